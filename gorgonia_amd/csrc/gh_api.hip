@@ -1,0 +1,336 @@
+// Context, memory, submission and graph entry points of libgorgonia_hip.so.
+// Replaces what Gorgonia's cuda.Engine gets from gorgonia.org/cu's
+// BatchedContext: context creation (cuda/external.go:112-170), queued copies,
+// kernel launch (cuda/arith.go:62) and DoWork/Signal (cuda/external.go:223).
+#include <cstdio>
+#include <cstring>
+
+#include "gh_internal.h"
+
+int gh_fail(gh_ctx* ctx, int code, const std::string& msg) {
+  if (ctx && ctx->err == GH_OK) {
+    ctx->err = code;
+    ctx->errmsg = msg;
+  }
+  return code;
+}
+
+int gh_check_hip(gh_ctx* ctx, hipError_t e, const char* what) {
+  if (e == hipSuccess) return GH_OK;
+  std::string m = std::string(what) + ": " + hipGetErrorString(e);
+  return gh_fail(ctx, GH_EDEVICE, m);
+}
+
+extern "C" {
+
+const char* gh_version(void) { return "gorgonia_hip 0.1 (gfx950)"; }
+
+int gh_device_count(int* out) {
+  if (!out) return GH_EINVAL;
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess) { *out = 0; return GH_EDEVICE; }
+  *out = n;
+  return GH_OK;
+}
+
+int gh_init(int device, int64_t arena_bytes, gh_ctx** out) {
+  if (!out || arena_bytes < 0) return GH_EINVAL;
+  *out = nullptr;
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || device < 0 || device >= n) return GH_EDEVICE;
+  if (hipSetDevice(device) != hipSuccess) return GH_EDEVICE;
+  gh_ctx* ctx = new gh_ctx();
+  ctx->device = device;
+  // Default priority only: mixed stream priorities are not used anywhere.
+  if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) {
+    delete ctx;
+    return GH_EDEVICE;
+  }
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->cu_count = prop.multiProcessorCount;
+  if (arena_bytes > 0) {
+    size_t free_b = 0, total_b = 0;
+    hipMemGetInfo(&free_b, &total_b);
+    if ((size_t)arena_bytes >= free_b) {  // cuda/external.go:159-161
+      hipStreamDestroy(ctx->stream);
+      delete ctx;
+      return GH_EOOM;
+    }
+    if (hipMalloc(&ctx->arena, (size_t)arena_bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      hipStreamDestroy(ctx->stream);
+      delete ctx;
+      return GH_EOOM;
+    }
+    ctx->arena_bytes = arena_bytes;
+  }
+  // Context-owned scratch: split-K partial sums and reduction flags.
+  ctx->workspace_bytes = 64ll << 20;
+  if (hipMalloc(&ctx->workspace, (size_t)ctx->workspace_bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    ctx->workspace = nullptr;
+    ctx->workspace_bytes = 0;
+  }
+  *out = ctx;
+  return GH_OK;
+}
+
+int gh_close(gh_ctx* ctx) {
+  if (!ctx) return GH_EINVAL;
+  hipSetDevice(ctx->device);
+  hipStreamSynchronize(ctx->stream);
+  for (auto& g : ctx->graphs) {
+    if (g.exec) hipGraphExecDestroy(g.exec);
+    if (g.graph) hipGraphDestroy(g.graph);
+  }
+  for (auto& e : ctx->events)
+    if (e) hipEventDestroy(e);
+  if (ctx->workspace) hipFree(ctx->workspace);
+  if (ctx->arena) hipFree(ctx->arena);
+  hipStreamDestroy(ctx->stream);
+  delete ctx;
+  return GH_OK;
+}
+
+int gh_device_info(gh_ctx* ctx, gh_devinfo* out) {
+  if (!ctx || !out) return GH_EINVAL;
+  hipDeviceProp_t p;
+  int rc = gh_check_hip(ctx, hipGetDeviceProperties(&p, ctx->device), "hipGetDeviceProperties");
+  if (rc) return rc;
+  memset(out, 0, sizeof(*out));
+  out->wavefront_size = p.warpSize;
+  out->max_threads_per_block = p.maxThreadsPerBlock;
+  out->max_grid_x = p.maxGridSize[0];
+  out->max_grid_y = p.maxGridSize[1];
+  out->max_grid_z = p.maxGridSize[2];
+  out->max_block_x = p.maxThreadsDim[0];
+  out->max_block_y = p.maxThreadsDim[1];
+  out->max_block_z = p.maxThreadsDim[2];
+  out->compute_units = p.multiProcessorCount;
+  out->lds_bytes_per_block = (int32_t)p.sharedMemPerBlock;
+  size_t f = 0, t = 0;
+  hipMemGetInfo(&f, &t);
+  out->free_mem = (int64_t)f;
+  out->total_mem = (int64_t)t;
+  snprintf(out->arch, sizeof(out->arch), "%s", p.gcnArchName);
+  return GH_OK;
+}
+
+gh_devptr gh_arena_base(gh_ctx* ctx) { return ctx ? (gh_devptr)(uintptr_t)ctx->arena : 0; }
+int64_t gh_arena_size(gh_ctx* ctx) { return ctx ? ctx->arena_bytes : 0; }
+
+int gh_malloc(gh_ctx* ctx, int64_t bytes, gh_devptr* out) {
+  if (!ctx || !out || bytes <= 0) return GH_EINVAL;
+  void* p = nullptr;
+  if (hipMalloc(&p, (size_t)bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return GH_EOOM;
+  }
+  *out = (gh_devptr)(uintptr_t)p;
+  return GH_OK;
+}
+
+int gh_free(gh_ctx* ctx, gh_devptr p) {
+  if (!ctx) return GH_EINVAL;
+  if (!p) return GH_OK;
+  return gh_check_hip(ctx, hipFree((void*)(uintptr_t)p), "hipFree");
+}
+
+int gh_host_alloc(gh_ctx* ctx, int64_t bytes, void** out) {
+  if (!ctx || !out || bytes <= 0) return GH_EINVAL;
+  if (hipHostMalloc(out, (size_t)bytes, hipHostMallocDefault) != hipSuccess) {
+    (void)hipGetLastError();
+    return GH_EOOM;
+  }
+  return GH_OK;
+}
+
+int gh_host_free(gh_ctx* ctx, void* p) {
+  if (!ctx) return GH_EINVAL;
+  if (!p) return GH_OK;
+  return gh_check_hip(ctx, hipHostFree(p), "hipHostFree");
+}
+
+int gh_memcpy_h2d(gh_ctx* ctx, gh_devptr dst, const void* src, int64_t bytes) {
+  if (!ctx || bytes < 0 || (bytes > 0 && (!dst || !src))) return GH_EINVAL;
+  if (ctx->err) return ctx->err;
+  if (bytes == 0) return GH_OK;
+  return gh_check_hip(ctx,
+                      hipMemcpyAsync((void*)(uintptr_t)dst, src, (size_t)bytes,
+                                     hipMemcpyHostToDevice, ctx->stream),
+                      "hipMemcpyAsync(H2D)");
+}
+
+int gh_memcpy_d2h(gh_ctx* ctx, void* dst, gh_devptr src, int64_t bytes) {
+  if (!ctx || bytes < 0 || (bytes > 0 && (!dst || !src))) return GH_EINVAL;
+  if (ctx->err) return ctx->err;
+  if (bytes == 0) return GH_OK;
+  return gh_check_hip(ctx,
+                      hipMemcpyAsync(dst, (const void*)(uintptr_t)src, (size_t)bytes,
+                                     hipMemcpyDeviceToHost, ctx->stream),
+                      "hipMemcpyAsync(D2H)");
+}
+
+int gh_memcpy_d2d(gh_ctx* ctx, gh_devptr dst, gh_devptr src, int64_t bytes) {
+  if (!ctx || bytes < 0 || (bytes > 0 && (!dst || !src))) return GH_EINVAL;
+  if (ctx->err) return ctx->err;
+  if (bytes == 0) return GH_OK;
+  return gh_check_hip(ctx,
+                      hipMemcpyAsync((void*)(uintptr_t)dst, (const void*)(uintptr_t)src,
+                                     (size_t)bytes, hipMemcpyDeviceToDevice, ctx->stream),
+                      "hipMemcpyAsync(D2D)");
+}
+
+static int dispatch(gh_ctx* ctx, const gh_cmd& c) {
+  switch (c.opcode) {
+    case GH_OP_NOP: return GH_OK;
+    case GH_OP_ELEM_BIN: return gh_launch_elem_bin(ctx, c);
+    case GH_OP_ELEM_UNARY: return gh_launch_elem_unary(ctx, c);
+    case GH_OP_BCAST_BIN: return gh_launch_bcast_bin(ctx, c);
+    case GH_OP_MEMCPY_D2D: return gh_memcpy_d2d(ctx, c.ptr[0], c.ptr[1], c.dim[0]);
+    case GH_OP_GEMM: return gh_launch_gemm(ctx, c);
+    case GH_OP_GEMV: return gh_launch_gemv(ctx, c);
+    case GH_OP_OUTER: return gh_launch_outer(ctx, c);
+    case GH_OP_CONV2D: return gh_launch_conv2d(ctx, c);
+    case GH_OP_MAXPOOL2D: return gh_launch_maxpool2d(ctx, c);
+    case GH_OP_BN_INFER: return gh_launch_bn_infer(ctx, c);
+    case GH_OP_RELU: return gh_launch_relu(ctx, c);
+    case GH_OP_LEAKY_RELU: return gh_launch_leaky_relu(ctx, c);
+    case GH_OP_SOFTMAX: return gh_launch_softmax(ctx, c);
+    case GH_OP_HAS_NAN:
+    case GH_OP_HAS_INF: return gh_launch_has_nan_inf(ctx, c);
+    case GH_OP_FILL: return gh_launch_fill(ctx, c);
+  }
+  return GH_ENOFUNC;
+}
+
+int gh_validate(const gh_cmd* cmds, int n, char* msg, int msg_len) {
+  if (n < 0 || (n > 0 && !cmds)) return GH_EINVAL;
+  for (int i = 0; i < n; i++) {
+    std::string m;
+    int rc = gh_validate_cmd(cmds[i], m);
+    if (rc) {
+      if (msg && msg_len > 0) snprintf(msg, (size_t)msg_len, "cmd %d: %s", i, m.c_str());
+      return rc;
+    }
+  }
+  if (msg && msg_len > 0) msg[0] = 0;
+  return GH_OK;
+}
+
+int gh_submit(gh_ctx* ctx, const gh_cmd* cmds, int n) {
+  if (!ctx || n < 0 || (n > 0 && !cmds)) return GH_EINVAL;
+  if (ctx->err) return ctx->err;
+  for (int i = 0; i < n; i++) {
+    std::string m;
+    int rc = gh_validate_cmd(cmds[i], m);
+    if (rc) return gh_fail(ctx, rc, "cmd " + std::to_string(i) + ": " + m);
+    rc = dispatch(ctx, cmds[i]);
+    if (rc) return rc;
+  }
+  return GH_OK;
+}
+
+int gh_sync(gh_ctx* ctx) {
+  if (!ctx) return GH_EINVAL;
+  if (ctx->capturing) return gh_fail(ctx, GH_ESTATE, "gh_sync during graph capture");
+  hipError_t e = hipStreamSynchronize(ctx->stream);
+  if (e != hipSuccess) gh_check_hip(ctx, e, "hipStreamSynchronize");
+  return ctx->err;
+}
+
+int gh_graph_begin(gh_ctx* ctx) {
+  if (!ctx) return GH_EINVAL;
+  if (ctx->err) return ctx->err;
+  if (ctx->capturing) return gh_fail(ctx, GH_ESTATE, "graph capture already active");
+  int rc = gh_check_hip(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal),
+                        "hipStreamBeginCapture");
+  if (rc) return rc;
+  ctx->capturing = true;
+  return GH_OK;
+}
+
+int gh_graph_end(gh_ctx* ctx, int* graph_id) {
+  if (!ctx || !graph_id) return GH_EINVAL;
+  if (!ctx->capturing) return gh_fail(ctx, GH_ESTATE, "no graph capture active");
+  ctx->capturing = false;
+  hipGraph_t g = nullptr;
+  hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+  if (e != hipSuccess) return gh_check_hip(ctx, e, "hipStreamEndCapture");
+  if (ctx->err) {  // a submit failed while capturing: drop the graph
+    if (g) hipGraphDestroy(g);
+    return ctx->err;
+  }
+  hipGraphExec_t ex = nullptr;
+  e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    hipGraphDestroy(g);
+    return gh_check_hip(ctx, e, "hipGraphInstantiate");
+  }
+  int id = -1;
+  for (size_t i = 0; i < ctx->graphs.size(); i++)
+    if (!ctx->graphs[i].used) { id = (int)i; break; }
+  if (id < 0) {
+    ctx->graphs.emplace_back();
+    id = (int)ctx->graphs.size() - 1;
+  }
+  ctx->graphs[id].graph = g;
+  ctx->graphs[id].exec = ex;
+  ctx->graphs[id].used = true;
+  *graph_id = id;
+  return GH_OK;
+}
+
+int gh_graph_launch(gh_ctx* ctx, int id) {
+  if (!ctx) return GH_EINVAL;
+  if (ctx->err) return ctx->err;
+  if (id < 0 || id >= (int)ctx->graphs.size() || !ctx->graphs[id].used)
+    return gh_fail(ctx, GH_EINVAL, "unknown graph id");
+  return gh_check_hip(ctx, hipGraphLaunch(ctx->graphs[id].exec, ctx->stream), "hipGraphLaunch");
+}
+
+int gh_graph_destroy(gh_ctx* ctx, int id) {
+  if (!ctx) return GH_EINVAL;
+  if (id < 0 || id >= (int)ctx->graphs.size() || !ctx->graphs[id].used) return GH_EINVAL;
+  hipStreamSynchronize(ctx->stream);
+  hipGraphExecDestroy(ctx->graphs[id].exec);
+  hipGraphDestroy(ctx->graphs[id].graph);
+  ctx->graphs[id] = gh_graph_slot();
+  return GH_OK;
+}
+
+int gh_last_error(gh_ctx* ctx, char* buf, int len) {
+  if (!ctx) return GH_EINVAL;
+  if (buf && len > 0) snprintf(buf, (size_t)len, "%s", ctx->errmsg.c_str());
+  return ctx->err;
+}
+
+int gh_clear_error(gh_ctx* ctx) {
+  if (!ctx) return GH_EINVAL;
+  ctx->err = GH_OK;
+  ctx->errmsg.clear();
+  (void)hipGetLastError();
+  return GH_OK;
+}
+
+int gh_event_record(gh_ctx* ctx, int slot) {
+  if (!ctx || slot < 0 || slot >= 64) return GH_EINVAL;
+  if (ctx->err) return ctx->err;
+  if (!ctx->events[slot]) {
+    int rc = gh_check_hip(ctx, hipEventCreate(&ctx->events[slot]), "hipEventCreate");
+    if (rc) return rc;
+  }
+  return gh_check_hip(ctx, hipEventRecord(ctx->events[slot], ctx->stream), "hipEventRecord");
+}
+
+int gh_event_elapsed_ms(gh_ctx* ctx, int start, int stop, float* ms) {
+  if (!ctx || !ms || start < 0 || start >= 64 || stop < 0 || stop >= 64) return GH_EINVAL;
+  if (!ctx->events[start] || !ctx->events[stop]) return GH_ESTATE;
+  int rc = gh_check_hip(ctx, hipEventSynchronize(ctx->events[stop]), "hipEventSynchronize");
+  if (rc) return rc;
+  return gh_check_hip(ctx, hipEventElapsedTime(ms, ctx->events[start], ctx->events[stop]),
+                      "hipEventElapsedTime");
+}
+
+}  // extern "C"

@@ -1,0 +1,65 @@
+// Internal declarations shared by the translation units of libgorgonia_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "gorgonia_hip.h"
+
+struct gh_graph_slot {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  bool used = false;
+};
+
+struct gh_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  void* arena = nullptr;
+  int64_t arena_bytes = 0;
+  int err = GH_OK;          // sticky status
+  std::string errmsg;
+  bool capturing = false;
+  std::vector<gh_graph_slot> graphs;
+  hipEvent_t events[64] = {};
+  int cu_count = 256;
+  // scratch owned by the context (split-K partials, reduction flags)
+  void* workspace = nullptr;
+  int64_t workspace_bytes = 0;
+};
+
+// Record a sticky error on the context and return its code.
+int gh_fail(gh_ctx* ctx, int code, const std::string& msg);
+int gh_check_hip(gh_ctx* ctx, hipError_t e, const char* what);
+
+// Per-family validators (host only) and launchers.  Launchers assume a
+// validated command.  Each returns GH_OK or a code with `msg` filled in.
+int gh_validate_cmd(const gh_cmd& c, std::string& msg);
+
+int gh_launch_elem_bin(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_elem_unary(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_bcast_bin(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_relu(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_leaky_relu(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_fill(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_has_nan_inf(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_gemv(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_outer(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_maxpool2d(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_bn_infer(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_softmax(gh_ctx* ctx, const gh_cmd& c);
+
+static inline uint32_t gh_fn(uint32_t flags) { return flags & 0xffu; }
+static inline uint32_t gh_mode(uint32_t flags) { return (flags >> 8) & 0xfu; }
+static inline uint32_t gh_dtype_of(uint32_t flags) { return (flags >> 12) & 0xfu; }
+
+// Output sizes shared by validators, launchers and the host mirror.
+static inline int64_t gh_conv_out(int64_t in, int64_t k, int64_t pad, int64_t stride, int64_t dil) {
+  return (in + 2 * pad - (dil * (k - 1) + 1)) / stride + 1;  // op_nn.go:311-315
+}
+static inline int64_t gh_pool_out(int64_t in, int64_t k, int64_t padA, int64_t padB, int64_t stride) {
+  return (in + padA + padB - (k - 1) - 1) / stride + 1;      // op_nn.go:810-816
+}

@@ -1,0 +1,547 @@
+// Elementwise kernels for gfx950: binary (vv/vs/sv/ss), unary, fused
+// broadcast, ReLU / LeakyReLU, fill and the NaN/Inf predicates.
+//
+// All of them are HBM-bound.  Each thread moves 16-byte vectors (float4 /
+// double2) in a grid-stride loop, several independent vectors per iteration so
+// that enough loads are in flight to cover HBM latency; a lane-contiguous
+// layout keeps every wavefront access a fully coalesced 1 KiB segment.
+//
+// Numerics: this file is compiled with -ffp-contract=off, denormals kept and
+// IEEE division, so add/sub/mul/div/compare are bit-identical to the CPU
+// engine (the reference builds its PTX the same way, cmd/cudagen/main.go:41-43).
+// Transcendentals are evaluated in float64 and rounded once, the form the CPU
+// engine uses for sigmoid (math_nooptim.go:36-44) and tanh (math_nooptim.go:22).
+#include "gh_internal.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;
+
+template <class T> struct VecOf;
+template <> struct VecOf<float> { typedef float type __attribute__((ext_vector_type(4))); static constexpr int N = 4; };
+template <> struct VecOf<double> { typedef double type __attribute__((ext_vector_type(2))); static constexpr int N = 2; };
+
+// ---- scalar functions ------------------------------------------------------
+
+template <int FN, class T>
+__device__ __forceinline__ T bin_apply(T a, T b) {
+  if constexpr (FN == GH_ADD) return a + b;
+  else if constexpr (FN == GH_SUB) return a - b;
+  else if constexpr (FN == GH_MUL) return a * b;
+  else if constexpr (FN == GH_DIV) return a / b;
+  else if constexpr (FN == GH_POW) return (T)pow((double)a, (double)b);
+  else if constexpr (FN == GH_LT) return a < b ? (T)1 : (T)0;
+  else if constexpr (FN == GH_LTE) return a <= b ? (T)1 : (T)0;
+  else if constexpr (FN == GH_GT) return a > b ? (T)1 : (T)0;
+  else if constexpr (FN == GH_GTE) return a >= b ? (T)1 : (T)0;
+  else if constexpr (FN == GH_EQ) return a == b ? (T)1 : (T)0;
+  else return a != b ? (T)1 : (T)0;
+}
+
+// tanh in float64 from one exp: 1 - 2/(e^{2x}+1); a short odd series near 0
+// where that form cancels.  Error stays far below half a float32 ulp.
+__device__ __forceinline__ double tanh_f64_for_f32(double x) {
+  double ax = fabs(x);
+  double r;
+  if (ax < 0.00390625) {  // 2^-8: |x^7 * 17/315| < 2^-60 relative
+    double x2 = ax * ax;
+    r = ax * (1.0 + x2 * (-1.0 / 3.0 + x2 * (2.0 / 15.0)));
+  } else if (ax > 20.0) {
+    r = 1.0;
+  } else {
+    r = 1.0 - 2.0 / (exp(2.0 * ax) + 1.0);
+  }
+  return x < 0 ? -r : r;
+}
+
+template <int FN>
+__device__ __forceinline__ float unary_apply(float x) {
+  if constexpr (FN == GH_ABS) return fabsf(x);
+  else if constexpr (FN == GH_SIGN) return (float)((x > 0.0f) - (x < 0.0f));
+  else if constexpr (FN == GH_CEIL) return ceilf(x);
+  else if constexpr (FN == GH_FLOOR) return floorf(x);
+  else if constexpr (FN == GH_SIN) return (float)sin((double)x);
+  else if constexpr (FN == GH_COS) return (float)cos((double)x);
+  else if constexpr (FN == GH_EXP) return (float)exp((double)x);
+  else if constexpr (FN == GH_LN) return (float)log((double)x);
+  else if constexpr (FN == GH_LOG2) return (float)log2((double)x);
+  else if constexpr (FN == GH_NEG) return -x;
+  else if constexpr (FN == GH_SQUARE) return x * x;
+  else if constexpr (FN == GH_SQRT) return sqrtf(x);
+  else if constexpr (FN == GH_INVERSE) return 1.0f / x;
+  else if constexpr (FN == GH_INVSQRT) return 1.0f / sqrtf(x);
+  else if constexpr (FN == GH_CUBE) return x * x * x;
+  else if constexpr (FN == GH_TANH) {
+    if (x != x) return x;
+    return (float)tanh_f64_for_f32((double)x);
+  } else if constexpr (FN == GH_SIGMOID) {
+    if (x < -88.0f) return 0.0f;
+    if (x > 15.0f) return 1.0f;
+    return (float)(1.0 / (1.0 + exp((double)(-x))));
+  } else if constexpr (FN == GH_LOG1P) return (float)log1p((double)x);
+  else if constexpr (FN == GH_EXPM1) return (float)expm1((double)x);
+  else {  // softplus
+    if (x < -103.0f) return 0.0f;
+    if (x > 14.0f) return x;
+    return (float)log1p(exp((double)x));
+  }
+}
+
+template <int FN>
+__device__ __forceinline__ double unary_apply(double x) {
+  if constexpr (FN == GH_ABS) return fabs(x);
+  else if constexpr (FN == GH_SIGN) return (double)((x > 0.0) - (x < 0.0));
+  else if constexpr (FN == GH_CEIL) return ceil(x);
+  else if constexpr (FN == GH_FLOOR) return floor(x);
+  else if constexpr (FN == GH_SIN) return sin(x);
+  else if constexpr (FN == GH_COS) return cos(x);
+  else if constexpr (FN == GH_EXP) return exp(x);
+  else if constexpr (FN == GH_LN) return log(x);
+  else if constexpr (FN == GH_LOG2) return log2(x);
+  else if constexpr (FN == GH_NEG) return -x;
+  else if constexpr (FN == GH_SQUARE) return x * x;
+  else if constexpr (FN == GH_SQRT) return sqrt(x);
+  else if constexpr (FN == GH_INVERSE) return 1.0 / x;
+  else if constexpr (FN == GH_INVSQRT) return 1.0 / sqrt(x);
+  else if constexpr (FN == GH_CUBE) return x * x * x;
+  else if constexpr (FN == GH_TANH) return tanh(x);
+  else if constexpr (FN == GH_SIGMOID) {
+    if (x < -709.0) return 0.0;
+    if (x > 19.0) return 1.0;
+    return 1.0 / (1.0 + exp(-x));
+  } else if constexpr (FN == GH_LOG1P) return log1p(x);
+  else if constexpr (FN == GH_EXPM1) return expm1(x);
+  else {
+    if (x < -708.0) return 0.0;
+    if (x > 16.0) return x;
+    return log1p(exp(x));
+  }
+}
+
+// ---- binary kernels ---------------------------------------------------------
+// MODE vv: A[i] = A[i] op B[i]   vs: A[i] = A[i] op B[0]
+//      sv: B[i] = A[0] op B[i]   ss: A[0] = A[0] op B[0]   (elembinop.cu:13-35)
+// POW2: vs mode only; the exponent was read as 2 by the kernel itself, so
+// x*x is used (equal to the correctly rounded pow(x,2)).
+
+template <int FN, class T, int MODE>
+__global__ __launch_bounds__(kBlock) void k_bin_vec(T* __restrict__ A, T* __restrict__ B, int64_t n) {
+  using V = typename VecOf<T>::type;
+  constexpr int N = VecOf<T>::N;
+  const int64_t nv = n / N;
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  T s = (T)0;
+  bool pow2 = false;
+  if constexpr (MODE == GH_VS) { s = B[0]; if constexpr (FN == GH_POW) pow2 = (s == (T)2); }
+  if constexpr (MODE == GH_SV) s = A[0];
+  V* __restrict__ Av = reinterpret_cast<V*>(A);
+  V* __restrict__ Bv = reinterpret_cast<V*>(B);
+  for (; i + (kUnroll - 1) * stride < nv; i += kUnroll * stride) {
+    V a[kUnroll], b[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      if constexpr (MODE != GH_SV) a[u] = __builtin_nontemporal_load(&Av[i + u * stride]);
+      if constexpr (MODE != GH_VS) b[u] = __builtin_nontemporal_load(&Bv[i + u * stride]);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      V r;
+#pragma unroll
+      for (int e = 0; e < N; e++) {
+        if constexpr (MODE == GH_VV) r[e] = bin_apply<FN, T>(a[u][e], b[u][e]);
+        else if constexpr (MODE == GH_VS) {
+          if constexpr (FN == GH_POW) r[e] = pow2 ? a[u][e] * a[u][e] : bin_apply<FN, T>(a[u][e], s);
+          else r[e] = bin_apply<FN, T>(a[u][e], s);
+        } else r[e] = bin_apply<FN, T>(s, b[u][e]);
+      }
+      if constexpr (MODE == GH_SV) __builtin_nontemporal_store(r, &Bv[i + u * stride]);
+      else __builtin_nontemporal_store(r, &Av[i + u * stride]);
+    }
+  }
+  for (; i < nv; i += stride) {
+    V a, b, r;
+    if constexpr (MODE != GH_SV) a = Av[i];
+    if constexpr (MODE != GH_VS) b = Bv[i];
+#pragma unroll
+    for (int e = 0; e < N; e++) {
+      if constexpr (MODE == GH_VV) r[e] = bin_apply<FN, T>(a[e], b[e]);
+      else if constexpr (MODE == GH_VS) {
+        if constexpr (FN == GH_POW) r[e] = pow2 ? a[e] * a[e] : bin_apply<FN, T>(a[e], s);
+        else r[e] = bin_apply<FN, T>(a[e], s);
+      } else r[e] = bin_apply<FN, T>(s, b[e]);
+    }
+    if constexpr (MODE == GH_SV) Bv[i] = r; else Av[i] = r;
+  }
+  // scalar tail (n % N elements)
+  const int64_t t = nv * N + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (t < n) {
+    if constexpr (MODE == GH_VV) A[t] = bin_apply<FN, T>(A[t], B[t]);
+    else if constexpr (MODE == GH_VS) {
+      if constexpr (FN == GH_POW) A[t] = pow2 ? A[t] * A[t] : bin_apply<FN, T>(A[t], s);
+      else A[t] = bin_apply<FN, T>(A[t], s);
+    } else B[t] = bin_apply<FN, T>(s, B[t]);
+  }
+}
+
+// Unaligned operands, or scalar-scalar: plain one-element-per-thread loop.
+template <int FN, class T, int MODE>
+__global__ __launch_bounds__(kBlock) void k_bin_scalar(T* A, T* B, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  T s = (T)0;
+  if constexpr (MODE == GH_VS) s = B[0];
+  if constexpr (MODE == GH_SV || MODE == GH_SS) s = A[0];
+  if constexpr (MODE == GH_SS) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) A[0] = bin_apply<FN, T>(s, B[0]);
+    return;
+  }
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    if constexpr (MODE == GH_VV) A[i] = bin_apply<FN, T>(A[i], B[i]);
+    else if constexpr (MODE == GH_VS) A[i] = bin_apply<FN, T>(A[i], s);
+    else if constexpr (MODE == GH_SV) B[i] = bin_apply<FN, T>(s, B[i]);
+  }
+}
+
+template <int FN, class T>
+__global__ __launch_bounds__(kBlock) void k_unary_vec(T* __restrict__ A, int64_t n) {
+  using V = typename VecOf<T>::type;
+  constexpr int N = VecOf<T>::N;
+  const int64_t nv = n / N;
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  V* __restrict__ Av = reinterpret_cast<V*>(A);
+  for (; i + (kUnroll - 1) * stride < nv; i += kUnroll * stride) {
+    V a[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) a[u] = __builtin_nontemporal_load(&Av[i + u * stride]);
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      V r;
+#pragma unroll
+      for (int e = 0; e < N; e++) r[e] = unary_apply<FN>(a[u][e]);
+      __builtin_nontemporal_store(r, &Av[i + u * stride]);
+    }
+  }
+  for (; i < nv; i += stride) {
+    V a = Av[i], r;
+#pragma unroll
+    for (int e = 0; e < N; e++) r[e] = unary_apply<FN>(a[e]);
+    Av[i] = r;
+  }
+  const int64_t t = nv * N + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (t < n) A[t] = unary_apply<FN>(A[t]);
+}
+
+template <int FN, class T>
+__global__ __launch_bounds__(kBlock) void k_unary_scalar(T* A, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride)
+    A[i] = unary_apply<FN>(A[i]);
+}
+
+// ---- fused broadcast --------------------------------------------------------
+// dst[o,m,i] = big[o,m,i] op small[m]  (or small op big with SMALL_LEFT).
+// Row form (inner == 1, mid % 4 == 0): each thread owns one float4 column
+// group, keeps its slice of `small` in registers and walks rows.
+template <int FN, bool LEFT>
+__global__ __launch_bounds__(kBlock) void k_bcast_row(float* __restrict__ dst,
+                                                      const float* __restrict__ big,
+                                                      const float* __restrict__ small,
+                                                      int64_t rows, int64_t colv) {
+  typedef float V __attribute__((ext_vector_type(4)));
+  const int64_t cv = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (cv >= colv) return;
+  const V s = reinterpret_cast<const V*>(small)[cv];
+  const V* __restrict__ bv = reinterpret_cast<const V*>(big);
+  V* __restrict__ dv = reinterpret_cast<V*>(dst);
+  int64_t r = blockIdx.y;
+  const int64_t rs = gridDim.y;
+  for (; r + (kUnroll - 1) * rs < rows; r += kUnroll * rs) {
+    V a[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) a[u] = __builtin_nontemporal_load(&bv[(r + u * rs) * colv + cv]);
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      V o;
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        o[e] = LEFT ? bin_apply<FN, float>(s[e], a[u][e]) : bin_apply<FN, float>(a[u][e], s[e]);
+      __builtin_nontemporal_store(o, &dv[(r + u * rs) * colv + cv]);
+    }
+  }
+  for (; r < rows; r += rs) {
+    V a = bv[r * colv + cv], o;
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      o[e] = LEFT ? bin_apply<FN, float>(s[e], a[e]) : bin_apply<FN, float>(a[e], s[e]);
+    dv[r * colv + cv] = o;
+  }
+}
+
+// General form: one element per thread, small index = (idx / inner) % mid.
+template <int FN, bool LEFT>
+__global__ __launch_bounds__(kBlock) void k_bcast_generic(float* dst, const float* big,
+                                                          const float* small, int64_t n,
+                                                          int64_t mid, int64_t inner) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    const float s = small[(i / inner) % mid];
+    const float a = big[i];
+    dst[i] = LEFT ? bin_apply<FN, float>(s, a) : bin_apply<FN, float>(a, s);
+  }
+}
+
+// ---- ReLU / LeakyReLU in the reference's arithmetic form --------------------
+// Rectify: x * float(x >= 0) (nn.go:136-163) - negative inputs give -0.0.
+// LeakyRelu: x*(x>=0) + (x*(x<0))*alpha (nn.go:83-131).
+__device__ __forceinline__ float relu_ref(float x) { return x * (x >= 0.0f ? 1.0f : 0.0f); }
+__device__ __forceinline__ float leaky_ref(float x, float alpha) {
+  const float pos = x * (x >= 0.0f ? 1.0f : 0.0f);
+  const float neg = x * (x < 0.0f ? 1.0f : 0.0f);
+  const float na = neg * alpha;
+  return pos + na;
+}
+
+template <bool LEAKY>
+__global__ __launch_bounds__(kBlock) void k_relu(const float* __restrict__ x, float* __restrict__ y,
+                                                 int64_t n, float alpha, int vec) {
+  typedef float V __attribute__((ext_vector_type(4)));
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (vec) {
+    const int64_t nv = n / 4;
+    const V* xv = reinterpret_cast<const V*>(x);
+    V* yv = reinterpret_cast<V*>(y);
+    for (; i < nv; i += stride) {
+      V a = xv[i], r;
+#pragma unroll
+      for (int e = 0; e < 4; e++) r[e] = LEAKY ? leaky_ref(a[e], alpha) : relu_ref(a[e]);
+      yv[i] = r;
+    }
+    const int64_t t = nv * 4 + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t < n) y[t] = LEAKY ? leaky_ref(x[t], alpha) : relu_ref(x[t]);
+  } else {
+    for (; i < n; i += stride) y[i] = LEAKY ? leaky_ref(x[i], alpha) : relu_ref(x[i]);
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void k_fill(float* A, int64_t n, float v) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) A[i] = v;
+}
+
+__global__ void k_set_flag(int* flag, int v) { *flag = v; }
+
+// misc.hasNaN / misc.hasInf (misc.cu:14-56).  The reference increments a
+// counter without atomics; here any matching lane stores 1 (a benign race on
+// a single value).
+template <class T, bool NAN_CHECK>
+__global__ __launch_bounds__(kBlock) void k_has(const T* __restrict__ A, int64_t n, int* flag) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  bool hit = false;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    const T v = A[i];
+    hit |= NAN_CHECK ? (v != v) : (v == (T)INFINITY || v == -(T)INFINITY);
+  }
+  if (hit) *flag = 1;
+}
+
+// ---- launch helpers ---------------------------------------------------------
+
+inline int grid_for(gh_ctx* ctx, int64_t work_items, int per_thread) {
+  int64_t blocks = (work_items + (int64_t)kBlock * per_thread - 1) / ((int64_t)kBlock * per_thread);
+  const int64_t cap = (int64_t)ctx->cu_count * 8;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return (int)blocks;
+}
+
+inline bool aligned16(uint64_t p) { return (p & 15u) == 0; }
+
+template <int FN, class T>
+int launch_bin_fn(gh_ctx* ctx, const gh_cmd& c) {
+  T* A = (T*)(uintptr_t)c.ptr[0];
+  T* B = (T*)(uintptr_t)c.ptr[1];
+  const int64_t n = c.dim[0];
+  const uint32_t mode = gh_mode(c.flags);
+  constexpr int N = VecOf<T>::N;
+  if (n == 0) return GH_OK;
+  bool vec = n >= N;
+  if (mode == GH_VV) vec = vec && aligned16(c.ptr[0]) && aligned16(c.ptr[1]);
+  if (mode == GH_VS) vec = vec && aligned16(c.ptr[0]);
+  if (mode == GH_SV) vec = vec && aligned16(c.ptr[1]);
+  if (mode == GH_SS) vec = false;
+  const int gv = grid_for(ctx, n / N + N, kUnroll);
+  const int gs = grid_for(ctx, n, 4);
+#define GH_LAUNCH_MODE(M)                                                                   \
+  if (vec) hipLaunchKernelGGL((k_bin_vec<FN, T, M>), dim3(gv), dim3(kBlock), 0, ctx->stream, A, B, n); \
+  else hipLaunchKernelGGL((k_bin_scalar<FN, T, M>), dim3(gs), dim3(kBlock), 0, ctx->stream, A, B, n);
+  switch (mode) {
+    case GH_VV: GH_LAUNCH_MODE(GH_VV) break;
+    case GH_VS: GH_LAUNCH_MODE(GH_VS) break;
+    case GH_SV: GH_LAUNCH_MODE(GH_SV) break;
+    default:
+      hipLaunchKernelGGL((k_bin_scalar<FN, T, GH_SS>), dim3(1), dim3(kBlock), 0, ctx->stream, A, B, n);
+  }
+#undef GH_LAUNCH_MODE
+  return gh_check_hip(ctx, hipGetLastError(), "elementwise binary launch");
+}
+
+template <class T>
+int launch_bin(gh_ctx* ctx, const gh_cmd& c) {
+  switch (gh_fn(c.flags)) {
+    case GH_ADD: return launch_bin_fn<GH_ADD, T>(ctx, c);
+    case GH_SUB: return launch_bin_fn<GH_SUB, T>(ctx, c);
+    case GH_MUL: return launch_bin_fn<GH_MUL, T>(ctx, c);
+    case GH_DIV: return launch_bin_fn<GH_DIV, T>(ctx, c);
+    case GH_POW: return launch_bin_fn<GH_POW, T>(ctx, c);
+    case GH_LT: return launch_bin_fn<GH_LT, T>(ctx, c);
+    case GH_LTE: return launch_bin_fn<GH_LTE, T>(ctx, c);
+    case GH_GT: return launch_bin_fn<GH_GT, T>(ctx, c);
+    case GH_GTE: return launch_bin_fn<GH_GTE, T>(ctx, c);
+    case GH_EQ: return launch_bin_fn<GH_EQ, T>(ctx, c);
+    case GH_NE: return launch_bin_fn<GH_NE, T>(ctx, c);
+  }
+  return gh_fail(ctx, GH_ENOFUNC, "unknown binary function");
+}
+
+template <int FN, class T>
+int launch_unary_fn(gh_ctx* ctx, const gh_cmd& c) {
+  T* A = (T*)(uintptr_t)c.ptr[0];
+  const int64_t n = c.dim[0];
+  constexpr int N = VecOf<T>::N;
+  if (n == 0) return GH_OK;
+  if (n >= N && aligned16(c.ptr[0]))
+    hipLaunchKernelGGL((k_unary_vec<FN, T>), dim3(grid_for(ctx, n / N + N, kUnroll)), dim3(kBlock), 0,
+                       ctx->stream, A, n);
+  else
+    hipLaunchKernelGGL((k_unary_scalar<FN, T>), dim3(grid_for(ctx, n, 4)), dim3(kBlock), 0,
+                       ctx->stream, A, n);
+  return gh_check_hip(ctx, hipGetLastError(), "elementwise unary launch");
+}
+
+template <class T>
+int launch_unary(gh_ctx* ctx, const gh_cmd& c) {
+  switch (gh_fn(c.flags)) {
+#define GH_U(F) case F: return launch_unary_fn<F, T>(ctx, c);
+    GH_U(GH_ABS) GH_U(GH_SIGN) GH_U(GH_CEIL) GH_U(GH_FLOOR) GH_U(GH_SIN) GH_U(GH_COS) GH_U(GH_EXP)
+    GH_U(GH_LN) GH_U(GH_LOG2) GH_U(GH_NEG) GH_U(GH_SQUARE) GH_U(GH_SQRT) GH_U(GH_INVERSE)
+    GH_U(GH_INVSQRT) GH_U(GH_CUBE) GH_U(GH_TANH) GH_U(GH_SIGMOID) GH_U(GH_LOG1P) GH_U(GH_EXPM1)
+    GH_U(GH_SOFTPLUS)
+#undef GH_U
+  }
+  return gh_fail(ctx, GH_ENOFUNC, "unknown unary function");
+}
+
+template <int FN>
+int launch_bcast_fn(gh_ctx* ctx, const gh_cmd& c) {
+  float* dst = (float*)(uintptr_t)c.ptr[0];
+  const float* big = (const float*)(uintptr_t)c.ptr[1];
+  const float* small = (const float*)(uintptr_t)c.ptr[2];
+  const int64_t outer = c.dim[0], mid = c.dim[1], inner = c.dim[2];
+  const int64_t n = outer * mid * inner;
+  const bool left = c.flags & GH_FLAG_SMALL_LEFT;
+  if (n == 0) return GH_OK;
+  const bool row = inner == 1 && (mid % 4) == 0 && aligned16(c.ptr[0]) && aligned16(c.ptr[1]) &&
+                   aligned16(c.ptr[2]);
+  if (row) {
+    const int64_t colv = mid / 4;
+    const int gx = (int)((colv + kBlock - 1) / kBlock);
+    int64_t gy = ((int64_t)ctx->cu_count * 8 + gx - 1) / gx;
+    const int64_t need = (outer + kUnroll - 1) / kUnroll;
+    if (gy > need) gy = need;
+    if (gy < 1) gy = 1;
+    if (gy > 65535) gy = 65535;
+    if (left)
+      hipLaunchKernelGGL((k_bcast_row<FN, true>), dim3(gx, (int)gy), dim3(kBlock), 0, ctx->stream, dst,
+                         big, small, outer, colv);
+    else
+      hipLaunchKernelGGL((k_bcast_row<FN, false>), dim3(gx, (int)gy), dim3(kBlock), 0, ctx->stream, dst,
+                         big, small, outer, colv);
+  } else {
+    const int g = grid_for(ctx, n, 4);
+    if (left)
+      hipLaunchKernelGGL((k_bcast_generic<FN, true>), dim3(g), dim3(kBlock), 0, ctx->stream, dst, big,
+                         small, n, mid, inner);
+    else
+      hipLaunchKernelGGL((k_bcast_generic<FN, false>), dim3(g), dim3(kBlock), 0, ctx->stream, dst, big,
+                         small, n, mid, inner);
+  }
+  return gh_check_hip(ctx, hipGetLastError(), "broadcast launch");
+}
+
+}  // namespace
+
+int gh_launch_elem_bin(gh_ctx* ctx, const gh_cmd& c) {
+  return gh_dtype_of(c.flags) == GH_F64 ? launch_bin<double>(ctx, c) : launch_bin<float>(ctx, c);
+}
+
+int gh_launch_elem_unary(gh_ctx* ctx, const gh_cmd& c) {
+  return gh_dtype_of(c.flags) == GH_F64 ? launch_unary<double>(ctx, c) : launch_unary<float>(ctx, c);
+}
+
+int gh_launch_bcast_bin(gh_ctx* ctx, const gh_cmd& c) {
+  switch (gh_fn(c.flags)) {
+    case GH_ADD: return launch_bcast_fn<GH_ADD>(ctx, c);
+    case GH_SUB: return launch_bcast_fn<GH_SUB>(ctx, c);
+    case GH_MUL: return launch_bcast_fn<GH_MUL>(ctx, c);
+    case GH_DIV: return launch_bcast_fn<GH_DIV>(ctx, c);
+    case GH_POW: return launch_bcast_fn<GH_POW>(ctx, c);
+    case GH_LT: return launch_bcast_fn<GH_LT>(ctx, c);
+    case GH_LTE: return launch_bcast_fn<GH_LTE>(ctx, c);
+    case GH_GT: return launch_bcast_fn<GH_GT>(ctx, c);
+    case GH_GTE: return launch_bcast_fn<GH_GTE>(ctx, c);
+    case GH_EQ: return launch_bcast_fn<GH_EQ>(ctx, c);
+    case GH_NE: return launch_bcast_fn<GH_NE>(ctx, c);
+  }
+  return gh_fail(ctx, GH_ENOFUNC, "unknown binary function");
+}
+
+int gh_launch_relu(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t n = c.dim[0];
+  if (n == 0) return GH_OK;
+  const int vec = aligned16(c.ptr[0]) && aligned16(c.ptr[1]) && n >= 4;
+  hipLaunchKernelGGL((k_relu<false>), dim3(grid_for(ctx, vec ? n / 4 + 4 : n, 2)), dim3(kBlock), 0,
+                     ctx->stream, (const float*)(uintptr_t)c.ptr[0], (float*)(uintptr_t)c.ptr[1], n,
+                     0.0f, vec);
+  return gh_check_hip(ctx, hipGetLastError(), "relu launch");
+}
+
+int gh_launch_leaky_relu(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t n = c.dim[0];
+  if (n == 0) return GH_OK;
+  const int vec = aligned16(c.ptr[0]) && aligned16(c.ptr[1]) && n >= 4;
+  hipLaunchKernelGGL((k_relu<true>), dim3(grid_for(ctx, vec ? n / 4 + 4 : n, 2)), dim3(kBlock), 0,
+                     ctx->stream, (const float*)(uintptr_t)c.ptr[0], (float*)(uintptr_t)c.ptr[1], n,
+                     c.f[0], vec);
+  return gh_check_hip(ctx, hipGetLastError(), "leaky relu launch");
+}
+
+int gh_launch_fill(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t n = c.dim[0];
+  if (n == 0) return GH_OK;
+  hipLaunchKernelGGL(k_fill, dim3(grid_for(ctx, n, 4)), dim3(kBlock), 0, ctx->stream,
+                     (float*)(uintptr_t)c.ptr[0], n, c.f[0]);
+  return gh_check_hip(ctx, hipGetLastError(), "fill launch");
+}
+
+int gh_launch_has_nan_inf(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t n = c.dim[0];
+  int* flag = (int*)(uintptr_t)c.ptr[1];
+  hipLaunchKernelGGL(k_set_flag, dim3(1), dim3(1), 0, ctx->stream, flag, 0);
+  if (n > 0) {
+    const int g = grid_for(ctx, n, 8);
+    const bool nanc = c.opcode == GH_OP_HAS_NAN;
+    if (gh_dtype_of(c.flags) == GH_F64) {
+      const double* A = (const double*)(uintptr_t)c.ptr[0];
+      if (nanc) hipLaunchKernelGGL((k_has<double, true>), dim3(g), dim3(kBlock), 0, ctx->stream, A, n, flag);
+      else hipLaunchKernelGGL((k_has<double, false>), dim3(g), dim3(kBlock), 0, ctx->stream, A, n, flag);
+    } else {
+      const float* A = (const float*)(uintptr_t)c.ptr[0];
+      if (nanc) hipLaunchKernelGGL((k_has<float, true>), dim3(g), dim3(kBlock), 0, ctx->stream, A, n, flag);
+      else hipLaunchKernelGGL((k_has<float, false>), dim3(g), dim3(kBlock), 0, ctx->stream, A, n, flag);
+    }
+  }
+  return gh_check_hip(ctx, hipGetLastError(), "hasNaN/hasInf launch");
+}

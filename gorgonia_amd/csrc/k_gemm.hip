@@ -1,0 +1,449 @@
+// fp32 MFMA contractions for gfx950: SGEMM / strided-batched GEMM and Conv2d
+// as implicit GEMM, plus GEMV and the outer product.
+//
+// Replaces cuBLAS Sgemm/Sgemv/Sger (cuda/linalg.go:102,223,282), the host loop
+// of per-slice Sgemm calls behind BatchedMatMul (operatorLinAlg.go:435-502) and
+// cuDNN ConvolutionForward (ops/nn/convolution_cuda.go:111-117).
+//
+// Tiling (one workgroup = 4 wavefronts of 64 lanes):
+//   block tile BM x BN, K step BK; LDS holds both operands k-major
+//   (As[k][m], Bs[k][n]) so that a v_mfma_f32_32x32x2f32 operand fetch is one
+//   conflict-free ds_read_b32 per lane (lane l reads [k0 + l/32][x0 + l%32]);
+//   each wavefront owns a (BM/2) x (BN/2) sub-tile = TM x TN MFMA tiles whose
+//   accumulators stay in registers for the whole K loop;
+//   global->register prefetch of tile k+1 overlaps the MFMAs on tile k, and
+//   LDS is double buffered so the loop needs one barrier per K step.
+//
+// Conv2d uses the same core with M = filters, N = B*oh*ow output pixels,
+// K = C*kh*kw: the "B" operand is gathered straight from the NCHW input (no
+// im2col buffer) and the result is written straight into NCHW (no transpose
+// pass), so lanes run along output pixels for coalesced loads and stores.
+#include <type_traits>
+
+#include "gh_internal.h"
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+
+// Epilogue activations in the reference's arithmetic form (nn.go:83-163).
+__device__ __forceinline__ float act_apply(float v, int act, float alpha) {
+  if (act == 1) return v * (v >= 0.0f ? 1.0f : 0.0f);
+  if (act == 2) {
+    const float pos = v * (v >= 0.0f ? 1.0f : 0.0f);
+    const float neg = v * (v < 0.0f ? 1.0f : 0.0f);
+    const float na = neg * alpha;
+    return pos + na;
+  }
+  return v;
+}
+
+// ---- operand loaders ---------------------------------------------------------
+// A loader moves one R x BK (or BK x R) operand tile: load() global->registers,
+// store() registers->LDS in k-major order with row stride S.
+
+// Operand stored [r][k] with k contiguous (A not transposed; B transposed).
+template <int R, int BK, bool VEC>
+struct LoadKContig {
+  static constexpr int S = R + 2;  // S % 32 == 2 keeps the transposing writes conflict-free
+  static constexpr int NV = (R * BK / 4) / kThreads;
+  const float* base; int ld; int rmax; int kmax;
+  f32x4 reg[NV];
+  __device__ __forceinline__ void load(int r0, int k0) {
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int f = threadIdx.x + j * kThreads;
+      const int r = r0 + f / (BK / 4);
+      const int k = k0 + (f % (BK / 4)) * 4;
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (r < rmax) {
+        const float* p = base + (int64_t)r * ld + k;
+        if (VEC) {
+          if (k < kmax) v = *reinterpret_cast<const f32x4*>(p);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) if (k + e < kmax) v[e] = p[e];
+        }
+      }
+      reg[j] = v;
+    }
+  }
+  __device__ __forceinline__ void store(float* lds) const {
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int f = threadIdx.x + j * kThreads;
+      const int r = f / (BK / 4);
+      const int kq = (f % (BK / 4)) * 4;
+#pragma unroll
+      for (int e = 0; e < 4; e++) lds[(kq + e) * S + r] = reg[j][e];
+    }
+  }
+};
+
+// Operand stored [k][c] with c contiguous (B not transposed; A transposed).
+template <int R, int BK, bool VEC>
+struct LoadMnContig {
+  static constexpr int S = R;
+  static constexpr int NV = (R * BK / 4) / kThreads;
+  const float* base; int ld; int rmax; int kmax;
+  f32x4 reg[NV];
+  __device__ __forceinline__ void load(int c0, int k0) {
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int f = threadIdx.x + j * kThreads;
+      const int k = k0 + f / (R / 4);
+      const int c = c0 + (f % (R / 4)) * 4;
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (k < kmax) {
+        const float* p = base + (int64_t)k * ld + c;
+        if (VEC) {
+          if (c < rmax) v = *reinterpret_cast<const f32x4*>(p);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) if (c + e < rmax) v[e] = p[e];
+        }
+      }
+      reg[j] = v;
+    }
+  }
+  __device__ __forceinline__ void store(float* lds) const {
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int f = threadIdx.x + j * kThreads;
+      const int k = f / (R / 4);
+      const int c = (f % (R / 4)) * 4;
+      *reinterpret_cast<f32x4*>(&lds[k * S + c]) = reg[j];
+    }
+  }
+};
+
+// im2col gather for Conv2d: logical operand [k][p], k = (c, kr, kc) in the
+// reference's order (op_nn.go:418-437), p = (b, oy, ox).  Each thread keeps
+// one output pixel for the whole kernel and walks k.  KH/KW > 0 are
+// compile-time kernel sizes; 0 means "use the runtime values".
+struct ConvGeom {
+  int C, H, W, oh, ow, kh, kw, padH, padW, strideH, strideW, dilH, dilW, P /* B*oh*ow */;
+};
+
+template <int R, int BK, int KH, int KW>
+struct LoadIm2col {
+  static constexpr int S = R;
+  static constexpr int KPT = BK / (kThreads / R);  // k values per thread per tile
+  const float* x; ConvGeom g; int kmax;
+  int pix_ok; int iy0, ix0; const float* xb;
+  float reg[KPT];
+  __device__ __forceinline__ void init(int p0) {
+    const int p = p0 + (threadIdx.x % R);
+    pix_ok = p < g.P;
+    const int pp = pix_ok ? p : 0;
+    const int b = pp / (g.oh * g.ow);
+    const int rem = pp - b * (g.oh * g.ow);
+    const int oy = rem / g.ow, ox = rem - oy * g.ow;
+    iy0 = oy * g.strideH - g.padH;
+    ix0 = ox * g.strideW - g.padW;
+    xb = x + (int64_t)b * g.C * g.H * g.W;
+  }
+  __device__ __forceinline__ void load(int /*p0*/, int k0) {
+    const int kh = KH ? KH : g.kh, kw = KW ? KW : g.kw;
+    const int kb = threadIdx.x / R;
+#pragma unroll
+    for (int j = 0; j < KPT; j++) {
+      const int k = k0 + kb + j * (kThreads / R);
+      float v = 0.f;
+      if (pix_ok && k < kmax) {
+        const int c = k / (kh * kw);
+        const int r = k - c * (kh * kw);
+        const int kr = r / kw, kc = r - kr * kw;
+        const int iy = iy0 + kr * g.dilH, ix = ix0 + kc * g.dilW;
+        if (iy >= 0 && iy < g.H && ix >= 0 && ix < g.W) v = xb[((int64_t)c * g.H + iy) * g.W + ix];
+      }
+      reg[j] = v;
+    }
+  }
+  __device__ __forceinline__ void store(float* lds) const {
+    const int kb = threadIdx.x / R, pl = threadIdx.x % R;
+#pragma unroll
+    for (int j = 0; j < KPT; j++) lds[(kb + j * (kThreads / R)) * S + pl] = reg[j];
+  }
+};
+
+// ---- result writers ------------------------------------------------------------
+struct StoreRowMajor {
+  float* C; int ldc;
+  __device__ __forceinline__ void put(int i, int j, float v) const { C[(int64_t)i * ldc + j] = v; }
+};
+
+// Conv result: row i = filter, column j = output pixel (b, oy, ox) -> NCHW.
+struct StoreNCHW {
+  float* y; int F; int plane /* oh*ow */;
+  __device__ __forceinline__ void put(int i, int j, float v) const {
+    const int b = j / plane, p = j - b * plane;
+    y[((int64_t)b * F + i) * plane + p] = v;
+  }
+};
+
+// ---- the MFMA core ---------------------------------------------------------------
+template <int BM, int BN, int BK, class LA, class LB, class SC>
+__device__ __forceinline__ void mfma_tile_loop(LA& la, LB& lb, const SC& sc, int M, int N, int K,
+                                               int m0, int n0, int act, float alpha) {
+  constexpr int WM = BM / 2, WN = BN / 2;      // 2 x 2 wavefronts
+  constexpr int TM = WM / 32, TN = WN / 32;    // MFMA tiles per wavefront
+  constexpr int SA = LA::S, SB = LB::S;
+  __shared__ float lds[2 * BK * (SA + SB)];
+  float* const As = lds;                 // two buffers of BK * SA floats
+  float* const Bs = lds + 2 * BK * SA;   // two buffers of BK * SB floats
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+  const int lr = lane & 31, lk = lane >> 5;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int a = 0; a < TM; a++)
+#pragma unroll
+    for (int b = 0; b < TN; b++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
+
+  const int nk = (K + BK - 1) / BK;
+  la.load(m0, 0);
+  lb.load(n0, 0);
+  la.store(As);
+  lb.store(Bs);
+  __syncthreads();
+
+  for (int kt = 0; kt < nk; kt++) {
+    const int cur = kt & 1;
+    const bool more = kt + 1 < nk;
+    if (more) {
+      la.load(m0, (kt + 1) * BK);
+      lb.load(n0, (kt + 1) * BK);
+    }
+    const float* a_s = As + cur * (BK * SA) + wm + lr;
+    const float* b_s = Bs + cur * (BK * SB) + wn + lr;
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      float af[TM], bf[TN];
+#pragma unroll
+      for (int a = 0; a < TM; a++) af[a] = a_s[(kk + lk) * SA + a * 32];
+#pragma unroll
+      for (int b = 0; b < TN; b++) bf[b] = b_s[(kk + lk) * SB + b * 32];
+#pragma unroll
+      for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int b = 0; b < TN; b++)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[a], bf[b], acc[a][b], 0, 0, 0);
+    }
+    if (more) {
+      la.store(As + (cur ^ 1) * (BK * SA));
+      lb.store(Bs + (cur ^ 1) * (BK * SB));
+    }
+    __syncthreads();
+  }
+
+  // Accumulator layout of v_mfma_f32_32x32x2f32: lane l holds column l%32 and,
+  // in register v, row 8*(v/4) + 4*(l/32) + v%4.
+#pragma unroll
+  for (int a = 0; a < TM; a++)
+#pragma unroll
+    for (int b = 0; b < TN; b++) {
+      const int j = n0 + wn + b * 32 + lr;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int i = m0 + wm + a * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+        if (i < M && j < N) sc.put(i, j, act_apply(acc[a][b][v], act, alpha));
+      }
+    }
+}
+
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC>
+__global__ __launch_bounds__(kThreads) void k_sgemm(const float* __restrict__ A,
+                                                    const float* __restrict__ B,
+                                                    float* __restrict__ C, int M, int N, int K,
+                                                    int lda, int ldb, int ldc, int64_t sA,
+                                                    int64_t sB, int64_t sC, int act, float alpha) {
+  using LA = typename std::conditional<TA, LoadMnContig<BM, BK, VEC>, LoadKContig<BM, BK, VEC>>::type;
+  using LB = typename std::conditional<TB, LoadKContig<BN, BK, VEC>, LoadMnContig<BN, BK, VEC>>::type;
+  const int bz = blockIdx.z;
+  LA la; la.base = A + bz * sA; la.ld = lda; la.rmax = M; la.kmax = K;
+  LB lb; lb.base = B + bz * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
+  StoreRowMajor sc{C + bz * sC, ldc};
+  mfma_tile_loop<BM, BN, BK, LA, LB, StoreRowMajor>(la, lb, sc, M, N, K, blockIdx.y * BM,
+                                                    blockIdx.x * BN, act, alpha);
+}
+
+template <int BM, int BN, int BK, int KH, int KW, bool VEC>
+__global__ __launch_bounds__(kThreads) void k_conv2d(const float* __restrict__ x,
+                                                     const float* __restrict__ w,
+                                                     float* __restrict__ y, ConvGeom g, int F, int K,
+                                                     int act, float alpha) {
+  using LA = LoadKContig<BM, BK, VEC>;
+  using LB = LoadIm2col<BN, BK, KH, KW>;
+  LA la; la.base = w; la.ld = K; la.rmax = F; la.kmax = K;
+  LB lb; lb.x = x; lb.g = g; lb.kmax = K;
+  const int n0 = blockIdx.x * BN;
+  lb.init(n0);
+  StoreNCHW sc{y, F, g.oh * g.ow};
+  mfma_tile_loop<BM, BN, BK, LA, LB, StoreNCHW>(la, lb, sc, F, g.P, K, blockIdx.y * BM, n0, act, alpha);
+}
+
+// ---- GEMV / outer ------------------------------------------------------------------
+// y(m) = A(m x n) x: one wavefront per row, float4 loads when the row is
+// 16-byte aligned, butterfly reduction across the 64 lanes.
+__global__ __launch_bounds__(256) void k_gemv_n(const float* __restrict__ A,
+                                                const float* __restrict__ x, float* __restrict__ y,
+                                                int m, int n, int lda, int vec) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= m) return;
+  const float* a = A + (int64_t)row * lda;
+  float acc = 0.f;
+  if (vec) {
+    const f32x4* av = reinterpret_cast<const f32x4*>(a);
+    const f32x4* xv = reinterpret_cast<const f32x4*>(x);
+    const int nv = n / 4;
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    for (int i = lane; i < nv; i += 64) {
+      const f32x4 p = __builtin_nontemporal_load(&av[i]) * xv[i];
+      s += p;
+    }
+    acc = (s[0] + s[1]) + (s[2] + s[3]);
+    for (int i = nv * 4 + lane; i < n; i += 64) acc += a[i] * x[i];
+  } else {
+    for (int i = lane; i < n; i += 64) acc += a[i] * x[i];
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (lane == 0) y[row] = acc;
+}
+
+// y(n) = A(m x n)^T x: each thread owns one column, walks rows; consecutive
+// lanes read consecutive addresses.
+__global__ __launch_bounds__(256) void k_gemv_t(const float* __restrict__ A,
+                                                const float* __restrict__ x, float* __restrict__ y,
+                                                int m, int n, int lda) {
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  if (col >= n) return;
+  float acc = 0.f;
+  for (int r = 0; r < m; r++) acc += A[(int64_t)r * lda + col] * x[r];
+  y[col] = acc;
+}
+
+__global__ __launch_bounds__(256) void k_outer(const float* __restrict__ x,
+                                               const float* __restrict__ y, float* __restrict__ A,
+                                               int64_t m, int64_t n) {
+  const int64_t total = m * n, stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride)
+    A[i] = x[i / n] * y[i % n];
+}
+
+inline bool al16(uint64_t p) { return (p & 15u) == 0; }
+
+template <int BM, int BN, int BK>
+int launch_sgemm_cfg(gh_ctx* ctx, const gh_cmd& c) {
+  const int M = (int)c.dim[0], N = (int)c.dim[1], K = (int)c.dim[2];
+  const int lda = (int)c.dim[3], ldb = (int)c.dim[4], ldc = (int)c.dim[5];
+  const int batch = c.dim[6] <= 0 ? 1 : (int)c.dim[6];
+  const bool ta = c.flags & GH_FLAG_TRANS_A, tb = c.flags & GH_FLAG_TRANS_B;
+  const float* A = (const float*)(uintptr_t)c.ptr[0];
+  const float* B = (const float*)(uintptr_t)c.ptr[1];
+  float* C = (float*)(uintptr_t)c.ptr[2];
+  const int64_t sA = batch > 1 ? c.dim[7] : 0, sB = batch > 1 ? c.dim[8] : 0, sC = batch > 1 ? c.dim[9] : 0;
+  // 16-byte vector loads need aligned bases, leading dimensions and batch
+  // strides, and a contiguous extent that is a multiple of four.
+  const bool vec = al16(c.ptr[0]) && al16(c.ptr[1]) && lda % 4 == 0 && ldb % 4 == 0 &&
+                   sA % 4 == 0 && sB % 4 == 0 && (ta ? M % 4 == 0 : K % 4 == 0) &&
+                   (tb ? K % 4 == 0 : N % 4 == 0);
+  const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
+  const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, batch);
+#define GH_GEMM_LAUNCH(TA_, TB_, V_)                                                              \
+  hipLaunchKernelGGL((k_sgemm<BM, BN, BK, TA_, TB_, V_>), grid, dim3(kThreads), 0, ctx->stream, A, B, \
+                     C, M, N, K, lda, ldb, ldc, sA, sB, sC, act, c.f[0])
+  if (vec) {
+    if (!ta && !tb) GH_GEMM_LAUNCH(false, false, true);
+    else if (!ta && tb) GH_GEMM_LAUNCH(false, true, true);
+    else if (ta && !tb) GH_GEMM_LAUNCH(true, false, true);
+    else GH_GEMM_LAUNCH(true, true, true);
+  } else {
+    if (!ta && !tb) GH_GEMM_LAUNCH(false, false, false);
+    else if (!ta && tb) GH_GEMM_LAUNCH(false, true, false);
+    else if (ta && !tb) GH_GEMM_LAUNCH(true, false, false);
+    else GH_GEMM_LAUNCH(true, true, false);
+  }
+#undef GH_GEMM_LAUNCH
+  return gh_check_hip(ctx, hipGetLastError(), "sgemm launch");
+}
+
+template <int BM, int BN, int BK, int KH, int KW>
+int launch_conv_cfg(gh_ctx* ctx, const gh_cmd& c, const ConvGeom& g, int F, int K) {
+  const bool vec = al16(c.ptr[1]) && K % 4 == 0;
+  const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
+  const dim3 grid((g.P + BN - 1) / BN, (F + BM - 1) / BM, 1);
+  const float* x = (const float*)(uintptr_t)c.ptr[0];
+  const float* w = (const float*)(uintptr_t)c.ptr[1];
+  float* y = (float*)(uintptr_t)c.ptr[2];
+  if (vec)
+    hipLaunchKernelGGL((k_conv2d<BM, BN, BK, KH, KW, true>), grid, dim3(kThreads), 0, ctx->stream, x, w,
+                       y, g, F, K, act, c.f[0]);
+  else
+    hipLaunchKernelGGL((k_conv2d<BM, BN, BK, KH, KW, false>), grid, dim3(kThreads), 0, ctx->stream, x,
+                       w, y, g, F, K, act, c.f[0]);
+  return gh_check_hip(ctx, hipGetLastError(), "conv2d launch");
+}
+
+template <int BM, int BN, int BK>
+int launch_conv_k(gh_ctx* ctx, const gh_cmd& c, const ConvGeom& g, int F, int K) {
+  if (g.kh == 3 && g.kw == 3) return launch_conv_cfg<BM, BN, BK, 3, 3>(ctx, c, g, F, K);
+  if (g.kh == 1 && g.kw == 1) return launch_conv_cfg<BM, BN, BK, 1, 1>(ctx, c, g, F, K);
+  return launch_conv_cfg<BM, BN, BK, 0, 0>(ctx, c, g, F, K);
+}
+
+}  // namespace
+
+int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t M = c.dim[0];
+  if (M <= 64) return launch_sgemm_cfg<64, 128, 16>(ctx, c);
+  return launch_sgemm_cfg<128, 128, 16>(ctx, c);
+}
+
+int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
+  ConvGeom g;
+  g.C = (int)c.dim[1]; g.H = (int)c.dim[2]; g.W = (int)c.dim[3];
+  g.kh = (int)c.dim[5]; g.kw = (int)c.dim[6];
+  g.padH = (int)c.dim[7]; g.padW = (int)c.dim[8];
+  g.strideH = (int)c.dim[9]; g.strideW = (int)c.dim[10];
+  g.dilH = (int)c.dim[11]; g.dilW = (int)c.dim[12];
+  g.oh = (int)gh_conv_out(g.H, g.kh, g.padH, g.strideH, g.dilH);
+  g.ow = (int)gh_conv_out(g.W, g.kw, g.padW, g.strideW, g.dilW);
+  g.P = (int)c.dim[0] * g.oh * g.ow;
+  const int F = (int)c.dim[4], K = g.C * g.kh * g.kw;
+  if (F <= 64) return launch_conv_k<64, 128, 16>(ctx, c, g, F, K);
+  return launch_conv_k<128, 128, 16>(ctx, c, g, F, K);
+}
+
+int gh_launch_gemv(gh_ctx* ctx, const gh_cmd& c) {
+  const int m = (int)c.dim[0], n = (int)c.dim[1], lda = (int)c.dim[2];
+  const float* A = (const float*)(uintptr_t)c.ptr[0];
+  const float* x = (const float*)(uintptr_t)c.ptr[1];
+  float* y = (float*)(uintptr_t)c.ptr[2];
+  if (c.flags & GH_FLAG_TRANS_A) {
+    hipLaunchKernelGGL(k_gemv_t, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, A, x, y, m, n, lda);
+  } else {
+    const int vec = al16(c.ptr[0]) && al16(c.ptr[1]) && lda % 4 == 0;
+    hipLaunchKernelGGL(k_gemv_n, dim3((m + 3) / 4), dim3(256), 0, ctx->stream, A, x, y, m, n, lda, vec);
+  }
+  return gh_check_hip(ctx, hipGetLastError(), "gemv launch");
+}
+
+int gh_launch_outer(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t m = c.dim[0], n = c.dim[1];
+  int64_t blocks = (m * n + 1023) / 1024;
+  if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
+  hipLaunchKernelGGL(k_outer, dim3((int)blocks), dim3(256), 0, ctx->stream,
+                     (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                     (float*)(uintptr_t)c.ptr[2], m, n);
+  return gh_check_hip(ctx, hipGetLastError(), "outer launch");
+}

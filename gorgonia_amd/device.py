@@ -1,0 +1,224 @@
+"""Thin Python view of the device C ABI: a context, raw device buffers and
+command builders.  Used by the tests, the benchmark and the Python mirror of
+the engine; it adds no numerics of its own - every result comes from the HIP
+library."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _ffi
+from ._ffi import GhCmd
+
+
+class DeviceError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"{_ffi.ERR_NAMES.get(code, code)}: {msg}")
+        self.code = code
+
+
+def make_cmd(opcode, flags=0, ptrs=(), dims=(), f=()):
+    c = GhCmd()
+    c.opcode = opcode
+    c.flags = flags
+    for i, p in enumerate(ptrs):
+        c.ptr[i] = int(p)
+    for i, d in enumerate(dims):
+        c.dim[i] = int(d)
+    for i, v in enumerate(f):
+        c.f[i] = float(v)
+    return c
+
+
+class Context:
+    """One gh_ctx: a device, its stream and (optionally) an arena reservation."""
+
+    def __init__(self, device=0, arena_bytes=0):
+        self.lib = _ffi.load()
+        h = C.c_void_p()
+        rc = self.lib.gh_init(device, arena_bytes, C.byref(h))
+        if rc != 0:
+            raise DeviceError(rc, f"gh_init(device={device}, arena_bytes={arena_bytes}) failed")
+        self.h = h
+        self._owned = []
+
+    # -- lifetime -----------------------------------------------------------
+    def close(self):
+        if self.h:
+            self.lib.gh_close(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    # -- errors ---------------------------------------------------------------
+    def check(self, rc):
+        if rc != 0:
+            buf = C.create_string_buffer(512)
+            self.lib.gh_last_error(self.h, buf, 512)
+            raise DeviceError(rc, buf.value.decode(errors="replace"))
+
+    def clear_error(self):
+        self.lib.gh_clear_error(self.h)
+
+    def info(self):
+        d = _ffi.GhDevInfo()
+        self.check(self.lib.gh_device_info(self.h, C.byref(d)))
+        return d
+
+    # -- memory -----------------------------------------------------------------
+    def malloc(self, nbytes):
+        p = C.c_uint64()
+        self.check(self.lib.gh_malloc(self.h, max(int(nbytes), 1), C.byref(p)))
+        return p.value
+
+    def free(self, ptr):
+        self.check(self.lib.gh_free(self.h, ptr))
+
+    def arena(self):
+        return self.lib.gh_arena_base(self.h), self.lib.gh_arena_size(self.h)
+
+    def h2d(self, dptr, arr):
+        arr = np.ascontiguousarray(arr)
+        self.check(self.lib.gh_memcpy_h2d(self.h, dptr, arr.ctypes.data_as(C.c_void_p), arr.nbytes))
+        self.sync()  # pageable numpy memory: do not return before the copy is done
+
+    def d2h(self, dptr, shape, dtype=np.float32):
+        out = np.empty(shape, dtype=dtype)
+        self.check(self.lib.gh_memcpy_d2h(self.h, out.ctypes.data_as(C.c_void_p), dptr, out.nbytes))
+        self.sync()
+        return out
+
+    def upload(self, arr):
+        """Allocate a device buffer holding `arr`; returns its address."""
+        arr = np.ascontiguousarray(arr)
+        p = self.malloc(arr.nbytes)
+        if arr.nbytes:
+            self.h2d(p, arr)
+        return p
+
+    # -- work ---------------------------------------------------------------------
+    def submit(self, cmds):
+        if isinstance(cmds, GhCmd):
+            cmds = [cmds]
+        n = len(cmds)
+        arr = (GhCmd * n)(*cmds)
+        self.check(self.lib.gh_submit(self.h, arr, n))
+
+    def sync(self):
+        self.check(self.lib.gh_sync(self.h))
+
+    def run(self, cmds):
+        self.submit(cmds)
+        self.sync()
+
+    def event(self, slot):
+        self.check(self.lib.gh_event_record(self.h, slot))
+
+    def elapsed_ms(self, a, b):
+        ms = C.c_float()
+        self.check(self.lib.gh_event_elapsed_ms(self.h, a, b, C.byref(ms)))
+        return ms.value
+
+    # -- graphs ---------------------------------------------------------------------
+    def graph_begin(self):
+        self.check(self.lib.gh_graph_begin(self.h))
+
+    def graph_end(self):
+        gid = C.c_int()
+        self.check(self.lib.gh_graph_end(self.h, C.byref(gid)))
+        return gid.value
+
+    def graph_launch(self, gid):
+        self.check(self.lib.gh_graph_launch(self.h, gid))
+
+    def graph_destroy(self, gid):
+        self.check(self.lib.gh_graph_destroy(self.h, gid))
+
+
+# ---- command builders -------------------------------------------------------------
+
+def cmd_bin(fn, mode, a, b, n, dtype=_ffi.F32):
+    fl = _ffi.flag_fn(_ffi.BIN_FN[fn]) | _ffi.flag_mode(_ffi.MODE[mode]) | _ffi.flag_dtype(dtype)
+    return make_cmd(_ffi.OP_ELEM_BIN, fl, (a, b), (n,))
+
+
+def cmd_unary(fn, a, n, dtype=_ffi.F32):
+    fl = _ffi.flag_fn(_ffi.UNARY_FN[fn]) | _ffi.flag_dtype(dtype)
+    return make_cmd(_ffi.OP_ELEM_UNARY, fl, (a,), (n,))
+
+
+def cmd_bcast(fn, dst, big, small, outer, mid, inner, small_left=False):
+    fl = _ffi.flag_fn(_ffi.BIN_FN[fn]) | (_ffi.FLAG_SMALL_LEFT if small_left else 0)
+    return make_cmd(_ffi.OP_BCAST_BIN, fl, (dst, big, small), (outer, mid, inner))
+
+
+def cmd_copy(dst, src, nbytes):
+    return make_cmd(_ffi.OP_MEMCPY_D2D, 0, (dst, src), (nbytes,))
+
+
+def cmd_gemm(a, b, c, m, n, k, lda=None, ldb=None, ldc=None, trans_a=False, trans_b=False,
+             batch=1, stride_a=0, stride_b=0, stride_c=0, act=None, alpha=0.0):
+    lda = lda if lda is not None else (m if trans_a else k)
+    ldb = ldb if ldb is not None else (k if trans_b else n)
+    ldc = ldc if ldc is not None else n
+    fl = (_ffi.FLAG_TRANS_A if trans_a else 0) | (_ffi.FLAG_TRANS_B if trans_b else 0)
+    fl |= {None: 0, "relu": _ffi.FLAG_ACT_RELU, "leaky": _ffi.FLAG_ACT_LEAKY}[act]
+    return make_cmd(_ffi.OP_GEMM, fl, (a, b, c), (m, n, k, lda, ldb, ldc, batch, stride_a, stride_b,
+                                                  stride_c), (alpha,))
+
+
+def cmd_gemv(a, x, y, m, n, lda=None, trans=False):
+    return make_cmd(_ffi.OP_GEMV, _ffi.FLAG_TRANS_A if trans else 0, (a, x, y),
+                    (m, n, lda if lda is not None else n))
+
+
+def cmd_outer(x, y, a, m, n):
+    return make_cmd(_ffi.OP_OUTER, 0, (x, y, a), (m, n))
+
+
+def cmd_conv2d(x, w, y, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dilation=(1, 1),
+               act=None, alpha=0.0):
+    fl = {None: 0, "relu": _ffi.FLAG_ACT_RELU, "leaky": _ffi.FLAG_ACT_LEAKY}[act]
+    return make_cmd(_ffi.OP_CONV2D, fl, (x, w, y),
+                    (B, Cin, H, W, F, kh, kw, pad[0], pad[1], stride[0], stride[1], dilation[0],
+                     dilation[1]), (alpha,))
+
+
+def cmd_maxpool2d(x, y, B, Cn, H, W, kh, kw, pad, stride):
+    """pad: 2 values (symmetric H, W) or 4 values (north, south, west, east) as in MaxPool2D."""
+    if len(pad) == 4:
+        p4, fl = tuple(pad), _ffi.FLAG_EXPLICIT_PAD
+    else:
+        p4, fl = (pad[0], pad[0], pad[1], pad[1]), 0
+    return make_cmd(_ffi.OP_MAXPOOL2D, fl, (x, y), (B, Cn, H, W, kh, kw) + p4 + tuple(stride))
+
+
+def cmd_bn_infer(x, y, mean, var, B, Cn, S, eps, gamma=0, beta=0):
+    fl = (_ffi.FLAG_HAS_GAMMA if gamma else 0) | (_ffi.FLAG_HAS_BETA if beta else 0)
+    return make_cmd(_ffi.OP_BN_INFER, fl, (x, y, mean, var, gamma, beta), (B, Cn, S), (eps,))
+
+
+def cmd_relu(x, y, n):
+    return make_cmd(_ffi.OP_RELU, 0, (x, y), (n,))
+
+
+def cmd_leaky_relu(x, y, n, alpha):
+    return make_cmd(_ffi.OP_LEAKY_RELU, 0, (x, y), (n,), (alpha,))
+
+
+def cmd_softmax(x, y, rows, cols):
+    return make_cmd(_ffi.OP_SOFTMAX, 0, (x, y), (rows, cols))
+
+
+def cmd_has(kind, a, flag, n, dtype=_ffi.F32):
+    op = _ffi.OP_HAS_NAN if kind == "nan" else _ffi.OP_HAS_INF
+    return make_cmd(op, _ffi.flag_dtype(dtype), (a, flag), (n,))
+
+
+def cmd_fill(a, n, value):
+    return make_cmd(_ffi.OP_FILL, 0, (a,), (n,), (value,))

@@ -1,0 +1,238 @@
+/*
+ * gorgonia_hip.h - C ABI of libgorgonia_hip.so, the gfx950 device engine that
+ * sits where Gorgonia's cuda/ package calls into gorgonia.org/cu, cuBLAS and
+ * cuDNN.
+ *
+ * The calling model follows Gorgonia's own "fill a command array in Go, drain
+ * it in one cgo call" precedent (blase/work.h:144-168): the host records one
+ * gh_cmd per operator while the tape machine walks a segment, and hands the
+ * whole array to gh_submit() when it reaches a flush point.  One cgo crossing
+ * per tape segment instead of one per operator.
+ *
+ * Conventions
+ *   - every entry point returns 0 on success, a GH_E* code otherwise;
+ *   - device errors are sticky per context (cuda/external.go:223-226,251-257):
+ *     once a call fails, later gh_submit()/gh_sync() calls return the same
+ *     code until gh_clear_error(); gh_last_error() returns the message;
+ *   - a context is used from one thread at a time (cuda/external.go:237);
+ *   - all work is stream-ordered on the context's single stream; results are
+ *     only guaranteed after gh_sync() (enqueue-then-flush, vm_tape.go:735-745);
+ *   - device addresses are plain uint64_t (tensor.Memory.Uintptr()).
+ */
+#ifndef GORGONIA_HIP_H
+#define GORGONIA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Exported from the shared library (everything else is built hidden). */
+#if defined(__GNUC__)
+#define GH_API __attribute__((visibility("default")))
+#else
+#define GH_API
+#endif
+
+typedef struct gh_ctx gh_ctx;
+typedef uint64_t gh_devptr;
+
+enum {
+  GH_OK = 0,
+  GH_EINVAL = 1,     /* bad argument / shape / opcode (cuda/utils.go:58-112) */
+  GH_EDEVICE = 2,    /* HIP runtime error (sticky) */
+  GH_EOOM = 3,       /* arena reservation failed (cuda/external.go:158-166) */
+  GH_ENOFUNC = 4,    /* no such kernel (cuda/arith.go:17-19) */
+  GH_ESTATE = 5      /* call not valid in the current state */
+};
+
+/* Device limits; replaces the attribute query at cuda/external.go:135-146. */
+typedef struct gh_devinfo {
+  int32_t wavefront_size;
+  int32_t max_threads_per_block;
+  int32_t max_grid_x, max_grid_y, max_grid_z;
+  int32_t max_block_x, max_block_y, max_block_z;
+  int32_t compute_units;
+  int32_t lds_bytes_per_block;
+  int64_t free_mem, total_mem;
+  char    arch[32];
+} gh_devinfo;
+
+/* ---- operator command -------------------------------------------------- */
+
+enum gh_opcode {
+  GH_OP_NOP = 0,
+  GH_OP_ELEM_BIN = 1,   /* elembinop.<fn>_{vv,vs,sv,ss}_f{32,64}              */
+  GH_OP_ELEM_UNARY = 2, /* elemunaryop.<fn>_f{32,64}                          */
+  GH_OP_BCAST_BIN = 3,  /* Broadcast{Add,Sub,HadamardProd,...}: fused repeat  */
+  GH_OP_MEMCPY_D2D = 4, /* Engine.memcpy (cuda/engine.go:129-131)             */
+  GH_OP_GEMM = 5,       /* Engine.MatMul / BatchedMatMul (cuda/linalg.go:110) */
+  GH_OP_GEMV = 6,       /* Engine.MatVecMul (cuda/linalg.go:47)               */
+  GH_OP_OUTER = 7,      /* Engine.Outer (cuda/linalg.go:232)                  */
+  GH_OP_CONV2D = 8,     /* ops/nn/convolution_cuda.go:95-121                  */
+  GH_OP_MAXPOOL2D = 9,  /* ops/nn/maxpool_cuda.go:94-111                      */
+  GH_OP_BN_INFER = 10,  /* ops/nn/batchnorm_cuda.go:101-111 (CPU semantics)   */
+  GH_OP_RELU = 11,      /* ops/nn/activation_cuda.go:72-94; nn.go:136-163     */
+  GH_OP_LEAKY_RELU = 12,/* nn.go:83-131                                       */
+  GH_OP_SOFTMAX = 13,   /* op_softmax.go:99-128                               */
+  GH_OP_HAS_NAN = 14,   /* misc.hasNaN (cuda/engine.go:144-166)               */
+  GH_OP_HAS_INF = 15,   /* misc.hasInf (cuda/engine.go:169-191)               */
+  GH_OP_FILL = 16,      /* Memset of a float value                            */
+  GH_OP__COUNT
+};
+
+/* flags for GH_OP_ELEM_BIN / GH_OP_BCAST_BIN: fn | mode<<8 | dtype<<12 | ... */
+enum gh_binfn {
+  GH_ADD = 0, GH_SUB = 1, GH_MUL = 2, GH_DIV = 3, GH_POW = 4,
+  GH_LT = 5, GH_LTE = 6, GH_GT = 7, GH_GTE = 8, GH_EQ = 9, GH_NE = 10,
+  GH_BINFN__COUNT
+};
+enum gh_binmode { GH_VV = 0, GH_VS = 1, GH_SV = 2, GH_SS = 3 };
+enum gh_dtype { GH_F32 = 0, GH_F64 = 1 };
+
+/* flags for GH_OP_ELEM_UNARY: fn | dtype<<12 */
+enum gh_unaryfn {
+  GH_ABS = 0, GH_SIGN = 1, GH_CEIL = 2, GH_FLOOR = 3, GH_SIN = 4, GH_COS = 5,
+  GH_EXP = 6, GH_LN = 7, GH_LOG2 = 8, GH_NEG = 9, GH_SQUARE = 10, GH_SQRT = 11,
+  GH_INVERSE = 12, GH_INVSQRT = 13, GH_CUBE = 14, GH_TANH = 15, GH_SIGMOID = 16,
+  GH_LOG1P = 17, GH_EXPM1 = 18, GH_SOFTPLUS = 19,
+  GH_UNARYFN__COUNT
+};
+
+#define GH_FLAG_FN(f)        ((uint32_t)(f) & 0xffu)
+#define GH_FLAG_MODE(m)      (((uint32_t)(m) & 0xfu) << 8)
+#define GH_FLAG_DTYPE(d)     (((uint32_t)(d) & 0xfu) << 12)
+#define GH_FLAG_TRANS_A      (1u << 16)   /* GEMM/GEMV: logical transpose of A */
+#define GH_FLAG_TRANS_B      (1u << 17)   /* GEMM: logical transpose of B      */
+#define GH_FLAG_SMALL_LEFT   (1u << 18)   /* BCAST_BIN: small operand on left  */
+#define GH_FLAG_EXPLICIT_PAD (1u << 19)   /* MAXPOOL2D: 4-value padding given  */
+#define GH_FLAG_HAS_GAMMA    (1u << 20)   /* BN_INFER: ptr[4] = gamma          */
+#define GH_FLAG_HAS_BETA     (1u << 21)   /* BN_INFER: ptr[5] = beta           */
+#define GH_FLAG_ACT_RELU     (1u << 22)   /* CONV2D/GEMM epilogue: x*(x>=0)    */
+#define GH_FLAG_ACT_LEAKY    (1u << 23)   /* epilogue: leaky relu, alpha=f[0]  */
+
+/*
+ * One operator.  Field use per opcode:
+ *
+ * ELEM_BIN    ptr[0]=A ptr[1]=B            dim[0]=n
+ *             vv/vs/ss write A, sv writes B (elembinop.cu:13-35)
+ * ELEM_UNARY  ptr[0]=A (in place)          dim[0]=n
+ * BCAST_BIN   ptr[0]=dst ptr[1]=big ptr[2]=small
+ *             dim[0]=outer dim[1]=mid dim[2]=inner; small has `mid` elements,
+ *             element (o,m,i) pairs big[o,m,i] with small[m]
+ * MEMCPY_D2D  ptr[0]=dst ptr[1]=src        dim[0]=bytes
+ * GEMM        ptr[0]=A ptr[1]=B ptr[2]=C   dim[0..2]=m,n,k  dim[3..5]=lda,ldb,ldc
+ *             dim[6]=batch (0/1 = single)  dim[7..9]=strideA,strideB,strideC
+ *             row-major; C(m x n) = op(A)(m x k) * op(B)(k x n)
+ * GEMV        ptr[0]=A ptr[1]=x ptr[2]=y   dim[0..2]=m,n,lda ; A is (m x n) row-major,
+ *             y(m)=A x, or with TRANS_A y(n)=A^T x
+ * OUTER       ptr[0]=x ptr[1]=y ptr[2]=A   dim[0..1]=m,n ; A(m x n) = x y^T
+ * CONV2D      ptr[0]=x ptr[1]=w ptr[2]=y   dim[0..3]=B,C,H,W dim[4]=F dim[5..6]=kh,kw
+ *             dim[7..8]=padH,padW dim[9..10]=strideH,strideW dim[11..12]=dilH,dilW
+ * MAXPOOL2D   ptr[0]=x ptr[1]=y            dim[0..3]=B,C,H,W dim[4..5]=kh,kw
+ *             dim[6..9]=padN,padS,padW,padE dim[10..11]=strideH,strideW
+ * BN_INFER    ptr[0]=x ptr[1]=y ptr[2]=mean ptr[3]=var [ptr[4]=gamma ptr[5]=beta]
+ *             dim[0..2]=B,C,S  f[0]=eps
+ * RELU        ptr[0]=x ptr[1]=y            dim[0]=n
+ * LEAKY_RELU  ptr[0]=x ptr[1]=y            dim[0]=n f[0]=alpha
+ * SOFTMAX     ptr[0]=x ptr[1]=y            dim[0]=rows dim[1]=cols
+ * HAS_NAN/INF ptr[0]=A ptr[1]=int32 flag (device)  dim[0]=n ; flag is set to 1
+ *             if any element matches, else 0
+ * FILL        ptr[0]=A                     dim[0]=n f[0]=value
+ */
+typedef struct gh_cmd {
+  uint32_t opcode;
+  uint32_t flags;
+  uint64_t ptr[6];
+  int64_t  dim[16];
+  float    f[4];
+} gh_cmd;
+
+/* ---- context / device -------------------------------------------------- */
+
+/* Engine.Init/doInit (cuda/external.go:88-170): make the device current,
+ * create the stream, reserve `arena_bytes` of device memory in one hipMalloc
+ * (arena_bytes may be 0: no reservation). */
+GH_API int gh_init(int device, int64_t arena_bytes, gh_ctx** out);
+/* Engine.Close (cuda/external.go:173-220). */
+GH_API int gh_close(gh_ctx* ctx);
+/* Device attribute query (cuda/external.go:135-146, cu.MemInfo :153). */
+GH_API int gh_device_info(gh_ctx* ctx, gh_devinfo* out);
+/* Number of visible devices; does not create a context. */
+GH_API int gh_device_count(int* out);
+
+/* Base and size of the reservation handed to the host-side BFC arena
+ * (bfc.reserve, cuda/external.go:166). */
+GH_API gh_devptr gh_arena_base(gh_ctx* ctx);
+GH_API int64_t gh_arena_size(gh_ctx* ctx);
+
+/* Stand-alone device allocations outside the arena (cu.MemAlloc). */
+GH_API int gh_malloc(gh_ctx* ctx, int64_t bytes, gh_devptr* out);
+GH_API int gh_free(gh_ctx* ctx, gh_devptr p);
+
+/* Pinned host staging memory for H2D/D2H (the reference relies on managed
+ * memory, cuda/external.go:162; explicit copies need a pinned source to be
+ * asynchronous). */
+GH_API int gh_host_alloc(gh_ctx* ctx, int64_t bytes, void** out);
+GH_API int gh_host_free(gh_ctx* ctx, void* p);
+
+/* Queued copies: cuda.go:141,186,199 and vm_tape_cuda.go:220-243
+ * (MemcpyHtoD / MemcpyDtoH), cuda/engine.go:103-127 (Memcpy D2D).  Stream
+ * ordered; the host buffer must stay valid until the next gh_sync(). */
+GH_API int gh_memcpy_h2d(gh_ctx* ctx, gh_devptr dst, const void* src, int64_t bytes);
+GH_API int gh_memcpy_d2h(gh_ctx* ctx, void* dst, gh_devptr src, int64_t bytes);
+GH_API int gh_memcpy_d2d(gh_ctx* ctx, gh_devptr dst, gh_devptr src, int64_t bytes);
+
+/* ---- work submission --------------------------------------------------- */
+
+/* Validate and enqueue n operators in order (replaces the per-operator
+ * BatchedContext.LaunchAndSync of cuda/arith.go:62, the cuBLAS calls at
+ * cuda/linalg.go:102,223,282 and the cuDNN calls in ops/nn/ *_cuda.go files).
+ * A command that fails validation enqueues nothing from that command on and
+ * returns GH_EINVAL/GH_ENOFUNC with the index in gh_last_error(). */
+GH_API int gh_submit(gh_ctx* ctx, const gh_cmd* cmds, int n);
+/* Validate only: same checks as gh_submit, touches no device. */
+GH_API int gh_validate(const gh_cmd* cmds, int n, char* msg, int msg_len);
+/* Engine.DoWork / Signal+Sync (cuda/external.go:223-226): block until the
+ * stream drains, return the sticky error. */
+GH_API int gh_sync(gh_ctx* ctx);
+
+/* Optional replay of a whole tape segment: record the submits between begin
+ * and end into a hipGraph, launch it again while the segment's pointer set is
+ * unchanged (arena offsets are deterministic, cuda/bfc.go:351-382). */
+GH_API int gh_graph_begin(gh_ctx* ctx);
+GH_API int gh_graph_end(gh_ctx* ctx, int* graph_id);
+GH_API int gh_graph_launch(gh_ctx* ctx, int graph_id);
+GH_API int gh_graph_destroy(gh_ctx* ctx, int graph_id);
+
+/* ---- kernel registry ---------------------------------------------------- */
+
+/* Engine.HasFunc (cuda/external.go:26) over the reference's kernel names,
+ * e.g. "elembinop.add_vv_f32", "elemunaryop.tanh_f32", "misc.hasNaN_f32"
+ * (cuda/utils.go:114-139, op_math_cuda.go:38).  Returns 1/0. */
+GH_API int gh_has_func(const char* name);
+/* Resolve such a name into opcode+flags for a gh_cmd. 0 on success. */
+GH_API int gh_lookup_func(const char* name, uint32_t* opcode, uint32_t* flags);
+
+/* ---- errors -------------------------------------------------------------- */
+
+/* Engine.Errors (cuda/engine.go:141): sticky status; copies the message. */
+GH_API int gh_last_error(gh_ctx* ctx, char* buf, int len);
+GH_API int gh_clear_error(gh_ctx* ctx);
+
+/* ---- timing (benchmark support; no reference counterpart) ---------------- */
+
+/* Record a HIP event on the context's stream into slot [0,64). */
+GH_API int gh_event_record(gh_ctx* ctx, int slot);
+/* Milliseconds between two recorded slots (synchronises on `stop`). */
+GH_API int gh_event_elapsed_ms(gh_ctx* ctx, int start, int stop, float* ms);
+
+/* Library version string. */
+GH_API const char* gh_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GORGONIA_HIP_H */

@@ -1,0 +1,243 @@
+"""ctypes binding of oracle/liboracle.so for the parity tests, the smoke check
+and the CPU-baseline leg of the benchmark.  TEST INFRASTRUCTURE ONLY: the
+product package never imports this module."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB = os.path.join(HERE, "liboracle.so")
+
+BIN = {"add": 0, "sub": 1, "mul": 2, "div": 3, "pow": 4, "lt": 5, "lte": 6, "gt": 7, "gte": 8,
+       "eq": 9, "ne": 10}
+MODE = {"vv": 0, "vs": 1, "sv": 2, "ss": 3}
+UNARY = {"abs": 0, "sign": 1, "ceil": 2, "floor": 3, "sin": 4, "cos": 5, "exp": 6, "ln": 7,
+         "log2": 8, "neg": 9, "square": 10, "sqrt": 11, "inverse": 12, "invsqrt": 13, "cube": 14,
+         "tanh": 15, "sigmoid": 16, "log1p": 17, "expm1": 18, "softplus": 19}
+
+_lib = None
+
+
+def build():
+    subprocess.run(["make", "-C", HERE, "-s"], check=True)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB):
+            build()
+        _lib = C.CDLL(LIB)
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _i64(*v):
+    return [C.c_int64(int(x)) for x in v]
+
+
+def set_threads(n):
+    lib().oracle_set_threads(int(n))
+
+
+def binop(fn, mode, a, b):
+    """Returns the array the device kernel writes (A for vv/vs/ss, B for sv)."""
+    dt = a.dtype
+    A = np.array(a, dtype=dt, copy=True).reshape(-1)
+    B = np.array(b, dtype=dt, copy=True).reshape(-1)
+    n = B.size if mode == "sv" else A.size
+    f = lib().oracle_binop_f32 if dt == np.float32 else lib().oracle_binop_f64
+    f(BIN[fn], MODE[mode], _p(A), _p(B), C.c_int64(n))
+    return B if mode == "sv" else A
+
+
+def bcast_binop(fn, big, small, outer, mid, inner, small_left=False):
+    big = np.ascontiguousarray(big, dtype=np.float32)
+    small = np.ascontiguousarray(small, dtype=np.float32)
+    dst = np.empty(outer * mid * inner, dtype=np.float32)
+    lib().oracle_bcast_binop_f32(BIN[fn], int(small_left), _p(dst), _p(big), _p(small),
+                                 *_i64(outer, mid, inner))
+    return dst
+
+
+def unary(fn, a):
+    A = np.array(a, copy=True).reshape(-1)
+    f = lib().oracle_unary_f32 if A.dtype == np.float32 else lib().oracle_unary_f64
+    f(UNARY[fn], _p(A), C.c_int64(A.size))
+    return A
+
+
+def relu(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty_like(x)
+    lib().oracle_relu_f32(_p(y), _p(x), C.c_int64(x.size))
+    return y
+
+
+def leaky_relu(x, alpha):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty_like(x)
+    lib().oracle_leaky_relu_f32(_p(y), _p(x), C.c_float(alpha), C.c_int64(x.size))
+    return y
+
+
+def gemm(A, B, trans_a=False, trans_b=False):
+    A = np.ascontiguousarray(A, dtype=np.float32)
+    B = np.ascontiguousarray(B, dtype=np.float32)
+    m, k = (A.shape[1], A.shape[0]) if trans_a else A.shape
+    n = B.shape[0] if trans_b else B.shape[1]
+    Cm = np.empty((m, n), dtype=np.float32)
+    lib().oracle_gemm_f32(int(trans_a), int(trans_b), *_i64(m, n, k), _p(A), C.c_int64(A.shape[1]),
+                          _p(B), C.c_int64(B.shape[1]), _p(Cm), C.c_int64(n))
+    return Cm
+
+
+def gemm_f64acc(A, B, trans_a=False, trans_b=False):
+    A = np.ascontiguousarray(A, dtype=np.float32)
+    B = np.ascontiguousarray(B, dtype=np.float32)
+    m, k = (A.shape[1], A.shape[0]) if trans_a else A.shape
+    n = B.shape[0] if trans_b else B.shape[1]
+    Cm = np.empty((m, n), dtype=np.float64)
+    lib().oracle_gemm_f64acc(int(trans_a), int(trans_b), *_i64(m, n, k), _p(A),
+                             C.c_int64(A.shape[1]), _p(B), C.c_int64(B.shape[1]), _p(Cm),
+                             C.c_int64(n))
+    return Cm
+
+
+def bmm(A, B, trans_a=False, trans_b=False):
+    A = np.ascontiguousarray(A, dtype=np.float32)
+    B = np.ascontiguousarray(B, dtype=np.float32)
+    batch = A.shape[0]
+    m, k = (A.shape[2], A.shape[1]) if trans_a else A.shape[1:]
+    n = B.shape[1] if trans_b else B.shape[2]
+    Cm = np.empty((batch, m, n), dtype=np.float32)
+    lib().oracle_bmm_f32(int(trans_a), int(trans_b), *_i64(batch, m, n, k), _p(A), _p(B), _p(Cm))
+    return Cm
+
+
+def gemv(A, x, trans=False):
+    A = np.ascontiguousarray(A, dtype=np.float32)
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    m, n = A.shape
+    y = np.empty(n if trans else m, dtype=np.float32)
+    lib().oracle_gemv_f32(int(trans), *_i64(m, n), _p(A), C.c_int64(n), _p(x), _p(y))
+    return y
+
+
+def outer(x, y):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    A = np.empty((x.size, y.size), dtype=np.float32)
+    lib().oracle_outer_f32(*_i64(x.size, y.size), _p(x), _p(y), _p(A))
+    return A
+
+
+def conv_out_hw(h, w, kh, kw, pad, stride, dil):
+    oh, ow = C.c_int64(), C.c_int64()
+    lib().oracle_conv_out_hw(*_i64(h, w, kh, kw, pad[0], pad[1], stride[0], stride[1], dil[0],
+                                   dil[1]), C.byref(oh), C.byref(ow))
+    return oh.value, ow.value
+
+
+def conv2d(x, w, pad=(0, 0), stride=(1, 1), dil=(1, 1)):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    B, Cn, H, W = x.shape
+    F, _, kh, kw = w.shape
+    oh, ow = conv_out_hw(H, W, kh, kw, pad, stride, dil)
+    y = np.empty((B, F, oh, ow), dtype=np.float32)
+    rc = lib().oracle_conv2d_f32(_p(x), _p(w), _p(y), *_i64(B, Cn, H, W, F, kh, kw, pad[0], pad[1],
+                                                           stride[0], stride[1], dil[0], dil[1]))
+    if rc != 0:
+        raise MemoryError("oracle conv2d scratch allocation failed")
+    return y
+
+
+def conv2d_direct_f64(x, w, pad=(0, 0), stride=(1, 1), dil=(1, 1)):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    B, Cn, H, W = x.shape
+    F, _, kh, kw = w.shape
+    oh, ow = conv_out_hw(H, W, kh, kw, pad, stride, dil)
+    y = np.empty((B, F, oh, ow), dtype=np.float64)
+    lib().oracle_conv2d_direct_f64(_p(x), _p(w), _p(y), *_i64(B, Cn, H, W, F, kh, kw, pad[0], pad[1],
+                                                             stride[0], stride[1], dil[0], dil[1]))
+    return y
+
+
+def _pad4(pad):
+    if len(pad) == 4:
+        return np.array(pad, dtype=np.int64), 1
+    return np.array([pad[0], pad[0], pad[1], pad[1]], dtype=np.int64), 0
+
+
+def maxpool_out_hw(h, w, kh, kw, pad, stride):
+    p4, _ = _pad4(pad)
+    oh, ow = C.c_int64(), C.c_int64()
+    lib().oracle_maxpool_out_hw(*_i64(h, w, kh, kw), _p(p4), *_i64(stride[0], stride[1]),
+                                C.byref(oh), C.byref(ow))
+    return oh.value, ow.value
+
+
+def maxpool2d(x, kernel, pad, stride):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    B, Cn, H, W = x.shape
+    p4, explicit = _pad4(pad)
+    oh, ow = maxpool_out_hw(H, W, kernel[0], kernel[1], pad, stride)
+    y = np.empty((B, Cn, oh, ow), dtype=np.float32)
+    lib().oracle_maxpool2d_f32(_p(x), _p(y), *_i64(B, Cn, H, W, kernel[0], kernel[1]), _p(p4),
+                               C.c_int(explicit), *_i64(stride[0], stride[1]))
+    return y
+
+
+def bn_infer(x, mean, var, eps, gamma=None, beta=None):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    B, Cn = x.shape[:2]
+    S = x.size // (B * Cn)
+    y = np.empty_like(x)
+    mean = np.ascontiguousarray(mean, dtype=np.float32)
+    var = np.ascontiguousarray(var, dtype=np.float32)
+    g = np.ascontiguousarray(gamma, dtype=np.float32) if gamma is not None else None
+    b = np.ascontiguousarray(beta, dtype=np.float32) if beta is not None else None
+    lib().oracle_bn_infer_f32(_p(x), _p(y), _p(mean), _p(var), _p(g) if g is not None else None,
+                              _p(b) if b is not None else None, C.c_float(eps), *_i64(B, Cn, S))
+    return y
+
+
+def bn_train(x, run_mean, run_var, momentum, eps):
+    """One training-mode forward; returns (y, new_running_mean, new_running_var)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    B, Cn = x.shape[:2]
+    S = x.size // (B * Cn)
+    y = np.empty_like(x)
+    rm = np.array(run_mean, dtype=np.float32, copy=True)
+    rv = np.array(run_var, dtype=np.float32, copy=True)
+    lib().oracle_bn_train_f32(_p(x), _p(y), _p(rm), _p(rv), C.c_float(momentum), C.c_float(eps),
+                              *_i64(B, Cn, S))
+    return y, rm, rv
+
+
+def softmax(x):
+    x = np.ascontiguousarray(x)
+    rows, cols = int(np.prod(x.shape[:-1])), x.shape[-1]
+    y = np.empty_like(x)
+    f = lib().oracle_softmax_f32 if x.dtype == np.float32 else lib().oracle_softmax_f64
+    f(_p(x), _p(y), *_i64(rows, cols))
+    return y
+
+
+def has_nan(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return bool(lib().oracle_has_nan_f32(_p(a), C.c_int64(a.size)))
+
+
+def has_inf(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return bool(lib().oracle_has_inf_f32(_p(a), C.c_int64(a.size)))

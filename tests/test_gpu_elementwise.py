@@ -1,0 +1,237 @@
+"""GPU parity: elementwise binary / unary / broadcast / relu kernels against the
+CPU oracle on the same seeded inputs, called through the C ABI (gh_submit).
+
+Bars: add/sub/mul/div/compare/relu/leaky/broadcast bit-exact; exp/tanh/sigmoid
+(and the other transcendentals) within 2 float32 ulp; pow(x, 2) bit-exact."""
+import numpy as np
+import pytest
+
+from gorgonia_amd import device as D
+from gorgonia_amd import synth
+from oracle import binding as O
+from tests.util import assert_bits_equal, ulp_diff
+
+pytestmark = pytest.mark.gpu
+
+EXACT_BIN = ["add", "sub", "mul", "div", "lt", "lte", "gt", "gte", "eq", "ne"]
+SIZES = [0, 1, 3, 4, 5, 255, 1024, 4099, 1 << 20, (1 << 20) + 7]
+
+
+def _special(n, seed):
+    """Seeded values salted with signed zeros, denormals, infinities, NaN, ties."""
+    a = synth.uniform(seed, (n,), -4.0, 4.0)
+    sp = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-42, -1e-42, 3.4e38, -3.4e38,
+                   1.17549435e-38, 2.0, 0.5], dtype=np.float32)
+    k = min(n, sp.size)
+    a[:k] = sp[:k]
+    return a
+
+
+def _operands(mode, n):
+    if mode == "vv":
+        return _special(n, 11), _special(n, 23)[::-1].copy()
+    if mode == "vs":
+        return _special(n, 11), np.array([1.5], dtype=np.float32)
+    if mode == "sv":
+        return np.array([-2.25], dtype=np.float32), _special(n, 23)
+    return np.array([3.0], dtype=np.float32), np.array([-0.75], dtype=np.float32)
+
+
+@pytest.mark.parametrize("fn", EXACT_BIN)
+@pytest.mark.parametrize("mode", ["vv", "vs", "sv", "ss"])
+def test_binary_bit_exact(ctx, fn, mode):
+    for n in ([1] if mode == "ss" else SIZES):
+        a, b = _operands(mode, n)
+        da, db = ctx.upload(a), ctx.upload(b)
+        ctx.run(D.cmd_bin(fn, mode, da, db, n))
+        dst, dst_host, src, src_host = (db, b, da, a) if mode == "sv" else (da, a, db, b)
+        got = ctx.d2h(dst, dst_host.shape)
+        assert_bits_equal(got, O.binop(fn, mode, a, b), f"{fn}_{mode} n={n}")
+        # the operand that is not the destination is left untouched
+        assert_bits_equal(ctx.d2h(src, src_host.shape), src_host, f"{fn}_{mode} source operand")
+        ctx.free(da)
+        ctx.free(db)
+
+
+def test_binary_unaligned_operands(ctx):
+    n = 1000
+    a = synth.uniform(5, (n + 3,), -4, 4)
+    b = synth.uniform(6, (n + 3,), -4, 4)
+    da, db = ctx.upload(a), ctx.upload(b)
+    ctx.run(D.cmd_bin("mul", "vv", da + 4, db + 8, n))  # 4- and 8-byte offsets
+    got = ctx.d2h(da, (n + 3,))
+    want = a.copy()
+    want[1:n + 1] = O.binop("mul", "vv", a[1:n + 1], b[2:n + 2])
+    assert_bits_equal(got, want, "unaligned mul")
+    ctx.free(da); ctx.free(db)
+
+
+def test_binary_f64(ctx):
+    n = 4099
+    rng = np.random.default_rng(3)
+    a = rng.uniform(-4, 4, n)
+    b = rng.uniform(-4, 4, n)
+    for fn in ["add", "sub", "mul", "div", "gte"]:
+        da, db = ctx.upload(a), ctx.upload(b)
+        ctx.run(D.cmd_bin(fn, "vv", da, db, n, dtype=1))
+        got = ctx.d2h(da, (n,), np.float64)
+        assert_bits_equal(got, O.binop(fn, "vv", a, b), f"{fn}_vv_f64")
+        ctx.free(da); ctx.free(db)
+
+
+def test_pow_scalar_two_is_exact_square(ctx):
+    n = (1 << 18) + 3
+    a = synth.uniform(7, (n,), 0.0, 1.0)
+    two = np.array([2.0], dtype=np.float32)
+    da, db = ctx.upload(a), ctx.upload(two)
+    ctx.run(D.cmd_bin("pow", "vs", da, db, n))
+    got = ctx.d2h(da, (n,))
+    assert_bits_equal(got, O.binop("pow", "vs", a, two), "pow(x,2) vs oracle")
+    assert_bits_equal(got, a * a, "pow(x,2) == x*x")
+    ctx.free(da); ctx.free(db)
+
+
+def test_pow_general(ctx):
+    n = 50000
+    a = synth.uniform(8, (n,), 0.01, 4.0)
+    b = synth.uniform(9, (n,), -3.0, 3.0)
+    da, db = ctx.upload(a), ctx.upload(b)
+    ctx.run(D.cmd_bin("pow", "vv", da, db, n))
+    got = ctx.d2h(da, (n,))
+    assert ulp_diff(got, O.binop("pow", "vv", a, b)).max() <= 2
+    ctx.free(da); ctx.free(db)
+
+
+ULP2 = ["exp", "tanh", "sigmoid", "ln", "log2", "sin", "cos", "log1p", "expm1", "softplus"]
+EXACT_UNARY = ["abs", "sign", "ceil", "floor", "neg", "square", "sqrt", "inverse", "invsqrt", "cube"]
+
+
+def _unary_input(fn, n, seed):
+    if fn in ("ln", "log2", "sqrt", "invsqrt"):
+        x = synth.uniform(seed, (n,), 1e-3, 50.0)
+    elif fn == "log1p":
+        x = synth.uniform(seed, (n,), -0.99, 50.0)
+    elif fn in ("exp", "expm1"):
+        x = synth.uniform(seed, (n,), -80.0, 80.0)
+    elif fn in ("sigmoid", "softplus"):
+        x = synth.uniform(seed, (n,), -110.0, 30.0)
+    elif fn == "tanh":
+        x = np.concatenate([synth.uniform(seed, (n // 2,), -12.0, 12.0),
+                            synth.uniform(seed + 1, (n - n // 2,), -0.01, 0.01)])
+    else:
+        x = synth.uniform(seed, (n,), -4.0, 4.0)
+    sp = np.array([0.0, -0.0, 1.0, -1.0, 0.5, -0.5, 1e-30, -1e-30, 15.0, 15.000001, -88.0,
+                   -88.00001, 14.0, -103.0, 20.0, -20.0], dtype=np.float32)
+    if fn not in ("ln", "log2", "sqrt", "invsqrt", "log1p", "inverse"):
+        x[:sp.size] = sp
+    return x.astype(np.float32)
+
+
+@pytest.mark.parametrize("fn", ULP2)
+def test_unary_within_2ulp(ctx, fn):
+    for n in [5, 4099, (1 << 20) + 3]:
+        x = _unary_input(fn, max(n, 32), 31)[:n] if n < 32 else _unary_input(fn, n, 31)
+        d = ctx.upload(x)
+        ctx.run(D.cmd_unary(fn, d, x.size))
+        got = ctx.d2h(d, (x.size,))
+        want = O.unary(fn, x)
+        u = ulp_diff(got, want)
+        assert u.max() <= 2, f"{fn}: max ulp {u.max()} at x={x[int(u.argmax())]!r}"
+        ctx.free(d)
+
+
+@pytest.mark.parametrize("fn", EXACT_UNARY)
+def test_unary_bit_exact(ctx, fn):
+    for n in [5, 4099, (1 << 20) + 3]:
+        x = _unary_input(fn, max(n, 32), 41)[:n]
+        d = ctx.upload(x)
+        ctx.run(D.cmd_unary(fn, d, x.size))
+        got = ctx.d2h(d, (x.size,))
+        assert_bits_equal(got, O.unary(fn, x), fn)
+        ctx.free(d)
+
+
+def test_sigmoid_identities(ctx):
+    """Closed-form pins of the sigmoid kernel itself: s(0)=1/2, cut-offs
+    (math_nooptim.go:36-44), monotone, s(x)+s(-x)=1 within rounding."""
+    x = np.linspace(-20, 15, 70001).astype(np.float32)
+    xs = np.concatenate([x, -x, np.array([0.0, -88.5, 15.5, -88.0, 15.0], np.float32)])
+    d = ctx.upload(xs)
+    ctx.run(D.cmd_unary("sigmoid", d, xs.size))
+    s = ctx.d2h(d, (xs.size,))
+    n = x.size
+    assert s[2 * n] == 0.5 and s[2 * n + 1] == 0.0 and s[2 * n + 2] == 1.0
+    assert s[2 * n + 3] > 0.0 and s[2 * n + 4] < 1.0
+    assert np.all(np.diff(s[:n]) >= 0)
+    ok = np.abs(x) <= 15
+    assert np.max(np.abs(s[:n][ok].astype(np.float64) + s[n:2 * n][ok] - 1.0)) <= 2 ** -23
+    ctx.free(d)
+
+
+@pytest.mark.parametrize("fn", ["add", "mul", "sub", "div"])
+@pytest.mark.parametrize("shape", [(64, 4096, 1), (7, 12, 1), (8, 16, 169), (3, 5, 64), (1, 4096, 1),
+                                   (4096, 8, 1)])
+@pytest.mark.parametrize("left", [False, True])
+def test_broadcast_bit_exact(ctx, fn, shape, left):
+    outer, mid, inner = shape
+    big = synth.uniform(51, (outer * mid * inner,), -4, 4)
+    small = synth.uniform(52, (mid,), -4, 4)
+    db, ds = ctx.upload(big), ctx.upload(small)
+    dd = ctx.malloc(big.nbytes)
+    ctx.run(D.cmd_bcast(fn, dd, db, ds, outer, mid, inner, small_left=left))
+    got = ctx.d2h(dd, big.shape)
+    assert_bits_equal(got, O.bcast_binop(fn, big, small, outer, mid, inner, left), f"bcast {fn}")
+    ctx.free(db); ctx.free(ds); ctx.free(dd)
+
+
+def test_relu_and_leaky_bit_exact(ctx):
+    for n in [1, 7, 4099, (1 << 20) + 1]:
+        x = _special(n, 61)
+        dx = ctx.upload(x)
+        dy = ctx.malloc(x.nbytes)
+        ctx.run(D.cmd_relu(dx, dy, n))
+        got = ctx.d2h(dy, (n,))
+        assert_bits_equal(got, O.relu(x), "relu")
+        ctx.run(D.cmd_leaky_relu(dx, dy, n, 0.1))
+        assert_bits_equal(ctx.d2h(dy, (n,)), O.leaky_relu(x, 0.1), "leaky")
+        ctx.free(dx); ctx.free(dy)
+    # negative inputs give -0.0 (x * 0), the CPU engine's form (nn.go:154-162)
+    x = np.array([-1.0, -0.0, 0.0, 2.0], np.float32)
+    dx = ctx.upload(x); dy = ctx.malloc(16)
+    ctx.run(D.cmd_relu(dx, dy, 4))
+    got = ctx.d2h(dy, (4,))
+    assert np.signbit(got[0]) and got[0] == 0.0 and got[3] == 2.0
+    ctx.free(dx); ctx.free(dy)
+
+
+def test_has_nan_inf(ctx):
+    n = 100003
+    x = synth.uniform(71, (n,), -4, 4)
+    flag = ctx.malloc(4)
+    for kind, val in [("nan", np.nan), ("inf", np.inf), ("inf", -np.inf)]:
+        d = ctx.upload(x)
+        ctx.run(D.cmd_has(kind, d, flag, n))
+        assert ctx.d2h(flag, (1,), np.int32)[0] == 0
+        y = x.copy(); y[n - 2] = val
+        ctx.h2d(d, y)
+        ctx.run(D.cmd_has(kind, d, flag, n))
+        assert ctx.d2h(flag, (1,), np.int32)[0] == 1
+        other = "inf" if kind == "nan" else "nan"
+        ctx.run(D.cmd_has(other, d, flag, n))
+        assert ctx.d2h(flag, (1,), np.int32)[0] == 0
+        ctx.free(d)
+    ctx.free(flag)
+
+
+def test_denormals_and_division_are_ieee(ctx):
+    """No flush-to-zero, correctly rounded division (the reference builds its
+    kernels with -ftz=false -prec-div=true, cmd/cudagen/main.go:41-43)."""
+    a = np.array([1e-40, 2e-45, 1.0, 1.0, 7.0, 1e-38], np.float32)
+    b = np.array([0.5, 1.0, 3.0, 7.0, 3.0, 0.1], np.float32)
+    for fn in ("mul", "div", "add"):
+        da, db = ctx.upload(a), ctx.upload(b)
+        ctx.run(D.cmd_bin(fn, "vv", da, db, a.size))
+        got = ctx.d2h(da, a.shape)
+        want = {"mul": a * b, "div": a / b, "add": a + b}[fn]
+        assert_bits_equal(got, want, f"ieee {fn}")
+        ctx.free(da); ctx.free(db)

@@ -1,0 +1,148 @@
+"""GPU parity: MatMul / BatchedMatMul / MatVecMul / Outer through the C ABI
+against the CPU oracle.  Bar: relative Frobenius error <= 1e-5 against the
+float64 product (the oracle's own float32 sequential-k result is held to the
+same bar), and exact equality on integer-valued inputs where every summation
+order is exact."""
+import numpy as np
+import pytest
+
+from gorgonia_amd import device as D
+from gorgonia_amd import synth
+from oracle import binding as O
+from tests.util import assert_bits_equal, rel_frobenius
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def _run_gemm(ctx, A, B, ta=False, tb=False, act=None, alpha=0.0):
+    m, k = (A.shape[1], A.shape[0]) if ta else A.shape
+    n = B.shape[0] if tb else B.shape[1]
+    dA, dB = ctx.upload(A), ctx.upload(B)
+    dC = ctx.malloc(m * n * 4)
+    ctx.run(D.cmd_fill(dC, m * n, np.nan))
+    ctx.run(D.cmd_gemm(dA, dB, dC, m, n, k, trans_a=ta, trans_b=tb, act=act, alpha=alpha))
+    out = ctx.d2h(dC, (m, n))
+    for p in (dA, dB, dC):
+        ctx.free(p)
+    return out
+
+
+SHAPES = [(1, 1, 1), (3, 5, 7), (32, 32, 2), (64, 64, 16), (65, 129, 33), (128, 128, 128),
+          (256, 784, 300), (256, 300, 100), (256, 100, 10), (128, 1152, 625), (130, 10, 625),
+          (512, 512, 512), (1000, 37, 259)]  # (m, k, n)
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_matmul_vs_oracle(ctx, ta, tb):
+    for (m, k, n) in SHAPES:
+        A = synth.normal(100 + m, (k, m) if ta else (m, k))
+        B = synth.normal(200 + n, (n, k) if tb else (k, n))
+        got = _run_gemm(ctx, A, B, ta, tb)
+        ref = O.gemm_f64acc(A, B, ta, tb)
+        err = rel_frobenius(got, ref)
+        assert err <= TOL, f"gemm {m}x{k}x{n} ta={ta} tb={tb}: rel frobenius {err:.3e}"
+        assert rel_frobenius(O.gemm(A, B, ta, tb), ref) <= TOL
+
+
+def test_matmul_integer_exact(ctx):
+    """Small-integer inputs: every partial sum is exactly representable, so any
+    accumulation order must give the oracle's bits."""
+    rng = np.random.default_rng(0)
+    for (m, k, n) in [(64, 64, 64), (100, 50, 30), (256, 300, 100), (7, 1, 5)]:
+        A = rng.integers(-8, 9, (m, k)).astype(np.float32)
+        B = rng.integers(-8, 9, (k, n)).astype(np.float32)
+        for ta, tb in [(False, False), (False, True), (True, False), (True, True)]:
+            As = A.T.copy() if ta else A
+            Bs = B.T.copy() if tb else B
+            got = _run_gemm(ctx, As, Bs, ta, tb)
+            assert_bits_equal(got, O.gemm(As, Bs, ta, tb), f"int gemm ta={ta} tb={tb}")
+            assert np.array_equal(got, (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32))
+
+
+def test_matmul_fused_relu_epilogue(ctx):
+    A = synth.normal(1, (256, 784))
+    B = synth.normal(2, (784, 300))
+    plain = _run_gemm(ctx, A, B)
+    fused = _run_gemm(ctx, A, B, act="relu")
+    assert_bits_equal(fused, O.relu(plain).reshape(plain.shape), "gemm+relu epilogue")
+    fusedl = _run_gemm(ctx, A, B, act="leaky", alpha=0.1)
+    assert_bits_equal(fusedl, O.leaky_relu(plain, 0.1).reshape(plain.shape), "gemm+leaky epilogue")
+
+
+def test_matmul_strided_ld(ctx):
+    """Leading dimensions larger than the logical width (sub-matrix views)."""
+    m, k, n = 70, 52, 44
+    Abig = synth.normal(3, (m, k + 12))
+    Bbig = synth.normal(4, (k, n + 8))
+    dA, dB = ctx.upload(Abig), ctx.upload(Bbig)
+    dC = ctx.malloc(m * (n + 4) * 4)
+    ctx.run(D.cmd_fill(dC, m * (n + 4), -7.0))
+    ctx.run(D.cmd_gemm(dA, dB, dC, m, n, k, lda=k + 12, ldb=n + 8, ldc=n + 4))
+    out = ctx.d2h(dC, (m, n + 4))
+    ref = O.gemm_f64acc(Abig[:, :k].copy(), Bbig[:, :n].copy())
+    assert rel_frobenius(out[:, :n], ref) <= TOL
+    assert np.all(out[:, n:] == -7.0)  # padding columns untouched
+    for p in (dA, dB, dC):
+        ctx.free(p)
+
+
+@pytest.mark.parametrize("shape", [(4, 32, 48, 40), (64, 64, 64, 64), (3, 130, 70, 50), (6, 2, 3, 2)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False)])
+def test_batched_matmul(ctx, shape, ta, tb):
+    batch, m, k, n = shape
+    A = synth.normal(5, (batch, k, m) if ta else (batch, m, k))
+    B = synth.normal(6, (batch, n, k) if tb else (batch, k, n))
+    dA, dB = ctx.upload(A), ctx.upload(B)
+    dC = ctx.malloc(batch * m * n * 4)
+    ctx.run(D.cmd_gemm(dA, dB, dC, m, n, k, trans_a=ta, trans_b=tb, batch=batch, stride_a=m * k,
+                       stride_b=k * n, stride_c=m * n))
+    got = ctx.d2h(dC, (batch, m, n))
+    want = O.bmm(A, B, ta, tb)
+    for b in range(batch):
+        ref = O.gemm_f64acc(A[b], B[b], ta, tb)
+        assert rel_frobenius(got[b], ref) <= TOL
+        assert rel_frobenius(want[b], ref) <= TOL
+    for p in (dA, dB, dC):
+        ctx.free(p)
+
+
+def test_batched_matmul_reference_example(ctx):
+    """example_linalg_test.go:11-92: BatchedMatMul of Range tensors."""
+    a = np.arange(2 * 3 * 2, dtype=np.float32).reshape(2, 3, 2)
+    b = np.arange(2 * 2 * 3, dtype=np.float32).reshape(2, 2, 3)
+    dA, dB = ctx.upload(a), ctx.upload(b)
+    dC = ctx.malloc(2 * 3 * 3 * 4)
+    ctx.run(D.cmd_gemm(dA, dB, dC, 3, 3, 2, batch=2, stride_a=6, stride_b=6, stride_c=9))
+    got = ctx.d2h(dC, (2, 3, 3))
+    assert np.array_equal(got, np.matmul(a, b))
+    for p in (dA, dB, dC):
+        ctx.free(p)
+
+
+@pytest.mark.parametrize("m,n", [(1, 1), (5, 3), (64, 64), (300, 784), (1000, 1001), (2048, 4096)])
+@pytest.mark.parametrize("trans", [False, True])
+def test_matvec(ctx, m, n, trans):
+    A = synth.normal(7, (m, n))
+    x = synth.normal(8, (m if trans else n,))
+    dA, dx = ctx.upload(A), ctx.upload(x)
+    dy = ctx.malloc((n if trans else m) * 4)
+    ctx.run(D.cmd_gemv(dA, dx, dy, m, n, trans=trans))
+    got = ctx.d2h(dy, (n if trans else m,))
+    ref = (A.T if trans else A).astype(np.float64) @ x.astype(np.float64)
+    assert rel_frobenius(got, ref) <= TOL
+    assert rel_frobenius(O.gemv(A, x, trans), ref) <= TOL
+    for p in (dA, dx, dy):
+        ctx.free(p)
+
+
+def test_outer_bit_exact(ctx):
+    x = synth.normal(9, (37,))
+    y = synth.normal(10, (53,))
+    dx, dy = ctx.upload(x), ctx.upload(y)
+    dA = ctx.malloc(37 * 53 * 4)
+    ctx.run(D.cmd_outer(dx, dy, dA, 37, 53))
+    assert_bits_equal(ctx.d2h(dA, (37, 53)), O.outer(x, y), "outer")
+    for p in (dx, dy, dA):
+        ctx.free(p)
