@@ -121,10 +121,9 @@ __global__ __launch_bounds__(kBlock) void k_bn_infer(const float* __restrict__ x
 }
 
 // Row softmax, one wavefront per row: max, exp(x - max) in float64 rounded
-// once, sum, scale by the rounded reciprocal.  Rows of at most 64
-// columns keep their exponentials in registers; the sum is taken in column
-// order by walking lanes, so it matches a sequential CPU loop exactly.
-
+// once, sum, scale by the rounded reciprocal.  The sum is taken in column
+// order (64 exponentials at a time, added lane by lane through readlane), so
+// it carries the same rounding as a sequential CPU loop.
 __global__ __launch_bounds__(kBlock) void k_softmax(const float* __restrict__ x,
                                                     float* __restrict__ y, int64_t rows, int cols) {
   const int lane = threadIdx.x & 63;
@@ -136,23 +135,23 @@ __global__ __launch_bounds__(kBlock) void k_softmax(const float* __restrict__ x,
   for (int j = lane; j < cols; j += 64) mx = fmaxf(mx, in[j]);
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-  if (cols <= 64) {
+  float sum = 0.f;
+  float keep = 0.f;  // this lane's exponential when the row fits one chunk
+  for (int j0 = 0; j0 < cols; j0 += 64) {
+    const int j = j0 + lane;
     float e = 0.f;
-    if (lane < cols) e = (float)exp((double)(in[lane] - mx));
-    float sum = 0.f;
-    for (int j = 0; j < cols; j++) sum = sum + __shfl(e, j, 64);  // column order
-    const float inv = 1.0f / sum;
-    if (lane < cols) out[lane] = e * inv;
-  } else {
-    float sum = 0.f;
-    for (int j = lane; j < cols; j += 64) {
-      const float e = (float)exp((double)(in[j] - mx));
-      out[j] = e;
-      sum += e;
+    if (j < cols) {
+      e = (float)exp((double)(in[j] - mx));
+      if (cols > 64) out[j] = e;
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    const float inv = 1.0f / sum;
+    keep = e;
+    const int lim = min(64, cols - j0);
+    for (int l = 0; l < lim; l++) sum = sum + __shfl(e, l, 64);
+  }
+  const float inv = 1.0f / sum;
+  if (cols <= 64) {
+    if (lane < cols) out[lane] = keep * inv;
+  } else {
     for (int j = lane; j < cols; j += 64) out[j] = out[j] * inv;
   }
 }
