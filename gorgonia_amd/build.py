@@ -103,7 +103,9 @@ def build_host(force=False):
     deps = srcs + _headers(HOST) + _headers(INCLUDE)
     if force or _newer(deps, out):
         cxx = shutil.which("g++") or "g++"
-        _run([cxx] + HOST_FLAGS + ["-shared", "-o", out] + srcs + ["-ldl"])
+        # links against the device library through its C ABI only
+        _run([cxx] + HOST_FLAGS + ["-shared", "-o", out] + srcs +
+             ["-L", LIBDIR, "-lgorgonia_hip", "-Wl,-rpath,$ORIGIN"])
     return out
 
 

@@ -126,7 +126,7 @@ __device__ __forceinline__ double unary_apply(double x) {
 // x*x is used (equal to the correctly rounded pow(x,2)).
 
 template <int FN, class T, int MODE>
-__global__ __launch_bounds__(kBlock) void k_bin_vec(T* __restrict__ A, T* __restrict__ B, int64_t n) {
+__global__ __launch_bounds__(kBlock) void k_bin_vec(const T* A, const T* B, T* D, int64_t n) {
   using V = typename VecOf<T>::type;
   constexpr int N = VecOf<T>::N;
   const int64_t nv = n / N;
@@ -136,8 +136,9 @@ __global__ __launch_bounds__(kBlock) void k_bin_vec(T* __restrict__ A, T* __rest
   bool pow2 = false;
   if constexpr (MODE == GH_VS) { s = B[0]; if constexpr (FN == GH_POW) pow2 = (s == (T)2); }
   if constexpr (MODE == GH_SV) s = A[0];
-  V* __restrict__ Av = reinterpret_cast<V*>(A);
-  V* __restrict__ Bv = reinterpret_cast<V*>(B);
+  const V* Av = reinterpret_cast<const V*>(A);
+  const V* Bv = reinterpret_cast<const V*>(B);
+  V* Dv = reinterpret_cast<V*>(D);
   for (; i + (kUnroll - 1) * stride < nv; i += kUnroll * stride) {
     V a[kUnroll], b[kUnroll];
 #pragma unroll
@@ -156,8 +157,7 @@ __global__ __launch_bounds__(kBlock) void k_bin_vec(T* __restrict__ A, T* __rest
           else r[e] = bin_apply<FN, T>(a[u][e], s);
         } else r[e] = bin_apply<FN, T>(s, b[u][e]);
       }
-      if constexpr (MODE == GH_SV) __builtin_nontemporal_store(r, &Bv[i + u * stride]);
-      else __builtin_nontemporal_store(r, &Av[i + u * stride]);
+      __builtin_nontemporal_store(r, &Dv[i + u * stride]);
     }
   }
   for (; i < nv; i += stride) {
@@ -172,45 +172,46 @@ __global__ __launch_bounds__(kBlock) void k_bin_vec(T* __restrict__ A, T* __rest
         else r[e] = bin_apply<FN, T>(a[e], s);
       } else r[e] = bin_apply<FN, T>(s, b[e]);
     }
-    if constexpr (MODE == GH_SV) Bv[i] = r; else Av[i] = r;
+    Dv[i] = r;
   }
   // scalar tail (n % N elements)
   const int64_t t = nv * N + (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (t < n) {
-    if constexpr (MODE == GH_VV) A[t] = bin_apply<FN, T>(A[t], B[t]);
+    if constexpr (MODE == GH_VV) D[t] = bin_apply<FN, T>(A[t], B[t]);
     else if constexpr (MODE == GH_VS) {
-      if constexpr (FN == GH_POW) A[t] = pow2 ? A[t] * A[t] : bin_apply<FN, T>(A[t], s);
-      else A[t] = bin_apply<FN, T>(A[t], s);
-    } else B[t] = bin_apply<FN, T>(s, B[t]);
+      if constexpr (FN == GH_POW) D[t] = pow2 ? A[t] * A[t] : bin_apply<FN, T>(A[t], s);
+      else D[t] = bin_apply<FN, T>(A[t], s);
+    } else D[t] = bin_apply<FN, T>(s, B[t]);
   }
 }
 
 // Unaligned operands, or scalar-scalar: plain one-element-per-thread loop.
 template <int FN, class T, int MODE>
-__global__ __launch_bounds__(kBlock) void k_bin_scalar(T* A, T* B, int64_t n) {
+__global__ __launch_bounds__(kBlock) void k_bin_scalar(const T* A, const T* B, T* D, int64_t n) {
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   T s = (T)0;
   if constexpr (MODE == GH_VS) s = B[0];
   if constexpr (MODE == GH_SV || MODE == GH_SS) s = A[0];
   if constexpr (MODE == GH_SS) {
-    if (blockIdx.x == 0 && threadIdx.x == 0) A[0] = bin_apply<FN, T>(s, B[0]);
+    if (blockIdx.x == 0 && threadIdx.x == 0) D[0] = bin_apply<FN, T>(s, B[0]);
     return;
   }
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
-    if constexpr (MODE == GH_VV) A[i] = bin_apply<FN, T>(A[i], B[i]);
-    else if constexpr (MODE == GH_VS) A[i] = bin_apply<FN, T>(A[i], s);
-    else if constexpr (MODE == GH_SV) B[i] = bin_apply<FN, T>(s, B[i]);
+    if constexpr (MODE == GH_VV) D[i] = bin_apply<FN, T>(A[i], B[i]);
+    else if constexpr (MODE == GH_VS) D[i] = bin_apply<FN, T>(A[i], s);
+    else if constexpr (MODE == GH_SV) D[i] = bin_apply<FN, T>(s, B[i]);
   }
 }
 
 template <int FN, class T>
-__global__ __launch_bounds__(kBlock) void k_unary_vec(T* __restrict__ A, int64_t n) {
+__global__ __launch_bounds__(kBlock) void k_unary_vec(const T* A, T* D, int64_t n) {
   using V = typename VecOf<T>::type;
   constexpr int N = VecOf<T>::N;
   const int64_t nv = n / N;
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  V* __restrict__ Av = reinterpret_cast<V*>(A);
+  const V* Av = reinterpret_cast<const V*>(A);
+  V* Dv = reinterpret_cast<V*>(D);
   for (; i + (kUnroll - 1) * stride < nv; i += kUnroll * stride) {
     V a[kUnroll];
 #pragma unroll
@@ -220,24 +221,24 @@ __global__ __launch_bounds__(kBlock) void k_unary_vec(T* __restrict__ A, int64_t
       V r;
 #pragma unroll
       for (int e = 0; e < N; e++) r[e] = unary_apply<FN>(a[u][e]);
-      __builtin_nontemporal_store(r, &Av[i + u * stride]);
+      __builtin_nontemporal_store(r, &Dv[i + u * stride]);
     }
   }
   for (; i < nv; i += stride) {
     V a = Av[i], r;
 #pragma unroll
     for (int e = 0; e < N; e++) r[e] = unary_apply<FN>(a[e]);
-    Av[i] = r;
+    Dv[i] = r;
   }
   const int64_t t = nv * N + (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (t < n) A[t] = unary_apply<FN>(A[t]);
+  if (t < n) D[t] = unary_apply<FN>(A[t]);
 }
 
 template <int FN, class T>
-__global__ __launch_bounds__(kBlock) void k_unary_scalar(T* A, int64_t n) {
+__global__ __launch_bounds__(kBlock) void k_unary_scalar(const T* A, T* D, int64_t n) {
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride)
-    A[i] = unary_apply<FN>(A[i]);
+    D[i] = unary_apply<FN>(A[i]);
 }
 
 // ---- fused broadcast --------------------------------------------------------
@@ -361,13 +362,17 @@ inline bool aligned16(uint64_t p) { return (p & 15u) == 0; }
 
 template <int FN, class T>
 int launch_bin_fn(gh_ctx* ctx, const gh_cmd& c) {
-  T* A = (T*)(uintptr_t)c.ptr[0];
-  T* B = (T*)(uintptr_t)c.ptr[1];
-  const int64_t n = c.dim[0];
+  const T* A = (const T*)(uintptr_t)c.ptr[0];
+  const T* B = (const T*)(uintptr_t)c.ptr[1];
   const uint32_t mode = gh_mode(c.flags);
+  // ptr[2] (optional) is a separate destination; without it the kernel works
+  // in place: on A for vv/vs/ss, on B for sv (elembinop.cu:13-35).
+  const uint64_t dptr = c.ptr[2] ? c.ptr[2] : (mode == GH_SV ? c.ptr[1] : c.ptr[0]);
+  T* Dst = (T*)(uintptr_t)dptr;
+  const int64_t n = c.dim[0];
   constexpr int N = VecOf<T>::N;
   if (n == 0) return GH_OK;
-  bool vec = n >= N;
+  bool vec = n >= N && aligned16(dptr);
   if (mode == GH_VV) vec = vec && aligned16(c.ptr[0]) && aligned16(c.ptr[1]);
   if (mode == GH_VS) vec = vec && aligned16(c.ptr[0]);
   if (mode == GH_SV) vec = vec && aligned16(c.ptr[1]);
@@ -375,14 +380,14 @@ int launch_bin_fn(gh_ctx* ctx, const gh_cmd& c) {
   const int gv = grid_for(ctx, n / N + N, kUnroll);
   const int gs = grid_for(ctx, n, 4);
 #define GH_LAUNCH_MODE(M)                                                                   \
-  if (vec) hipLaunchKernelGGL((k_bin_vec<FN, T, M>), dim3(gv), dim3(kBlock), 0, ctx->stream, A, B, n); \
-  else hipLaunchKernelGGL((k_bin_scalar<FN, T, M>), dim3(gs), dim3(kBlock), 0, ctx->stream, A, B, n);
+  if (vec) hipLaunchKernelGGL((k_bin_vec<FN, T, M>), dim3(gv), dim3(kBlock), 0, ctx->stream, A, B, Dst, n); \
+  else hipLaunchKernelGGL((k_bin_scalar<FN, T, M>), dim3(gs), dim3(kBlock), 0, ctx->stream, A, B, Dst, n);
   switch (mode) {
     case GH_VV: GH_LAUNCH_MODE(GH_VV) break;
     case GH_VS: GH_LAUNCH_MODE(GH_VS) break;
     case GH_SV: GH_LAUNCH_MODE(GH_SV) break;
     default:
-      hipLaunchKernelGGL((k_bin_scalar<FN, T, GH_SS>), dim3(1), dim3(kBlock), 0, ctx->stream, A, B, n);
+      hipLaunchKernelGGL((k_bin_scalar<FN, T, GH_SS>), dim3(1), dim3(kBlock), 0, ctx->stream, A, B, Dst, n);
   }
 #undef GH_LAUNCH_MODE
   return gh_check_hip(ctx, hipGetLastError(), "elementwise binary launch");
@@ -408,16 +413,18 @@ int launch_bin(gh_ctx* ctx, const gh_cmd& c) {
 
 template <int FN, class T>
 int launch_unary_fn(gh_ctx* ctx, const gh_cmd& c) {
-  T* A = (T*)(uintptr_t)c.ptr[0];
+  const T* A = (const T*)(uintptr_t)c.ptr[0];
+  const uint64_t dptr = c.ptr[1] ? c.ptr[1] : c.ptr[0];  // optional separate destination
+  T* Dst = (T*)(uintptr_t)dptr;
   const int64_t n = c.dim[0];
   constexpr int N = VecOf<T>::N;
   if (n == 0) return GH_OK;
-  if (n >= N && aligned16(c.ptr[0]))
+  if (n >= N && aligned16(c.ptr[0]) && aligned16(dptr))
     hipLaunchKernelGGL((k_unary_vec<FN, T>), dim3(grid_for(ctx, n / N + N, kUnroll)), dim3(kBlock), 0,
-                       ctx->stream, A, n);
+                       ctx->stream, A, Dst, n);
   else
     hipLaunchKernelGGL((k_unary_scalar<FN, T>), dim3(grid_for(ctx, n, 4)), dim3(kBlock), 0,
-                       ctx->stream, A, n);
+                       ctx->stream, A, Dst, n);
   return gh_check_hip(ctx, hipGetLastError(), "elementwise unary launch");
 }
 

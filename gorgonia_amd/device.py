@@ -142,14 +142,14 @@ class Context:
 
 # ---- command builders -------------------------------------------------------------
 
-def cmd_bin(fn, mode, a, b, n, dtype=_ffi.F32):
+def cmd_bin(fn, mode, a, b, n, dtype=_ffi.F32, dst=0):
     fl = _ffi.flag_fn(_ffi.BIN_FN[fn]) | _ffi.flag_mode(_ffi.MODE[mode]) | _ffi.flag_dtype(dtype)
-    return make_cmd(_ffi.OP_ELEM_BIN, fl, (a, b), (n,))
+    return make_cmd(_ffi.OP_ELEM_BIN, fl, (a, b, dst), (n,))
 
 
-def cmd_unary(fn, a, n, dtype=_ffi.F32):
+def cmd_unary(fn, a, n, dtype=_ffi.F32, dst=0):
     fl = _ffi.flag_fn(_ffi.UNARY_FN[fn]) | _ffi.flag_dtype(dtype)
-    return make_cmd(_ffi.OP_ELEM_UNARY, fl, (a,), (n,))
+    return make_cmd(_ffi.OP_ELEM_UNARY, fl, (a, dst), (n,))
 
 
 def cmd_bcast(fn, dst, big, small, outer, mid, inner, small_left=False):

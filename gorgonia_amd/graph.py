@@ -1,0 +1,233 @@
+"""Graph-building API and tape machine, named after the Gorgonia functions they
+stand in for (api_gen.go, operations.go, nn.go, ops/nn/api_cuda.go, vm_tape.go).
+Only what the device path needs: forward graphs of operators that have a
+device implementation.  Nodes are plain handles; all logic is in
+libgorgonia_host.so."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _ffi
+from .engine import Engine, EngineError, GhhOp, load_host
+
+(K_ELEMBIN, K_ELEMUNARY, K_BCAST, K_MATMUL, K_MATVEC, K_OUTER, K_BMM, K_CONV2D, K_MAXPOOL, K_BN,
+ K_RECTIFY, K_LEAKY, K_SOFTMAX, K_RESHAPE) = range(14)
+
+
+class Node:
+    def __init__(self, g, nid):
+        self.g, self.id = g, nid
+
+    def Shape(self):
+        return self.g.shape_of(self.id)
+
+
+class ExprGraph:
+    def __init__(self):
+        self.lib = load_host()
+        self.h = self.lib.ghh_graph_new()
+        self._keep = []  # host arrays bound to nodes must outlive the graph
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.lib.ghh_graph_destroy(self.h)
+            self.h = None
+
+    def _check(self, rc):
+        if rc != 0:
+            raise EngineError(rc, self.lib.ghh_graph_last_error(self.h).decode(errors="replace"))
+
+    def shape_of(self, nid):
+        buf = (C.c_int64 * 8)()
+        n = self.lib.ghh_graph_node_shape(self.h, nid, buf, 8)
+        return tuple(buf[i] for i in range(n))
+
+    def apply(self, kind, inputs, fn=0, name="", trans_a=False, trans_b=False, ints=(), f0=0.0):
+        op = GhhOp()
+        op.kind, op.fn, op.name = kind, fn, name.encode()
+        op.trans_a, op.trans_b = int(trans_a), int(trans_b)
+        op.n_ints = len(ints)
+        for i, v in enumerate(ints):
+            op.ints[i] = int(v)
+        op.f0 = float(f0)
+        arr = (C.c_int * len(inputs))(*[n.id for n in inputs])
+        out = C.c_int()
+        self._check(self.lib.ghh_graph_apply(self.h, C.byref(op), arr, len(inputs), C.byref(out)))
+        return Node(self, out.value)
+
+
+def NewGraph():
+    return ExprGraph()
+
+
+def NewTensor(g, value, resident=False):
+    """NewTensor(g, dt, dims, WithShape(...), WithValue(value)): an input node
+    bound to a host array.  resident=True keeps it on the device across runs
+    (weights); the reference re-uploads every input on every run."""
+    value = np.asarray(value)
+    if value.ndim:  # ascontiguousarray would turn a 0-d scalar into shape (1,)
+        value = np.ascontiguousarray(value)
+    g._keep.append(value)
+    shp = (C.c_int64 * max(value.ndim, 1))(*value.shape)
+    dt = {np.dtype(np.float32): 0, np.dtype(np.float64): 1}.get(value.dtype, 2)
+    nid = g.lib.ghh_graph_new_tensor(g.h, shp, value.ndim, dt, value.ctypes.data_as(C.c_void_p),
+                                     int(resident))
+    return Node(g, nid)
+
+
+def NewScalar(g, value, dtype=np.float32, resident=True):
+    return NewTensor(g, np.array(value, dtype=dtype), resident)
+
+
+def Let(node, value):
+    value = np.ascontiguousarray(value)
+    node.g._keep.append(value)
+    node.g._check(node.g.lib.ghh_graph_let(node.g.h, node.id, value.ctypes.data_as(C.c_void_p)))
+
+
+def Read(node, dtype=np.float32):
+    """gorgonia.Read: returns the host array the value lands in after RunAll."""
+    out = np.empty(node.Shape(), dtype=dtype)
+    node.g._keep.append(out)
+    node.g._check(node.g.lib.ghh_graph_read(node.g.h, node.id, out.ctypes.data_as(C.c_void_p)))
+    return out
+
+
+def _bin(fn):
+    return lambda a, b: a.g.apply(K_ELEMBIN, [a, b], fn=_ffi.BIN_FN[fn])
+
+
+def _un(name):
+    return lambda a: a.g.apply(K_ELEMUNARY, [a], name=name)
+
+
+def _bc(fn):
+    return lambda a, b: a.g.apply(K_BCAST, [a, b], fn=_ffi.BIN_FN[fn])
+
+
+# api_gen.go names
+Add, Sub, HadamardProd, HadamardDiv, Pow = _bin("add"), _bin("sub"), _bin("mul"), _bin("div"), _bin("pow")
+Lt, Lte, Gt, Gte, Eq, Ne = _bin("lt"), _bin("lte"), _bin("gt"), _bin("gte"), _bin("eq"), _bin("ne")
+BroadcastAdd, BroadcastSub = _bc("add"), _bc("sub")
+BroadcastHadamardProd, BroadcastHadamardDiv = _bc("mul"), _bc("div")
+Abs, Sign, Ceil, Floor, Sin, Cos, Exp, Log, Log2 = (_un(n) for n in
+                                                     ("abs", "sign", "ceil", "floor", "sin", "cos", "exp", "ln", "log2"))
+Neg, Square, Sqrt, Inverse, InverseSqrt, Cube = (_un(n) for n in
+                                                 ("neg", "square", "sqrt", "inv", "invSqrt", "cube"))
+Tanh, Sigmoid, Log1p, Expm1, Softplus = (_un(n) for n in ("tanh", "sigmoid", "log1p", "expm1", "softplus"))
+
+
+def Mul(a, b, transA=False, transB=False):
+    """operations.go:52-130: matrix-matrix, matrix-vector or vector-vector (outer) product."""
+    sa, sb = a.Shape(), b.Shape()
+    if len(sa) == 2 and len(sb) == 2:
+        return a.g.apply(K_MATMUL, [a, b], trans_a=transA, trans_b=transB)
+    if len(sa) == 2 and len(sb) == 1:
+        return a.g.apply(K_MATVEC, [a, b], trans_a=transA)
+    if len(sa) == 1 and len(sb) == 1:
+        return a.g.apply(K_OUTER, [a, b])
+    raise EngineError(_ffi.GH_EINVAL, f"Mul: unsupported shapes {sa} x {sb}")
+
+
+def OuterProd(a, b):
+    return a.g.apply(K_OUTER, [a, b])
+
+
+def BatchedMatMul(a, b, transA=False, transB=False):
+    return a.g.apply(K_BMM, [a, b], trans_a=transA, trans_b=transB)
+
+
+def Conv2d(im, filter, kernelShape, pad=None, stride=(1, 1), dilation=None):
+    """nnops.Conv2d (ops/nn/api_cuda.go:10-16; nn.go:211-305)."""
+    pad = (0, 0) if pad is None else pad
+    dilation = (1, 1) if dilation is None else dilation
+    return im.g.apply(K_CONV2D, [im, filter], ints=list(kernelShape) + list(pad) + list(stride) + list(dilation))
+
+
+def MaxPool2D(x, kernel, pad, stride):
+    """nnops.MaxPool2D (nn.go:322-375): pad has 2 values (symmetric) or 4 (N, S, W, E)."""
+    return x.g.apply(K_MAXPOOL, [x], ints=list(kernel) + [len(pad)] + list(pad) + list(stride))
+
+
+def BatchNorm(x, scale, bias, runningMean, runningVariance, epsilon=1e-5):
+    """nnops.BatchNorm in EvalMode with SetStats(runningMean, runningVariance)
+    (nn.go:386-441, op_nn.go:1286-1313): y = scale * ((x - mean)/sqrt(var + eps)) + bias."""
+    ins = [x, runningMean, runningVariance] + ([scale, bias] if scale is not None else [])
+    return x.g.apply(K_BN, ins, f0=epsilon)
+
+
+def Rectify(x):
+    return x.g.apply(K_RECTIFY, [x])
+
+
+def LeakyRelu(x, alpha):
+    return x.g.apply(K_LEAKY, [x], f0=alpha)
+
+
+def SoftMax(x):
+    return x.g.apply(K_SOFTMAX, [x])
+
+
+def Reshape(x, shape):
+    return x.g.apply(K_RESHAPE, [x], ints=list(shape))
+
+
+class TapeMachine:
+    """NewTapeMachine(g, ...) / RunAll / Reset / Close (vm_tape.go:45-249)."""
+
+    def __init__(self, g, graph_replay=False, reupload_resident=False, fuse_activations=False,
+                 device=0, compile_only=False):
+        self.g = g
+        self.lib = g.lib
+        self.fused = self.lib.ghh_graph_fuse_activations(g.h) if fuse_activations else 0
+        self.h = self.lib.ghh_tape_new(g.h, int(graph_replay), int(reupload_resident))
+        if compile_only:
+            self._check(self.lib.ghh_tape_compile_only(self.h))
+        else:
+            self._check(self.lib.ghh_tape_init(self.h, device))
+
+    def _check(self, rc):
+        if rc != 0:
+            raise EngineError(rc, self.lib.ghh_tape_last_error(self.h).decode(errors="replace"))
+
+    def RunAll(self):
+        self._check(self.lib.ghh_tape_run_all(self.h))
+
+    def Reset(self):
+        self._check(self.lib.ghh_tape_reset(self.h))
+
+    def Close(self):
+        if self.h:
+            self.lib.ghh_tape_close(self.h)
+            self.lib.ghh_tape_destroy(self.h)
+            self.h = None
+
+    def engine(self):
+        return Engine(self.lib.ghh_tape_engine(self.h))
+
+    def gpumem(self):
+        return self.lib.ghh_tape_gpumem(self.h)
+
+    def segments(self):
+        return self.lib.ghh_tape_segments(self.h)
+
+    def graph_launches(self):
+        return self.lib.ghh_tape_graph_launches(self.h)
+
+    def submit_calls(self):
+        return self.lib.ghh_tape_submit_calls(self.h)
+
+    def register_address(self, node):
+        return self.lib.ghh_tape_register_address(self.h, node.id)
+
+    def program(self):
+        n = self.lib.ghh_tape_program_string(self.h, None, 0)
+        buf = C.create_string_buffer(n + 1)
+        self.lib.ghh_tape_program_string(self.h, buf, n + 1)
+        return buf.value.decode()
+
+
+def NewTapeMachine(g, **kw):
+    return TapeMachine(g, **kw)

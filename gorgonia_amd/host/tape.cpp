@@ -1,0 +1,634 @@
+#include "tape.hpp"
+
+#include <algorithm>
+#include <cstring>
+#include <sstream>
+
+namespace gorgonia {
+
+static Status bad(const std::string& m) { return Status::Err(GH_EINVAL, m); }
+
+static int64_t conv_out(int64_t in, int64_t k, int64_t pad, int64_t stride, int64_t dil) {
+  return (in + 2 * pad - (dil * (k - 1) + 1)) / stride + 1;  // op_nn.go:311-315
+}
+static int64_t pool_out(int64_t in, int64_t k, int64_t pa, int64_t pb, int64_t stride) {
+  return (in + pa + pb - (k - 1) - 1) / stride + 1;  // op_nn.go:810-816
+}
+
+// Broadcast decomposition: the small operand has size-1 dims everywhere except
+// one contiguous run of axes, which must match the big operand.
+static bool bcast_decompose(const Shape& big, const Shape& small, int64_t* outer, int64_t* mid,
+                            int64_t* inner) {
+  if (big.Dims() != small.Dims()) return false;
+  int first = -1, last = -1;
+  for (int i = 0; i < big.Dims(); i++) {
+    if (small[i] == big[i] && big[i] != 1) { if (first < 0) first = i; last = i; }
+    else if (small[i] != 1) return false;
+  }
+  if (first < 0) { *outer = big.TotalSize(); *mid = 1; *inner = 1; return true; }
+  for (int i = first; i <= last; i++) if (small[i] != big[i]) return false;
+  *outer = *mid = *inner = 1;
+  for (int i = 0; i < first; i++) *outer *= big[i];
+  for (int i = first; i <= last; i++) *mid *= big[i];
+  for (int i = last + 1; i < big.Dims(); i++) *inner *= big[i];
+  return true;
+}
+
+Status InferShape(const OpSpec& op, const std::vector<const Shape*>& in, Shape* out) {
+  auto need = [&](size_t n) { return in.size() == n; };
+  switch (op.kind) {
+    case OpKind::ElemBin:
+      if (!need(2)) return bad("binary op needs 2 inputs");
+      if (in[0]->IsScalar()) { *out = *in[1]; return Status::OK(); }
+      if (in[1]->IsScalar()) { *out = *in[0]; return Status::OK(); }
+      if (!in[0]->Eq(*in[1]))
+        return bad("Shape mismatch. Expected " + in[0]->String() + ". Got " + in[1]->String());
+      *out = *in[0];
+      return Status::OK();
+    case OpKind::ElemUnary:
+    case OpKind::Rectify:
+    case OpKind::LeakyRelu:
+      if (!need(1)) return bad("unary op needs 1 input");
+      *out = *in[0];
+      return Status::OK();
+    case OpKind::BroadcastBin: {
+      if (!need(2)) return bad("broadcast op needs 2 inputs");
+      int64_t o, m, i;
+      const bool left_small = in[0]->TotalSize() < in[1]->TotalSize();
+      const Shape& big = left_small ? *in[1] : *in[0];
+      const Shape& small = left_small ? *in[0] : *in[1];
+      if (!bcast_decompose(big, small, &o, &m, &i))
+        return bad("cannot broadcast " + small.String() + " to " + big.String());
+      *out = big;
+      return Status::OK();
+    }
+    case OpKind::MatMul: {
+      if (!need(2) || in[0]->Dims() != 2 || in[1]->Dims() != 2) return bad("MatMul needs two matrices");
+      const int64_t m = op.transA ? (*in[0])[1] : (*in[0])[0], k = op.transA ? (*in[0])[0] : (*in[0])[1];
+      const int64_t kb = op.transB ? (*in[1])[1] : (*in[1])[0], n = op.transB ? (*in[1])[0] : (*in[1])[1];
+      if (k != kb) return bad("MatMul: inner dimensions differ");
+      *out = Shape{m, n};
+      return Status::OK();
+    }
+    case OpKind::MatVecMul: {
+      if (!need(2) || in[0]->Dims() != 2 || in[1]->Dims() != 1) return bad("MatVecMul needs a matrix and a vector");
+      const int64_t m = op.transA ? (*in[0])[1] : (*in[0])[0], n = op.transA ? (*in[0])[0] : (*in[0])[1];
+      if ((*in[1])[0] != n) return bad("MatVecMul: dimension mismatch");
+      *out = Shape{m};
+      return Status::OK();
+    }
+    case OpKind::Outer:
+      if (!need(2) || in[0]->Dims() != 1 || in[1]->Dims() != 1) return bad("Outer needs two vectors");
+      *out = Shape{(*in[0])[0], (*in[1])[0]};
+      return Status::OK();
+    case OpKind::BatchedMatMul: {
+      if (!need(2) || in[0]->Dims() < 3 || in[0]->Dims() != in[1]->Dims()) return bad("BatchedMatMul needs equal rank >= 3");
+      const int d = in[0]->Dims();
+      std::vector<int64_t> o(in[0]->d.begin(), in[0]->d.end() - 2);
+      const int64_t ar = (*in[0])[d - 2], ac = (*in[0])[d - 1], br = (*in[1])[d - 2], bc = (*in[1])[d - 1];
+      const int64_t m = op.transA ? ac : ar, k = op.transA ? ar : ac, kb = op.transB ? bc : br,
+                    n = op.transB ? br : bc;
+      if (k != kb) return bad("BatchedMatMul: inner dimensions differ");
+      o.push_back(m); o.push_back(n);
+      *out = Shape(o);
+      return Status::OK();
+    }
+    case OpKind::Conv2d: {
+      if (!need(2)) return bad("Conv2d needs image and filter");
+      if (in[0]->Dims() != 4) return bad("im should have 4 dims, got " + std::to_string(in[0]->Dims()) + " dims");
+      if (in[1]->Dims() != 4) return bad("filter should have 4 dims, got " + std::to_string(in[1]->Dims()) + " dims");
+      if (op.ints.size() != 8) return bad("Conv2d needs kernel, pad, stride, dilation");
+      const auto& p = op.ints;
+      if (p[4] <= 0 || p[5] <= 0) return bad("Cannot use strides of less than or equal 0");
+      if (p[2] < 0 || p[3] < 0) return bad("Cannot use padding of less than 0");
+      if (p[6] <= 0 || p[7] <= 0) return bad("Cannot use dilation less than or eq 0");
+      if ((*in[1])[1] != (*in[0])[1] || (*in[1])[2] != p[0] || (*in[1])[3] != p[1])
+        return bad("filter shape " + in[1]->String() + " does not fit image " + in[0]->String());
+      const int64_t oh = conv_out((*in[0])[2], p[0], p[2], p[4], p[6]);
+      const int64_t ow = conv_out((*in[0])[3], p[1], p[3], p[5], p[7]);
+      if (oh <= 0 || ow <= 0) return bad("Conv2d: empty output");
+      *out = Shape{(*in[0])[0], (*in[1])[0], oh, ow};
+      return Status::OK();
+    }
+    case OpKind::MaxPool2D: {
+      if (!need(1)) return bad("MaxPool2D needs 1 input");
+      if (in[0]->Dims() != 4) return bad("Expected input to have a shape with dimension 4");
+      const auto& p = op.ints;  // kh kw npad pads... sh sw
+      if (p.size() < 3 || (p[2] != 2 && p[2] != 4) || (int64_t)p.size() != 3 + p[2] + 2)
+        return bad("MaxPool2D needs kernel, 2 or 4 pads, stride");
+      const int64_t np = p[2];
+      const int64_t pn = p[3], ps = np == 4 ? p[4] : p[3], pw = np == 4 ? p[5] : p[4], pe = np == 4 ? p[6] : p[4];
+      const int64_t sh = p[3 + np], sw = p[4 + np];
+      if (sh <= 0 || sw <= 0) return bad("Cannot use strides of less than or equal 0");
+      for (int64_t i = 0; i < np; i++) if (p[3 + i] < 0) return bad("Cannot use padding of less than 0");
+      if ((*in[0])[2] - p[0] + pn + ps < 0) return bad("Impossible height/kernel/pad combination");
+      if ((*in[0])[3] - p[1] + pw + pe < 0) return bad("Impossible width/kernel/pad combination");
+      *out = Shape{(*in[0])[0], (*in[0])[1], pool_out((*in[0])[2], p[0], pn, ps, sh),
+                   pool_out((*in[0])[3], p[1], pw, pe, sw)};
+      return Status::OK();
+    }
+    case OpKind::BatchNorm: {
+      if (in.size() != 3 && in.size() != 5) return bad("BatchNorm needs x, mean, var[, scale, bias]");
+      if (in[0]->Dims() != 2 && in[0]->Dims() != 4) return bad("BatchNorm input must be (B, N) or (B, C, H, W)");
+      const int64_t C = (*in[0])[1];
+      for (size_t i = 1; i < in.size(); i++)
+        if (in[i]->TotalSize() != C)
+          return bad("invalid runningMean shape " + in[i]->String() + ". Expected: (" + std::to_string(C) + ")");
+      *out = *in[0];
+      return Status::OK();
+    }
+    case OpKind::SoftMax:
+      if (!need(1) || in[0]->IsScalar()) return bad("SoftMax needs a tensor");
+      *out = *in[0];
+      return Status::OK();
+    case OpKind::Reshape: {
+      if (!need(1)) return bad("Reshape needs 1 input");
+      Shape s(op.ints);
+      if (s.TotalSize() != in[0]->TotalSize()) return bad("Reshape: size mismatch " + in[0]->String() + " -> " + s.String());
+      *out = s;
+      return Status::OK();
+    }
+  }
+  return bad("unknown op");
+}
+
+int OverwritesInput(const OpSpec& op) {
+  // elementwise ops may overwrite their tensor argument (op_math.go:285-294,
+  // 476-481); everything else writes a fresh value
+  if (op.kind == OpKind::ElemUnary) return 0;
+  if (op.kind == OpKind::ElemBin) return 0;
+  return -1;
+}
+
+static std::string op_name(const OpSpec& op) {
+  static const char* bins[] = {"add", "sub", "mul", "div", "pow", "lt", "lte", "gt", "gte", "eq", "ne"};
+  switch (op.kind) {
+    case OpKind::ElemBin: return std::string("elembin.") + bins[op.fn];
+    case OpKind::ElemUnary: return "elemunary." + op.name;
+    case OpKind::BroadcastBin: return std::string("broadcast.") + bins[op.fn];
+    case OpKind::MatMul: return "matmul";
+    case OpKind::MatVecMul: return "matvecmul";
+    case OpKind::Outer: return "outer";
+    case OpKind::BatchedMatMul: return "batchedmatmul";
+    case OpKind::Conv2d: return op.fuse_act_relu ? "conv2d+rectify" : op.fuse_act_leaky ? "conv2d+leakyrelu" : "conv2d";
+    case OpKind::MaxPool2D: return "maxpool2d";
+    case OpKind::BatchNorm: return "batchnorm(eval)";
+    case OpKind::Rectify: return "rectify";
+    case OpKind::LeakyRelu: return "leakyrelu";
+    case OpKind::SoftMax: return "softmax";
+    case OpKind::Reshape: return "reshape";
+  }
+  return "?";
+}
+
+Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<Tensor*>& in) {
+  switch (op.kind) {
+    case OpKind::ElemBin: {
+      Tensor& a = *in[0];
+      Tensor& b = *in[1];
+      static const char* names[] = {"Add", "Sub", "Mul", "Div", "Pow", "Lt", "Lte", "Gt", "Gte", "ElEq", "ElNe"};
+      const bool as = a.shape.IsScalar(), bs = b.shape.IsScalar();
+      if (as != bs) {  // tensor-scalar: the *Scalar methods (operatorPointwise_binary.go:359-426)
+        Tensor& t = as ? b : a;
+        Tensor& s = as ? a : b;
+        FuncOpts o = prealloc.mem == t.mem ? FuncOpts::UseUnsafe() : FuncOpts::WithReuse(&prealloc);
+        return e.BinOpScalar(op.fn, names[op.fn], t, s.mem, /*leftTensor=*/!as, o, nullptr);
+      }
+      FuncOpts o = prealloc.mem == a.mem ? FuncOpts::UseUnsafe() : FuncOpts::WithReuse(&prealloc);
+      return e.BinOp(op.fn, names[op.fn], a, b, o, nullptr);
+    }
+    case OpKind::ElemUnary:
+      return e.UnaryTo(op.name, *in[0], prealloc.mem);
+    case OpKind::BroadcastBin: {
+      const bool left_small = in[0]->shape.TotalSize() < in[1]->shape.TotalSize();
+      Tensor& big = left_small ? *in[1] : *in[0];
+      Tensor& small = left_small ? *in[0] : *in[1];
+      int64_t o, m, i;
+      if (!bcast_decompose(big.shape, small.shape, &o, &m, &i)) return bad("cannot broadcast");
+      return e.BroadcastBinOp(op.fn, big, small, o, m, i, left_small, prealloc.mem);
+    }
+    case OpKind::MatMul: {
+      // op.transA/transB are applied as transposed views (op_math_cuda.go:210-224)
+      Tensor a = *in[0], b = *in[1];
+      if (op.transA) { std::swap(a.shape.d[0], a.shape.d[1]); a.transposed = !a.transposed; }
+      if (op.transB) { std::swap(b.shape.d[0], b.shape.d[1]); b.transposed = !b.transposed; }
+      const int act = op.fuse_act_relu ? 1 : op.fuse_act_leaky ? 2 : 0;
+      return e.MatMul(a, b, prealloc, act, (float)op.f0);
+    }
+    case OpKind::MatVecMul: {
+      Tensor a = *in[0];
+      if (op.transA) { std::swap(a.shape.d[0], a.shape.d[1]); a.transposed = !a.transposed; }
+      return e.MatVecMul(a, *in[1], prealloc);
+    }
+    case OpKind::Outer:
+      return e.Outer(*in[0], *in[1], prealloc);
+    case OpKind::BatchedMatMul:
+      return e.BatchedMatMul(*in[0], *in[1], prealloc, op.transA, op.transB);
+    case OpKind::Conv2d: {
+      const Tensor& x = *in[0];
+      const Tensor& w = *in[1];
+      if (x.dt != Dtype::Float32) return bad("Conv2d: Unsupported Dtype");
+      gh_cmd c{};
+      c.opcode = GH_OP_CONV2D;
+      c.flags = op.fuse_act_relu ? GH_FLAG_ACT_RELU : op.fuse_act_leaky ? GH_FLAG_ACT_LEAKY : 0;
+      c.f[0] = (float)op.f0;
+      c.ptr[0] = x.mem; c.ptr[1] = w.mem; c.ptr[2] = prealloc.mem;
+      for (int i = 0; i < 4; i++) c.dim[i] = x.shape[i];
+      c.dim[4] = w.shape[0];
+      for (int i = 0; i < 8; i++) c.dim[5 + i] = op.ints[(size_t)i];
+      e.Enqueue(c);
+      return Status::OK();
+    }
+    case OpKind::MaxPool2D: {
+      const Tensor& x = *in[0];
+      if (x.dt != Dtype::Float32) return bad("MaxPool2D: Unsupported Dtype");
+      const auto& p = op.ints;
+      const int64_t np = p[2];
+      gh_cmd c{};
+      c.opcode = GH_OP_MAXPOOL2D;
+      c.flags = np == 4 ? GH_FLAG_EXPLICIT_PAD : 0;
+      c.ptr[0] = x.mem; c.ptr[1] = prealloc.mem;
+      for (int i = 0; i < 4; i++) c.dim[i] = x.shape[i];
+      c.dim[4] = p[0]; c.dim[5] = p[1];
+      if (np == 4) { c.dim[6] = p[3]; c.dim[7] = p[4]; c.dim[8] = p[5]; c.dim[9] = p[6]; }
+      else { c.dim[6] = c.dim[7] = p[3]; c.dim[8] = c.dim[9] = p[4]; }
+      c.dim[10] = p[3 + np]; c.dim[11] = p[4 + np];
+      e.Enqueue(c);
+      return Status::OK();
+    }
+    case OpKind::BatchNorm: {
+      const Tensor& x = *in[0];
+      if (x.dt != Dtype::Float32) return bad("BatchNorm: Unsupported Dtype");
+      gh_cmd c{};
+      c.opcode = GH_OP_BN_INFER;
+      c.ptr[0] = x.mem; c.ptr[1] = prealloc.mem; c.ptr[2] = in[1]->mem; c.ptr[3] = in[2]->mem;
+      if (in.size() == 5) {
+        c.flags = GH_FLAG_HAS_GAMMA | GH_FLAG_HAS_BETA;
+        c.ptr[4] = in[3]->mem; c.ptr[5] = in[4]->mem;
+      }
+      const int64_t B = x.shape[0], C = x.shape[1];
+      c.dim[0] = B; c.dim[1] = C; c.dim[2] = x.shape.TotalSize() / (B * C);
+      c.f[0] = (float)op.f0;
+      e.Enqueue(c);
+      return Status::OK();
+    }
+    case OpKind::Rectify:
+    case OpKind::LeakyRelu: {
+      gh_cmd c{};
+      c.opcode = op.kind == OpKind::Rectify ? GH_OP_RELU : GH_OP_LEAKY_RELU;
+      c.ptr[0] = in[0]->mem; c.ptr[1] = prealloc.mem;
+      c.dim[0] = in[0]->DataSize();
+      c.f[0] = (float)op.f0;
+      e.Enqueue(c);
+      return Status::OK();
+    }
+    case OpKind::SoftMax: {
+      const Tensor& x = *in[0];
+      gh_cmd c{};
+      c.opcode = GH_OP_SOFTMAX;
+      c.ptr[0] = x.mem; c.ptr[1] = prealloc.mem;
+      const int64_t cols = x.shape[x.shape.Dims() - 1];
+      c.dim[0] = x.shape.TotalSize() / cols; c.dim[1] = cols;
+      e.Enqueue(c);
+      return Status::OK();
+    }
+    case OpKind::Reshape:
+      return Status::OK();  // metadata only (op_tensor.go:1226-1246)
+  }
+  return bad("unknown op");
+}
+
+// ---- Graph ------------------------------------------------------------------------
+
+int Graph::NewTensor(const Shape& s, Dtype dt, const void* host, bool resident) {
+  Node n;
+  n.id = (int)nodes_.size();
+  n.shape = s; n.dt = dt; n.is_input = true; n.host = host; n.resident = resident;
+  nodes_.push_back(n);
+  return n.id;
+}
+
+Status Graph::Apply(const OpSpec& op, const std::vector<int>& inputs, int* out) {
+  std::vector<const Shape*> shapes;
+  for (int i : inputs) {
+    if (i < 0 || i >= (int)nodes_.size()) return bad("Apply: unknown input node");
+    shapes.push_back(&nodes_[(size_t)i].shape);
+  }
+  Node n;
+  Status st = InferShape(op, shapes, &n.shape);
+  if (!st.ok()) return st;
+  n.id = (int)nodes_.size();
+  n.dt = inputs.empty() ? Dtype::Float32 : nodes_[(size_t)inputs[0]].dt;
+  n.op = op;
+  n.inputs = inputs;
+  if (op.kind == OpKind::Reshape) n.alias_of = inputs[0];
+  nodes_.push_back(n);
+  if (out) *out = n.id;
+  return Status::OK();
+}
+
+Status Graph::Let(int node, const void* host) {
+  if (node < 0 || node >= (int)nodes_.size() || !nodes_[(size_t)node].is_input) return bad("Let: not an input node");
+  nodes_[(size_t)node].host = host;
+  return Status::OK();
+}
+
+Status Graph::Read(int node, void* host_out) {
+  if (node < 0 || node >= (int)nodes_.size()) return bad("Read: unknown node");
+  nodes_[(size_t)node].read_into = host_out;
+  return Status::OK();
+}
+
+int Graph::FuseActivations() {
+  int fused = 0;
+  std::vector<int> uses(nodes_.size(), 0);
+  for (auto& n : nodes_) for (int i : n.inputs) uses[(size_t)i]++;
+  for (auto& n : nodes_) {
+    if (n.is_input || n.fused_away) continue;
+    if (n.op.kind != OpKind::Rectify && n.op.kind != OpKind::LeakyRelu) continue;
+    Node& p = nodes_[(size_t)n.inputs[0]];
+    if (p.is_input || p.read_into || uses[(size_t)p.id] != 1) continue;
+    if (p.op.kind != OpKind::Conv2d && p.op.kind != OpKind::MatMul) continue;
+    if (p.op.fuse_act_relu || p.op.fuse_act_leaky) continue;
+    if (n.op.kind == OpKind::Rectify) p.op.fuse_act_relu = true;
+    else { p.op.fuse_act_leaky = true; p.op.f0 = n.op.f0; }
+    n.fused_away = true;
+    n.alias_of = p.id;
+    fused++;
+  }
+  return fused;
+}
+
+// ---- TapeMachine --------------------------------------------------------------------
+
+TapeMachine::~TapeMachine() { Close(); }
+
+Status TapeMachine::Compile() {
+  auto& nodes = g_->Nodes();
+  const int N = (int)nodes.size();
+  prog_.clear();
+  auto bytes_of = [&](const Node& n) {
+    return (n.shape.IsScalar() ? 1 : n.shape.TotalSize()) * dtype_size(n.dt);
+  };
+  // root value of a node: aliases (Reshape, fused activations) are views of it
+  std::vector<int> root((size_t)N);
+  for (int i = 0; i < N; i++) root[(size_t)i] = nodes[(size_t)i].alias_of >= 0 ? root[(size_t)nodes[(size_t)i].alias_of] : i;
+  // last instruction that reads each root value
+  std::vector<int> last_reader((size_t)N, -1);
+  for (int i = 0; i < N; i++)
+    for (int in : nodes[(size_t)i].inputs) last_reader[(size_t)root[(size_t)in]] = i;
+  std::vector<char> value_kept((size_t)N, 0);  // read by the host, or a resident input
+  for (int i = 0; i < N; i++)
+    if (nodes[(size_t)i].read_into || (nodes[(size_t)i].is_input && nodes[(size_t)i].resident))
+      value_kept[(size_t)root[(size_t)i]] = 1;
+
+  // registers: a node that overwrites a dead input takes over that input's
+  // register (regalloc.go:211-243); every other node gets a fresh one
+  node_reg_.assign((size_t)N, -1);
+  std::vector<char> inplace((size_t)N, 0);
+  int nreg = 0;
+  for (int i = 0; i < N; i++) {
+    Node& n = nodes[(size_t)i];
+    if (n.alias_of >= 0) { node_reg_[(size_t)i] = node_reg_[(size_t)root[(size_t)i]]; continue; }
+    const int ow = n.is_input ? -1 : OverwritesInput(n.op);
+    if (ow >= 0 && ow < (int)n.inputs.size()) {
+      int src = n.inputs[(size_t)ow];
+      if (n.op.kind == OpKind::ElemBin && n.inputs.size() == 2 && nodes[(size_t)src].shape.IsScalar())
+        src = n.inputs[1];  // scalar (op) tensor: the tensor operand is the one overwritten
+      const int rs = root[(size_t)src];
+      if (last_reader[(size_t)rs] == i && !value_kept[(size_t)rs] && bytes_of(nodes[(size_t)src]) == bytes_of(n)) {
+        node_reg_[(size_t)i] = node_reg_[(size_t)rs];
+        inplace[(size_t)i] = 1;
+        continue;
+      }
+    }
+    node_reg_[(size_t)i] = nreg++;
+  }
+  // register liveness: last instruction touching any value held in it
+  std::vector<int> reg_last((size_t)nreg, -1);
+  std::vector<char> reg_kept((size_t)nreg, 0);
+  for (int i = 0; i < N; i++) {
+    const int r = node_reg_[(size_t)i];
+    reg_last[(size_t)r] = std::max(reg_last[(size_t)r], std::max(i, last_reader[(size_t)root[(size_t)i]]));
+    if (value_kept[(size_t)root[(size_t)i]]) reg_kept[(size_t)r] = 1;
+  }
+  regs_.assign((size_t)nreg, Tensor());
+  reg_live_.assign((size_t)nreg, 0);
+  resident_done_.assign((size_t)N, 0);
+  std::vector<int64_t> reg_bytes((size_t)nreg, 0);
+  gpumem_ = 0;
+
+  for (int i = 0; i < N; i++) {
+    Node& n = nodes[(size_t)i];
+    if (n.alias_of >= 0) continue;
+    const int r = node_reg_[(size_t)i];
+    const int64_t bytes = bytes_of(n);
+    if (n.is_input) {
+      prog_.push_back({InstrKind::LoadArg, i, r, bytes, false});
+      prog_.push_back({InstrKind::Alloc, i, r, bytes, false});
+      prog_.push_back({InstrKind::Transport, i, r, bytes, false});
+      reg_bytes[(size_t)r] = bytes;
+      gpumem_ += bytes;
+    } else {
+      if (!inplace[(size_t)i]) {
+        prog_.push_back({InstrKind::Alloc, i, r, bytes, false});
+        reg_bytes[(size_t)r] = bytes;
+        gpumem_ += bytes;
+      }
+      prog_.push_back({InstrKind::ExecOp, i, r, bytes, inplace[(size_t)i] != 0});
+    }
+    // registers whose last use is this instruction die here
+    for (int q = 0; q < nreg; q++)
+      if (reg_last[(size_t)q] == i && !reg_kept[(size_t)q] && reg_bytes[(size_t)q] > 0)
+        prog_.push_back({InstrKind::Free, i, q, reg_bytes[(size_t)q], false});
+  }
+  // host reads: one flush, then the copies (compile.go:437-462 puts a flush in
+  // front of every consumer that needs a finished value)
+  prog_.push_back({InstrKind::Flush, -1, -1, 0, false});
+  std::vector<int> freed;
+  for (int i = 0; i < N; i++)
+    if (nodes[(size_t)i].read_into)
+      prog_.push_back({InstrKind::Read, i, node_reg_[(size_t)i], bytes_of(nodes[(size_t)i]), false});
+  for (int i = 0; i < N; i++) {
+    Node& n = nodes[(size_t)i];
+    const int r = node_reg_[(size_t)i];
+    if (!n.read_into) continue;
+    bool resident_reg = false;
+    for (int j = 0; j < N; j++)
+      if (node_reg_[(size_t)j] == r && nodes[(size_t)j].is_input && nodes[(size_t)j].resident) resident_reg = true;
+    if (resident_reg || std::find(freed.begin(), freed.end(), r) != freed.end()) continue;
+    prog_.push_back({InstrKind::Free, i, r, reg_bytes[(size_t)r], false});
+    freed.push_back(r);
+  }
+  return Status::OK();
+}
+
+Status TapeMachine::Init(int device) {
+  Status st = Compile();
+  if (!st.ok()) return st;
+  // every register is 32-byte aligned in the arena: size the reservation on
+  // aligned sizes so that "2.5x the program's need" still holds for many small
+  // tensors (the reference sums raw sizes, compile.go:148-216)
+  int64_t need = 0;
+  for (auto& in : prog_)
+    if (in.kind == InstrKind::Alloc) need += (in.size + 31) / 32 * 32;
+  return eng_.Init(device, need > gpumem_ ? need : gpumem_);
+}
+
+uint64_t TapeMachine::RegisterAddress(int node) const {
+  if (node < 0 || node >= (int)node_reg_.size()) return 0;
+  return regs_[(size_t)node_reg_[(size_t)node]].mem;
+}
+
+Status TapeMachine::flush() {
+  segments_++;
+  if (!opt_.graph_replay) return eng_.DoWork();
+  const size_t idx = (size_t)seg_index_++;
+  if (seg_cache_.size() <= idx) seg_cache_.resize(idx + 1);
+  SegCache& sc = seg_cache_[idx];
+  const std::vector<gh_cmd>& cur = eng_.Segment();
+  const bool same = sc.cmds.size() == cur.size() &&
+                    (cur.empty() || std::memcmp(sc.cmds.data(), cur.data(), cur.size() * sizeof(gh_cmd)) == 0);
+  if (cur.empty()) return eng_.Sync();
+  if (sc.graph_id >= 0 && same) {
+    eng_.DropSegment();
+    Status st = eng_.GraphLaunch(sc.graph_id);
+    if (!st.ok()) return st;
+    graph_launches_++;
+    return eng_.Sync();
+  }
+  if (same && runs_ >= 1) {
+    // second identical run of this segment: capture it, then launch the capture
+    Status st = eng_.GraphBegin();
+    if (!st.ok()) return st;
+    st = eng_.SubmitPending();
+    int id = -1;
+    Status st2 = eng_.GraphEnd(&id);
+    if (!st.ok()) return st;
+    if (!st2.ok()) return st2;
+    sc.graph_id = id;
+    st = eng_.GraphLaunch(id);
+    if (!st.ok()) return st;
+    graph_launches_++;
+    return eng_.Sync();
+  }
+  sc.cmds = cur;  // first sight (or the pointer set changed): run eagerly, remember
+  sc.graph_id = -1;
+  return eng_.DoWork();
+}
+
+Status TapeMachine::RunAll() {
+  if (!eng_.Initialized()) return Status::Err(GH_ESTATE, "tape machine not initialised");
+  auto& nodes = g_->Nodes();
+  segments_ = 0;
+  seg_index_ = 0;
+  for (size_t pc = 0; pc < prog_.size(); pc++) {
+    const Instr& in = prog_[pc];
+    Status st;
+    switch (in.kind) {
+      case InstrKind::LoadArg:
+        if (!nodes[(size_t)in.node].host)
+          return Status::Err(GH_EINVAL, "PC " + std::to_string(pc) + ": input node " +
+                                            std::to_string(in.node) + " has no value bound");
+        break;
+      case InstrKind::Alloc:
+        if (!reg_live_[(size_t)in.reg]) {  // skipped when the register still holds a value (vm_tape.go:594-597)
+          uint64_t mem = 0;
+          st = eng_.Get(in.size, &mem);
+          if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": alloc");
+          regs_[(size_t)in.reg].mem = mem;
+          reg_live_[(size_t)in.reg] = 1;
+        }
+        break;
+      case InstrKind::Transport: {
+        Node& n = nodes[(size_t)in.node];
+        if (n.resident && resident_done_[(size_t)in.node] && !opt_.reupload_resident) break;
+        st = eng_.MemcpyHtoD(regs_[(size_t)in.reg].mem, n.host, in.size);
+        if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": devTrans");
+        resident_done_[(size_t)in.node] = 1;
+        break;
+      }
+      case InstrKind::ExecOp: {
+        Node& n = nodes[(size_t)in.node];
+        Tensor out;
+        out.mem = regs_[(size_t)in.reg].mem;
+        out.dt = n.dt;
+        out.shape = n.shape;
+        std::vector<Tensor> ins(n.inputs.size());
+        std::vector<Tensor*> inp(n.inputs.size());
+        for (size_t k = 0; k < n.inputs.size(); k++) {
+          const Node& s = nodes[(size_t)n.inputs[k]];
+          ins[k].mem = regs_[(size_t)node_reg_[(size_t)s.id]].mem;
+          ins[k].dt = s.dt;
+          ins[k].shape = s.shape;
+          inp[k] = &ins[k];
+        }
+        st = CUDADo(eng_, n.op, out, inp);
+        if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": " + op_name(n.op));
+        break;
+      }
+      case InstrKind::Free:
+        if (reg_live_[(size_t)in.reg]) {
+          eng_.Put(regs_[(size_t)in.reg].mem, in.size);
+          reg_live_[(size_t)in.reg] = 0;
+        }
+        break;
+      case InstrKind::Flush:
+        st = flush();
+        if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": flush");
+        break;
+      case InstrKind::Read: {
+        Node& n = nodes[(size_t)in.node];
+        st = eng_.MemcpyDtoH(n.read_into, regs_[(size_t)in.reg].mem, in.size, false);
+        if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": read");
+        bool last = pc + 1 >= prog_.size() || prog_[pc + 1].kind != InstrKind::Read;
+        if (last) {
+          st = eng_.Sync();
+          if (!st.ok()) return st;
+        }
+        break;
+      }
+    }
+  }
+  Status st = eng_.DoWork();  // final DoWork (vm_tape.go:236)
+  runs_++;
+  // Leave the arena in a state that depends only on what is still held
+  // (resident inputs): merge the holes and zero the free/alloc counters, so the
+  // next run's first-fit walk hands out the same addresses again and a captured
+  // segment stays replayable.
+  eng_.Allocator().coalesce();
+  eng_.Allocator().reset_stats();
+  return st;
+}
+
+Status TapeMachine::Reset() {
+  if (!eng_.Initialized()) return Status::OK();
+  eng_.DropSegment();
+  eng_.ResetAllocator();
+  std::fill(reg_live_.begin(), reg_live_.end(), 0);
+  std::fill(resident_done_.begin(), resident_done_.end(), 0);
+  return Status::OK();
+}
+
+Status TapeMachine::Close() { return eng_.Close(); }
+
+std::string TapeMachine::ProgramString() const {
+  static const char* names[] = {"loadArg", "alloc", "devTrans", "execOp", "free", "flush", "read"};
+  std::ostringstream os;
+  os << "Instructions:\n";
+  const auto& nodes = g_->Nodes();
+  for (size_t pc = 0; pc < prog_.size(); pc++) {
+    const Instr& in = prog_[pc];
+    os << pc << "\t" << names[(int)in.kind];
+    if (in.node >= 0) os << " node " << in.node;
+    if (in.reg >= 0) os << " GPU" << in.reg;
+    if (in.kind == InstrKind::ExecOp)
+      os << " " << op_name(nodes[(size_t)in.node].op) << (in.use_unsafe ? " [unsafe]" : " [reuse]");
+    if (in.size) os << " " << in.size << "B";
+    os << "\n";
+  }
+  os << "GPU Memories: " << gpumem_ << "\n";
+  return os.str();
+}
+
+}  // namespace gorgonia

@@ -1,0 +1,147 @@
+// Operators with a device path (the reference's CUDADoer implementers) and a
+// tape machine that runs them in segments.
+//
+// What this mirrors:
+//   - Op::CUDADo(extern, dev, prealloc, inputs...)            op.go:153-155
+//       elemBinOp / elemUnaryOp / linAlgBinOp                 op_math_cuda.go:23-240
+//       reshapeOp (metadata only)                             op_tensor.go:1226-1246
+//       ops/nn convolution, maxpool, BatchNormOp, activation  ops/nn/*_cuda.go
+//   - the tape program: loadArg / alloc / deviceTransport / execOp / free /
+//     flushInstr / readInstr                                  vm_tape.go:584-793
+//   - register reuse only when the overwritten input is dead  regalloc.go:211-243
+//   - flushInstr only where a host read needs a finished value compile.go:437-462
+//   - RunAll / Reset                                          vm_tape.go:123-134,213-249
+//
+// The expression-graph front end (type system, differentiation, CSE) is out of
+// scope; Graph below is the minimum needed to produce the same instruction
+// stream for forward graphs: nodes are appended in topological order, each
+// with an Op and its input nodes.
+#pragma once
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "engine.hpp"
+
+namespace gorgonia {
+
+enum class OpKind : int32_t {
+  ElemBin = 0,      // Add, Sub, HadamardProd, HadamardDiv, Pow, Lt, Lte, Gt, Gte, Eq, Ne
+  ElemUnary = 1,    // Sigmoid, Tanh, Exp, ... (by the op's String() name)
+  BroadcastBin = 2, // BroadcastAdd / BroadcastHadamardProd ... (broadcast.go:69-129)
+  MatMul = 3,       // linAlgBinOp matMulOperator (+transA/transB)
+  MatVecMul = 4,
+  Outer = 5,
+  BatchedMatMul = 6,
+  Conv2d = 7,       // nnops.Conv2d
+  MaxPool2D = 8,    // nnops.MaxPool2D
+  BatchNorm = 9,    // nnops.BatchNorm in eval mode (+ the gamma/beta wrap of nn.go:429-440)
+  Rectify = 10,     // nnops.Rectify
+  LeakyRelu = 11,   // gorgonia.LeakyRelu
+  SoftMax = 12,     // gorgonia.SoftMax (last axis)
+  Reshape = 13      // gorgonia.Reshape
+};
+
+struct OpSpec {
+  OpKind kind = OpKind::ElemBin;
+  int32_t fn = 0;             // gh_binfn for ElemBin / BroadcastBin
+  std::string name;           // unary op name ("sigmoid", "tanh", ...)
+  bool transA = false, transB = false;
+  std::vector<int64_t> ints;  // kernel/pad/stride/dilation, new shape, broadcast axes ...
+  double f0 = 0.0;            // epsilon / alpha
+  bool fuse_act_relu = false;   // batcher-fused epilogue (set by Graph::FuseActivations)
+  bool fuse_act_leaky = false;
+};
+
+// Output shape of an op (InferShape of each reference op); error if the inputs
+// do not fit.
+Status InferShape(const OpSpec& op, const std::vector<const Shape*>& in, Shape* out);
+// Which input the op may overwrite, -1 for none (OverwritesInput,
+// op_math.go:285-294,476-481; the nn ops return -1).
+int OverwritesInput(const OpSpec& op);
+// Record the op's device work on the engine (one or more gh_cmd).
+Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<Tensor*>& inputs);
+
+struct Node {
+  int id = -1;
+  Shape shape;
+  Dtype dt = Dtype::Float32;
+  bool is_input = false;
+  bool resident = false;          // uploaded once and kept (weights); else re-uploaded per run
+  const void* host = nullptr;     // bound host value (Let / WithValue)
+  OpSpec op;
+  std::vector<int> inputs;
+  void* read_into = nullptr;      // Read(node, &host) target
+  bool fused_away = false;        // activation folded into its producer
+  int alias_of = -1;              // Reshape shares its input's register
+};
+
+class Graph {
+ public:
+  int NewTensor(const Shape& s, Dtype dt, const void* host, bool resident);
+  Status Apply(const OpSpec& op, const std::vector<int>& inputs, int* out);
+  Status Let(int node, const void* host);              // rebind an input value
+  Status Read(int node, void* host_out);               // gorgonia.Read
+  // Fold Rectify/LeakyRelu into the Conv2d/MatMul that feeds them when nothing
+  // else reads the un-activated value (bit-identical epilogue).
+  int FuseActivations();
+  const std::vector<Node>& Nodes() const { return nodes_; }
+  std::vector<Node>& Nodes() { return nodes_; }
+
+ private:
+  std::vector<Node> nodes_;
+};
+
+enum class InstrKind : int32_t { LoadArg, Alloc, Transport, ExecOp, Free, Flush, Read };
+
+struct Instr {
+  InstrKind kind;
+  int node = -1;    // node the instruction is about
+  int reg = -1;     // register written / freed
+  int64_t size = 0; // bytes for Alloc/Free/Transport/Read
+  bool use_unsafe = false;  // ExecOp reuses input 0's register
+};
+
+struct TapeOptions {
+  bool graph_replay = false;      // capture each segment into a hipGraph and replay it
+  bool reupload_resident = false; // treat resident inputs like the reference does (H2D every run)
+};
+
+class TapeMachine {
+ public:
+  TapeMachine(Graph* g, const TapeOptions& o) : g_(g), opt_(o) {}
+  ~TapeMachine();
+  // Compile (compile.go:16-60 for forward graphs), size the arena from the
+  // program (compile.go:148-216) and create the engine (vm_tape_cuda.go:17-41).
+  Status Init(int device);
+  Status Compile();  // program only, no device
+  Status RunAll();
+  Status Reset();   // vm_tape.go:123-134: pc = 0, arena reset
+  Status Close();
+  Engine& Eng() { return eng_; }
+  const std::vector<Instr>& Program() const { return prog_; }
+  int64_t GpuMem() const { return gpumem_; }
+  int Segments() const { return segments_; }      // flush points in the last run
+  int GraphLaunches() const { return graph_launches_; }
+  uint64_t RegisterAddress(int node) const;
+  std::string ProgramString() const;              // program.String() (vm_tape.go:493-522)
+
+ private:
+  Status flush();
+  Graph* g_;
+  TapeOptions opt_;
+  Engine eng_;
+  std::vector<Instr> prog_;
+  std::vector<Tensor> regs_;       // one per register
+  std::vector<int> node_reg_;      // node -> register
+  std::vector<char> reg_live_;     // register currently holds arena memory
+  std::vector<char> resident_done_;
+  int64_t gpumem_ = 0;
+  int runs_ = 0, segments_ = 0, graph_launches_ = 0;
+  // per-segment replay cache
+  struct SegCache { std::vector<gh_cmd> cmds; int graph_id = -1; };
+  std::vector<SegCache> seg_cache_;
+  int seg_index_ = 0;
+};
+
+}  // namespace gorgonia

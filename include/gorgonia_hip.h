@@ -116,9 +116,11 @@ enum gh_unaryfn {
 /*
  * One operator.  Field use per opcode:
  *
- * ELEM_BIN    ptr[0]=A ptr[1]=B            dim[0]=n
- *             vv/vs/ss write A, sv writes B (elembinop.cu:13-35)
- * ELEM_UNARY  ptr[0]=A (in place)          dim[0]=n
+ * ELEM_BIN    ptr[0]=A ptr[1]=B [ptr[2]=dst]  dim[0]=n
+ *             without dst: vv/vs/ss write A, sv writes B (elembinop.cu:13-35);
+ *             with dst the operands are left alone (the reference reaches the
+ *             same state by memcpy(reuse <- a) + in-place op, cuda/arith.go:36-44)
+ * ELEM_UNARY  ptr[0]=A [ptr[1]=dst]        dim[0]=n ; in place without dst
  * BCAST_BIN   ptr[0]=dst ptr[1]=big ptr[2]=small
  *             dim[0]=outer dim[1]=mid dim[2]=inner; small has `mid` elements,
  *             element (o,m,i) pairs big[o,m,i] with small[m]

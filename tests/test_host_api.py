@@ -1,0 +1,162 @@
+"""Host mirror checks that need no GPU: exported symbols, the engine's argument
+checks and error texts (cuda/utils.go:22-112, cuda/arith.go:17-49,
+cuda/linalg.go:17-45), shape inference of the operators and the compiled tape
+program (register reuse, flush placement)."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+from gorgonia_amd import configs, graph as G
+from gorgonia_amd.engine import HOST_SYMBOLS, Engine, EngineError, Tensor, load_host
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_header_symbols_all_exported():
+    hdr = open(os.path.join(ROOT, "include", "gorgonia_host.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    declared = set(re.findall(r"\b(ghh_[a-z0-9_]+)\s*\(", hdr))
+    lib = load_host()
+    for name in sorted(declared):
+        assert hasattr(lib, name), name
+    assert declared == set(HOST_SYMBOLS), declared ^ set(HOST_SYMBOLS)
+
+
+@pytest.fixture()
+def eng():
+    e = Engine()  # not initialised: every check below happens before any device call
+    yield e
+    e.destroy()
+
+
+def T(shape, dtype=np.float32, mem=0x1000, **kw):
+    return Tensor(mem, shape, dtype, **kw)
+
+
+def test_binary_checks(eng):
+    with pytest.raises(EngineError, match=r"Basic checks failed for Add: Shape mismatch. Expected \(4\). Got \(2\)"):
+        eng.Add(T((2,)), T((4,)), unsafe=True)
+    with pytest.raises(EngineError, match="TypeMismatch: a float64 and b float32"):
+        eng.Gt(T((2,), np.float64), T((2,), np.float32), unsafe=True)
+    with pytest.raises(EngineError, match="Unsupported Dtype for a"):
+        eng.Mul(T((2,), np.int32), T((2,), np.int32), unsafe=True)
+    with pytest.raises(EngineError, match="a requires an iterator"):
+        eng.Sub(T((2,), needs_iterator=True), T((2,)), unsafe=True)
+    # safe without reuse is an error; incr is unsupported (cuda/arith.go:47-49)
+    with pytest.raises(EngineError, match="Impossible state: A reuse tensor must be passed in"):
+        eng.Add(T((2,)), T((2,)))
+    with pytest.raises(EngineError, match="Incr"):
+        eng.Add(T((2,)), T((2,)), reuse=T((2,), mem=0x2000), incr=True)
+    # reuse checks (cuda/utils.go:35-47)
+    with pytest.raises(EngineError, match="Cannot use reuse: shape mismatch"):
+        eng.Add(T((4,)), T((4,)), reuse=T((3,), mem=0x2000))
+    with pytest.raises(EngineError, match="Cannot use reuse: TypeMismatch"):
+        eng.Add(T((4,)), T((4,)), reuse=T((4,), np.float64, mem=0x2000))
+    # mod has no kernel (elembinop.cu:201-210)
+    with pytest.raises(EngineError, match=r'does not have the function "elembinop.mod_vv_f32"'):
+        eng.Mod(T((4,)), T((4,)), unsafe=True)
+    with pytest.raises(EngineError, match="b has to be a tensor.Memory"):
+        eng.AddScalar(T((4,)), None, True, unsafe=True)
+    # a valid call only records a command
+    eng.Add(T((4,)), T((4,)), unsafe=True)
+    eng.MulScalar(T((4,)), 0x3000, False, reuse=T((4,), mem=0x2000))
+    assert eng.pending() == 2
+
+
+def test_linalg_checks(eng):
+    a, b, c = T((3, 4)), T((4, 5)), T((3, 5))
+    with pytest.raises(EngineError, match="a isn't"):
+        eng.MatMul(T((3, 4), managed=False), b, c)
+    with pytest.raises(EngineError, match="same Dtype"):
+        eng.MatMul(a, T((4, 5), np.float64), c)
+    with pytest.raises(EngineError, match="Shape mismatch"):
+        eng.MatMul(a, T((3, 5)), c)
+    with pytest.raises(EngineError, match="Shape mismatch"):
+        eng.MatMul(a, b, T((5, 3)))
+    eng.MatMul(a, b, c)
+    eng.MatMul(T((4, 3)).T(), b, c)          # transposed view of a (4,3) buffer
+    eng.MatVecMul(a, T((4,)), T((3,)))
+    eng.Outer(T((3,)), T((5,)), c)
+    assert eng.pending() == 4
+
+
+def test_has_func_and_unknown_unary(eng):
+    assert eng.HasFunc("elembinop.add_vv_f32") and eng.HasFunc("elemunaryop.tanh_f64")
+    assert not eng.HasFunc("elembinop.mod_vv_f32")
+    with pytest.raises(EngineError, match="does not have the function"):
+        eng.Unary("erf", T((4,)))
+    assert eng.AllocAccessible() is False
+
+
+def test_elem_grid_size_matches_reference_rule(eng):
+    """cuda/external.go:52-85 with the device limits defaulted (1024 threads)."""
+    assert eng.ElemGridSize(100) == (1, 1, 1, 100, 1, 1)
+    assert eng.ElemGridSize(1024) == (1, 1, 1, 1024, 1, 1)
+    assert eng.ElemGridSize(1025) == (2, 1, 1, 1024, 1, 1)
+    assert eng.ElemGridSize(1 << 24) == (16384, 1, 1, 1024, 1, 1)
+
+
+def test_shape_inference_and_errors():
+    g = G.NewGraph()
+    x = G.NewTensor(g, np.zeros((2, 3, 8, 8), np.float32))
+    w = G.NewTensor(g, np.zeros((5, 3, 3, 3), np.float32))
+    assert G.Conv2d(x, w, (3, 3), (1, 1), (1, 1), (1, 1)).Shape() == (2, 5, 8, 8)
+    assert G.Conv2d(x, w, (3, 3), (0, 0), (2, 2), (1, 1)).Shape() == (2, 5, 3, 3)
+    assert G.MaxPool2D(x, (2, 2), (0, 0), (2, 2)).Shape() == (2, 3, 4, 4)
+    assert G.MaxPool2D(x, (2, 2), (1, 0, 1, 0), (1, 1)).Shape() == (2, 3, 8, 8)
+    with pytest.raises(EngineError, match="Cannot use strides of less than or equal 0"):
+        G.Conv2d(x, w, (3, 3), (1, 1), (0, 1), (1, 1))
+    with pytest.raises(EngineError, match="Cannot use padding of less than 0"):
+        G.MaxPool2D(x, (2, 2), (-1, 0), (2, 2))
+    with pytest.raises(EngineError, match="Impossible height/kernel/pad combination"):
+        G.MaxPool2D(x, (9, 2), (0, 0), (1, 1))
+    with pytest.raises(EngineError, match="im should have 4 dims, got 2 dims"):
+        G.Conv2d(G.NewTensor(g, np.zeros((2, 3), np.float32)), w, (3, 3))
+    a = G.NewTensor(g, np.zeros((4, 6), np.float32))
+    b = G.NewTensor(g, np.zeros((1, 6), np.float32))
+    assert G.BroadcastAdd(a, b).Shape() == (4, 6)
+    assert G.Mul(a, G.NewTensor(g, np.zeros((6, 2), np.float32))).Shape() == (4, 2)
+    assert G.Mul(a, G.NewTensor(g, np.zeros((5, 6), np.float32)), transB=True).Shape() == (4, 5)
+    with pytest.raises(EngineError, match="Shape mismatch"):
+        G.Add(a, b)
+    assert G.Reshape(a, (2, 12)).Shape() == (2, 12)
+    with pytest.raises(EngineError, match="invalid runningMean shape"):
+        G.BatchNorm(x, None, None, G.NewTensor(g, np.zeros((2, 2), np.float32)),
+                    G.NewTensor(g, np.zeros(3, np.float32)))
+
+
+def test_tape_program_keeps_live_values():
+    """Config 2: z feeds both Tanh and Pow, so Sigmoid may overwrite its dead
+    input but Tanh must not overwrite z (regalloc.go:211-243)."""
+    inp = configs.elementwise_inputs(8)
+    g, outs = configs.build_elementwise(inp)
+    m = G.NewTapeMachine(g, compile_only=True)
+    prog = m.program()
+    lines = [l for l in prog.splitlines() if "execOp" in l]
+    assert len(lines) == 5
+    assert "elembin.mul [unsafe]" in lines[0]          # x*y overwrites x (dead afterwards)
+    assert "broadcast.add" in lines[1]
+    assert "elemunary.sigmoid [unsafe]" in lines[2]    # its input is dead
+    assert "elemunary.tanh [reuse]" in lines[3]        # z is still needed by Pow
+    assert "elembin.pow [reuse]" in lines[4]           # z is read by the host afterwards
+    # one flush, in front of the host reads
+    assert prog.count("flush") == 1
+    assert prog.index("flush") < prog.index("read")
+    m.Close()
+
+
+def test_tape_program_convnet_fusion():
+    inp = configs.convnet_inputs(2)
+    g, _ = configs.build_convnet(inp)
+    m = G.NewTapeMachine(g, compile_only=True, fuse_activations=True)
+    assert m.fused == 4
+    prog = m.program()
+    assert prog.count("conv2d+rectify") == 3 and prog.count(" rectify") == 0
+    assert prog.count("maxpool2d") == 3 and prog.count("softmax") == 1
+    m.Close()
+    g2, _ = configs.build_convnet(inp)
+    m2 = G.NewTapeMachine(g2, compile_only=True)
+    assert m2.program().count(" rectify") == 4
+    m2.Close()
