@@ -1,0 +1,279 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X tensor-engine hot path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu]
+
+A step is one forward pass of the convnet configuration (batch 128x1x28x28,
+3x[Conv2d 3x3 + ReLU + MaxPool 2x2] + 2 dense layers + SoftMax) on the tape
+machine, with weights and the input batch already resident in HBM.  The same
+run also measures the other two parts of the headline metric - the elementwise
+chain on 4096x4096 tensors (HBM GB/s) and SGEMM 4096^3 (TFLOP/s) - with HIP
+events on the engine's own stream, and times the CPU oracle on the host cores
+as a reported baseline.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
+MFMA_F32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_cmds(ctx, cmds, iters, warm=3):
+    """Average milliseconds per submission of `cmds`, HIP events on the engine stream."""
+    for _ in range(warm):
+        ctx.submit(cmds)
+    ctx.sync()
+    ctx.event(0)
+    for _ in range(iters):
+        ctx.submit(cmds)
+    ctx.event(1)
+    return ctx.elapsed_ms(0, 1) / iters
+
+
+def bench_elementwise(ctx, iters):
+    """Config 2: z = Sigmoid(x*y + b); Tanh(z); Pow(z, 2) on 4096x4096 float32."""
+    from gorgonia_amd import configs, device as D
+    inp = configs.elementwise_inputs(4096)
+    N = 4096 * 4096
+    x, y, b = ctx.upload(inp["x"]), ctx.upload(inp["y"]), ctx.upload(inp["b"])
+    z, t, p = ctx.malloc(4 * N), ctx.malloc(4 * N), ctx.malloc(4 * N)
+    two = ctx.upload(np.array([2.0], np.float32))
+    ctx.run([D.cmd_bin("mul", "vv", x, y, N, dst=z), D.cmd_bcast("add", z, z, b, 4096, 4096, 1),
+             D.cmd_unary("sigmoid", z, N)])
+    kernels = [
+        ("HadamardProd", D.cmd_bin("mul", "vv", x, y, N, dst=p), 3 * 4 * N),
+        ("BroadcastAdd", D.cmd_bcast("add", p, p, b, 4096, 4096, 1), 2 * 4 * N + 4 * 4096),
+        ("Sigmoid", D.cmd_unary("sigmoid", p, N, dst=t), 2 * 4 * N),
+        ("Tanh", D.cmd_unary("tanh", z, N, dst=t), 2 * 4 * N),
+        ("Pow2", D.cmd_bin("pow", "vs", z, two, N, dst=p), 2 * 4 * N),
+    ]
+    out, total_ms, total_bytes = {}, 0.0, 0
+    for name, cmd, nbytes in kernels:
+        ms = time_cmds(ctx, [cmd], iters)
+        out[name] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1),
+                     "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "bytes": nbytes}
+        total_ms += ms
+        total_bytes += nbytes
+    # device copy of the same size as a measured ceiling next to the nominal one
+    ms = time_cmds(ctx, [D.cmd_copy(t, x, 4 * N)], iters)
+    copy_gbps = 2 * 4 * N / ms / 1e6
+    for q in (x, y, b, z, t, p, two):
+        ctx.free(q)
+    return {"chain_GBps": round(total_bytes / total_ms / 1e6, 1), "chain_bytes": total_bytes,
+            "chain_us": round(total_ms * 1e3, 1), "frac_hbm": round(total_bytes / total_ms / 1e6 / HBM_PEAK_GBPS, 4),
+            "device_copy_GBps": round(copy_gbps, 1), "kernels": out}
+
+
+def bench_linalg(ctx, iters):
+    """Config 3: SGEMM 4096^3, BatchedMatMul 64 x 512^3, MatVecMul 8192^2."""
+    from gorgonia_amd import device as D, synth
+    res = {}
+    for name, (m, n, k, batch) in {"sgemm_4096": (4096, 4096, 4096, 1), "bmm_64x512": (512, 512, 512, 64)}.items():
+        A = ctx.upload(synth.normal(1, (batch * m * k,)))
+        B = ctx.upload(synth.normal(2, (batch * k * n,)))
+        Cm = ctx.malloc(batch * m * n * 4)
+        cmd = D.cmd_gemm(A, B, Cm, m, n, k, batch=batch, stride_a=m * k, stride_b=k * n, stride_c=m * n)
+        ms = time_cmds(ctx, [cmd], max(5, iters // 2))
+        fl = 2.0 * m * n * k * batch
+        res[name] = {"us": round(ms * 1e3, 1), "TFLOPs": round(fl / ms / 1e9, 2),
+                     "frac_mfma": round(fl / ms / 1e9 / MFMA_F32_PEAK_TFLOPS, 4), "flop": fl}
+        for q in (A, B, Cm):
+            ctx.free(q)
+    m = n = 8192
+    A = ctx.upload(synth.normal(3, (m * n,)))
+    xv, yv = ctx.upload(synth.normal(4, (n,))), ctx.malloc(4 * m)
+    ms = time_cmds(ctx, [D.cmd_gemv(A, xv, yv, m, n)], iters)
+    nb = 4 * (m * n + m + n)
+    res["gemv_8192"] = {"us": round(ms * 1e3, 1), "GBps": round(nb / ms / 1e6, 1),
+                        "frac_hbm": round(nb / ms / 1e6 / HBM_PEAK_GBPS, 4), "bytes": nb}
+    for q in (A, xv, yv):
+        ctx.free(q)
+    return res
+
+
+CONVNET_LAYERS = [  # (name, B-relative shape) of configuration 4
+    ("conv0", 1, 28, 32), ("conv1", 32, 14, 64), ("conv2", 64, 7, 128),
+]
+
+
+def bench_convnet_kernels(ctx, batch, iters):
+    """Per-kernel time of the conv layers of the convnet step (for the roofline object)."""
+    from gorgonia_amd import device as D, synth
+    out = {}
+    for name, cin, hw, f in CONVNET_LAYERS:
+        x = ctx.upload(synth.uniform01(1, (batch * cin * hw * hw,)))
+        w = ctx.upload(synth.normal(2, (f * cin * 9,)))
+        y = ctx.malloc(batch * f * hw * hw * 4)
+        ms = time_cmds(ctx, [D.cmd_conv2d(x, w, y, batch, cin, hw, hw, f, 3, 3, (1, 1), act="relu")], iters)
+        fl = 2.0 * batch * hw * hw * f * cin * 9
+        nb = 4 * (batch * cin * hw * hw + f * cin * 9 + batch * f * hw * hw)
+        out[name] = {"us": round(ms * 1e3, 2), "TFLOPs": round(fl / ms / 1e9, 2), "flop": fl,
+                     "GBps": round(nb / ms / 1e6, 1), "bytes": nb}
+        for q in (x, w, y):
+            ctx.free(q)
+    return out
+
+
+def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=True):
+    from gorgonia_amd import configs, graph as G
+    inp = configs.convnet_inputs(batch)
+    g = G.NewGraph()
+    # same graph as configs.build_convnet, with the input batch optionally resident
+    h = G.NewTensor(g, inp["x"], resident=resident_input)
+    for i in range(3):
+        w = G.NewTensor(g, inp[f"w{i}"], True)
+        h = G.MaxPool2D(G.Rectify(G.Conv2d(h, w, (3, 3), (1, 1), (1, 1), (1, 1))), (2, 2), (0, 0), (2, 2))
+    h = G.Reshape(h, (batch, 128 * 3 * 3))
+    h = G.Rectify(G.Mul(h, G.NewTensor(g, inp["w3"], True)))
+    out = G.Read(G.SoftMax(G.Mul(h, G.NewTensor(g, inp["w4"], True))))
+    m = G.NewTapeMachine(g, graph_replay=graph_replay, fuse_activations=True)
+    for _ in range(max(warmup, 3)):  # first run eager, second captures, third replays
+        m.RunAll()
+    eng = m.engine()
+    eng.DoWork()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        m.RunAll()
+    eng.DoWork()
+    dt = time.perf_counter() - t0
+    result = out.copy()
+    launches = m.graph_launches()
+    m.Close()
+    return dt / steps * 1e3, result, inp, launches
+
+
+def cpu_baseline_convnet(inp, budget_s=12.0):
+    """The CPU oracle's forward pass of the same configuration on the host cores."""
+    from oracle import binding as O, forward as F
+    threads = min(os.cpu_count() or 1, 16)
+    O.set_threads(threads)
+    t0 = time.perf_counter()
+    ref = F.convnet(inp)
+    one = time.perf_counter() - t0
+    reps = 1
+    while (reps + 1) * one < budget_s and reps < 50:
+        F.convnet(inp)
+        reps += 1
+    total = time.perf_counter() - t0
+    O.set_threads(1)
+    return ref, inp["x"].shape[0] * reps / total, threads, reps
+
+
+def cpu_baseline_micro():
+    """Oracle timings of the other two metric parts on a bounded sample."""
+    from oracle import binding as O
+    from gorgonia_amd import synth
+    res = {}
+    n = 1 << 22  # 4 Mi elements of the 16 Mi-element chain, single thread like the reference's loops
+    x, y = synth.uniform(1, (n,), -4, 4), synth.uniform(2, (n,), -4, 4)
+    b = synth.uniform(3, (4096,), -4, 4)
+    t0 = time.perf_counter()
+    z = O.unary("sigmoid", O.bcast_binop("add", O.binop("mul", "vv", x, y), b, n // 4096, 4096, 1))
+    O.unary("tanh", z)
+    O.binop("pow", "vs", z, np.array([2.0], np.float32))
+    dt = time.perf_counter() - t0
+    res["elementwise_chain_GBps"] = round(738_213_888 * (n / (4096 * 4096)) / dt / 1e9, 3)
+    res["elementwise_sample"] = "4 Mi of 16 Mi elements, 1 thread"
+    threads = min(os.cpu_count() or 1, 16)
+    O.set_threads(threads)
+    m, k, nn = 256, 4096, 4096  # a 256-row slab of the 4096^3 product
+    A, B = synth.normal(4, (m, k)), synth.normal(5, (k, nn))
+    t0 = time.perf_counter()
+    O.gemm(A, B)
+    dt = time.perf_counter() - t0
+    O.set_threads(1)
+    res["sgemm_TFLOPs"] = round(2.0 * m * k * nn / dt / 1e12, 4)
+    res["sgemm_sample"] = f"256x4096x4096 slab, {threads} threads"
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="comma list of: convnet,elementwise,linalg")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this engine runs on one GPU; --gpus must be 1 (no multi-GPU path is built)")
+    only = set(filter(None, a.only.split(",")))
+
+    from gorgonia_amd.device import Context
+    ctx = Context(0, 0)
+    info = ctx.info()
+    log(f"device {info.arch.decode()} CUs={info.compute_units}")
+
+    ms_step, gpu_out, inp, launches = bench_convnet(a.steps, a.warmup)
+    images_s = 128 / ms_step * 1e3
+    log(f"convnet: {ms_step:.4f} ms/step  {images_s:.0f} images/s  (graph launches {launches})")
+    ms_h2d, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False)
+    ms_eager, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, graph_replay=False)
+
+    iters = 30
+    conv_k = bench_convnet_kernels(ctx, 128, iters) if not only or "convnet" in only else {}
+    elem = bench_elementwise(ctx, iters) if not only or "elementwise" in only else {}
+    lin = bench_linalg(ctx, iters) if not only or "linalg" in only else {}
+    ctx.close()
+
+    # the dominant kernel of the step: the conv layer with the largest time
+    roofline = None
+    if conv_k:
+        name = max(conv_k, key=lambda k: conv_k[k]["us"])
+        r = conv_k[name]
+        roofline = {"kernel": f"k_conv2d ({name} of the convnet step, fused ReLU)", "bound": "mfma",
+                    "achieved": r["TFLOPs"], "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(r["TFLOPs"] / MFMA_F32_PEAK_TFLOPS, 4), "traffic": None,
+                    "launch_us": r["us"], "algorithmic_flop": r["flop"]}
+
+    cpu = None
+    parity = None
+    if not a.skip_cpu:
+        ref, cpu_images_s, threads, reps = cpu_baseline_convnet(inp)
+        err = float(np.linalg.norm(gpu_out.astype(np.float64) - ref) / np.linalg.norm(ref))
+        parity = {"convnet_rel_frobenius_vs_oracle": err, "tolerance": 1e-5, "ok": err <= 1e-5}
+        cpu = {"value": round(cpu_images_s, 1), "unit": "images/s", "cores": threads, "kind": "port",
+               "sample": f"{reps} forward passes of the same 128-image batch (CPU oracle, OpenMP)"}
+        cpu.update(cpu_baseline_micro())
+
+    line = {
+        "metric": "convnet fwd images/s (1 GPU); elementwise HBM GB/s; SGEMM TFLOP/s",
+        "value": round(images_s, 1), "unit": "images/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "convnet forward, float32 NCHW batch 128x1x28x28 (config 4): "
+                               "3x[Conv2d 3x3 pad1 + ReLU + MaxPool 2x2] -> Dense 625 ReLU -> Dense 10 SoftMax; "
+                               "tape machine, one segment, hipGraph replay, weights and input resident",
+                   "batch": 128, "flop_per_step": 2_093_410_816},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "extra": {
+            "elementwise_hbm_GBps": elem.get("chain_GBps"), "elementwise_frac_hbm": elem.get("frac_hbm"),
+            "sgemm_TFLOPs": lin.get("sgemm_4096", {}).get("TFLOPs"),
+            "sgemm_frac_mfma": lin.get("sgemm_4096", {}).get("frac_mfma"),
+            "convnet_ms_per_step_with_input_h2d": round(ms_h2d, 5),
+            "convnet_images_s_with_input_h2d": round(128 / ms_h2d * 1e3, 1),
+            "convnet_ms_per_step_eager_no_graph": round(ms_eager, 5),
+            "convnet_kernels": conv_k, "elementwise": elem, "linalg": lin, "parity": parity,
+        },
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
