@@ -4,7 +4,9 @@
 // All of them are HBM-bound.  Each thread moves 16-byte vectors (float4 /
 // double2) in a grid-stride loop, several independent vectors per iteration so
 // that enough loads are in flight to cover HBM latency; a lane-contiguous
-// layout keeps every wavefront access a fully coalesced 1 KiB segment.
+// layout keeps every wavefront access a fully coalesced 1 KiB segment.  Plain
+// (cached) loads and stores with about 32 workgroups per CU measured fastest:
+// non-temporal accesses bypass the 256 MB last-level cache and lost ~15 %.
 //
 // Numerics: this file is compiled with -ffp-contract=off, denormals kept and
 // IEEE division, so add/sub/mul/div/compare are bit-identical to the CPU
@@ -16,7 +18,7 @@
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kUnroll = 4;
+constexpr int kUnroll = 2;
 
 template <class T> struct VecOf;
 template <> struct VecOf<float> { typedef float type __attribute__((ext_vector_type(4))); static constexpr int N = 4; };
@@ -39,20 +41,83 @@ __device__ __forceinline__ T bin_apply(T a, T b) {
   else return a != b ? (T)1 : (T)0;
 }
 
-// tanh in float64 from one exp: 1 - 2/(e^{2x}+1); a short odd series near 0
-// where that form cancels.  Error stays far below half a float32 ulp.
+// exp in float64 for results that are rounded to float32 afterwards.
+// Range reduction x = n ln2 + r with |r| <= ln2/2: n comes from the
+// "add 1.5*2^52" trick (the integer sits in the low mantissa bits, so no
+// round/convert instructions), exp(r) - 1 from a degree-10 Taylor polynomial
+// (relative error below 2^-41, far under half a float32 ulp), and the scaling
+// by 2^n is an integer add on the exponent field.  Valid for |x| <= 700;
+// callers clamp.  Explicit fma() so the -ffp-contract=off build still gets
+// fused steps here.  Conversion, reciprocal and ldexp instructions run at a
+// quarter of the FMA rate on this hardware, which is why they are avoided:
+// sigmoid/tanh/exp stay memory-bound.
+struct ExpParts { double q; int n; };  // exp(x) = (1 + q) * 2^n
+
+// A float64 constant pinned in a scalar register pair.  As a plain literal each
+// Horner step costs an extra 64-bit vector move (the compiler materialises the
+// coefficient into the accumulator of v_fmac_f64); from a scalar register the
+// step is a single v_fma_f64.  The empty asm only hides the value's origin.
+__device__ __forceinline__ double sconst(double v) {
+  asm("" : "+s"(v));
+  return v;
+}
+
+__device__ __forceinline__ ExpParts exp_parts(double x) {
+  const double kShift = sconst(6755399441055744.0);  // 1.5 * 2^52
+  const double t = fma(x, sconst(1.4426950408889634), kShift);
+  const double n = t - kShift;
+  double r = fma(-n, sconst(0.6931471803691238), x);   // ln2 high part
+  r = fma(-n, sconst(1.9082149292705877e-10), r);      // ln2 low part
+  double p = sconst(2.7557319223985893e-07);           // 1/10!
+  p = fma(p, r, sconst(2.7557319223985888e-06));       // 1/9!
+  p = fma(p, r, sconst(2.4801587301587302e-05));       // 1/8!
+  p = fma(p, r, sconst(1.9841269841269841e-04));       // 1/7!
+  p = fma(p, r, sconst(1.3888888888888889e-03));       // 1/6!
+  p = fma(p, r, sconst(8.3333333333333332e-03));       // 1/5!
+  p = fma(p, r, sconst(4.1666666666666664e-02));       // 1/4!
+  p = fma(p, r, sconst(1.6666666666666666e-01));       // 1/3!
+  p = fma(p, r, 0.5);
+  p = fma(p, r, 1.0);
+  ExpParts e;
+  e.q = p * r;
+  e.n = (int)(unsigned)__double_as_longlong(t);    // low 32 bits of t hold n
+  return e;
+}
+
+__device__ __forceinline__ double scale_pow2(double v, int n) {  // v * 2^n, result normal
+  return __longlong_as_double(__double_as_longlong(v) + ((long long)n << 52));
+}
+
+__device__ __forceinline__ double exp_f64_fast(double x) {
+  const ExpParts e = exp_parts(x);
+  return scale_pow2(1.0 + e.q, e.n);
+}
+
+// 1/s in float64 to ~2^-50: hardware reciprocal estimate plus one Newton step.
+__device__ __forceinline__ double rcp_f64_fast(double s) {
+  const double r = __builtin_amdgcn_rcp(s);
+  return fma(fma(-s, r, 1.0), r, r);
+}
+
+// exp(x) for a float32 argument, rounded once from float64.
+__device__ __forceinline__ float exp_f32_via_f64(float x) {
+  double xd = (double)x;
+  xd = xd < -110.0 ? -110.0 : xd;  // beyond the clamps the rounded result is 0 / +inf
+  xd = xd > 90.0 ? 90.0 : xd;      // (NaN fails both compares and propagates)
+  return (float)exp_f64_fast(xd);
+}
+
+// tanh in float64 from one exp, branch free: with a = 2|x|,
+// tanh|x| = (e^a - 1)/(e^a + 1) = em1/(em1 + 2).  For n == 0 the polynomial
+// yields e^a - 1 directly (no cancellation near zero); otherwise e^a >= sqrt(2)
+// and the subtraction is harmless.  Error stays far below half a float32 ulp.
 __device__ __forceinline__ double tanh_f64_for_f32(double x) {
-  double ax = fabs(x);
-  double r;
-  if (ax < 0.00390625) {  // 2^-8: |x^7 * 17/315| < 2^-60 relative
-    double x2 = ax * ax;
-    r = ax * (1.0 + x2 * (-1.0 / 3.0 + x2 * (2.0 / 15.0)));
-  } else if (ax > 20.0) {
-    r = 1.0;
-  } else {
-    r = 1.0 - 2.0 / (exp(2.0 * ax) + 1.0);
-  }
-  return x < 0 ? -r : r;
+  double a = 2.0 * fabs(x);
+  a = a > 44.0 ? 44.0 : a;  // tanh rounds to 1 long before; NaN propagates
+  const ExpParts e = exp_parts(a);
+  const double em1 = e.n == 0 ? e.q : scale_pow2(1.0 + e.q, e.n) - 1.0;
+  const double r = em1 * rcp_f64_fast(em1 + 2.0);
+  return copysign(r, x);
 }
 
 template <int FN>
@@ -63,7 +128,7 @@ __device__ __forceinline__ float unary_apply(float x) {
   else if constexpr (FN == GH_FLOOR) return floorf(x);
   else if constexpr (FN == GH_SIN) return (float)sin((double)x);
   else if constexpr (FN == GH_COS) return (float)cos((double)x);
-  else if constexpr (FN == GH_EXP) return (float)exp((double)x);
+  else if constexpr (FN == GH_EXP) return exp_f32_via_f64(x);
   else if constexpr (FN == GH_LN) return (float)log((double)x);
   else if constexpr (FN == GH_LOG2) return (float)log2((double)x);
   else if constexpr (FN == GH_NEG) return -x;
@@ -72,13 +137,10 @@ __device__ __forceinline__ float unary_apply(float x) {
   else if constexpr (FN == GH_INVERSE) return 1.0f / x;
   else if constexpr (FN == GH_INVSQRT) return 1.0f / sqrtf(x);
   else if constexpr (FN == GH_CUBE) return x * x * x;
-  else if constexpr (FN == GH_TANH) {
-    if (x != x) return x;
-    return (float)tanh_f64_for_f32((double)x);
-  } else if constexpr (FN == GH_SIGMOID) {
+  else if constexpr (FN == GH_TANH) return (float)tanh_f64_for_f32((double)x); else if constexpr (FN == GH_SIGMOID) {
     if (x < -88.0f) return 0.0f;
     if (x > 15.0f) return 1.0f;
-    return (float)(1.0 / (1.0 + exp((double)(-x))));
+    return (float)rcp_f64_fast(1.0 + exp_f64_fast((double)(-x)));  // NaN propagates
   } else if constexpr (FN == GH_LOG1P) return (float)log1p((double)x);
   else if constexpr (FN == GH_EXPM1) return (float)expm1((double)x);
   else {  // softplus
@@ -143,8 +205,8 @@ __global__ __launch_bounds__(kBlock) void k_bin_vec(const T* A, const T* B, T* D
     V a[kUnroll], b[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-      if constexpr (MODE != GH_SV) a[u] = __builtin_nontemporal_load(&Av[i + u * stride]);
-      if constexpr (MODE != GH_VS) b[u] = __builtin_nontemporal_load(&Bv[i + u * stride]);
+      if constexpr (MODE != GH_SV) a[u] = Av[i + u * stride];
+      if constexpr (MODE != GH_VS) b[u] = Bv[i + u * stride];
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
@@ -157,7 +219,7 @@ __global__ __launch_bounds__(kBlock) void k_bin_vec(const T* A, const T* B, T* D
           else r[e] = bin_apply<FN, T>(a[u][e], s);
         } else r[e] = bin_apply<FN, T>(s, b[u][e]);
       }
-      __builtin_nontemporal_store(r, &Dv[i + u * stride]);
+      Dv[i + u * stride] = r;
     }
   }
   for (; i < nv; i += stride) {
@@ -215,13 +277,13 @@ __global__ __launch_bounds__(kBlock) void k_unary_vec(const T* A, T* D, int64_t 
   for (; i + (kUnroll - 1) * stride < nv; i += kUnroll * stride) {
     V a[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; u++) a[u] = __builtin_nontemporal_load(&Av[i + u * stride]);
+    for (int u = 0; u < kUnroll; u++) a[u] = Av[i + u * stride];
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
       V r;
 #pragma unroll
       for (int e = 0; e < N; e++) r[e] = unary_apply<FN>(a[u][e]);
-      __builtin_nontemporal_store(r, &Dv[i + u * stride]);
+      Dv[i + u * stride] = r;
     }
   }
   for (; i < nv; i += stride) {
@@ -261,14 +323,14 @@ __global__ __launch_bounds__(kBlock) void k_bcast_row(float* __restrict__ dst,
   for (; r + (kUnroll - 1) * rs < rows; r += kUnroll * rs) {
     V a[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; u++) a[u] = __builtin_nontemporal_load(&bv[(r + u * rs) * colv + cv]);
+    for (int u = 0; u < kUnroll; u++) a[u] = bv[(r + u * rs) * colv + cv];
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
       V o;
 #pragma unroll
       for (int e = 0; e < 4; e++)
         o[e] = LEFT ? bin_apply<FN, float>(s[e], a[u][e]) : bin_apply<FN, float>(a[u][e], s[e]);
-      __builtin_nontemporal_store(o, &dv[(r + u * rs) * colv + cv]);
+      dv[(r + u * rs) * colv + cv] = o;
     }
   }
   for (; r < rows; r += rs) {
@@ -352,7 +414,7 @@ __global__ __launch_bounds__(kBlock) void k_has(const T* __restrict__ A, int64_t
 
 inline int grid_for(gh_ctx* ctx, int64_t work_items, int per_thread) {
   int64_t blocks = (work_items + (int64_t)kBlock * per_thread - 1) / ((int64_t)kBlock * per_thread);
-  const int64_t cap = (int64_t)ctx->cu_count * 8;
+  const int64_t cap = (int64_t)ctx->cu_count * 64;
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
   return (int)blocks;
@@ -455,7 +517,7 @@ int launch_bcast_fn(gh_ctx* ctx, const gh_cmd& c) {
   if (row) {
     const int64_t colv = mid / 4;
     const int gx = (int)((colv + kBlock - 1) / kBlock);
-    int64_t gy = ((int64_t)ctx->cu_count * 8 + gx - 1) / gx;
+    int64_t gy = ((int64_t)ctx->cu_count * 64 + gx - 1) / gx;
     const int64_t need = (outer + kUnroll - 1) / kUnroll;
     if (gy > need) gy = need;
     if (gy < 1) gy = 1;

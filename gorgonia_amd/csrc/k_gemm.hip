@@ -18,6 +18,8 @@
 // K = C*kh*kw: the "B" operand is gathered straight from the NCHW input (no
 // im2col buffer) and the result is written straight into NCHW (no transpose
 // pass), so lanes run along output pixels for coalesced loads and stores.
+#include <cstdio>
+#include <cstdlib>
 #include <type_traits>
 
 #include "gh_internal.h"
@@ -49,7 +51,8 @@ __device__ __forceinline__ float act_apply(float v, int act, float alpha) {
 template <int R, int BK, bool VEC>
 struct LoadKContig {
   static constexpr int S = R + 2;  // S % 32 == 2 keeps the transposing writes conflict-free
-  static constexpr int NV = (R * BK / 4) / kThreads;
+  static constexpr int TOTAL = R * BK / 4;  // float4 slots in a tile
+  static constexpr int NV = (TOTAL + kThreads - 1) / kThreads;
   const float* base; int ld; int rmax; int kmax;
   f32x4 reg[NV];
   __device__ __forceinline__ void load(int r0, int k0) {
@@ -59,7 +62,7 @@ struct LoadKContig {
       const int r = r0 + f / (BK / 4);
       const int k = k0 + (f % (BK / 4)) * 4;
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
-      if (r < rmax) {
+      if ((TOTAL % kThreads == 0 || f < TOTAL) && r < rmax) {
         const float* p = base + (int64_t)r * ld + k;
         if (VEC) {
           if (k < kmax) v = *reinterpret_cast<const f32x4*>(p);
@@ -75,6 +78,7 @@ struct LoadKContig {
 #pragma unroll
     for (int j = 0; j < NV; j++) {
       const int f = threadIdx.x + j * kThreads;
+      if (TOTAL % kThreads != 0 && f >= TOTAL) continue;
       const int r = f / (BK / 4);
       const int kq = (f % (BK / 4)) * 4;
 #pragma unroll
@@ -87,7 +91,8 @@ struct LoadKContig {
 template <int R, int BK, bool VEC>
 struct LoadMnContig {
   static constexpr int S = R;
-  static constexpr int NV = (R * BK / 4) / kThreads;
+  static constexpr int TOTAL = R * BK / 4;
+  static constexpr int NV = (TOTAL + kThreads - 1) / kThreads;
   const float* base; int ld; int rmax; int kmax;
   f32x4 reg[NV];
   __device__ __forceinline__ void load(int c0, int k0) {
@@ -97,7 +102,7 @@ struct LoadMnContig {
       const int k = k0 + f / (R / 4);
       const int c = c0 + (f % (R / 4)) * 4;
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
-      if (k < kmax) {
+      if ((TOTAL % kThreads == 0 || f < TOTAL) && k < kmax) {
         const float* p = base + (int64_t)k * ld + c;
         if (VEC) {
           if (c < rmax) v = *reinterpret_cast<const f32x4*>(p);
@@ -113,6 +118,7 @@ struct LoadMnContig {
 #pragma unroll
     for (int j = 0; j < NV; j++) {
       const int f = threadIdx.x + j * kThreads;
+      if (TOTAL % kThreads != 0 && f >= TOTAL) continue;
       const int k = f / (R / 4);
       const int c = (f % (R / 4)) * 4;
       *reinterpret_cast<f32x4*>(&lds[k * S + c]) = reg[j];
@@ -122,8 +128,10 @@ struct LoadMnContig {
 
 // im2col gather for Conv2d: logical operand [k][p], k = (c, kr, kc) in the
 // reference's order (op_nn.go:418-437), p = (b, oy, ox).  Each thread keeps
-// one output pixel for the whole kernel and walks k.  KH/KW > 0 are
-// compile-time kernel sizes; 0 means "use the runtime values".
+// one output pixel for the whole kernel and walks k.  What depends only on
+// the pixel - its base offset and which of the kh*kw taps fall inside the
+// image - is computed once; per element only k -> (c, tap) remains.
+// KH/KW > 0 are compile-time kernel sizes; 0 means "use the runtime values".
 struct ConvGeom {
   int C, H, W, oh, ow, kh, kw, padH, padW, strideH, strideW, dilH, dilW, P /* B*oh*ow */;
 };
@@ -131,34 +139,56 @@ struct ConvGeom {
 template <int R, int BK, int KH, int KW>
 struct LoadIm2col {
   static constexpr int S = R;
-  static constexpr int KPT = BK / (kThreads / R);  // k values per thread per tile
+  static constexpr int KSTEP = kThreads / R;  // k distance between a thread's elements
+  static constexpr int KPT = BK / KSTEP;      // k values per thread per tile
   const float* x; ConvGeom g; int kmax;
-  int pix_ok; int iy0, ix0; const float* xb;
+  int pix_off;          // offset of the window's (0,0) tap inside the batch item; may be negative
+  int iy0, ix0;
+  uint64_t tap_mask;    // bit r set: tap r = kr*kw + kc lies inside the image
+  const float* xb;
   float reg[KPT];
   __device__ __forceinline__ void init(int p0) {
+    const int kh = KH ? KH : g.kh, kw = KW ? KW : g.kw;
     const int p = p0 + (threadIdx.x % R);
-    pix_ok = p < g.P;
-    const int pp = pix_ok ? p : 0;
+    const bool ok = p < g.P;
+    const int pp = ok ? p : 0;
     const int b = pp / (g.oh * g.ow);
     const int rem = pp - b * (g.oh * g.ow);
     const int oy = rem / g.ow, ox = rem - oy * g.ow;
     iy0 = oy * g.strideH - g.padH;
     ix0 = ox * g.strideW - g.padW;
+    pix_off = iy0 * g.W + ix0;
     xb = x + (int64_t)b * g.C * g.H * g.W;
+    tap_mask = 0;
+    if (ok && kh * kw <= 64) {
+      for (int kr = 0; kr < kh; kr++)
+        for (int kc = 0; kc < kw; kc++) {
+          const int iy = iy0 + kr * g.dilH, ix = ix0 + kc * g.dilW;
+          if (iy >= 0 && iy < g.H && ix >= 0 && ix < g.W) tap_mask |= 1ull << (kr * kw + kc);
+        }
+    }
+    if (!ok) kmax = 0;  // out-of-range pixel: every element reads as zero
   }
   __device__ __forceinline__ void load(int /*p0*/, int k0) {
     const int kh = KH ? KH : g.kh, kw = KW ? KW : g.kw;
+    const int kk = kh * kw;
     const int kb = threadIdx.x / R;
+    const int HW = g.H * g.W;
 #pragma unroll
     for (int j = 0; j < KPT; j++) {
-      const int k = k0 + kb + j * (kThreads / R);
+      const int k = k0 + kb + j * KSTEP;
       float v = 0.f;
-      if (pix_ok && k < kmax) {
-        const int c = k / (kh * kw);
-        const int r = k - c * (kh * kw);
+      if (k < kmax) {
+        const int c = k / kk;
+        const int r = k - c * kk;
         const int kr = r / kw, kc = r - kr * kw;
-        const int iy = iy0 + kr * g.dilH, ix = ix0 + kc * g.dilW;
-        if (iy >= 0 && iy < g.H && ix >= 0 && ix < g.W) v = xb[((int64_t)c * g.H + iy) * g.W + ix];
+        bool in;
+        if (kk <= 64) in = (tap_mask >> r) & 1;
+        else {
+          const int iy = iy0 + kr * g.dilH, ix = ix0 + kc * g.dilW;
+          in = iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+        }
+        if (in) v = xb[c * HW + kr * g.dilH * g.W + kc * g.dilW + pix_off];
       }
       reg[j] = v;
     }
@@ -166,7 +196,7 @@ struct LoadIm2col {
   __device__ __forceinline__ void store(float* lds) const {
     const int kb = threadIdx.x / R, pl = threadIdx.x % R;
 #pragma unroll
-    for (int j = 0; j < KPT; j++) lds[(kb + j * (kThreads / R)) * S + pl] = reg[j];
+    for (int j = 0; j < KPT; j++) lds[(kb + j * KSTEP) * S + pl] = reg[j];
   }
 };
 
@@ -185,19 +215,29 @@ struct StoreNCHW {
   }
 };
 
+// Split-K partial sums: slab `split` of a [splits][M][N] workspace.
+struct StorePartial {
+  float* ws; int N;
+  __device__ __forceinline__ void put(int i, int j, float v) const { ws[(int64_t)i * N + j] = v; }
+};
+
 // ---- the MFMA core ---------------------------------------------------------------
-template <int BM, int BN, int BK, class LA, class LB, class SC>
-__device__ __forceinline__ void mfma_tile_loop(LA& la, LB& lb, const SC& sc, int M, int N, int K,
-                                               int m0, int n0, int act, float alpha) {
-  constexpr int WM = BM / 2, WN = BN / 2;      // 2 x 2 wavefronts
+// WAVES_M x WAVES_N wavefronts (4 in all) tile the BM x BN block; k-tiles
+// [kt0, kt1) are accumulated (a split-K slice, or the whole K range).
+template <int BM, int BN, int BK, int WAVES_M, class LA, class LB, class SC>
+__device__ __forceinline__ void mfma_tile_loop(LA& la, LB& lb, const SC& sc, int M, int N, int kt0,
+                                               int kt1, int m0, int n0, int act, float alpha) {
+  constexpr int WAVES_N = 4 / WAVES_M;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;    // MFMA tiles per wavefront
+  static_assert(TM >= 1 && TN >= 1 && WM % 32 == 0 && WN % 32 == 0, "bad wave tiling");
   constexpr int SA = LA::S, SB = LB::S;
   __shared__ float lds[2 * BK * (SA + SB)];
   float* const As = lds;                 // two buffers of BK * SA floats
   float* const Bs = lds + 2 * BK * SA;   // two buffers of BK * SB floats
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+  const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
   const int lr = lane & 31, lk = lane >> 5;
 
   f32x16 acc[TM][TN];
@@ -208,16 +248,15 @@ __device__ __forceinline__ void mfma_tile_loop(LA& la, LB& lb, const SC& sc, int
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
 
-  const int nk = (K + BK - 1) / BK;
-  la.load(m0, 0);
-  lb.load(n0, 0);
+  la.load(m0, kt0 * BK);
+  lb.load(n0, kt0 * BK);
   la.store(As);
   lb.store(Bs);
   __syncthreads();
 
-  for (int kt = 0; kt < nk; kt++) {
-    const int cur = kt & 1;
-    const bool more = kt + 1 < nk;
+  for (int kt = kt0; kt < kt1; kt++) {
+    const int cur = (kt - kt0) & 1;
+    const bool more = kt + 1 < kt1;
     if (more) {
       la.load(m0, (kt + 1) * BK);
       lb.load(n0, (kt + 1) * BK);
@@ -259,35 +298,80 @@ __device__ __forceinline__ void mfma_tile_loop(LA& la, LB& lb, const SC& sc, int
     }
 }
 
-template <int BM, int BN, int BK, bool TA, bool TB, bool VEC>
+// k-tile range of split `s` out of `splits` over nk tiles.
+__device__ __forceinline__ void split_range(int nk, int splits, int s, int* kt0, int* kt1) {
+  const int per = (nk + splits - 1) / splits;
+  *kt0 = s * per;
+  *kt1 = min(nk, *kt0 + per);
+}
+
+// blockIdx.z is the batch index (splits == 1) or the split-K slice (batch == 1).
+template <int BM, int BN, int BK, int WAVES_M, bool TA, bool TB, bool VEC>
 __global__ __launch_bounds__(kThreads) void k_sgemm(const float* __restrict__ A,
                                                     const float* __restrict__ B,
                                                     float* __restrict__ C, int M, int N, int K,
                                                     int lda, int ldb, int ldc, int64_t sA,
-                                                    int64_t sB, int64_t sC, int act, float alpha) {
+                                                    int64_t sB, int64_t sC, int act, float alpha,
+                                                    int splits, float* __restrict__ ws) {
   using LA = typename std::conditional<TA, LoadMnContig<BM, BK, VEC>, LoadKContig<BM, BK, VEC>>::type;
   using LB = typename std::conditional<TB, LoadKContig<BN, BK, VEC>, LoadMnContig<BN, BK, VEC>>::type;
   const int bz = blockIdx.z;
-  LA la; la.base = A + bz * sA; la.ld = lda; la.rmax = M; la.kmax = K;
-  LB lb; lb.base = B + bz * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
-  StoreRowMajor sc{C + bz * sC, ldc};
-  mfma_tile_loop<BM, BN, BK, LA, LB, StoreRowMajor>(la, lb, sc, M, N, K, blockIdx.y * BM,
-                                                    blockIdx.x * BN, act, alpha);
+  const int nk = (K + BK - 1) / BK;
+  if (splits > 1) {
+    int kt0, kt1;
+    split_range(nk, splits, bz, &kt0, &kt1);
+    LA la; la.base = A; la.ld = lda; la.rmax = M; la.kmax = K;
+    LB lb; lb.base = B; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
+    StorePartial sc{ws + (int64_t)bz * M * N, N};
+    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StorePartial>(la, lb, sc, M, N, kt0, kt1,
+                                                              blockIdx.y * BM, blockIdx.x * BN, 0, 0.f);
+  } else {
+    LA la; la.base = A + bz * sA; la.ld = lda; la.rmax = M; la.kmax = K;
+    LB lb; lb.base = B + bz * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
+    StoreRowMajor sc{C + bz * sC, ldc};
+    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreRowMajor>(la, lb, sc, M, N, 0, nk, blockIdx.y * BM,
+                                                               blockIdx.x * BN, act, alpha);
+  }
 }
 
-template <int BM, int BN, int BK, int KH, int KW, bool VEC>
+template <int BM, int BN, int BK, int WAVES_M, int KH, int KW, bool VEC>
 __global__ __launch_bounds__(kThreads) void k_conv2d(const float* __restrict__ x,
                                                      const float* __restrict__ w,
                                                      float* __restrict__ y, ConvGeom g, int F, int K,
-                                                     int act, float alpha) {
+                                                     int act, float alpha, int splits,
+                                                     float* __restrict__ ws) {
   using LA = LoadKContig<BM, BK, VEC>;
   using LB = LoadIm2col<BN, BK, KH, KW>;
   LA la; la.base = w; la.ld = K; la.rmax = F; la.kmax = K;
   LB lb; lb.x = x; lb.g = g; lb.kmax = K;
   const int n0 = blockIdx.x * BN;
   lb.init(n0);
-  StoreNCHW sc{y, F, g.oh * g.ow};
-  mfma_tile_loop<BM, BN, BK, LA, LB, StoreNCHW>(la, lb, sc, F, g.P, K, blockIdx.y * BM, n0, act, alpha);
+  const int nk = (K + BK - 1) / BK;
+  if (splits > 1) {
+    int kt0, kt1;
+    split_range(nk, splits, blockIdx.z, &kt0, &kt1);
+    StorePartial sc{ws + (int64_t)blockIdx.z * F * g.P, g.P};
+    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StorePartial>(la, lb, sc, F, g.P, kt0, kt1,
+                                                              blockIdx.y * BM, n0, 0, 0.f);
+  } else {
+    StoreNCHW sc{y, F, g.oh * g.ow};
+    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreNCHW>(la, lb, sc, F, g.P, 0, nk, blockIdx.y * BM,
+                                                           n0, act, alpha);
+  }
+}
+
+// Sum the split-K slabs in slab order (deterministic), apply the epilogue and
+// write through the same result writer as the unsplit kernel.
+template <class SC>
+__global__ __launch_bounds__(256) void k_splitk_reduce(const float* __restrict__ ws, int splits, int M,
+                                                       int N, SC sc, int act, float alpha) {
+  const int64_t total = (int64_t)M * N, stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    float acc = ws[e];
+    for (int s = 1; s < splits; s++) acc = acc + ws[(int64_t)s * total + e];
+    const int i = (int)(e / N), j = (int)(e - (int64_t)i * N);
+    sc.put(i, j, act_apply(acc, act, alpha));
+  }
 }
 
 // ---- GEMV / outer ------------------------------------------------------------------
@@ -307,7 +391,7 @@ __global__ __launch_bounds__(256) void k_gemv_n(const float* __restrict__ A,
     const int nv = n / 4;
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
     for (int i = lane; i < nv; i += 64) {
-      const f32x4 p = __builtin_nontemporal_load(&av[i]) * xv[i];
+      const f32x4 p = av[i] * xv[i];
       s += p;
     }
     acc = (s[0] + s[1]) + (s[2] + s[3]);
@@ -342,8 +426,59 @@ __global__ __launch_bounds__(256) void k_outer(const float* __restrict__ x,
 
 inline bool al16(uint64_t p) { return (p & 15u) == 0; }
 
-template <int BM, int BN, int BK>
-int launch_sgemm_cfg(gh_ctx* ctx, const gh_cmd& c) {
+// ---- tile plan -------------------------------------------------------------------
+// Three block shapes: 128x128 (each wavefront 64x64: the throughput shape),
+// 64x64 (each wavefront 32x32: more, smaller blocks for problems that would
+// leave CUs idle) and 32x256 (all four wavefronts along N: few filters, many
+// pixels).  When even the small shape yields too few blocks, K is split across
+// grid.z and a second kernel sums the slabs.
+enum { kTile128 = 0, kTile64 = 1, kTile32x256 = 2 };
+struct TilePlan { int tile; int splits; };
+
+inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Largest split count whose [splits][M][N] slabs fit the context workspace.
+inline int clamp_splits(gh_ctx* ctx, int64_t splits, int64_t M, int64_t N, int64_t K, int64_t batch) {
+  if (batch > 1 || splits < 1) return 1;
+  const int64_t nk = cdiv(K, 16);
+  if (splits > nk) splits = nk;
+  if (splits > 64) splits = 64;
+  const int64_t slab = M * N * 4;
+  if (slab <= 0 || !ctx->workspace) return 1;
+  const int64_t fit = ctx->workspace_bytes / slab;
+  if (splits > fit) splits = fit;
+  return splits < 1 ? 1 : (int)splits;
+}
+
+TilePlan plan_tiles(gh_ctx* ctx, int64_t M, int64_t N, int64_t K, int64_t batch, bool allow_32x256) {
+  TilePlan p{kTile128, 1};
+  if (const char* env = getenv("GORGONIA_HIP_GEMM_PLAN")) {  // tuning override: "tile,splits"
+    int t = 0, sp = 1;
+    if (sscanf(env, "%d,%d", &t, &sp) == 2 && t >= 0 && t <= 2 && sp >= 1) {
+      p.tile = (t == kTile32x256 && !allow_32x256) ? kTile64 : t;
+      p.splits = clamp_splits(ctx, sp, M, N, K, batch);
+      return p;
+    }
+  }
+  const int64_t cus = ctx->cu_count;
+  const int64_t big = cdiv(M, 128) * cdiv(N, 128) * batch;
+  if (big >= cus && M > 64) return p;
+  if (allow_32x256 && M <= 32) p.tile = kTile32x256;
+  else p.tile = kTile64;
+  const int64_t blocks = p.tile == kTile64 ? cdiv(M, 64) * cdiv(N, 64) * batch : cdiv(M, 32) * cdiv(N, 256);
+  if (batch == 1 && blocks < 2 * cus) {
+    const int64_t nk = cdiv(K, 16);
+    int64_t sp = cdiv(2 * cus, blocks);
+    const int64_t max_sp = nk / 4 > 0 ? nk / 4 : 1;  // at least 4 k-tiles per slice
+    if (sp > max_sp) sp = max_sp;
+    p.splits = clamp_splits(ctx, sp, M, N, K, batch);
+  }
+  return p;
+}
+
+template <int BM, int BN, int WAVES_M>
+int launch_sgemm_cfg(gh_ctx* ctx, const gh_cmd& c, int splits) {
+  constexpr int BK = 16;
   const int M = (int)c.dim[0], N = (int)c.dim[1], K = (int)c.dim[2];
   const int lda = (int)c.dim[3], ldb = (int)c.dim[4], ldc = (int)c.dim[5];
   const int batch = c.dim[6] <= 0 ? 1 : (int)c.dim[6];
@@ -358,10 +493,13 @@ int launch_sgemm_cfg(gh_ctx* ctx, const gh_cmd& c) {
                    sA % 4 == 0 && sB % 4 == 0 && (ta ? M % 4 == 0 : K % 4 == 0) &&
                    (tb ? K % 4 == 0 : N % 4 == 0);
   const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
-  const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, batch);
-#define GH_GEMM_LAUNCH(TA_, TB_, V_)                                                              \
-  hipLaunchKernelGGL((k_sgemm<BM, BN, BK, TA_, TB_, V_>), grid, dim3(kThreads), 0, ctx->stream, A, B, \
-                     C, M, N, K, lda, ldb, ldc, sA, sB, sC, act, c.f[0])
+  float* ws = (float*)ctx->workspace;
+  if (splits > 1 && (batch > 1 || (int64_t)splits * M * N * 4 > ctx->workspace_bytes))
+    return gh_fail(ctx, GH_ESTATE, "sgemm: split-K slabs do not fit the workspace");
+  const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, splits > 1 ? splits : batch);
+#define GH_GEMM_LAUNCH(TA_, TB_, V_)                                                                 \
+  hipLaunchKernelGGL((k_sgemm<BM, BN, BK, WAVES_M, TA_, TB_, V_>), grid, dim3(kThreads), 0, ctx->stream, \
+                     A, B, C, M, N, K, lda, ldb, ldc, sA, sB, sC, act, c.f[0], splits, ws)
   if (vec) {
     if (!ta && !tb) GH_GEMM_LAUNCH(false, false, true);
     else if (!ta && tb) GH_GEMM_LAUNCH(false, true, true);
@@ -374,39 +512,58 @@ int launch_sgemm_cfg(gh_ctx* ctx, const gh_cmd& c) {
     else GH_GEMM_LAUNCH(true, true, false);
   }
 #undef GH_GEMM_LAUNCH
-  return gh_check_hip(ctx, hipGetLastError(), "sgemm launch");
+  int rc = gh_check_hip(ctx, hipGetLastError(), "sgemm launch");
+  if (rc || splits <= 1) return rc;
+  const int64_t total = (int64_t)M * N;
+  int64_t blocks = cdiv(total, 256);
+  if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
+  hipLaunchKernelGGL((k_splitk_reduce<StoreRowMajor>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws,
+                     splits, M, N, StoreRowMajor{C, ldc}, act, c.f[0]);
+  return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
 }
 
-template <int BM, int BN, int BK, int KH, int KW>
-int launch_conv_cfg(gh_ctx* ctx, const gh_cmd& c, const ConvGeom& g, int F, int K) {
+template <int BM, int BN, int WAVES_M, int KH, int KW>
+int launch_conv_cfg(gh_ctx* ctx, const gh_cmd& c, const ConvGeom& g, int F, int K, int splits) {
+  constexpr int BK = 16;
   const bool vec = al16(c.ptr[1]) && K % 4 == 0;
   const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
-  const dim3 grid((g.P + BN - 1) / BN, (F + BM - 1) / BM, 1);
+  const dim3 grid((g.P + BN - 1) / BN, (F + BM - 1) / BM, splits);
   const float* x = (const float*)(uintptr_t)c.ptr[0];
   const float* w = (const float*)(uintptr_t)c.ptr[1];
   float* y = (float*)(uintptr_t)c.ptr[2];
+  float* ws = (float*)ctx->workspace;
+  if (splits > 1 && (int64_t)splits * F * g.P * 4 > ctx->workspace_bytes)
+    return gh_fail(ctx, GH_ESTATE, "conv2d: split-K slabs do not fit the workspace");
   if (vec)
-    hipLaunchKernelGGL((k_conv2d<BM, BN, BK, KH, KW, true>), grid, dim3(kThreads), 0, ctx->stream, x, w,
-                       y, g, F, K, act, c.f[0]);
+    hipLaunchKernelGGL((k_conv2d<BM, BN, BK, WAVES_M, KH, KW, true>), grid, dim3(kThreads), 0,
+                       ctx->stream, x, w, y, g, F, K, act, c.f[0], splits, ws);
   else
-    hipLaunchKernelGGL((k_conv2d<BM, BN, BK, KH, KW, false>), grid, dim3(kThreads), 0, ctx->stream, x,
-                       w, y, g, F, K, act, c.f[0]);
-  return gh_check_hip(ctx, hipGetLastError(), "conv2d launch");
+    hipLaunchKernelGGL((k_conv2d<BM, BN, BK, WAVES_M, KH, KW, false>), grid, dim3(kThreads), 0,
+                       ctx->stream, x, w, y, g, F, K, act, c.f[0], splits, ws);
+  int rc = gh_check_hip(ctx, hipGetLastError(), "conv2d launch");
+  if (rc || splits <= 1) return rc;
+  const int64_t total = (int64_t)F * g.P;
+  int64_t blocks = cdiv(total, 256);
+  if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
+  hipLaunchKernelGGL((k_splitk_reduce<StoreNCHW>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws,
+                     splits, F, g.P, StoreNCHW{y, F, g.oh * g.ow}, act, c.f[0]);
+  return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
 }
 
-template <int BM, int BN, int BK>
-int launch_conv_k(gh_ctx* ctx, const gh_cmd& c, const ConvGeom& g, int F, int K) {
-  if (g.kh == 3 && g.kw == 3) return launch_conv_cfg<BM, BN, BK, 3, 3>(ctx, c, g, F, K);
-  if (g.kh == 1 && g.kw == 1) return launch_conv_cfg<BM, BN, BK, 1, 1>(ctx, c, g, F, K);
-  return launch_conv_cfg<BM, BN, BK, 0, 0>(ctx, c, g, F, K);
+template <int BM, int BN, int WAVES_M>
+int launch_conv_k(gh_ctx* ctx, const gh_cmd& c, const ConvGeom& g, int F, int K, int splits) {
+  if (g.kh == 3 && g.kw == 3) return launch_conv_cfg<BM, BN, WAVES_M, 3, 3>(ctx, c, g, F, K, splits);
+  if (g.kh == 1 && g.kw == 1) return launch_conv_cfg<BM, BN, WAVES_M, 1, 1>(ctx, c, g, F, K, splits);
+  return launch_conv_cfg<BM, BN, WAVES_M, 0, 0>(ctx, c, g, F, K, splits);
 }
 
 }  // namespace
 
 int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
-  const int64_t M = c.dim[0];
-  if (M <= 64) return launch_sgemm_cfg<64, 128, 16>(ctx, c);
-  return launch_sgemm_cfg<128, 128, 16>(ctx, c);
+  const int64_t batch = c.dim[6] <= 0 ? 1 : c.dim[6];
+  const TilePlan p = plan_tiles(ctx, c.dim[0], c.dim[1], c.dim[2], batch, false);
+  if (p.tile == kTile128) return launch_sgemm_cfg<128, 128, 2>(ctx, c, p.splits);
+  return launch_sgemm_cfg<64, 64, 2>(ctx, c, p.splits);
 }
 
 int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
@@ -420,8 +577,10 @@ int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
   g.ow = (int)gh_conv_out(g.W, g.kw, g.padW, g.strideW, g.dilW);
   g.P = (int)c.dim[0] * g.oh * g.ow;
   const int F = (int)c.dim[4], K = g.C * g.kh * g.kw;
-  if (F <= 64) return launch_conv_k<64, 128, 16>(ctx, c, g, F, K);
-  return launch_conv_k<128, 128, 16>(ctx, c, g, F, K);
+  const TilePlan p = plan_tiles(ctx, F, g.P, K, 1, true);
+  if (p.tile == kTile128) return launch_conv_k<128, 128, 2>(ctx, c, g, F, K, p.splits);
+  if (p.tile == kTile32x256) return launch_conv_k<32, 256, 1>(ctx, c, g, F, K, p.splits);
+  return launch_conv_k<64, 64, 2>(ctx, c, g, F, K, p.splits);
 }
 
 int gh_launch_gemv(gh_ctx* ctx, const gh_cmd& c) {

@@ -58,8 +58,8 @@ __global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2(const float* __restric
     const int64_t bc = row / oh;
     const int ph = (int)(row - bc * oh);
     const float* in = x + (bc * H + 2 * ph) * (int64_t)W + 4 * pp;
-    const f4 r0 = __builtin_nontemporal_load(reinterpret_cast<const f4*>(in));
-    const f4 r1 = __builtin_nontemporal_load(reinterpret_cast<const f4*>(in + W));
+    const f4 r0 = *(reinterpret_cast<const f4*>(in));
+    const f4 r1 = *(reinterpret_cast<const f4*>(in + W));
     f2 o;
 #pragma unroll
     for (int e = 0; e < 2; e++) {
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kBlock) void k_bn_infer(const float* __restrict__ x
     if (VEC) {
       const int64_t sv = S / 4;
       for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < sv; i += stride) {
-        f4 v = __builtin_nontemporal_load(reinterpret_cast<const f4*>(in) + i);
+        f4 v = *(reinterpret_cast<const f4*>(in) + i);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           float t = v[e] * a;
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(kBlock) void k_bn_infer(const float* __restrict__ x
           if (hb) t = t + bt;
           v[e] = t;
         }
-        __builtin_nontemporal_store(v, reinterpret_cast<f4*>(out) + i);
+        *(reinterpret_cast<f4*>(out) + i) = v;
       }
     } else {
       for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < S; i += stride) {
