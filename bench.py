@@ -33,15 +33,22 @@ def log(*a):
 
 
 def time_cmds(ctx, cmds, iters, warm=3):
-    """Average milliseconds per submission of `cmds`, HIP events on the engine stream."""
-    for _ in range(warm):
-        ctx.submit(cmds)
+    """Average milliseconds per pass over `cmds`: `iters` passes are captured
+    into one hipGraph (so host enqueue time is out of the picture) and the
+    replay is bracketed by HIP events on the engine's stream."""
+    ctx.submit(list(cmds) * warm)
+    ctx.sync()
+    ctx.graph_begin()
+    ctx.submit(list(cmds) * iters)
+    gid = ctx.graph_end()
+    ctx.graph_launch(gid)
     ctx.sync()
     ctx.event(0)
-    for _ in range(iters):
-        ctx.submit(cmds)
+    ctx.graph_launch(gid)
     ctx.event(1)
-    return ctx.elapsed_ms(0, 1) / iters
+    ms = ctx.elapsed_ms(0, 1) / iters
+    ctx.graph_destroy(gid)
+    return ms
 
 
 def bench_elementwise(ctx, iters):

@@ -225,14 +225,13 @@ struct StorePartial {
 // WAVES_M x WAVES_N wavefronts (4 in all) tile the BM x BN block; k-tiles
 // [kt0, kt1) are accumulated (a split-K slice, or the whole K range).
 template <int BM, int BN, int BK, int WAVES_M, class LA, class LB, class SC>
-__device__ __forceinline__ void mfma_tile_loop(LA& la, LB& lb, const SC& sc, int M, int N, int kt0,
-                                               int kt1, int m0, int n0, int act, float alpha) {
+__device__ __forceinline__ void mfma_tile_loop(float* lds, LA& la, LB& lb, const SC& sc, int M, int N,
+                                               int kt0, int kt1, int m0, int n0, int act, float alpha) {
   constexpr int WAVES_N = 4 / WAVES_M;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;    // MFMA tiles per wavefront
   static_assert(TM >= 1 && TN >= 1 && WM % 32 == 0 && WN % 32 == 0, "bad wave tiling");
   constexpr int SA = LA::S, SB = LB::S;
-  __shared__ float lds[2 * BK * (SA + SB)];
   float* const As = lds;                 // two buffers of BK * SA floats
   float* const Bs = lds + 2 * BK * SA;   // two buffers of BK * SB floats
 
@@ -263,18 +262,26 @@ __device__ __forceinline__ void mfma_tile_loop(LA& la, LB& lb, const SC& sc, int
     }
     const float* a_s = As + cur * (BK * SA) + wm + lr;
     const float* b_s = Bs + cur * (BK * SB) + wn + lr;
+    // operand fragments are fetched one k-step ahead of the MFMAs that use them
+    float af[2][TM], bf[2][TN];
+#pragma unroll
+    for (int a = 0; a < TM; a++) af[0][a] = a_s[lk * SA + a * 32];
+#pragma unroll
+    for (int b = 0; b < TN; b++) bf[0][b] = b_s[lk * SB + b * 32];
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 2) {
-      float af[TM], bf[TN];
+      const int cb = (kk >> 1) & 1, nb = cb ^ 1;
+      if (kk + 2 < BK) {
 #pragma unroll
-      for (int a = 0; a < TM; a++) af[a] = a_s[(kk + lk) * SA + a * 32];
+        for (int a = 0; a < TM; a++) af[nb][a] = a_s[(kk + 2 + lk) * SA + a * 32];
 #pragma unroll
-      for (int b = 0; b < TN; b++) bf[b] = b_s[(kk + lk) * SB + b * 32];
+        for (int b = 0; b < TN; b++) bf[nb][b] = b_s[(kk + 2 + lk) * SB + b * 32];
+      }
 #pragma unroll
       for (int a = 0; a < TM; a++)
 #pragma unroll
         for (int b = 0; b < TN; b++)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[a], bf[b], acc[a][b], 0, 0, 0);
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cb][a], bf[cb][b], acc[a][b], 0, 0, 0);
     }
     if (more) {
       la.store(As + (cur ^ 1) * (BK * SA));
@@ -317,19 +324,22 @@ __global__ __launch_bounds__(kThreads) void k_sgemm(const float* __restrict__ A,
   using LB = typename std::conditional<TB, LoadKContig<BN, BK, VEC>, LoadMnContig<BN, BK, VEC>>::type;
   const int bz = blockIdx.z;
   const int nk = (K + BK - 1) / BK;
+  // one LDS allocation shared by both call sites below (a static array inside
+  // the tile loop would be instantiated once per call site)
+  __shared__ float lds[2 * BK * (LA::S + LB::S)];
   if (splits > 1) {
     int kt0, kt1;
     split_range(nk, splits, bz, &kt0, &kt1);
     LA la; la.base = A; la.ld = lda; la.rmax = M; la.kmax = K;
     LB lb; lb.base = B; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
     StorePartial sc{ws + (int64_t)bz * M * N, N};
-    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StorePartial>(la, lb, sc, M, N, kt0, kt1,
+    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StorePartial>(lds, la, lb, sc, M, N, kt0, kt1,
                                                               blockIdx.y * BM, blockIdx.x * BN, 0, 0.f);
   } else {
     LA la; la.base = A + bz * sA; la.ld = lda; la.rmax = M; la.kmax = K;
     LB lb; lb.base = B + bz * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
     StoreRowMajor sc{C + bz * sC, ldc};
-    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreRowMajor>(la, lb, sc, M, N, 0, nk, blockIdx.y * BM,
+    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreRowMajor>(lds, la, lb, sc, M, N, 0, nk, blockIdx.y * BM,
                                                                blockIdx.x * BN, act, alpha);
   }
 }
@@ -347,15 +357,16 @@ __global__ __launch_bounds__(kThreads) void k_conv2d(const float* __restrict__ x
   const int n0 = blockIdx.x * BN;
   lb.init(n0);
   const int nk = (K + BK - 1) / BK;
+  __shared__ float lds[2 * BK * (LA::S + LB::S)];
   if (splits > 1) {
     int kt0, kt1;
     split_range(nk, splits, blockIdx.z, &kt0, &kt1);
     StorePartial sc{ws + (int64_t)blockIdx.z * F * g.P, g.P};
-    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StorePartial>(la, lb, sc, F, g.P, kt0, kt1,
+    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StorePartial>(lds, la, lb, sc, F, g.P, kt0, kt1,
                                                               blockIdx.y * BM, n0, 0, 0.f);
   } else {
     StoreNCHW sc{y, F, g.oh * g.ow};
-    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreNCHW>(la, lb, sc, F, g.P, 0, nk, blockIdx.y * BM,
+    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreNCHW>(lds, la, lb, sc, F, g.P, 0, nk, blockIdx.y * BM,
                                                            n0, act, alpha);
   }
 }
@@ -371,6 +382,218 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(const float* __restrict__
     for (int s = 1; s < splits; s++) acc = acc + ws[(int64_t)s * total + e];
     const int i = (int)(e / N), j = (int)(e - (int64_t)i * N);
     sc.put(i, j, act_apply(acc, act, alpha));
+  }
+}
+
+// ---- Conv2d 3x3 / stride 1 with the input staged in LDS -----------------------------
+// Same GEMM view as k_conv2d (M = filters, N = B*oh*ow output pixels in
+// flattened order, K = C*9), but the B operand is not gathered element by
+// element.  Per chunk of CC input channels the block copies into LDS
+//   - the weights of its BM filters for those channels, k-major, and
+//   - every input row its BN pixels touch, as rows of a zero-padded image:
+//     image b contributes H+2p padded rows of W+2p padded columns, stacked over
+//     b, so padded row b*(H+2p) + oy + kr, column ox + kc is tap (kr, kc) of
+//     output pixel (b, oy, ox) and the zero halo needs no test in the hot loop.
+// A lane then fetches its B value with one ds_read at (pixel base + tap offset);
+// the two lane halves of a 32x32x2 MFMA take channels c and c + CC/2 of the same
+// tap, which keeps both operands' offsets lane-constant plus a uniform term.
+// One barrier pair per chunk (CC*9 = 72 k-values) instead of one per 16.
+struct Conv3Geom {
+  int C, H, W, F, oh, ow, pad, P /* B*oh*ow */, B;
+  int Hp, PW;      // padded image height, padded row pitch (W + 2 pad)
+  int R;           // patch rows held in LDS (upper bound over all blocks)
+  int CP;          // floats per channel plane of the patch (R * PW)
+  int K;           // C * 9
+  int nchunks;     // ceil(C / CC)
+};
+
+template <int BM, int BN, int CC, int WAVES_M, int PMAX, bool VEC, class SC>
+__device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const float* __restrict__ w,
+                                           const SC& sc, const Conv3Geom& g, int chunk0, int chunk1,
+                                           int m0, int n0, int act, float alpha) {
+  constexpr int WAVES_N = 4 / WAVES_M;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int KC = CC * 9;          // k-values per chunk
+  constexpr int KHALF = KC / 2;       // MFMA steps per chunk
+  constexpr int SA = BM + 2;          // (BM + 2) % 32 == 2: conflict-free transposing writes
+  constexpr int QPR = KC / 4;         // float4 slots per filter row
+  constexpr int QG = (QPR + 3) / 4;   // groups of four slots
+  constexpr int WTOTAL = BM * QG * 4; // weight float4 slots per chunk (some past QPR)
+  constexpr int NW = (WTOTAL + kThreads - 1) / kThreads;
+  static_assert(CC % 2 == 0 && BM % 32 == 0 && TM >= 1 && TN >= 1, "bad conv tile");
+  extern __shared__ float lds[];
+  float* const As = lds;                       // [KC][SA]
+  float* const Ps = lds + KC * SA;             // [CC][CP]
+  int* const rowoff = reinterpret_cast<int*>(Ps + CC * g.CP);  // [R] offset of the row in x, -1 = zero row
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
+  const int lr = lane & 31, lk = lane >> 5;
+  const int plane = g.oh * g.ow;
+  const int HW = g.H * g.W;
+
+  // padded-row window of this block's pixels
+  const int b_lo = n0 / plane;
+  const int gp_lo = b_lo * g.Hp + (n0 - b_lo * plane) / g.ow;
+  for (int r = threadIdx.x; r < g.R; r += kThreads) {
+    const int gpr = gp_lo + r;
+    const int b = gpr / g.Hp;
+    const int iy = gpr - b * g.Hp - g.pad;
+    rowoff[r] = (b < g.B && iy >= 0 && iy < g.H) ? (b * g.C * g.H + iy) * g.W : -1;
+  }
+  __syncthreads();
+
+  // What each thread copies per chunk never changes except for the channel
+  // base, so it is decoded once: patch element e = tid + j*256 of the
+  // [CC][R][PW] patch comes from x[c0*HW + psrc[j]] (or is a halo zero), and
+  // weight slot f = tid + j*256 from w[wsrc[j] + c0*9].
+  const int patch_total = CC * g.CP;
+  int psrc[PMAX];
+#pragma unroll
+  for (int j = 0; j < PMAX; j++) {
+    const int e = threadIdx.x + j * kThreads;
+    int src = -1;
+    if (e < patch_total) {
+      const int c = e / g.CP;
+      const int rem = e - c * g.CP;
+      const int r = rem / g.PW;
+      const int ix = rem - r * g.PW - g.pad;
+      const int ro = rowoff[r];
+      if (ro >= 0 && ix >= 0 && ix < g.W) src = c * HW + ro + ix;
+    }
+    psrc[j] = src;
+  }
+  int wsrc[NW];   // element offset into w at c0 = 0, -1 = nothing to copy
+  int wdst[NW];   // LDS offset of the slot's first element
+#pragma unroll
+  for (int j = 0; j < NW; j++) {
+    const int f = threadIdx.x + j * kThreads;
+    const int q_lo = f & 3;
+    const int row = (f >> 2) % BM;
+    const int q = ((f >> 2) / BM) * 4 + q_lo;
+    const bool ok = f < WTOTAL && q < QPR && m0 + row < g.F;
+    wsrc[j] = ok ? (m0 + row) * g.K + q * 4 : -1;
+    wdst[j] = (q * 4) * SA + row;
+  }
+
+  // per-lane pixel bases inside the patch (one per MFMA column group)
+  int pbase[TN];
+#pragma unroll
+  for (int t = 0; t < TN; t++) {
+    int j = n0 + wn + t * 32 + lr;
+    j = j < g.P ? j : g.P - 1;
+    const int b = j / plane;
+    const int rem = j - b * plane;
+    const int oy = rem / g.ow, ox = rem - oy * g.ow;
+    pbase[t] = (b * g.Hp + oy - gp_lo) * g.PW + ox + lk * (CC / 2) * g.CP;
+  }
+  const int abase = lk * KHALF * SA + wm + lr;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int a = 0; a < TM; a++)
+#pragma unroll
+    for (int b = 0; b < TN; b++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
+
+  float preg[PMAX];
+  f32x4 wreg[NW];
+  auto stage_load = [&](int chunk) {
+    const int c0 = chunk * CC;
+    const float* xc = x + (int64_t)c0 * HW;
+    const float* wc = w + c0 * 9;
+#pragma unroll
+    for (int j = 0; j < PMAX; j++) preg[j] = psrc[j] >= 0 ? xc[psrc[j]] : 0.f;
+#pragma unroll
+    for (int j = 0; j < NW; j++) {
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (wsrc[j] >= 0) {
+        const float* src = wc + wsrc[j];
+        if (VEC) v = *reinterpret_cast<const f32x4*>(src);
+        else { v[0] = src[0]; v[1] = src[1]; v[2] = src[2]; v[3] = src[3]; }
+      }
+      wreg[j] = v;
+    }
+  };
+  auto stage_store = [&]() {
+#pragma unroll
+    for (int j = 0; j < PMAX; j++) {
+      const int e = threadIdx.x + j * kThreads;
+      if (e < patch_total) Ps[e] = preg[j];
+    }
+#pragma unroll
+    for (int j = 0; j < NW; j++) {
+      const int f = threadIdx.x + j * kThreads;
+      const int q = ((f >> 2) / BM) * 4 + (f & 3);
+      if (f < WTOTAL && q < QPR) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) As[wdst[j] + e * SA] = wreg[j][e];
+      }
+    }
+  };
+
+  if (chunk0 < chunk1) stage_load(chunk0);
+  for (int chunk = chunk0; chunk < chunk1; chunk++) {
+    __syncthreads();           // the previous chunk's LDS reads are done
+    stage_store();
+    __syncthreads();
+    if (chunk + 1 < chunk1) stage_load(chunk + 1);  // in flight during the MFMAs below
+    // ---- MFMA over the chunk: step s pairs k = s (channel s/9) with k = s + KHALF
+    float af[2][TM], bf[2][TN];  // fragments run one step ahead of the MFMAs
+#pragma unroll
+    for (int a = 0; a < TM; a++) af[0][a] = As[abase + a * 32];
+#pragma unroll
+    for (int t = 0; t < TN; t++) bf[0][t] = Ps[pbase[t]];
+#pragma unroll
+    for (int s = 0; s < KHALF; s++) {
+      const int cb = s & 1, nb = cb ^ 1;
+      if (s + 1 < KHALF) {
+        const int s1 = s + 1;
+        const int cs = s1 / 9, tap = s1 % 9, kr = tap / 3, kc = tap % 3;
+        const int boff = cs * g.CP + kr * g.PW + kc;
+#pragma unroll
+        for (int a = 0; a < TM; a++) af[nb][a] = As[abase + s1 * SA + a * 32];
+#pragma unroll
+        for (int t = 0; t < TN; t++) bf[nb][t] = Ps[pbase[t] + boff];
+      }
+#pragma unroll
+      for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int t = 0; t < TN; t++)
+          acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cb][a], bf[cb][t], acc[a][t], 0, 0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int a = 0; a < TM; a++)
+#pragma unroll
+    for (int t = 0; t < TN; t++) {
+      const int j = n0 + wn + t * 32 + lr;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int i = m0 + wm + a * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+        if (i < g.F && j < g.P) sc.put(i, j, act_apply(acc[a][t][v], act, alpha));
+      }
+    }
+}
+
+template <int BM, int BN, int CC, int WAVES_M, int PMAX, bool VEC>
+__global__ __launch_bounds__(kThreads) void k_conv3x3_lds(const float* __restrict__ x,
+                                                          const float* __restrict__ w,
+                                                          float* __restrict__ y, Conv3Geom g, int act,
+                                                          float alpha, int splits,
+                                                          float* __restrict__ ws) {
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  if (splits > 1) {
+    const int per = (g.nchunks + splits - 1) / splits;
+    const int c0 = blockIdx.z * per, c1 = min(g.nchunks, c0 + per);
+    StorePartial sc{ws + (int64_t)blockIdx.z * g.F * g.P, g.P};
+    conv3_tile<BM, BN, CC, WAVES_M, PMAX, VEC, StorePartial>(x, w, sc, g, c0, c1, m0, n0, 0, 0.f);
+  } else {
+    StoreNCHW sc{y, g.F, g.oh * g.ow};
+    conv3_tile<BM, BN, CC, WAVES_M, PMAX, VEC, StoreNCHW>(x, w, sc, g, 0, g.nchunks, m0, n0, act, alpha);
   }
 }
 
@@ -557,6 +780,99 @@ int launch_conv_k(gh_ctx* ctx, const gh_cmd& c, const ConvGeom& g, int F, int K,
   return launch_conv_cfg<BM, BN, WAVES_M, 0, 0>(ctx, c, g, F, K, splits);
 }
 
+// Exact number of padded rows the widest block window needs.
+int conv3_patch_rows(const Conv3Geom& g, int BN) {
+  const int plane = g.oh * g.ow;
+  int best = 0;
+  for (int n0 = 0; n0 < g.P; n0 += BN) {
+    const int pl = (n0 + BN < g.P ? n0 + BN : g.P) - 1;
+    const int b0 = n0 / plane, b1 = pl / plane;
+    const int gp0 = b0 * g.Hp + (n0 - b0 * plane) / g.ow;
+    const int gp1 = b1 * g.Hp + (pl - b1 * plane) / g.ow;
+    const int need = gp1 - gp0 + 3;
+    if (need > best) best = need;
+  }
+  return best;
+}
+
+template <int BM, int BN, int CC, int WAVES_M, int PMAX>
+int launch_conv3_cfg(gh_ctx* ctx, const gh_cmd& c, Conv3Geom g, int splits, size_t lds_bytes) {
+  const bool vec = al16(c.ptr[1]) && g.K % 4 == 0;
+  const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
+  const dim3 grid((g.P + BN - 1) / BN, (g.F + BM - 1) / BM, splits);
+  const float* x = (const float*)(uintptr_t)c.ptr[0];
+  const float* w = (const float*)(uintptr_t)c.ptr[1];
+  float* y = (float*)(uintptr_t)c.ptr[2];
+  float* ws = (float*)ctx->workspace;
+  if (splits > 1 && (int64_t)splits * g.F * g.P * 4 > ctx->workspace_bytes)
+    return gh_fail(ctx, GH_ESTATE, "conv2d: split-K slabs do not fit the workspace");
+  if (vec)
+    hipLaunchKernelGGL((k_conv3x3_lds<BM, BN, CC, WAVES_M, PMAX, true>), grid, dim3(kThreads), lds_bytes,
+                       ctx->stream, x, w, y, g, act, c.f[0], splits, ws);
+  else
+    hipLaunchKernelGGL((k_conv3x3_lds<BM, BN, CC, WAVES_M, PMAX, false>), grid, dim3(kThreads), lds_bytes,
+                       ctx->stream, x, w, y, g, act, c.f[0], splits, ws);
+  int rc = gh_check_hip(ctx, hipGetLastError(), "conv3x3 launch");
+  if (rc || splits <= 1) return rc;
+  const int64_t total = (int64_t)g.F * g.P;
+  int64_t blocks = cdiv(total, 256);
+  if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
+  hipLaunchKernelGGL((k_splitk_reduce<StoreNCHW>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws,
+                     splits, g.F, g.P, StoreNCHW{y, g.F, g.oh * g.ow}, act, c.f[0]);
+  return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
+}
+
+// Returns -1 when the shape is not one the LDS-staged kernel takes.
+int try_launch_conv3(gh_ctx* ctx, const gh_cmd& c) {
+  const int B = (int)c.dim[0], C = (int)c.dim[1], H = (int)c.dim[2], W = (int)c.dim[3], F = (int)c.dim[4];
+  const int pad = (int)c.dim[7];
+  if (c.dim[5] != 3 || c.dim[6] != 3 || c.dim[9] != 1 || c.dim[10] != 1 || c.dim[11] != 1 ||
+      c.dim[12] != 1 || c.dim[8] != pad || pad > 1 || C < 8 || C % 8 != 0)
+    return -1;
+  if (getenv("GORGONIA_HIP_CONV_GATHER")) return -1;  // tuning switch: force the gather kernel
+  Conv3Geom g;
+  g.B = B; g.C = C; g.H = H; g.W = W; g.F = F; g.pad = pad;
+  g.oh = H + 2 * pad - 2; g.ow = W + 2 * pad - 2;
+  if (g.oh <= 0 || g.ow <= 0) return -1;
+  g.P = B * g.oh * g.ow;
+  g.Hp = H + 2 * pad; g.PW = W + 2 * pad;
+  g.K = C * 9;
+  constexpr int CC = 8;
+  g.nchunks = (C + CC - 1) / CC;
+  // Tile choice: 64x64 blocks measured fastest on every 3x3 layer of the
+  // benchmark configurations (more, smaller blocks hide the staging latency
+  // better than 128-wide ones); the channel chunks are split across grid.z
+  // when even those leave the chip under-filled.
+  const int64_t cus = ctx->cu_count;
+  int BM = 64, BN = 64;
+  if (const char* env = getenv("GORGONIA_HIP_CONV_TILE")) {  // tuning override: 0 = 128 wide, 1 = 64x64
+    if (atoi(env) == 0) { BM = F > 64 ? 128 : 64; BN = 128; }
+  }
+  g.R = conv3_patch_rows(g, BN);
+  g.CP = g.R * g.PW;
+  const size_t lds = ((size_t)CC * 9 * (BM + 2) + (size_t)CC * g.CP + g.R) * 4;
+  if (lds > 64 * 1024) return -1;
+  const int per_thread = (CC * g.CP + kThreads - 1) / kThreads;  // patch elements each thread stages
+  if (per_thread > 16) return -1;  // wide images: the gather kernel does better
+  const int64_t blocks = cdiv(F, BM) * cdiv(g.P, BN);
+  int splits = 1;
+  if (const char* env = getenv("GORGONIA_HIP_CONV_SPLITS")) splits = atoi(env);
+  else {
+    splits = (int)((5 * cus / 2 + blocks / 2) / blocks);       // aim at ~2.5 blocks per CU
+    if (splits > g.nchunks / 4) splits = g.nchunks / 4;        // at least 4 chunks per slice
+  }
+  if (splits > g.nchunks) splits = g.nchunks;
+  if (splits < 1) splits = 1;
+  while (splits > 1 && (int64_t)splits * F * g.P * 4 > ctx->workspace_bytes) splits--;
+#define GH_CONV3(BM_, BN_)                                                                        \
+  (per_thread <= 8 ? launch_conv3_cfg<BM_, BN_, CC, 2, 8>(ctx, c, g, splits, lds)                 \
+                   : launch_conv3_cfg<BM_, BN_, CC, 2, 16>(ctx, c, g, splits, lds))
+  if (BN == 64) return GH_CONV3(64, 64);
+  if (BM == 128) return GH_CONV3(128, 128);
+  return GH_CONV3(64, 128);
+#undef GH_CONV3
+}
+
 }  // namespace
 
 int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
@@ -567,6 +883,8 @@ int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
+  const int rc3 = try_launch_conv3(ctx, c);
+  if (rc3 >= 0) return rc3;
   ConvGeom g;
   g.C = (int)c.dim[1]; g.H = (int)c.dim[2]; g.W = (int)c.dim[3];
   g.kh = (int)c.dim[5]; g.kw = (int)c.dim[6];
