@@ -312,6 +312,25 @@ __device__ __forceinline__ void split_range(int nk, int splits, int s, int* kt0,
   *kt1 = min(nk, *kt0 + per);
 }
 
+// Which output tile a workgroup computes.  Workgroup ids are dealt round-robin
+// over the 8 XCDs, each with its own L2, so ids are first regrouped to give
+// every XCD one contiguous range of tiles; inside a range, tiles are walked in
+// groups of 8 tile-rows so that co-resident workgroups share A rows and B
+// columns (a plain row-major walk re-read A and B ~6x from HBM at 4096^3).
+__device__ __forceinline__ void tile_coords(int* tm, int* tn) {
+  const int gx = gridDim.x, gy = gridDim.y;  // tiles along N, along M
+  const int total = gx * gy;
+  int id = blockIdx.y * gx + blockIdx.x;
+  constexpr int kXcd = 8, kGroup = 8;
+  if (total % kXcd == 0) id = (id % kXcd) * (total / kXcd) + id / kXcd;
+  const int per_group = kGroup * gx;
+  const int first_m = (id / per_group) * kGroup;
+  const int gsz = min(gy - first_m, kGroup);
+  const int in_group = id % per_group;
+  *tm = first_m + in_group % gsz;
+  *tn = in_group / gsz;
+}
+
 // blockIdx.z is the batch index (splits == 1) or the split-K slice (batch == 1).
 template <int BM, int BN, int BK, int WAVES_M, bool TA, bool TB, bool VEC>
 __global__ __launch_bounds__(kThreads) void k_sgemm(const float* __restrict__ A,
@@ -324,6 +343,8 @@ __global__ __launch_bounds__(kThreads) void k_sgemm(const float* __restrict__ A,
   using LB = typename std::conditional<TB, LoadKContig<BN, BK, VEC>, LoadMnContig<BN, BK, VEC>>::type;
   const int bz = blockIdx.z;
   const int nk = (K + BK - 1) / BK;
+  int tile_m, tile_n;
+  tile_coords(&tile_m, &tile_n);
   // one LDS allocation shared by both call sites below (a static array inside
   // the tile loop would be instantiated once per call site)
   __shared__ float lds[2 * BK * (LA::S + LB::S)];
@@ -334,13 +355,13 @@ __global__ __launch_bounds__(kThreads) void k_sgemm(const float* __restrict__ A,
     LB lb; lb.base = B; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
     StorePartial sc{ws + (int64_t)bz * M * N, N};
     mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StorePartial>(lds, la, lb, sc, M, N, kt0, kt1,
-                                                              blockIdx.y * BM, blockIdx.x * BN, 0, 0.f);
+                                                              tile_m * BM, tile_n * BN, 0, 0.f);
   } else {
     LA la; la.base = A + bz * sA; la.ld = lda; la.rmax = M; la.kmax = K;
     LB lb; lb.base = B + bz * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
     StoreRowMajor sc{C + bz * sC, ldc};
-    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreRowMajor>(lds, la, lb, sc, M, N, 0, nk, blockIdx.y * BM,
-                                                               blockIdx.x * BN, act, alpha);
+    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreRowMajor>(lds, la, lb, sc, M, N, 0, nk, tile_m * BM,
+                                                               tile_n * BN, act, alpha);
   }
 }
 
