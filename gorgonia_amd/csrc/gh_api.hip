@@ -172,13 +172,29 @@ int gh_memcpy_d2h(gh_ctx* ctx, void* dst, gh_devptr src, int64_t bytes) {
                       "hipMemcpyAsync(D2H)");
 }
 
+// Word copy for small transfers: a kernel node costs less inside a captured
+// graph than a copy-engine node, and it can write pinned host memory too.
+__global__ __launch_bounds__(256) void k_copy_words(uint32_t* __restrict__ dst,
+                                                    const uint32_t* __restrict__ src, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
 int gh_memcpy_d2d(gh_ctx* ctx, gh_devptr dst, gh_devptr src, int64_t bytes) {
   if (!ctx || bytes < 0 || (bytes > 0 && (!dst || !src))) return GH_EINVAL;
   if (ctx->err) return ctx->err;
   if (bytes == 0) return GH_OK;
+  if (bytes <= (1 << 20) && ((dst | src | (uint64_t)bytes) & 3) == 0) {
+    const int64_t n = bytes / 4;
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 256) blocks = 256;
+    hipLaunchKernelGGL(k_copy_words, dim3((int)blocks), dim3(256), 0, ctx->stream,
+                       (uint32_t*)(uintptr_t)dst, (const uint32_t*)(uintptr_t)src, n);
+    return gh_check_hip(ctx, hipGetLastError(), "copy launch");
+  }
   return gh_check_hip(ctx,
                       hipMemcpyAsync((void*)(uintptr_t)dst, (const void*)(uintptr_t)src,
-                                     (size_t)bytes, hipMemcpyDeviceToDevice, ctx->stream),
+                                     (size_t)bytes, hipMemcpyDefault, ctx->stream),
                       "hipMemcpyAsync(D2D)");
 }
 

@@ -406,6 +406,73 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(const float* __restrict__
   }
 }
 
+// ---- small-output GEMM: the K range is split across the wavefronts of one block ------
+// C(M x N) = A(M x K) B(K x N), both row-major, for products whose output has
+// too few 32x32 tiles to fill the chip when each tile walks all of K.  One
+// workgroup of WV wavefronts owns one 32x32 tile; wavefront w takes the 16-wide
+// k-chunks w, w + WV, ... with operands loaded straight from global memory in
+// MFMA lane order (every element is used once per tile, so LDS staging buys
+// nothing), then the WV partial tiles are summed through LDS in wavefront order
+// - a fixed order, so results repeat bit for bit - and the epilogue is applied.
+template <int WV>
+__global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict__ A,
+                                                         const float* __restrict__ B,
+                                                         float* __restrict__ C, int M, int N, int K,
+                                                         int lda, int ldb, int ldc, int act,
+                                                         float alpha, int vec_a) {
+  __shared__ float part[WV * 1024];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+  const int m = m0 + r, n = n0 + r;
+  const int nchunks = (K + 15) / 16;
+  const float* arow = A + (int64_t)m * lda;
+
+  // lane (r, h) feeds k = 16*chunk + 8*h + t at MFMA step t of a chunk
+  auto load = [&](int chunk, float (&a)[8], float (&b)[8]) {
+    const int k0 = chunk * 16 + 8 * h;
+    if (m < M && vec_a && k0 + 8 <= K) {
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(arow + k0);
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(arow + k0 + 4);
+#pragma unroll
+      for (int t = 0; t < 4; t++) { a[t] = lo[t]; a[4 + t] = hi[t]; }
+    } else {
+#pragma unroll
+      for (int t = 0; t < 8; t++) a[t] = (m < M && k0 + t < K) ? arow[k0 + t] : 0.f;
+    }
+#pragma unroll
+    for (int t = 0; t < 8; t++) b[t] = (n < N && k0 + t < K) ? B[(int64_t)(k0 + t) * ldb + n] : 0.f;
+  };
+
+  f32x16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; v++) acc[v] = 0.f;
+  float a[8], b[8], an[8], bn[8];
+  int c = wave;
+  if (c < nchunks) load(c, a, b);
+  for (; c < nchunks; c += WV) {
+    const bool more = c + WV < nchunks;
+    if (more) load(c + WV, an, bn);
+#pragma unroll
+    for (int t = 0; t < 8; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b[t], acc, 0, 0, 0);
+    if (more) {
+#pragma unroll
+      for (int t = 0; t < 8; t++) { a[t] = an[t]; b[t] = bn[t]; }
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 16; v++) part[(wave * 16 + v) * 64 + lane] = acc[v];
+  __syncthreads();
+  for (int e = threadIdx.x; e < 1024; e += WV * 64) {
+    float sum = part[e];
+#pragma unroll
+    for (int w = 1; w < WV; w++) sum = sum + part[w * 1024 + e];
+    const int v = e >> 6, l = e & 63;
+    const int i = m0 + 8 * (v / 4) + 4 * (l >> 5) + (v % 4), j = n0 + (l & 31);
+    if (i < M && j < N) C[(int64_t)i * ldc + j] = act_apply(sum, act, alpha);
+  }
+}
+
 // ---- Conv2d 3x3 / stride 1 with the input staged in LDS -----------------------------
 // Same GEMM view as k_conv2d (M = filters, N = B*oh*ow output pixels in
 // flattened order, K = C*9), but the B operand is not gathered element by
@@ -896,7 +963,28 @@ int try_launch_conv3(gh_ctx* ctx, const gh_cmd& c) {
 
 }  // namespace
 
+// Small-output products (dense layers of a small batch): returns -1 when the
+// shape belongs to the tiled kernel.
+static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t batch = c.dim[6] <= 0 ? 1 : c.dim[6];
+  if (batch != 1 || (c.flags & (GH_FLAG_TRANS_A | GH_FLAG_TRANS_B))) return -1;
+  const int M = (int)c.dim[0], N = (int)c.dim[1], K = (int)c.dim[2];
+  const int64_t tiles = cdiv(M, 32) * cdiv(N, 32);
+  if (tiles > ctx->cu_count || K < 32) return -1;
+  if (getenv("GORGONIA_HIP_GEMM_PLAN")) return -1;  // a forced tile plan means the tiled kernel
+  const int lda = (int)c.dim[3], ldb = (int)c.dim[4], ldc = (int)c.dim[5];
+  const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
+  const int vec_a = al16(c.ptr[0]) && lda % 4 == 0;
+  constexpr int WV = 8;
+  hipLaunchKernelGGL((k_gemm_skinny<WV>), dim3((N + 31) / 32, (M + 31) / 32), dim3(WV * 64), 0, ctx->stream,
+                     (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                     (float*)(uintptr_t)c.ptr[2], M, N, K, lda, ldb, ldc, act, c.f[0], vec_a);
+  return gh_check_hip(ctx, hipGetLastError(), "skinny gemm launch");
+}
+
 int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
+  const int rs = try_launch_gemm_skinny(ctx, c);
+  if (rs >= 0) return rs;
   const int64_t batch = c.dim[6] <= 0 ? 1 : c.dim[6];
   const TilePlan p = plan_tiles(ctx, c.dim[0], c.dim[1], c.dim[2], batch, false);
   if (p.tile == kTile128) return launch_sgemm_cfg<128, 128, 2>(ctx, c, p.splits);

@@ -171,6 +171,23 @@ Status Engine::MemcpyDtoH(void* dst, uint64_t src, int64_t bytes, bool synchrono
   return synchronous ? DoWork() : Status::OK();
 }
 
+Status Engine::HostAlloc(int64_t bytes, void** out) {
+  if (!ctx_) return Status::Err(GH_ESTATE, "engine not initialised");
+  int rc = gh_host_alloc(ctx_, bytes, out);
+  return rc == GH_OK ? Status::OK() : fail(rc, "HostAlloc");
+}
+
+void Engine::HostFree(void* p) {
+  if (ctx_ && p) gh_host_free(ctx_, p);
+}
+
+void Engine::RecordCopy(uint64_t dst, uint64_t src, int64_t bytes) {
+  gh_cmd c{};
+  c.opcode = GH_OP_MEMCPY_D2D;
+  c.ptr[0] = dst; c.ptr[1] = src; c.dim[0] = bytes;
+  Enqueue(c);
+}
+
 // ---- checks (cuda/utils.go:22-112) ---------------------------------------------------
 static Status binaryCheck(const Tensor& a, const Tensor& b) {
   if (a.dt == Dtype::Other) return Status::Err(GH_EINVAL, "Unsupported Dtype for a: " + dtype_name(a.dt));

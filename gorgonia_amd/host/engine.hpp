@@ -107,6 +107,11 @@ class Engine {
   // behind the segment recorded so far.  `synchronous` flushes like Signal().
   Status MemcpyHtoD(uint64_t dst, const void* src, int64_t bytes);
   Status MemcpyDtoH(void* dst, uint64_t src, int64_t bytes, bool synchronous = true);
+  // Pinned host memory the device can write; a copy into it can be recorded in
+  // the segment like any operator (and so be captured and replayed with it).
+  Status HostAlloc(int64_t bytes, void** out);
+  void HostFree(void* p);
+  void RecordCopy(uint64_t dst, uint64_t src, int64_t bytes);
 
   // ---- arithmetic and comparison (cuda/arith.go, cuda/cmp.go) -----------------------
   // fn is a gh_binfn.  Tensor-tensor form: Add/Sub/Mul/Div/Pow/Lt/Lte/Gt/Gte/ElEq/ElNe.

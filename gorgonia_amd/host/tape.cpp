@@ -6,6 +6,9 @@
 
 namespace gorgonia {
 
+// outputs up to this size leave through a pinned staging buffer
+static constexpr int64_t kStageLimit = 1 << 20;
+
 static Status bad(const std::string& m) { return Status::Err(GH_EINVAL, m); }
 
 static int64_t conv_out(int64_t in, int64_t k, int64_t pad, int64_t stride, int64_t dil) {
@@ -444,6 +447,10 @@ Status TapeMachine::Compile() {
   }
   // host reads: one flush, then the copies (compile.go:437-462 puts a flush in
   // front of every consumer that needs a finished value)
+  for (int i = 0; i < N; i++)
+    if (nodes[(size_t)i].read_into && bytes_of(nodes[(size_t)i]) <= kStageLimit &&
+        bytes_of(nodes[(size_t)i]) % 4 == 0)
+      prog_.push_back({InstrKind::StageOut, i, node_reg_[(size_t)i], bytes_of(nodes[(size_t)i]), false});
   prog_.push_back({InstrKind::Flush, -1, -1, 0, false});
   std::vector<int> freed;
   for (int i = 0; i < N; i++)
@@ -472,7 +479,15 @@ Status TapeMachine::Init(int device) {
   int64_t need = 0;
   for (auto& in : prog_)
     if (in.kind == InstrKind::Alloc) need += (in.size + 31) / 32 * 32;
-  return eng_.Init(device, need > gpumem_ ? need : gpumem_);
+  st = eng_.Init(device, need > gpumem_ ? need : gpumem_);
+  if (!st.ok()) return st;
+  stage_.assign(g_->Nodes().size(), nullptr);
+  for (auto& in : prog_)
+    if (in.kind == InstrKind::StageOut) {
+      st = eng_.HostAlloc(in.size, &stage_[(size_t)in.node]);
+      if (!st.ok()) return st;
+    }
+  return Status::OK();
 }
 
 uint64_t TapeMachine::RegisterAddress(int node) const {
@@ -577,8 +592,16 @@ Status TapeMachine::RunAll() {
         st = flush();
         if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": flush");
         break;
+      case InstrKind::StageOut:
+        eng_.RecordCopy((uint64_t)(uintptr_t)stage_[(size_t)in.node], regs_[(size_t)in.reg].mem, in.size);
+        break;
       case InstrKind::Read: {
         Node& n = nodes[(size_t)in.node];
+        if (in.node < (int)stage_.size() && stage_[(size_t)in.node]) {
+          // the flush in front of the reads has waited for the staging copy
+          std::memcpy(n.read_into, stage_[(size_t)in.node], (size_t)in.size);
+          break;
+        }
         st = eng_.MemcpyDtoH(n.read_into, regs_[(size_t)in.reg].mem, in.size, false);
         if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": read");
         bool last = pc + 1 >= prog_.size() || prog_[pc + 1].kind != InstrKind::Read;
@@ -610,10 +633,16 @@ Status TapeMachine::Reset() {
   return Status::OK();
 }
 
-Status TapeMachine::Close() { return eng_.Close(); }
+Status TapeMachine::Close() {
+  for (void*& p : stage_) {
+    eng_.HostFree(p);
+    p = nullptr;
+  }
+  return eng_.Close();
+}
 
 std::string TapeMachine::ProgramString() const {
-  static const char* names[] = {"loadArg", "alloc", "devTrans", "execOp", "free", "flush", "read"};
+  static const char* names[] = {"loadArg", "alloc", "devTrans", "execOp", "free", "flush", "read", "stageOut"};
   std::ostringstream os;
   os << "Instructions:\n";
   const auto& nodes = g_->Nodes();

@@ -92,7 +92,7 @@ class Graph {
   std::vector<Node> nodes_;
 };
 
-enum class InstrKind : int32_t { LoadArg, Alloc, Transport, ExecOp, Free, Flush, Read };
+enum class InstrKind : int32_t { LoadArg, Alloc, Transport, ExecOp, Free, Flush, Read, StageOut };
 
 struct Instr {
   InstrKind kind;
@@ -136,6 +136,10 @@ class TapeMachine {
   std::vector<int> node_reg_;      // node -> register
   std::vector<char> reg_live_;     // register currently holds arena memory
   std::vector<char> resident_done_;
+  // Small outputs leave through pinned host buffers written by a copy at the
+  // end of the segment, so a replayed run is one graph launch and one wait;
+  // node -> buffer (null: the output is read with a D2H copy after the flush).
+  std::vector<void*> stage_;
   int64_t gpumem_ = 0;
   int runs_ = 0, segments_ = 0, graph_launches_ = 0;
   // per-segment replay cache
