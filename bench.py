@@ -163,6 +163,28 @@ def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=Tr
     return dt / steps * 1e3, result, inp, launches
 
 
+def bench_yolo(steps, warmup):
+    """Config 5: Tiny-YOLO-v2-shaped forward, batch 8 x 3 x 416 x 416, on the tape
+    machine with conv+BatchNorm+LeakyReLU(+MaxPool) folded, graph replay,
+    weights and input resident."""
+    from gorgonia_amd import configs, graph as G
+    inp = configs.yolo_inputs(8, 416)
+    g, outs = configs.build_yolo(inp, resident_input=True)
+    m = G.NewTapeMachine(g, graph_replay=True, fuse_activations=True)
+    for _ in range(max(warmup, 3)):
+        m.RunAll()
+    eng = m.engine()
+    eng.DoWork()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        m.RunAll()
+    eng.DoWork()
+    dt = time.perf_counter() - t0
+    result = outs["out"].copy()
+    m.Close()
+    return dt / steps * 1e3, result, inp
+
+
 def cpu_baseline_convnet(inp, budget_s=12.0):
     """The CPU oracle's forward pass of the same configuration on the host cores."""
     from oracle import binding as O, forward as F
@@ -214,7 +236,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of: convnet,elementwise,linalg")
+    ap.add_argument("--only", default="", help="comma list of: convnet,elementwise,linalg,yolo")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this engine runs on one GPU; --gpus must be 1 (no multi-GPU path is built)")
@@ -230,6 +252,13 @@ def main():
     log(f"convnet: {ms_step:.4f} ms/step  {images_s:.0f} images/s  (graph launches {launches})")
     ms_h2d, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False)
     ms_eager, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, graph_replay=False)
+
+    yolo = None
+    if not only or "yolo" in only:
+        ms_yolo, yolo_out, yolo_inp = bench_yolo(max(20, a.steps // 4), a.warmup)
+        yolo = {"ms_per_step": round(ms_yolo, 4), "images_s": round(8 / ms_yolo * 1e3, 1),
+                "TFLOPs": round(31_080_857_600 / ms_yolo / 1e9, 2), "flop_per_step": 31_080_857_600}
+        log(f"yolo-shaped: {ms_yolo:.4f} ms/step  {8 / ms_yolo * 1e3:.0f} images/s")
 
     iters = 30
     conv_k = bench_convnet_kernels(ctx, 128, iters) if not only or "convnet" in only else {}
@@ -256,6 +285,18 @@ def main():
         cpu = {"value": round(cpu_images_s, 1), "unit": "images/s", "cores": threads, "kind": "port",
                "sample": f"{reps} forward passes of the same 128-image batch (CPU oracle, OpenMP)"}
         cpu.update(cpu_baseline_micro())
+        if yolo is not None:
+            from oracle import binding as O, forward as F
+            O.set_threads(threads)
+            t0 = time.perf_counter()
+            yref = F.yolo(yolo_inp)
+            ydt = time.perf_counter() - t0
+            O.set_threads(1)
+            cpu["yolo_images_s"] = round(8 / ydt, 2)
+            cpu["yolo_sample"] = f"1 forward pass of the same 8-image batch, {threads} threads"
+            yerr = float(np.linalg.norm(yolo_out.astype(np.float64) - yref) / np.linalg.norm(yref))
+            parity["yolo_rel_frobenius_vs_oracle"] = yerr
+            parity["ok"] = parity["ok"] and yerr <= 1e-5
 
     line = {
         "metric": "convnet fwd images/s (1 GPU); elementwise HBM GB/s; SGEMM TFLOP/s",
@@ -276,7 +317,7 @@ def main():
             "convnet_ms_per_step_with_input_h2d": round(ms_h2d, 5),
             "convnet_images_s_with_input_h2d": round(128 / ms_h2d * 1e3, 1),
             "convnet_ms_per_step_eager_no_graph": round(ms_eager, 5),
-            "convnet_kernels": conv_k, "elementwise": elem, "linalg": lin, "parity": parity,
+            "yolo_shaped_forward": yolo, "convnet_kernels": conv_k, "elementwise": elem, "linalg": lin, "parity": parity,
         },
     }
     print(json.dumps(line), flush=True)

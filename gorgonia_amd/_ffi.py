@@ -37,6 +37,8 @@ FLAG_HAS_GAMMA = 1 << 20
 FLAG_HAS_BETA = 1 << 21
 FLAG_ACT_RELU = 1 << 22
 FLAG_ACT_LEAKY = 1 << 23
+FLAG_CONV_BN = 1 << 24
+FLAG_CONV_POOL2 = 1 << 25
 
 
 def flag_fn(f):
@@ -52,7 +54,7 @@ def flag_dtype(d):
 
 
 class GhCmd(C.Structure):
-    _fields_ = [("opcode", C.c_uint32), ("flags", C.c_uint32), ("ptr", C.c_uint64 * 6),
+    _fields_ = [("opcode", C.c_uint32), ("flags", C.c_uint32), ("ptr", C.c_uint64 * 8),
                 ("dim", C.c_int64 * 16), ("f", C.c_float * 4)]
 
 
@@ -82,6 +84,7 @@ SYMBOLS = {
     "gh_memcpy_d2d": (C.c_int, [_P, C.c_uint64, C.c_uint64, C.c_int64]),
     "gh_submit": (C.c_int, [_P, C.POINTER(GhCmd), C.c_int]),
     "gh_validate": (C.c_int, [C.POINTER(GhCmd), C.c_int, C.c_char_p, C.c_int]),
+    "gh_conv2d_can_pool": (C.c_int, [C.POINTER(GhCmd)]),
     "gh_sync": (C.c_int, [_P]),
     "gh_graph_begin": (C.c_int, [_P]),
     "gh_graph_end": (C.c_int, [_P, C.POINTER(C.c_int)]),

@@ -105,15 +105,14 @@ def build_convnet(inp, resident=True):
     return g, {"out": G.Read(out)}
 
 
-def build_yolo(inp, resident=True):
+def build_yolo(inp, resident=True, resident_input=False):
     g = G.NewGraph()
-    h = G.NewTensor(g, inp["x"])
+    h = G.NewTensor(g, inp["x"], resident_input)
     for i in range(7):
         w = G.NewTensor(g, inp[f"w{i}"], resident)
         h = G.Conv2d(h, w, (3, 3), (1, 1), (1, 1), (1, 1))
-        if True:
-            m, v, ga, be = (G.NewTensor(g, inp[f"{k}{i}"], resident) for k in ("mean", "var", "gamma", "beta"))
-            h = G.BatchNorm(h, ga, be, m, v, 1e-5)
+        m, v, ga, be = (G.NewTensor(g, inp[f"{k}{i}"], resident) for k in ("mean", "var", "gamma", "beta"))
+        h = G.BatchNorm(h, ga, be, m, v, 1e-5)
         h = G.LeakyRelu(h, 0.1)
         if i < 5:
             h = G.MaxPool2D(h, (2, 2), (0, 0), (2, 2))

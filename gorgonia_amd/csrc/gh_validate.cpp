@@ -80,6 +80,13 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
         return bad("conv2d: tensor too large for 32-bit indexing");
       if ((c.flags & GH_FLAG_ACT_RELU) && (c.flags & GH_FLAG_ACT_LEAKY))
         return bad("conv2d: two activations requested");
+      if (c.flags & GH_FLAG_CONV_BN) {
+        if (!c.ptr[3] || !c.ptr[4]) return bad("conv2d: fused BatchNorm needs mean and variance");
+        if ((c.flags & GH_FLAG_HAS_GAMMA) && !c.ptr[5]) return bad("conv2d: fused BatchNorm gamma is null");
+        if ((c.flags & GH_FLAG_HAS_BETA) && !c.ptr[6]) return bad("conv2d: fused BatchNorm beta is null");
+      }
+      if ((c.flags & GH_FLAG_CONV_POOL2) && !gh_conv2d_can_pool(&c))
+        return bad("conv2d: no fused pooling for this shape");
       return GH_OK;
     }
     case GH_OP_MAXPOOL2D: {

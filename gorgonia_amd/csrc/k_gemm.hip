@@ -43,6 +43,27 @@ __device__ __forceinline__ float act_apply(float v, int act, float alpha) {
   return v;
 }
 
+// Operators riding in a convolution's epilogue, applied per stored value in this
+// order: BatchNorm in eval mode with BN_INFER's arithmetic (op_nn.go:1559-1584:
+// a = 1/sqrt(var+eps), b = -mean*a, y = x*a + b, then gamma*y, then + beta, each
+// step rounded), then the activation.  Null mean: no BatchNorm.
+struct ConvTail {
+  const float* mean; const float* var; const float* gamma; const float* beta;
+  float eps; int act; float alpha;
+};
+
+__device__ __forceinline__ float tail_apply(const ConvTail& t, int f, float v) {
+  if (t.mean) {
+    const float a = 1.0f / sqrtf(t.var[f] + t.eps);
+    const float b = -t.mean[f] * a;
+    v = v * a;
+    v = v + b;
+    if (t.gamma) v = t.gamma[f] * v;
+    if (t.beta) v = v + t.beta[f];
+  }
+  return act_apply(v, t.act, t.alpha);
+}
+
 // ---- operand loaders ---------------------------------------------------------
 // A loader moves one R x BK (or BK x R) operand tile: load() global->registers,
 // store() registers->LDS in k-major order with row stride S.
@@ -209,9 +230,10 @@ struct StoreRowMajor {
 // Conv result: row i = filter, column j = output pixel (b, oy, ox) -> NCHW.
 struct StoreNCHW {
   float* y; int F; int plane /* oh*ow */;
+  ConvTail tail;
   __device__ __forceinline__ void put(int i, int j, float v) const {
     const int b = j / plane, p = j - b * plane;
-    y[((int64_t)b * F + i) * plane + p] = v;
+    y[((int64_t)b * F + i) * plane + p] = tail_apply(tail, i, v);
   }
 };
 
@@ -295,11 +317,11 @@ __device__ __forceinline__ void mfma_tile_loop(float* lds, LA& la, LB& lb, const
 #pragma unroll
   for (int a = 0; a < TM; a++)
 #pragma unroll
-    for (int b = 0; b < TN; b++) {
-      const int j = n0 + wn + b * 32 + lr;
+    for (int v = 0; v < 16; v++) {
+      const int i = m0 + wm + a * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
 #pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const int i = m0 + wm + a * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+      for (int b = 0; b < TN; b++) {
+        const int j = n0 + wn + b * 32 + lr;
         if (i < M && j < N) sc.put(i, j, act_apply(acc[a][b][v], act, alpha));
       }
     }
@@ -369,7 +391,7 @@ template <int BM, int BN, int BK, int WAVES_M, int KH, int KW, bool VEC>
 __global__ __launch_bounds__(kThreads) void k_conv2d(const float* __restrict__ x,
                                                      const float* __restrict__ w,
                                                      float* __restrict__ y, ConvGeom g, int F, int K,
-                                                     int act, float alpha, int splits,
+                                                     ConvTail tail, int splits,
                                                      float* __restrict__ ws) {
   using LA = LoadKContig<BM, BK, VEC>;
   using LB = LoadIm2col<BN, BK, KH, KW>;
@@ -386,9 +408,9 @@ __global__ __launch_bounds__(kThreads) void k_conv2d(const float* __restrict__ x
     mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StorePartial>(lds, la, lb, sc, F, g.P, kt0, kt1,
                                                               blockIdx.y * BM, n0, 0, 0.f);
   } else {
-    StoreNCHW sc{y, F, g.oh * g.ow};
+    StoreNCHW sc{y, F, g.oh * g.ow, tail};
     mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreNCHW>(lds, la, lb, sc, F, g.P, 0, nk, blockIdx.y * BM,
-                                                           n0, act, alpha);
+                                                           n0, 0, 0.f);
   }
 }
 
@@ -420,7 +442,9 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
                                                          float* __restrict__ C, int M, int N, int K,
                                                          int lda, int ldb, int ldc, int act,
                                                          float alpha, int vec_a) {
-  __shared__ float part[WV * 1024];
+  constexpr int G = 4;                       // k-chunks whose loads are in flight together
+  constexpr int HALF = WV / 2;
+  __shared__ float part[HALF * 1024];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 31, h = lane >> 5;
   const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
@@ -447,26 +471,38 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
   f32x16 acc;
 #pragma unroll
   for (int v = 0; v < 16; v++) acc[v] = 0.f;
-  float a[8], b[8], an[8], bn[8];
-  int c = wave;
-  if (c < nchunks) load(c, a, b);
-  for (; c < nchunks; c += WV) {
-    const bool more = c + WV < nchunks;
-    if (more) load(c + WV, an, bn);
+  for (int c = wave; c < nchunks; c += G * WV) {
+    float a[G][8], b[G][8];
 #pragma unroll
-    for (int t = 0; t < 8; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b[t], acc, 0, 0, 0);
-    if (more) {
+    for (int g = 0; g < G; g++)
+      if (c + g * WV < nchunks) load(c + g * WV, a[g], b[g]);
 #pragma unroll
-      for (int t = 0; t < 8; t++) { a[t] = an[t]; b[t] = bn[t]; }
+    for (int g = 0; g < G; g++)
+      if (c + g * WV < nchunks) {
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[g][t], b[g][t], acc, 0, 0, 0);
+      }
+  }
+  // upper half of the wavefronts hands its tiles to the lower half, then the
+  // HALF sums are added in wavefront order
+  if (wave >= HALF) {
+#pragma unroll
+    for (int v = 0; v < 16; v++) part[((wave - HALF) * 16 + v) * 64 + lane] = acc[v];
+  }
+  __syncthreads();
+  if (wave < HALF) {
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int at = (wave * 16 + v) * 64 + lane;
+      part[at] = acc[v] + part[at];
     }
   }
-#pragma unroll
-  for (int v = 0; v < 16; v++) part[(wave * 16 + v) * 64 + lane] = acc[v];
   __syncthreads();
   for (int e = threadIdx.x; e < 1024; e += WV * 64) {
     float sum = part[e];
 #pragma unroll
-    for (int w = 1; w < WV; w++) sum = sum + part[w * 1024 + e];
+    for (int w = 1; w < HALF; w++) sum = sum + part[w * 1024 + e];
     const int v = e >> 6, l = e & 63;
     const int i = m0 + 8 * (v / 4) + 4 * (l >> 5) + (v % 4), j = n0 + (l & 31);
     if (i < M && j < N) C[(int64_t)i * ldc + j] = act_apply(sum, act, alpha);
@@ -657,11 +693,11 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
 #pragma unroll
   for (int a = 0; a < TM; a++)
 #pragma unroll
-    for (int t = 0; t < TN; t++) {
-      const int j = n0 + wn + t * 32 + lr;
+    for (int v = 0; v < 16; v++) {
+      const int i = m0 + wm + a * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
 #pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const int i = m0 + wm + a * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+      for (int t = 0; t < TN; t++) {
+        const int j = n0 + wn + t * 32 + lr;
         if (i < g.F && j < g.P) sc.put(i, j, act_apply(acc[a][t][v], act, alpha));
       }
     }
@@ -670,8 +706,8 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
 template <int BM, int BN, int CC, int WAVES_M, int PMAX, bool VEC>
 __global__ __launch_bounds__(kThreads) void k_conv3x3_lds(const float* __restrict__ x,
                                                           const float* __restrict__ w,
-                                                          float* __restrict__ y, Conv3Geom g, int act,
-                                                          float alpha, int splits,
+                                                          float* __restrict__ y, Conv3Geom g,
+                                                          ConvTail tail, int splits,
                                                           float* __restrict__ ws) {
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   if (splits > 1) {
@@ -680,8 +716,76 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_lds(const float* __restric
     StorePartial sc{ws + (int64_t)blockIdx.z * g.F * g.P, g.P};
     conv3_tile<BM, BN, CC, WAVES_M, PMAX, VEC, StorePartial>(x, w, sc, g, c0, c1, m0, n0, 0, 0.f);
   } else {
-    StoreNCHW sc{y, g.F, g.oh * g.ow};
-    conv3_tile<BM, BN, CC, WAVES_M, PMAX, VEC, StoreNCHW>(x, w, sc, g, 0, g.nchunks, m0, n0, act, alpha);
+    StoreNCHW sc{y, g.F, g.oh * g.ow, tail};
+    conv3_tile<BM, BN, CC, WAVES_M, PMAX, VEC, StoreNCHW>(x, w, sc, g, 0, g.nchunks, m0, n0, 0, 0.f);
+  }
+}
+
+// ---- Conv2d 3x3 / stride 1 over a few input channels, on the vector ALUs ------------
+// With C*9 <= 36 the contraction is too short for the matrix cores to pay, and
+// the layer is bound by writing y.  One thread owns one stored pixel: it holds
+// the input patch in registers, walks this workgroup's filters (weights are
+// uniform across the wavefront, so they come through scalar loads) and applies
+// the epilogue.  With WS == 2 the stored pixel is the 2x2/stride-2 max-pool
+// window of four convolution results (scan order and strict > of the pooling
+// kernel), which cuts the bytes written by four.
+template <int C, int WS>
+__global__ __launch_bounds__(256) void k_conv3x3_direct(const float* __restrict__ x,
+                                                        const float* __restrict__ w,
+                                                        float* __restrict__ y, int B, int H, int W,
+                                                        int F, int pad, int yh, int yw, int fper,
+                                                        ConvTail tail) {
+  constexpr int PS = WS + 2;
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= (int64_t)B * yh * yw) return;
+  const int px = (int)(t % yw), py = (int)((t / yw) % yh), b = (int)(t / ((int64_t)yw * yh));
+  const int iy0 = py * WS - pad, ix0 = px * WS - pad;
+  float patch[C][PS][PS];
+#pragma unroll
+  for (int c = 0; c < C; c++)
+#pragma unroll
+    for (int r = 0; r < PS; r++)
+#pragma unroll
+      for (int q = 0; q < PS; q++) {
+        const int iy = iy0 + r, ix = ix0 + q;
+        const bool in = iy >= 0 && iy < H && ix >= 0 && ix < W;
+        patch[c][r][q] = in ? x[(((int64_t)b * C + c) * H + iy) * W + ix] : 0.f;
+      }
+  const int f0 = blockIdx.y * fper, f1 = min(F, f0 + fper);
+  for (int f = f0; f < f1; f++) {
+    const float* wf = w + (int64_t)f * (C * 9);
+    float acc[WS][WS];
+#pragma unroll
+    for (int dy = 0; dy < WS; dy++)
+#pragma unroll
+      for (int dx = 0; dx < WS; dx++) acc[dy][dx] = 0.f;
+#pragma unroll
+    for (int c = 0; c < C; c++)
+#pragma unroll
+      for (int kr = 0; kr < 3; kr++)
+#pragma unroll
+        for (int kc = 0; kc < 3; kc++) {
+          const float wv = wf[(c * 3 + kr) * 3 + kc];
+#pragma unroll
+          for (int dy = 0; dy < WS; dy++)
+#pragma unroll
+            for (int dx = 0; dx < WS; dx++)
+              acc[dy][dx] = __builtin_fmaf(patch[c][dy + kr][dx + kc], wv, acc[dy][dx]);
+        }
+    float out;
+    if (WS == 2) {
+      out = -3.402823466e+38f;
+#pragma unroll
+      for (int dy = 0; dy < WS; dy++)
+#pragma unroll
+        for (int dx = 0; dx < WS; dx++) {
+          const float v = tail_apply(tail, f, acc[dy][dx]);
+          if (v > out) out = v;
+        }
+    } else {
+      out = tail_apply(tail, f, acc[0][0]);
+    }
+    y[(((int64_t)b * F + f) * yh + py) * yw + px] = out;
   }
 }
 
@@ -745,6 +849,20 @@ inline bool al16(uint64_t p) { return (p & 15u) == 0; }
 // grid.z and a second kernel sums the slabs.
 enum { kTile128 = 0, kTile64 = 1, kTile32x256 = 2 };
 struct TilePlan { int tile; int splits; };
+
+inline ConvTail conv_tail(const gh_cmd& c) {
+  ConvTail t{};
+  if (c.flags & GH_FLAG_CONV_BN) {
+    t.mean = (const float*)(uintptr_t)c.ptr[3];
+    t.var = (const float*)(uintptr_t)c.ptr[4];
+    t.gamma = (c.flags & GH_FLAG_HAS_GAMMA) ? (const float*)(uintptr_t)c.ptr[5] : nullptr;
+    t.beta = (c.flags & GH_FLAG_HAS_BETA) ? (const float*)(uintptr_t)c.ptr[6] : nullptr;
+    t.eps = c.f[1];
+  }
+  t.act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
+  t.alpha = c.f[0];
+  return t;
+}
 
 inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
@@ -837,7 +955,7 @@ template <int BM, int BN, int WAVES_M, int KH, int KW>
 int launch_conv_cfg(gh_ctx* ctx, const gh_cmd& c, const ConvGeom& g, int F, int K, int splits) {
   constexpr int BK = 16;
   const bool vec = al16(c.ptr[1]) && K % 4 == 0;
-  const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
+  const ConvTail tail = conv_tail(c);
   const dim3 grid((g.P + BN - 1) / BN, (F + BM - 1) / BM, splits);
   const float* x = (const float*)(uintptr_t)c.ptr[0];
   const float* w = (const float*)(uintptr_t)c.ptr[1];
@@ -847,17 +965,17 @@ int launch_conv_cfg(gh_ctx* ctx, const gh_cmd& c, const ConvGeom& g, int F, int 
     return gh_fail(ctx, GH_ESTATE, "conv2d: split-K slabs do not fit the workspace");
   if (vec)
     hipLaunchKernelGGL((k_conv2d<BM, BN, BK, WAVES_M, KH, KW, true>), grid, dim3(kThreads), 0,
-                       ctx->stream, x, w, y, g, F, K, act, c.f[0], splits, ws);
+                       ctx->stream, x, w, y, g, F, K, tail, splits, ws);
   else
     hipLaunchKernelGGL((k_conv2d<BM, BN, BK, WAVES_M, KH, KW, false>), grid, dim3(kThreads), 0,
-                       ctx->stream, x, w, y, g, F, K, act, c.f[0], splits, ws);
+                       ctx->stream, x, w, y, g, F, K, tail, splits, ws);
   int rc = gh_check_hip(ctx, hipGetLastError(), "conv2d launch");
   if (rc || splits <= 1) return rc;
   const int64_t total = (int64_t)F * g.P;
   int64_t blocks = cdiv(total, 256);
   if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
   hipLaunchKernelGGL((k_splitk_reduce<StoreNCHW>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws,
-                     splits, F, g.P, StoreNCHW{y, F, g.oh * g.ow}, act, c.f[0]);
+                     splits, F, g.P, StoreNCHW{y, F, g.oh * g.ow, tail}, 0, 0.f);
   return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
 }
 
@@ -886,7 +1004,7 @@ int conv3_patch_rows(const Conv3Geom& g, int BN) {
 template <int BM, int BN, int CC, int WAVES_M, int PMAX>
 int launch_conv3_cfg(gh_ctx* ctx, const gh_cmd& c, Conv3Geom g, int splits, size_t lds_bytes) {
   const bool vec = al16(c.ptr[1]) && g.K % 4 == 0;
-  const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
+  const ConvTail tail = conv_tail(c);
   const dim3 grid((g.P + BN - 1) / BN, (g.F + BM - 1) / BM, splits);
   const float* x = (const float*)(uintptr_t)c.ptr[0];
   const float* w = (const float*)(uintptr_t)c.ptr[1];
@@ -896,17 +1014,17 @@ int launch_conv3_cfg(gh_ctx* ctx, const gh_cmd& c, Conv3Geom g, int splits, size
     return gh_fail(ctx, GH_ESTATE, "conv2d: split-K slabs do not fit the workspace");
   if (vec)
     hipLaunchKernelGGL((k_conv3x3_lds<BM, BN, CC, WAVES_M, PMAX, true>), grid, dim3(kThreads), lds_bytes,
-                       ctx->stream, x, w, y, g, act, c.f[0], splits, ws);
+                       ctx->stream, x, w, y, g, tail, splits, ws);
   else
     hipLaunchKernelGGL((k_conv3x3_lds<BM, BN, CC, WAVES_M, PMAX, false>), grid, dim3(kThreads), lds_bytes,
-                       ctx->stream, x, w, y, g, act, c.f[0], splits, ws);
+                       ctx->stream, x, w, y, g, tail, splits, ws);
   int rc = gh_check_hip(ctx, hipGetLastError(), "conv3x3 launch");
   if (rc || splits <= 1) return rc;
   const int64_t total = (int64_t)g.F * g.P;
   int64_t blocks = cdiv(total, 256);
   if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
   hipLaunchKernelGGL((k_splitk_reduce<StoreNCHW>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws,
-                     splits, g.F, g.P, StoreNCHW{y, g.F, g.oh * g.ow}, act, c.f[0]);
+                     splits, g.F, g.P, StoreNCHW{y, g.F, g.oh * g.ow, tail}, 0, 0.f);
   return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
 }
 
@@ -975,7 +1093,7 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   const int lda = (int)c.dim[3], ldb = (int)c.dim[4], ldc = (int)c.dim[5];
   const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
   const int vec_a = al16(c.ptr[0]) && lda % 4 == 0;
-  constexpr int WV = 8;
+  constexpr int WV = 8;  // 512 threads leave each wavefront 256 registers for the grouped loads
   hipLaunchKernelGGL((k_gemm_skinny<WV>), dim3((N + 31) / 32, (M + 31) / 32), dim3(WV * 64), 0, ctx->stream,
                      (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
                      (float*)(uintptr_t)c.ptr[2], M, N, K, lda, ldb, ldc, act, c.f[0], vec_a);
@@ -991,7 +1109,55 @@ int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
   return launch_sgemm_cfg<64, 64, 2>(ctx, c, p.splits);
 }
 
+// The direct kernel's shapes: 3x3, stride 1, no dilation, square padding, at
+// most four input channels.
+static bool conv_direct_shape(const gh_cmd& c) {
+  return c.dim[5] == 3 && c.dim[6] == 3 && c.dim[9] == 1 && c.dim[10] == 1 && c.dim[11] == 1 &&
+         c.dim[12] == 1 && c.dim[7] == c.dim[8] && c.dim[1] >= 1 && c.dim[1] <= 4;
+}
+
+static int launch_conv_direct(gh_ctx* ctx, const gh_cmd& c) {
+  const int B = (int)c.dim[0], C = (int)c.dim[1], H = (int)c.dim[2], W = (int)c.dim[3], F = (int)c.dim[4];
+  const int pad = (int)c.dim[7];
+  const int oh = H + 2 * pad - 2, ow = W + 2 * pad - 2;
+  const bool pool = c.flags & GH_FLAG_CONV_POOL2;
+  const int yh = pool ? oh / 2 : oh, yw = pool ? ow / 2 : ow;
+  const int64_t pix = (int64_t)B * yh * yw;
+  if (pix == 0 || F == 0) return GH_OK;
+  const int64_t bx = cdiv(pix, 256);
+  // enough filter groups to give every SIMD a few wavefronts, at least 4 filters each
+  int64_t groups = cdiv((int64_t)ctx->cu_count * 16, bx * 4);
+  if (groups > F / 4) groups = F / 4;
+  if (groups < 1) groups = 1;
+  const int fper = (int)cdiv(F, groups);
+  const dim3 grid((unsigned)bx, (unsigned)cdiv(F, fper));
+  const float* x = (const float*)(uintptr_t)c.ptr[0];
+  const float* w = (const float*)(uintptr_t)c.ptr[1];
+  float* y = (float*)(uintptr_t)c.ptr[2];
+  const ConvTail tail = conv_tail(c);
+#define GH_DIRECT(C_)                                                                                \
+  do {                                                                                               \
+    if (pool)                                                                                        \
+      hipLaunchKernelGGL((k_conv3x3_direct<C_, 2>), grid, dim3(256), 0, ctx->stream, x, w, y, B, H, W, \
+                         F, pad, yh, yw, fper, tail);                                                \
+    else                                                                                             \
+      hipLaunchKernelGGL((k_conv3x3_direct<C_, 1>), grid, dim3(256), 0, ctx->stream, x, w, y, B, H, W, \
+                         F, pad, yh, yw, fper, tail);                                                \
+  } while (0)
+  switch (C) {
+    case 1: GH_DIRECT(1); break;
+    case 2: GH_DIRECT(2); break;
+    case 3: GH_DIRECT(3); break;
+    default: GH_DIRECT(4); break;
+  }
+#undef GH_DIRECT
+  return gh_check_hip(ctx, hipGetLastError(), "direct conv launch");
+}
+
 int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
+  if (conv_direct_shape(c) && !getenv("GORGONIA_HIP_CONV_NO_DIRECT")) return launch_conv_direct(ctx, c);
+  if (c.flags & GH_FLAG_CONV_POOL2)
+    return gh_fail(ctx, GH_EINVAL, "conv2d: no fused pooling for this shape (see gh_conv2d_can_pool)");
   const int rc3 = try_launch_conv3(ctx, c);
   if (rc3 >= 0) return rc3;
   ConvGeom g;
@@ -1032,4 +1198,10 @@ int gh_launch_outer(gh_ctx* ctx, const gh_cmd& c) {
                      (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
                      (float*)(uintptr_t)c.ptr[2], m, n);
   return gh_check_hip(ctx, hipGetLastError(), "outer launch");
+}
+
+extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {
+  if (!c || c->opcode != GH_OP_CONV2D || !conv_direct_shape(*c)) return 0;
+  const int64_t oh = c->dim[2] + 2 * c->dim[7] - 2, ow = c->dim[3] + 2 * c->dim[7] - 2;
+  return oh >= 2 && ow >= 2;
 }

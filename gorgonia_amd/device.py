@@ -182,11 +182,21 @@ def cmd_outer(x, y, a, m, n):
 
 
 def cmd_conv2d(x, w, y, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dilation=(1, 1),
-               act=None, alpha=0.0):
+               act=None, alpha=0.0, bn=None, eps=1e-5, pool2=False):
+    """bn = (mean, var, gamma or 0, beta or 0) device pointers: BatchNorm (eval)
+    on the result; pool2: 2x2 stride-2 MaxPool2D on the result (y is then
+    B x F x oh/2 x ow/2).  Order: conv, bn, activation, pool."""
     fl = {None: 0, "relu": _ffi.FLAG_ACT_RELU, "leaky": _ffi.FLAG_ACT_LEAKY}[act]
-    return make_cmd(_ffi.OP_CONV2D, fl, (x, w, y),
+    ptrs = [x, w, y]
+    if bn is not None:
+        mean, var, gamma, beta = bn
+        fl |= _ffi.FLAG_CONV_BN | (_ffi.FLAG_HAS_GAMMA if gamma else 0) | (_ffi.FLAG_HAS_BETA if beta else 0)
+        ptrs += [mean, var, gamma, beta]
+    if pool2:
+        fl |= _ffi.FLAG_CONV_POOL2
+    return make_cmd(_ffi.OP_CONV2D, fl, ptrs,
                     (B, Cin, H, W, F, kh, kw, pad[0], pad[1], stride[0], stride[1], dilation[0],
-                     dilation[1]), (alpha,))
+                     dilation[1]), (alpha, eps))
 
 
 def cmd_maxpool2d(x, y, B, Cn, H, W, kh, kw, pad, stride):

@@ -173,7 +173,10 @@ static std::string op_name(const OpSpec& op) {
     case OpKind::MatVecMul: return "matvecmul";
     case OpKind::Outer: return "outer";
     case OpKind::BatchedMatMul: return "batchedmatmul";
-    case OpKind::Conv2d: return op.fuse_act_relu ? "conv2d+rectify" : op.fuse_act_leaky ? "conv2d+leakyrelu" : "conv2d";
+    case OpKind::Conv2d:
+      return std::string("conv2d") + (op.fuse_bn ? "+batchnorm(eval)" : "") +
+             (op.fuse_act_relu ? "+rectify" : op.fuse_act_leaky ? "+leakyrelu" : "") +
+             (op.fuse_pool2 ? "+maxpool2d" : "");
     case OpKind::MaxPool2D: return "maxpool2d";
     case OpKind::BatchNorm: return "batchnorm(eval)";
     case OpKind::Rectify: return "rectify";
@@ -236,6 +239,17 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       c.flags = op.fuse_act_relu ? GH_FLAG_ACT_RELU : op.fuse_act_leaky ? GH_FLAG_ACT_LEAKY : 0;
       c.f[0] = (float)op.f0;
       c.ptr[0] = x.mem; c.ptr[1] = w.mem; c.ptr[2] = prealloc.mem;
+      if (op.fuse_bn) {
+        if (in.size() != 4 && in.size() != 6) return bad("Conv2d: fused BatchNorm needs mean, var[, scale, bias]");
+        c.flags |= GH_FLAG_CONV_BN;
+        c.ptr[3] = in[2]->mem; c.ptr[4] = in[3]->mem;
+        if (in.size() == 6) {
+          c.flags |= GH_FLAG_HAS_GAMMA | GH_FLAG_HAS_BETA;
+          c.ptr[5] = in[4]->mem; c.ptr[6] = in[5]->mem;
+        }
+        c.f[1] = (float)op.f1;
+      }
+      if (op.fuse_pool2) c.flags |= GH_FLAG_CONV_POOL2;
       for (int i = 0; i < 4; i++) c.dim[i] = x.shape[i];
       c.dim[4] = w.shape[0];
       for (int i = 0; i < 8; i++) c.dim[5 + i] = op.ints[(size_t)i];
@@ -347,16 +361,45 @@ int Graph::FuseActivations() {
   std::vector<int> uses(nodes_.size(), 0);
   for (auto& n : nodes_) for (int i : n.inputs) uses[(size_t)i]++;
   for (auto& n : nodes_) {
-    if (n.is_input || n.fused_away) continue;
-    if (n.op.kind != OpKind::Rectify && n.op.kind != OpKind::LeakyRelu) continue;
+    if (n.is_input || n.fused_away || n.inputs.empty()) continue;
+    const OpKind k = n.op.kind;
+    if (k != OpKind::Rectify && k != OpKind::LeakyRelu && k != OpKind::BatchNorm && k != OpKind::MaxPool2D)
+      continue;
     Node& p = nodes_[(size_t)n.inputs[0]];
-    if (p.is_input || p.read_into || uses[(size_t)p.id] != 1) continue;
+    if (p.is_input || p.fused_away || p.read_into || uses[(size_t)p.id] != 1) continue;
     if (p.op.kind != OpKind::Conv2d && p.op.kind != OpKind::MatMul) continue;
-    if (p.op.fuse_act_relu || p.op.fuse_act_leaky) continue;
-    if (n.op.kind == OpKind::Rectify) p.op.fuse_act_relu = true;
-    else { p.op.fuse_act_leaky = true; p.op.f0 = n.op.f0; }
-    n.fused_away = true;
-    n.alias_of = p.id;
+    OpSpec op = p.op;
+    std::vector<int> inputs = p.inputs;
+    const bool has_act = op.fuse_act_relu || op.fuse_act_leaky;
+    if (k == OpKind::BatchNorm) {
+      if (op.kind != OpKind::Conv2d || op.fuse_bn || has_act || op.fuse_pool2) continue;
+      if (n.shape.Dims() != 4) continue;
+      op.fuse_bn = true;
+      op.f1 = n.op.f0;
+      for (size_t i = 1; i < n.inputs.size(); i++) inputs.push_back(n.inputs[i]);
+    } else if (k == OpKind::Rectify || k == OpKind::LeakyRelu) {
+      if (has_act || op.fuse_pool2) continue;
+      if (k == OpKind::Rectify) op.fuse_act_relu = true;
+      else { op.fuse_act_leaky = true; op.f0 = n.op.f0; }
+    } else {  // MaxPool2D: 2x2 window, stride 2, no padding, and a kernel that can take it
+      if (op.kind != OpKind::Conv2d || op.fuse_pool2) continue;
+      const auto& q = n.op.ints;  // kh kw npad pads... sh sw
+      bool plain = q.size() >= 5 && q[0] == 2 && q[1] == 2;
+      for (size_t i = 3; plain && i < q.size(); i++) plain = q[i] == (i >= 3 + (size_t)q[2] ? 2 : 0);
+      if (!plain) continue;
+      const Shape& xs = nodes_[(size_t)inputs[0]].shape;
+      const Shape& ws = nodes_[(size_t)inputs[1]].shape;
+      gh_cmd c{};
+      c.opcode = GH_OP_CONV2D;
+      for (int i = 0; i < 4; i++) c.dim[i] = xs[i];
+      c.dim[4] = ws[0];
+      for (int i = 0; i < 8; i++) c.dim[5 + i] = op.ints[(size_t)i];
+      if (!gh_conv2d_can_pool(&c)) continue;
+      op.fuse_pool2 = true;
+    }
+    n.op = op;
+    n.inputs = inputs;
+    p.fused_away = true;
     fused++;
   }
   return fused;
@@ -378,8 +421,10 @@ Status TapeMachine::Compile() {
   for (int i = 0; i < N; i++) root[(size_t)i] = nodes[(size_t)i].alias_of >= 0 ? root[(size_t)nodes[(size_t)i].alias_of] : i;
   // last instruction that reads each root value
   std::vector<int> last_reader((size_t)N, -1);
-  for (int i = 0; i < N; i++)
+  for (int i = 0; i < N; i++) {
+    if (nodes[(size_t)i].fused_away) continue;  // its inputs are read by the node that absorbed it
     for (int in : nodes[(size_t)i].inputs) last_reader[(size_t)root[(size_t)in]] = i;
+  }
   std::vector<char> value_kept((size_t)N, 0);  // read by the host, or a resident input
   for (int i = 0; i < N; i++)
     if (nodes[(size_t)i].read_into || (nodes[(size_t)i].is_input && nodes[(size_t)i].resident))
@@ -392,6 +437,7 @@ Status TapeMachine::Compile() {
   int nreg = 0;
   for (int i = 0; i < N; i++) {
     Node& n = nodes[(size_t)i];
+    if (n.fused_away) continue;
     if (n.alias_of >= 0) { node_reg_[(size_t)i] = node_reg_[(size_t)root[(size_t)i]]; continue; }
     const int ow = n.is_input ? -1 : OverwritesInput(n.op);
     if (ow >= 0 && ow < (int)n.inputs.size()) {
@@ -412,6 +458,7 @@ Status TapeMachine::Compile() {
   std::vector<char> reg_kept((size_t)nreg, 0);
   for (int i = 0; i < N; i++) {
     const int r = node_reg_[(size_t)i];
+    if (r < 0) continue;
     reg_last[(size_t)r] = std::max(reg_last[(size_t)r], std::max(i, last_reader[(size_t)root[(size_t)i]]));
     if (value_kept[(size_t)root[(size_t)i]]) reg_kept[(size_t)r] = 1;
   }
@@ -423,7 +470,7 @@ Status TapeMachine::Compile() {
 
   for (int i = 0; i < N; i++) {
     Node& n = nodes[(size_t)i];
-    if (n.alias_of >= 0) continue;
+    if (n.alias_of >= 0 || n.fused_away) continue;
     const int r = node_reg_[(size_t)i];
     const int64_t bytes = bytes_of(n);
     if (n.is_input) {
@@ -491,7 +538,7 @@ Status TapeMachine::Init(int device) {
 }
 
 uint64_t TapeMachine::RegisterAddress(int node) const {
-  if (node < 0 || node >= (int)node_reg_.size()) return 0;
+  if (node < 0 || node >= (int)node_reg_.size() || node_reg_[(size_t)node] < 0) return 0;
   return regs_[(size_t)node_reg_[(size_t)node]].mem;
 }
 

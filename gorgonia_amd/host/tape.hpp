@@ -49,8 +49,14 @@ struct OpSpec {
   bool transA = false, transB = false;
   std::vector<int64_t> ints;  // kernel/pad/stride/dilation, new shape, broadcast axes ...
   double f0 = 0.0;            // epsilon / alpha
-  bool fuse_act_relu = false;   // batcher-fused epilogue (set by Graph::FuseActivations)
+  // Followers folded into a Conv2d/MatMul epilogue by Graph::FuseActivations,
+  // applied in this order: BatchNorm (Conv2d only; inputs 2.. = mean, var[,
+  // scale, bias], f1 = epsilon), activation (f0 = alpha), 2x2/2 MaxPool2D.
+  bool fuse_bn = false;
+  double f1 = 0.0;
+  bool fuse_act_relu = false;
   bool fuse_act_leaky = false;
+  bool fuse_pool2 = false;
 };
 
 // Output shape of an op (InferShape of each reference op); error if the inputs
@@ -72,7 +78,7 @@ struct Node {
   OpSpec op;
   std::vector<int> inputs;
   void* read_into = nullptr;      // Read(node, &host) target
-  bool fused_away = false;        // activation folded into its producer
+  bool fused_away = false;        // absorbed into the follower that now computes both: no register, no instruction
   int alias_of = -1;              // Reshape shares its input's register
 };
 
@@ -82,8 +88,11 @@ class Graph {
   Status Apply(const OpSpec& op, const std::vector<int>& inputs, int* out);
   Status Let(int node, const void* host);              // rebind an input value
   Status Read(int node, void* host_out);               // gorgonia.Read
-  // Fold Rectify/LeakyRelu into the Conv2d/MatMul that feeds them when nothing
-  // else reads the un-activated value (bit-identical epilogue).
+  // Fold BatchNorm (eval), Rectify/LeakyRelu and a 2x2/2 MaxPool2D into the
+  // Conv2d that feeds them (activations into MatMul too) when nothing else reads
+  // the intermediate value.  The follower takes over the producer's operator
+  // and inputs; the values it stores are bit-identical to the unfused chain's.
+  // Returns the number of operators folded away.
   int FuseActivations();
   const std::vector<Node>& Nodes() const { return nodes_; }
   std::vector<Node>& Nodes() { return nodes_; }

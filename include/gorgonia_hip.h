@@ -112,6 +112,8 @@ enum gh_unaryfn {
 #define GH_FLAG_HAS_BETA     (1u << 21)   /* BN_INFER: ptr[5] = beta           */
 #define GH_FLAG_ACT_RELU     (1u << 22)   /* CONV2D/GEMM epilogue: x*(x>=0)    */
 #define GH_FLAG_ACT_LEAKY    (1u << 23)   /* epilogue: leaky relu, alpha=f[0]  */
+#define GH_FLAG_CONV_BN      (1u << 24)   /* CONV2D: BatchNorm (eval) on the result, ptr[3..6] */
+#define GH_FLAG_CONV_POOL2   (1u << 25)   /* CONV2D: 2x2 stride-2 unpadded MaxPool2D on the result */
 
 /*
  * One operator.  Field use per opcode:
@@ -133,6 +135,12 @@ enum gh_unaryfn {
  * OUTER       ptr[0]=x ptr[1]=y ptr[2]=A   dim[0..1]=m,n ; A(m x n) = x y^T
  * CONV2D      ptr[0]=x ptr[1]=w ptr[2]=y   dim[0..3]=B,C,H,W dim[4]=F dim[5..6]=kh,kw
  *             dim[7..8]=padH,padW dim[9..10]=strideH,strideW dim[11..12]=dilH,dilW
+ *             Operators that follow the convolution can ride in its epilogue; the
+ *             stored values are bit for bit those of the separate commands, in
+ *             this order: CONV_BN (ptr[3]=mean ptr[4]=var, with HAS_GAMMA ptr[5]=gamma,
+ *             with HAS_BETA ptr[6]=beta, f[1]=eps; BN_INFER's arithmetic per filter),
+ *             then ACT_RELU / ACT_LEAKY, then CONV_POOL2 (y then has the pooled
+ *             shape B,F,oh/2,ow/2; only where gh_conv2d_can_pool says so)
  * MAXPOOL2D   ptr[0]=x ptr[1]=y            dim[0..3]=B,C,H,W dim[4..5]=kh,kw
  *             dim[6..9]=padN,padS,padW,padE dim[10..11]=strideH,strideW
  * BN_INFER    ptr[0]=x ptr[1]=y ptr[2]=mean ptr[3]=var [ptr[4]=gamma ptr[5]=beta]
@@ -147,7 +155,7 @@ enum gh_unaryfn {
 typedef struct gh_cmd {
   uint32_t opcode;
   uint32_t flags;
-  uint64_t ptr[6];
+  uint64_t ptr[8];
   int64_t  dim[16];
   float    f[4];
 } gh_cmd;
@@ -197,6 +205,11 @@ GH_API int gh_memcpy_d2d(gh_ctx* ctx, gh_devptr dst, gh_devptr src, int64_t byte
 GH_API int gh_submit(gh_ctx* ctx, const gh_cmd* cmds, int n);
 /* Validate only: same checks as gh_submit, touches no device. */
 GH_API int gh_validate(const gh_cmd* cmds, int n, char* msg, int msg_len);
+/* 1 when this CONV2D command may carry GH_FLAG_CONV_POOL2 (a convolution whose
+ * kernel keeps a whole pooling window in one thread), else 0.  Host only.  The
+ * reference has no fused form: this folds maxpool.CUDADo
+ * (ops/nn/maxpool_cuda.go:94-111) into convolution.CUDADo (convolution_cuda.go:95-121). */
+GH_API int gh_conv2d_can_pool(const gh_cmd* conv);
 /* Engine.DoWork / Signal+Sync (cuda/external.go:223-226): block until the
  * stream drains, return the sticky error. */
 GH_API int gh_sync(gh_ctx* ctx);

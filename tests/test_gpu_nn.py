@@ -97,6 +97,98 @@ def test_conv_fused_activation_epilogue(ctx):
                       O.leaky_relu(plain, 0.1).reshape(plain.shape), "conv+leaky")
 
 
+def gpu_conv_tail(ctx, x, w, pad, bn=None, act=None, alpha=0.0, pool2=False, eps=1e-5):
+    """Conv2d with followers in its epilogue: bn = (mean, var, gamma|None, beta|None) host arrays."""
+    B, C, H, W = x.shape
+    F, _, kh, kw = w.shape
+    oh, ow = O.conv_out_hw(H, W, kh, kw, pad, (1, 1), (1, 1))
+    yh, yw = (oh // 2, ow // 2) if pool2 else (oh, ow)
+    held = [ctx.upload(x), ctx.upload(w)]
+    dbn = None
+    if bn is not None:
+        dbn = tuple(0 if a is None else ctx.upload(a) for a in bn)
+        held += [p for p in dbn if p]
+    dy = ctx.malloc(B * F * yh * yw * 4)
+    held.append(dy)
+    ctx.run(D.cmd_fill(dy, B * F * yh * yw, np.nan))
+    ctx.run(D.cmd_conv2d(held[0], held[1], dy, B, C, H, W, F, kh, kw, pad, act=act, alpha=alpha, bn=dbn,
+                         eps=eps, pool2=pool2))
+    y = ctx.d2h(dy, (B, F, yh, yw))
+    for p in held:
+        ctx.free(p)
+    return y
+
+
+def gpu_bn(ctx, x, mean, var, gamma, beta, eps):
+    B, C = x.shape[:2]
+    S = x.size // (B * C)
+    dx, dm, dv = ctx.upload(x), ctx.upload(mean), ctx.upload(var)
+    dg = ctx.upload(gamma) if gamma is not None else 0
+    db = ctx.upload(beta) if beta is not None else 0
+    ctx.run(D.cmd_bn_infer(dx, dx, dm, dv, B, C, S, eps, gamma=dg, beta=db))
+    y = ctx.d2h(dx, x.shape)
+    for p in (dx, dm, dv, dg, db):
+        if p:
+            ctx.free(p)
+    return y
+
+
+# shapes that reach each convolution kernel: the direct one (C <= 4), the
+# LDS-staged 3x3 one with and without split-K, the gather one (1x1)
+TAIL_CASES = [(2, 3, 20, 22, 16, 3, 1), (3, 1, 28, 28, 32, 3, 1), (2, 4, 9, 9, 5, 3, 0),
+              (2, 16, 26, 26, 32, 3, 1), (2, 256, 13, 13, 64, 3, 1), (2, 64, 13, 13, 40, 1, 0)]
+
+
+@pytest.mark.parametrize("cfg", TAIL_CASES)
+def test_conv_epilogue_batchnorm_activation_bit_exact(ctx, cfg):
+    """conv -> BatchNorm(eval) -> LeakyReLU as one command stores the bits of the three separate commands."""
+    B, C, H, W, F, k, pad = cfg
+    x = synth.uniform(11, (B, C, H, W), -1, 1)
+    w = synth.he_normal(12, (F, C, k, k))
+    mean, var = synth.normal(13, (F,), 0.0, 0.1), synth.uniform(14, (F,), 0.5, 1.5)
+    gamma, beta = synth.uniform(15, (F,), 0.5, 1.5), synth.normal(16, (F,), 0.0, 0.1)
+    plain = gpu_conv(ctx, x, w, (pad, pad), (1, 1), (1, 1))
+    for g, b in ((gamma, beta), (None, None)):
+        bn = gpu_bn(ctx, plain.copy(), mean, var, g, b, 1e-5)
+        assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, g, b)), bn, f"conv+bn {cfg}")
+        assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, g, b), act="leaky", alpha=0.1),
+                          O.leaky_relu(bn, 0.1).reshape(bn.shape), f"conv+bn+leaky {cfg}")
+    # and against the oracle's own batch norm of the same convolution result
+    want = O.bn_infer(plain, mean, var, 1e-5, gamma, beta)
+    assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, gamma, beta)), want, "vs oracle bn")
+
+
+@pytest.mark.parametrize("cfg", [(3, 1, 28, 28, 32, 1), (2, 3, 21, 19, 16, 1), (2, 4, 10, 12, 6, 0),
+                                 (1, 2, 7, 7, 9, 1)])
+def test_conv_epilogue_pool_bit_exact(ctx, cfg):
+    """conv -> ReLU -> MaxPool 2x2/2 as one command (odd sizes drop the last row/column)."""
+    B, C, H, W, F, pad = cfg
+    x = synth.uniform(21, (B, C, H, W), -1, 1)
+    w = synth.he_normal(22, (F, C, 3, 3))
+    cmd = D.cmd_conv2d(1, 1, 1, B, C, H, W, F, 3, 3, (pad, pad))
+    assert ctx.lib.gh_conv2d_can_pool(cmd) == 1
+    act = gpu_conv(ctx, x, w, (pad, pad), (1, 1), (1, 1), act="relu")
+    want = gpu_pool(ctx, act, (2, 2), (0, 0), (2, 2))
+    got = gpu_conv_tail(ctx, x, w, (pad, pad), act="relu", pool2=True)
+    assert_bits_equal(got, want, f"conv+relu+pool {cfg}")
+    assert_bits_equal(want, O.maxpool2d(O.relu(act).reshape(act.shape), (2, 2), (0, 0), (2, 2)), "pool vs oracle")
+    mean, var = synth.normal(23, (F,), 0.0, 0.1), synth.uniform(24, (F,), 0.5, 1.5)
+    plain = gpu_conv(ctx, x, w, (pad, pad), (1, 1), (1, 1))
+    chain = gpu_pool(ctx, O.leaky_relu(gpu_bn(ctx, plain.copy(), mean, var, None, None, 1e-5), 0.1).reshape(plain.shape),
+                     (2, 2), (0, 0), (2, 2))
+    assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, None, None), act="leaky", alpha=0.1,
+                                    pool2=True), chain, f"conv+bn+leaky+pool {cfg}")
+
+
+def test_conv_pool_flag_needs_a_pooling_kernel(ctx):
+    cmd = D.cmd_conv2d(0x1000, 0x2000, 0x3000, 2, 8, 14, 14, 16, 3, 3, (1, 1), pool2=True)
+    assert ctx.lib.gh_conv2d_can_pool(cmd) == 0
+    import ctypes as C
+    buf = C.create_string_buffer(256)
+    assert ctx.lib.gh_validate(C.byref(cmd), 1, buf, 256) != 0
+    assert b"pooling" in buf.value
+
+
 def gpu_pool(ctx, x, kernel, pad, stride):
     B, C, H, W = x.shape
     oh, ow = O.maxpool_out_hw(H, W, kernel[0], kernel[1], pad, stride)

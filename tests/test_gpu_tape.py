@@ -47,7 +47,7 @@ def test_convnet_forward_fused_and_unfused(ctx):
     m2, _, r2 = run_once(configs.build_convnet, inp, fuse_activations=True)
     assert rel_frobenius(r1["out"], want) <= 1e-5
     assert_bits_equal(r1["out"], r2["out"], "fused activations change nothing")
-    assert m2.fused == 4
+    assert m2.fused == 5  # 4 activations + the first pool
     m1.Close(); m2.Close()
 
 
@@ -58,7 +58,17 @@ def test_yolo_shaped_forward_reduced(ctx):
     m, _, res = run_once(configs.build_yolo, inp, fuse_activations=True)
     assert res["out"].shape == want.shape == (1, 425, 3, 3)
     assert rel_frobenius(res["out"], want) <= 1e-5
+    # conv -> batchnorm -> leakyrelu (-> maxpool after the 3-channel layer) run as
+    # single commands; the folded program stores the bits of the plain one
+    prog = m.program()
+    assert prog.count("conv2d+batchnorm(eval)+leakyrelu") == 7
+    assert prog.count("conv2d+batchnorm(eval)+leakyrelu+maxpool2d") == 1
+    assert " batchnorm" not in prog and " leakyrelu" not in prog
     m.Close()
+    m0, _, plain = run_once(configs.build_yolo, inp)
+    assert "conv2d+" not in m0.program()
+    assert_bits_equal(res["out"], plain["out"], "folded yolo-shaped forward == plain")
+    m0.Close()
 
 
 def test_graph_replay_matches_eager_every_time(ctx):
