@@ -32,12 +32,20 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+EAGER_TIMING = False  # --eager-timing: no hipGraph anywhere (for hardware-counter runs)
+
+
 def time_cmds(ctx, cmds, iters, warm=3):
     """Average milliseconds per pass over `cmds`: `iters` passes are captured
     into one hipGraph (so host enqueue time is out of the picture) and the
     replay is bracketed by HIP events on the engine's stream."""
     ctx.submit(list(cmds) * warm)
     ctx.sync()
+    if EAGER_TIMING:
+        ctx.event(0)
+        ctx.submit(list(cmds) * iters)
+        ctx.event(1)
+        return ctx.elapsed_ms(0, 1) / iters
     ctx.graph_begin()
     ctx.submit(list(cmds) * iters)
     gid = ctx.graph_end()
@@ -112,6 +120,16 @@ def bench_linalg(ctx, iters):
     return res
 
 
+# HBM bytes per launch of each conv layer's kernels (the split-K reduce
+# included), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
+# (KiB per dispatch; FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0, the factors a
+# 64 MiB device copy in the same runs gives).
+MEASURED_TRAFFIC_BYTES = {
+    "conv0": (2 * 295.9 + 12544.0) * 1024,
+    "conv1": (2 * 4508.5 + 6784.0) * 1024,
+    "conv2": (2 * 4073.0 + 6272.0 + 2 * 3156.5 + 3360.0) * 1024,
+}
+
 CONVNET_LAYERS = [  # (name, B-relative shape) of configuration 4
     ("conv0", 1, 28, 32), ("conv1", 32, 14, 64), ("conv2", 64, 7, 128),
 ]
@@ -170,7 +188,7 @@ def bench_yolo(steps, warmup):
     from gorgonia_amd import configs, graph as G
     inp = configs.yolo_inputs(8, 416)
     g, outs = configs.build_yolo(inp, resident_input=True)
-    m = G.NewTapeMachine(g, graph_replay=True, fuse_activations=True)
+    m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING, fuse_activations=True)
     for _ in range(max(warmup, 3)):
         m.RunAll()
     eng = m.engine()
@@ -236,18 +254,22 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--eager-timing", action="store_true",
+                    help="launch every kernel eagerly, no hipGraph (use under rocprofv3 --pmc)")
     ap.add_argument("--only", default="", help="comma list of: convnet,elementwise,linalg,yolo")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this engine runs on one GPU; --gpus must be 1 (no multi-GPU path is built)")
     only = set(filter(None, a.only.split(",")))
+    global EAGER_TIMING
+    EAGER_TIMING = a.eager_timing
 
     from gorgonia_amd.device import Context
     ctx = Context(0, 0)
     info = ctx.info()
     log(f"device {info.arch.decode()} CUs={info.compute_units}")
 
-    ms_step, gpu_out, inp, launches = bench_convnet(a.steps, a.warmup)
+    ms_step, gpu_out, inp, launches = bench_convnet(a.steps, a.warmup, graph_replay=not a.eager_timing)
     images_s = 128 / ms_step * 1e3
     log(f"convnet: {ms_step:.4f} ms/step  {images_s:.0f} images/s  (graph launches {launches})")
     ms_h2d, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False)
@@ -271,9 +293,11 @@ def main():
     if conv_k:
         name = max(conv_k, key=lambda k: conv_k[k]["us"])
         r = conv_k[name]
-        roofline = {"kernel": f"k_conv2d ({name} of the convnet step, fused ReLU)", "bound": "mfma",
+        kname = "k_conv3x3_direct" if name == "conv0" else "k_conv3x3_lds (+ k_splitk_reduce)"
+        roofline = {"kernel": f"{kname}: {name} of the convnet step with ReLU in the epilogue", "bound": "mfma",
                     "achieved": r["TFLOPs"], "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(r["TFLOPs"] / MFMA_F32_PEAK_TFLOPS, 4), "traffic": None,
+                    "frac": round(r["TFLOPs"] / MFMA_F32_PEAK_TFLOPS, 4),
+                    "traffic": int(MEASURED_TRAFFIC_BYTES[name]),
                     "launch_us": r["us"], "algorithmic_flop": r["flop"]}
 
     cpu = None
