@@ -233,6 +233,82 @@ def softmax(x):
     return y
 
 
+def maxpool2d_bwd(x, dy, kernel, pad, stride):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    B, Cn, H, W = x.shape
+    p4, explicit = _pad4(pad)
+    dx = np.empty_like(x)
+    lib().oracle_maxpool2d_bwd_f32(_p(x), _p(dy), _p(dx), *_i64(B, Cn, H, W, kernel[0], kernel[1]), _p(p4),
+                                   C.c_int(explicit), *_i64(stride[0], stride[1]))
+    return dx
+
+
+def conv2d_bwd(x, w, dy, pad=(0, 0), stride=(1, 1), dil=(1, 1)):
+    """(dx, dw) of Conv2d as the reference's graph differentiates it, float32."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    B, Cn, H, W = x.shape
+    F, _, kh, kw = w.shape
+    dx, dw = np.empty_like(x), np.empty_like(w)
+    rc = lib().oracle_conv2d_bwd_f32(_p(x), _p(w), _p(dy), _p(dx), _p(dw),
+                                     *_i64(B, Cn, H, W, F, kh, kw, pad[0], pad[1], stride[0], stride[1],
+                                           dil[0], dil[1]))
+    if rc != 0:
+        raise MemoryError("oracle conv2d backward scratch allocation failed")
+    return dx, dw
+
+
+def conv2d_bwd_direct_f64(x, w, dy, pad=(0, 0), stride=(1, 1), dil=(1, 1)):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    B, Cn, H, W = x.shape
+    F, _, kh, kw = w.shape
+    dx, dw = np.empty(x.shape, np.float64), np.empty(w.shape, np.float64)
+    lib().oracle_conv2d_bwd_direct_f64(_p(x), _p(w), _p(dy), _p(dx), _p(dw),
+                                       *_i64(B, Cn, H, W, F, kh, kw, pad[0], pad[1], stride[0], stride[1],
+                                             dil[0], dil[1]))
+    return dx, dw
+
+
+def bn_train_stats(x, run_mean, run_var, momentum, eps):
+    """Training-mode forward; returns (y, running_mean, running_var, save_mean, save_var_sum)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    B, Cn = x.shape[:2]
+    S = x.size // (B * Cn)
+    y = np.empty_like(x)
+    rm = np.array(run_mean, dtype=np.float32, copy=True)
+    rv = np.array(run_var, dtype=np.float32, copy=True)
+    sm, sv = np.empty(Cn, np.float32), np.empty(Cn, np.float32)
+    lib().oracle_bn_train_stats_f32(_p(x), _p(y), _p(rm), _p(rv), _p(sm), _p(sv), C.c_float(momentum),
+                                    C.c_float(eps), *_i64(B, Cn, S))
+    return y, rm, rv, sm, sv
+
+
+def bn_bwd(x, dy, save_mean, save_var, eps, training=True):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    B, Cn = x.shape[:2]
+    S = x.size // (B * Cn)
+    dx = np.empty_like(x)
+    sm = np.ascontiguousarray(save_mean, dtype=np.float32)
+    sv = np.ascontiguousarray(save_var, dtype=np.float32)
+    lib().oracle_bn_bwd_f32(_p(x), _p(dy), _p(dx), _p(sm), _p(sv), C.c_float(eps), C.c_int(int(training)),
+                            *_i64(B, Cn, S))
+    return dx
+
+
+def softmax_bwd(y, dy):
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    rows, cols = int(np.prod(y.shape[:-1])), y.shape[-1]
+    dx = np.empty_like(y)
+    lib().oracle_softmax_bwd_f32(_p(y), _p(dy), _p(dx), *_i64(rows, cols))
+    return dx
+
+
 def has_nan(a):
     a = np.ascontiguousarray(a, dtype=np.float32)
     return bool(lib().oracle_has_nan_f32(_p(a), C.c_int64(a.size)))

@@ -591,6 +591,250 @@ EXPORT void oracle_bn_train_f32(const float* x, float* y, float* run_mean, float
 /* ------------------------------------------------------------------ */
 /* SoftMax over the last axis (op_softmax.go:99-128 -> tensor.SoftMax): */
 /* max-subtracted exp, sum, divide.                                    */
+/* ================================================================== */
+/* Backward passes (the reference's diff ops on the CPU engine).       */
+/* ================================================================== */
+
+/* MaxPool2D backward: maxPoolDiffOp.f32s (op_nn.go:1067-1093) driven by the
+ * argmax mask the forward pass records (op_nn.go:860-907: first element in
+ * row-major window order that is strictly greater than everything before,
+ * starting from -FLT_MAX; -1 when nothing wins, which contributes nothing
+ * here).  dx is zeroed, then every window adds its dy into its argmax in
+ * (ph, pw) order. */
+EXPORT void oracle_maxpool2d_bwd_f32(const float* x, const float* dy, float* dx, int64_t B,
+                                     int64_t C, int64_t H, int64_t W, int64_t kh, int64_t kw,
+                                     const int64_t* pad4, int explicit_padding, int64_t strideH,
+                                     int64_t strideW) {
+  int64_t oh, ow, bc;
+  oracle_maxpool_out_hw(H, W, kh, kw, pad4, strideH, strideW, &oh, &ow);
+  int64_t padH = explicit_padding ? pad4[1] : pad4[0];
+  int64_t padW = explicit_padding ? pad4[3] : pad4[2];
+#pragma omp parallel for if (g_threads > 1) schedule(static)
+  for (bc = 0; bc < B * C; bc++) {
+    const float* in = x + bc * H * W;
+    const float* g = dy + bc * oh * ow;
+    float* out = dx + bc * H * W;
+    int64_t ph, pw, hi, wi, i;
+    for (i = 0; i < H * W; i++) out[i] = 0.0f;
+    for (ph = 0; ph < oh; ph++)
+      for (pw = 0; pw < ow; pw++) {
+        int64_t hs = ph * strideH - padH, ws = pw * strideW - padW;
+        int64_t he = hs + kh < H ? hs + kh : H;
+        int64_t we = ws + kw < W ? ws + kw : W;
+        if (hs < 0) hs = 0;
+        if (ws < 0) ws = 0;
+        float best = -FLT_MAX;
+        int64_t arg = -1;
+        for (hi = hs; hi < he; hi++)
+          for (wi = ws; wi < we; wi++)
+            if (in[hi * W + wi] > best) { best = in[hi * W + wi]; arg = hi * W + wi; }
+        if (arg >= 0) out[arg] = out[arg] + g[ph * ow + pw];
+      }
+  }
+}
+
+/* col2im: col2imOp.f32s (op_nn.go:605-640), per image, accumulation in
+ * (outputRow, outputCol, channel, kernelRow, kernelCol) order. */
+static void col2im_one_f32(const float* col, float* im, int64_t C, int64_t H, int64_t W,
+                           int64_t kh, int64_t kw, int64_t padH, int64_t padW, int64_t strideH,
+                           int64_t strideW, int64_t dilH, int64_t dilW, int64_t oh, int64_t ow) {
+  int64_t i, r, c, ch, kr, kc, idx = 0;
+  for (i = 0; i < C * H * W; i++) im[i] = 0.0f;
+  for (r = 0; r < oh; r++)
+    for (c = 0; c < ow; c++)
+      for (ch = 0; ch < C; ch++)
+        for (kr = 0; kr < kh; kr++) {
+          int64_t ir = -padH + kr * dilH + r * strideH;
+          for (kc = 0; kc < kw; kc++) {
+            int64_t ic = -padW + kc * dilW + c * strideW;
+            if (ir >= 0 && ir < H && ic >= 0 && ic < W) {
+              float* t = &im[(ch * H + ir) * W + ic];
+              *t = *t + col[idx];
+            }
+            idx++;
+          }
+        }
+}
+
+/* Conv2d backward as the reference's graph differentiates it (nn.go:211-305):
+ * y = transpose(reshape(col . Wflat^T)), so with dY2d = (B*oh*ow, F):
+ *   dCol = dY2d . Wflat          (linAlgBinOp diff wrt the first operand)
+ *   dX   = col2im(dCol)          (im2colOp.DoDiff, op_nn.go:267-291)
+ *   dW   = dY2d^T . col          (diff wrt the second, transposed operand)
+ * Either output pointer may be NULL. */
+EXPORT int oracle_conv2d_bwd_f32(const float* x, const float* w, const float* dy, float* dx,
+                                 float* dw, int64_t B, int64_t C, int64_t H, int64_t W, int64_t F,
+                                 int64_t kh, int64_t kw, int64_t padH, int64_t padW,
+                                 int64_t strideH, int64_t strideW, int64_t dilH, int64_t dilW) {
+  int64_t oh, ow;
+  oracle_conv_out_hw(H, W, kh, kw, padH, padW, strideH, strideW, dilH, dilW, &oh, &ow);
+  int64_t K = C * kh * kw, P = oh * ow, M = B * P;
+  float* dy2 = (float*)malloc((size_t)M * F * sizeof(float));
+  float* col = (float*)malloc((size_t)M * K * sizeof(float));
+  if (!dy2 || !col) { free(dy2); free(col); return -1; }
+  int64_t b, f, p;
+#pragma omp parallel for if (g_threads > 1) schedule(static)
+  for (b = 0; b < B; b++)
+    for (f = 0; f < F; f++)
+      for (p = 0; p < P; p++) dy2[(b * P + p) * F + f] = dy[(b * F + f) * P + p];
+  if (dw) {
+    oracle_im2col_f32(x, col, B, C, H, W, kh, kw, padH, padW, strideH, strideW, dilH, dilW);
+    oracle_gemm_f32(1, 0, F, K, M, dy2, F, col, K, dw, K);
+  }
+  if (dx) {
+    oracle_gemm_f32(0, 0, M, K, F, dy2, F, w, K, col, K);
+#pragma omp parallel for if (g_threads > 1) schedule(static)
+    for (b = 0; b < B; b++)
+      col2im_one_f32(col + b * P * K, dx + b * C * H * W, C, H, W, kh, kw, padH, padW, strideH,
+                     strideW, dilH, dilW, oh, ow);
+  }
+  free(dy2);
+  free(col);
+  return 0;
+}
+
+/* The same two gradients from the definition, in float64: the yardstick that
+ * pins oracle_conv2d_bwd_f32 (every product x*w*dy of the forward sum is
+ * attributed to its x and its w). */
+EXPORT void oracle_conv2d_bwd_direct_f64(const float* x, const float* w, const float* dy,
+                                         double* dx, double* dw, int64_t B, int64_t C, int64_t H,
+                                         int64_t W, int64_t F, int64_t kh, int64_t kw,
+                                         int64_t padH, int64_t padW, int64_t strideH,
+                                         int64_t strideW, int64_t dilH, int64_t dilW) {
+  int64_t oh, ow, b, f, r, c, ch, kr, kc, i;
+  oracle_conv_out_hw(H, W, kh, kw, padH, padW, strideH, strideW, dilH, dilW, &oh, &ow);
+  for (i = 0; i < B * C * H * W; i++) dx[i] = 0.0;
+  for (i = 0; i < F * C * kh * kw; i++) dw[i] = 0.0;
+  for (b = 0; b < B; b++)
+    for (f = 0; f < F; f++)
+      for (r = 0; r < oh; r++)
+        for (c = 0; c < ow; c++) {
+          const double g = (double)dy[((b * F + f) * oh + r) * ow + c];
+          for (ch = 0; ch < C; ch++)
+            for (kr = 0; kr < kh; kr++)
+              for (kc = 0; kc < kw; kc++) {
+                int64_t ir = r * strideH - padH + kr * dilH;
+                int64_t ic = c * strideW - padW + kc * dilW;
+                if (ir < 0 || ir >= H || ic < 0 || ic >= W) continue;
+                int64_t xi = ((b * C + ch) * H + ir) * W + ic;
+                int64_t wi = ((f * C + ch) * kh + kr) * kw + kc;
+                dx[xi] += g * (double)w[wi];
+                dw[wi] += g * (double)x[xi];
+              }
+        }
+}
+
+/* BatchNorm forward in training mode with the saved statistics exposed:
+ * updateStatsF32 (op_nn.go:1489-1555) + calculateAlphaAndBetaF32 + the apply
+ * loop (op_nn.go:1559-1635).  save_var receives the SUM of squared deviations
+ * (the reference divides by n only where it is used). */
+EXPORT void oracle_bn_train_stats_f32(const float* x, float* y, float* run_mean, float* run_var,
+                                      float* save_mean, float* save_var, float momentum,
+                                      float eps, int64_t B, int64_t C, int64_t S) {
+  int64_t n = B * S, c;
+  for (c = 0; c < C; c++) {
+    float mean = 0.0f, var = 0.0f;
+    int64_t s, d;
+    for (s = 0; s < B; s++)
+      for (d = 0; d < S; d++) mean = mean + x[(s * C + c) * S + d];
+    mean = mean / (float)n;
+    for (s = 0; s < B; s++)
+      for (d = 0; d < S; d++) {
+        float t = x[(s * C + c) * S + d] - mean;
+        float t2 = t * t;
+        var = var + t2;
+      }
+    save_mean[c] = mean;
+    save_var[c] = var;
+    {
+      float m1 = momentum * mean;
+      float m2 = (1.0f - momentum) * run_mean[c];
+      run_mean[c] = m1 + m2;
+      float unb = var / (float)(n - 1);
+      float v1 = momentum * unb;
+      float v2 = (1.0f - momentum) * run_var[c];
+      run_var[c] = v1 + v2;
+    }
+    float vb = var / (float)n;
+    float inv = 1.0f / sqrtf(vb + eps);
+    float a = inv;
+    float b = -mean * a;
+    for (s = 0; s < B; s++)
+      for (d = 0; d < S; d++) {
+        int64_t i = (s * C + c) * S + d;
+        float t = x[i] * a;
+        y[i] = t + b;
+      }
+  }
+}
+
+/* BatchNorm backward, training branch of batchnormDiffOp.f32s for inputs with
+ * a spatial extent (op_nn.go:1893-1926; the S == 1 branch, op_nn.go:1850-1878,
+ * differs only in how the dot product is written and is followed when S == 1):
+ *   sum = SUM dy, dotp = SUM (x*dy - mean*dy), invstd = 1/sqrt(save_var/n + eps),
+ *   k = dotp*invstd*invstd/n, gradMean = sum/n,
+ *   dx = (dy - gradMean - (x - mean)*k) * invstd.
+ * training == 0: dx = dy * invstd (op_nn.go:1928-1936). */
+EXPORT void oracle_bn_bwd_f32(const float* x, const float* dy, float* dx, const float* save_mean,
+                              const float* save_var, float eps, int training, int64_t B,
+                              int64_t C, int64_t S) {
+  int64_t n = B * S, c;
+  for (c = 0; c < C; c++) {
+    float dotp = 0.0f, sum = 0.0f;
+    int64_t s, d;
+    const float mean = save_mean[c];
+    for (s = 0; s < B; s++)
+      for (d = 0; d < S; d++) {
+        int64_t i = (s * C + c) * S + d;
+        sum = sum + dy[i];
+        float partial;
+        if (S == 1) {
+          float t = x[i] - mean;
+          partial = t * dy[i];
+        } else {
+          float t1 = x[i] * dy[i];
+          float t2 = mean * dy[i];
+          partial = t1 - t2;
+        }
+        dotp = dotp + partial;
+      }
+    float vb = save_var[c] / (float)n;
+    float invstd = 1.0f / sqrtf(vb + eps);
+    float kk = dotp * invstd;
+    kk = kk * invstd;
+    kk = kk / (float)n;
+    float gradMean = sum / (float)n;
+    for (s = 0; s < B; s++)
+      for (d = 0; d < S; d++) {
+        int64_t i = (s * C + c) * S + d;
+        if (training) {
+          float t = x[i] - mean;
+          t = t * kk;
+          float u;
+          if (S == 1) { u = dy[i] - t; u = u - gradMean; }
+          else { u = dy[i] - gradMean; u = u - t; }
+          dx[i] = u * invstd;
+        } else {
+          dx[i] = dy[i] * invstd;
+        }
+      }
+  }
+}
+
+/* SoftMax backward over the last axis (softmaxDiffOp -> tensor.SoftMaxB,
+ * op_softmax.go:266-279): dx_i = y_i * (dy_i - SUM_j dy_j*y_j). */
+EXPORT void oracle_softmax_bwd_f32(const float* y, const float* dy, float* dx, int64_t rows,
+                                   int64_t cols) {
+  int64_t r, j;
+  for (r = 0; r < rows; r++) {
+    const float* yy = y + r * cols;
+    const float* g = dy + r * cols;
+    float dot = 0.0f;
+    for (j = 0; j < cols; j++) { float t = g[j] * yy[j]; dot = dot + t; }
+    for (j = 0; j < cols; j++) { float t = g[j] - dot; dx[r * cols + j] = yy[j] * t; }
+  }
+}
+
 /* ------------------------------------------------------------------ */
 EXPORT void oracle_softmax_f32(const float* x, float* y, int64_t rows, int64_t cols) {
   int64_t r, j;

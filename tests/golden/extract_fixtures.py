@@ -159,7 +159,9 @@ def batchnorm():
                 "expected_train_result": lit("ExpectedTrainResult"),
                 "expected_eval_result": lit("ExpectedEvalResult"),
                 "expected_scale_grad": lit("ExpectedScaleGrad"),
-                "expected_bias_grad": lit("ExpectedBiasGrad")}
+                "expected_bias_grad": lit("ExpectedBiasGrad"),
+                "expected_output_grad": lit("ExpectedOutputGrad"),
+                "expected_input_grad": lit("ExpectedInputGrad")}
         m = re.match(r"RangedFromWithStep\(([^,]*),\s*([^)]*)\)", x)
         if m:
             case["x_ranged"] = [float(m.group(1)), float(m.group(2))]

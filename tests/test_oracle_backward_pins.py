@@ -1,0 +1,224 @@
+"""Pins the oracle's backward passes (MaxPool2D, Conv2d, BatchNorm, SoftMax
+gradients) before the GPU kernels are compared to them: the reference's own
+gradient goldens where its tests hold any (BatchNorm input gradients), the
+definition in float64 / brute force on small inputs, adjoint identities against
+the already pinned forward oracle, and finite differences.  No GPU."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import binding as O
+from tests.test_oracle_pins import _init, _ranged
+
+G = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def load(name):
+    with open(os.path.join(G, name)) as f:
+        return json.load(f)
+
+
+# ---- MaxPool2D -----------------------------------------------------------------
+
+POOL_CASES = [((2, 2), (0, 0), (2, 2), (5, 6)), ((2, 2), (0, 0), (1, 1), (3, 4)), ((3, 3), (1, 1), (2, 2), (7, 7)),
+              ((2, 2), (1, 0, 1, 0), (1, 1), (6, 5)), ((3, 2), (1, 1), (1, 2), (6, 7))]
+
+
+def _pool_bwd_bruteforce(x, dy, kernel, pad, stride):
+    """Pure-Python restatement from the definition: argmax = first strictly larger element."""
+    B, C, H, W = x.shape
+    if len(pad) == 4:
+        ph_, pw_ = pad[1], pad[3]  # explicit padding offsets by south / east (op_nn.go:871-875)
+    else:
+        ph_, pw_ = pad
+    oh, ow = dy.shape[2:]
+    dx = np.zeros_like(x)
+    for b in range(B):
+        for c in range(C):
+            for ph in range(oh):
+                for pw in range(ow):
+                    best, arg = -np.finfo(np.float32).max, None
+                    for hi in range(max(ph * stride[0] - ph_, 0), min(ph * stride[0] - ph_ + kernel[0], H)):
+                        for wi in range(max(pw * stride[1] - pw_, 0), min(pw * stride[1] - pw_ + kernel[1], W)):
+                            if x[b, c, hi, wi] > best:
+                                best, arg = x[b, c, hi, wi], (hi, wi)
+                    if arg is not None:
+                        dx[b, c, arg[0], arg[1]] = np.float32(dx[b, c, arg[0], arg[1]] + dy[b, c, ph, pw])
+    return dx
+
+
+@pytest.mark.parametrize("kernel,pad,stride,hw", POOL_CASES)
+def test_maxpool_bwd_bruteforce(kernel, pad, stride, hw):
+    rng = np.random.default_rng(3)
+    x = rng.integers(-3, 4, (2, 3) + hw).astype(np.float32)  # many ties: the first maximum must win
+    y = O.maxpool2d(x, kernel, pad, stride)
+    dy = rng.standard_normal(y.shape).astype(np.float32)
+    got = O.maxpool2d_bwd(x, dy, kernel, pad, stride)
+    assert np.array_equal(got, _pool_bwd_bruteforce(x, dy, kernel, pad, stride))
+    # every dy lands somewhere: plane sums agree (float64 sums of float32 values)
+    assert np.allclose(got.sum(axis=(2, 3), dtype=np.float64), dy.sum(axis=(2, 3), dtype=np.float64), atol=1e-5)
+
+
+def test_maxpool_bwd_reference_example():
+    """nn_test.go:140-193 TestMaxPool2D: x = 0..23 as (1,2,3,4), 2x2 window, stride 1, cost = Sum(y):
+    each window's maximum is its bottom-right element, so the gradient counts windows per element."""
+    x = np.arange(24, dtype=np.float32).reshape(1, 2, 3, 4)
+    dy = np.ones((1, 2, 2, 3), np.float32)
+    dx = O.maxpool2d_bwd(x, dy, (2, 2), (0, 0), (1, 1))
+    want = np.zeros((3, 4), np.float32)
+    want[1:, 1:] = 1.0
+    assert np.array_equal(dx[0, 0], want) and np.array_equal(dx[0, 1], want)
+
+
+def test_maxpool_bwd_on_golden_forward():
+    """The 3072-float darknet-style pool of nn_test.go:91-138: gradient of Sum(y) puts, on every
+    element, the number of windows it wins; the wins reproduce the golden forward output."""
+    g = load("maxpool_asym.json")
+    x = np.array(g["x"], dtype=np.float32).reshape(g["shape"])
+    y = np.array(g["y"], dtype=np.float32).reshape(g["shape"])
+    dx = O.maxpool2d_bwd(x, np.ones_like(y), g["kernel"], g["pad"], g["stride"])
+    assert dx.sum() == y.size
+    assert np.isclose((dx * x).sum(dtype=np.float64), y.sum(dtype=np.float64))
+
+
+# ---- Conv2d ---------------------------------------------------------------------
+
+CONV_BWD_CASES = [
+    (2, 3, 8, 9, 5, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (1, 4, 7, 7, 6, 1, 1, (0, 0), (1, 1), (1, 1)),
+    (2, 2, 10, 11, 3, 3, 2, (2, 1), (2, 3), (1, 1)),
+    (1, 3, 12, 12, 4, 3, 3, (2, 2), (1, 1), (2, 2)),
+    (2, 5, 9, 9, 7, 5, 5, (2, 2), (1, 1), (1, 1)),
+    (3, 8, 6, 6, 16, 3, 3, (0, 0), (2, 2), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("cfg", CONV_BWD_CASES)
+def test_conv_bwd_definition_and_adjoint(cfg):
+    B, C, H, W, F, kh, kw, pad, stride, dil = cfg
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    w = rng.standard_normal((F, C, kh, kw)).astype(np.float32)
+    y64 = O.conv2d_direct_f64(x, w, pad, stride, dil)
+    dy = rng.standard_normal(y64.shape).astype(np.float32)
+    dx, dw = O.conv2d_bwd(x, w, dy, pad, stride, dil)
+    dx64, dw64 = O.conv2d_bwd_direct_f64(x, w, dy, pad, stride, dil)
+    for got, ref in ((dx, dx64), (dw, dw64)):
+        assert np.linalg.norm(got - ref) <= 1e-5 * np.linalg.norm(ref)
+    # adjoint identities against the pinned forward pass: <conv(x, w), dy> = <x, dx> = <w, dw>
+    lhs = float((y64 * dy).sum())
+    assert np.isclose(lhs, float((x.astype(np.float64) * dx64).sum()), rtol=1e-9)
+    assert np.isclose(lhs, float((w.astype(np.float64) * dw64).sum()), rtol=1e-9)
+    # integer data: the float32 port is exact whatever its summation order
+    xi = rng.integers(-3, 4, x.shape).astype(np.float32)
+    wi = rng.integers(-3, 4, w.shape).astype(np.float32)
+    di = rng.integers(-3, 4, dy.shape).astype(np.float32)
+    dxi, dwi = O.conv2d_bwd(xi, wi, di, pad, stride, dil)
+    rx, rw = O.conv2d_bwd_direct_f64(xi, wi, di, pad, stride, dil)
+    assert np.array_equal(dxi, rx.astype(np.float32)) and np.array_equal(dwi, rw.astype(np.float32))
+
+
+def test_conv_bwd_finite_difference():
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((1, 2, 5, 5)).astype(np.float32)
+    w = rng.standard_normal((3, 2, 3, 3)).astype(np.float32)
+    dy = rng.standard_normal((1, 3, 5, 5)).astype(np.float32)
+    dx64, dw64 = O.conv2d_bwd_direct_f64(x, w, dy, (1, 1))
+    f = lambda xx, ww: float((O.conv2d_direct_f64(xx, ww, (1, 1)) * dy).sum())
+    for idx in [(0, 0, 0, 0), (0, 1, 2, 3), (0, 1, 4, 4)]:
+        xp, xm = x.copy(), x.copy()
+        xp[idx] += 0.25; xm[idx] -= 0.25   # the loss is linear in x: any step is exact up to rounding
+        assert np.isclose((f(xp, w) - f(xm, w)) / 0.5, dx64[idx], rtol=1e-6)
+    for idx in [(0, 0, 0, 0), (2, 1, 1, 2)]:
+        wp, wm = w.copy(), w.copy()
+        wp[idx] += 0.25; wm[idx] -= 0.25
+        assert np.isclose((f(x, wp) - f(x, wm)) / 0.5, dw64[idx], rtol=1e-6)
+
+
+# ---- BatchNorm ------------------------------------------------------------------
+
+@pytest.mark.parametrize("idx", range(6))
+def test_batchnorm_input_grad_goldens(idx):
+    """nn_amd64_test.go bnAllCases ExpectedOutputGrad / ExpectedInputGrad through the graph of
+    nn_test.go:319-417: out = (gamma*BN(x) + beta) . fcWeight^T, cost = Mean(out)."""
+    c = load("batchnorm.json")["cases"][idx]
+    shp = c["x_shape"]
+    n = int(np.prod(shp))
+    x = (_ranged(*c["x_ranged"], n) if "x_ranged" in c else np.array(c["x"], np.float32)).reshape(shp)
+    B, Cn = shp[0], shp[1]
+    feat = n // B
+    S = feat // Cn
+    gamma = _init(c["scale_init"], Cn)
+    fcw = _init(c["scale_init"], B * feat).reshape(B, feat)
+    y, rm, rv, sm, sv = O.bn_train_stats(x, np.zeros(Cn, np.float32), np.ones(Cn, np.float32), 0.9, 1e-5)
+    y0, rm0, rv0 = O.bn_train(x, np.zeros(Cn, np.float32), np.ones(Cn, np.float32), 0.9, 1e-5)
+    assert np.array_equal(y, y0) and np.array_equal(rm, rm0) and np.array_equal(rv, rv0)
+    dout = np.full((B, B), 1.0 / (B * B), np.float32)
+    assert np.allclose(dout.reshape(-1), c["expected_output_grad"])
+    dz = (dout @ fcw).astype(np.float32)                           # out = z . fcw^T
+    dbn = (dz.reshape(B, Cn, S) * gamma[None, :, None]).astype(np.float32).reshape(shp)
+    dx = O.bn_bwd(x, dbn, sm, sv, 1e-5, training=True)
+    want = np.array(c["expected_input_grad"], np.float32).reshape(shp)
+    assert np.allclose(dx, want, rtol=2e-3, atol=2e-6), (dx.reshape(-1), want.reshape(-1))
+
+
+def _bn_train_f64(x, eps):
+    B, Cn = x.shape[:2]
+    x3 = x.reshape(B, Cn, -1).astype(np.float64)
+    mean = x3.mean(axis=(0, 2), keepdims=True)
+    var = ((x3 - mean) ** 2).mean(axis=(0, 2), keepdims=True)
+    return ((x3 - mean) / np.sqrt(var + eps)).reshape(x.shape)
+
+
+@pytest.mark.parametrize("shape", [(4, 3, 5, 5), (6, 4)])
+def test_batchnorm_bwd_is_the_gradient_of_the_training_forward(shape):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal(shape).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    Cn = shape[1]
+    y, _, _, sm, sv = O.bn_train_stats(x, np.zeros(Cn, np.float32), np.ones(Cn, np.float32), 0.9, 1e-5)
+    assert np.allclose(y, _bn_train_f64(x, 1e-5), atol=1e-5)
+    x3 = x.reshape(shape[0], Cn, -1).astype(np.float64)
+    assert np.allclose(sm, x3.mean(axis=(0, 2)), atol=1e-6)
+    assert np.allclose(sv, ((x3 - x3.mean(axis=(0, 2), keepdims=True)) ** 2).sum(axis=(0, 2)), rtol=1e-5)
+    dx = O.bn_bwd(x, dy, sm, sv, 1e-5, training=True)
+    loss = lambda xx: float((_bn_train_f64(xx, 1e-5) * dy).sum())
+    h = 1e-3
+    for idx in [tuple(0 for _ in shape), tuple(s - 1 for s in shape), tuple(s // 2 for s in shape)]:
+        xp, xm = x.astype(np.float64), x.astype(np.float64)
+        xp[idx] += h; xm[idx] -= h
+        fd = (loss(xp) - loss(xm)) / (2 * h)
+        assert np.isclose(dx[idx], fd, rtol=2e-3, atol=2e-5), (idx, dx[idx], fd)
+    # a gradient of a function that ignores the batch mean and scale: orthogonal to 1 and to x - mean
+    d3 = dx.reshape(shape[0], Cn, -1).astype(np.float64)
+    assert np.allclose(d3.sum(axis=(0, 2)), 0, atol=1e-4)
+    # eval branch: dy / sqrt(var + eps)
+    de = O.bn_bwd(x, dy, sm, sv, 1e-5, training=False)
+    n = x.size // Cn
+    inv = 1.0 / np.sqrt(sv.astype(np.float64) / n + 1e-5)
+    assert np.allclose(de.reshape(shape[0], Cn, -1), dy.reshape(shape[0], Cn, -1) * inv[None, :, None], rtol=1e-6)
+
+
+# ---- SoftMax ----------------------------------------------------------------------
+
+def test_softmax_bwd_finite_difference_and_identities():
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((5, 10))
+    dy = rng.standard_normal((5, 10)).astype(np.float32)
+    y64 = O.softmax(x)                                  # float64 oracle, pinned by the goldens
+    dx = O.softmax_bwd(y64.astype(np.float32), dy)
+    jac = y64[:, :, None] * (np.eye(10)[None] - y64[:, None, :])       # dy_i/dx_j = y_i (delta_ij - y_j)
+    want = np.einsum("ri,rij->rj", dy.astype(np.float64), jac)
+    assert np.allclose(dx, want, rtol=1e-5, atol=1e-7)
+    h = 1e-6
+    for (r, j) in [(0, 0), (2, 7), (4, 9)]:
+        xp, xm = x.copy(), x.copy()
+        xp[r, j] += h; xm[r, j] -= h
+        fd = ((O.softmax(xp) - O.softmax(xm)) * dy).sum() / (2 * h)
+        assert np.isclose(dx[r, j], fd, rtol=1e-4, atol=1e-7)
+    assert np.allclose(dx.sum(axis=1), 0, atol=1e-6)   # softmax ignores a shift of its input
+    # old-vs-new softmax example of op_softmax_test.go:283-290: cost = Sum(softmax(a)) has zero gradient
+    a = np.array([[0.1, 0.1, 0.3, 0.1, 0.4]])
+    assert np.allclose(O.softmax_bwd(O.softmax(a).astype(np.float32), np.ones((1, 5), np.float32)), 0, atol=1e-7)
