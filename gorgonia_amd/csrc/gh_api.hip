@@ -217,6 +217,12 @@ static int dispatch(gh_ctx* ctx, const gh_cmd& c) {
     case GH_OP_HAS_NAN:
     case GH_OP_HAS_INF: return gh_launch_has_nan_inf(ctx, c);
     case GH_OP_FILL: return gh_launch_fill(ctx, c);
+    case GH_OP_MAXPOOL2D_BWD: return gh_launch_maxpool2d_bwd(ctx, c);
+    case GH_OP_CONV2D_BWD_DATA: return gh_launch_conv2d_bwd_data(ctx, c);
+    case GH_OP_CONV2D_BWD_FILTER: return gh_launch_conv2d_bwd_filter(ctx, c);
+    case GH_OP_BN_TRAIN: return gh_launch_bn_train(ctx, c);
+    case GH_OP_BN_BWD: return gh_launch_bn_bwd(ctx, c);
+    case GH_OP_SOFTMAX_BWD: return gh_launch_softmax_bwd(ctx, c);
   }
   return GH_ENOFUNC;
 }

@@ -51,6 +51,12 @@ int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_maxpool2d(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_bn_infer(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_softmax(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_maxpool2d_bwd(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_conv2d_bwd_data(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_bn_train(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_bn_bwd(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_softmax_bwd(gh_ctx* ctx, const gh_cmd& c);
 
 static inline uint32_t gh_fn(uint32_t flags) { return flags & 0xffu; }
 static inline uint32_t gh_mode(uint32_t flags) { return (flags >> 8) & 0xfu; }

@@ -64,6 +64,11 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
       if (!pos(c.dim[0]) || !pos(c.dim[1])) return bad("outer: m, n must be positive");
       return GH_OK;
+    case GH_OP_CONV2D_BWD_DATA:
+    case GH_OP_CONV2D_BWD_FILTER:
+      if (c.flags & (GH_FLAG_CONV_BN | GH_FLAG_CONV_POOL2 | GH_FLAG_ACT_RELU | GH_FLAG_ACT_LEAKY))
+        return bad("conv2d backward takes no epilogue flags");
+      [[fallthrough]];
     case GH_OP_CONV2D: {
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
       for (int i = 0; i <= 6; i++)
@@ -89,6 +94,9 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
         return bad("conv2d: no fused pooling for this shape");
       return GH_OK;
     }
+    case GH_OP_MAXPOOL2D_BWD:
+      if (!c.ptr[2]) return bad("null operand");
+      [[fallthrough]];
     case GH_OP_MAXPOOL2D: {
       if (!c.ptr[0] || !c.ptr[1]) return bad("null operand");
       for (int i = 0; i <= 5; i++)
@@ -109,6 +117,23 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if ((c.flags & GH_FLAG_HAS_GAMMA) && !c.ptr[4]) return bad("null gamma");
       if ((c.flags & GH_FLAG_HAS_BETA) && !c.ptr[5]) return bad("null beta");
       if (!pos(c.dim[0]) || !pos(c.dim[1]) || !pos(c.dim[2])) return bad("bn: B,C,S must be positive");
+      return GH_OK;
+    case GH_OP_BN_TRAIN:
+      for (int i = 0; i < 6; i++)
+        if (!c.ptr[i]) return bad("null operand");
+      if (!pos(c.dim[0]) || !pos(c.dim[1]) || !pos(c.dim[2])) return bad("bn: B,C,S must be positive");
+      if (c.dim[1] > 65535) return bad("bn: more than 65535 channels");
+      if (c.dim[0] * c.dim[2] < 2) return bad("bn: training statistics need at least two values per channel");
+      return GH_OK;
+    case GH_OP_BN_BWD:
+      for (int i = 0; i < 5; i++)
+        if (!c.ptr[i]) return bad("null operand");
+      if (!pos(c.dim[0]) || !pos(c.dim[1]) || !pos(c.dim[2])) return bad("bn: B,C,S must be positive");
+      if (c.dim[1] > 65535) return bad("bn: more than 65535 channels");
+      return GH_OK;
+    case GH_OP_SOFTMAX_BWD:
+      if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
+      if (c.dim[0] < 0 || !pos(c.dim[1])) return bad("softmax: bad shape");
       return GH_OK;
     case GH_OP_RELU:
     case GH_OP_LEAKY_RELU:

@@ -1,0 +1,330 @@
+// Backward passes of MaxPool2D, BatchNorm and SoftMax, and BatchNorm's
+// training-mode forward, for gfx950.  They stand where the reference calls
+// cuDNN PoolingBackward (ops/nn/maxpool_cuda.go:177-188),
+// BatchNormalizationForwardTraining / Backward (ops/nn/batchnorm_cuda.go:87-100,
+// 192-219) and where its CPU engine runs maxPoolDiffOp (op_nn.go:1042-1093),
+// BatchNormOp.updateStatsF32 (op_nn.go:1489-1555), batchnormDiffOp.f32s
+// (op_nn.go:1834-1943) and softmaxDiffOp (op_softmax.go:266-279); the
+// arithmetic follows the CPU engine.  All of them are HBM-bound.
+#include <cfloat>
+
+#include "gh_internal.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+
+struct PoolGeom {
+  int H, W, oh, ow, kh, kw, padH, padW, strideH, strideW;
+};
+
+// One thread per input element.  The reference zeroes dx and lets every
+// window, in (ph, pw) order, add its dy into the window's argmax (the first
+// element in row-major window order that beats everything before it, from
+// -FLT_MAX).  Gathering the same contributions per element in the same window
+// order gives the same bits without atomics, overlapping windows included.
+__global__ __launch_bounds__(kBlock) void k_maxpool2d_bwd(const float* __restrict__ x,
+                                                          const float* __restrict__ dy,
+                                                          float* __restrict__ dx, PoolGeom g,
+                                                          int64_t total) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  const int plane = g.H * g.W;
+  for (int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += stride) {
+    const int64_t bc = idx / plane;
+    const int me = (int)(idx - bc * plane);
+    const int iy = me / g.W, ix = me - iy * g.W;
+    const float* in = x + bc * (int64_t)plane;
+    const float* gy = dy + bc * (int64_t)g.oh * g.ow;
+    // windows whose extent [p*s - pad, p*s - pad + k) holds this row / column
+    const int ny = iy + g.padH - g.kh + 1, nx = ix + g.padW - g.kw + 1;
+    const int ph0 = ny > 0 ? (ny + g.strideH - 1) / g.strideH : 0;
+    const int pw0 = nx > 0 ? (nx + g.strideW - 1) / g.strideW : 0;
+    const int ph1 = min(g.oh - 1, (iy + g.padH) / g.strideH);
+    const int pw1 = min(g.ow - 1, (ix + g.padW) / g.strideW);
+    float acc = 0.0f;
+    for (int ph = ph0; ph <= ph1; ph++)
+      for (int pw = pw0; pw <= pw1; pw++) {
+        int hs = ph * g.strideH - g.padH, ws = pw * g.strideW - g.padW;
+        const int he = min(hs + g.kh, g.H), we = min(ws + g.kw, g.W);
+        hs = max(hs, 0);
+        ws = max(ws, 0);
+        float best = -FLT_MAX;
+        int arg = -1;
+        for (int hi = hs; hi < he; hi++)
+          for (int wi = ws; wi < we; wi++) {
+            const float v = in[hi * g.W + wi];
+            if (v > best) { best = v; arg = hi * g.W + wi; }
+          }
+        if (arg == me) acc = acc + gy[ph * g.ow + pw];
+      }
+    dx[idx] = acc;
+  }
+}
+
+// ---- BatchNorm: per-channel reductions ----------------------------------------------
+// A channel's n = B*S values are split over G workgroups; each reduces its share
+// with a fixed tree (so results repeat run to run), the consumers add the G
+// partial sums in index order.
+
+__device__ __forceinline__ float block_sum(float v, float* sh) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) sh[wave] = v;
+  __syncthreads();
+  const float r = (sh[0] + sh[1]) + (sh[2] + sh[3]);
+  __syncthreads();
+  return r;
+}
+
+__device__ __forceinline__ float sum_partials(const float* p, int G) {
+  float s = 0.0f;
+  for (int g = 0; g < G; g++) s = s + p[g];
+  return s;
+}
+
+// MODE 0: part[c][g] = sum x.  MODE 1: part[c][g] = sum (x - mean)^2 with
+// mean = (sum of the MODE 0 partials) / n.
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void k_bn_reduce(const float* __restrict__ x,
+                                                      const float* __restrict__ part_sum,
+                                                      float* __restrict__ part, int C, int64_t S,
+                                                      int64_t n) {
+  __shared__ float sh[4];
+  const int c = blockIdx.y, G = gridDim.x;
+  float mean = 0.0f;
+  if (MODE == 1) mean = sum_partials(part_sum + (int64_t)c * G, G) / (float)n;
+  float acc = 0.0f;
+  for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n; e += (int64_t)G * kBlock) {
+    const int64_t b = e / S, d = e - b * S;
+    const float v = x[(b * C + c) * S + d];
+    if (MODE == 0) acc = acc + v;
+    else {
+      const float t = v - mean;
+      acc = acc + t * t;
+    }
+  }
+  const float r = block_sum(acc, sh);
+  if (threadIdx.x == 0) part[(int64_t)c * G + blockIdx.x] = r;
+}
+
+// save_mean, save_var (the SUM of squared deviations, as the reference keeps
+// it), the running statistics (momentum weights the NEW value; unbiased
+// variance, op_nn.go:1547-1550) and the biased batch variance the apply pass
+// normalises with (op_nn.go:1573).
+__global__ __launch_bounds__(kBlock) void k_bn_train_finalize(const float* __restrict__ part_sum,
+                                                              const float* __restrict__ part_sq,
+                                                              float* __restrict__ run_mean,
+                                                              float* __restrict__ run_var,
+                                                              float* __restrict__ save_mean,
+                                                              float* __restrict__ save_var,
+                                                              float* __restrict__ batch_var,
+                                                              float momentum, int C, int G,
+                                                              int64_t n) {
+  const int c = blockIdx.x * kBlock + threadIdx.x;
+  if (c >= C) return;
+  const float mean = sum_partials(part_sum + (int64_t)c * G, G) / (float)n;
+  const float var = sum_partials(part_sq + (int64_t)c * G, G);
+  save_mean[c] = mean;
+  save_var[c] = var;
+  const float m1 = momentum * mean, m2 = (1.0f - momentum) * run_mean[c];
+  run_mean[c] = m1 + m2;
+  const float unb = var / (float)(n - 1);
+  const float v1 = momentum * unb, v2 = (1.0f - momentum) * run_var[c];
+  run_var[c] = v1 + v2;
+  batch_var[c] = var / (float)n;
+}
+
+// part[c][g][0] = sum dy, part[c][g][1] = sum (x*dy - mean*dy)  (op_nn.go:1897-1906;
+// for S == 1 the reference writes (x - mean)*dy, op_nn.go:1864-1866).
+__global__ __launch_bounds__(kBlock) void k_bn_bwd_reduce(const float* __restrict__ x,
+                                                          const float* __restrict__ dy,
+                                                          const float* __restrict__ save_mean,
+                                                          float* __restrict__ part, int C,
+                                                          int64_t S, int64_t n) {
+  __shared__ float sh[4];
+  const int c = blockIdx.y, G = gridDim.x;
+  const float mean = save_mean[c];
+  float s = 0.0f, dot = 0.0f;
+  for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n; e += (int64_t)G * kBlock) {
+    const int64_t b = e / S, d = e - b * S;
+    const int64_t i = (b * C + c) * S + d;
+    const float xv = x[i], g = dy[i];
+    s = s + g;
+    float p;
+    if (S == 1) {
+      const float t = xv - mean;
+      p = t * g;
+    } else {
+      const float t1 = xv * g, t2 = mean * g;
+      p = t1 - t2;
+    }
+    dot = dot + p;
+  }
+  const float rs = block_sum(s, sh);
+  const float rd = block_sum(dot, sh);
+  if (threadIdx.x == 0) {
+    part[((int64_t)c * G + blockIdx.x) * 2] = rs;
+    part[((int64_t)c * G + blockIdx.x) * 2 + 1] = rd;
+  }
+}
+
+// dx = (dy - gradMean - (x - mean)*k) * invstd in training mode, dy * invstd in
+// eval mode (op_nn.go:1908-1936), one (b, c) plane per blockIdx.y.
+__global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const float* __restrict__ x,
+                                                         const float* __restrict__ dy,
+                                                         float* __restrict__ dx,
+                                                         const float* __restrict__ save_mean,
+                                                         const float* __restrict__ save_var,
+                                                         const float* __restrict__ part, float eps,
+                                                         int training, int64_t BC, int C, int64_t S,
+                                                         int G, int64_t n) {
+  for (int64_t bc = blockIdx.y; bc < BC; bc += gridDim.y) {
+    const int c = (int)(bc % C);
+    float s = 0.0f, dot = 0.0f;
+    for (int g = 0; g < G; g++) {
+      s = s + part[((int64_t)c * G + g) * 2];
+      dot = dot + part[((int64_t)c * G + g) * 2 + 1];
+    }
+    const float mean = save_mean[c];
+    const float vb = save_var[c] / (float)n;
+    const float invstd = 1.0f / sqrtf(vb + eps);
+    float k = dot * invstd;
+    k = k * invstd;
+    k = k / (float)n;
+    const float grad_mean = s / (float)n;
+    const float* xi = x + bc * S;
+    const float* gi = dy + bc * S;
+    float* out = dx + bc * S;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < S; i += (int64_t)gridDim.x * kBlock) {
+      if (training) {
+        float t = xi[i] - mean;
+        t = t * k;
+        float u;
+        if (S == 1) { u = gi[i] - t; u = u - grad_mean; }
+        else { u = gi[i] - grad_mean; u = u - t; }
+        out[i] = u * invstd;
+      } else {
+        out[i] = gi[i] * invstd;
+      }
+    }
+  }
+}
+
+// SoftMax backward over the last axis, one wavefront per row:
+// dx_i = y_i * (dy_i - sum_j dy_j*y_j), the sum taken in column order (lane by
+// lane through readlane) like the forward kernel's, so it equals a sequential loop.
+__global__ __launch_bounds__(kBlock) void k_softmax_bwd(const float* __restrict__ y,
+                                                        const float* __restrict__ dy,
+                                                        float* __restrict__ dx, int64_t rows,
+                                                        int cols) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float* yy = y + row * cols;
+  const float* g = dy + row * cols;
+  float dot = 0.0f;
+  for (int j0 = 0; j0 < cols; j0 += 64) {
+    const int j = j0 + lane;
+    const float p = j < cols ? g[j] * yy[j] : 0.0f;
+    const int lim = min(64, cols - j0);
+    for (int l = 0; l < lim; l++) dot = dot + __shfl(p, l, 64);
+  }
+  for (int j = lane; j < cols; j += 64) {
+    const float t = g[j] - dot;
+    dx[row * cols + j] = yy[j] * t;
+  }
+}
+
+// how many workgroups share one channel's reduction
+int bn_groups(int64_t n) {
+  int64_t g = n / 4096;
+  if (g < 1) g = 1;
+  if (g > 64) g = 64;
+  return (int)g;
+}
+
+}  // namespace
+
+int gh_launch_maxpool2d_bwd(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t B = c.dim[0], C = c.dim[1];
+  PoolGeom g;
+  g.H = (int)c.dim[2]; g.W = (int)c.dim[3]; g.kh = (int)c.dim[4]; g.kw = (int)c.dim[5];
+  const int64_t padN = c.dim[6], padS = c.dim[7], padW = c.dim[8], padE = c.dim[9];
+  g.strideH = (int)c.dim[10]; g.strideW = (int)c.dim[11];
+  g.oh = (int)gh_pool_out(g.H, g.kh, padN, padS, g.strideH);
+  g.ow = (int)gh_pool_out(g.W, g.kw, padW, padE, g.strideW);
+  const bool explicit_pad = c.flags & GH_FLAG_EXPLICIT_PAD;  // south/east offsets, op_nn.go:871-875
+  g.padH = (int)(explicit_pad ? padS : padN);
+  g.padW = (int)(explicit_pad ? padE : padW);
+  const int64_t total = B * C * g.H * g.W;
+  if (total == 0) return GH_OK;
+  int64_t blocks = (total + kBlock - 1) / kBlock;
+  if (blocks > (int64_t)ctx->cu_count * 64) blocks = (int64_t)ctx->cu_count * 64;
+  hipLaunchKernelGGL(k_maxpool2d_bwd, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
+                     (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                     (float*)(uintptr_t)c.ptr[2], g, total);
+  return gh_check_hip(ctx, hipGetLastError(), "maxpool backward launch");
+}
+
+int gh_launch_bn_train(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t B = c.dim[0], C = c.dim[1], S = c.dim[2], n = B * S;
+  const int G = bn_groups(n);
+  // scratch: [C][G] sums, [C][G] squared deviations, [C] batch variance
+  const int64_t need = (2 * C * G + C) * 4;
+  if (need > ctx->workspace_bytes) return gh_fail(ctx, GH_ESTATE, "batchnorm: reduction scratch does not fit the workspace");
+  float* part_sum = (float*)ctx->workspace;
+  float* part_sq = part_sum + C * G;
+  float* batch_var = part_sq + C * G;
+  const float* x = (const float*)(uintptr_t)c.ptr[0];
+  hipLaunchKernelGGL((k_bn_reduce<0>), dim3(G, (int)C), dim3(kBlock), 0, ctx->stream, x, nullptr, part_sum,
+                     (int)C, S, n);
+  hipLaunchKernelGGL((k_bn_reduce<1>), dim3(G, (int)C), dim3(kBlock), 0, ctx->stream, x, part_sum, part_sq,
+                     (int)C, S, n);
+  hipLaunchKernelGGL(k_bn_train_finalize, dim3((int)((C + kBlock - 1) / kBlock)), dim3(kBlock), 0, ctx->stream,
+                     part_sum, part_sq, (float*)(uintptr_t)c.ptr[2], (float*)(uintptr_t)c.ptr[3],
+                     (float*)(uintptr_t)c.ptr[4], (float*)(uintptr_t)c.ptr[5], batch_var, c.f[1], (int)C, G, n);
+  int rc = gh_check_hip(ctx, hipGetLastError(), "batchnorm statistics launch");
+  if (rc) return rc;
+  // y = x*a + b with a = 1/sqrt(batch_var + eps), b = -mean*a: the inference kernel
+  gh_cmd a{};
+  a.opcode = GH_OP_BN_INFER;
+  a.ptr[0] = c.ptr[0]; a.ptr[1] = c.ptr[1]; a.ptr[2] = c.ptr[4]; a.ptr[3] = (uint64_t)(uintptr_t)batch_var;
+  a.dim[0] = B; a.dim[1] = C; a.dim[2] = S;
+  a.f[0] = c.f[0];
+  return gh_launch_bn_infer(ctx, a);
+}
+
+int gh_launch_bn_bwd(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t B = c.dim[0], C = c.dim[1], S = c.dim[2], n = B * S;
+  const int G = bn_groups(n);
+  if (2 * C * G * 4 > ctx->workspace_bytes) return gh_fail(ctx, GH_ESTATE, "batchnorm: reduction scratch does not fit the workspace");
+  float* part = (float*)ctx->workspace;
+  const float* x = (const float*)(uintptr_t)c.ptr[0];
+  const float* dy = (const float*)(uintptr_t)c.ptr[1];
+  float* dx = (float*)(uintptr_t)c.ptr[2];
+  const float* save_mean = (const float*)(uintptr_t)c.ptr[3];
+  const float* save_var = (const float*)(uintptr_t)c.ptr[4];
+  hipLaunchKernelGGL(k_bn_bwd_reduce, dim3(G, (int)C), dim3(kBlock), 0, ctx->stream, x, dy, save_mean, part,
+                     (int)C, S, n);
+  const int64_t BC = B * C;
+  int gx = (int)((S + kBlock * 4 - 1) / (kBlock * 4));
+  if (gx < 1) gx = 1;
+  if (gx > 1024) gx = 1024;
+  const int64_t gy = BC > 65535 ? 65535 : BC;
+  const int training = (c.flags & GH_FLAG_BN_EVAL) ? 0 : 1;
+  hipLaunchKernelGGL(k_bn_bwd_apply, dim3(gx, (int)gy), dim3(kBlock), 0, ctx->stream, x, dy, dx, save_mean,
+                     save_var, part, c.f[0], training, BC, (int)C, S, G, n);
+  return gh_check_hip(ctx, hipGetLastError(), "batchnorm backward launch");
+}
+
+int gh_launch_softmax_bwd(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t rows = c.dim[0];
+  const int cols = (int)c.dim[1];
+  if (rows == 0) return GH_OK;
+  const int64_t blocks = (rows + (kBlock / 64) - 1) / (kBlock / 64);
+  hipLaunchKernelGGL(k_softmax_bwd, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
+                     (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                     (float*)(uintptr_t)c.ptr[2], rows, cols);
+  return gh_check_hip(ctx, hipGetLastError(), "softmax backward launch");
+}

@@ -789,6 +789,168 @@ __global__ __launch_bounds__(256) void k_conv3x3_direct(const float* __restrict_
   }
 }
 
+// ---- Conv2d backward ---------------------------------------------------------------
+// The reference differentiates Conv2d through its im2col + MatMul graph
+// (nn.go:211-305): dW = dY2d^T . col and dX = col2im(dY2d . Wflat)
+// (op_nn.go:267-291, 605-640).  Here both are implicit GEMMs on the matrix
+// cores with no col buffer.
+//
+// Filter gradient: dW(F x CKK) = sum over pixels j = (b, oy, ox) of
+// dy[b][f][oy][ox] * x[b][c][oy*s - p + kr*d][ox*s - p + kc*d]: M = F, N = C*kh*kw,
+// K = B*oh*ow, split over K.
+
+// A operand: row f, k = pixel index across the batch, from NCHW dy.
+template <int R, int BK>
+struct LoadDyRows {
+  static constexpr int S = R + 2;
+  static constexpr int RSTEP = kThreads / BK;   // row distance between a thread's elements
+  static constexpr int RPT = R / RSTEP;
+  const float* dy; int F; int plane; int kmax /* B*plane */;
+  float reg[RPT];
+  __device__ __forceinline__ void load(int r0, int k0) {
+    const int kk = threadIdx.x % BK, rb = threadIdx.x / BK;
+    const int j = k0 + kk;
+    const bool ok = j < kmax;
+    const int b = ok ? j / plane : 0;
+    const int p = ok ? j - b * plane : 0;
+    const float* base = dy + (int64_t)b * F * plane + p;
+#pragma unroll
+    for (int i = 0; i < RPT; i++) {
+      const int f = r0 + rb + i * RSTEP;
+      reg[i] = (ok && f < F) ? base[(int64_t)f * plane] : 0.f;
+    }
+  }
+  __device__ __forceinline__ void store(float* lds) const {
+    const int kk = threadIdx.x % BK, rb = threadIdx.x / BK;
+#pragma unroll
+    for (int i = 0; i < RPT; i++) lds[kk * S + rb + i * RSTEP] = reg[i];
+  }
+};
+
+// B operand: column n = (c, kr, kc), k = pixel index: the im2col gather read the
+// other way round.  What depends only on the column is computed once.
+template <int R, int BK>
+struct LoadIm2colT {
+  static constexpr int S = R + 2;
+  static constexpr int RSTEP = kThreads / BK;
+  static constexpr int RPT = R / RSTEP;
+  const float* x; ConvGeom g; int nmax /* C*kh*kw */; int kmax /* B*oh*ow */;
+  int coff[RPT];   // c*H*W + kr*dilH*W + kc*dilW, or -1 for a column past the end
+  int dyo[RPT], dxo[RPT];
+  float reg[RPT];
+  __device__ __forceinline__ void init(int n0) {
+    const int rb = threadIdx.x / BK;
+    const int kk = g.kh * g.kw;
+#pragma unroll
+    for (int i = 0; i < RPT; i++) {
+      const int n = n0 + rb + i * RSTEP;
+      if (n < nmax) {
+        const int c = n / kk, r = n - c * kk;
+        const int kr = r / g.kw, kc = r - kr * g.kw;
+        dyo[i] = kr * g.dilH;
+        dxo[i] = kc * g.dilW;
+        coff[i] = c * g.H * g.W + dyo[i] * g.W + dxo[i];
+      } else {
+        coff[i] = -1; dyo[i] = 0; dxo[i] = 0;
+      }
+    }
+  }
+  __device__ __forceinline__ void load(int /*n0*/, int k0) {
+    const int j = k0 + threadIdx.x % BK;
+    const bool ok = j < kmax;
+    const int plane = g.oh * g.ow;
+    const int b = ok ? j / plane : 0;
+    const int rem = ok ? j - b * plane : 0;
+    const int oy = rem / g.ow, ox = rem - oy * g.ow;
+    const int iy0 = oy * g.strideH - g.padH, ix0 = ox * g.strideW - g.padW;
+    const float* xb = x + (int64_t)b * g.C * g.H * g.W + iy0 * g.W + ix0;
+#pragma unroll
+    for (int i = 0; i < RPT; i++) {
+      const int iy = iy0 + dyo[i], ix = ix0 + dxo[i];
+      const bool in = ok && coff[i] >= 0 && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+      reg[i] = in ? xb[coff[i]] : 0.f;
+    }
+  }
+  __device__ __forceinline__ void store(float* lds) const {
+    const int kk = threadIdx.x % BK, rb = threadIdx.x / BK;
+#pragma unroll
+    for (int i = 0; i < RPT; i++) lds[kk * S + rb + i * RSTEP] = reg[i];
+  }
+};
+
+template <int BM, int BN, int BK, int WAVES_M>
+__global__ __launch_bounds__(kThreads) void k_conv2d_wgrad(const float* __restrict__ x,
+                                                           const float* __restrict__ dy,
+                                                           float* __restrict__ dw, ConvGeom g,
+                                                           int F, int CKK, int splits,
+                                                           float* __restrict__ ws) {
+  using LA = LoadDyRows<BM, BK>;
+  using LB = LoadIm2colT<BN, BK>;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  LA la; la.dy = dy; la.F = F; la.plane = g.oh * g.ow; la.kmax = g.P;
+  LB lb; lb.x = x; lb.g = g; lb.nmax = CKK; lb.kmax = g.P;
+  lb.init(n0);
+  const int nk = (g.P + BK - 1) / BK;
+  __shared__ float lds[2 * BK * (LA::S + LB::S)];
+  if (splits > 1) {
+    int kt0, kt1;
+    split_range(nk, splits, blockIdx.z, &kt0, &kt1);
+    StorePartial sc{ws + (int64_t)blockIdx.z * F * CKK, CKK};
+    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StorePartial>(lds, la, lb, sc, F, CKK, kt0, kt1, m0, n0, 0, 0.f);
+  } else {
+    StoreRowMajor sc{dw, CKK};
+    mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreRowMajor>(lds, la, lb, sc, F, CKK, 0, nk, m0, n0, 0, 0.f);
+  }
+}
+
+// Input gradient, stride 1: dX is the forward convolution of dy with the
+// filters mirrored and their channel axes swapped, under padding
+// dil*(k-1) - pad, so the forward kernels compute it.  This writes those filters:
+// wt[c][f][kr][kc] = w[f][c][kh-1-kr][kw-1-kc].
+__global__ __launch_bounds__(256) void k_flip_filters(const float* __restrict__ w,
+                                                      float* __restrict__ wt, int F, int C, int kh,
+                                                      int kw) {
+  const int64_t total = (int64_t)F * C * kh * kw;
+  const int kk = kh * kw;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int r = (int)(i % kk);
+    const int64_t cf = i / kk;
+    const int f = (int)(cf % F), c = (int)(cf / F);
+    wt[i] = w[((int64_t)f * C + c) * kk + (kk - 1 - r)];
+  }
+}
+
+// Input gradient for any stride: one thread per dx element gathers the
+// (f, kr, kc) terms whose window position divides evenly.  Not on the matrix
+// cores; strided convolutions are rare on this path.
+__global__ __launch_bounds__(256) void k_conv2d_dgrad_gather(const float* __restrict__ dy,
+                                                             const float* __restrict__ w,
+                                                             float* __restrict__ dx, ConvGeom g,
+                                                             int B, int F) {
+  const int64_t total = (int64_t)B * g.C * g.H * g.W;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int ix = (int)(i % g.W), iy = (int)((i / g.W) % g.H);
+    const int c = (int)((i / ((int64_t)g.W * g.H)) % g.C), b = (int)(i / ((int64_t)g.W * g.H * g.C));
+    float acc = 0.f;
+    for (int kr = 0; kr < g.kh; kr++) {
+      const int ty = iy + g.padH - kr * g.dilH;
+      if (ty < 0 || ty % g.strideH) continue;
+      const int oy = ty / g.strideH;
+      if (oy >= g.oh) continue;
+      for (int kc = 0; kc < g.kw; kc++) {
+        const int tx = ix + g.padW - kc * g.dilW;
+        if (tx < 0 || tx % g.strideW) continue;
+        const int ox = tx / g.strideW;
+        if (ox >= g.ow) continue;
+        for (int f = 0; f < F; f++)
+          acc = __builtin_fmaf(dy[(((int64_t)b * F + f) * g.oh + oy) * g.ow + ox],
+                               w[(((int64_t)f * g.C + c) * g.kh + kr) * g.kw + kc], acc);
+      }
+    }
+    dx[i] = acc;
+  }
+}
+
 // ---- GEMV / outer ------------------------------------------------------------------
 // y(m) = A(m x n) x: one wavefront per row, float4 loads when the row is
 // 16-byte aligned, butterfly reduction across the 64 lanes.
@@ -1174,6 +1336,85 @@ int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
   if (p.tile == kTile128) return launch_conv_k<128, 128, 2>(ctx, c, g, F, K, p.splits);
   if (p.tile == kTile32x256) return launch_conv_k<32, 256, 1>(ctx, c, g, F, K, p.splits);
   return launch_conv_k<64, 64, 2>(ctx, c, g, F, K, p.splits);
+}
+
+static ConvGeom conv_geom(const gh_cmd& c) {
+  ConvGeom g;
+  g.C = (int)c.dim[1]; g.H = (int)c.dim[2]; g.W = (int)c.dim[3];
+  g.kh = (int)c.dim[5]; g.kw = (int)c.dim[6];
+  g.padH = (int)c.dim[7]; g.padW = (int)c.dim[8];
+  g.strideH = (int)c.dim[9]; g.strideW = (int)c.dim[10];
+  g.dilH = (int)c.dim[11]; g.dilW = (int)c.dim[12];
+  g.oh = (int)gh_conv_out(g.H, g.kh, g.padH, g.strideH, g.dilH);
+  g.ow = (int)gh_conv_out(g.W, g.kw, g.padW, g.strideW, g.dilW);
+  g.P = (int)c.dim[0] * g.oh * g.ow;
+  return g;
+}
+
+// dW = dY2d^T . col  (ptr[0] = x, ptr[1] = dy, ptr[2] = dw)
+int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
+  const ConvGeom g = conv_geom(c);
+  const int F = (int)c.dim[4], CKK = g.C * g.kh * g.kw;
+  constexpr int BM = 64, BN = 64, BK = 16;
+  const int64_t tiles = cdiv(F, BM) * cdiv(CKK, BN);
+  const int64_t nk = cdiv(g.P, BK);
+  int64_t splits = cdiv(5 * (int64_t)ctx->cu_count / 2, tiles);   // ~2.5 workgroups per CU
+  if (splits > nk / 4) splits = nk / 4;
+  if (splits > 64) splits = 64;
+  const int64_t slab = (int64_t)F * CKK * 4;
+  if (ctx->workspace_bytes / slab < splits) splits = ctx->workspace_bytes / slab;
+  if (splits < 1) splits = 1;
+  const float* x = (const float*)(uintptr_t)c.ptr[0];
+  const float* dy = (const float*)(uintptr_t)c.ptr[1];
+  float* dw = (float*)(uintptr_t)c.ptr[2];
+  float* ws = (float*)ctx->workspace;
+  const dim3 grid((unsigned)cdiv(CKK, BN), (unsigned)cdiv(F, BM), (unsigned)splits);
+  hipLaunchKernelGGL((k_conv2d_wgrad<BM, BN, BK, 2>), grid, dim3(kThreads), 0, ctx->stream, x, dy, dw, g, F,
+                     CKK, (int)splits, ws);
+  int rc = gh_check_hip(ctx, hipGetLastError(), "conv filter-gradient launch");
+  if (rc || splits <= 1) return rc;
+  int64_t blocks = cdiv((int64_t)F * CKK, 256);
+  if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
+  hipLaunchKernelGGL((k_splitk_reduce<StoreRowMajor>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws,
+                     (int)splits, F, CKK, StoreRowMajor{dw, CKK}, 0, 0.f);
+  return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
+}
+
+// dX = col2im(dY2d . Wflat)  (ptr[0] = dy, ptr[1] = w, ptr[2] = dx)
+int gh_launch_conv2d_bwd_data(gh_ctx* ctx, const gh_cmd& c) {
+  const ConvGeom g = conv_geom(c);
+  const int B = (int)c.dim[0], F = (int)c.dim[4];
+  const float* dy = (const float*)(uintptr_t)c.ptr[0];
+  const float* w = (const float*)(uintptr_t)c.ptr[1];
+  float* dx = (float*)(uintptr_t)c.ptr[2];
+  const int64_t wbytes = ((int64_t)F * g.C * g.kh * g.kw * 4 + 255) / 256 * 256;
+  const int padH = g.dilH * (g.kh - 1) - g.padH, padW = g.dilW * (g.kw - 1) - g.padW;
+  if (g.strideH == 1 && g.strideW == 1 && padH >= 0 && padW >= 0 && wbytes <= ctx->workspace_bytes / 4) {
+    // mirrored filters live at the top of the workspace; the forward launch
+    // below may use what is left of it for its own split-K slabs
+    float* wt = (float*)((char*)ctx->workspace + ctx->workspace_bytes - wbytes);
+    int64_t blocks = cdiv((int64_t)F * g.C * g.kh * g.kw, 256);
+    if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
+    hipLaunchKernelGGL(k_flip_filters, dim3((int)blocks), dim3(256), 0, ctx->stream, w, wt, F, g.C, g.kh, g.kw);
+    int rc = gh_check_hip(ctx, hipGetLastError(), "filter mirror launch");
+    if (rc) return rc;
+    gh_cmd f{};
+    f.opcode = GH_OP_CONV2D;
+    f.ptr[0] = c.ptr[0]; f.ptr[1] = (uint64_t)(uintptr_t)wt; f.ptr[2] = c.ptr[2];
+    f.dim[0] = B; f.dim[1] = F; f.dim[2] = g.oh; f.dim[3] = g.ow; f.dim[4] = g.C;
+    f.dim[5] = g.kh; f.dim[6] = g.kw; f.dim[7] = padH; f.dim[8] = padW;
+    f.dim[9] = 1; f.dim[10] = 1; f.dim[11] = g.dilH; f.dim[12] = g.dilW;
+    const int64_t keep = ctx->workspace_bytes;
+    ctx->workspace_bytes = keep - wbytes;
+    rc = gh_launch_conv2d(ctx, f);
+    ctx->workspace_bytes = keep;
+    return rc;
+  }
+  const int64_t total = (int64_t)B * g.C * g.H * g.W;
+  int64_t blocks = cdiv(total, 256);
+  if (blocks > (int64_t)ctx->cu_count * 32) blocks = (int64_t)ctx->cu_count * 32;
+  hipLaunchKernelGGL(k_conv2d_dgrad_gather, dim3((int)blocks), dim3(256), 0, ctx->stream, dy, w, dx, g, B, F);
+  return gh_check_hip(ctx, hipGetLastError(), "conv input-gradient launch");
 }
 
 int gh_launch_gemv(gh_ctx* ctx, const gh_cmd& c) {

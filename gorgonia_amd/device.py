@@ -225,6 +225,39 @@ def cmd_softmax(x, y, rows, cols):
     return make_cmd(_ffi.OP_SOFTMAX, 0, (x, y), (rows, cols))
 
 
+def cmd_maxpool2d_bwd(x, dy, dx, B, Cn, H, W, kh, kw, pad, stride):
+    c = cmd_maxpool2d(x, dy, B, Cn, H, W, kh, kw, pad, stride)
+    c.opcode = _ffi.OP_MAXPOOL2D_BWD
+    c.ptr[2] = int(dx)
+    return c
+
+
+def _conv_dims(B, Cin, H, W, F, kh, kw, pad, stride, dilation):
+    return (B, Cin, H, W, F, kh, kw, pad[0], pad[1], stride[0], stride[1], dilation[0], dilation[1])
+
+
+def cmd_conv2d_bwd_data(dy, w, dx, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dilation=(1, 1)):
+    """dx of Conv2d; B, Cin, H, W describe x (and dx)."""
+    return make_cmd(_ffi.OP_CONV2D_BWD_DATA, 0, (dy, w, dx), _conv_dims(B, Cin, H, W, F, kh, kw, pad, stride, dilation))
+
+
+def cmd_conv2d_bwd_filter(x, dy, dw, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dilation=(1, 1)):
+    return make_cmd(_ffi.OP_CONV2D_BWD_FILTER, 0, (x, dy, dw), _conv_dims(B, Cin, H, W, F, kh, kw, pad, stride, dilation))
+
+
+def cmd_bn_train(x, y, run_mean, run_var, save_mean, save_var, B, Cn, S, eps, momentum):
+    return make_cmd(_ffi.OP_BN_TRAIN, 0, (x, y, run_mean, run_var, save_mean, save_var), (B, Cn, S), (eps, momentum))
+
+
+def cmd_bn_bwd(x, dy, dx, save_mean, save_var, B, Cn, S, eps, training=True):
+    return make_cmd(_ffi.OP_BN_BWD, 0 if training else _ffi.FLAG_BN_EVAL, (x, dy, dx, save_mean, save_var),
+                    (B, Cn, S), (eps,))
+
+
+def cmd_softmax_bwd(y, dy, dx, rows, cols):
+    return make_cmd(_ffi.OP_SOFTMAX_BWD, 0, (y, dy, dx), (rows, cols))
+
+
 def cmd_has(kind, a, flag, n, dtype=_ffi.F32):
     op = _ffi.OP_HAS_NAN if kind == "nan" else _ffi.OP_HAS_INF
     return make_cmd(op, _ffi.flag_dtype(dtype), (a, flag), (n,))

@@ -80,6 +80,13 @@ enum gh_opcode {
   GH_OP_HAS_NAN = 14,   /* misc.hasNaN (cuda/engine.go:144-166)               */
   GH_OP_HAS_INF = 15,   /* misc.hasInf (cuda/engine.go:169-191)               */
   GH_OP_FILL = 16,      /* Memset of a float value                            */
+  /* backward passes and the training-mode BatchNorm forward */
+  GH_OP_MAXPOOL2D_BWD = 17,     /* ops/nn/maxpool_cuda.go:177-188; CPU op_nn.go:1042-1093      */
+  GH_OP_CONV2D_BWD_DATA = 18,   /* ops/nn/convolution_cuda.go:192-229; CPU col2im op_nn.go:605 */
+  GH_OP_CONV2D_BWD_FILTER = 19, /* ops/nn/convolution_cuda.go:230-267                          */
+  GH_OP_BN_TRAIN = 20,          /* ops/nn/batchnorm_cuda.go:87-100; CPU op_nn.go:1489-1635     */
+  GH_OP_BN_BWD = 21,            /* ops/nn/batchnorm_cuda.go:192-219; CPU op_nn.go:1834-1943    */
+  GH_OP_SOFTMAX_BWD = 22,       /* softmaxDiffOp, op_softmax.go:266-279                        */
   GH_OP__COUNT
 };
 
@@ -113,6 +120,7 @@ enum gh_unaryfn {
 #define GH_FLAG_ACT_RELU     (1u << 22)   /* CONV2D/GEMM epilogue: x*(x>=0)    */
 #define GH_FLAG_ACT_LEAKY    (1u << 23)   /* epilogue: leaky relu, alpha=f[0]  */
 #define GH_FLAG_CONV_BN      (1u << 24)   /* CONV2D: BatchNorm (eval) on the result, ptr[3..6] */
+#define GH_FLAG_BN_EVAL      (1u << 26)   /* BN_BWD: eval-mode gradient dy/sqrt(var+eps)       */
 #define GH_FLAG_CONV_POOL2   (1u << 25)   /* CONV2D: 2x2 stride-2 unpadded MaxPool2D on the result */
 
 /*
@@ -151,6 +159,16 @@ enum gh_unaryfn {
  * HAS_NAN/INF ptr[0]=A ptr[1]=int32 flag (device)  dim[0]=n ; flag is set to 1
  *             if any element matches, else 0
  * FILL        ptr[0]=A                     dim[0]=n f[0]=value
+ * MAXPOOL2D_BWD     ptr[0]=x ptr[1]=dy ptr[2]=dx ; dims as MAXPOOL2D.  dx gets, per element,
+ *             the dy of every window whose argmax it is (first maximum in scan order)
+ * CONV2D_BWD_DATA   ptr[0]=dy ptr[1]=w ptr[2]=dx ; dims as CONV2D (B,C,H,W describe x / dx)
+ * CONV2D_BWD_FILTER ptr[0]=x ptr[1]=dy ptr[2]=dw ; dims as CONV2D
+ * BN_TRAIN    ptr[0]=x ptr[1]=y ptr[2]=running_mean ptr[3]=running_var (both updated)
+ *             ptr[4]=save_mean ptr[5]=save_var (outputs; save_var is the SUM of squared
+ *             deviations, op_nn.go:1536-1541)  dim[0..2]=B,C,S  f[0]=eps f[1]=momentum
+ * BN_BWD      ptr[0]=x ptr[1]=dy ptr[2]=dx ptr[3]=save_mean ptr[4]=save_var
+ *             dim[0..2]=B,C,S  f[0]=eps ; BN_EVAL selects dx = dy/sqrt(save_var/n + eps)
+ * SOFTMAX_BWD ptr[0]=y ptr[1]=dy ptr[2]=dx        dim[0]=rows dim[1]=cols
  */
 typedef struct gh_cmd {
   uint32_t opcode;

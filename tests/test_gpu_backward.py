@@ -1,0 +1,158 @@
+"""GPU parity of the backward passes and the training-mode BatchNorm forward,
+through the C ABI against the CPU oracle.  Bars: max-pool gradient bit-exact
+(pure selection and ordered adds); softmax gradient <= 2 ulp; conv gradients
+<= 1e-5 relative Frobenius against the float64 definition (exact on integer
+data); BatchNorm statistics, output and gradient <= 1e-5 relative (parallel
+reduction order differs from the CPU's sequential sums)."""
+import numpy as np
+import pytest
+
+from gorgonia_amd import device as D
+from gorgonia_amd import synth
+from oracle import binding as O
+from tests.util import assert_bits_equal, rel_frobenius, ulp_diff
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+POOL_CASES = [
+    # B, C, H, W, kernel, pad, stride
+    (2, 3, 8, 10, (2, 2), (0, 0), (2, 2)),
+    (2, 3, 9, 11, (2, 2), (0, 0), (2, 2)),
+    (1, 2, 3, 4, (2, 2), (0, 0), (1, 1)),
+    (2, 4, 13, 13, (2, 2), (1, 0, 1, 0), (1, 1)),   # darknet stride-1 pool
+    (2, 3, 12, 9, (3, 3), (1, 1), (2, 2)),
+    (1, 2, 7, 8, (3, 2), (1, 1), (1, 2)),
+    (16, 32, 28, 28, (2, 2), (0, 0), (2, 2)),        # convnet pool 0 (batch trimmed)
+]
+
+
+@pytest.mark.parametrize("cfg", POOL_CASES)
+def test_maxpool_backward_bit_exact(ctx, cfg):
+    B, C, H, W, kernel, pad, stride = cfg
+    rng = np.random.default_rng(1)
+    for x in (synth.normal(7, (B, C, H, W)), rng.integers(-2, 3, (B, C, H, W)).astype(np.float32)):
+        oh, ow = O.maxpool_out_hw(H, W, kernel[0], kernel[1], pad, stride)
+        dy = synth.normal(8, (B, C, oh, ow))
+        dx_, dy_, dd = ctx.upload(x), ctx.upload(dy), ctx.malloc(x.size * 4)
+        ctx.run(D.cmd_fill(dd, x.size, np.nan))
+        ctx.run(D.cmd_maxpool2d_bwd(dx_, dy_, dd, B, C, H, W, kernel[0], kernel[1], pad, stride))
+        got = ctx.d2h(dd, x.shape)
+        for p in (dx_, dy_, dd):
+            ctx.free(p)
+        assert_bits_equal(got, O.maxpool2d_bwd(x, dy, kernel, pad, stride), f"maxpool backward {cfg}")
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (7, 10), (128, 10), (5, 64), (3, 65), (4, 1000)])
+def test_softmax_backward(ctx, shape):
+    x = synth.normal(3, shape)
+    y = O.softmax(x)
+    dy = synth.normal(4, shape)
+    py, pg, pd = ctx.upload(y), ctx.upload(dy), ctx.malloc(y.size * 4)
+    ctx.run(D.cmd_softmax_bwd(py, pg, pd, shape[0], shape[1]))
+    got = ctx.d2h(pd, shape)
+    for p in (py, pg, pd):
+        ctx.free(p)
+    want = O.softmax_bwd(y, dy)
+    assert ulp_diff(got, want).max() <= 2
+    assert np.allclose(got.sum(axis=1), 0, atol=1e-5)
+
+
+CONV_BWD_CASES = [
+    # B, C, H, W, F, kh, kw, pad, stride, dil
+    (2, 3, 8, 9, 5, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (1, 4, 7, 7, 6, 1, 1, (0, 0), (1, 1), (1, 1)),
+    (2, 2, 10, 11, 3, 3, 2, (2, 1), (2, 3), (1, 1)),       # strided: gather kernel for dx
+    (1, 3, 12, 12, 4, 3, 3, (2, 2), (1, 1), (2, 2)),
+    (2, 5, 9, 9, 7, 5, 5, (2, 2), (1, 1), (1, 1)),
+    (2, 4, 9, 9, 3, 3, 3, (3, 3), (1, 1), (1, 1)),          # padding wider than the kernel reach: gather kernel
+    (16, 1, 28, 28, 32, 3, 3, (1, 1), (1, 1), (1, 1)),      # convnet layers, batch trimmed
+    (16, 32, 14, 14, 64, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (16, 64, 7, 7, 128, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (2, 16, 52, 52, 32, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (2, 256, 13, 13, 512, 3, 3, (1, 1), (1, 1), (1, 1)),
+]
+
+
+def gpu_conv_bwd(ctx, x, w, dy, pad, stride, dil):
+    B, C, H, W = x.shape
+    F, _, kh, kw = w.shape
+    px, pw, pg = ctx.upload(x), ctx.upload(w), ctx.upload(dy)
+    pdx, pdw = ctx.malloc(x.size * 4), ctx.malloc(w.size * 4)
+    ctx.run([D.cmd_fill(pdx, x.size, np.nan), D.cmd_fill(pdw, w.size, np.nan)])
+    ctx.run([D.cmd_conv2d_bwd_data(pg, pw, pdx, B, C, H, W, F, kh, kw, pad, stride, dil),
+             D.cmd_conv2d_bwd_filter(px, pg, pdw, B, C, H, W, F, kh, kw, pad, stride, dil)])
+    dx, dw = ctx.d2h(pdx, x.shape), ctx.d2h(pdw, w.shape)
+    for p in (px, pw, pg, pdx, pdw):
+        ctx.free(p)
+    return dx, dw
+
+
+@pytest.mark.parametrize("cfg", CONV_BWD_CASES)
+def test_conv_backward_vs_oracle(ctx, cfg):
+    B, C, H, W, F, kh, kw, pad, stride, dil = cfg
+    x = synth.uniform(300 + C, (B, C, H, W), -1, 1)
+    w = synth.he_normal(400 + F, (F, C, kh, kw))
+    oh, ow = O.conv_out_hw(H, W, kh, kw, pad, stride, dil)
+    dy = synth.normal(500 + F, (B, F, oh, ow))
+    dx, dw = gpu_conv_bwd(ctx, x, w, dy, pad, stride, dil)
+    if B * C * H * W * F * kh * kw <= 4e8:
+        rx, rw = O.conv2d_bwd_direct_f64(x, w, dy, pad, stride, dil)   # float64 definition
+    else:
+        rx, rw = O.conv2d_bwd(x, w, dy, pad, stride, dil)              # float32 port (pinned to the definition)
+    assert rel_frobenius(dx, rx) <= TOL, f"dx {cfg}: {rel_frobenius(dx, rx):.3e}"
+    assert rel_frobenius(dw, rw) <= TOL, f"dw {cfg}: {rel_frobenius(dw, rw):.3e}"
+    # integer data: exact whatever the accumulation order
+    rng = np.random.default_rng(7)
+    xi = rng.integers(-3, 4, x.shape).astype(np.float32)
+    wi = rng.integers(-3, 4, w.shape).astype(np.float32)
+    di = rng.integers(-2, 3, dy.shape).astype(np.float32)
+    dxi, dwi = gpu_conv_bwd(ctx, xi, wi, di, pad, stride, dil)
+    oxi, owi = O.conv2d_bwd(xi, wi, di, pad, stride, dil)
+    assert_bits_equal(dxi, oxi, f"integer dx {cfg}")
+    assert_bits_equal(dwi, owi, f"integer dw {cfg}")
+
+
+BN_CASES = [(3, 2, 1), (6, 4, 1), (2, 2, 4), (4, 3, 25), (8, 16, 26 * 26), (2, 32, 104 * 104), (128, 10, 1)]
+
+
+@pytest.mark.parametrize("B,C,S", BN_CASES)
+def test_batchnorm_training_forward_and_backward(ctx, B, C, S):
+    x = synth.normal(21, (B, C, S), 0.5, 2.0)
+    dy = synth.normal(22, (B, C, S))
+    rm0, rv0 = synth.normal(23, (C,), 0.0, 0.1), synth.uniform(24, (C,), 0.5, 1.5)
+    px, pg = ctx.upload(x), ctx.upload(dy)
+    py, pdx = ctx.malloc(x.size * 4), ctx.malloc(x.size * 4)
+    prm, prv = ctx.upload(rm0), ctx.upload(rv0)
+    psm, psv = ctx.malloc(C * 4), ctx.malloc(C * 4)
+    ctx.run(D.cmd_bn_train(px, py, prm, prv, psm, psv, B, C, S, 1e-5, 0.9))
+    y, rm, rv = ctx.d2h(py, x.shape), ctx.d2h(prm, (C,)), ctx.d2h(prv, (C,))
+    sm, sv = ctx.d2h(psm, (C,)), ctx.d2h(psv, (C,))
+    wy, wrm, wrv, wsm, wsv = O.bn_train_stats(x, rm0, rv0, 0.9, 1e-5)
+    assert np.allclose(sm, wsm, rtol=1e-5, atol=1e-6) and np.allclose(sv, wsv, rtol=1e-5)
+    assert np.allclose(rm, wrm, rtol=1e-5, atol=1e-6) and np.allclose(rv, wrv, rtol=1e-5)
+    assert rel_frobenius(y, wy) <= TOL
+    # the reductions also agree with float64 sums of the same data
+    x64 = x.astype(np.float64)
+    assert np.allclose(sm, x64.mean(axis=(0, 2)), rtol=1e-5, atol=1e-6)
+    assert np.allclose(sv, ((x64 - x64.mean(axis=(0, 2), keepdims=True)) ** 2).sum(axis=(0, 2)), rtol=1e-5)
+    for training in (True, False):
+        ctx.run(D.cmd_bn_bwd(px, pg, pdx, psm, psv, B, C, S, 1e-5, training=training))
+        dx = ctx.d2h(pdx, x.shape)
+        want = O.bn_bwd(x, dy, sm, sv, 1e-5, training=training)   # same saved statistics as the device used
+        assert rel_frobenius(dx, want) <= TOL, f"bn backward training={training}: {rel_frobenius(dx, want):.3e}"
+    for p in (px, pg, py, pdx, prm, prv, psm, psv):
+        ctx.free(p)
+
+
+def test_backward_commands_validate(ctx):
+    import ctypes as C
+    buf = C.create_string_buffer(256)
+    bad = D.cmd_conv2d_bwd_data(0x1000, 0x2000, 0x3000, 2, 8, 14, 14, 16, 3, 3, (1, 1))
+    bad.flags |= 1 << 22
+    assert ctx.lib.gh_validate(C.byref(bad), 1, buf, 256) != 0
+    ok = D.cmd_conv2d_bwd_filter(0x1000, 0x2000, 0x3000, 2, 8, 14, 14, 16, 3, 3, (1, 1))
+    assert ctx.lib.gh_validate(C.byref(ok), 1, buf, 256) == 0
+    assert ctx.lib.gh_validate(C.byref(D.cmd_bn_train(1, 2, 3, 4, 5, 6, 1, 4, 1, 1e-5, 0.9)), 1, buf, 256) != 0
+    assert ctx.lib.gh_validate(C.byref(D.cmd_softmax_bwd(1, 2, 0, 4, 4)), 1, buf, 256) != 0
