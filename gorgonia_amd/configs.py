@@ -105,6 +105,52 @@ def build_convnet(inp, resident=True):
     return g, {"out": G.Read(out)}
 
 
+def build_convnet_train(inp, onehot, lr, read_grads=True):
+    """Config 4 as one training step (examples/convnet/main.go:57-180 with vanilla
+    SGD): forward, the diff ops the reference's symbolic differentiation would
+    insert, and w <- w - lr * dw through Set, so the resident weights carry over
+    to the next RunAll.  cost = -Mean(out * onehot)."""
+    g = G.NewGraph()
+    b = inp["x"].shape[0]
+    x = G.NewTensor(g, inp["x"], True)
+    y = G.NewTensor(g, onehot, True)
+    w = [G.NewTensor(g, inp[f"w{i}"], True) for i in range(5)]
+    zero = G.NewScalar(g, 0.0)
+    lr_s = G.NewScalar(g, lr)
+    scale = G.NewScalar(g, -1.0 / onehot.size)
+    conv = dict(kernelShape=(3, 3), pad=(1, 1), stride=(1, 1), dilation=(1, 1))
+    acts, h = [], x
+    for i in range(3):
+        z = G.Conv2d(h, w[i], (3, 3), (1, 1), (1, 1), (1, 1))
+        a = G.Rectify(z)
+        acts.append((h, z, a))
+        h = G.MaxPool2D(a, (2, 2), (0, 0), (2, 2))
+    r = G.Reshape(h, (b, 128 * 3 * 3))
+    z3 = G.Mul(r, w[3])
+    a3 = G.Rectify(z3)
+    out = G.SoftMax(G.Mul(a3, w[4]))
+    outs = {"out": G.Read(out)}
+    # backward
+    g4 = G.SoftMaxDiff(out, G.HadamardProd(y, scale))
+    dw = {4: G.Mul(a3, g4, transA=True)}
+    dz3 = G.HadamardProd(G.Mul(g4, w[4], transB=True), G.Gte(z3, zero))
+    dw[3] = G.Mul(r, dz3, transA=True)
+    grad = G.Reshape(G.Mul(dz3, w[3], transB=True), h.Shape())
+    for i in (2, 1, 0):
+        x_in, z, a = acts[i]
+        dz = G.HadamardProd(G.MaxPool2DDiff(a, grad, (2, 2), (0, 0), (2, 2)), G.Gte(z, zero))
+        dw[i] = G.Conv2dDiffFilter(x_in, dz, **conv)
+        if i:
+            grad = G.Conv2dDiffImage(dz, w[i], x_in.Shape(), **conv)
+    if read_grads:
+        for i in range(5):
+            outs[f"dw{i}"] = G.Read(dw[i])
+    # updates last: every gradient above was taken at the old weights
+    for i in range(5):
+        G.Set(w[i], G.Sub(w[i], G.HadamardProd(dw[i], lr_s)))
+    return g, outs
+
+
 def build_yolo(inp, resident=True, resident_input=False):
     g = G.NewGraph()
     h = G.NewTensor(g, inp["x"], resident_input)

@@ -13,7 +13,8 @@ from . import _ffi
 from .engine import Engine, EngineError, GhhOp, load_host
 
 (K_ELEMBIN, K_ELEMUNARY, K_BCAST, K_MATMUL, K_MATVEC, K_OUTER, K_BMM, K_CONV2D, K_MAXPOOL, K_BN,
- K_RECTIFY, K_LEAKY, K_SOFTMAX, K_RESHAPE) = range(14)
+ K_RECTIFY, K_LEAKY, K_SOFTMAX, K_RESHAPE, K_MAXPOOL_DIFF, K_CONV_DIFF_DATA, K_CONV_DIFF_FILTER, K_BN_TRAIN,
+ K_BN_DIFF, K_SOFTMAX_DIFF, K_SET) = range(21)
 
 
 class Node:
@@ -44,7 +45,7 @@ class ExprGraph:
         n = self.lib.ghh_graph_node_shape(self.h, nid, buf, 8)
         return tuple(buf[i] for i in range(n))
 
-    def apply(self, kind, inputs, fn=0, name="", trans_a=False, trans_b=False, ints=(), f0=0.0):
+    def apply(self, kind, inputs, fn=0, name="", trans_a=False, trans_b=False, ints=(), f0=0.0, f1=0.0):
         op = GhhOp()
         op.kind, op.fn, op.name = kind, fn, name.encode()
         op.trans_a, op.trans_b = int(trans_a), int(trans_b)
@@ -52,6 +53,7 @@ class ExprGraph:
         for i, v in enumerate(ints):
             op.ints[i] = int(v)
         op.f0 = float(f0)
+        op.f1 = float(f1)
         arr = (C.c_int * len(inputs))(*[n.id for n in inputs])
         out = C.c_int()
         self._check(self.lib.ghh_graph_apply(self.h, C.byref(op), arr, len(inputs), C.byref(out)))
@@ -172,6 +174,47 @@ def SoftMax(x):
 
 def Reshape(x, shape):
     return x.g.apply(K_RESHAPE, [x], ints=list(shape))
+
+
+# ---- the diff ops symbolic differentiation inserts, for hand-built training graphs ----
+
+def MaxPool2DDiff(x, grad, kernel, pad, stride):
+    """maxPoolDiffOp (op_nn.go:962-1093): gradient of MaxPool2D(x, kernel, pad, stride) wrt x."""
+    return x.g.apply(K_MAXPOOL_DIFF, [x, grad], ints=list(kernel) + [len(pad)] + list(pad) + list(stride))
+
+
+def Conv2dDiffImage(grad, filter, imageShape, kernelShape, pad=(0, 0), stride=(1, 1), dilation=(1, 1)):
+    """Gradient of Conv2d wrt the image (col2im of grad2d . filter, op_nn.go:267-291, 605-640)."""
+    ints = list(kernelShape) + list(pad) + list(stride) + list(dilation) + list(imageShape)
+    return grad.g.apply(K_CONV_DIFF_DATA, [grad, filter], ints=ints)
+
+
+def Conv2dDiffFilter(im, grad, kernelShape, pad=(0, 0), stride=(1, 1), dilation=(1, 1)):
+    """Gradient of Conv2d wrt the filter (grad2d^T . im2col(im))."""
+    return im.g.apply(K_CONV_DIFF_FILTER, [im, grad], ints=list(kernelShape) + list(pad) + list(stride) + list(dilation))
+
+
+def BatchNormTrain(x, runningMean, runningVariance, saveMean, saveVariance, momentum=0.9, epsilon=1e-5):
+    """nnops.BatchNorm in training mode (op_nn.go:1489-1635): returns the normalised
+    value; the four statistics tensors (resident inputs) are updated in place."""
+    op_inputs = [x, runningMean, runningVariance, saveMean, saveVariance]
+    return x.g.apply(K_BN_TRAIN, op_inputs, f0=epsilon, f1=momentum)
+
+
+def BatchNormDiff(x, grad, saveMean, saveVariance, epsilon=1e-5):
+    """batchnormDiffOp (op_nn.go:1834-1943), training branch."""
+    return x.g.apply(K_BN_DIFF, [x, grad, saveMean, saveVariance], f0=epsilon)
+
+
+def SoftMaxDiff(y, grad):
+    """softmaxDiffOp (op_softmax.go:184-279): y = SoftMax(x), returns the gradient wrt x."""
+    return y.g.apply(K_SOFTMAX_DIFF, [y, grad])
+
+
+def Set(a, b):
+    """gorgonia.Set(a, b): a's value becomes b's; a keeps its register, so a
+    resident input updated this way carries the new value into the next run."""
+    return a.g.apply(K_SET, [a, b])
 
 
 class TapeMachine:

@@ -184,6 +184,7 @@ int ghh_graph_apply(ghh_graph* g, const ghh_op* op, const int* inputs, int n_inp
   s.transB = op->trans_b != 0;
   for (int i = 0; i < op->n_ints && i < 16; i++) s.ints.push_back(op->ints[i]);
   s.f0 = op->f0;
+  s.f1 = op->f1;
   std::vector<int> in(inputs, inputs + n_inputs);
   return ret(g, g->g.Apply(s, in, out));
 }

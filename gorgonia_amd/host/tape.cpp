@@ -144,6 +144,68 @@ Status InferShape(const OpSpec& op, const std::vector<const Shape*>& in, Shape* 
       if (!need(1) || in[0]->IsScalar()) return bad("SoftMax needs a tensor");
       *out = *in[0];
       return Status::OK();
+    case OpKind::MaxPool2DDiff: {
+      if (!need(2)) return bad("MaxPool2DDiff needs input and gradient");
+      OpSpec fwd = op;
+      fwd.kind = OpKind::MaxPool2D;
+      Shape pooled;
+      std::vector<const Shape*> one{in[0]};
+      Status st = InferShape(fwd, one, &pooled);
+      if (!st.ok()) return st;
+      if (!pooled.Eq(*in[1])) return bad("MaxPool2DDiff: gradient shape " + in[1]->String() + ", expected " + pooled.String());
+      *out = *in[0];
+      return Status::OK();
+    }
+    case OpKind::Conv2dDiffData: {
+      if (!need(2) || op.ints.size() != 12) return bad("Conv2dDiffData needs gradient, filter and the image shape");
+      Shape xs{op.ints[8], op.ints[9], op.ints[10], op.ints[11]};
+      OpSpec fwd = op;
+      fwd.kind = OpKind::Conv2d;
+      fwd.ints.resize(8);
+      Shape ys;
+      std::vector<const Shape*> two{&xs, in[1]};
+      Status st = InferShape(fwd, two, &ys);
+      if (!st.ok()) return st;
+      if (!ys.Eq(*in[0])) return bad("Conv2dDiffData: gradient shape " + in[0]->String() + ", expected " + ys.String());
+      *out = xs;
+      return Status::OK();
+    }
+    case OpKind::Conv2dDiffFilter: {
+      if (!need(2) || op.ints.size() != 8) return bad("Conv2dDiffFilter needs image, gradient and the conv parameters");
+      if (in[0]->Dims() != 4 || in[1]->Dims() != 4) return bad("Conv2dDiffFilter: 4-D operands expected");
+      Shape ws{(*in[1])[1], (*in[0])[1], op.ints[0], op.ints[1]};
+      OpSpec fwd = op;
+      fwd.kind = OpKind::Conv2d;
+      Shape ys;
+      std::vector<const Shape*> two{in[0], &ws};
+      Status st = InferShape(fwd, two, &ys);
+      if (!st.ok()) return st;
+      if (!ys.Eq(*in[1])) return bad("Conv2dDiffFilter: gradient shape " + in[1]->String() + ", expected " + ys.String());
+      *out = ws;
+      return Status::OK();
+    }
+    case OpKind::BatchNormTrain:
+    case OpKind::BatchNormDiff: {
+      const size_t want = op.kind == OpKind::BatchNormTrain ? 5 : 4;
+      if (in.size() != want) return bad("BatchNorm training ops need x[, grad] and the statistics tensors");
+      if (in[0]->Dims() != 2 && in[0]->Dims() != 4) return bad("BatchNorm input must be (B, N) or (B, C, H, W)");
+      const int64_t C = (*in[0])[1];
+      const size_t first = op.kind == OpKind::BatchNormTrain ? 1 : 2;
+      if (op.kind == OpKind::BatchNormDiff && !in[1]->Eq(*in[0])) return bad("BatchNormDiff: gradient shape mismatch");
+      for (size_t i = first; i < in.size(); i++)
+        if (in[i]->TotalSize() != C)
+          return bad("invalid runningMean shape " + in[i]->String() + ". Expected: (" + std::to_string(C) + ")");
+      *out = *in[0];
+      return Status::OK();
+    }
+    case OpKind::SoftMaxDiff:
+      if (!need(2) || !in[0]->Eq(*in[1])) return bad("SoftMaxDiff needs output and gradient of one shape");
+      *out = *in[0];
+      return Status::OK();
+    case OpKind::Set:
+      if (!need(2) || in[0]->TotalSize() != in[1]->TotalSize()) return bad("Set: sizes differ");
+      *out = *in[0];
+      return Status::OK();
     case OpKind::Reshape: {
       if (!need(1)) return bad("Reshape needs 1 input");
       Shape s(op.ints);
@@ -183,6 +245,13 @@ static std::string op_name(const OpSpec& op) {
     case OpKind::LeakyRelu: return "leakyrelu";
     case OpKind::SoftMax: return "softmax";
     case OpKind::Reshape: return "reshape";
+    case OpKind::MaxPool2DDiff: return "maxpool2d.diff";
+    case OpKind::Conv2dDiffData: return "conv2d.diff.image";
+    case OpKind::Conv2dDiffFilter: return "conv2d.diff.filter";
+    case OpKind::BatchNormTrain: return "batchnorm(train)";
+    case OpKind::BatchNormDiff: return "batchnorm.diff";
+    case OpKind::SoftMaxDiff: return "softmax.diff";
+    case OpKind::Set: return "set";
   }
   return "?";
 }
@@ -311,6 +380,72 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     }
     case OpKind::Reshape:
       return Status::OK();  // metadata only (op_tensor.go:1226-1246)
+    case OpKind::MaxPool2DDiff: {
+      const Tensor& x = *in[0];
+      const auto& p = op.ints;
+      const int64_t np = p[2];
+      gh_cmd c{};
+      c.opcode = GH_OP_MAXPOOL2D_BWD;
+      c.flags = np == 4 ? GH_FLAG_EXPLICIT_PAD : 0;
+      c.ptr[0] = x.mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
+      for (int i = 0; i < 4; i++) c.dim[i] = x.shape[i];
+      c.dim[4] = p[0]; c.dim[5] = p[1];
+      if (np == 4) { c.dim[6] = p[3]; c.dim[7] = p[4]; c.dim[8] = p[5]; c.dim[9] = p[6]; }
+      else { c.dim[6] = c.dim[7] = p[3]; c.dim[8] = c.dim[9] = p[4]; }
+      c.dim[10] = p[3 + np]; c.dim[11] = p[4 + np];
+      e.Enqueue(c);
+      return Status::OK();
+    }
+    case OpKind::Conv2dDiffData:
+    case OpKind::Conv2dDiffFilter: {
+      const bool data = op.kind == OpKind::Conv2dDiffData;
+      gh_cmd c{};
+      c.opcode = data ? GH_OP_CONV2D_BWD_DATA : GH_OP_CONV2D_BWD_FILTER;
+      c.ptr[0] = in[0]->mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
+      const Shape& xs = data ? prealloc.shape : in[0]->shape;
+      for (int i = 0; i < 4; i++) c.dim[i] = xs[i];
+      c.dim[4] = data ? in[1]->shape[0] : prealloc.shape[0];
+      for (int i = 0; i < 8; i++) c.dim[5 + i] = op.ints[(size_t)i];
+      e.Enqueue(c);
+      return Status::OK();
+    }
+    case OpKind::BatchNormTrain:
+    case OpKind::BatchNormDiff: {
+      const Tensor& x = *in[0];
+      if (x.dt != Dtype::Float32) return bad("BatchNorm: Unsupported Dtype");
+      gh_cmd c{};
+      const int64_t B = x.shape[0], C = x.shape[1];
+      c.dim[0] = B; c.dim[1] = C; c.dim[2] = x.shape.TotalSize() / (B * C);
+      c.f[0] = (float)op.f0;
+      if (op.kind == OpKind::BatchNormTrain) {
+        c.opcode = GH_OP_BN_TRAIN;
+        c.ptr[0] = x.mem; c.ptr[1] = prealloc.mem;
+        for (int i = 0; i < 4; i++) c.ptr[2 + i] = in[(size_t)(1 + i)]->mem;
+        c.f[1] = (float)op.f1;
+      } else {
+        c.opcode = GH_OP_BN_BWD;
+        c.ptr[0] = x.mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
+        c.ptr[3] = in[2]->mem; c.ptr[4] = in[3]->mem;
+      }
+      e.Enqueue(c);
+      return Status::OK();
+    }
+    case OpKind::SoftMaxDiff: {
+      const Tensor& y = *in[0];
+      gh_cmd c{};
+      c.opcode = GH_OP_SOFTMAX_BWD;
+      c.ptr[0] = y.mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
+      const int64_t cols = y.shape[y.shape.Dims() - 1];
+      c.dim[0] = y.shape.TotalSize() / cols; c.dim[1] = cols;
+      e.Enqueue(c);
+      return Status::OK();
+    }
+    case OpKind::Set: {
+      // prealloc is a's register (the node aliases a); copy b's bytes into it
+      const int64_t bytes = in[1]->DataSize() * dtype_size(in[1]->dt);
+      e.RecordCopy(prealloc.mem, in[1]->mem, bytes);
+      return Status::OK();
+    }
   }
   return bad("unknown op");
 }
@@ -338,7 +473,7 @@ Status Graph::Apply(const OpSpec& op, const std::vector<int>& inputs, int* out) 
   n.dt = inputs.empty() ? Dtype::Float32 : nodes_[(size_t)inputs[0]].dt;
   n.op = op;
   n.inputs = inputs;
-  if (op.kind == OpKind::Reshape) n.alias_of = inputs[0];
+  if (op.kind == OpKind::Reshape || op.kind == OpKind::Set) n.alias_of = inputs[0];
   nodes_.push_back(n);
   if (out) *out = n.id;
   return Status::OK();
@@ -470,10 +605,14 @@ Status TapeMachine::Compile() {
 
   for (int i = 0; i < N; i++) {
     Node& n = nodes[(size_t)i];
-    if (n.alias_of >= 0 || n.fused_away) continue;
+    if (n.fused_away) continue;
+    if (n.alias_of >= 0 && n.op.kind != OpKind::Set) continue;  // a view: nothing to run
     const int r = node_reg_[(size_t)i];
     const int64_t bytes = bytes_of(n);
-    if (n.is_input) {
+    if (n.alias_of >= 0) {
+      // Set writes into the register it aliases
+      prog_.push_back({InstrKind::ExecOp, i, r, bytes, true});
+    } else if (n.is_input) {
       prog_.push_back({InstrKind::LoadArg, i, r, bytes, false});
       prog_.push_back({InstrKind::Alloc, i, r, bytes, false});
       prog_.push_back({InstrKind::Transport, i, r, bytes, false});

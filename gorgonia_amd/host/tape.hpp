@@ -39,7 +39,16 @@ enum class OpKind : int32_t {
   Rectify = 10,     // nnops.Rectify
   LeakyRelu = 11,   // gorgonia.LeakyRelu
   SoftMax = 12,     // gorgonia.SoftMax (last axis)
-  Reshape = 13      // gorgonia.Reshape
+  Reshape = 13,     // gorgonia.Reshape
+  // the diff ops the reference's symbolic differentiation inserts, and Set
+  MaxPool2DDiff = 14,    // maxPoolDiffOp (op_nn.go:962-1093): inputs x, grad
+  Conv2dDiffData = 15,   // gradient of Conv2d wrt the image: inputs grad, filter; ints = conv params + image shape
+  Conv2dDiffFilter = 16, // gradient wrt the filter: inputs image, grad; ints = conv params
+  BatchNormTrain = 17,   // BatchNormOp in training mode (op_nn.go:1489-1635): inputs x, runningMean,
+                         // runningVar, saveMean, saveVar; the four statistics tensors are updated in place
+  BatchNormDiff = 18,    // batchnormDiffOp (op_nn.go:1834-1943): inputs x, grad, saveMean, saveVar
+  SoftMaxDiff = 19,      // softmaxDiffOp (op_softmax.go:184-279): inputs y, grad
+  Set = 20               // gorgonia.Set(a, b): a's value becomes b's (operations.go); inputs a, b
 };
 
 struct OpSpec {

@@ -98,6 +98,7 @@ typedef struct ghh_op {
   int32_t n_ints;
   int64_t ints[16];
   double  f0;
+  double  f1;      /* second scalar parameter (BatchNorm momentum) */
 } ghh_op;
 
 GH_API ghh_graph* ghh_graph_new(void);

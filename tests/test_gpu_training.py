@@ -1,0 +1,73 @@
+"""GPU parity of a whole training step: convnet forward, the diff ops of every
+layer, and the in-place SGD update through Set, on the tape machine, against
+the CPU oracle's step on the same seeded inputs (<= 1e-5 relative Frobenius per
+gradient; every kernel on the way has its own tighter test)."""
+import numpy as np
+import pytest
+
+from gorgonia_amd import configs, graph as G
+from oracle import forward as F
+from tests.util import assert_bits_equal, rel_frobenius
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def _onehot(batch):
+    y = np.zeros((batch, 10), np.float32)
+    y[np.arange(batch), (np.arange(batch) * 7 + 3) % 10] = 1.0
+    return y
+
+
+def test_convnet_training_step_gradients(ctx):
+    inp = configs.convnet_inputs(32)
+    y = _onehot(32)
+    g, outs = configs.build_convnet_train(inp, y, 0.05)
+    m = G.NewTapeMachine(g)
+    m.RunAll()
+    out, cost, grads, new = F.convnet_train_step(inp, y, 0.05)
+    assert rel_frobenius(outs["out"], out) <= TOL
+    for i in range(5):
+        err = rel_frobenius(outs[f"dw{i}"], grads[f"w{i}"])
+        assert err <= TOL, f"dw{i}: {err:.3e}"
+    # the weights moved on the device: the second step's forward pass sees them
+    m.RunAll()
+    inp2 = dict(inp, **new)
+    out2, _, grads2, _ = F.convnet_train_step(inp2, y, 0.05)
+    assert rel_frobenius(outs["out"], out2) <= TOL
+    for i in range(5):
+        assert rel_frobenius(outs[f"dw{i}"], grads2[f"w{i}"]) <= 5 * TOL
+    assert not np.array_equal(out, out2)
+    m.Close()
+
+
+def test_training_steps_replayed_from_a_graph(ctx):
+    """Steps 2.. run as hipGraph replays; the in-place weight updates persist
+    between replays and the cost goes down."""
+    inp = configs.convnet_inputs(16)
+    y = _onehot(16)
+    g, outs = configs.build_convnet_train(inp, y, 0.5, read_grads=False)
+    m = G.NewTapeMachine(g, graph_replay=True)
+    cur = dict(inp)
+    costs = []
+    for step in range(5):
+        m.RunAll()
+        want, cost, _, new = F.convnet_train_step(cur, y, 0.5)
+        assert rel_frobenius(outs["out"], want) <= 2 * TOL * (step + 1), f"step {step}"
+        costs.append(-float((outs["out"] * y).mean()))
+        cur = dict(cur, **new)
+    assert m.graph_launches() >= 3
+    assert costs[-1] < costs[0]
+    m.Close()
+
+
+def test_set_updates_a_resident_input_in_place(ctx):
+    g = G.NewGraph()
+    a = G.NewTensor(g, np.arange(8, dtype=np.float32), resident=True)
+    one = G.NewScalar(g, 1.0)
+    out = G.Read(G.Set(a, G.Add(a, one)))
+    m = G.NewTapeMachine(g)
+    for k in range(1, 4):
+        m.RunAll()
+        assert_bits_equal(out, np.arange(8, dtype=np.float32) + k, f"after {k} runs")
+    m.Close()
