@@ -203,6 +203,65 @@ def bench_yolo(steps, warmup):
     return dt / steps * 1e3, result, inp
 
 
+def bench_convnet_train(steps, warmup, batch=128):
+    """Config 4 as a training step: forward, every layer's gradient, SGD update
+    of the resident weights; only the 128x10 output leaves the device."""
+    from gorgonia_amd import configs, graph as G
+    inp = configs.convnet_inputs(batch)
+    onehot = np.zeros((batch, 10), np.float32)
+    onehot[np.arange(batch), np.arange(batch) % 10] = 1.0
+    g, outs = configs.build_convnet_train(inp, onehot, 0.01, read_grads=False)
+    m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING)
+    for _ in range(max(warmup, 3)):
+        m.RunAll()
+    eng = m.engine()
+    eng.DoWork()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        m.RunAll()
+    eng.DoWork()
+    dt = time.perf_counter() - t0
+    m.Close()
+    return dt / steps * 1e3, inp, onehot
+
+
+def bench_backward_kernels(ctx, iters):
+    """Per-kernel time of the backward passes at the convnet's and the
+    yolo-shaped stack's layer shapes."""
+    from gorgonia_amd import device as D, synth
+    out = {}
+    for name, (B, C, HW, F) in {"convnet_conv1": (128, 32, 14, 64), "convnet_conv2": (128, 64, 7, 128),
+                                "yolo_conv3": (8, 64, 52, 128), "yolo_conv6": (8, 512, 13, 1024)}.items():
+        x = ctx.upload(synth.uniform01(1, (B * C * HW * HW,)))
+        w = ctx.upload(synth.normal(2, (F * C * 9,)))
+        dy = ctx.upload(synth.normal(3, (B * F * HW * HW,)))
+        dx, dw = ctx.malloc(B * C * HW * HW * 4), ctx.malloc(F * C * 9 * 4)
+        fl = 2.0 * B * HW * HW * F * C * 9
+        ms = time_cmds(ctx, [D.cmd_conv2d_bwd_filter(x, dy, dw, B, C, HW, HW, F, 3, 3, (1, 1))], iters)
+        out[name + "_filter_grad"] = {"us": round(ms * 1e3, 2), "TFLOPs": round(fl / ms / 1e9, 2)}
+        ms = time_cmds(ctx, [D.cmd_conv2d_bwd_data(dy, w, dx, B, C, HW, HW, F, 3, 3, (1, 1))], iters)
+        out[name + "_image_grad"] = {"us": round(ms * 1e3, 2), "TFLOPs": round(fl / ms / 1e9, 2)}
+        for q in (x, w, dy, dx, dw):
+            ctx.free(q)
+    B, C, HW = 8, 32, 208
+    n = B * C * HW * HW
+    x, dy = ctx.upload(synth.normal(4, (n,))), ctx.upload(synth.normal(5, (n // 4,)))
+    dx = ctx.malloc(n * 4)
+    ms = time_cmds(ctx, [D.cmd_maxpool2d_bwd(x, dy, dx, B, C, HW, HW, 2, 2, (0, 0), (2, 2))], iters)
+    out["maxpool_bwd_8x32x208x208"] = {"us": round(ms * 1e3, 2), "GBps": round(4 * (2 * n + n // 4) / ms / 1e6, 1)}
+    g = ctx.upload(synth.normal(6, (n,)))
+    st = [ctx.upload(np.zeros(C, np.float32)) for _ in range(4)]
+    ms = time_cmds(ctx, [D.cmd_bn_train(x, dx, st[0], st[1], st[2], st[3], B, C, HW * HW, 1e-5, 0.9)], iters)
+    out["bn_train_8x32x208x208"] = {"us": round(ms * 1e3, 2), "GBps": round(4 * 4 * n / ms / 1e6, 1),
+                                    "bytes": "3 reads + 1 write of x"}
+    ms = time_cmds(ctx, [D.cmd_bn_bwd(x, g, dx, st[2], st[3], B, C, HW * HW, 1e-5)], iters)
+    out["bn_bwd_8x32x208x208"] = {"us": round(ms * 1e3, 2), "GBps": round(4 * 5 * n / ms / 1e6, 1),
+                                  "bytes": "2 reads of x and dy + 1 write"}
+    for q in [x, dy, dx, g] + st:
+        ctx.free(q)
+    return out
+
+
 def cpu_baseline_convnet(inp, budget_s=12.0):
     """The CPU oracle's forward pass of the same configuration on the host cores."""
     from oracle import binding as O, forward as F
@@ -256,7 +315,7 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager-timing", action="store_true",
                     help="launch every kernel eagerly, no hipGraph (use under rocprofv3 --pmc)")
-    ap.add_argument("--only", default="", help="comma list of: convnet,elementwise,linalg,yolo")
+    ap.add_argument("--only", default="", help="comma list of: convnet,elementwise,linalg,yolo,train")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this engine runs on one GPU; --gpus must be 1 (no multi-GPU path is built)")
@@ -282,10 +341,17 @@ def main():
                 "TFLOPs": round(31_080_857_600 / ms_yolo / 1e9, 2), "flop_per_step": 31_080_857_600}
         log(f"yolo-shaped: {ms_yolo:.4f} ms/step  {8 / ms_yolo * 1e3:.0f} images/s")
 
+    train = None
+    if not only or "train" in only:
+        ms_train, train_inp, train_y = bench_convnet_train(max(20, a.steps // 4), a.warmup)
+        train = {"ms_per_step": round(ms_train, 4), "images_s": round(128 / ms_train * 1e3, 1)}
+        log(f"convnet training step: {ms_train:.4f} ms/step  {128 / ms_train * 1e3:.0f} images/s")
+
     iters = 30
     conv_k = bench_convnet_kernels(ctx, 128, iters) if not only or "convnet" in only else {}
     elem = bench_elementwise(ctx, iters) if not only or "elementwise" in only else {}
     lin = bench_linalg(ctx, iters) if not only or "linalg" in only else {}
+    bwd = bench_backward_kernels(ctx, iters) if not only or "train" in only else {}
     ctx.close()
 
     # the dominant kernel of the step: the conv layer with the largest time
@@ -309,6 +375,18 @@ def main():
         cpu = {"value": round(cpu_images_s, 1), "unit": "images/s", "cores": threads, "kind": "port",
                "sample": f"{reps} forward passes of the same 128-image batch (CPU oracle, OpenMP)"}
         cpu.update(cpu_baseline_micro())
+        if train is not None:
+            from oracle import binding as O, forward as F
+            O.set_threads(threads)
+            t0 = time.perf_counter()
+            reps_t = 0
+            while reps_t < 20 and time.perf_counter() - t0 < 6.0:
+                F.convnet_train_step(train_inp, train_y, 0.01)
+                reps_t += 1
+            tdt = time.perf_counter() - t0
+            O.set_threads(1)
+            cpu["convnet_train_images_s"] = round(128 * reps_t / tdt, 1)
+            cpu["convnet_train_sample"] = f"{reps_t} training steps of the same 128-image batch, {threads} threads"
         if yolo is not None:
             from oracle import binding as O, forward as F
             O.set_threads(threads)
@@ -341,7 +419,7 @@ def main():
             "convnet_ms_per_step_with_input_h2d": round(ms_h2d, 5),
             "convnet_images_s_with_input_h2d": round(128 / ms_h2d * 1e3, 1),
             "convnet_ms_per_step_eager_no_graph": round(ms_eager, 5),
-            "yolo_shaped_forward": yolo, "convnet_kernels": conv_k, "elementwise": elem, "linalg": lin, "parity": parity,
+            "yolo_shaped_forward": yolo, "convnet_training_step": train, "backward_kernels": bwd, "convnet_kernels": conv_k, "elementwise": elem, "linalg": lin, "parity": parity,
         },
     }
     print(json.dumps(line), flush=True)

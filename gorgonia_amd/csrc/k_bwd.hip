@@ -61,6 +61,47 @@ __global__ __launch_bounds__(kBlock) void k_maxpool2d_bwd(const float* __restric
   }
 }
 
+// 2x2 / stride 2 / no padding with even H and W % 4 == 0: windows do not
+// overlap, so one thread owns two adjacent windows - two float4 row loads, one
+// float2 of dy, two float4 stores - with the generic kernel's scan order
+// (r0c0, r0c1, r1c0, r1c1), strict >, and its "0 + dy" for the winner.
+__global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2_bwd(const float* __restrict__ x,
+                                                              const float* __restrict__ dy,
+                                                              float* __restrict__ dx, int H, int W,
+                                                              int64_t pairs) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  const int oh = H / 2, ow = W / 2, owp = ow / 2;
+  for (int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x; idx < pairs; idx += stride) {
+    const int64_t row = idx / owp;  // (bc, ph) flattened
+    const int pp = (int)(idx - row * owp);
+    const int64_t bc = row / oh;
+    const int ph = (int)(row - bc * oh);
+    const int64_t at = (bc * H + 2 * ph) * (int64_t)W + 4 * pp;
+    const f4 r0 = *reinterpret_cast<const f4*>(x + at);
+    const f4 r1 = *reinterpret_cast<const f4*>(x + at + W);
+    const f2 g = *reinterpret_cast<const f2*>(dy + (bc * oh + ph) * (int64_t)ow + 2 * pp);
+    f4 o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+      float best = -FLT_MAX;
+      int arg = -1;
+      if (r0[2 * e] > best) { best = r0[2 * e]; arg = 0; }
+      if (r0[2 * e + 1] > best) { best = r0[2 * e + 1]; arg = 1; }
+      if (r1[2 * e] > best) { best = r1[2 * e]; arg = 2; }
+      if (r1[2 * e + 1] > best) { best = r1[2 * e + 1]; arg = 3; }
+      const float v = 0.0f + g[e];
+      o0[2 * e] = arg == 0 ? v : 0.0f;
+      o0[2 * e + 1] = arg == 1 ? v : 0.0f;
+      o1[2 * e] = arg == 2 ? v : 0.0f;
+      o1[2 * e + 1] = arg == 3 ? v : 0.0f;
+    }
+    *reinterpret_cast<f4*>(dx + at) = o0;
+    *reinterpret_cast<f4*>(dx + at + W) = o1;
+  }
+}
+
 // ---- BatchNorm: per-channel reductions ----------------------------------------------
 // A channel's n = B*S values are split over G workgroups; each reduces its share
 // with a fixed tree (so results repeat run to run), the consumers add the G
@@ -95,13 +136,32 @@ __global__ __launch_bounds__(kBlock) void k_bn_reduce(const float* __restrict__ 
   float mean = 0.0f;
   if (MODE == 1) mean = sum_partials(part_sum + (int64_t)c * G, G) / (float)n;
   float acc = 0.0f;
-  for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n; e += (int64_t)G * kBlock) {
-    const int64_t b = e / S, d = e - b * S;
-    const float v = x[(b * C + c) * S + d];
-    if (MODE == 0) acc = acc + v;
-    else {
-      const float t = v - mean;
-      acc = acc + t * t;
+  const int64_t B = n / S;
+  // workgroup g takes every G-th 256-wide strip of each image's plane; planes
+  // narrower than a strip (dense layers: S == 1) are walked over the batch instead
+  if (S >= kBlock) {
+    for (int64_t b = 0; b < B; b++) {
+      const float* p = x + (b * C + c) * S;
+      for (int64_t d = (int64_t)blockIdx.x * kBlock + threadIdx.x; d < S; d += (int64_t)G * kBlock) {
+        const float v = p[d];
+        if (MODE == 0) acc = acc + v;
+        else {
+          const float t = v - mean;
+          acc = acc + t * t;
+        }
+      }
+    }
+  } else {
+    for (int64_t b = (int64_t)blockIdx.x * kBlock + threadIdx.x; b < B; b += (int64_t)G * kBlock) {
+      const float* p = x + (b * C + c) * S;
+      for (int64_t d = 0; d < S; d++) {
+        const float v = p[d];
+        if (MODE == 0) acc = acc + v;
+        else {
+          const float t = v - mean;
+          acc = acc + t * t;
+        }
+      }
     }
   }
   const float r = block_sum(acc, sh);
@@ -146,9 +206,8 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_reduce(const float* __restric
   const int c = blockIdx.y, G = gridDim.x;
   const float mean = save_mean[c];
   float s = 0.0f, dot = 0.0f;
-  for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n; e += (int64_t)G * kBlock) {
-    const int64_t b = e / S, d = e - b * S;
-    const int64_t i = (b * C + c) * S + d;
+  const int64_t B = n / S;
+  auto term = [&](int64_t i) {
     const float xv = x[i], g = dy[i];
     s = s + g;
     float p;
@@ -160,6 +219,14 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_reduce(const float* __restric
       p = t1 - t2;
     }
     dot = dot + p;
+  };
+  if (S >= kBlock) {
+    for (int64_t b = 0; b < B; b++)
+      for (int64_t d = (int64_t)blockIdx.x * kBlock + threadIdx.x; d < S; d += (int64_t)G * kBlock)
+        term((b * C + c) * S + d);
+  } else {
+    for (int64_t b = (int64_t)blockIdx.x * kBlock + threadIdx.x; b < B; b += (int64_t)G * kBlock)
+      for (int64_t d = 0; d < S; d++) term((b * C + c) * S + d);
   }
   const float rs = block_sum(s, sh);
   const float rd = block_sum(dot, sh);
@@ -237,8 +304,9 @@ __global__ __launch_bounds__(kBlock) void k_softmax_bwd(const float* __restrict_
 }
 
 // how many workgroups share one channel's reduction
-int bn_groups(int64_t n) {
-  int64_t g = n / 4096;
+int bn_groups(int64_t n, int64_t S) {
+  // strips of a plane when planes are wide, slices of the batch otherwise
+  int64_t g = (S >= kBlock ? S : n / S) / 1024;
   if (g < 1) g = 1;
   if (g > 64) g = 64;
   return (int)g;
@@ -259,6 +327,16 @@ int gh_launch_maxpool2d_bwd(gh_ctx* ctx, const gh_cmd& c) {
   g.padW = (int)(explicit_pad ? padE : padW);
   const int64_t total = B * C * g.H * g.W;
   if (total == 0) return GH_OK;
+  if (g.kh == 2 && g.kw == 2 && g.strideH == 2 && g.strideW == 2 && g.padH == 0 && g.padW == 0 &&
+      g.H % 2 == 0 && g.W % 4 == 0 && ((c.ptr[0] | c.ptr[2]) & 15) == 0 && (c.ptr[1] & 7) == 0) {
+    const int64_t pairs = total / 8;
+    int64_t blocks = (pairs + kBlock - 1) / kBlock;
+    if (blocks > (int64_t)ctx->cu_count * 64) blocks = (int64_t)ctx->cu_count * 64;
+    hipLaunchKernelGGL(k_maxpool_2x2s2_bwd, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
+                       (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                       (float*)(uintptr_t)c.ptr[2], g.H, g.W, pairs);
+    return gh_check_hip(ctx, hipGetLastError(), "maxpool backward launch");
+  }
   int64_t blocks = (total + kBlock - 1) / kBlock;
   if (blocks > (int64_t)ctx->cu_count * 64) blocks = (int64_t)ctx->cu_count * 64;
   hipLaunchKernelGGL(k_maxpool2d_bwd, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
@@ -269,7 +347,7 @@ int gh_launch_maxpool2d_bwd(gh_ctx* ctx, const gh_cmd& c) {
 
 int gh_launch_bn_train(gh_ctx* ctx, const gh_cmd& c) {
   const int64_t B = c.dim[0], C = c.dim[1], S = c.dim[2], n = B * S;
-  const int G = bn_groups(n);
+  const int G = bn_groups(n, S);
   // scratch: [C][G] sums, [C][G] squared deviations, [C] batch variance
   const int64_t need = (2 * C * G + C) * 4;
   if (need > ctx->workspace_bytes) return gh_fail(ctx, GH_ESTATE, "batchnorm: reduction scratch does not fit the workspace");
@@ -297,7 +375,7 @@ int gh_launch_bn_train(gh_ctx* ctx, const gh_cmd& c) {
 
 int gh_launch_bn_bwd(gh_ctx* ctx, const gh_cmd& c) {
   const int64_t B = c.dim[0], C = c.dim[1], S = c.dim[2], n = B * S;
-  const int G = bn_groups(n);
+  const int G = bn_groups(n, S);
   if (2 * C * G * 4 > ctx->workspace_bytes) return gh_fail(ctx, GH_ESTATE, "batchnorm: reduction scratch does not fit the workspace");
   float* part = (float*)ctx->workspace;
   const float* x = (const float*)(uintptr_t)c.ptr[0];

@@ -1389,7 +1389,7 @@ int gh_launch_conv2d_bwd_data(gh_ctx* ctx, const gh_cmd& c) {
   float* dx = (float*)(uintptr_t)c.ptr[2];
   const int64_t wbytes = ((int64_t)F * g.C * g.kh * g.kw * 4 + 255) / 256 * 256;
   const int padH = g.dilH * (g.kh - 1) - g.padH, padW = g.dilW * (g.kw - 1) - g.padW;
-  if (g.strideH == 1 && g.strideW == 1 && padH >= 0 && padW >= 0 && wbytes <= ctx->workspace_bytes / 4) {
+  if (g.strideH == 1 && g.strideW == 1 && padH >= 0 && padW >= 0 && wbytes <= ctx->workspace_bytes / 2) {
     // mirrored filters live at the top of the workspace; the forward launch
     // below may use what is left of it for its own split-K slabs
     float* wt = (float*)((char*)ctx->workspace + ctx->workspace_bytes - wbytes);
