@@ -428,6 +428,26 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(const float* __restrict__
   }
 }
 
+// Many slabs, few results (filter gradients): four lanes share one result.
+// Lane q adds slabs q, q+4, q+8, ... in that order, then the four sums are
+// combined as (s0 + s1) + (s2 + s3): a fixed order, so results repeat.
+template <class SC>
+__global__ __launch_bounds__(256) void k_splitk_reduce4(const float* __restrict__ ws, int splits, int M,
+                                                        int N, SC sc, int act, float alpha) {
+  const int64_t total = (int64_t)M * N;
+  const int q = threadIdx.x & 3;
+  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 2;
+  float acc = 0.f;
+  if (e < total)
+    for (int s = q; s < splits; s += 4) acc = acc + ws[(int64_t)s * total + e];
+  const float pair = acc + __shfl_xor(acc, 1, 64);      // lanes 0,1 -> s0+s1 ; lanes 2,3 -> s2+s3 (commutative)
+  const float sum = pair + __shfl_xor(pair, 2, 64);
+  if (e < total && q == 0) {
+    const int i = (int)(e / N), j = (int)(e - (int64_t)i * N);
+    sc.put(i, j, act_apply(sum, act, alpha));
+  }
+}
+
 // ---- small-output GEMM: the K range is split across the wavefronts of one block ------
 // C(M x N) = A(M x K) B(K x N), both row-major, for products whose output has
 // too few 32x32 tiles to fill the chip when each tile walks all of K.  One
@@ -799,26 +819,34 @@ __global__ __launch_bounds__(256) void k_conv3x3_direct(const float* __restrict_
 // dy[b][f][oy][ox] * x[b][c][oy*s - p + kr*d][ox*s - p + kc*d]: M = F, N = C*kh*kw,
 // K = B*oh*ow, split over K.
 
-// A operand: row f, k = pixel index across the batch, from NCHW dy.
+// A operand: row f, k = pixel index across the batch, from NCHW dy.  The tile
+// loop asks for consecutive k-tiles, so after the first call the (image, pixel)
+// position is advanced by carries instead of being divided out again.
 template <int R, int BK>
 struct LoadDyRows {
   static constexpr int S = R + 2;
   static constexpr int RSTEP = kThreads / BK;   // row distance between a thread's elements
   static constexpr int RPT = R / RSTEP;
   const float* dy; int F; int plane; int kmax /* B*plane */;
+  int next_k = -1, b = 0, p = 0;
   float reg[RPT];
   __device__ __forceinline__ void load(int r0, int k0) {
     const int kk = threadIdx.x % BK, rb = threadIdx.x / BK;
     const int j = k0 + kk;
+    if (k0 != next_k) {
+      b = j / plane;
+      p = j - b * plane;
+    }
+    next_k = k0 + BK;
     const bool ok = j < kmax;
-    const int b = ok ? j / plane : 0;
-    const int p = ok ? j - b * plane : 0;
     const float* base = dy + (int64_t)b * F * plane + p;
 #pragma unroll
     for (int i = 0; i < RPT; i++) {
       const int f = r0 + rb + i * RSTEP;
       reg[i] = (ok && f < F) ? base[(int64_t)f * plane] : 0.f;
     }
+    p += BK;
+    while (p >= plane) { p -= plane; b++; }
   }
   __device__ __forceinline__ void store(float* lds) const {
     const int kk = threadIdx.x % BK, rb = threadIdx.x / BK;
@@ -828,7 +856,8 @@ struct LoadDyRows {
 };
 
 // B operand: column n = (c, kr, kc), k = pixel index: the im2col gather read the
-// other way round.  What depends only on the column is computed once.
+// other way round.  What depends only on the column is computed once; the
+// pixel position (image, oy, ox) is carried from tile to tile.
 template <int R, int BK>
 struct LoadIm2colT {
   static constexpr int S = R + 2;
@@ -837,6 +866,7 @@ struct LoadIm2colT {
   const float* x; ConvGeom g; int nmax /* C*kh*kw */; int kmax /* B*oh*ow */;
   int coff[RPT];   // c*H*W + kr*dilH*W + kc*dilW, or -1 for a column past the end
   int dyo[RPT], dxo[RPT];
+  int next_k = -1, b = 0, oy = 0, ox = 0;
   float reg[RPT];
   __device__ __forceinline__ void init(int n0) {
     const int rb = threadIdx.x / BK;
@@ -844,24 +874,26 @@ struct LoadIm2colT {
 #pragma unroll
     for (int i = 0; i < RPT; i++) {
       const int n = n0 + rb + i * RSTEP;
-      if (n < nmax) {
-        const int c = n / kk, r = n - c * kk;
-        const int kr = r / g.kw, kc = r - kr * g.kw;
-        dyo[i] = kr * g.dilH;
-        dxo[i] = kc * g.dilW;
-        coff[i] = c * g.H * g.W + dyo[i] * g.W + dxo[i];
-      } else {
-        coff[i] = -1; dyo[i] = 0; dxo[i] = 0;
-      }
+      const bool okn = n < nmax;
+      const int nn = okn ? n : 0;
+      const int c = nn / kk, r = nn - c * kk;
+      const int kr = r / g.kw, kc = r - kr * g.kw;
+      dyo[i] = kr * g.dilH;
+      dxo[i] = kc * g.dilW;
+      coff[i] = okn ? c * g.H * g.W + dyo[i] * g.W + dxo[i] : -1;
     }
   }
   __device__ __forceinline__ void load(int /*n0*/, int k0) {
     const int j = k0 + threadIdx.x % BK;
+    if (k0 != next_k) {
+      const int plane = g.oh * g.ow;
+      b = j / plane;
+      const int rem = j - b * plane;
+      oy = rem / g.ow;
+      ox = rem - oy * g.ow;
+    }
+    next_k = k0 + BK;
     const bool ok = j < kmax;
-    const int plane = g.oh * g.ow;
-    const int b = ok ? j / plane : 0;
-    const int rem = ok ? j - b * plane : 0;
-    const int oy = rem / g.ow, ox = rem - oy * g.ow;
     const int iy0 = oy * g.strideH - g.padH, ix0 = ox * g.strideW - g.padW;
     const float* xb = x + (int64_t)b * g.C * g.H * g.W + iy0 * g.W + ix0;
 #pragma unroll
@@ -870,6 +902,9 @@ struct LoadIm2colT {
       const bool in = ok && coff[i] >= 0 && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
       reg[i] = in ? xb[coff[i]] : 0.f;
     }
+    ox += BK;
+    while (ox >= g.ow) { ox -= g.ow; oy++; }
+    while (oy >= g.oh) { oy -= g.oh; b++; }
   }
   __device__ __forceinline__ void store(float* lds) const {
     const int kk = threadIdx.x % BK, rb = threadIdx.x / BK;
@@ -900,6 +935,58 @@ __global__ __launch_bounds__(kThreads) void k_conv2d_wgrad(const float* __restri
   } else {
     StoreRowMajor sc{dw, CKK};
     mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreRowMajor>(lds, la, lb, sc, F, CKK, 0, nk, m0, n0, 0, 0.f);
+  }
+}
+
+// Filter gradient for the direct kernel's shapes (3x3, stride 1, at most four
+// input channels): only F*C*9 results, each a sum over all output pixels, so
+// this is a reduction on the vector ALUs.  Workgroup (g, f) walks every G-th
+// image: a thread adds dy * x-patch into its C*9 accumulators, the workgroup
+// folds them with a fixed tree, and slab g of the [G][F][C*9] workspace gets the
+// partial; the split-K reduce kernel adds the slabs in order.
+template <int C>
+__global__ __launch_bounds__(256) void k_conv3x3_wgrad_direct(const float* __restrict__ x,
+                                                              const float* __restrict__ dy,
+                                                              float* __restrict__ ws, int B, int H,
+                                                              int W, int F, int pad, int oh, int ow) {
+  constexpr int Q = C * 9;
+  __shared__ float sh[4][Q];
+  const int f = blockIdx.y, G = gridDim.x;
+  const int plane = oh * ow;
+  float acc[Q];
+#pragma unroll
+  for (int q = 0; q < Q; q++) acc[q] = 0.f;
+  for (int b = blockIdx.x; b < B; b += G) {
+    const float* gy = dy + ((int64_t)b * F + f) * plane;
+    const float* xb = x + (int64_t)b * C * H * W;
+    for (int p = threadIdx.x; p < plane; p += 256) {
+      const int oy = p / ow, ox = p - oy * ow;
+      const float g = gy[p];
+#pragma unroll
+      for (int c = 0; c < C; c++)
+#pragma unroll
+        for (int kr = 0; kr < 3; kr++)
+#pragma unroll
+          for (int kc = 0; kc < 3; kc++) {
+            const int iy = oy - pad + kr, ix = ox - pad + kc;
+            const bool in = iy >= 0 && iy < H && ix >= 0 && ix < W;
+            const float xv = in ? xb[(c * H + iy) * W + ix] : 0.f;
+            acc[(c * 3 + kr) * 3 + kc] = __builtin_fmaf(g, xv, acc[(c * 3 + kr) * 3 + kc]);
+          }
+    }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int q = 0; q < Q; q++) {
+    float v = acc[q];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    if (lane == 0) sh[wave][q] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x < Q) {
+    const int q = threadIdx.x;
+    ws[((int64_t)blockIdx.x * F + f) * Q + q] = (sh[0][q] + sh[1][q]) + (sh[2][q] + sh[3][q]);
   }
 }
 
@@ -1355,7 +1442,31 @@ static ConvGeom conv_geom(const gh_cmd& c) {
 int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
   const ConvGeom g = conv_geom(c);
   const int F = (int)c.dim[4], CKK = g.C * g.kh * g.kw;
-  constexpr int BM = 64, BN = 64, BK = 16;
+  if (conv_direct_shape(c) && F <= 65535) {
+    const int B = (int)c.dim[0];
+    int G = B < 64 ? B : 64;
+    while (G > 1 && (int64_t)G * F * CKK * 4 > ctx->workspace_bytes) G--;
+    float* wsd = (float*)ctx->workspace;
+    const float* xd = (const float*)(uintptr_t)c.ptr[0];
+    const float* dyd = (const float*)(uintptr_t)c.ptr[1];
+    const dim3 grid((unsigned)G, (unsigned)F);
+#define GH_WGRAD_DIRECT(C_)                                                                          \
+  hipLaunchKernelGGL((k_conv3x3_wgrad_direct<C_>), grid, dim3(256), 0, ctx->stream, xd, dyd, wsd, B, g.H, \
+                     g.W, F, g.padH, g.oh, g.ow)
+    switch (g.C) {
+      case 1: GH_WGRAD_DIRECT(1); break;
+      case 2: GH_WGRAD_DIRECT(2); break;
+      case 3: GH_WGRAD_DIRECT(3); break;
+      default: GH_WGRAD_DIRECT(4); break;
+    }
+#undef GH_WGRAD_DIRECT
+    int rc = gh_check_hip(ctx, hipGetLastError(), "direct filter-gradient launch");
+    if (rc) return rc;
+    hipLaunchKernelGGL((k_splitk_reduce4<StoreRowMajor>), dim3((int)cdiv((int64_t)F * CKK * 4, 256)), dim3(256),
+                       0, ctx->stream, wsd, G, F, CKK, StoreRowMajor{(float*)(uintptr_t)c.ptr[2], CKK}, 0, 0.f);
+    return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
+  }
+  constexpr int BM = 64, BN = 64, BK = 32;
   const int64_t tiles = cdiv(F, BM) * cdiv(CKK, BN);
   const int64_t nk = cdiv(g.P, BK);
   int64_t splits = cdiv(5 * (int64_t)ctx->cu_count / 2, tiles);   // ~2.5 workgroups per CU
@@ -1373,10 +1484,15 @@ int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
                      CKK, (int)splits, ws);
   int rc = gh_check_hip(ctx, hipGetLastError(), "conv filter-gradient launch");
   if (rc || splits <= 1) return rc;
-  int64_t blocks = cdiv((int64_t)F * CKK, 256);
-  if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
-  hipLaunchKernelGGL((k_splitk_reduce<StoreRowMajor>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws,
-                     (int)splits, F, CKK, StoreRowMajor{dw, CKK}, 0, 0.f);
+  if (splits >= 8) {
+    hipLaunchKernelGGL((k_splitk_reduce4<StoreRowMajor>), dim3((int)cdiv((int64_t)F * CKK * 4, 256)), dim3(256),
+                       0, ctx->stream, ws, (int)splits, F, CKK, StoreRowMajor{dw, CKK}, 0, 0.f);
+  } else {
+    int64_t blocks = cdiv((int64_t)F * CKK, 256);
+    if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
+    hipLaunchKernelGGL((k_splitk_reduce<StoreRowMajor>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws,
+                       (int)splits, F, CKK, StoreRowMajor{dw, CKK}, 0, 0.f);
+  }
   return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
 }
 
