@@ -137,31 +137,34 @@ __global__ __launch_bounds__(kBlock) void k_bn_reduce(const float* __restrict__ 
   if (MODE == 1) mean = sum_partials(part_sum + (int64_t)c * G, G) / (float)n;
   float acc = 0.0f;
   const int64_t B = n / S;
-  // workgroup g takes every G-th 256-wide strip of each image's plane; planes
-  // narrower than a strip (dense layers: S == 1) are walked over the batch instead
+  auto term = [&](float v) {
+    if (MODE == 0) return v;
+    const float t = v - mean;
+    return t * t;
+  };
+  // A plane is cut into 256-wide strips; workgroup g takes strips g, g + G, ...
+  // of every image.  Planes narrower than a strip (dense layers: S == 1) are
+  // walked over the batch instead.
   if (S >= kBlock) {
-    for (int64_t b = 0; b < B; b++) {
-      const float* p = x + (b * C + c) * S;
-      for (int64_t d = (int64_t)blockIdx.x * kBlock + threadIdx.x; d < S; d += (int64_t)G * kBlock) {
-        const float v = p[d];
-        if (MODE == 0) acc = acc + v;
-        else {
-          const float t = v - mean;
-          acc = acc + t * t;
-        }
+    float a4[4] = {0.f, 0.f, 0.f, 0.f};
+    const int64_t img = (int64_t)C * S;
+    for (int64_t d = (int64_t)blockIdx.x * kBlock + threadIdx.x; d < S; d += (int64_t)G * kBlock) {
+      const float* p = x + (int64_t)c * S + d;
+      int64_t b = 0;
+      for (; b + 4 <= B; b += 4) {   // four images at a time: four loads in flight
+        const float v0 = p[b * img], v1 = p[(b + 1) * img], v2 = p[(b + 2) * img], v3 = p[(b + 3) * img];
+        a4[0] = a4[0] + term(v0);
+        a4[1] = a4[1] + term(v1);
+        a4[2] = a4[2] + term(v2);
+        a4[3] = a4[3] + term(v3);
       }
+      for (; b < B; b++) a4[0] = a4[0] + term(p[b * img]);
     }
+    acc = (a4[0] + a4[1]) + (a4[2] + a4[3]);
   } else {
     for (int64_t b = (int64_t)blockIdx.x * kBlock + threadIdx.x; b < B; b += (int64_t)G * kBlock) {
       const float* p = x + (b * C + c) * S;
-      for (int64_t d = 0; d < S; d++) {
-        const float v = p[d];
-        if (MODE == 0) acc = acc + v;
-        else {
-          const float t = v - mean;
-          acc = acc + t * t;
-        }
-      }
+      for (int64_t d = 0; d < S; d++) acc = acc + term(p[d]);
     }
   }
   const float r = block_sum(acc, sh);
@@ -207,6 +210,18 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_reduce(const float* __restric
   const float mean = save_mean[c];
   float s = 0.0f, dot = 0.0f;
   const int64_t B = n / S;
+  auto term2 = [&](float xv, float g) {
+    s = s + g;
+    float p;
+    if (S == 1) {
+      const float t = xv - mean;
+      p = t * g;
+    } else {
+      const float t1 = xv * g, t2 = mean * g;
+      p = t1 - t2;
+    }
+    dot = dot + p;
+  };
   auto term = [&](int64_t i) {
     const float xv = x[i], g = dy[i];
     s = s + g;
@@ -221,9 +236,18 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_reduce(const float* __restric
     dot = dot + p;
   };
   if (S >= kBlock) {
-    for (int64_t b = 0; b < B; b++)
-      for (int64_t d = (int64_t)blockIdx.x * kBlock + threadIdx.x; d < S; d += (int64_t)G * kBlock)
-        term((b * C + c) * S + d);
+    const int64_t img = (int64_t)C * S;
+    for (int64_t d = (int64_t)blockIdx.x * kBlock + threadIdx.x; d < S; d += (int64_t)G * kBlock) {
+      const int64_t at = (int64_t)c * S + d;
+      int64_t b = 0;
+      for (; b + 2 <= B; b += 2) {
+        const float x0 = x[at + b * img], g0 = dy[at + b * img];
+        const float x1 = x[at + (b + 1) * img], g1 = dy[at + (b + 1) * img];
+        term2(x0, g0);
+        term2(x1, g1);
+      }
+      for (; b < B; b++) term2(x[at + b * img], dy[at + b * img]);
+    }
   } else {
     for (int64_t b = (int64_t)blockIdx.x * kBlock + threadIdx.x; b < B; b += (int64_t)G * kBlock)
       for (int64_t d = 0; d < S; d++) term((b * C + c) * S + d);
@@ -245,7 +269,7 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const float* __restrict
                                                          const float* __restrict__ save_var,
                                                          const float* __restrict__ part, float eps,
                                                          int training, int64_t BC, int C, int64_t S,
-                                                         int G, int64_t n) {
+                                                         int G, int64_t n, int vec) {
   for (int64_t bc = blockIdx.y; bc < BC; bc += gridDim.y) {
     const int c = (int)(bc % C);
     float s = 0.0f, dot = 0.0f;
@@ -263,17 +287,27 @@ __global__ __launch_bounds__(kBlock) void k_bn_bwd_apply(const float* __restrict
     const float* xi = x + bc * S;
     const float* gi = dy + bc * S;
     float* out = dx + bc * S;
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < S; i += (int64_t)gridDim.x * kBlock) {
-      if (training) {
-        float t = xi[i] - mean;
-        t = t * k;
-        float u;
-        if (S == 1) { u = gi[i] - t; u = u - grad_mean; }
-        else { u = gi[i] - grad_mean; u = u - t; }
-        out[i] = u * invstd;
-      } else {
-        out[i] = gi[i] * invstd;
+    auto one = [&](float xv, float g) {
+      if (!training) return g * invstd;
+      float t = xv - mean;
+      t = t * k;
+      float u;
+      if (S == 1) { u = g - t; u = u - grad_mean; }
+      else { u = g - grad_mean; u = u - t; }
+      return u * invstd;
+    };
+    if (vec) {
+      typedef float f4 __attribute__((ext_vector_type(4)));
+      for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < S / 4; i += (int64_t)gridDim.x * kBlock) {
+        const f4 xv = *(reinterpret_cast<const f4*>(xi) + i), gv = *(reinterpret_cast<const f4*>(gi) + i);
+        f4 o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = one(xv[e], gv[e]);
+        *(reinterpret_cast<f4*>(out) + i) = o;
       }
+    } else {
+      for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < S; i += (int64_t)gridDim.x * kBlock)
+        out[i] = one(xi[i], gi[i]);
     }
   }
 }
@@ -305,8 +339,8 @@ __global__ __launch_bounds__(kBlock) void k_softmax_bwd(const float* __restrict_
 
 // how many workgroups share one channel's reduction
 int bn_groups(int64_t n, int64_t S) {
-  // strips of a plane when planes are wide, slices of the batch otherwise
-  int64_t g = (S >= kBlock ? S : n / S) / 1024;
+  // wide planes: two 256-wide strips of every image per workgroup; else 1024 images per workgroup
+  int64_t g = S >= kBlock ? (S + kBlock - 1) / kBlock / 2 : (n / S) / 1024;
   if (g < 1) g = 1;
   if (g > 64) g = 64;
   return (int)g;
@@ -386,13 +420,14 @@ int gh_launch_bn_bwd(gh_ctx* ctx, const gh_cmd& c) {
   hipLaunchKernelGGL(k_bn_bwd_reduce, dim3(G, (int)C), dim3(kBlock), 0, ctx->stream, x, dy, save_mean, part,
                      (int)C, S, n);
   const int64_t BC = B * C;
-  int gx = (int)((S + kBlock * 4 - 1) / (kBlock * 4));
+  const int vec = S % 4 == 0 && ((c.ptr[0] | c.ptr[1] | c.ptr[2]) & 15) == 0;
+  int gx = (int)(((vec ? S / 4 : S) + kBlock * 4 - 1) / (kBlock * 4));
   if (gx < 1) gx = 1;
   if (gx > 1024) gx = 1024;
   const int64_t gy = BC > 65535 ? 65535 : BC;
   const int training = (c.flags & GH_FLAG_BN_EVAL) ? 0 : 1;
   hipLaunchKernelGGL(k_bn_bwd_apply, dim3(gx, (int)gy), dim3(kBlock), 0, ctx->stream, x, dy, dx, save_mean,
-                     save_var, part, c.f[0], training, BC, (int)C, S, G, n);
+                     save_var, part, c.f[0], training, BC, (int)C, S, G, n, vec);
   return gh_check_hip(ctx, hipGetLastError(), "batchnorm backward launch");
 }
 
