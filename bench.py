@@ -204,13 +204,14 @@ def bench_yolo(steps, warmup):
 
 
 def bench_convnet_train(steps, warmup, batch=128):
-    """Config 4 as a training step: forward, every layer's gradient, SGD update
-    of the resident weights; only the 128x10 output leaves the device."""
+    """Config 4 as a training step: forward, every layer's gradient, RMSProp
+    update (examples/convnet/main.go:195) of the resident weights; only the
+    128x10 output leaves the device."""
     from gorgonia_amd import configs, graph as G
     inp = configs.convnet_inputs(batch)
     onehot = np.zeros((batch, 10), np.float32)
     onehot[np.arange(batch), np.arange(batch) % 10] = 1.0
-    g, outs = configs.build_convnet_train(inp, onehot, 0.01, read_grads=False)
+    g, outs = configs.build_convnet_train(inp, onehot, 0.01, read_grads=False, solver="rmsprop")
     m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING)
     for _ in range(max(warmup, 3)):
         m.RunAll()

@@ -105,7 +105,7 @@ def build_convnet(inp, resident=True):
     return g, {"out": G.Read(out)}
 
 
-def build_convnet_train(inp, onehot, lr, read_grads=True):
+def build_convnet_train(inp, onehot, lr, read_grads=True, solver="set"):
     """Config 4 as one training step (examples/convnet/main.go:57-180 with vanilla
     SGD): forward, the diff ops the reference's symbolic differentiation would
     insert, and w <- w - lr * dw through Set, so the resident weights carry over
@@ -147,7 +147,13 @@ def build_convnet_train(inp, onehot, lr, read_grads=True):
             outs[f"dw{i}"] = G.Read(dw[i])
     # updates last: every gradient above was taken at the old weights
     for i in range(5):
-        G.Set(w[i], G.Sub(w[i], G.HadamardProd(dw[i], lr_s)))
+        if solver == "set":      # w <- w - lr*dw spelled with graph ops
+            G.Set(w[i], G.Sub(w[i], G.HadamardProd(dw[i], lr_s)))
+        elif solver == "vanilla":
+            G.SolverStep("vanilla", w[i], dw[i], eta=lr)
+        else:                     # RMSProp as in examples/convnet/main.go:195
+            cache = G.NewTensor(g, np.zeros_like(inp[f"w{i}"]), True)
+            G.SolverStep("rmsprop", w[i], dw[i], [cache], eta=lr, l2reg=1e-6, clip=5.0)
     return g, outs
 
 

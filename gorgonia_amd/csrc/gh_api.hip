@@ -223,6 +223,7 @@ static int dispatch(gh_ctx* ctx, const gh_cmd& c) {
     case GH_OP_BN_TRAIN: return gh_launch_bn_train(ctx, c);
     case GH_OP_BN_BWD: return gh_launch_bn_bwd(ctx, c);
     case GH_OP_SOFTMAX_BWD: return gh_launch_softmax_bwd(ctx, c);
+    case GH_OP_SOLVER_STEP: return gh_launch_solver_step(ctx, c);
   }
   return GH_ENOFUNC;
 }

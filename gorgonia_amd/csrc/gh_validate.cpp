@@ -135,6 +135,13 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
       if (c.dim[0] < 0 || !pos(c.dim[1])) return bad("softmax: bad shape");
       return GH_OK;
+    case GH_OP_SOLVER_STEP:
+      if (fn >= GH_SOLVER__COUNT) { msg = "unknown solver"; return GH_ENOFUNC; }
+      if (!c.ptr[0] || !c.ptr[1]) return bad("null operand");
+      if (fn >= GH_SOLVER_RMSPROP && !c.ptr[2]) return bad("solver cache is null");
+      if (fn == GH_SOLVER_ADAM && !c.ptr[3]) return bad("Adam second-moment cache is null");
+      if (c.dim[0] < 0) return bad("negative size");
+      return GH_OK;
     case GH_OP_RELU:
     case GH_OP_LEAKY_RELU:
       if (!c.ptr[0] || !c.ptr[1]) return bad("null operand");

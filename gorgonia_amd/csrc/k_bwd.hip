@@ -337,6 +337,70 @@ __global__ __launch_bounds__(kBlock) void k_softmax_bwd(const float* __restrict_
   }
 }
 
+// ---- solver steps ---------------------------------------------------------------------
+// One fused pass per tensor instead of the reference's 6-15 tensor ops
+// (solvers.go:273-372, 461-640, 780-870); every intermediate is rounded where
+// a tensor op of the reference would round it, so the weights and caches get
+// the reference's bits.
+struct SolverPar { float eta, eps, l1reg, l2reg, clip, one_per_batch, a, b, corr1, corr2; };
+
+__device__ __forceinline__ float clampf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+__device__ __forceinline__ float prep_grad(float g, float w, int use, const SolverPar& p) {
+  if (use & 1) { const float t = p.l1reg * (float)((w > 0.0f) - (w < 0.0f)); g = g + t; }
+  if (use & 2) { const float t = w * p.l2reg; g = g + t; }
+  if (use & 8) g = g * p.one_per_batch;
+  if ((use & 4) && p.clip > 0.0f) g = clampf(g, -p.clip, p.clip);
+  return g;
+}
+
+template <int KIND>
+__global__ __launch_bounds__(kBlock) void k_solver_step(float* __restrict__ w, const float* __restrict__ g,
+                                                        float* __restrict__ c1, float* __restrict__ c2,
+                                                        int64_t n, int use, SolverPar p) {
+  const float neg_eta = -p.eta;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    if (KIND == GH_SOLVER_VANILLA) {
+      float gi = prep_grad(g[i], w[i], use, p);
+      gi = gi * neg_eta;
+      w[i] = w[i] + gi;
+    } else if (KIND == GH_SOLVER_RMSPROP) {
+      float gi = g[i];
+      float gt2 = gi * gi;
+      float cw = c1[i] * p.a;
+      gt2 = gt2 * p.b;
+      cw = cw + gt2;
+      c1[i] = cw;
+      if (use & 4) gi = clampf(gi, -p.clip, p.clip);
+      float upd = cw + p.eps;
+      upd = 1.0f / sqrtf(upd);
+      gi = gi * neg_eta;
+      upd = upd * gi;
+      if (use & 2) { const float reg = w[i] * p.l2reg; upd = upd - reg; }
+      w[i] = w[i] + upd;
+    } else {
+      const float gi = prep_grad(g[i], w[i], use, p);
+      const float omb1 = 1.0f - p.a, omb2 = 1.0f - p.b;
+      float t1 = gi * omb1;
+      float g2 = gi * gi;
+      g2 = g2 * omb2;
+      const float mb = c1[i] * p.a;
+      t1 = t1 + mb;
+      const float vb = c2[i] * p.b;
+      g2 = g2 + vb;
+      c1[i] = t1;
+      c2[i] = g2;
+      float mh = t1 * p.corr1;
+      float vh = g2 * p.corr2;
+      vh = sqrtf(vh);
+      vh = vh + p.eps;
+      mh = mh * neg_eta;
+      mh = mh / vh;
+      w[i] = w[i] + mh;
+    }
+  }
+}
+
 // how many workgroups share one channel's reduction
 int bn_groups(int64_t n, int64_t S) {
   // wide planes: two 256-wide strips of every image per workgroup; else 1024 images per workgroup
@@ -440,4 +504,25 @@ int gh_launch_softmax_bwd(gh_ctx* ctx, const gh_cmd& c) {
                      (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
                      (float*)(uintptr_t)c.ptr[2], rows, cols);
   return gh_check_hip(ctx, hipGetLastError(), "softmax backward launch");
+}
+
+int gh_launch_solver_step(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t n = c.dim[0];
+  if (n == 0) return GH_OK;
+  const int kind = (int)gh_fn(c.flags), use = (int)gh_mode(c.flags);
+  SolverPar p{c.f[0], c.f[1], c.f[2], c.f[3], c.f[4], c.f[5], c.f[6], c.f[7], c.f[8], c.f[9]};
+  float* w = (float*)(uintptr_t)c.ptr[0];
+  const float* g = (const float*)(uintptr_t)c.ptr[1];
+  float* c1 = (float*)(uintptr_t)c.ptr[2];
+  float* c2 = (float*)(uintptr_t)c.ptr[3];
+  int64_t blocks = (n + kBlock - 1) / kBlock;
+  if (blocks > (int64_t)ctx->cu_count * 32) blocks = (int64_t)ctx->cu_count * 32;
+  const dim3 grid((int)blocks), block(kBlock);
+  if (kind == GH_SOLVER_VANILLA)
+    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_VANILLA>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p);
+  else if (kind == GH_SOLVER_RMSPROP)
+    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_RMSPROP>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p);
+  else
+    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_ADAM>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p);
+  return gh_check_hip(ctx, hipGetLastError(), "solver step launch");
 }

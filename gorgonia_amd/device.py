@@ -258,6 +258,15 @@ def cmd_softmax_bwd(y, dy, dx, rows, cols):
     return make_cmd(_ffi.OP_SOFTMAX_BWD, 0, (y, dy, dx), (rows, cols))
 
 
+SOLVER = {"vanilla": 0, "rmsprop": 1, "adam": 2}
+
+
+def cmd_solver_step(kind, w, g, n, par, use, cache=0, cache2=0):
+    """par: the ten float32 constants of gorgonia_hip.h's SOLVER_STEP row; use: option mask."""
+    fl = _ffi.flag_fn(SOLVER[kind]) | _ffi.flag_mode(use)
+    return make_cmd(_ffi.OP_SOLVER_STEP, fl, (w, g, cache, cache2), (n,), tuple(float(v) for v in par))
+
+
 def cmd_has(kind, a, flag, n, dtype=_ffi.F32):
     op = _ffi.OP_HAS_NAN if kind == "nan" else _ffi.OP_HAS_INF
     return make_cmd(op, _ffi.flag_dtype(dtype), (a, flag), (n,))

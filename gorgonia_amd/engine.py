@@ -23,7 +23,7 @@ class GhhTensor(C.Structure):
 class GhhOp(C.Structure):
     _fields_ = [("kind", C.c_int32), ("fn", C.c_int32), ("name", C.c_char * 24),
                 ("trans_a", C.c_int32), ("trans_b", C.c_int32), ("n_ints", C.c_int32),
-                ("ints", C.c_int64 * 16), ("f0", C.c_double), ("f1", C.c_double)]
+                ("ints", C.c_int64 * 16), ("f0", C.c_double), ("f1", C.c_double), ("fs", C.c_double * 10)]
 
 
 T_NOT_MANAGED, T_TRANSPOSED, T_NEEDS_ITER = 1, 2, 4

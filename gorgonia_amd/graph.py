@@ -14,7 +14,7 @@ from .engine import Engine, EngineError, GhhOp, load_host
 
 (K_ELEMBIN, K_ELEMUNARY, K_BCAST, K_MATMUL, K_MATVEC, K_OUTER, K_BMM, K_CONV2D, K_MAXPOOL, K_BN,
  K_RECTIFY, K_LEAKY, K_SOFTMAX, K_RESHAPE, K_MAXPOOL_DIFF, K_CONV_DIFF_DATA, K_CONV_DIFF_FILTER, K_BN_TRAIN,
- K_BN_DIFF, K_SOFTMAX_DIFF, K_SET) = range(21)
+ K_BN_DIFF, K_SOFTMAX_DIFF, K_SET, K_SOLVER) = range(22)
 
 
 class Node:
@@ -45,7 +45,7 @@ class ExprGraph:
         n = self.lib.ghh_graph_node_shape(self.h, nid, buf, 8)
         return tuple(buf[i] for i in range(n))
 
-    def apply(self, kind, inputs, fn=0, name="", trans_a=False, trans_b=False, ints=(), f0=0.0, f1=0.0):
+    def apply(self, kind, inputs, fn=0, name="", trans_a=False, trans_b=False, ints=(), f0=0.0, f1=0.0, fs=()):
         op = GhhOp()
         op.kind, op.fn, op.name = kind, fn, name.encode()
         op.trans_a, op.trans_b = int(trans_a), int(trans_b)
@@ -54,6 +54,8 @@ class ExprGraph:
             op.ints[i] = int(v)
         op.f0 = float(f0)
         op.f1 = float(f1)
+        for i, v in enumerate(fs):
+            op.fs[i] = float(v)
         arr = (C.c_int * len(inputs))(*[n.id for n in inputs])
         out = C.c_int()
         self._check(self.lib.ghh_graph_apply(self.h, C.byref(op), arr, len(inputs), C.byref(out)))
@@ -215,6 +217,22 @@ def Set(a, b):
     """gorgonia.Set(a, b): a's value becomes b's; a keeps its register, so a
     resident input updated this way carries the new value into the next run."""
     return a.g.apply(K_SET, [a, b])
+
+
+def SolverStep(kind, weights, grad, caches=(), eta=0.001, eps=1e-8, l1reg=0.0, l2reg=0.0, clip=0.0, batch=1.0,
+               decay=0.999, beta1=0.9, beta2=0.999, iteration=1):
+    """One Step of NewVanillaSolver / NewRMSPropSolver / NewAdamSolver (solvers.go) on one
+    weight tensor, on the device: the weights (a resident input) and the solver's caches
+    (resident inputs, zero at the start) are updated in place.  The constants are
+    rounded to float32 the way the reference rounds them; Adam's bias corrections
+    depend on `iteration`, so an Adam step is a new command every run."""
+    f = np.float32
+    a, b = (f(decay), f(1.0 - decay)) if kind == "rmsprop" else (f(beta1), f(beta2))
+    fs = [f(eta), f(eps), f(l1reg), f(l2reg), f(clip), f(1) / f(batch), a, b,
+          f(1) / f(1 - beta1 ** iteration), f(1) / f(1 - beta2 ** iteration)]
+    use = (1 if l1reg else 0) | (2 if l2reg else 0) | (4 if clip else 0) | (8 if batch > 1 else 0)
+    fn = {"vanilla": 0, "rmsprop": 1, "adam": 2}[kind]
+    return weights.g.apply(K_SOLVER, [weights, grad] + list(caches), fn=fn, ints=[use], fs=fs)
 
 
 class TapeMachine:

@@ -185,6 +185,7 @@ int ghh_graph_apply(ghh_graph* g, const ghh_op* op, const int* inputs, int n_inp
   for (int i = 0; i < op->n_ints && i < 16; i++) s.ints.push_back(op->ints[i]);
   s.f0 = op->f0;
   s.f1 = op->f1;
+  s.fs.assign(op->fs, op->fs + 10);
   std::vector<int> in(inputs, inputs + n_inputs);
   return ret(g, g->g.Apply(s, in, out));
 }

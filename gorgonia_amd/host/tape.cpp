@@ -206,6 +206,15 @@ Status InferShape(const OpSpec& op, const std::vector<const Shape*>& in, Shape* 
       if (!need(2) || in[0]->TotalSize() != in[1]->TotalSize()) return bad("Set: sizes differ");
       *out = *in[0];
       return Status::OK();
+    case OpKind::SolverStep: {
+      if (op.fn < 0 || op.fn >= GH_SOLVER__COUNT) return bad("SolverStep: unknown solver");
+      if (in.size() != (size_t)(2 + op.fn)) return bad("SolverStep: weights, grad and the solver's caches expected");
+      for (size_t i = 1; i < in.size(); i++)
+        if (in[i]->TotalSize() != in[0]->TotalSize()) return bad("SolverStep: sizes differ");
+      if (op.fs.size() < 10 || op.ints.empty()) return bad("SolverStep: constants missing");
+      *out = *in[0];
+      return Status::OK();
+    }
     case OpKind::Reshape: {
       if (!need(1)) return bad("Reshape needs 1 input");
       Shape s(op.ints);
@@ -252,6 +261,7 @@ static std::string op_name(const OpSpec& op) {
     case OpKind::BatchNormDiff: return "batchnorm.diff";
     case OpKind::SoftMaxDiff: return "softmax.diff";
     case OpKind::Set: return "set";
+    case OpKind::SolverStep: return op.fn == GH_SOLVER_ADAM ? "solver.adam" : op.fn == GH_SOLVER_RMSPROP ? "solver.rmsprop" : "solver.vanilla";
   }
   return "?";
 }
@@ -440,6 +450,16 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       e.Enqueue(c);
       return Status::OK();
     }
+    case OpKind::SolverStep: {
+      gh_cmd c{};
+      c.opcode = GH_OP_SOLVER_STEP;
+      c.flags = GH_FLAG_FN(op.fn) | GH_FLAG_MODE(op.ints[0]);
+      for (size_t i = 0; i < in.size(); i++) c.ptr[i] = in[i]->mem;
+      c.dim[0] = in[0]->DataSize();
+      for (int i = 0; i < 10; i++) c.f[i] = (float)op.fs[(size_t)i];
+      e.Enqueue(c);
+      return Status::OK();
+    }
     case OpKind::Set: {
       // prealloc is a's register (the node aliases a); copy b's bytes into it
       const int64_t bytes = in[1]->DataSize() * dtype_size(in[1]->dt);
@@ -473,7 +493,7 @@ Status Graph::Apply(const OpSpec& op, const std::vector<int>& inputs, int* out) 
   n.dt = inputs.empty() ? Dtype::Float32 : nodes_[(size_t)inputs[0]].dt;
   n.op = op;
   n.inputs = inputs;
-  if (op.kind == OpKind::Reshape || op.kind == OpKind::Set) n.alias_of = inputs[0];
+  if (op.kind == OpKind::Reshape || op.kind == OpKind::Set || op.kind == OpKind::SolverStep) n.alias_of = inputs[0];
   nodes_.push_back(n);
   if (out) *out = n.id;
   return Status::OK();
@@ -606,11 +626,11 @@ Status TapeMachine::Compile() {
   for (int i = 0; i < N; i++) {
     Node& n = nodes[(size_t)i];
     if (n.fused_away) continue;
-    if (n.alias_of >= 0 && n.op.kind != OpKind::Set) continue;  // a view: nothing to run
+    if (n.alias_of >= 0 && n.op.kind != OpKind::Set && n.op.kind != OpKind::SolverStep) continue;  // a view: nothing to run
     const int r = node_reg_[(size_t)i];
     const int64_t bytes = bytes_of(n);
     if (n.alias_of >= 0) {
-      // Set writes into the register it aliases
+      // Set and SolverStep write into the register they alias
       prog_.push_back({InstrKind::ExecOp, i, r, bytes, true});
     } else if (n.is_input) {
       prog_.push_back({InstrKind::LoadArg, i, r, bytes, false});

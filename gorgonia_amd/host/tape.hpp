@@ -48,7 +48,10 @@ enum class OpKind : int32_t {
                          // runningVar, saveMean, saveVar; the four statistics tensors are updated in place
   BatchNormDiff = 18,    // batchnormDiffOp (op_nn.go:1834-1943): inputs x, grad, saveMean, saveVar
   SoftMaxDiff = 19,      // softmaxDiffOp (op_softmax.go:184-279): inputs y, grad
-  Set = 20               // gorgonia.Set(a, b): a's value becomes b's (operations.go); inputs a, b
+  Set = 20,              // gorgonia.Set(a, b): a's value becomes b's (operations.go); inputs a, b
+  SolverStep = 21        // one Step of VanillaSolver / RMSPropSolver / AdamSolver on one weight tensor
+                         // (solvers.go:273-870): inputs weights, grad[, cache[, cache2]]; fn = gh_solver,
+                         // ints[0] = use mask, fs = the ten constants; the weights are updated in place
 };
 
 struct OpSpec {
@@ -58,6 +61,7 @@ struct OpSpec {
   bool transA = false, transB = false;
   std::vector<int64_t> ints;  // kernel/pad/stride/dilation, new shape, broadcast axes ...
   double f0 = 0.0;            // epsilon / alpha
+  std::vector<double> fs;     // SolverStep constants
   // Followers folded into a Conv2d/MatMul epilogue by Graph::FuseActivations,
   // applied in this order: BatchNorm (Conv2d only; inputs 2.. = mean, var[,
   // scale, bias], f1 = epsilon), activation (f0 = alpha), 2x2/2 MaxPool2D.

@@ -87,8 +87,12 @@ enum gh_opcode {
   GH_OP_BN_TRAIN = 20,          /* ops/nn/batchnorm_cuda.go:87-100; CPU op_nn.go:1489-1635     */
   GH_OP_BN_BWD = 21,            /* ops/nn/batchnorm_cuda.go:192-219; CPU op_nn.go:1834-1943    */
   GH_OP_SOFTMAX_BWD = 22,       /* softmaxDiffOp, op_softmax.go:266-279                        */
+  GH_OP_SOLVER_STEP = 23,       /* Vanilla/RMSProp/Adam Step on a float32 tensor, solvers.go:273-870 */
   GH_OP__COUNT
 };
+
+/* GH_OP_SOLVER_STEP: which solver (flags FN field) */
+enum gh_solver { GH_SOLVER_VANILLA = 0, GH_SOLVER_RMSPROP = 1, GH_SOLVER_ADAM = 2, GH_SOLVER__COUNT };
 
 /* flags for GH_OP_ELEM_BIN / GH_OP_BCAST_BIN: fn | mode<<8 | dtype<<12 | ... */
 enum gh_binfn {
@@ -169,13 +173,19 @@ enum gh_unaryfn {
  * BN_BWD      ptr[0]=x ptr[1]=dy ptr[2]=dx ptr[3]=save_mean ptr[4]=save_var
  *             dim[0..2]=B,C,S  f[0]=eps ; BN_EVAL selects dx = dy/sqrt(save_var/n + eps)
  * SOFTMAX_BWD ptr[0]=y ptr[1]=dy ptr[2]=dx        dim[0]=rows dim[1]=cols
+ * SOLVER_STEP ptr[0]=weights ptr[1]=grad [ptr[2]=cache (RMSProp cache / Adam m) ptr[3]=Adam v]
+ *             dim[0]=n ; flags: FN = gh_solver, MODE = use mask (1 l1reg, 2 l2reg, 4 clip,
+ *             8 batch) ; f[0]=eta f[1]=eps f[2]=l1reg f[3]=l2reg f[4]=clip f[5]=1/batch
+ *             f[6]=decay|beta1 f[7]=(1-decay)|beta2 f[8]=1/(1-beta1^t) f[9]=1/(1-beta2^t).
+ *             Weights and caches are updated in place with the reference's sequence of
+ *             tensor ops, one rounding each; grad is left untouched (the reference zeroes it)
  */
 typedef struct gh_cmd {
   uint32_t opcode;
   uint32_t flags;
   uint64_t ptr[8];
   int64_t  dim[16];
-  float    f[4];
+  float    f[12];
 } gh_cmd;
 
 /* ---- context / device -------------------------------------------------- */

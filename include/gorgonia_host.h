@@ -99,6 +99,7 @@ typedef struct ghh_op {
   int64_t ints[16];
   double  f0;
   double  f1;      /* second scalar parameter (BatchNorm momentum) */
+  double  fs[10];  /* SolverStep: the constants of GH_OP_SOLVER_STEP's f[0..9] */
 } ghh_op;
 
 GH_API ghh_graph* ghh_graph_new(void);

@@ -309,6 +309,37 @@ def softmax_bwd(y, dy):
     return dx
 
 
+SOLVER = {"vanilla": 0, "rmsprop": 1, "adam": 2}
+
+
+def solver_params(eta, eps=1e-8, l1reg=0.0, l2reg=0.0, clip=0.0, batch=1.0, decay=0.999, beta1=0.9, beta2=0.999,
+                  kind="vanilla", iteration=1):
+    """The float32 constants a solver step uses, computed the way the reference does
+    (float64 first, then one cast; solvers.go:307-314, 492-525, 793-806), and its use mask."""
+    f = np.float32
+    if kind == "rmsprop":
+        a, b = f(decay), f(1.0 - decay)
+    else:
+        a, b = f(beta1), f(beta2)
+    c1 = f(1) / f(1 - beta1 ** iteration)
+    c2 = f(1) / f(1 - beta2 ** iteration)
+    par = np.array([f(eta), f(eps), f(l1reg), f(l2reg), f(clip), f(1) / f(batch), a, b, c1, c2], dtype=np.float32)
+    use = (1 if l1reg else 0) | (2 if l2reg else 0) | (4 if clip else 0) | (8 if batch > 1 else 0)
+    return par, use
+
+
+def solver_step(kind, w, g, c1=None, c2=None, **kw):
+    """One solver step in place on copies; returns (w, g, c1, c2)."""
+    par, use = solver_params(kind=kind, **kw)
+    w = np.array(w, dtype=np.float32, copy=True)
+    g = np.array(g, dtype=np.float32, copy=True)
+    c1 = np.zeros_like(w) if c1 is None else np.array(c1, dtype=np.float32, copy=True)
+    c2 = np.zeros_like(w) if c2 is None else np.array(c2, dtype=np.float32, copy=True)
+    lib().oracle_solver_step_f32(C.c_int(SOLVER[kind]), _p(w), _p(g), _p(c1), _p(c2), C.c_int64(w.size),
+                                 C.c_int(use), _p(par))
+    return w, g, c1, c2
+
+
 def has_nan(a):
     a = np.ascontiguousarray(a, dtype=np.float32)
     return bool(lib().oracle_has_nan_f32(_p(a), C.c_int64(a.size)))

@@ -835,6 +835,76 @@ EXPORT void oracle_softmax_bwd_f32(const float* y, const float* dy, float* dx, i
   }
 }
 
+/* ================================================================== */
+/* Solver steps on float32 tensors: the *tensor.Dense branches of      */
+/* VanillaSolver.Step (solvers.go:780-870), RMSPropSolver.Step         */
+/* (solvers.go:273-372) and AdamSolver.Step (solvers.go:461-640), one  */
+/* element at a time with every tensor op's rounding kept.             */
+/* par: 0 eta, 1 eps, 2 l1reg, 3 l2reg, 4 clip, 5 1/batch,             */
+/*      6 decay | beta1, 7 1-decay | beta2, 8 1/correction1,           */
+/*      9 1/correction2.  use: bit0 l1, bit1 l2, bit2 clip, bit3 batch */
+/* The gradient is left as the reference leaves it before g.Zero().    */
+/* ================================================================== */
+static float clampf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
+static float signf(float v) { return v > 0.0f ? 1.0f : (v < 0.0f ? -1.0f : 0.0f); }
+
+static float prep_grad(float g, float w, int use, const float* par) {
+  if (use & 1) { float t = par[2] * signf(w); g = g + t; }
+  if (use & 2) { float t = w * par[3]; g = g + t; }
+  if (use & 8) g = g * par[5];
+  if ((use & 4) && par[4] > 0.0f) g = clampf(g, -par[4], par[4]);
+  return g;
+}
+
+EXPORT void oracle_solver_step_f32(int kind, float* w, float* g, float* c1, float* c2, int64_t n,
+                                   int use, const float* par) {
+  int64_t i;
+  const float neg_eta = -par[0];
+  for (i = 0; i < n; i++) {
+    if (kind == 0) {            /* vanilla */
+      float gi = prep_grad(g[i], w[i], use, par);
+      gi = gi * neg_eta;
+      w[i] = w[i] + gi;
+      g[i] = gi;
+    } else if (kind == 1) {     /* RMSProp */
+      float gi = g[i];
+      float gt2 = gi * gi;
+      float cw = c1[i] * par[6];
+      gt2 = gt2 * par[7];
+      cw = cw + gt2;
+      c1[i] = cw;
+      if (use & 4) gi = clampf(gi, -par[4], par[4]);
+      float upd = cw + par[1];
+      upd = 1.0f / sqrtf(upd);
+      gi = gi * neg_eta;
+      upd = upd * gi;
+      if (use & 2) { float reg = w[i] * par[3]; upd = upd - reg; }
+      w[i] = w[i] + upd;
+      g[i] = gi;
+    } else {                    /* Adam */
+      float gi = prep_grad(g[i], w[i], use, par);
+      float omb1 = 1.0f - par[6], omb2 = 1.0f - par[7];
+      float t1 = gi * omb1;
+      float g2 = gi * gi;
+      g2 = g2 * omb2;
+      float mb = c1[i] * par[6];
+      t1 = t1 + mb;
+      float vb = c2[i] * par[7];
+      g2 = g2 + vb;
+      c1[i] = t1;
+      c2[i] = g2;
+      float mh = t1 * par[8];
+      float vh = g2 * par[9];
+      vh = sqrtf(vh);
+      vh = vh + par[1];
+      mh = mh * neg_eta;
+      mh = mh / vh;
+      w[i] = w[i] + mh;
+      g[i] = g2;
+    }
+  }
+}
+
 /* ------------------------------------------------------------------ */
 EXPORT void oracle_softmax_f32(const float* x, float* y, int64_t rows, int64_t cols) {
   int64_t r, j;

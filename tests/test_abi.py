@@ -25,7 +25,7 @@ def test_header_symbols_all_exported():
 
 
 def test_struct_layout_matches_header():
-    assert C.sizeof(_ffi.GhCmd) == 4 + 4 + 8 * 8 + 16 * 8 + 4 * 4
+    assert C.sizeof(_ffi.GhCmd) == 4 + 4 + 8 * 8 + 16 * 8 + 12 * 4
     assert _ffi.GhCmd.ptr.offset == 8 and _ffi.GhCmd.dim.offset == 72 and _ffi.GhCmd.f.offset == 200
 
 

@@ -146,6 +146,40 @@ def test_batchnorm_training_forward_and_backward(ctx, B, C, S):
         ctx.free(p)
 
 
+@pytest.mark.parametrize("kind,kw", [
+    ("vanilla", dict(eta=0.05)),
+    ("vanilla", dict(eta=0.05, l1reg=0.01, l2reg=0.02, clip=0.5, batch=4.0)),
+    ("rmsprop", dict(eta=0.01, l2reg=1e-6, clip=5.0, decay=0.999)),
+    ("rmsprop", dict(eta=0.001)),
+    ("adam", dict(eta=0.1, iteration=1)),
+    ("adam", dict(eta=0.02, l1reg=0.001, l2reg=0.002, clip=1.0, batch=2.0, iteration=7)),
+])
+def test_solver_steps_bit_exact(ctx, kind, kw):
+    """Three consecutive steps on the device against the oracle's (which is pinned by the
+    reference's RMSProp closed form and Adam golden): weights and caches bit for bit."""
+    n = 100003
+    w = synth.normal(31, (n,))
+    c1 = np.zeros(n, np.float32)
+    c2 = np.zeros(n, np.float32)
+    pw, pc1, pc2 = ctx.upload(w), ctx.upload(c1), ctx.upload(c2)
+    for step in range(3):
+        g = synth.normal(40 + step, (n,), 0.0, 3.0)
+        if kind == "adam":
+            kw = dict(kw, iteration=kw["iteration"] + (1 if step else 0))
+        par, use = O.solver_params(kind=kind, **kw)
+        pg = ctx.upload(g)
+        ctx.run(D.cmd_solver_step(kind, pw, pg, n, par, use, pc1, pc2))
+        ctx.free(pg)
+        w, _, c1, c2 = O.solver_step(kind, w, g, c1, c2, **kw)
+        assert_bits_equal(ctx.d2h(pw, (n,)), w, f"{kind} weights, step {step}")
+        if kind != "vanilla":
+            assert_bits_equal(ctx.d2h(pc1, (n,)), c1, f"{kind} cache, step {step}")
+        if kind == "adam":
+            assert_bits_equal(ctx.d2h(pc2, (n,)), c2, f"adam v, step {step}")
+    for p in (pw, pc1, pc2):
+        ctx.free(p)
+
+
 def test_backward_commands_validate(ctx):
     import ctypes as C
     buf = C.create_string_buffer(256)

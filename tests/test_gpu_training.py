@@ -61,6 +61,38 @@ def test_training_steps_replayed_from_a_graph(ctx):
     m.Close()
 
 
+def test_training_with_device_solver_steps(ctx):
+    """The same step with the update done by the fused solver kernels: vanilla equals the
+    Set-spelled update bit for bit; RMSProp (the example's solver) follows the oracle."""
+    inp = configs.convnet_inputs(16)
+    y = _onehot(16)
+    outs_by = {}
+    for solver in ("set", "vanilla", "rmsprop"):
+        g, outs = configs.build_convnet_train(inp, y, 0.05 if solver != "rmsprop" else 0.01, read_grads=False,
+                                              solver=solver)
+        m = G.NewTapeMachine(g, graph_replay=True)
+        hist = []
+        for _ in range(4):
+            m.RunAll()
+            hist.append(outs["out"].copy())
+        assert m.graph_launches() >= 2
+        outs_by[solver] = hist
+        m.Close()
+    for a, b in zip(outs_by["set"], outs_by["vanilla"]):
+        assert_bits_equal(a, b, "vanilla solver step == w - lr*dw through Set")
+    # RMSProp against the oracle: forward/backward by the oracle step, update by the oracle solver
+    cur = dict(inp)
+    caches = {k: np.zeros_like(inp[k]) for k in ("w0", "w1", "w2", "w3", "w4")}
+    from oracle import binding as O
+    for step in range(4):
+        want, _, grads, _ = F.convnet_train_step(cur, y, 0.0)
+        assert rel_frobenius(outs_by["rmsprop"][step], want) <= 2 * TOL * (step + 1), f"rmsprop step {step}"
+        for k in caches:
+            wn, _, cn, _ = O.solver_step("rmsprop", cur[k].reshape(-1), grads[k].reshape(-1), caches[k].reshape(-1),
+                                         eta=0.01, l2reg=1e-6, clip=5.0)
+            cur[k], caches[k] = wn.reshape(cur[k].shape), cn.reshape(cur[k].shape)
+
+
 def test_set_updates_a_resident_input_in_place(ctx):
     g = G.NewGraph()
     a = G.NewTensor(g, np.arange(8, dtype=np.float32), resident=True)

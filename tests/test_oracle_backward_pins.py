@@ -222,3 +222,57 @@ def test_softmax_bwd_finite_difference_and_identities():
     # old-vs-new softmax example of op_softmax_test.go:283-290: cost = Sum(softmax(a)) has zero gradient
     a = np.array([[0.1, 0.1, 0.3, 0.1, 0.4]])
     assert np.allclose(O.softmax_bwd(O.softmax(a).astype(np.float32), np.ones((1, 5), np.float32)), 0, atol=1e-7)
+
+
+# ---- solvers ------------------------------------------------------------------------
+
+def test_rmsprop_manual_closed_form():
+    """solvers_test.go:100-143 manualRMSProp32 (TestRMSPropSolverManual): lr 0.01, l2reg 1e-6, clip 5,
+    weights [1,2,3,4], gradients [0.5,-10,10,0.5] (zeroed by the first step), five iterations, 1e-4."""
+    f = np.float32
+    w = np.array([1, 2, 3, 4], f)
+    g = np.array([0.5, -10, 10, 0.5], f)
+    cache = np.zeros(4, f)
+    correct_w, correct_c = w.copy(), np.zeros(4, f)
+    decay, l2reg, eta, eps, clip = f(0.999), f(1e-6), f(0.01), f(1e-8), f(5.0)
+    grad = g.copy()
+    for it in range(5):
+        for j in range(4):
+            decayed = f(correct_c[j] * decay + f(f(f(1.0) - decay) * grad[j]) * grad[j])
+            correct_c[j] = decayed
+            gc = min(max(grad[j], -clip), clip)
+            upd = f(f(f(-eta * gc) / np.sqrt(f(decayed + eps))) - f(l2reg * correct_w[j]))
+            correct_w[j] = f(correct_w[j] + upd)
+        w, _, cache, _ = O.solver_step("rmsprop", w, grad, cache, eta=0.01, l2reg=1e-6, clip=5.0, decay=0.999)
+        grad = np.zeros(4, f)   # gt.Zero() at the end of Step (solvers.go:366)
+        assert np.allclose(w, correct_w, rtol=1e-4, atol=0), it
+        assert np.allclose(cache, correct_c, rtol=1e-4, atol=0), it
+
+
+def test_adam_precision_golden():
+    """solvers_test.go:355-437 TestAdamSolverPrecision float32: weights ones(4), the gradient of
+    Mean(x . w) wrt w is x = d for d = 0, 0.1, ... (float32 accumulation) < 1; lr 0.1; ten steps."""
+    f = np.float32
+    w, m, v = np.ones(4, f), np.zeros(4, f), np.zeros(4, f)
+    d, it = f(0.0), 0
+    while d < f(1.0):
+        it += 1
+        w, _, m, v = O.solver_step("adam", w, np.full(4, d, f), m, v, eta=0.1, iteration=it)
+        d = f(d + f(0.1))
+    assert it == 10
+    assert np.allclose(w, [0.18293014] * 4, rtol=1e-5, atol=1e-6), w
+
+
+def test_vanilla_step_is_w_minus_eta_g_with_the_options_in_order():
+    f = np.float32
+    rng = np.random.default_rng(11)
+    w = rng.standard_normal(1000).astype(f)
+    g = rng.standard_normal(1000).astype(f)
+    w1, _, _, _ = O.solver_step("vanilla", w, g, eta=0.05)
+    assert np.array_equal(w1, (w + g * f(-0.05)).astype(f))
+    w2, _, _, _ = O.solver_step("vanilla", w, g, eta=0.05, l1reg=0.01, l2reg=0.02, clip=0.5, batch=4.0)
+    gg = g + f(0.01) * np.sign(w).astype(f)
+    gg = gg + w * f(0.02)
+    gg = gg * (f(1) / f(4))
+    gg = np.clip(gg, f(-0.5), f(0.5))
+    assert np.array_equal(w2, (w + gg * f(-0.05)).astype(f))
