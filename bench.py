@@ -108,6 +108,17 @@ def bench_linalg(ctx, iters):
                      "frac_mfma": round(fl / ms / 1e9 / MFMA_F32_PEAK_TFLOPS, 4), "flop": fl}
         for q in (A, B, Cm):
             ctx.free(q)
+    # float64 product (Dgemm path), against the fp64 matrix peak of 78.6 TFLOP/s
+    from gorgonia_amd import _ffi
+    m = n = k = 2048
+    A = ctx.upload(synth.normal(6, (m * k,)).astype(np.float64))
+    B = ctx.upload(synth.normal(7, (k * n,)).astype(np.float64))
+    Cm = ctx.malloc(m * n * 8)
+    ms = time_cmds(ctx, [D.cmd_gemm(A, B, Cm, m, n, k, dtype=_ffi.F64)], max(5, iters // 2))
+    res["dgemm_2048"] = {"us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * m * n * k / ms / 1e9, 2),
+                         "frac_mfma_f64": round(2.0 * m * n * k / ms / 1e9 / 78.6, 4)}
+    for q in (A, B, Cm):
+        ctx.free(q)
     m = n = 8192
     A = ctx.upload(synth.normal(3, (m * n,)))
     xv, yv = ctx.upload(synth.normal(4, (n,))), ctx.malloc(4 * m)

@@ -53,6 +53,10 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (batch > 1 && (c.dim[7] < 0 || c.dim[8] < 0 || c.dim[9] < m * n))
         return bad("gemm: bad batch strides");
       if (batch > 65535 * 16) return bad("gemm: batch too large");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
+      if (dt == GH_F64 && (c.flags & (GH_FLAG_ACT_RELU | GH_FLAG_ACT_LEAKY)))
+        return bad("gemm: no fused activation for float64");
+      if (dt == GH_F64 && batch > 65535) return bad("gemm: batch too large");
       return GH_OK;
     }
     case GH_OP_GEMV:

@@ -809,6 +809,81 @@ __global__ __launch_bounds__(256) void k_conv3x3_direct(const float* __restrict_
   }
 }
 
+// ---- float64 GEMM -----------------------------------------------------------------
+// C = op(A) op(B) in float64 on the matrix cores (v_mfma_f64_16x16x4f64: lane l
+// feeds A[l%16][l/16] and B[l/16][l%16]; accumulator register v of lane l is
+// C[4*v + l/16][l%16]).  64x64 block tile, four wavefronts of 32x32, operands
+// staged k-major through LDS with plain bounds-checked loads (any transpose, any
+// leading dimension).  Present for the float64 engine path; not tuned.
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(kThreads) void k_dgemm(const double* __restrict__ A,
+                                                    const double* __restrict__ B,
+                                                    double* __restrict__ C, int M, int N, int K,
+                                                    int lda, int ldb, int ldc, int64_t sA, int64_t sB,
+                                                    int64_t sC, int ta, int tb) {
+  constexpr int BM = 64, BN = 64, BK = 16, S = 66;
+  __shared__ double As[BK * S], Bs[BK * S];
+  A += blockIdx.z * sA;
+  B += blockIdx.z * sB;
+  C += blockIdx.z * sC;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+  const int lr = lane & 15, lk = lane >> 4;
+  f64x4 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; a++)
+#pragma unroll
+    for (int b = 0; b < 2; b++) acc[a][b] = f64x4{0.0, 0.0, 0.0, 0.0};
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    // 64 x 16 elements per operand, 4 per thread; consecutive threads walk the
+    // operand's contiguous axis
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const int f = threadIdx.x + e * kThreads;
+      {
+        const int r = ta ? f % BM : f / BK, k = ta ? f / BM : f % BK;
+        const int i = m0 + r, kk = k0 + k;
+        double v = 0.0;
+        if (i < M && kk < K) v = ta ? A[(int64_t)kk * lda + i] : A[(int64_t)i * lda + kk];
+        As[k * S + r] = v;
+      }
+      {
+        const int c = tb ? f / BK : f % BN, k = tb ? f % BK : f / BN;
+        const int j = n0 + c, kk = k0 + k;
+        double v = 0.0;
+        if (j < N && kk < K) v = tb ? B[(int64_t)j * ldb + kk] : B[(int64_t)kk * ldb + j];
+        Bs[k * S + c] = v;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 4) {
+      double af[2], bf[2];
+#pragma unroll
+      for (int a = 0; a < 2; a++) af[a] = As[(kk + lk) * S + wm + a * 16 + lr];
+#pragma unroll
+      for (int b = 0; b < 2; b++) bf[b] = Bs[(kk + lk) * S + wn + b * 16 + lr];
+#pragma unroll
+      for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+          acc[a][b] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[a], bf[b], acc[a][b], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int a = 0; a < 2; a++)
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        const int i = m0 + wm + a * 16 + 4 * v + lk, j = n0 + wn + b * 16 + lr;
+        if (i < M && j < N) C[(int64_t)i * ldc + j] = acc[a][b][v];
+      }
+}
+
 // ---- Conv2d backward ---------------------------------------------------------------
 // The reference differentiates Conv2d through its im2col + MatMul graph
 // (nn.go:211-305): dW = dY2d^T . col and dX = col2im(dY2d . Wflat)
@@ -1350,6 +1425,17 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) {
+    const int M = (int)c.dim[0], N = (int)c.dim[1], K = (int)c.dim[2];
+    const int64_t batch = c.dim[6] <= 0 ? 1 : c.dim[6];
+    const dim3 grid((N + 63) / 64, (M + 63) / 64, (unsigned)batch);
+    hipLaunchKernelGGL(k_dgemm, grid, dim3(kThreads), 0, ctx->stream, (const double*)(uintptr_t)c.ptr[0],
+                       (const double*)(uintptr_t)c.ptr[1], (double*)(uintptr_t)c.ptr[2], M, N, K, (int)c.dim[3],
+                       (int)c.dim[4], (int)c.dim[5], batch > 1 ? c.dim[7] : 0, batch > 1 ? c.dim[8] : 0,
+                       batch > 1 ? c.dim[9] : 0, (c.flags & GH_FLAG_TRANS_A) ? 1 : 0,
+                       (c.flags & GH_FLAG_TRANS_B) ? 1 : 0);
+    return gh_check_hip(ctx, hipGetLastError(), "dgemm launch");
+  }
   const int rs = try_launch_gemm_skinny(ctx, c);
   if (rs >= 0) return rs;
   const int64_t batch = c.dim[6] <= 0 ? 1 : c.dim[6];

@@ -403,7 +403,8 @@ Status Engine::MatVecMul(Tensor& a, Tensor& b, Tensor& prealloc) {
 Status Engine::MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act, float alpha) {
   Status st = checkThreeFloat(a, b, prealloc);
   if (!st.ok()) return st.Wrap("MatMul failed pre check");
-  if (a.dt != Dtype::Float32) return Status::Err(GH_EINVAL, "Unsupported Dtype " + dtype_name(a.dt));
+  if (a.dt == Dtype::Other) return Status::Err(GH_EINVAL, "Unsupported Dtype " + dtype_name(a.dt));
+  if (a.dt == Dtype::Float64 && act) return Status::Err(GH_EINVAL, "MatMul: no fused activation for float64");
   if (a.shape.Dims() != 2 || b.shape.Dims() != 2 || prealloc.shape.Dims() != 2)
     return Status::Err(GH_EINVAL, "MatMul: operands must be matrices");
   const int64_t m = a.shape[0], k = a.shape[1], n = b.shape[1];
@@ -417,7 +418,8 @@ Status Engine::MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act, float alp
   gh_cmd c{};
   c.opcode = GH_OP_GEMM;
   c.flags = (a.transposed ? GH_FLAG_TRANS_A : 0) | (b.transposed ? GH_FLAG_TRANS_B : 0) |
-            (act == 1 ? GH_FLAG_ACT_RELU : act == 2 ? GH_FLAG_ACT_LEAKY : 0);
+            (act == 1 ? GH_FLAG_ACT_RELU : act == 2 ? GH_FLAG_ACT_LEAKY : 0) |
+            GH_FLAG_DTYPE(a.dt == Dtype::Float64 ? GH_F64 : GH_F32);  // Dgemm / Sgemm, cuda/linalg.go:204-227
   c.f[0] = alpha;
   c.ptr[0] = a.mem; c.ptr[1] = b.mem; c.ptr[2] = prealloc.mem;
   c.dim[0] = m; c.dim[1] = n; c.dim[2] = k;
@@ -447,7 +449,7 @@ Status Engine::Outer(Tensor& a, Tensor& b, Tensor& prealloc) {
 Status Engine::BatchedMatMul(Tensor& a, Tensor& b, Tensor& c, bool transA, bool transB) {
   Status st = checkThreeFloat(a, b, c);
   if (!st.ok()) return st.Wrap("BatchedMatMul failed pre check");
-  if (a.dt != Dtype::Float32) return Status::Err(GH_EINVAL, "Unsupported Dtype");
+  if (a.dt == Dtype::Other) return Status::Err(GH_EINVAL, "Unsupported Dtype");
   const int da = a.shape.Dims(), db = b.shape.Dims();
   if (da < 3 || db != da) return Status::Err(GH_EINVAL, "BatchedMatMul: operands need equal rank >= 3");
   int64_t batch = 1;
@@ -462,7 +464,8 @@ Status Engine::BatchedMatMul(Tensor& a, Tensor& b, Tensor& c, bool transA, bool 
   if (c.DataSize() != batch * m * n) return Status::Err(GH_EINVAL, "BatchedMatMul: bad result shape");
   gh_cmd cmd{};
   cmd.opcode = GH_OP_GEMM;
-  cmd.flags = (transA ? GH_FLAG_TRANS_A : 0) | (transB ? GH_FLAG_TRANS_B : 0);
+  cmd.flags = (transA ? GH_FLAG_TRANS_A : 0) | (transB ? GH_FLAG_TRANS_B : 0) |
+              GH_FLAG_DTYPE(a.dt == Dtype::Float64 ? GH_F64 : GH_F32);
   cmd.ptr[0] = a.mem; cmd.ptr[1] = b.mem; cmd.ptr[2] = c.mem;
   cmd.dim[0] = m; cmd.dim[1] = n; cmd.dim[2] = k;
   cmd.dim[3] = ac; cmd.dim[4] = bc; cmd.dim[5] = n;

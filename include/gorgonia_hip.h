@@ -142,6 +142,7 @@ enum gh_unaryfn {
  * GEMM        ptr[0]=A ptr[1]=B ptr[2]=C   dim[0..2]=m,n,k  dim[3..5]=lda,ldb,ldc
  *             dim[6]=batch (0/1 = single)  dim[7..9]=strideA,strideB,strideC
  *             row-major; C(m x n) = op(A)(m x k) * op(B)(k x n)
+ *             float64 with GH_FLAG_DTYPE(GH_F64) (no fused activation)
  * GEMV        ptr[0]=A ptr[1]=x ptr[2]=y   dim[0..2]=m,n,lda ; A is (m x n) row-major,
  *             y(m)=A x, or with TRANS_A y(n)=A^T x
  * OUTER       ptr[0]=x ptr[1]=y ptr[2]=A   dim[0..1]=m,n ; A(m x n) = x y^T

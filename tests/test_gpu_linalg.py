@@ -146,3 +146,42 @@ def test_outer_bit_exact(ctx):
     assert_bits_equal(ctx.d2h(dA, (37, 53)), O.outer(x, y), "outer")
     for p in (dx, dy, dA):
         ctx.free(p)
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_matmul_float64(ctx, ta, tb):
+    """Dgemm path of Engine.MatMul (cuda/linalg.go:204-227): float64 on the matrix cores,
+    against numpy's float64 product (1e-13 relative) and exactly on integer data."""
+    from gorgonia_amd import _ffi
+    rng = np.random.default_rng(17)
+    for (m, k, n) in [(1, 1, 1), (3, 5, 7), (16, 4, 16), (65, 129, 33), (128, 128, 128), (256, 300, 100), (100, 37, 259)]:
+        for integer in (False, True):
+            A = rng.integers(-8, 9, (k, m) if ta else (m, k)).astype(np.float64) if integer else \
+                rng.standard_normal((k, m) if ta else (m, k))
+            B = rng.integers(-8, 9, (n, k) if tb else (k, n)).astype(np.float64) if integer else \
+                rng.standard_normal((n, k) if tb else (k, n))
+            dA, dB = ctx.upload(A), ctx.upload(B)
+            dC = ctx.malloc(m * n * 8)
+            ctx.run(D.cmd_gemm(dA, dB, dC, m, n, k, trans_a=ta, trans_b=tb, dtype=_ffi.F64))
+            got = ctx.d2h(dC, (m, n), dtype=np.float64)
+            for p in (dA, dB, dC):
+                ctx.free(p)
+            want = (A.T if ta else A) @ (B.T if tb else B)
+            if integer:
+                assert np.array_equal(got, want), f"integer dgemm {m}x{k}x{n} ta={ta} tb={tb}"
+            else:
+                assert rel_frobenius(got, want) <= 1e-13, f"dgemm {m}x{k}x{n} ta={ta} tb={tb}"
+
+
+def test_batched_matmul_float64(ctx):
+    from gorgonia_amd import _ffi
+    rng = np.random.default_rng(18)
+    A, B = rng.standard_normal((5, 40, 24)), rng.standard_normal((5, 24, 36))
+    dA, dB, dC = ctx.upload(A), ctx.upload(B), ctx.malloc(5 * 40 * 36 * 8)
+    ctx.run(D.cmd_gemm(dA, dB, dC, 40, 36, 24, batch=5, stride_a=40 * 24, stride_b=24 * 36, stride_c=40 * 36,
+                       dtype=_ffi.F64))
+    got = ctx.d2h(dC, (5, 40, 36), dtype=np.float64)
+    for p in (dA, dB, dC):
+        ctx.free(p)
+    assert rel_frobenius(got, A @ B) <= 1e-13
