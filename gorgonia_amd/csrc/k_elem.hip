@@ -120,6 +120,92 @@ __device__ __forceinline__ double tanh_f64_for_f32(double x) {
   return copysign(r, x);
 }
 
+// ---- float32 sigmoid / tanh without float64 ---------------------------------------
+// The float64 forms above are within half an ulp but cost two quarter-rate
+// conversions, a float64 reciprocal and ~20 half-rate FMAs per element, which
+// makes a streaming kernel ALU-bound on this part.  These stay in float32 and
+// within 2 ulp of the correctly rounded result (measured: the dense sweep in
+// the GPU tests), and leave the kernels memory-bound.
+//
+// exp(t) = 2^n * (1 + q): n = round(t / ln2) through the 1.5*2^23 shift (the
+// integer also sits in the low mantissa bits), Cody-Waite reduction with a
+// short-mantissa ln2 high part so that n*ln2_hi is exact, and
+// exp(r) - 1 = r + r^2 P(r) with the classic degree-5 float32 coefficients.
+struct ExpF { float q; int n; };
+
+__device__ __forceinline__ ExpF expf_parts(float t) {
+  const float kShift = 12582912.0f;  // 1.5 * 2^23
+  const float shifted = __builtin_fmaf(t, 1.44269504088896341f, kShift);
+  const float nf = shifted - kShift;
+  float r = __builtin_fmaf(-nf, 0.693145751953125f, t);
+  r = __builtin_fmaf(-nf, 1.428606765330187e-06f, r);
+  float p = 1.9875691500e-4f;
+  p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+  p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+  p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+  p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+  p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+  ExpF e;
+  e.q = __builtin_fmaf(r * r, p, r);
+  e.n = __float_as_int(shifted) - __float_as_int(kShift);
+  return e;
+}
+
+// 1/d to about half an ulp (hardware estimate + one Newton step), then corrected
+// for `derr`, the rounding error of d itself: 1/(d + derr) = r - r^2 derr.
+__device__ __forceinline__ float rcp_f32_comp(float d, float derr) {
+  float r = __builtin_amdgcn_rcpf(d);
+  r = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+  return __builtin_fmaf(-(r * r), derr, r);
+}
+
+// sigmoid with the reference's cut-offs (math_nooptim.go:36-44): with
+// e = exp(-|x|) <= 1, 1/(1+e) for x >= 0 and e/(1+e) for x < 0.  e and 1+e are
+// carried as (high, low) pairs and the quotient gets one residual correction,
+// which leaves the polynomial's own error (about 0.3 ulp) plus the final
+// rounding: within 1 ulp of the correctly rounded value over the dense sweep.
+__device__ __forceinline__ float sigmoid_f32_fast(float x) {
+  const ExpF p = expf_parts(-fabsf(x));
+  const float t = 1.0f + p.q;
+  const float tl = p.q - (t - 1.0f);           // exact: |q| < 1
+  const float e_hi = ldexpf(t, p.n);           // denormal below exp(-87.3), rounded once
+  const float e_lo = ldexpf(tl, p.n);
+  const float d_hi = 1.0f + e_hi;
+  const float d_lo = (e_hi - (d_hi - 1.0f)) + e_lo;
+  float r = __builtin_amdgcn_rcpf(d_hi);
+  r = __builtin_fmaf(__builtin_fmaf(-d_hi, r, 1.0f), r, r);
+  const bool neg = x < 0.0f;
+  const float num_hi = neg ? e_hi : 1.0f, num_lo = neg ? e_lo : 0.0f;
+  const float q0 = num_hi * r;
+  const float rem = __builtin_fmaf(-q0, d_hi, num_hi);          // exact remainder of the first quotient
+  float s = __builtin_fmaf((rem + num_lo) - q0 * d_lo, r, q0);
+  s = x < -88.0f ? 0.0f : s;
+  s = x > 15.0f ? 1.0f : s;
+  return s;                                    // NaN fails every compare and propagates
+}
+
+// tanh: below 0.55 an odd polynomial x + x^3 R(x^2) (R fitted on [0, 0.56^2],
+// approximation error 0.07 ulp); above it 1 - 2/(e^(2|x|) + 1), where the result
+// is at least 0.5 and the subtraction costs no accuracy.
+__device__ __forceinline__ float tanh_f32_fast(float x) {
+  const float ax = fabsf(x);
+  const float s = ax * ax;
+  float R = 0.0024976127315312624f;
+  R = __builtin_fmaf(R, s, -0.008506525307893753f);
+  R = __builtin_fmaf(R, s, 0.02181374467909336f);
+  R = __builtin_fmaf(R, s, -0.05396425351500511f);
+  R = __builtin_fmaf(R, s, 0.133333221077919f);
+  R = __builtin_fmaf(R, s, -0.3333333432674408f);
+  const float small = __builtin_fmaf(ax * s, R, ax);
+  const float a = (ax > 10.0f ? 10.0f : ax) * 2.0f;   // tanh(10) rounds to 1; NaN stays NaN
+  const ExpF p = expf_parts(a);
+  const float e = ldexpf(1.0f + p.q, p.n);
+  const float d = e + 1.0f;
+  const float r = rcp_f32_comp(d, 1.0f - (d - e));
+  const float large = __builtin_fmaf(-2.0f, r, 1.0f);
+  return copysignf(ax < 0.55f ? small : large, x);
+}
+
 template <int FN>
 __device__ __forceinline__ float unary_apply(float x) {
   if constexpr (FN == GH_ABS) return fabsf(x);
@@ -137,11 +223,9 @@ __device__ __forceinline__ float unary_apply(float x) {
   else if constexpr (FN == GH_INVERSE) return 1.0f / x;
   else if constexpr (FN == GH_INVSQRT) return 1.0f / sqrtf(x);
   else if constexpr (FN == GH_CUBE) return x * x * x;
-  else if constexpr (FN == GH_TANH) return (float)tanh_f64_for_f32((double)x); else if constexpr (FN == GH_SIGMOID) {
-    if (x < -88.0f) return 0.0f;
-    if (x > 15.0f) return 1.0f;
-    return (float)rcp_f64_fast(1.0 + exp_f64_fast((double)(-x)));  // NaN propagates
-  } else if constexpr (FN == GH_LOG1P) return (float)log1p((double)x);
+  else if constexpr (FN == GH_TANH) return tanh_f32_fast(x);
+  else if constexpr (FN == GH_SIGMOID) return sigmoid_f32_fast(x);
+  else if constexpr (FN == GH_LOG1P) return (float)log1p((double)x);
   else if constexpr (FN == GH_EXPM1) return (float)expm1((double)x);
   else {  // softplus
     if (x < -103.0f) return 0.0f;
