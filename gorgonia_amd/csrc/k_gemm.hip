@@ -284,26 +284,29 @@ __device__ __forceinline__ void mfma_tile_loop(float* lds, LA& la, LB& lb, const
     }
     const float* a_s = As + cur * (BK * SA) + wm + lr;
     const float* b_s = Bs + cur * (BK * SB) + wn + lr;
-    // operand fragments are fetched one k-step ahead of the MFMAs that use them
-    float af[2][TM], bf[2][TN];
+    // operand fragments are fetched kAhead k-steps ahead of the MFMAs that use
+    // them (an LDS read outlasts one MFMA); the scheduling barriers keep the
+    // compiler from sinking the reads back to their uses
+    constexpr int kSteps = BK / 2, kAhead = (TM * TN >= 4) ? 2 : 4, kRing = 8;
+    float af[kRing][TM], bf[kRing][TN];
+    auto fetch = [&](int st) {
 #pragma unroll
-    for (int a = 0; a < TM; a++) af[0][a] = a_s[lk * SA + a * 32];
+      for (int a = 0; a < TM; a++) af[st % kRing][a] = a_s[(2 * st + lk) * SA + a * 32];
 #pragma unroll
-    for (int b = 0; b < TN; b++) bf[0][b] = b_s[lk * SB + b * 32];
+      for (int b = 0; b < TN; b++) bf[st % kRing][b] = b_s[(2 * st + lk) * SB + b * 32];
+    };
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 2) {
-      const int cb = (kk >> 1) & 1, nb = cb ^ 1;
-      if (kk + 2 < BK) {
+    for (int st = 0; st < kAhead && st < kSteps; st++) fetch(st);
 #pragma unroll
-        for (int a = 0; a < TM; a++) af[nb][a] = a_s[(kk + 2 + lk) * SA + a * 32];
-#pragma unroll
-        for (int b = 0; b < TN; b++) bf[nb][b] = b_s[(kk + 2 + lk) * SB + b * 32];
-      }
+    for (int st = 0; st < kSteps; st++) {
+      if (st + kAhead < kSteps) fetch(st + kAhead);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int a = 0; a < TM; a++)
 #pragma unroll
         for (int b = 0; b < TN; b++)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cb][a], bf[cb][b], acc[a][b], 0, 0, 0);
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[st % kRing][a], bf[st % kRing][b], acc[a][b], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (more) {
       la.store(As + (cur ^ 1) * (BK * SA));
