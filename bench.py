@@ -136,9 +136,9 @@ def bench_linalg(ctx, iters):
 # (KiB per dispatch; FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0, the factors a
 # 64 MiB device copy in the same runs gives).
 MEASURED_TRAFFIC_BYTES = {
-    "conv0": (2 * 295.9 + 12544.0) * 1024,
-    "conv1": (2 * 4508.5 + 6784.0) * 1024,
-    "conv2": (2 * 4073.0 + 6272.0 + 2 * 3156.5 + 3360.0) * 1024,
+    "conv0": (2 * 284.3 + 12544.0) * 1024,
+    "conv1": (2 * 4496.5 + 6784.0) * 1024,
+    "conv2": (2 * 4069.0 + 6272.0 + 2 * 3160.0 + 3360.0) * 1024,
 }
 
 CONVNET_LAYERS = [  # (name, B-relative shape) of configuration 4
