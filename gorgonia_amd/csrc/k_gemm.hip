@@ -552,6 +552,11 @@ struct Conv3Geom {
   int CP;          // floats per channel plane of the patch (R * PW)
   int K;           // C * 9
   int nchunks;     // ceil(C / CC)
+  // Wide images: a block's BN pixels are a TH x TW rectangle of one image
+  // instead of BN consecutive flattened pixels, and the patch is the
+  // (TH+2) x (TW+2) window under it (PW, R, CP then describe that window).
+  // TW == 0: the row-stacked layout above.
+  int TH, TW, tiles_x, tiles_y;
 };
 
 template <int BM, int BN, int CC, int WAVES_M, int PMAX, bool VEC, class SC>
@@ -580,13 +585,29 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
   const int plane = g.oh * g.ow;
   const int HW = g.H * g.W;
 
-  // padded-row window of this block's pixels
+  // patch rows: the padded-row window of this block's pixels, or in the tiled
+  // layout the TH+2 input rows under the tile
+  const bool tiled = g.TW > 0;
+  int tb = 0, oy0 = 0, ox0 = 0;   // tiled: image, first output row / column of the tile
+  if (tiled) {
+    const int t = blockIdx.x;
+    const int tx = t % g.tiles_x, ty = (t / g.tiles_x) % g.tiles_y;
+    tb = t / (g.tiles_x * g.tiles_y);
+    oy0 = ty * g.TH;
+    ox0 = tx * g.TW;
+  }
   const int b_lo = n0 / plane;
   const int gp_lo = b_lo * g.Hp + (n0 - b_lo * plane) / g.ow;
   for (int r = threadIdx.x; r < g.R; r += kThreads) {
-    const int gpr = gp_lo + r;
-    const int b = gpr / g.Hp;
-    const int iy = gpr - b * g.Hp - g.pad;
+    int b, iy;
+    if (tiled) {
+      b = tb;
+      iy = oy0 + r - g.pad;
+    } else {
+      const int gpr = gp_lo + r;
+      b = gpr / g.Hp;
+      iy = gpr - b * g.Hp - g.pad;
+    }
     rowoff[r] = (b < g.B && iy >= 0 && iy < g.H) ? (b * g.C * g.H + iy) * g.W : -1;
   }
   __syncthreads();
@@ -605,7 +626,7 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
       const int c = e / g.CP;
       const int rem = e - c * g.CP;
       const int r = rem / g.PW;
-      const int ix = rem - r * g.PW - g.pad;
+      const int ix = ox0 + rem - r * g.PW - g.pad;
       const int ro = rowoff[r];
       if (ro >= 0 && ix >= 0 && ix < g.W) src = c * HW + ro + ix;
     }
@@ -624,16 +645,26 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
     wdst[j] = (q * 4) * SA + row;
   }
 
-  // per-lane pixel bases inside the patch (one per MFMA column group)
-  int pbase[TN];
+  // per-lane pixel bases inside the patch (one per MFMA column group) and the
+  // flattened index of that pixel in y (-1: outside the image)
+  int pbase[TN], jout[TN];
 #pragma unroll
   for (int t = 0; t < TN; t++) {
-    int j = n0 + wn + t * 32 + lr;
-    j = j < g.P ? j : g.P - 1;
-    const int b = j / plane;
-    const int rem = j - b * plane;
-    const int oy = rem / g.ow, ox = rem - oy * g.ow;
-    pbase[t] = (b * g.Hp + oy - gp_lo) * g.PW + ox + lk * (CC / 2) * g.CP;
+    if (tiled) {
+      const int n = wn + t * 32 + lr;
+      const int ty = n / g.TW, tx = n - ty * g.TW;
+      const int oy = oy0 + ty, ox = ox0 + tx;
+      jout[t] = (oy < g.oh && ox < g.ow) ? tb * plane + oy * g.ow + ox : -1;
+      pbase[t] = ty * g.PW + tx + lk * (CC / 2) * g.CP;
+    } else {
+      int j = n0 + wn + t * 32 + lr;
+      jout[t] = j < g.P ? j : -1;
+      j = j < g.P ? j : g.P - 1;
+      const int b = j / plane;
+      const int rem = j - b * plane;
+      const int oy = rem / g.ow, ox = rem - oy * g.ow;
+      pbase[t] = (b * g.Hp + oy - gp_lo) * g.PW + ox + lk * (CC / 2) * g.CP;
+    }
   }
   const int abase = lk * KHALF * SA + wm + lr;
 
@@ -723,10 +754,8 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
     for (int v = 0; v < 16; v++) {
       const int i = m0 + wm + a * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
 #pragma unroll
-      for (int t = 0; t < TN; t++) {
-        const int j = n0 + wn + t * 32 + lr;
-        if (i < g.F && j < g.P) sc.put(i, j, act_apply(acc[a][t][v], act, alpha));
-      }
+      for (int t = 0; t < TN; t++)
+        if (i < g.F && jout[t] >= 0) sc.put(i, jout[t], act_apply(acc[a][t][v], act, alpha));
     }
 }
 
@@ -1336,7 +1365,8 @@ template <int BM, int BN, int CC, int WAVES_M, int PMAX>
 int launch_conv3_cfg(gh_ctx* ctx, const gh_cmd& c, Conv3Geom g, int splits, size_t lds_bytes) {
   const bool vec = al16(c.ptr[1]) && g.K % 4 == 0;
   const ConvTail tail = conv_tail(c);
-  const dim3 grid((g.P + BN - 1) / BN, (g.F + BM - 1) / BM, splits);
+  const unsigned pixel_tiles = g.TW > 0 ? (unsigned)(g.B * g.tiles_y * g.tiles_x) : (unsigned)((g.P + BN - 1) / BN);
+  const dim3 grid(pixel_tiles, (g.F + BM - 1) / BM, splits);
   const float* x = (const float*)(uintptr_t)c.ptr[0];
   const float* w = (const float*)(uintptr_t)c.ptr[1];
   float* y = (float*)(uintptr_t)c.ptr[2];
@@ -1386,13 +1416,36 @@ int try_launch_conv3_cc(gh_ctx* ctx, const gh_cmd& c) {
     if (atoi(env) == 0) { BM = F > 64 ? 128 : 64; BN = 128; }
     if (atoi(env) == 2 && F > 64) { BM = 128; BN = 64; }
   }
+  g.TH = g.TW = g.tiles_x = g.tiles_y = 0;
   g.R = conv3_patch_rows(g, BN);
   g.CP = g.R * g.PW;
+  int64_t pixel_tiles = cdiv(g.P, BN);
+  // Wide rows: BN consecutive pixels touch only one or two image rows, and the
+  // row-stacked patch would hold whole rows for them.  Cut the image into
+  // TH x TW rectangles instead (the shape that wastes the fewest pixels on
+  // partial tiles, then the smallest patch) and stage the window under each.
+  if (g.ow >= 64 && !getenv("GORGONIA_HIP_CONV_GATHER_WIDE") && !getenv("GORGONIA_HIP_CONV_TILE")) {
+    if (F <= 32) { BM = 32; BN = 128; }
+    int best_th = 0, best_tw = 0;
+    int64_t best_tiles = 0, best_patch = 0;
+    for (int tw = 4; tw <= BN; tw *= 2) {
+      const int th = BN / tw;
+      const int64_t tiles = cdiv(g.oh, th) * cdiv(g.ow, tw);
+      const int64_t patch = (int64_t)(th + 2) * (tw + 2);
+      if (!best_tw || tiles < best_tiles || (tiles == best_tiles && patch < best_patch)) {
+        best_th = th; best_tw = tw; best_tiles = tiles; best_patch = patch;
+      }
+    }
+    g.TH = best_th; g.TW = best_tw;
+    g.tiles_x = (int)cdiv(g.ow, g.TW); g.tiles_y = (int)cdiv(g.oh, g.TH);
+    g.PW = g.TW + 2; g.R = g.TH + 2; g.CP = g.R * g.PW;
+    pixel_tiles = (int64_t)B * g.tiles_x * g.tiles_y;
+  }
   const size_t lds = ((size_t)CC * 9 * (BM + 2) + (size_t)CC * g.CP + g.R) * 4;
   if (lds > 64 * 1024) return -1;
   const int per_thread = (CC * g.CP + kThreads - 1) / kThreads;  // patch elements each thread stages
-  if (per_thread > 16) return -1;  // wide images: the gather kernel does better
-  const int64_t blocks = cdiv(F, BM) * cdiv(g.P, BN);
+  if (per_thread > 16) return -1;  // the gather kernel does better
+  const int64_t blocks = cdiv(F, BM) * pixel_tiles;
   int splits = 1;
   if (const char* env = getenv("GORGONIA_HIP_CONV_SPLITS")) splits = atoi(env);
   else {
@@ -1405,6 +1458,9 @@ int try_launch_conv3_cc(gh_ctx* ctx, const gh_cmd& c) {
 #define GH_CONV3(BM_, BN_)                                                                        \
   (per_thread <= 8 ? launch_conv3_cfg<BM_, BN_, CC, 2, 8>(ctx, c, g, splits, lds)                 \
                    : launch_conv3_cfg<BM_, BN_, CC, 2, 16>(ctx, c, g, splits, lds))
+  if (BM == 32)
+    return per_thread <= 8 ? launch_conv3_cfg<32, 128, CC, 1, 8>(ctx, c, g, splits, lds)
+                           : launch_conv3_cfg<32, 128, CC, 1, 16>(ctx, c, g, splits, lds);
   if (BN == 64 && BM == 128) return GH_CONV3(128, 64);
   if (BN == 64) return GH_CONV3(64, 64);
   if (BM == 128) return GH_CONV3(128, 128);

@@ -64,6 +64,11 @@ CONV_CASES = [
     (2, 16, 52, 52, 32, 3, 3, (1, 1), (1, 1), (1, 1)),
     (2, 256, 13, 13, 512, 3, 3, (1, 1), (1, 1), (1, 1)),
     (2, 1024, 13, 13, 425, 1, 1, (0, 0), (1, 1), (1, 1)),
+    # wide rows: the LDS kernel's rectangular-tile layout, partial tiles on both axes
+    (1, 8, 71, 75, 16, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (2, 16, 66, 68, 40, 3, 3, (0, 0), (1, 1), (1, 1)),
+    (1, 8, 104, 104, 64, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (1, 16, 70, 130, 96, 3, 3, (1, 1), (1, 1), (1, 1)),
 ]
 
 
@@ -136,7 +141,8 @@ def gpu_bn(ctx, x, mean, var, gamma, beta, eps):
 # shapes that reach each convolution kernel: the direct one (C <= 4), the
 # LDS-staged 3x3 one with and without split-K, the gather one (1x1)
 TAIL_CASES = [(2, 3, 20, 22, 16, 3, 1), (3, 1, 28, 28, 32, 3, 1), (2, 4, 9, 9, 5, 3, 0),
-              (2, 16, 26, 26, 32, 3, 1), (2, 256, 13, 13, 64, 3, 1), (2, 64, 13, 13, 40, 1, 0)]
+              (2, 16, 26, 26, 32, 3, 1), (2, 256, 13, 13, 64, 3, 1), (2, 64, 13, 13, 40, 1, 0),
+              (1, 16, 60, 72, 32, 3, 1), (1, 64, 52, 80, 72, 3, 1)]
 
 
 @pytest.mark.parametrize("cfg", TAIL_CASES)
