@@ -33,6 +33,25 @@
  *                                            math32 (not vendored).  Oracle is
  *                                            float64 libm rounded once; the
  *                                            2-ulp budget covers the gap.
+ *   batch norm backward                    - nn_amd64_test.go ExpectedInputGrad
+ *                                            goldens; finite differences of the
+ *                                            training forward
+ *   solver steps (vanilla, RMSProp, Adam)  - solvers_test.go:100-143 closed form,
+ *                                            solvers_test.go:355-437 Adam golden
+ *   max-pool backward                      - nn_test.go:140-193 example, brute
+ *                                            force on tied inputs, the 3072-float
+ *                                            golden's windows
+ *   conv2d backward (image, filter)        - the reference's tests are only
+ *                                            differential (tape vs lisp machine):
+ *                                            pinned by the float64 definition,
+ *                                            adjoint identities against the
+ *                                            pinned forward pass, finite
+ *                                            differences, integer-exact cases
+ *   softmax backward                       - no reference golden: Jacobian and
+ *                                            finite differences of the pinned
+ *                                            forward pass.  tensor.SoftMaxB
+ *                                            itself is not vendored: PARITY
+ *                                            UNPINNED bit-for-bit.
  */
 #include <math.h>
 #include <stdint.h>
