@@ -224,6 +224,9 @@ static int dispatch(gh_ctx* ctx, const gh_cmd& c) {
     case GH_OP_BN_BWD: return gh_launch_bn_bwd(ctx, c);
     case GH_OP_SOFTMAX_BWD: return gh_launch_softmax_bwd(ctx, c);
     case GH_OP_SOLVER_STEP: return gh_launch_solver_step(ctx, c);
+    case GH_OP_RAND_UNIFORM: return gh_launch_rand_uniform(ctx, c);
+    case GH_OP_DROPOUT: return gh_launch_dropout(ctx, c);
+    case GH_OP_DROPOUT_BWD: return gh_launch_dropout_bwd(ctx, c);
   }
   return GH_ENOFUNC;
 }

@@ -58,6 +58,9 @@ int gh_launch_bn_train(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_bn_bwd(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_softmax_bwd(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_solver_step(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_rand_uniform(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_dropout(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_dropout_bwd(gh_ctx* ctx, const gh_cmd& c);
 
 static inline uint32_t gh_fn(uint32_t flags) { return flags & 0xffu; }
 static inline uint32_t gh_mode(uint32_t flags) { return (flags >> 8) & 0xfu; }

@@ -146,6 +146,17 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (fn == GH_SOLVER_ADAM && !c.ptr[3]) return bad("Adam second-moment cache is null");
       if (c.dim[0] < 0) return bad("negative size");
       return GH_OK;
+    case GH_OP_RAND_UNIFORM:
+      if (!c.ptr[0]) return bad("null operand");
+      if (c.dim[0] < 0) return bad("negative size");
+      if (c.ptr[1] & 7) return bad("rand: state must be 8-byte aligned");
+      return GH_OK;
+    case GH_OP_DROPOUT:
+    case GH_OP_DROPOUT_BWD:
+      if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
+      if (c.dim[0] < 0) return bad("negative size");
+      if (!(c.f[0] >= 0.0f && c.f[0] < 1.0f)) return bad("dropout: probability must be in [0, 1)");
+      return GH_OK;
     case GH_OP_RELU:
     case GH_OP_LEAKY_RELU:
       if (!c.ptr[0] || !c.ptr[1]) return bad("null operand");

@@ -401,6 +401,37 @@ __global__ __launch_bounds__(kBlock) void k_solver_step(float* __restrict__ w, c
   }
 }
 
+// ---- dropout and its random source -------------------------------------------------------
+// Counter-based: element i is a pure function of (seed, offset + i), so the
+// numbers do not depend on the launch shape and a CPU twin can reproduce them.
+__global__ __launch_bounds__(kBlock) void k_rand_uniform(float* __restrict__ out, int64_t n, uint64_t seed,
+                                                         uint64_t offset, const uint64_t* __restrict__ state) {
+  if (state) offset = *state;
+  const uint64_t base = seed * 0xD1342543DE82EF95ull;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    uint64_t z = base + (offset + (uint64_t)i + 1) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z = z ^ (z >> 31);
+    out[i] = (float)(uint32_t)(z >> 40) * 5.9604644775390625e-08f;
+  }
+}
+
+__global__ void k_rand_advance(uint64_t* state, uint64_t n) { *state += n; }
+
+__global__ __launch_bounds__(kBlock) void k_dropout(const float* __restrict__ x, const float* __restrict__ r,
+                                                    float* __restrict__ y, int64_t n, float keep,
+                                                    int identity) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
+    y[i] = identity ? x[i] : (r[i] < keep ? x[i] / keep : 0.0f);
+}
+
+__global__ __launch_bounds__(kBlock) void k_dropout_bwd(const float* __restrict__ y, const float* __restrict__ dy,
+                                                        float* __restrict__ dx, int64_t n, float prob) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
+    dx[i] = (prob != 0.0f && y[i] != 0.0f) ? dy[i] / prob : 0.0f;
+}
+
 // how many workgroups share one channel's reduction
 int bn_groups(int64_t n, int64_t S) {
   // wide planes: two 256-wide strips of every image per workgroup; else 1024 images per workgroup
@@ -525,4 +556,40 @@ int gh_launch_solver_step(gh_ctx* ctx, const gh_cmd& c) {
   else
     hipLaunchKernelGGL((k_solver_step<GH_SOLVER_ADAM>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p);
   return gh_check_hip(ctx, hipGetLastError(), "solver step launch");
+}
+
+static int stream_blocks(gh_ctx* ctx, int64_t n) {
+  int64_t blocks = (n + kBlock - 1) / kBlock;
+  if (blocks > (int64_t)ctx->cu_count * 32) blocks = (int64_t)ctx->cu_count * 32;
+  return (int)(blocks < 1 ? 1 : blocks);
+}
+
+int gh_launch_rand_uniform(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t n = c.dim[0];
+  uint64_t* state = (uint64_t*)(uintptr_t)c.ptr[1];
+  if (n > 0)
+    hipLaunchKernelGGL(k_rand_uniform, dim3(stream_blocks(ctx, n)), dim3(kBlock), 0, ctx->stream,
+                       (float*)(uintptr_t)c.ptr[0], n, (uint64_t)c.dim[1], (uint64_t)c.dim[2], state);
+  if (state && n > 0) hipLaunchKernelGGL(k_rand_advance, dim3(1), dim3(1), 0, ctx->stream, state, (uint64_t)n);
+  return gh_check_hip(ctx, hipGetLastError(), "uniform generator launch");
+}
+
+int gh_launch_dropout(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t n = c.dim[0];
+  if (n == 0) return GH_OK;
+  const int identity = (c.flags & GH_FLAG_BN_EVAL) || c.f[0] == 0.0f;
+  const float keep = (float)(1.0 - (double)c.f[0]);
+  hipLaunchKernelGGL(k_dropout, dim3(stream_blocks(ctx, n)), dim3(kBlock), 0, ctx->stream,
+                     (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[2],
+                     (float*)(uintptr_t)c.ptr[1], n, keep, identity);
+  return gh_check_hip(ctx, hipGetLastError(), "dropout launch");
+}
+
+int gh_launch_dropout_bwd(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t n = c.dim[0];
+  if (n == 0) return GH_OK;
+  hipLaunchKernelGGL(k_dropout_bwd, dim3(stream_blocks(ctx, n)), dim3(kBlock), 0, ctx->stream,
+                     (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                     (float*)(uintptr_t)c.ptr[2], n, c.f[0]);
+  return gh_check_hip(ctx, hipGetLastError(), "dropout backward launch");
 }

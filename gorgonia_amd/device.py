@@ -267,6 +267,18 @@ def cmd_solver_step(kind, w, g, n, par, use, cache=0, cache2=0):
     return make_cmd(_ffi.OP_SOLVER_STEP, fl, (w, g, cache, cache2), (n,), tuple(float(v) for v in par))
 
 
+def cmd_rand_uniform(out, n, seed, offset=0, state=0):
+    return make_cmd(_ffi.OP_RAND_UNIFORM, 0, (out, state), (n, seed, offset))
+
+
+def cmd_dropout(x, y, r, n, prob, training=True):
+    return make_cmd(_ffi.OP_DROPOUT, 0 if training else _ffi.FLAG_BN_EVAL, (x, y, r), (n,), (prob,))
+
+
+def cmd_dropout_bwd(y, dy, dx, n, prob):
+    return make_cmd(_ffi.OP_DROPOUT_BWD, 0, (y, dy, dx), (n,), (prob,))
+
+
 def cmd_has(kind, a, flag, n, dtype=_ffi.F32):
     op = _ffi.OP_HAS_NAN if kind == "nan" else _ffi.OP_HAS_INF
     return make_cmd(op, _ffi.flag_dtype(dtype), (a, flag), (n,))

@@ -14,7 +14,7 @@ from .engine import Engine, EngineError, GhhOp, load_host
 
 (K_ELEMBIN, K_ELEMUNARY, K_BCAST, K_MATMUL, K_MATVEC, K_OUTER, K_BMM, K_CONV2D, K_MAXPOOL, K_BN,
  K_RECTIFY, K_LEAKY, K_SOFTMAX, K_RESHAPE, K_MAXPOOL_DIFF, K_CONV_DIFF_DATA, K_CONV_DIFF_FILTER, K_BN_TRAIN,
- K_BN_DIFF, K_SOFTMAX_DIFF, K_SET, K_SOLVER) = range(22)
+ K_BN_DIFF, K_SOFTMAX_DIFF, K_SET, K_SOLVER, K_RAND_UNIFORM, K_DROPOUT, K_DROPOUT_DIFF) = range(25)
 
 
 class Node:
@@ -233,6 +233,35 @@ def SolverStep(kind, weights, grad, caches=(), eta=0.001, eps=1e-8, l1reg=0.0, l
     use = (1 if l1reg else 0) | (2 if l2reg else 0) | (4 if clip else 0) | (8 if batch > 1 else 0)
     fn = {"vanilla": 0, "rmsprop": 1, "adam": 2}[kind]
     return weights.g.apply(K_SOLVER, [weights, grad] + list(caches), fn=fn, ints=[use], fs=fs)
+
+
+def RandUniform(g, shape, seed, offset=0, counter=None):
+    """The uniform [0, 1) numbers gorgonia.Dropout draws (nn.go:71-77), generated on the
+    device: element i is a function of (seed, offset + i) only.  With `counter` (from
+    NewCounter) the offset lives on the device and moves on by the tensor's size every
+    run, so a replayed tape draws fresh numbers each time."""
+    inputs = [] if counter is None else [counter]
+    return g.apply(K_RAND_UNIFORM, inputs, ints=[int(seed), int(offset)] + [int(d) for d in shape])
+
+
+def NewCounter(g, start=0):
+    """One 8-byte position of a random stream, resident on the device."""
+    return NewTensor(g, np.array([start], dtype=np.uint64).view(np.float64), resident=True)
+
+
+def Dropout(x, prob, rand=None, seed=0, training=True):
+    """gorgonia.Dropout(x, dropProb) (nn.go:71-77, op_dropout.go:107-132):
+    y = r < 1-p ? x/(1-p) : 0 with r uniform in [0, 1).  `rand` supplies the numbers
+    (a node of x's size); without it a device generator seeded with `seed` and its own
+    counter is added to the graph.  The reference seeds from the wall clock."""
+    if rand is None:
+        rand = RandUniform(x.g, x.Shape(), seed, counter=NewCounter(x.g))
+    return x.g.apply(K_DROPOUT, [x, rand], fn=int(training), f0=float(prob))
+
+
+def DropoutDiff(y, grad, prob):
+    """dropoutDiffOp (op_dropout.go:205-238): dx = dy/p where y is non-zero, else 0."""
+    return y.g.apply(K_DROPOUT_DIFF, [y, grad], f0=float(prob))
 
 
 class TapeMachine:

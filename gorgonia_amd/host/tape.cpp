@@ -215,6 +215,20 @@ Status InferShape(const OpSpec& op, const std::vector<const Shape*>& in, Shape* 
       *out = *in[0];
       return Status::OK();
     }
+    case OpKind::RandUniform: {
+      if (in.size() > 1 || (in.size() == 1 && in[0]->TotalSize() != 1)) return bad("RandUniform: at most one counter input");
+      if (op.ints.size() < 2) return bad("RandUniform: seed and offset missing");
+      Shape s(std::vector<int64_t>(op.ints.begin() + 2, op.ints.end()));
+      for (int64_t d : s.d) if (d < 0) return bad("RandUniform: negative dimension");
+      *out = s;
+      return Status::OK();
+    }
+    case OpKind::Dropout:
+    case OpKind::DropoutDiff:
+      if (!need(2) || in[0]->TotalSize() != in[1]->TotalSize()) return bad("Dropout: operand sizes differ");
+      if (!(op.f0 >= 0.0 && op.f0 < 1.0)) return bad("Dropout: probability must be in [0, 1)");
+      *out = *in[0];
+      return Status::OK();
     case OpKind::Reshape: {
       if (!need(1)) return bad("Reshape needs 1 input");
       Shape s(op.ints);
@@ -261,6 +275,9 @@ static std::string op_name(const OpSpec& op) {
     case OpKind::BatchNormDiff: return "batchnorm.diff";
     case OpKind::SoftMaxDiff: return "softmax.diff";
     case OpKind::Set: return "set";
+    case OpKind::RandUniform: return "rand.uniform";
+    case OpKind::Dropout: return "dropout";
+    case OpKind::DropoutDiff: return "dropoutDiff";
     case OpKind::SolverStep: return op.fn == GH_SOLVER_ADAM ? "solver.adam" : op.fn == GH_SOLVER_RMSPROP ? "solver.rmsprop" : "solver.vanilla";
   }
   return "?";
@@ -460,6 +477,32 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       e.Enqueue(c);
       return Status::OK();
     }
+    case OpKind::RandUniform: {
+      if (!in.empty() && in[0]->dt != Dtype::Float64) return bad("RandUniform: the counter must be an 8-byte scalar");
+      gh_cmd c{};
+      c.opcode = GH_OP_RAND_UNIFORM;
+      c.ptr[0] = prealloc.mem;
+      c.ptr[1] = in.empty() ? 0 : in[0]->mem;
+      c.dim[0] = prealloc.shape.TotalSize(); c.dim[1] = op.ints[0]; c.dim[2] = op.ints[1];
+      e.Enqueue(c);
+      return Status::OK();
+    }
+    case OpKind::Dropout:
+    case OpKind::DropoutDiff: {
+      if (in[0]->dt != Dtype::Float32 || in[1]->dt != Dtype::Float32) return bad("Dropout: Unsupported Dtype");
+      gh_cmd c{};
+      c.opcode = op.kind == OpKind::Dropout ? GH_OP_DROPOUT : GH_OP_DROPOUT_BWD;
+      if (op.kind == OpKind::Dropout) {
+        if (!op.fn) c.flags = GH_FLAG_BN_EVAL;
+        c.ptr[0] = in[0]->mem; c.ptr[1] = prealloc.mem; c.ptr[2] = in[1]->mem;
+      } else {
+        c.ptr[0] = in[0]->mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
+      }
+      c.dim[0] = in[0]->shape.TotalSize();
+      c.f[0] = (float)op.f0;
+      e.Enqueue(c);
+      return Status::OK();
+    }
     case OpKind::Set: {
       // prealloc is a's register (the node aliases a); copy b's bytes into it
       const int64_t bytes = in[1]->DataSize() * dtype_size(in[1]->dt);
@@ -490,7 +533,7 @@ Status Graph::Apply(const OpSpec& op, const std::vector<int>& inputs, int* out) 
   Status st = InferShape(op, shapes, &n.shape);
   if (!st.ok()) return st;
   n.id = (int)nodes_.size();
-  n.dt = inputs.empty() ? Dtype::Float32 : nodes_[(size_t)inputs[0]].dt;
+  n.dt = inputs.empty() || op.kind == OpKind::RandUniform ? Dtype::Float32 : nodes_[(size_t)inputs[0]].dt;
   n.op = op;
   n.inputs = inputs;
   if (op.kind == OpKind::Reshape || op.kind == OpKind::Set || op.kind == OpKind::SolverStep) n.alias_of = inputs[0];

@@ -49,9 +49,15 @@ enum class OpKind : int32_t {
   BatchNormDiff = 18,    // batchnormDiffOp (op_nn.go:1834-1943): inputs x, grad, saveMean, saveVar
   SoftMaxDiff = 19,      // softmaxDiffOp (op_softmax.go:184-279): inputs y, grad
   Set = 20,              // gorgonia.Set(a, b): a's value becomes b's (operations.go); inputs a, b
-  SolverStep = 21        // one Step of VanillaSolver / RMSPropSolver / AdamSolver on one weight tensor
+  SolverStep = 21,       // one Step of VanillaSolver / RMSPropSolver / AdamSolver on one weight tensor
                          // (solvers.go:273-870): inputs weights, grad[, cache[, cache2]]; fn = gh_solver,
                          // ints[0] = use mask, fs = the ten constants; the weights are updated in place
+  RandUniform = 22,      // the uniform [0,1) source gorgonia.Dropout draws from (nn.go:71-77), generated on
+                         // the device: ints = seed, offset, shape...; optional input = one 8-byte counter
+                         // (a Float64 scalar used as raw bits) read as the offset and advanced by the size
+  Dropout = 23,          // dropoutOp (op_dropout.go:107-132): inputs x, uniform numbers; f0 = probability,
+                         // fn = 1 while training, 0 for the identity of evaluation
+  DropoutDiff = 24       // dropoutDiffOp (op_dropout.go:205-238): inputs y, grad; f0 = probability
 };
 
 struct OpSpec {

@@ -88,6 +88,9 @@ enum gh_opcode {
   GH_OP_BN_BWD = 21,            /* ops/nn/batchnorm_cuda.go:192-219; CPU op_nn.go:1834-1943    */
   GH_OP_SOFTMAX_BWD = 22,       /* softmaxDiffOp, op_softmax.go:266-279                        */
   GH_OP_SOLVER_STEP = 23,       /* Vanilla/RMSProp/Adam Step on a float32 tensor, solvers.go:273-870 */
+  GH_OP_RAND_UNIFORM = 24,      /* the random source of Dropout (nn.go:71-77), generated on the device */
+  GH_OP_DROPOUT = 25,           /* dropoutOp.do, op_dropout.go:107-132; ops/nn/dropout_cuda.go    */
+  GH_OP_DROPOUT_BWD = 26,       /* dropoutDiffOp, op_dropout.go:205-238                            */
   GH_OP__COUNT
 };
 
@@ -174,6 +177,15 @@ enum gh_unaryfn {
  * BN_BWD      ptr[0]=x ptr[1]=dy ptr[2]=dx ptr[3]=save_mean ptr[4]=save_var
  *             dim[0..2]=B,C,S  f[0]=eps ; BN_EVAL selects dx = dy/sqrt(save_var/n + eps)
  * SOFTMAX_BWD ptr[0]=y ptr[1]=dy ptr[2]=dx        dim[0]=rows dim[1]=cols
+ * RAND_UNIFORM ptr[0]=out [ptr[1]=state]          dim[0]=n dim[1]=seed dim[2]=offset
+ *             float32 in [0,1) with 24 random bits, element i = SplitMix64 output function
+ *             of seed*0xD1342543DE82EF95 + (offset + i + 1)*0x9E3779B97F4A7C15.  With a
+ *             state pointer (one uint64 on the device) the offset is read from it and n
+ *             is added to it afterwards, so a replayed segment draws fresh numbers
+ * DROPOUT     ptr[0]=x ptr[1]=y ptr[2]=r (uniform numbers, one per element)  dim[0]=n
+ *             f[0]=drop probability ; y = r < 1-p ? x/(1-p) : 0 ; BN_EVAL or p == 0: y = x
+ * DROPOUT_BWD ptr[0]=y ptr[1]=dy ptr[2]=dx         dim[0]=n f[0]=drop probability
+ *             dx = (p != 0 && y != 0) ? dy/p : 0   (the reference divides by p)
  * SOLVER_STEP ptr[0]=weights ptr[1]=grad [ptr[2]=cache (RMSProp cache / Adam m) ptr[3]=Adam v]
  *             dim[0]=n ; flags: FN = gh_solver, MODE = use mask (1 l1reg, 2 l2reg, 4 clip,
  *             8 batch) ; f[0]=eta f[1]=eps f[2]=l1reg f[3]=l2reg f[4]=clip f[5]=1/batch

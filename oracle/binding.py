@@ -340,6 +340,28 @@ def solver_step(kind, w, g, c1=None, c2=None, **kw):
     return w, g, c1, c2
 
 
+def dropout(x, r, prob, training=True):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    r = np.ascontiguousarray(r, dtype=np.float32)
+    y = np.empty_like(x)
+    lib().oracle_dropout_f32(_p(x), _p(r), _p(y), C.c_int64(x.size), C.c_double(prob), C.c_int(int(training)))
+    return y
+
+
+def dropout_bwd(y, dy, prob):
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    dx = np.empty_like(y)
+    lib().oracle_dropout_bwd_f32(_p(y), _p(dy), _p(dx), C.c_int64(y.size), C.c_double(prob))
+    return dx
+
+
+def uniform01(n, seed, offset=0):
+    out = np.empty(n, np.float32)
+    lib().oracle_uniform01_f32(_p(out), C.c_int64(n), C.c_uint64(seed), C.c_uint64(offset))
+    return out
+
+
 def has_nan(a):
     a = np.ascontiguousarray(a, dtype=np.float32)
     return bool(lib().oracle_has_nan_f32(_p(a), C.c_int64(a.size)))

@@ -47,6 +47,9 @@
  *                                            adjoint identities against the
  *                                            pinned forward pass, finite
  *                                            differences, integer-exact cases
+ *   dropout forward / backward             - op_dropout_test.go:14-102 goldens with
+ *                                            the injected random sequence
+ *   uniform01 (the engine's own generator) - equals gorgonia_amd/synth.py's stream
  *   softmax backward                       - no reference golden: Jacobian and
  *                                            finite differences of the pinned
  *                                            forward pass.  tensor.SoftMaxB
@@ -921,6 +924,44 @@ EXPORT void oracle_solver_step_f32(int kind, float* w, float* g, float* c1, floa
       w[i] = w[i] + mh;
       g[i] = g2;
     }
+  }
+}
+
+/* ================================================================== */
+/* Dropout: dropoutOp.do (op_dropout.go:107-132) and dropoutDiffOp     */
+/* (op_dropout.go:205-238).  r holds the values the op's random source */
+/* returns, one per element in order.  Outputs that are not kept stay  */
+/* at the zero a fresh tensor holds.  The gradient divides by the DROP */
+/* probability, as the reference does.                                 */
+/* ================================================================== */
+EXPORT void oracle_dropout_f32(const float* x, const float* r, float* y, int64_t n, double prob,
+                               int training) {
+  int64_t i;
+  if (prob == 0.0 || !training) { for (i = 0; i < n; i++) y[i] = x[i]; return; }
+  const float keep = (float)(1.0 - prob);
+  for (i = 0; i < n; i++) y[i] = r[i] < keep ? x[i] / keep : 0.0f;
+}
+
+EXPORT void oracle_dropout_bwd_f32(const float* y, const float* dy, float* dx, int64_t n, double prob) {
+  int64_t i;
+  const float p = (float)prob;
+  for (i = 0; i < n; i++) dx[i] = (prob != 0.0 && y[i] != 0.0f) ? dy[i] / p : 0.0f;
+}
+
+/* Counter-based uniform source in [0, 1) with 24 random bits: element i of
+ * stream (seed, offset) is SplitMix64's output function applied to
+ * seed*0xD1342543DE82EF95 + (offset + i + 1)*0x9E3779B97F4A7C15, top 24 bits.
+ * Not the reference's generator (that one is seeded from the wall clock,
+ * nn.go:72); this is the engine's own, stated here so the device can be
+ * checked bit for bit. */
+EXPORT void oracle_uniform01_f32(float* out, int64_t n, uint64_t seed, uint64_t offset) {
+  int64_t i;
+  for (i = 0; i < n; i++) {
+    uint64_t z = seed * 0xD1342543DE82EF95ull + (offset + (uint64_t)i + 1) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z = z ^ (z >> 31);
+    out[i] = (float)(z >> 40) * 5.9604644775390625e-08f;
   }
 }
 

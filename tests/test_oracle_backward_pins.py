@@ -276,3 +276,29 @@ def test_vanilla_step_is_w_minus_eta_g_with_the_options_in_order():
     gg = gg * (f(1) / f(4))
     gg = np.clip(gg, f(-0.5), f(0.5))
     assert np.array_equal(w2, (w + gg * f(-0.05)).astype(f))
+
+
+# ---- dropout -------------------------------------------------------------------------
+
+@pytest.mark.parametrize("prob,expected,input_grad", [
+    (0.2, [1.25, 1.25, 1.25, 0.0, 0.0], [1, 1, 1, 0, 0]),
+    (0.5, [2.0, 2.0, 0.0, 0.0, 0.0], [0.4, 0.4, 0, 0, 0]),
+])
+def test_dropout_goldens(prob, expected, input_grad):
+    """op_dropout_test.go:14-102 TestDropoutAll, Float32 rows: x = ones(5), the random source
+    returns 0, 0.2, 0.5, 0.8, 1.0, cost = Mean(y) so the output gradient is 0.2 everywhere."""
+    x = np.ones(5, np.float32)
+    r = np.array([0.0, 0.2, 0.5, 0.8, 1.0], np.float32)
+    y = O.dropout(x, r, prob)
+    assert np.array_equal(y, np.array(expected, np.float32))
+    dx = O.dropout_bwd(y, np.full(5, 0.2, np.float32), prob)
+    assert np.array_equal(dx, np.array(input_grad, np.float32))
+    assert np.array_equal(O.dropout(x, r, 0.0), x) and np.array_equal(O.dropout(x, r, prob, training=False), x)
+
+
+def test_uniform_source_is_the_synthetic_stream():
+    from gorgonia_amd import synth
+    assert np.array_equal(O.uniform01(1000, 77), synth.uniform01(77, (1000,)))
+    a = O.uniform01(1 << 16, 5)
+    assert np.array_equal(O.uniform01(100, 5, offset=1000), a[1000:1100])
+    assert 0.0 <= a.min() and a.max() < 1.0 and abs(a.mean() - 0.5) < 0.01
