@@ -465,7 +465,7 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
                                                          float* __restrict__ C, int M, int N, int K,
                                                          int lda, int ldb, int ldc, int act,
                                                          float alpha, int vec_a) {
-  constexpr int G = 4;                       // k-chunks whose loads are in flight together
+  constexpr int G = 5;                       // k-chunks per group; two groups of loads are in flight
   constexpr int HALF = WV / 2;
   __shared__ float part[HALF * 1024];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -490,15 +490,17 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
 #pragma unroll
     for (int t = 0; t < 8; t++) b[t] = (n < N && k0 + t < K) ? B[(int64_t)(k0 + t) * ldb + n] : 0.f;
   };
-
-  f32x16 acc;
-#pragma unroll
-  for (int v = 0; v < 16; v++) acc[v] = 0.f;
-  for (int c = wave; c < nchunks; c += G * WV) {
-    float a[G][8], b[G][8];
+  // group = chunks c, c + WV, ... (G of them); the chunk order per wavefront is
+  // fixed, so the sum is the same whatever the grouping
+  auto load_group = [&](int c, float (&a)[G][8], float (&b)[G][8]) {
 #pragma unroll
     for (int g = 0; g < G; g++)
       if (c + g * WV < nchunks) load(c + g * WV, a[g], b[g]);
+  };
+  f32x16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; v++) acc[v] = 0.f;
+  auto mfma_group = [&](int c, float (&a)[G][8], float (&b)[G][8]) {
 #pragma unroll
     for (int g = 0; g < G; g++)
       if (c + g * WV < nchunks) {
@@ -506,6 +508,21 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
         for (int t = 0; t < 8; t++)
           acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[g][t], b[g][t], acc, 0, 0, 0);
       }
+  };
+
+  // The MFMAs of one group form a dependent chain of 8*G*64 cycles; the next
+  // group's loads are issued before it so their latency runs underneath.
+  float a0[G][8], b0[G][8], a1[G][8], b1[G][8];
+  int c0 = wave;
+  if (c0 < nchunks) load_group(c0, a0, b0);
+  while (c0 < nchunks) {
+    const int c1 = c0 + G * WV;
+    if (c1 < nchunks) load_group(c1, a1, b1);
+    mfma_group(c0, a0, b0);
+    if (c1 >= nchunks) break;
+    c0 = c1 + G * WV;
+    if (c0 < nchunks) load_group(c0, a0, b0);
+    mfma_group(c1, a1, b1);
   }
   // upper half of the wavefronts hands its tiles to the lower half, then the
   // HALF sums are added in wavefront order
@@ -557,7 +574,27 @@ struct Conv3Geom {
   // (TH+2) x (TW+2) window under it (PW, R, CP then describe that window).
   // TW == 0: the row-stacked layout above.
   int TH, TW, tiles_x, tiles_y;
+  // ceil(2^32 / d) for d = CP, PW, Hp: the staging decode divides by them once
+  // per element (see div_magic)
+  unsigned mCP, mPW, mHp;
+  // Row-stacked layout: a block owns BNU <= BN consecutive pixels (BNU = BN
+  // unless the tile is cut to whole output rows for the fused pooling).
+  int BNU;
+  // Fused 2x2/stride-2 max-pool: pool != 0, y has the pooled shape (ph x pw per
+  // plane) and every block's pixels form whole pooling windows - row-stacked: a
+  // multiple of two rows starting on an even row (oh even) or whole images (oh
+  // odd); tiled: TH and TW even.  NPR = pooled rows a block produces.
+  int pool, ph, pw, NPR;
+  int vsplits;   // pool only: K slices of the unfused launch of this layer (see conv3_tile)
 };
+
+// n / d through one high multiply, exact while n * d < 2^32; magic 0 stands for d = 1.
+__host__ __device__ __forceinline__ unsigned div_magic_of(unsigned d) {
+  return d <= 1 ? 0u : (unsigned)((0x100000000ull + d - 1) / d);
+}
+__device__ __forceinline__ int div_magic(int n, unsigned magic) {
+  return magic ? (int)__umulhi((unsigned)n, magic) : n;
+}
 
 template <int BM, int BN, int CC, int WAVES_M, int PMAX, bool VEC, class SC>
 __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const float* __restrict__ w,
@@ -577,7 +614,6 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
   extern __shared__ float lds[];
   float* const As = lds;                       // [KC][SA]
   float* const Ps = lds + KC * SA;             // [CC][CP]
-  int* const rowoff = reinterpret_cast<int*>(Ps + CC * g.CP);  // [R] offset of the row in x, -1 = zero row
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
@@ -585,8 +621,9 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
   const int plane = g.oh * g.ow;
   const int HW = g.H * g.W;
 
-  // patch rows: the padded-row window of this block's pixels, or in the tiled
-  // layout the TH+2 input rows under the tile
+  // patch rows: the padded-row window of this block's pixels (row r of the patch
+  // is padded row gp_lo + r of the stacked images), or in the tiled layout the
+  // TH+2 input rows under the tile
   const bool tiled = g.TW > 0;
   int tb = 0, oy0 = 0, ox0 = 0;   // tiled: image, first output row / column of the tile
   if (tiled) {
@@ -598,19 +635,6 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
   }
   const int b_lo = n0 / plane;
   const int gp_lo = b_lo * g.Hp + (n0 - b_lo * plane) / g.ow;
-  for (int r = threadIdx.x; r < g.R; r += kThreads) {
-    int b, iy;
-    if (tiled) {
-      b = tb;
-      iy = oy0 + r - g.pad;
-    } else {
-      const int gpr = gp_lo + r;
-      b = gpr / g.Hp;
-      iy = gpr - b * g.Hp - g.pad;
-    }
-    rowoff[r] = (b < g.B && iy >= 0 && iy < g.H) ? (b * g.C * g.H + iy) * g.W : -1;
-  }
-  __syncthreads();
 
   // What each thread copies per chunk never changes except for the channel
   // base, so it is decoded once: patch element e = tid + j*256 of the
@@ -623,12 +647,17 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
     const int e = threadIdx.x + j * kThreads;
     int src = -1;
     if (e < patch_total) {
-      const int c = e / g.CP;
+      const int c = div_magic(e, g.mCP);
       const int rem = e - c * g.CP;
-      const int r = rem / g.PW;
+      const int r = div_magic(rem, g.mPW);
       const int ix = ox0 + rem - r * g.PW - g.pad;
-      const int ro = rowoff[r];
-      if (ro >= 0 && ix >= 0 && ix < g.W) src = c * HW + ro + ix;
+      int b = tb, iy = oy0 + r - g.pad;
+      if (!tiled) {
+        const int gpr = gp_lo + r;
+        b = div_magic(gpr, g.mHp);
+        iy = gpr - b * g.Hp - g.pad;
+      }
+      if (b < g.B && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W) src = c * HW + (b * g.C * g.H + iy) * g.W + ix;
     }
     psrc[j] = src;
   }
@@ -657,9 +686,11 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
       jout[t] = (oy < g.oh && ox < g.ow) ? tb * plane + oy * g.ow + ox : -1;
       pbase[t] = ty * g.PW + tx + lk * (CC / 2) * g.CP;
     } else {
-      int j = n0 + wn + t * 32 + lr;
-      jout[t] = j < g.P ? j : -1;
-      j = j < g.P ? j : g.P - 1;
+      const int nl = wn + t * 32 + lr;
+      int j = n0 + nl;
+      const bool ok = nl < g.BNU && j < g.P;
+      jout[t] = ok ? j : -1;
+      j = ok ? j : n0;   // idle lanes read the block's first pixel
       const int b = j / plane;
       const int rem = j - b * plane;
       const int oy = rem / g.ow, ox = rem - oy * g.ow;
@@ -712,12 +743,31 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
     }
   };
 
-  if (chunk0 < chunk1) stage_load(chunk0);
-  for (int chunk = chunk0; chunk < chunk1; chunk++) {
+  // With fused pooling the whole K range is summed here, but in the slices a
+  // split-K launch of the same layer would use (vsplits of them, added in slab
+  // order), so the stored bits do not depend on whether the pool was fused.
+  const int vsplits = (g.pool && g.vsplits > 1) ? g.vsplits : 1;
+  const int vper = (chunk1 - chunk0 + vsplits - 1) / vsplits;
+  f32x16 tot[TM][TN];
+  for (int vz = 0; vz < vsplits; vz++) {
+  const int vc0 = chunk0 + vz * vper, vc1 = min(chunk1, vc0 + vper);
+  if (vz > 0) {
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+      for (int b = 0; b < TN; b++) {
+        if (vz == 1) tot[a][b] = acc[a][b];
+        else tot[a][b] = tot[a][b] + acc[a][b];
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
+      }
+  }
+  if (vc0 < vc1) stage_load(vc0);
+  for (int chunk = vc0; chunk < vc1; chunk++) {
     __syncthreads();           // the previous chunk's LDS reads are done
     stage_store();
     __syncthreads();
-    if (chunk + 1 < chunk1) stage_load(chunk + 1);  // in flight during the MFMAs below
+    if (chunk + 1 < vc1) stage_load(chunk + 1);  // in flight during the MFMAs below
     // ---- MFMA over the chunk: step s pairs k = s (channel s/9) with k = s + KHALF
     // Operand fragments run kAhead steps ahead of the MFMAs that use them: an LDS
     // read takes longer than one 32x32x2 MFMA, so a distance of one left the
@@ -747,7 +797,74 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
       __builtin_amdgcn_sched_barrier(0);
     }
   }
+  }
+  if (vsplits > 1) {
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+      for (int b = 0; b < TN; b++) acc[a][b] = tot[a][b] + acc[a][b];
+  }
 
+  if constexpr (std::is_same<SC, StoreNCHW>::value) {
+    if (g.pool) {
+      // The block's results (after BatchNorm / activation) go to LDS as
+      // S[filter][pixel]; then each thread owns one pooled pixel and walks
+      // filters: window scan order and strict > of the pooling kernel.
+      constexpr int SP = BN + 1;
+      constexpr int QL = BN / 4;            // pooled pixels per block, at most
+      constexpr int FSTEP = kThreads / QL;  // filters advance by this per thread
+      float* const S = lds;
+      __syncthreads();                      // operand reads of the last chunk are done
+#pragma unroll
+      for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int il = wm + a * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+          if (m0 + il < g.F) {
+#pragma unroll
+            for (int t = 0; t < TN; t++) S[il * SP + wn + t * 32 + lr] = tail_apply(sc.tail, m0 + il, acc[a][t][v]);
+          }
+        }
+      __syncthreads();
+      const int q = threadIdx.x % QL;
+      int nl, rowstep, b;
+      int64_t obase;   // offset of the pooled pixel inside its (b, f) plane
+      bool ok;
+      if (tiled) {
+        const int hw = g.TW / 2;
+        const int pr = q / hw, pc = q - pr * hw;
+        ok = pr < g.NPR && oy0 + 2 * pr + 1 < g.oh && ox0 + 2 * pc + 1 < g.ow;
+        nl = 2 * pr * g.TW + 2 * pc;
+        rowstep = g.TW;
+        b = tb;
+        obase = (int64_t)(oy0 / 2 + pr) * g.pw + ox0 / 2 + pc;
+      } else {
+        const int pr = q / g.pw, pc = q - pr * g.pw;
+        int rr = 2 * pr;   // local row of the window's top
+        if (g.oh & 1) { const int k = pr / g.ph; rr = k * g.oh + 2 * (pr - k * g.ph); }
+        const int gr = n0 / g.ow + rr;   // stacked output row
+        b = gr / g.oh;
+        const int oy = gr - b * g.oh;
+        ok = pr < g.NPR && b < g.B;
+        nl = rr * g.ow + 2 * pc;
+        rowstep = g.ow;
+        obase = (int64_t)(oy / 2) * g.pw + pc;
+      }
+      if (ok) {
+        const int64_t pplane = (int64_t)g.ph * g.pw;
+        for (int il = threadIdx.x / QL; il < BM && m0 + il < g.F; il += FSTEP) {
+          const float* s0 = S + il * SP + nl;
+          float out = -3.402823466e+38f;
+          if (s0[0] > out) out = s0[0];
+          if (s0[1] > out) out = s0[1];
+          if (s0[rowstep] > out) out = s0[rowstep];
+          if (s0[rowstep + 1] > out) out = s0[rowstep + 1];
+          sc.y[((int64_t)b * g.F + m0 + il) * pplane + obase] = out;
+        }
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int a = 0; a < TM; a++)
 #pragma unroll
@@ -765,7 +882,7 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_lds(const float* __restric
                                                           float* __restrict__ y, Conv3Geom g,
                                                           ConvTail tail, int splits,
                                                           float* __restrict__ ws) {
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * g.BNU;
   if (splits > 1) {
     const int per = (g.nchunks + splits - 1) / splits;
     const int c0 = blockIdx.z * per, c1 = min(g.nchunks, c0 + per);
@@ -1347,11 +1464,11 @@ int launch_conv_k(gh_ctx* ctx, const gh_cmd& c, const ConvGeom& g, int F, int K,
 }
 
 // Exact number of padded rows the widest block window needs.
-int conv3_patch_rows(const Conv3Geom& g, int BN) {
+int conv3_patch_rows(const Conv3Geom& g, int BNU) {
   const int plane = g.oh * g.ow;
   int best = 0;
-  for (int n0 = 0; n0 < g.P; n0 += BN) {
-    const int pl = (n0 + BN < g.P ? n0 + BN : g.P) - 1;
+  for (int n0 = 0; n0 < g.P; n0 += BNU) {
+    const int pl = (n0 + BNU < g.P ? n0 + BNU : g.P) - 1;
     const int b0 = n0 / plane, b1 = pl / plane;
     const int gp0 = b0 * g.Hp + (n0 - b0 * plane) / g.ow;
     const int gp1 = b1 * g.Hp + (pl - b1 * plane) / g.ow;
@@ -1365,7 +1482,7 @@ template <int BM, int BN, int CC, int WAVES_M, int PMAX>
 int launch_conv3_cfg(gh_ctx* ctx, const gh_cmd& c, Conv3Geom g, int splits, size_t lds_bytes) {
   const bool vec = al16(c.ptr[1]) && g.K % 4 == 0;
   const ConvTail tail = conv_tail(c);
-  const unsigned pixel_tiles = g.TW > 0 ? (unsigned)(g.B * g.tiles_y * g.tiles_x) : (unsigned)((g.P + BN - 1) / BN);
+  const unsigned pixel_tiles = g.TW > 0 ? (unsigned)(g.B * g.tiles_y * g.tiles_x) : (unsigned)((g.P + g.BNU - 1) / g.BNU);
   const dim3 grid(pixel_tiles, (g.F + BM - 1) / BM, splits);
   const float* x = (const float*)(uintptr_t)c.ptr[0];
   const float* w = (const float*)(uintptr_t)c.ptr[1];
@@ -1389,47 +1506,48 @@ int launch_conv3_cfg(gh_ctx* ctx, const gh_cmd& c, Conv3Geom g, int splits, size
   return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
 }
 
-// Returns -1 when the shape is not one the LDS-staged kernel takes.
+// Geometry, tile shape and LDS need of the LDS-staged kernel for one command;
+// false when the shape is not one it takes (or, with `pool`, when the result
+// cannot be cut into blocks of whole pooling windows).
 template <int CC>
-int try_launch_conv3_cc(gh_ctx* ctx, const gh_cmd& c) {
+bool conv3_plan(const gh_cmd& c, bool pool, Conv3Geom* gout, int* BMo, int* BNo, size_t* lds_out, int* per_thread_out) {
   const int B = (int)c.dim[0], C = (int)c.dim[1], H = (int)c.dim[2], W = (int)c.dim[3], F = (int)c.dim[4];
   const int pad = (int)c.dim[7];
   if (c.dim[5] != 3 || c.dim[6] != 3 || c.dim[9] != 1 || c.dim[10] != 1 || c.dim[11] != 1 ||
       c.dim[12] != 1 || c.dim[8] != pad || pad > 1 || C < CC || C % CC != 0)
-    return -1;
-  if (getenv("GORGONIA_HIP_CONV_GATHER")) return -1;  // tuning switch: force the gather kernel
-  Conv3Geom g;
+    return false;
+  if (getenv("GORGONIA_HIP_CONV_GATHER")) return false;  // tuning switch: force the gather kernel
+  Conv3Geom g{};
   g.B = B; g.C = C; g.H = H; g.W = W; g.F = F; g.pad = pad;
   g.oh = H + 2 * pad - 2; g.ow = W + 2 * pad - 2;
-  if (g.oh <= 0 || g.ow <= 0) return -1;
+  if (g.oh <= 0 || g.ow <= 0) return false;
+  if (pool && (g.oh < 2 || g.ow < 2)) return false;
   g.P = B * g.oh * g.ow;
   g.Hp = H + 2 * pad; g.PW = W + 2 * pad;
   g.K = C * 9;
   g.nchunks = (C + CC - 1) / CC;
+  g.pool = pool ? 1 : 0; g.ph = g.oh / 2; g.pw = g.ow / 2;
   // Tile choice: 64x64 blocks measured fastest on every 3x3 layer of the
   // benchmark configurations (more, smaller blocks hide the staging latency
-  // better than 128-wide ones); the channel chunks are split across grid.z
-  // when even those leave the chip under-filled.
-  const int64_t cus = ctx->cu_count;
+  // better than 128-wide ones).
   int BM = 64, BN = 64;
-  if (const char* env = getenv("GORGONIA_HIP_CONV_TILE")) {  // tuning override: 0 = 128 wide, 1 = 64x64, 2 = 128x64
-    if (atoi(env) == 0) { BM = F > 64 ? 128 : 64; BN = 128; }
-    if (atoi(env) == 2 && F > 64) { BM = 128; BN = 64; }
+  const char* tile_env = getenv("GORGONIA_HIP_CONV_TILE");  // tuning override: 0 = 128 wide, 1 = 64x64, 2 = 128x64
+  if (tile_env && !pool) {
+    if (atoi(tile_env) == 0) { BM = F > 64 ? 128 : 64; BN = 128; }
+    if (atoi(tile_env) == 2 && F > 64) { BM = 128; BN = 64; }
   }
-  g.TH = g.TW = g.tiles_x = g.tiles_y = 0;
-  g.R = conv3_patch_rows(g, BN);
-  g.CP = g.R * g.PW;
-  int64_t pixel_tiles = cdiv(g.P, BN);
-  // Wide rows: BN consecutive pixels touch only one or two image rows, and the
-  // row-stacked patch would hold whole rows for them.  Cut the image into
-  // TH x TW rectangles instead (the shape that wastes the fewest pixels on
-  // partial tiles, then the smallest patch) and stage the window under each.
-  if (g.ow >= 64 && !getenv("GORGONIA_HIP_CONV_GATHER_WIDE") && !getenv("GORGONIA_HIP_CONV_TILE")) {
+  g.BNU = BN;
+  if (g.ow >= 64 && !getenv("GORGONIA_HIP_CONV_GATHER_WIDE") && (!tile_env || pool)) {
+    // Wide rows: BN consecutive pixels touch only one or two image rows, and the
+    // row-stacked patch would hold whole rows for them.  Cut the image into
+    // TH x TW rectangles instead (the shape that wastes the fewest pixels on
+    // partial tiles, then the smallest patch) and stage the window under each.
     if (F <= 32) { BM = 32; BN = 128; }
     int best_th = 0, best_tw = 0;
     int64_t best_tiles = 0, best_patch = 0;
     for (int tw = 4; tw <= BN; tw *= 2) {
       const int th = BN / tw;
+      if (pool && th < 2) continue;   // a block must hold whole 2x2 windows
       const int64_t tiles = cdiv(g.oh, th) * cdiv(g.ow, tw);
       const int64_t patch = (int64_t)(th + 2) * (tw + 2);
       if (!best_tw || tiles < best_tiles || (tiles == best_tiles && patch < best_patch)) {
@@ -1439,12 +1557,48 @@ int try_launch_conv3_cc(gh_ctx* ctx, const gh_cmd& c) {
     g.TH = best_th; g.TW = best_tw;
     g.tiles_x = (int)cdiv(g.ow, g.TW); g.tiles_y = (int)cdiv(g.oh, g.TH);
     g.PW = g.TW + 2; g.R = g.TH + 2; g.CP = g.R * g.PW;
-    pixel_tiles = (int64_t)B * g.tiles_x * g.tiles_y;
+    g.BNU = BN;
+    g.NPR = g.TH / 2;
+  } else {
+    if (pool) {
+      // rows per block: an even count when oh is even (stacked rows then pair
+      // up inside every image), whole images when it is odd
+      const int unit = (g.oh & 1) ? g.oh : 2;
+      int rt = (BN / g.ow) / unit * unit;
+      if (rt == 0) { BN = 128; rt = (BN / g.ow) / unit * unit; }
+      if (rt == 0) return false;
+      g.BNU = rt * g.ow;
+      g.NPR = (g.oh & 1) ? (rt / g.oh) * g.ph : rt / 2;
+    }
+    g.R = conv3_patch_rows(g, g.BNU);
+    g.CP = g.R * g.PW;
   }
-  const size_t lds = ((size_t)CC * 9 * (BM + 2) + (size_t)CC * g.CP + g.R) * 4;
-  if (lds > 64 * 1024) return -1;
+  size_t lds = ((size_t)CC * 9 * (BM + 2) + (size_t)CC * g.CP) * 4;
+  if (pool && lds < (size_t)BM * (BN + 1) * 4) lds = (size_t)BM * (BN + 1) * 4;
+  if (lds > 64 * 1024) return false;
+  // the staging decode's multiply-high divisions are exact below 2^32
+  if ((int64_t)CC * g.CP * g.CP >= (1ll << 32) || ((int64_t)B * g.Hp + g.R) * g.Hp >= (1ll << 32)) return false;
+  g.mCP = div_magic_of((unsigned)g.CP); g.mPW = div_magic_of((unsigned)g.PW); g.mHp = div_magic_of((unsigned)g.Hp);
   const int per_thread = (CC * g.CP + kThreads - 1) / kThreads;  // patch elements each thread stages
-  if (per_thread > 16) return -1;  // the gather kernel does better
+  if (per_thread > 16) return false;  // the gather kernel does better
+  *gout = g; *BMo = BM; *BNo = BN; *lds_out = lds; *per_thread_out = per_thread;
+  return true;
+}
+
+// Returns -1 when the shape is not one the LDS-staged kernel takes.
+template <int CC>
+int try_launch_conv3_cc(gh_ctx* ctx, const gh_cmd& c) {
+  Conv3Geom g;
+  int BM, BN, per_thread;
+  size_t lds;
+  const bool pool = c.flags & GH_FLAG_CONV_POOL2;
+  if (!conv3_plan<CC>(c, pool, &g, &BM, &BN, &lds, &per_thread)) return -1;
+  const int F = g.F;
+  const int64_t cus = ctx->cu_count;
+  const int64_t pixel_tiles = g.TW > 0 ? (int64_t)g.B * g.tiles_x * g.tiles_y : cdiv(g.P, g.BNU);
+  // the channel chunks are split across grid.z when the tiles alone leave the
+  // chip under-filled (never with fused pooling: the pooled epilogue needs the
+  // finished sums)
   const int64_t blocks = cdiv(F, BM) * pixel_tiles;
   int splits = 1;
   if (const char* env = getenv("GORGONIA_HIP_CONV_SPLITS")) splits = atoi(env);
@@ -1454,6 +1608,27 @@ int try_launch_conv3_cc(gh_ctx* ctx, const gh_cmd& c) {
   }
   if (splits > g.nchunks) splits = g.nchunks;
   if (splits < 1) splits = 1;
+  if (pool) {
+    // the K slices the same layer gets without the pool (its own block count)
+    Conv3Geom g0;
+    int BM0, BN0, pt0;
+    size_t lds0;
+    int vs = 1;
+    if (conv3_plan<CC>(c, false, &g0, &BM0, &BN0, &lds0, &pt0)) {
+      const int64_t tiles0 = g0.TW > 0 ? (int64_t)g0.B * g0.tiles_x * g0.tiles_y : cdiv(g0.P, g0.BNU);
+      const int64_t blocks0 = cdiv(F, BM0) * tiles0;
+      if (const char* env = getenv("GORGONIA_HIP_CONV_SPLITS")) vs = atoi(env);
+      else {
+        vs = (int)((5 * cus / 2 + blocks0 / 2) / blocks0);
+        if (vs > g.nchunks / 4) vs = g.nchunks / 4;
+      }
+      if (vs > g.nchunks) vs = g.nchunks;
+      if (vs < 1) vs = 1;
+      while (vs > 1 && (int64_t)vs * F * g.P * 4 > ctx->workspace_bytes) vs--;
+    }
+    g.vsplits = vs;
+    splits = 1;
+  }
   while (splits > 1 && (int64_t)splits * F * g.P * 4 > ctx->workspace_bytes) splits--;
 #define GH_CONV3(BM_, BN_)                                                                        \
   (per_thread <= 8 ? launch_conv3_cfg<BM_, BN_, CC, 2, 8>(ctx, c, g, splits, lds)                 \
@@ -1560,10 +1735,10 @@ static int launch_conv_direct(gh_ctx* ctx, const gh_cmd& c) {
 
 int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
   if (conv_direct_shape(c) && !getenv("GORGONIA_HIP_CONV_NO_DIRECT")) return launch_conv_direct(ctx, c);
-  if (c.flags & GH_FLAG_CONV_POOL2)
-    return gh_fail(ctx, GH_EINVAL, "conv2d: no fused pooling for this shape (see gh_conv2d_can_pool)");
   const int rc3 = try_launch_conv3(ctx, c);
   if (rc3 >= 0) return rc3;
+  if (c.flags & GH_FLAG_CONV_POOL2)
+    return gh_fail(ctx, GH_EINVAL, "conv2d: no fused pooling for this shape (see gh_conv2d_can_pool)");
   ConvGeom g;
   g.C = (int)c.dim[1]; g.H = (int)c.dim[2]; g.W = (int)c.dim[3];
   g.kh = (int)c.dim[5]; g.kw = (int)c.dim[6];
@@ -1713,7 +1888,14 @@ int gh_launch_outer(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {
-  if (!c || c->opcode != GH_OP_CONV2D || !conv_direct_shape(*c)) return 0;
-  const int64_t oh = c->dim[2] + 2 * c->dim[7] - 2, ow = c->dim[3] + 2 * c->dim[7] - 2;
-  return oh >= 2 && ow >= 2;
+  if (!c || c->opcode != GH_OP_CONV2D) return 0;
+  if (conv_direct_shape(*c) && !getenv("GORGONIA_HIP_CONV_NO_DIRECT")) {
+    const int64_t oh = c->dim[2] + 2 * c->dim[7] - 2, ow = c->dim[3] + 2 * c->dim[7] - 2;
+    return oh >= 2 && ow >= 2;
+  }
+  if (getenv("GORGONIA_HIP_CONV_NO_POOL")) return 0;  // tuning switch: keep MaxPool2D a kernel of its own
+  Conv3Geom g;
+  int BM, BN, per_thread;
+  size_t lds;
+  return conv3_plan<8>(*c, true, &g, &BM, &BN, &lds, &per_thread) ? 1 : 0;
 }

@@ -165,7 +165,12 @@ def test_conv_epilogue_batchnorm_activation_bit_exact(ctx, cfg):
 
 
 @pytest.mark.parametrize("cfg", [(3, 1, 28, 28, 32, 1), (2, 3, 21, 19, 16, 1), (2, 4, 10, 12, 6, 0),
-                                 (1, 2, 7, 7, 9, 1)])
+                                 (1, 2, 7, 7, 9, 1),
+                                 # the matrix-core kernel: blocks of whole rows (even height, blocks crossing
+                                 # images), whole images (odd height), 128-pixel blocks, rectangular tiles
+                                 (5, 32, 14, 14, 64, 1), (3, 16, 7, 7, 40, 1), (130, 8, 7, 7, 8, 1),
+                                 (2, 8, 26, 26, 16, 1), (2, 8, 16, 16, 70, 0), (2, 8, 52, 52, 8, 1),
+                                 (1, 8, 70, 66, 24, 1), (1, 16, 64, 66, 48, 0), (2, 8, 9, 5, 16, 1)])
 def test_conv_epilogue_pool_bit_exact(ctx, cfg):
     """conv -> ReLU -> MaxPool 2x2/2 as one command (odd sizes drop the last row/column)."""
     B, C, H, W, F, pad = cfg
@@ -187,7 +192,8 @@ def test_conv_epilogue_pool_bit_exact(ctx, cfg):
 
 
 def test_conv_pool_flag_needs_a_pooling_kernel(ctx):
-    cmd = D.cmd_conv2d(0x1000, 0x2000, 0x3000, 2, 8, 14, 14, 16, 3, 3, (1, 1), pool2=True)
+    # 13 rows of 13: no block of at most 128 pixels holds a whole image
+    cmd = D.cmd_conv2d(0x1000, 0x2000, 0x3000, 2, 8, 13, 13, 16, 3, 3, (1, 1), pool2=True)
     assert ctx.lib.gh_conv2d_can_pool(cmd) == 0
     import ctypes as C
     buf = C.create_string_buffer(256)

@@ -47,7 +47,7 @@ def test_convnet_forward_fused_and_unfused(ctx):
     m2, _, r2 = run_once(configs.build_convnet, inp, fuse_activations=True)
     assert rel_frobenius(r1["out"], want) <= 1e-5
     assert_bits_equal(r1["out"], r2["out"], "fused activations change nothing")
-    assert m2.fused == 5  # 4 activations + the first pool
+    assert m2.fused == 7  # 4 activations + the three pools
     m1.Close(); m2.Close()
 
 
@@ -58,11 +58,11 @@ def test_yolo_shaped_forward_reduced(ctx):
     m, _, res = run_once(configs.build_yolo, inp, fuse_activations=True)
     assert res["out"].shape == want.shape == (1, 425, 3, 3)
     assert rel_frobenius(res["out"], want) <= 1e-5
-    # conv -> batchnorm -> leakyrelu (-> maxpool after the 3-channel layer) run as
+    # conv -> batchnorm -> leakyrelu (-> maxpool where it is 2x2 stride 2) run as
     # single commands; the folded program stores the bits of the plain one
     prog = m.program()
     assert prog.count("conv2d+batchnorm(eval)+leakyrelu") == 7
-    assert prog.count("conv2d+batchnorm(eval)+leakyrelu+maxpool2d") == 1
+    assert prog.count("conv2d+batchnorm(eval)+leakyrelu+maxpool2d") == 5
     assert " batchnorm" not in prog and " leakyrelu" not in prog
     m.Close()
     m0, _, plain = run_once(configs.build_yolo, inp)
