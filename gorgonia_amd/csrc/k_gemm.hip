@@ -459,36 +459,69 @@ __global__ __launch_bounds__(256) void k_splitk_reduce4(const float* __restrict_
 // MFMA lane order (every element is used once per tile, so LDS staging buys
 // nothing), then the WV partial tiles are summed through LDS in wavefront order
 // - a fixed order, so results repeat bit for bit - and the epilogue is applied.
-template <int WV>
+// (Cutting K across workgroups as well, with the last one to arrive at a
+// per-tile counter adding the slices, was measured: the device-wide fences it
+// needs cost ~35 us per launch on this part, four times the whole kernel.)
+template <int WV, bool VEC>
 __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict__ A,
                                                          const float* __restrict__ B,
                                                          float* __restrict__ C, int M, int N, int K,
                                                          int lda, int ldb, int ldc, int act,
-                                                         float alpha, int vec_a) {
+                                                         float alpha) {
   constexpr int G = 5;                       // k-chunks per group; two groups of loads are in flight
   constexpr int HALF = WV / 2;
   __shared__ float part[HALF * 1024];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // the wavefront index as a scalar: every branch on chunk numbers below is then
+  // a scalar branch, and a load in one arm does not look pending in the other
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 31, h = lane >> 5;
   const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
   const int m = m0 + r, n = n0 + r;
   const int nchunks = (K + 15) / 16;
-  const float* arow = A + (int64_t)m * lda;
 
-  // lane (r, h) feeds k = 16*chunk + 8*h + t at MFMA step t of a chunk
+  // Lane (r, h) feeds k = 16*chunk + 8*h + t at MFMA step t of a chunk.  B comes
+  // in that order straight from memory (32 consecutive columns per k).  A would
+  // be one row per lane - 64 cache lines per load instruction - so a chunk of A
+  // (32 rows x 16 k) is loaded with k fastest across lanes and turned into MFMA
+  // order through a wavefront-private LDS tile just before use.  Loads never
+  // branch per lane: rows, columns and k past the matrix are clamped to the
+  // last valid one and replaced by zero just before the MFMA, so nothing makes
+  // the compiler wait for one load before it issues the next.
+  constexpr int TP = 20;                     // pitch of the transposing tile: rows stay 16-byte aligned
+  __shared__ __attribute__((aligned(16))) float tbuf[WV][32 * TP];
+  float* const T = tbuf[wave];
+  const int n_c = min(n, N - 1);
+  const float* const a_vec = A + (int64_t)min(m0 + (lane >> 2), M - 1) * lda + (lane & 3) * 4;   // + 16 rows for the second load
+  const int64_t a_vec_step = (int64_t)(min(m0 + 16 + (lane >> 2), M - 1) - min(m0 + (lane >> 2), M - 1)) * lda;
   auto load = [&](int chunk, float (&a)[8], float (&b)[8]) {
-    const int k0 = chunk * 16 + 8 * h;
-    if (m < M && vec_a && k0 + 8 <= K) {
-      const f32x4 lo = *reinterpret_cast<const f32x4*>(arow + k0);
-      const f32x4 hi = *reinterpret_cast<const f32x4*>(arow + k0 + 4);
+    if (VEC) {   // 16-byte aligned rows and K a multiple of 16: every chunk is whole
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(a_vec + chunk * 16);
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(a_vec + a_vec_step + chunk * 16);
 #pragma unroll
       for (int t = 0; t < 4; t++) { a[t] = lo[t]; a[4 + t] = hi[t]; }
     } else {
+      const int kk = min(chunk * 16 + (lane & 15), K - 1);
 #pragma unroll
-      for (int t = 0; t < 8; t++) a[t] = (m < M && k0 + t < K) ? arow[k0 + t] : 0.f;
+      for (int t = 0; t < 8; t++) a[t] = A[(int64_t)min(m0 + t * 4 + (lane >> 4), M - 1) * lda + kk];
     }
+    const int k0 = chunk * 16 + 8 * h;
 #pragma unroll
-    for (int t = 0; t < 8; t++) b[t] = (n < N && k0 + t < K) ? B[(int64_t)(k0 + t) * ldb + n] : 0.f;
+    for (int t = 0; t < 8; t++) b[t] = B[(int64_t)min(k0 + t, K - 1) * ldb + n_c];
+  };
+  // load order -> MFMA order, in place
+  auto transpose_a = [&](int chunk, float (&a)[8]) {
+    if (VEC) {
+      f32x4 lo = {a[0], a[1], a[2], a[3]}, hi = {a[4], a[5], a[6], a[7]};
+      *reinterpret_cast<f32x4*>(T + (lane >> 2) * TP + (lane & 3) * 4) = lo;
+      *reinterpret_cast<f32x4*>(T + (16 + (lane >> 2)) * TP + (lane & 3) * 4) = hi;
+    } else {
+#pragma unroll
+      for (int t = 0; t < 8; t++) T[(t * 4 + (lane >> 4)) * TP + (lane & 15)] = a[t];
+    }
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(T + r * TP + 8 * h);
+    const f32x4 hi = *reinterpret_cast<const f32x4*>(T + r * TP + 8 * h + 4);
+#pragma unroll
+    for (int t = 0; t < 4; t++) { a[t] = lo[t]; a[4 + t] = hi[t]; }
   };
   // group = chunks c, c + WV, ... (G of them); the chunk order per wavefront is
   // fixed, so the sum is the same whatever the grouping
@@ -504,9 +537,14 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
 #pragma unroll
     for (int g = 0; g < G; g++)
       if (c + g * WV < nchunks) {
+        transpose_a(c + g * WV, a[g]);
+        const int left = K - ((c + g * WV) * 16 + 8 * h);   // valid k of this lane's eight
 #pragma unroll
-        for (int t = 0; t < 8; t++)
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[g][t], b[g][t], acc, 0, 0, 0);
+        for (int t = 0; t < 8; t++) {
+          const float av = (m < M && t < left) ? a[g][t] : 0.f;
+          const float bv = (n < N && t < left) ? b[g][t] : 0.f;
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
+        }
       }
   };
 
@@ -709,6 +747,14 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
 
   float preg[PMAX];
   f32x4 wreg[NW];
+  // Variants of this staging that were measured and not kept (MI355X, the 3x3
+  // layers of the benchmark configurations): a second register set so loads get
+  // two chunks to land (185 registers instead of 87, large layers 30 % slower);
+  // branch-free loads with the zero chosen at the LDS write, and loads spread
+  // between the MFMAs (a few percent slower); eight wavefronts per block with
+  // the k-steps of a chunk split between two quads (MFMA phase at its ideal
+  // length, but the wait for the next chunk's loads grows by as much; large
+  // layers 8-25 % slower); a per-block rotation of the chunk order (no change).
   auto stage_load = [&](int chunk) {
     const int c0 = chunk * CC;
     const float* xc = x + (int64_t)c0 * HW;
@@ -1660,11 +1706,18 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   if (getenv("GORGONIA_HIP_GEMM_PLAN")) return -1;  // a forced tile plan means the tiled kernel
   const int lda = (int)c.dim[3], ldb = (int)c.dim[4], ldc = (int)c.dim[5];
   const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
-  const int vec_a = al16(c.ptr[0]) && lda % 4 == 0;
+  const bool vec_a = al16(c.ptr[0]) && lda % 4 == 0 && K % 16 == 0;
   constexpr int WV = 8;  // 512 threads leave each wavefront 256 registers for the grouped loads
-  hipLaunchKernelGGL((k_gemm_skinny<WV>), dim3((N + 31) / 32, (M + 31) / 32), dim3(WV * 64), 0, ctx->stream,
-                     (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
-                     (float*)(uintptr_t)c.ptr[2], M, N, K, lda, ldb, ldc, act, c.f[0], vec_a);
+  const dim3 grid((N + 31) / 32, (M + 31) / 32);
+  const float* A = (const float*)(uintptr_t)c.ptr[0];
+  const float* B = (const float*)(uintptr_t)c.ptr[1];
+  float* C = (float*)(uintptr_t)c.ptr[2];
+  if (vec_a)
+    hipLaunchKernelGGL((k_gemm_skinny<WV, true>), grid, dim3(WV * 64), 0, ctx->stream, A, B, C, M, N, K, lda, ldb,
+                       ldc, act, c.f[0]);
+  else
+    hipLaunchKernelGGL((k_gemm_skinny<WV, false>), grid, dim3(WV * 64), 0, ctx->stream, A, B, C, M, N, K, lda, ldb,
+                       ldc, act, c.f[0]);
   return gh_check_hip(ctx, hipGetLastError(), "skinny gemm launch");
 }
 
