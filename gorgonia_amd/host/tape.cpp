@@ -660,6 +660,19 @@ Status TapeMachine::Compile() {
     reg_last[(size_t)r] = std::max(reg_last[(size_t)r], std::max(i, last_reader[(size_t)root[(size_t)i]]));
     if (value_kept[(size_t)root[(size_t)i]]) reg_kept[(size_t)r] = 1;
   }
+  // A small result that only the host reads is written by its kernel straight
+  // into pinned host memory: no arena register, no staging copy at the end of
+  // the segment.
+  std::vector<char> host_out((size_t)N, 0);
+  for (int i = 0; i < N; i++) {
+    const Node& n = nodes[(size_t)i];
+    if (!n.read_into || n.is_input || n.fused_away || n.alias_of >= 0 || inplace[(size_t)i]) continue;
+    if (bytes_of(n) > kStageLimit || bytes_of(n) % 4 != 0 || last_reader[(size_t)i] >= 0) continue;
+    bool shared = false;
+    for (int j = 0; j < N; j++)
+      if (j != i && (root[(size_t)j] == i || node_reg_[(size_t)j] == node_reg_[(size_t)i])) shared = true;
+    if (!shared) host_out[(size_t)i] = 1;
+  }
   regs_.assign((size_t)nreg, Tensor());
   reg_live_.assign((size_t)nreg, 0);
   resident_done_.assign((size_t)N, 0);
@@ -682,7 +695,9 @@ Status TapeMachine::Compile() {
       reg_bytes[(size_t)r] = bytes;
       gpumem_ += bytes;
     } else {
-      if (!inplace[(size_t)i]) {
+      if (host_out[(size_t)i]) {
+        prog_.push_back({InstrKind::AllocHost, i, r, bytes, false});
+      } else if (!inplace[(size_t)i]) {
         prog_.push_back({InstrKind::Alloc, i, r, bytes, false});
         reg_bytes[(size_t)r] = bytes;
         gpumem_ += bytes;
@@ -697,7 +712,7 @@ Status TapeMachine::Compile() {
   // host reads: one flush, then the copies (compile.go:437-462 puts a flush in
   // front of every consumer that needs a finished value)
   for (int i = 0; i < N; i++)
-    if (nodes[(size_t)i].read_into && bytes_of(nodes[(size_t)i]) <= kStageLimit &&
+    if (nodes[(size_t)i].read_into && !host_out[(size_t)i] && bytes_of(nodes[(size_t)i]) <= kStageLimit &&
         bytes_of(nodes[(size_t)i]) % 4 == 0)
       prog_.push_back({InstrKind::StageOut, i, node_reg_[(size_t)i], bytes_of(nodes[(size_t)i]), false});
   prog_.push_back({InstrKind::Flush, -1, -1, 0, false});
@@ -708,7 +723,7 @@ Status TapeMachine::Compile() {
   for (int i = 0; i < N; i++) {
     Node& n = nodes[(size_t)i];
     const int r = node_reg_[(size_t)i];
-    if (!n.read_into) continue;
+    if (!n.read_into || host_out[(size_t)i]) continue;
     bool resident_reg = false;
     for (int j = 0; j < N; j++)
       if (node_reg_[(size_t)j] == r && nodes[(size_t)j].is_input && nodes[(size_t)j].resident) resident_reg = true;
@@ -732,7 +747,7 @@ Status TapeMachine::Init(int device) {
   if (!st.ok()) return st;
   stage_.assign(g_->Nodes().size(), nullptr);
   for (auto& in : prog_)
-    if (in.kind == InstrKind::StageOut) {
+    if (in.kind == InstrKind::StageOut || in.kind == InstrKind::AllocHost) {
       st = eng_.HostAlloc(in.size, &stage_[(size_t)in.node]);
       if (!st.ok()) return st;
     }
@@ -841,6 +856,9 @@ Status TapeMachine::RunAll() {
         st = flush();
         if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": flush");
         break;
+      case InstrKind::AllocHost:
+        regs_[(size_t)in.reg].mem = (uint64_t)(uintptr_t)stage_[(size_t)in.node];
+        break;
       case InstrKind::StageOut:
         eng_.RecordCopy((uint64_t)(uintptr_t)stage_[(size_t)in.node], regs_[(size_t)in.reg].mem, in.size);
         break;
@@ -891,7 +909,7 @@ Status TapeMachine::Close() {
 }
 
 std::string TapeMachine::ProgramString() const {
-  static const char* names[] = {"loadArg", "alloc", "devTrans", "execOp", "free", "flush", "read", "stageOut"};
+  static const char* names[] = {"loadArg", "alloc", "devTrans", "execOp", "free", "flush", "read", "stageOut", "allocHost"};
   std::ostringstream os;
   os << "Instructions:\n";
   const auto& nodes = g_->Nodes();

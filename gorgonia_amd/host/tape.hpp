@@ -120,7 +120,7 @@ class Graph {
   std::vector<Node> nodes_;
 };
 
-enum class InstrKind : int32_t { LoadArg, Alloc, Transport, ExecOp, Free, Flush, Read, StageOut };
+enum class InstrKind : int32_t { LoadArg, Alloc, Transport, ExecOp, Free, Flush, Read, StageOut, AllocHost };
 
 struct Instr {
   InstrKind kind;
