@@ -41,6 +41,7 @@ FLAG_ACT_LEAKY = 1 << 23
 FLAG_CONV_BN = 1 << 24
 FLAG_CONV_POOL2 = 1 << 25
 FLAG_BN_EVAL = 1 << 26
+FLAG_GEMM_SOFTMAX = 1 << 27
 
 
 def flag_fn(f):
@@ -87,6 +88,7 @@ SYMBOLS = {
     "gh_submit": (C.c_int, [_P, C.POINTER(GhCmd), C.c_int]),
     "gh_validate": (C.c_int, [C.POINTER(GhCmd), C.c_int, C.c_char_p, C.c_int]),
     "gh_conv2d_can_pool": (C.c_int, [C.POINTER(GhCmd)]),
+    "gh_gemm_can_softmax": (C.c_int, [C.POINTER(GhCmd)]),
     "gh_sync": (C.c_int, [_P]),
     "gh_graph_begin": (C.c_int, [_P]),
     "gh_graph_end": (C.c_int, [_P, C.POINTER(C.c_int)]),

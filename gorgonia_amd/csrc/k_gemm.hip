@@ -467,7 +467,7 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
                                                          const float* __restrict__ B,
                                                          float* __restrict__ C, int M, int N, int K,
                                                          int lda, int ldb, int ldc, int act,
-                                                         float alpha) {
+                                                         float alpha, int softmax) {
   constexpr int G = 5;                       // k-chunks per group; two groups of loads are in flight
   constexpr int HALF = WV / 2;
   __shared__ float part[HALF * 1024];
@@ -489,6 +489,7 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
   // the compiler wait for one load before it issues the next.
   constexpr int TP = 20;                     // pitch of the transposing tile: rows stay 16-byte aligned
   __shared__ __attribute__((aligned(16))) float tbuf[WV][32 * TP];
+  __shared__ float sm_x[32 * 33], sm_e[32 * 33];   // the tile and its exponentials when a softmax follows
   float* const T = tbuf[wave];
   const int n_c = min(n, N - 1);
   const float* const a_vec = A + (int64_t)min(m0 + (lane >> 2), M - 1) * lda + (lane & 3) * 4;   // + 16 rows for the second load
@@ -582,8 +583,29 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
 #pragma unroll
     for (int w = 1; w < HALF; w++) sum = sum + part[w * 1024 + e];
     const int v = e >> 6, l = e & 63;
-    const int i = m0 + 8 * (v / 4) + 4 * (l >> 5) + (v % 4), j = n0 + (l & 31);
-    if (i < M && j < N) C[(int64_t)i * ldc + j] = act_apply(sum, act, alpha);
+    const int il = 8 * (v / 4) + 4 * (l >> 5) + (v % 4), jl = l & 31;
+    const int i = m0 + il, j = n0 + jl;
+    if (softmax) sm_x[il * 33 + jl] = act_apply(sum, act, alpha);
+    else if (i < M && j < N) C[(int64_t)i * ldc + j] = act_apply(sum, act, alpha);
+  }
+  if (!softmax) return;
+  // Row softmax of the tile (N <= 32: the tile holds whole rows) with the
+  // arithmetic of the softmax kernel: max, exp(x - max) in float64 rounded
+  // once, the sum taken in column order, one rounded reciprocal.
+  __syncthreads();
+  for (int e = threadIdx.x; e < 1024; e += WV * 64) {
+    const int il = e >> 5, jl = e & 31;
+    float mx = -INFINITY;
+    for (int j = 0; j < N; j++) mx = fmaxf(mx, sm_x[il * 33 + j]);
+    sm_e[il * 33 + jl] = jl < N ? (float)exp((double)(sm_x[il * 33 + jl] - mx)) : 0.f;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < 1024; e += WV * 64) {
+    const int il = e >> 5, jl = e & 31;
+    float sum = 0.f;
+    for (int j = 0; j < N; j++) sum = sum + sm_e[il * 33 + j];
+    const float inv = 1.0f / sum;
+    if (m0 + il < M && jl < N) C[(int64_t)(m0 + il) * ldc + jl] = sm_e[il * 33 + jl] * inv;
   }
 }
 
@@ -1709,15 +1731,16 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   const bool vec_a = al16(c.ptr[0]) && lda % 4 == 0 && K % 16 == 0;
   constexpr int WV = 8;  // 512 threads leave each wavefront 256 registers for the grouped loads
   const dim3 grid((N + 31) / 32, (M + 31) / 32);
+  const int softmax = (c.flags & GH_FLAG_GEMM_SOFTMAX) ? 1 : 0;
   const float* A = (const float*)(uintptr_t)c.ptr[0];
   const float* B = (const float*)(uintptr_t)c.ptr[1];
   float* C = (float*)(uintptr_t)c.ptr[2];
   if (vec_a)
     hipLaunchKernelGGL((k_gemm_skinny<WV, true>), grid, dim3(WV * 64), 0, ctx->stream, A, B, C, M, N, K, lda, ldb,
-                       ldc, act, c.f[0]);
+                       ldc, act, c.f[0], softmax);
   else
     hipLaunchKernelGGL((k_gemm_skinny<WV, false>), grid, dim3(WV * 64), 0, ctx->stream, A, B, C, M, N, K, lda, ldb,
-                       ldc, act, c.f[0]);
+                       ldc, act, c.f[0], softmax);
   return gh_check_hip(ctx, hipGetLastError(), "skinny gemm launch");
 }
 
@@ -1735,6 +1758,8 @@ int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
   }
   const int rs = try_launch_gemm_skinny(ctx, c);
   if (rs >= 0) return rs;
+  if (c.flags & GH_FLAG_GEMM_SOFTMAX)
+    return gh_fail(ctx, GH_EINVAL, "gemm: no fused softmax for this shape (see gh_gemm_can_softmax)");
   const int64_t batch = c.dim[6] <= 0 ? 1 : c.dim[6];
   const TilePlan p = plan_tiles(ctx, c.dim[0], c.dim[1], c.dim[2], batch, false);
   if (p.tile == kTile128) return launch_sgemm_cfg<128, 128, 2>(ctx, c, p.splits);
@@ -1938,6 +1963,15 @@ int gh_launch_outer(gh_ctx* ctx, const gh_cmd& c) {
                      (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
                      (float*)(uintptr_t)c.ptr[2], m, n);
   return gh_check_hip(ctx, hipGetLastError(), "outer launch");
+}
+
+extern "C" int gh_gemm_can_softmax(const gh_cmd* c) {
+  if (!c || c->opcode != GH_OP_GEMM || gh_dtype_of(c->flags) != GH_F32) return 0;
+  if (c->flags & (GH_FLAG_TRANS_A | GH_FLAG_TRANS_B)) return 0;
+  const int64_t batch = c->dim[6] <= 0 ? 1 : c->dim[6];
+  if (batch != 1 || getenv("GORGONIA_HIP_GEMM_PLAN")) return 0;
+  // the small-output kernel must take the product (one workgroup per 32 rows)
+  return c->dim[1] >= 1 && c->dim[1] <= 32 && c->dim[0] >= 1 && c->dim[0] <= 2048 && c->dim[2] >= 32;
 }
 
 extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {

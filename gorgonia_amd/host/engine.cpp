@@ -400,7 +400,7 @@ Status Engine::MatVecMul(Tensor& a, Tensor& b, Tensor& prealloc) {
   return Status::OK();
 }
 
-Status Engine::MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act, float alpha) {
+Status Engine::MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act, float alpha, bool softmax) {
   Status st = checkThreeFloat(a, b, prealloc);
   if (!st.ok()) return st.Wrap("MatMul failed pre check");
   if (a.dt == Dtype::Other) return Status::Err(GH_EINVAL, "Unsupported Dtype " + dtype_name(a.dt));
@@ -419,6 +419,7 @@ Status Engine::MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act, float alp
   c.opcode = GH_OP_GEMM;
   c.flags = (a.transposed ? GH_FLAG_TRANS_A : 0) | (b.transposed ? GH_FLAG_TRANS_B : 0) |
             (act == 1 ? GH_FLAG_ACT_RELU : act == 2 ? GH_FLAG_ACT_LEAKY : 0) |
+            (softmax ? GH_FLAG_GEMM_SOFTMAX : 0) |
             GH_FLAG_DTYPE(a.dt == Dtype::Float64 ? GH_F64 : GH_F32);  // Dgemm / Sgemm, cuda/linalg.go:204-227
   c.f[0] = alpha;
   c.ptr[0] = a.mem; c.ptr[1] = b.mem; c.ptr[2] = prealloc.mem;

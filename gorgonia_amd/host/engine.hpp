@@ -151,7 +151,7 @@ class Engine {
   // ---- linalg (cuda/linalg.go:47-285) -----------------------------------------------------
   Status MatVecMul(Tensor& a, Tensor& b, Tensor& prealloc);
   // act: 0 none, 1 Rectify, 2 LeakyRelu(alpha) applied to the product (fused epilogue).
-  Status MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act = 0, float alpha = 0.f);
+  Status MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act = 0, float alpha = 0.f, bool softmax = false);
   Status Outer(Tensor& a, Tensor& b, Tensor& prealloc);
   // batchedMatMul (operatorLinAlg.go:435-502): one strided-batched launch.
   Status BatchedMatMul(Tensor& a, Tensor& b, Tensor& c, bool transA, bool transB);

@@ -254,7 +254,9 @@ static std::string op_name(const OpSpec& op) {
     case OpKind::ElemBin: return std::string("elembin.") + bins[op.fn];
     case OpKind::ElemUnary: return "elemunary." + op.name;
     case OpKind::BroadcastBin: return std::string("broadcast.") + bins[op.fn];
-    case OpKind::MatMul: return "matmul";
+    case OpKind::MatMul:
+      return std::string("matmul") + (op.fuse_act_relu ? "+rectify" : op.fuse_act_leaky ? "+leakyrelu" : "") +
+             (op.fuse_softmax ? "+softmax" : "");
     case OpKind::MatVecMul: return "matvecmul";
     case OpKind::Outer: return "outer";
     case OpKind::BatchedMatMul: return "batchedmatmul";
@@ -315,7 +317,7 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       if (op.transA) { std::swap(a.shape.d[0], a.shape.d[1]); a.transposed = !a.transposed; }
       if (op.transB) { std::swap(b.shape.d[0], b.shape.d[1]); b.transposed = !b.transposed; }
       const int act = op.fuse_act_relu ? 1 : op.fuse_act_leaky ? 2 : 0;
-      return e.MatMul(a, b, prealloc, act, (float)op.f0);
+      return e.MatMul(a, b, prealloc, act, (float)op.f0, op.fuse_softmax);
     }
     case OpKind::MatVecMul: {
       Tensor a = *in[0];
@@ -561,7 +563,8 @@ int Graph::FuseActivations() {
   for (auto& n : nodes_) {
     if (n.is_input || n.fused_away || n.inputs.empty()) continue;
     const OpKind k = n.op.kind;
-    if (k != OpKind::Rectify && k != OpKind::LeakyRelu && k != OpKind::BatchNorm && k != OpKind::MaxPool2D)
+    if (k != OpKind::Rectify && k != OpKind::LeakyRelu && k != OpKind::BatchNorm && k != OpKind::MaxPool2D &&
+        k != OpKind::SoftMax)
       continue;
     Node& p = nodes_[(size_t)n.inputs[0]];
     if (p.is_input || p.fused_away || p.read_into || uses[(size_t)p.id] != 1) continue;
@@ -569,7 +572,17 @@ int Graph::FuseActivations() {
     OpSpec op = p.op;
     std::vector<int> inputs = p.inputs;
     const bool has_act = op.fuse_act_relu || op.fuse_act_leaky;
-    if (k == OpKind::BatchNorm) {
+    if (op.fuse_softmax) continue;   // nothing rides behind a softmax
+    if (k == OpKind::SoftMax) {
+      if (op.kind != OpKind::MatMul || op.transA || op.transB || n.shape.Dims() != 2) continue;
+      gh_cmd c{};
+      c.opcode = GH_OP_GEMM;
+      c.flags = GH_FLAG_DTYPE(p.dt == Dtype::Float64 ? GH_F64 : GH_F32);
+      c.dim[0] = n.shape[0]; c.dim[1] = n.shape[1]; c.dim[2] = nodes_[(size_t)inputs[0]].shape[1];
+      c.dim[6] = 1;
+      if (!gh_gemm_can_softmax(&c)) continue;
+      op.fuse_softmax = true;
+    } else if (k == OpKind::BatchNorm) {
       if (op.kind != OpKind::Conv2d || op.fuse_bn || has_act || op.fuse_pool2) continue;
       if (n.shape.Dims() != 4) continue;
       op.fuse_bn = true;

@@ -76,6 +76,7 @@ struct OpSpec {
   bool fuse_act_relu = false;
   bool fuse_act_leaky = false;
   bool fuse_pool2 = false;
+  bool fuse_softmax = false;  // MatMul only: the SoftMax that follows, where gh_gemm_can_softmax allows
 };
 
 // Output shape of an op (InferShape of each reference op); error if the inputs

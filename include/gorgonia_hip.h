@@ -129,6 +129,7 @@ enum gh_unaryfn {
 #define GH_FLAG_CONV_BN      (1u << 24)   /* CONV2D: BatchNorm (eval) on the result, ptr[3..6] */
 #define GH_FLAG_BN_EVAL      (1u << 26)   /* BN_BWD: eval-mode gradient dy/sqrt(var+eps)       */
 #define GH_FLAG_CONV_POOL2   (1u << 25)   /* CONV2D: 2x2 stride-2 unpadded MaxPool2D on the result */
+#define GH_FLAG_GEMM_SOFTMAX (1u << 27)   /* GEMM: row SoftMax on the result (after the activation) */
 
 /*
  * One operator.  Field use per opcode:
@@ -251,6 +252,12 @@ GH_API int gh_validate(const gh_cmd* cmds, int n, char* msg, int msg_len);
  * reference has no fused form: this folds maxpool.CUDADo
  * (ops/nn/maxpool_cuda.go:94-111) into convolution.CUDADo (convolution_cuda.go:95-121). */
 GH_API int gh_conv2d_can_pool(const gh_cmd* conv);
+
+/* 1 when this GEMM command may carry GH_FLAG_GEMM_SOFTMAX: a float32 product of
+ * untransposed operands with at most 32 columns and at most 2048 rows, whose
+ * rows are whole inside one workgroup.  The stored values are those of the
+ * SOFTMAX command applied to the plain product. */
+GH_API int gh_gemm_can_softmax(const gh_cmd* gemm);
 /* Engine.DoWork / Signal+Sync (cuda/external.go:223-226): block until the
  * stream drains, return the sticky error. */
 GH_API int gh_sync(gh_ctx* ctx);

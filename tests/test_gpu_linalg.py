@@ -15,13 +15,13 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-5
 
 
-def _run_gemm(ctx, A, B, ta=False, tb=False, act=None, alpha=0.0):
+def _run_gemm(ctx, A, B, ta=False, tb=False, act=None, alpha=0.0, softmax=False):
     m, k = (A.shape[1], A.shape[0]) if ta else A.shape
     n = B.shape[0] if tb else B.shape[1]
     dA, dB = ctx.upload(A), ctx.upload(B)
     dC = ctx.malloc(m * n * 4)
     ctx.run(D.cmd_fill(dC, m * n, np.nan))
-    ctx.run(D.cmd_gemm(dA, dB, dC, m, n, k, trans_a=ta, trans_b=tb, act=act, alpha=alpha))
+    ctx.run(D.cmd_gemm(dA, dB, dC, m, n, k, trans_a=ta, trans_b=tb, act=act, alpha=alpha, softmax=softmax))
     out = ctx.d2h(dC, (m, n))
     for p in (dA, dB, dC):
         ctx.free(p)
@@ -69,6 +69,32 @@ def test_matmul_fused_relu_epilogue(ctx):
     assert_bits_equal(fused, O.relu(plain).reshape(plain.shape), "gemm+relu epilogue")
     fusedl = _run_gemm(ctx, A, B, act="leaky", alpha=0.1)
     assert_bits_equal(fusedl, O.leaky_relu(plain, 0.1).reshape(plain.shape), "gemm+leaky epilogue")
+
+
+@pytest.mark.parametrize("m,k,n", [(128, 625, 10), (1, 32, 1), (33, 100, 32), (2048, 64, 7), (50, 48, 31)])
+def test_matmul_fused_softmax_epilogue(ctx, m, k, n):
+    """MatMul -> SoftMax as one command stores the bits of the two commands."""
+    A = synth.normal(3, (m, k))
+    B = synth.normal(4, (k, n), 0.0, 0.3)
+    assert ctx.lib.gh_gemm_can_softmax(D.cmd_gemm(1, 1, 1, m, n, k)) == 1
+    plain = _run_gemm(ctx, A, B)
+    dx, dy = ctx.upload(plain), ctx.malloc(m * n * 4)
+    ctx.run(D.cmd_softmax(dx, dy, m, n))
+    want = ctx.d2h(dy, (m, n))
+    ctx.free(dx); ctx.free(dy)
+    assert_bits_equal(_run_gemm(ctx, A, B, softmax=True), want, "gemm+softmax epilogue")
+    assert_bits_equal(want, O.softmax(plain), "softmax kernel vs oracle")
+    relu = _run_gemm(ctx, A, B, act="relu", softmax=True)
+    assert_bits_equal(relu, O.softmax(O.relu(plain).reshape(plain.shape)), "gemm+relu+softmax epilogue")
+
+
+def test_matmul_softmax_flag_needs_whole_rows_in_a_tile(ctx):
+    import ctypes as C
+    buf = C.create_string_buffer(256)
+    for cmd in (D.cmd_gemm(1, 1, 1, 64, 33, 64, softmax=True), D.cmd_gemm(1, 1, 1, 64, 10, 16, softmax=True),
+                D.cmd_gemm(1, 1, 1, 64, 10, 64, trans_b=True, softmax=True), D.cmd_gemm(1, 1, 1, 4096, 10, 64, softmax=True)):
+        assert ctx.lib.gh_gemm_can_softmax(cmd) == 0
+        assert ctx.lib.gh_validate(C.byref(cmd), 1, buf, 256) != 0 and b"softmax" in buf.value
 
 
 def test_matmul_strided_ld(ctx):

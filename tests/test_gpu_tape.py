@@ -47,7 +47,7 @@ def test_convnet_forward_fused_and_unfused(ctx):
     m2, _, r2 = run_once(configs.build_convnet, inp, fuse_activations=True)
     assert rel_frobenius(r1["out"], want) <= 1e-5
     assert_bits_equal(r1["out"], r2["out"], "fused activations change nothing")
-    assert m2.fused == 7  # 4 activations + the three pools
+    assert m2.fused == 8  # 4 activations, the three pools and the softmax
     m1.Close(); m2.Close()
 
 

@@ -151,7 +151,7 @@ def test_tape_program_convnet_fusion():
     inp = configs.convnet_inputs(2)
     g, _ = configs.build_convnet(inp)
     m = G.NewTapeMachine(g, compile_only=True, fuse_activations=True)
-    assert m.fused == 7  # 4 activations + the three pools
+    assert m.fused == 8  # 4 activations, the three pools and the softmax
     prog = m.program()
     assert prog.count("conv2d+rectify") == 3 and prog.count(" rectify") == 0
     assert prog.count("maxpool2d") == 3 and prog.count("softmax") == 1
