@@ -131,14 +131,14 @@ def bench_linalg(ctx, iters):
     return res
 
 
-# HBM bytes per launch of each conv layer's kernels (the split-K reduce
-# included), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
-# (KiB per dispatch; FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0, the factors a
-# 64 MiB device copy in the same runs gives).
+# HBM bytes per launch of each conv layer's kernel as the step issues it (conv +
+# ReLU + 2x2 max-pool in one launch), from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs of this script (KiB per dispatch; FETCH_SIZE scaled by 2.0,
+# WRITE_SIZE by 1.0, the factors a 64 MiB device copy in the same runs gives).
 MEASURED_TRAFFIC_BYTES = {
-    "conv0": (2 * 284.3 + 12544.0) * 1024,
-    "conv1": (2 * 4496.5 + 6784.0) * 1024,
-    "conv2": (2 * 4069.0 + 6272.0 + 2 * 3160.0 + 3360.0) * 1024,
+    "conv0": (2 * 929.7 + 3232.0) * 1024,
+    "conv1": (2 * 4351.7 + 2464.0) * 1024,
+    "conv2": (2 * 2108.3 + 576.0) * 1024,
 }
 
 CONVNET_LAYERS = [  # (name, B-relative shape) of configuration 4
@@ -147,18 +147,22 @@ CONVNET_LAYERS = [  # (name, B-relative shape) of configuration 4
 
 
 def bench_convnet_kernels(ctx, batch, iters):
-    """Per-kernel time of the conv layers of the convnet step (for the roofline object)."""
+    """Per-kernel time of the conv layers of the convnet step (for the roofline object):
+    the commands the step itself issues - conv + ReLU + 2x2 max-pool in one launch where
+    the library offers it.  FLOPs are the convolution's own (2*B*oh*ow*F*C*9)."""
     from gorgonia_amd import device as D, synth
     out = {}
     for name, cin, hw, f in CONVNET_LAYERS:
         x = ctx.upload(synth.uniform01(1, (batch * cin * hw * hw,)))
         w = ctx.upload(synth.normal(2, (f * cin * 9,)))
         y = ctx.malloc(batch * f * hw * hw * 4)
-        ms = time_cmds(ctx, [D.cmd_conv2d(x, w, y, batch, cin, hw, hw, f, 3, 3, (1, 1), act="relu")], iters)
+        pool = bool(ctx.lib.gh_conv2d_can_pool(D.cmd_conv2d(x, w, y, batch, cin, hw, hw, f, 3, 3, (1, 1))))
+        ms = time_cmds(ctx, [D.cmd_conv2d(x, w, y, batch, cin, hw, hw, f, 3, 3, (1, 1), act="relu", pool2=pool)], iters)
         fl = 2.0 * batch * hw * hw * f * cin * 9
-        nb = 4 * (batch * cin * hw * hw + f * cin * 9 + batch * f * hw * hw)
+        out_hw = (hw // 2) if pool else hw
+        nb = 4 * (batch * cin * hw * hw + f * cin * 9 + batch * f * out_hw * out_hw)
         out[name] = {"us": round(ms * 1e3, 2), "TFLOPs": round(fl / ms / 1e9, 2), "flop": fl,
-                     "GBps": round(nb / ms / 1e6, 1), "bytes": nb}
+                     "GBps": round(nb / ms / 1e6, 1), "bytes": nb, "pool_fused": pool}
         for q in (x, w, y):
             ctx.free(q)
     return out
@@ -371,8 +375,9 @@ def main():
     if conv_k:
         name = max(conv_k, key=lambda k: conv_k[k]["us"])
         r = conv_k[name]
-        kname = "k_conv3x3_direct" if name == "conv0" else "k_conv3x3_lds (+ k_splitk_reduce)"
-        roofline = {"kernel": f"{kname}: {name} of the convnet step with ReLU in the epilogue", "bound": "mfma",
+        kname = "k_conv3x3_direct" if name == "conv0" else "k_conv3x3_lds"
+        tail = "ReLU and the 2x2 max-pool in the epilogue" if r["pool_fused"] else "ReLU in the epilogue"
+        roofline = {"kernel": f"{kname}: {name} of the convnet step with {tail}", "bound": "mfma",
                     "achieved": r["TFLOPs"], "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(r["TFLOPs"] / MFMA_F32_PEAK_TFLOPS, 4),
                     "traffic": int(MEASURED_TRAFFIC_BYTES[name]),
