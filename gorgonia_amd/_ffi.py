@@ -22,7 +22,7 @@ ERR_NAMES = {0: "GH_OK", 1: "GH_EINVAL", 2: "GH_EDEVICE", 3: "GH_EOOM", 4: "GH_E
  OP_FILL, OP_MAXPOOL2D_BWD, OP_CONV2D_BWD_DATA, OP_CONV2D_BWD_FILTER, OP_BN_TRAIN, OP_BN_BWD,
  OP_SOFTMAX_BWD, OP_SOLVER_STEP, OP_RAND_UNIFORM, OP_DROPOUT, OP_DROPOUT_BWD) = range(27)
 
-BIN_FN = {"add": 0, "sub": 1, "mul": 2, "div": 3, "pow": 4, "lt": 5, "lte": 6, "gt": 7, "gte": 8,
+BIN_FN = {"mod": 11, "add": 0, "sub": 1, "mul": 2, "div": 3, "pow": 4, "lt": 5, "lte": 6, "gt": 7, "gte": 8,
           "eq": 9, "ne": 10}
 MODE = {"vv": 0, "vs": 1, "sv": 2, "ss": 3}
 F32, F64 = 0, 1

@@ -65,10 +65,12 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
       if (!pos(c.dim[0]) || !pos(c.dim[1])) return bad("gemv: m, n must be positive");
       if (c.dim[2] < c.dim[1]) return bad("gemv: lda too small");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     case GH_OP_OUTER:
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
       if (!pos(c.dim[0]) || !pos(c.dim[1])) return bad("outer: m, n must be positive");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     case GH_OP_CONV2D_BWD_DATA:
     case GH_OP_CONV2D_BWD_FILTER:
@@ -187,11 +189,11 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
 // The reference names kernels "<module>.<fn>_<mode>_f<bits>" for binary ops
 // (cuda/utils.go:114-139) and "<module>.<fn>_f<bits>" for unary ops
 // (op_math_cuda.go:38).  "mod" is declared by the engine
-// (cuda/arith.go:589-701) but its kernel is absent from elembinop.cu:201-210;
-// it is absent here too, so HasFunc reports false for it as in the reference.
+// (cuda/arith.go:589-701) but its kernel is absent from elembinop.cu:201-210,
+// so HasFunc is false for it there; here the kernel exists.
 
 static const char* kBinNames[GH_BINFN__COUNT] = {"add", "sub", "mul", "div", "pow", "lt",
-                                                 "lte", "gt",  "gte", "eq",  "ne"};
+                                                 "lte", "gt",  "gte", "eq",  "ne",  "mod"};
 static const char* kModeNames[4] = {"vv", "vs", "sv", "ss"};
 // Kernel-file names (elemunaryop.cu:109-193) ...
 static const char* kUnaryNames[GH_UNARYFN__COUNT] = {

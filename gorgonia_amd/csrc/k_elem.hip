@@ -38,6 +38,7 @@ __device__ __forceinline__ T bin_apply(T a, T b) {
   else if constexpr (FN == GH_GT) return a > b ? (T)1 : (T)0;
   else if constexpr (FN == GH_GTE) return a >= b ? (T)1 : (T)0;
   else if constexpr (FN == GH_EQ) return a == b ? (T)1 : (T)0;
+  else if constexpr (FN == GH_MOD) return (T)fmod((double)a, (double)b);   // exact in either width
   else return a != b ? (T)1 : (T)0;
 }
 
@@ -553,6 +554,7 @@ int launch_bin(gh_ctx* ctx, const gh_cmd& c) {
     case GH_GTE: return launch_bin_fn<GH_GTE, T>(ctx, c);
     case GH_EQ: return launch_bin_fn<GH_EQ, T>(ctx, c);
     case GH_NE: return launch_bin_fn<GH_NE, T>(ctx, c);
+    case GH_MOD: return launch_bin_fn<GH_MOD, T>(ctx, c);
   }
   return gh_fail(ctx, GH_ENOFUNC, "unknown binary function");
 }
@@ -647,6 +649,7 @@ int gh_launch_bcast_bin(gh_ctx* ctx, const gh_cmd& c) {
     case GH_GTE: return launch_bcast_fn<GH_GTE>(ctx, c);
     case GH_EQ: return launch_bcast_fn<GH_EQ>(ctx, c);
     case GH_NE: return launch_bcast_fn<GH_NE>(ctx, c);
+    case GH_MOD: return launch_bcast_fn<GH_MOD>(ctx, c);
   }
   return gh_fail(ctx, GH_ENOFUNC, "unknown binary function");
 }

@@ -1384,6 +1384,36 @@ __global__ __launch_bounds__(256) void k_outer(const float* __restrict__ x,
     A[i] = x[i / n] * y[i % n];
 }
 
+// float64 twins (Dgemv / Dger, cuda/linalg.go:94-159): same shapes, plain loads.
+__global__ __launch_bounds__(256) void k_dgemv_n(const double* __restrict__ A, const double* __restrict__ x,
+                                                 double* __restrict__ y, int m, int n, int lda) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= m) return;
+  const double* a = A + (int64_t)row * lda;
+  double acc = 0.0;
+  for (int i = lane; i < n; i += 64) acc += a[i] * x[i];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (lane == 0) y[row] = acc;
+}
+
+__global__ __launch_bounds__(256) void k_dgemv_t(const double* __restrict__ A, const double* __restrict__ x,
+                                                 double* __restrict__ y, int m, int n, int lda) {
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  if (col >= n) return;
+  double acc = 0.0;
+  for (int r = 0; r < m; r++) acc += A[(int64_t)r * lda + col] * x[r];
+  y[col] = acc;
+}
+
+__global__ __launch_bounds__(256) void k_douter(const double* __restrict__ x, const double* __restrict__ y,
+                                                double* __restrict__ A, int64_t m, int64_t n) {
+  const int64_t total = m * n, stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride)
+    A[i] = x[i / n] * y[i % n];
+}
+
 inline bool al16(uint64_t p) { return (p & 15u) == 0; }
 
 // ---- tile plan -------------------------------------------------------------------
@@ -1943,6 +1973,16 @@ int gh_launch_conv2d_bwd_data(gh_ctx* ctx, const gh_cmd& c) {
 
 int gh_launch_gemv(gh_ctx* ctx, const gh_cmd& c) {
   const int m = (int)c.dim[0], n = (int)c.dim[1], lda = (int)c.dim[2];
+  if (gh_dtype_of(c.flags) == GH_F64) {
+    const double* A = (const double*)(uintptr_t)c.ptr[0];
+    const double* x = (const double*)(uintptr_t)c.ptr[1];
+    double* y = (double*)(uintptr_t)c.ptr[2];
+    if (c.flags & GH_FLAG_TRANS_A)
+      hipLaunchKernelGGL(k_dgemv_t, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, A, x, y, m, n, lda);
+    else
+      hipLaunchKernelGGL(k_dgemv_n, dim3((m + 3) / 4), dim3(256), 0, ctx->stream, A, x, y, m, n, lda);
+    return gh_check_hip(ctx, hipGetLastError(), "dgemv launch");
+  }
   const float* A = (const float*)(uintptr_t)c.ptr[0];
   const float* x = (const float*)(uintptr_t)c.ptr[1];
   float* y = (float*)(uintptr_t)c.ptr[2];
@@ -1959,6 +1999,12 @@ int gh_launch_outer(gh_ctx* ctx, const gh_cmd& c) {
   const int64_t m = c.dim[0], n = c.dim[1];
   int64_t blocks = (m * n + 1023) / 1024;
   if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
+  if (gh_dtype_of(c.flags) == GH_F64) {
+    hipLaunchKernelGGL(k_douter, dim3((int)blocks), dim3(256), 0, ctx->stream,
+                       (const double*)(uintptr_t)c.ptr[0], (const double*)(uintptr_t)c.ptr[1],
+                       (double*)(uintptr_t)c.ptr[2], m, n);
+    return gh_check_hip(ctx, hipGetLastError(), "outer launch");
+  }
   hipLaunchKernelGGL(k_outer, dim3((int)blocks), dim3(256), 0, ctx->stream,
                      (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
                      (float*)(uintptr_t)c.ptr[2], m, n);

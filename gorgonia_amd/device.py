@@ -174,13 +174,13 @@ def cmd_gemm(a, b, c, m, n, k, lda=None, ldb=None, ldc=None, trans_a=False, tran
                                                   stride_c), (alpha,))
 
 
-def cmd_gemv(a, x, y, m, n, lda=None, trans=False):
-    return make_cmd(_ffi.OP_GEMV, _ffi.FLAG_TRANS_A if trans else 0, (a, x, y),
+def cmd_gemv(a, x, y, m, n, lda=None, trans=False, dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_GEMV, (_ffi.FLAG_TRANS_A if trans else 0) | _ffi.flag_dtype(dtype), (a, x, y),
                     (m, n, lda if lda is not None else n))
 
 
-def cmd_outer(x, y, a, m, n):
-    return make_cmd(_ffi.OP_OUTER, 0, (x, y, a), (m, n))
+def cmd_outer(x, y, a, m, n, dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_OUTER, _ffi.flag_dtype(dtype), (x, y, a), (m, n))
 
 
 def cmd_conv2d(x, w, y, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dilation=(1, 1),

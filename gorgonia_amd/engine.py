@@ -161,7 +161,7 @@ class Tensor:
         return d
 
 
-BIN_FN = dict(_ffi.BIN_FN, mod=11)
+BIN_FN = dict(_ffi.BIN_FN)
 
 
 class Engine:
@@ -303,8 +303,7 @@ for _go, _fn in [("Add", "add"), ("Sub", "sub"), ("Mul", "mul"), ("Div", "div"),
                  ("ElNe", "ne"), ("Mod", "mod")]:
     _tt, _ts = _mk(_fn)
     setattr(Engine, _go, _tt)
-    if _fn != "mod":
-        setattr(Engine, _go + "Scalar", _ts)
+    setattr(Engine, _go + "Scalar", _ts)
 
 
 class BFC:

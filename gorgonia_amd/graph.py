@@ -114,6 +114,7 @@ def _bc(fn):
 # api_gen.go names
 Add, Sub, HadamardProd, HadamardDiv, Pow = _bin("add"), _bin("sub"), _bin("mul"), _bin("div"), _bin("pow")
 Lt, Lte, Gt, Gte, Eq, Ne = _bin("lt"), _bin("lte"), _bin("gt"), _bin("gte"), _bin("eq"), _bin("ne")
+Mod = _bin("mod")
 BroadcastAdd, BroadcastSub = _bc("add"), _bc("sub")
 BroadcastHadamardProd, BroadcastHadamardDiv = _bc("mul"), _bc("div")
 Abs, Sign, Ceil, Floor, Sin, Cos, Exp, Log, Log2 = (_un(n) for n in

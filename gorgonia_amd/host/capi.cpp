@@ -119,8 +119,8 @@ int ghh_engine_binop(ghh_engine* e, int fn, const ghh_tensor* a, const ghh_tenso
 int ghh_engine_binop_scalar(ghh_engine* e, int fn, const ghh_tensor* a, uint64_t b_mem, int left_tensor,
                             const ghh_tensor* reuse, int safe, uint64_t* ret_mem) {
   static const char* names[] = {"AddScalar", "SubScalar", "MulScalar", "DivScalar", "PowScalar", "LtScalar",
-                                "LteScalar", "GtScalar", "GteScalar", "ElEqScalar", "ElNeScalar"};
-  if (fn < 0 || fn > 10) { e->err = "unknown function"; return GH_ENOFUNC; }
+                                "LteScalar", "GtScalar", "GteScalar", "ElEqScalar", "ElNeScalar", "ModScalar"};
+  if (fn < 0 || fn > 11) { e->err = "unknown function"; return GH_ENOFUNC; }
   Tensor ta = to_tensor(a), tr;
   if (reuse) tr = to_tensor(reuse);
   FuncOpts o = make_opts(reuse ? &tr : nullptr, safe, 0);

@@ -225,7 +225,7 @@ static std::string binName(const char* fn, int mode, Dtype dt) {
 }
 
 static const char* kFnNames[GH_BINFN__COUNT] = {"add", "sub", "mul", "div", "pow", "lt",
-                                                "lte", "gt",  "gte", "eq",  "ne"};
+                                                "lte", "gt",  "gte", "eq",  "ne",  "mod"};
 
 // Destination selection shared by all arithmetic methods (cuda/arith.go:34-49):
 // with a reuse tensor the result lands there and a is left alone (the
@@ -300,11 +300,8 @@ Status Engine::BinOpScalar(int fn, const char* go_name, Tensor& a, uint64_t b_me
   return Status::OK();
 }
 
-Status Engine::Mod(Tensor& a, Tensor& b, const FuncOpts&, Tensor**) {
-  const int mode = a.shape.IsScalar() ? (b.shape.IsScalar() ? GH_SS : GH_SV)
-                                      : (b.shape.IsScalar() ? GH_VS : GH_VV);
-  return Status::Err(GH_ENOFUNC, "Unable to perform Mod(). The tensor engine does not have the function \"" +
-                                     binName("mod", mode, a.dt) + "\"");
+Status Engine::Mod(Tensor& a, Tensor& b, const FuncOpts& o, Tensor** ret) {
+  return BinOp(GH_MOD, "Mod", a, b, o, ret);
 }
 
 Status Engine::UnaryTo(const std::string& op_name, Tensor& a, uint64_t dst_mem) {
@@ -382,7 +379,7 @@ static Status checkThreeFloat(const Tensor& a, const Tensor& b, const Tensor& re
 Status Engine::MatVecMul(Tensor& a, Tensor& b, Tensor& prealloc) {
   Status st = checkThreeFloat(a, b, prealloc);
   if (!st.ok()) return st.Wrap("MatVecMul failed pre check");
-  if (a.dt != Dtype::Float32) return Status::Err(GH_EINVAL, "Unsupported Dtype");
+  if (a.dt == Dtype::Other) return Status::Err(GH_EINVAL, "Unsupported Dtype");
   if (a.shape.Dims() != 2) return Status::Err(GH_EINVAL, "MatVecMul: a must be a matrix");
   const int64_t m = a.shape[0], n = a.shape[1];  // logical shape
   if (b.DataSize() != n || prealloc.DataSize() != m)
@@ -390,8 +387,9 @@ Status Engine::MatVecMul(Tensor& a, Tensor& b, Tensor& prealloc) {
   gh_cmd c{};
   c.opcode = GH_OP_GEMV;
   c.ptr[0] = a.mem; c.ptr[1] = b.mem; c.ptr[2] = prealloc.mem;
+  c.flags = GH_FLAG_DTYPE(a.dt == Dtype::Float64 ? GH_F64 : GH_F32);  // Dgemv / Sgemv, cuda/linalg.go:94-127
   if (a.transposed) {  // stored (n x m) row-major: y = A_stored^T x
-    c.flags = GH_FLAG_TRANS_A;
+    c.flags |= GH_FLAG_TRANS_A;
     c.dim[0] = n; c.dim[1] = m; c.dim[2] = m;
   } else {
     c.dim[0] = m; c.dim[1] = n; c.dim[2] = n;
@@ -435,12 +433,13 @@ Status Engine::MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act, float alp
 Status Engine::Outer(Tensor& a, Tensor& b, Tensor& prealloc) {
   Status st = checkThreeFloat(a, b, prealloc);
   if (!st.ok()) return st.Wrap("Outer failed pre check");
-  if (a.dt != Dtype::Float32) return Status::Err(GH_EINVAL, "Unsupported Dtype");
+  if (a.dt == Dtype::Other) return Status::Err(GH_EINVAL, "Unsupported Dtype");
   const int64_t m = a.DataSize(), n = b.DataSize();
   if (prealloc.DataSize() != m * n)
     return Status::Err(GH_EINVAL, fmt2(kShapeMismatch, Shape{m, n}.String(), prealloc.shape.String()));
   gh_cmd c{};
   c.opcode = GH_OP_OUTER;
+  c.flags = GH_FLAG_DTYPE(a.dt == Dtype::Float64 ? GH_F64 : GH_F32);  // Dger / Sger, cuda/linalg.go:129-159
   c.ptr[0] = a.mem; c.ptr[1] = b.mem; c.ptr[2] = prealloc.mem;
   c.dim[0] = m; c.dim[1] = n;
   Enqueue(c);

@@ -132,7 +132,7 @@ class Engine {
   GORGONIA_BINOP(Lte, GH_LTE) GORGONIA_BINOP(Gt, GH_GT) GORGONIA_BINOP(Gte, GH_GTE)
   GORGONIA_BINOP(ElEq, GH_EQ) GORGONIA_BINOP(ElNe, GH_NE)
 #undef GORGONIA_BINOP
-  // Mod is declared by the reference engine but has no kernel
+  // Mod: the reference engine declares it but ships no kernel; here it runs
   // (cuda/arith.go:589-701, elembinop.cu:201-210): same error here.
   Status Mod(Tensor& a, Tensor& b, const FuncOpts& o, Tensor** ret = nullptr);
 

@@ -249,7 +249,7 @@ int OverwritesInput(const OpSpec& op) {
 }
 
 static std::string op_name(const OpSpec& op) {
-  static const char* bins[] = {"add", "sub", "mul", "div", "pow", "lt", "lte", "gt", "gte", "eq", "ne"};
+  static const char* bins[] = {"add", "sub", "mul", "div", "pow", "lt", "lte", "gt", "gte", "eq", "ne", "mod"};
   switch (op.kind) {
     case OpKind::ElemBin: return std::string("elembin.") + bins[op.fn];
     case OpKind::ElemUnary: return "elemunary." + op.name;

@@ -101,6 +101,8 @@ enum gh_solver { GH_SOLVER_VANILLA = 0, GH_SOLVER_RMSPROP = 1, GH_SOLVER_ADAM = 
 enum gh_binfn {
   GH_ADD = 0, GH_SUB = 1, GH_MUL = 2, GH_DIV = 3, GH_POW = 4,
   GH_LT = 5, GH_LTE = 6, GH_GT = 7, GH_GTE = 8, GH_EQ = 9, GH_NE = 10,
+  GH_MOD = 11, /* Engine.Mod / ModScalar (cuda/arith.go:589-701): the reference declares the
+                  methods but ships no "mod" kernel, so they fail there; math.Mod semantics */
   GH_BINFN__COUNT
 };
 enum gh_binmode { GH_VV = 0, GH_VS = 1, GH_SV = 2, GH_SS = 3 };

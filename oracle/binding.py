@@ -12,7 +12,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "liboracle.so")
 
-BIN = {"add": 0, "sub": 1, "mul": 2, "div": 3, "pow": 4, "lt": 5, "lte": 6, "gt": 7, "gte": 8,
+BIN = {"mod": 11, "add": 0, "sub": 1, "mul": 2, "div": 3, "pow": 4, "lt": 5, "lte": 6, "gt": 7, "gte": 8,
        "eq": 9, "ne": 10}
 MODE = {"vv": 0, "vs": 1, "sv": 2, "ss": 3}
 UNARY = {"abs": 0, "sign": 1, "ceil": 2, "floor": 3, "sin": 4, "cos": 5, "exp": 6, "ln": 7,

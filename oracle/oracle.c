@@ -87,7 +87,7 @@ EXPORT int oracle_get_threads(void) { return g_threads; }
 /* comparisons return 1/0 in the operand dtype (retSame,               */
 /* operatorPointwise_binary.go:305-317).                               */
 /* op codes: 0 add 1 sub 2 mul 3 div 4 pow 5 lt 6 lte 7 gt 8 gte 9 eq  */
-/*           10 ne                                                     */
+/*           10 ne   11 mod (Go's math.Mod = C fmod: sign of the dividend) */
 /* ------------------------------------------------------------------ */
 
 static inline float binop_f32(int op, float a, float b) {
@@ -103,6 +103,7 @@ static inline float binop_f32(int op, float a, float b) {
     case 8: return a >= b ? 1.0f : 0.0f;
     case 9: return a == b ? 1.0f : 0.0f;
     case 10: return a != b ? 1.0f : 0.0f;
+    case 11: return (float)fmod((double)a, (double)b); /* math32.Mod: math.Mod in float64, exact */
   }
   return NAN;
 }
@@ -120,6 +121,7 @@ static inline double binop_f64(int op, double a, double b) {
     case 8: return a >= b ? 1.0 : 0.0;
     case 9: return a == b ? 1.0 : 0.0;
     case 10: return a != b ? 1.0 : 0.0;
+    case 11: return fmod(a, b); /* math.Mod */
   }
   return NAN;
 }

@@ -33,7 +33,7 @@ def test_kernel_name_registry():
     """Names built by constructName2/constructName1 (cuda/utils.go:114-139) and
     by elemUnaryOp.CUDADo (op_math_cuda.go:38)."""
     lib = _ffi.load()
-    for fn in ["add", "sub", "mul", "div", "pow", "lt", "lte", "gt", "gte", "eq", "ne"]:
+    for fn in ["add", "sub", "mul", "div", "pow", "lt", "lte", "gt", "gte", "eq", "ne", "mod"]:
         for mode in ["vv", "vs", "sv", "ss"]:
             for bits in (32, 64):
                 assert lib.gh_has_func(f"elembinop.{fn}_{mode}_f{bits}".encode()) == 1
@@ -42,8 +42,7 @@ def test_kernel_name_registry():
                "softplus"]:
         assert lib.gh_has_func(f"elemunaryop.{fn}_f32".encode()) == 1, fn
     assert lib.gh_has_func(b"misc.hasNaN_f32") == 1 and lib.gh_has_func(b"misc.hasInf_f64") == 1
-    # mod is declared by the reference engine but has no kernel (elembinop.cu:201-210)
-    assert lib.gh_has_func(b"elembinop.mod_vv_f32") == 0
+    # (mod is declared by the reference engine without a kernel, elembinop.cu:201-210; it has one here)
     assert lib.gh_has_func(b"elembinop.add_vv_f16") == 0
     assert lib.gh_has_func(b"nosuch.add_vv_f32") == 0
     op, fl = C.c_uint32(), C.c_uint32()

@@ -6,6 +6,7 @@ Bars: add/sub/mul/div/compare/relu/leaky/broadcast bit-exact; exp/tanh/sigmoid
 import numpy as np
 import pytest
 
+from gorgonia_amd import _ffi
 from gorgonia_amd import device as D
 from gorgonia_amd import synth
 from oracle import binding as O
@@ -89,6 +90,30 @@ def test_pow_scalar_two_is_exact_square(ctx):
     assert_bits_equal(got, O.binop("pow", "vs", a, two), "pow(x,2) vs oracle")
     assert_bits_equal(got, a * a, "pow(x,2) == x*x")
     ctx.free(da); ctx.free(db)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_mod_bit_exact(ctx, dtype):
+    """Engine.Mod (cuda/arith.go:589-640): math.Mod semantics, exact in both widths."""
+    n = 100_003
+    a = (synth.uniform(31, (n,), -50, 50)).astype(dtype)
+    b = (synth.uniform(32, (n,), -7, 7)).astype(dtype)
+    special = np.array([0.0, -0.0, 5.5, -5.5, np.inf, -np.inf, np.nan, 1e30, 3.0], dtype=dtype)
+    a[:81] = np.repeat(special, 9)
+    b[:81] = np.tile(special, 9)
+    dt = _ffi.F32 if dtype == np.float32 else _ffi.F64
+    for mode in ("vv", "vs", "sv"):
+        A = a.copy() if mode != "sv" else a[:1].copy()
+        B = b.copy() if mode != "vs" else b[3:4].copy()
+        da, db = ctx.upload(A), ctx.upload(B)
+        ctx.run(D.cmd_bin("mod", mode, da, db, n, dtype=dt))
+        got = ctx.d2h(db if mode == "sv" else da, (n,), dtype)
+        ctx.free(da); ctx.free(db)
+        want = O.binop("mod", mode, A, B)
+        assert_bits_equal(got, want, f"mod {mode} {dtype.__name__}")
+        with np.errstate(invalid="ignore", divide="ignore"):
+            ref = np.fmod(A if mode != "sv" else np.full(n, A[0], dtype), B if mode != "vs" else np.full(n, B[0], dtype))
+        assert_bits_equal(got, ref.astype(dtype), f"mod {mode} against fmod")
 
 
 def test_pow_general(ctx):

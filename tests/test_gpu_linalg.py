@@ -174,6 +174,32 @@ def test_outer_bit_exact(ctx):
         ctx.free(p)
 
 
+@pytest.mark.parametrize("m,n,trans", [(64, 64, False), (300, 784, False), (100, 300, True), (5, 3, True), (1, 1, False)])
+def test_matvec_and_outer_float64(ctx, m, n, trans):
+    """Dgemv / Dger paths of Engine.MatVecMul / Outer (cuda/linalg.go:94-159)."""
+    from gorgonia_amd import _ffi
+    A = synth.normal(7, (m, n)).astype(np.float64) + 1e-9 * synth.normal(17, (m, n)).astype(np.float64)
+    x = synth.normal(8, (m if trans else n,)).astype(np.float64)
+    dA, dx = ctx.upload(A), ctx.upload(x)
+    dy = ctx.malloc((n if trans else m) * 8)
+    ctx.run(D.cmd_gemv(dA, dx, dy, m, n, trans=trans, dtype=_ffi.F64))
+    got = ctx.d2h(dy, (n if trans else m,), np.float64)
+    ref = (A.T if trans else A) @ x
+    assert rel_frobenius(got, ref) <= 1e-13
+    Ai = np.round(A * 4)
+    xi = np.round(x * 4)
+    ctx.h2d(dA, Ai); ctx.h2d(dx, xi)
+    ctx.run(D.cmd_gemv(dA, dx, dy, m, n, trans=trans, dtype=_ffi.F64))
+    assert np.array_equal(ctx.d2h(dy, (n if trans else m,), np.float64), (Ai.T if trans else Ai) @ xi)
+    # outer: one product per element, exact
+    y = synth.normal(9, (n,)).astype(np.float64) * 1.000000001
+    dyv, dO = ctx.upload(y), ctx.malloc(x.size * n * 8)
+    ctx.run(D.cmd_outer(dx, dyv, dO, x.size, n, dtype=_ffi.F64))
+    assert_bits_equal(ctx.d2h(dO, (x.size, n), np.float64), np.multiply.outer(xi, y), "float64 outer")
+    for p in (dA, dx, dy, dyv, dO):
+        ctx.free(p)
+
+
 @pytest.mark.parametrize("ta", [False, True])
 @pytest.mark.parametrize("tb", [False, True])
 def test_matmul_float64(ctx, ta, tb):

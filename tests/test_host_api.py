@@ -54,9 +54,10 @@ def test_binary_checks(eng):
         eng.Add(T((4,)), T((4,)), reuse=T((3,), mem=0x2000))
     with pytest.raises(EngineError, match="Cannot use reuse: TypeMismatch"):
         eng.Add(T((4,)), T((4,)), reuse=T((4,), np.float64, mem=0x2000))
-    # mod has no kernel (elembinop.cu:201-210)
-    with pytest.raises(EngineError, match=r'does not have the function "elembinop.mod_vv_f32"'):
-        eng.Mod(T((4,)), T((4,)), unsafe=True)
+    # the reference's Mod stops at "does not have the function" (no kernel in elembinop.cu:201-210);
+    # here it goes through the same checks as every other binary method
+    with pytest.raises(EngineError, match=r"Basic checks failed for Mod: Shape mismatch"):
+        eng.Mod(T((2,)), T((4,)), unsafe=True)
     with pytest.raises(EngineError, match="b has to be a tensor.Memory"):
         eng.AddScalar(T((4,)), None, True, unsafe=True)
     # a valid call only records a command
@@ -84,7 +85,7 @@ def test_linalg_checks(eng):
 
 def test_has_func_and_unknown_unary(eng):
     assert eng.HasFunc("elembinop.add_vv_f32") and eng.HasFunc("elemunaryop.tanh_f64")
-    assert not eng.HasFunc("elembinop.mod_vv_f32")
+    assert eng.HasFunc("elembinop.mod_vv_f32") and eng.HasFunc("elembinop.mod_sv_f64")
     with pytest.raises(EngineError, match="does not have the function"):
         eng.Unary("erf", T((4,)))
     assert eng.AllocAccessible() is False

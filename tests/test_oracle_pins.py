@@ -331,3 +331,26 @@ def test_has_nan_inf():
     assert O.has_nan(a) and not O.has_inf(a)
     a[7] = -np.inf
     assert O.has_inf(a) and not O.has_nan(a)
+
+
+def test_mod_is_go_math_mod():
+    """math.Mod's documented special cases (Go standard library, math/mod.go: Mod(±Inf, y) = NaN,
+    Mod(NaN, y) = NaN, Mod(x, 0) = NaN, Mod(x, ±Inf) = x, Mod(x, NaN) = NaN; the result takes
+    the sign of x) and exactness: x - trunc(x/y)*y evaluated in integers."""
+    from oracle import binding as O
+    f = np.float32
+    a = np.array([7.5, -7.5, 7.5, -7.5, 5.0, np.inf, -np.inf, np.nan, 3.0, 3.0, -3.0, 3.0, 0.0, -0.0], f)
+    b = np.array([2.0, 2.0, -2.0, -2.0, 0.0, 2.0, 2.0, 2.0, np.inf, -np.inf, np.inf, np.nan, 3.0, 3.0], f)
+    got = O.binop("mod", "vv", a, b)
+    want = np.array([1.5, -1.5, 1.5, -1.5, np.nan, np.nan, np.nan, np.nan, 3.0, 3.0, -3.0, np.nan, 0.0, -0.0], f)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32))
+    # exact remainders on integers scaled by powers of two
+    rng = np.random.default_rng(5)
+    x = rng.integers(-10**6, 10**6, 5000)
+    y = rng.integers(1, 5000, 5000) * rng.choice([-1, 1], 5000)
+    for dt, scale in ((np.float32, 0.25), (np.float64, 2.0 ** -20)):
+        r = O.binop("mod", "vv", (x * scale).astype(dt), (y * scale).astype(dt))
+        exact = np.sign(x) * (np.abs(x) % np.abs(y)) * scale
+        assert np.array_equal(r, exact.astype(dt))
