@@ -59,6 +59,12 @@ int gh_launch_bn_bwd(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_softmax_bwd(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_solver_step(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_rand_uniform(gh_ctx* ctx, const gh_cmd& c);
+// float64 twins of the forward neural-network operators (k_nn64.hip)
+int gh_launch_relu_f64(gh_ctx* ctx, const gh_cmd& c, bool leaky);
+int gh_launch_maxpool2d_f64(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_bn_infer_f64(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_softmax_f64(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_conv2d_f64(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_dropout(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_dropout_bwd(gh_ctx* ctx, const gh_cmd& c);
 

@@ -98,6 +98,10 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
         if ((c.flags & GH_FLAG_HAS_GAMMA) && !c.ptr[5]) return bad("conv2d: fused BatchNorm gamma is null");
         if ((c.flags & GH_FLAG_HAS_BETA) && !c.ptr[6]) return bad("conv2d: fused BatchNorm beta is null");
       }
+      if (dt > GH_F64) return bad("Unsupported Dtype");
+      if (dt == GH_F64 && c.opcode != GH_OP_CONV2D) return bad("conv2d backward: float32 only");
+      if (dt == GH_F64 && (c.flags & (GH_FLAG_CONV_BN | GH_FLAG_CONV_POOL2 | GH_FLAG_ACT_RELU | GH_FLAG_ACT_LEAKY)))
+        return bad("conv2d: no epilogue operators for float64");
       if ((c.flags & GH_FLAG_CONV_POOL2) && !gh_conv2d_can_pool(&c))
         return bad("conv2d: no fused pooling for this shape");
       return GH_OK;
@@ -118,6 +122,7 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
         return bad("Impossible width/kernel/pad combination");
       if (c.dim[0] * c.dim[1] * c.dim[2] * c.dim[3] > INT32_MAX)
         return bad("maxpool2d: tensor too large for 32-bit indexing");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     }
     case GH_OP_BN_INFER:
@@ -125,6 +130,7 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if ((c.flags & GH_FLAG_HAS_GAMMA) && !c.ptr[4]) return bad("null gamma");
       if ((c.flags & GH_FLAG_HAS_BETA) && !c.ptr[5]) return bad("null beta");
       if (!pos(c.dim[0]) || !pos(c.dim[1]) || !pos(c.dim[2])) return bad("bn: B,C,S must be positive");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     case GH_OP_BN_TRAIN:
       for (int i = 0; i < 6; i++)
@@ -165,10 +171,12 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
     case GH_OP_LEAKY_RELU:
       if (!c.ptr[0] || !c.ptr[1]) return bad("null operand");
       if (c.dim[0] < 0) return bad("negative size");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     case GH_OP_SOFTMAX:
       if (!c.ptr[0] || !c.ptr[1]) return bad("null operand");
       if (c.dim[0] < 0 || !pos(c.dim[1])) return bad("softmax: bad shape");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     case GH_OP_HAS_NAN:
     case GH_OP_HAS_INF:

@@ -1842,6 +1842,7 @@ static int launch_conv_direct(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_conv2d_f64(ctx, c);
   if (conv_direct_shape(c) && !getenv("GORGONIA_HIP_CONV_NO_DIRECT")) return launch_conv_direct(ctx, c);
   const int rc3 = try_launch_conv3(ctx, c);
   if (rc3 >= 0) return rc3;
@@ -2021,7 +2022,7 @@ extern "C" int gh_gemm_can_softmax(const gh_cmd* c) {
 }
 
 extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {
-  if (!c || c->opcode != GH_OP_CONV2D) return 0;
+  if (!c || c->opcode != GH_OP_CONV2D || gh_dtype_of(c->flags) != GH_F32) return 0;
   if (conv_direct_shape(*c) && !getenv("GORGONIA_HIP_CONV_NO_DIRECT")) {
     const int64_t oh = c->dim[2] + 2 * c->dim[7] - 2, ow = c->dim[3] + 2 * c->dim[7] - 2;
     return oh >= 2 && ow >= 2;

@@ -161,6 +161,7 @@ inline bool al16(uint64_t p) { return (p & 15u) == 0; }
 }  // namespace
 
 int gh_launch_maxpool2d(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_maxpool2d_f64(ctx, c);
   const int64_t B = c.dim[0], C = c.dim[1];
   PoolGeom g;
   g.H = (int)c.dim[2]; g.W = (int)c.dim[3]; g.kh = (int)c.dim[4]; g.kw = (int)c.dim[5];
@@ -195,6 +196,7 @@ int gh_launch_maxpool2d(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_bn_infer(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_bn_infer_f64(ctx, c);
   const int64_t B = c.dim[0], C = c.dim[1], S = c.dim[2];
   const float* x = (const float*)(uintptr_t)c.ptr[0];
   float* y = (float*)(uintptr_t)c.ptr[1];
@@ -220,6 +222,7 @@ int gh_launch_bn_infer(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_softmax(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_softmax_f64(ctx, c);
   const int64_t rows = c.dim[0];
   const int cols = (int)c.dim[1];
   if (rows == 0) return GH_OK;

@@ -183,12 +183,17 @@ def cmd_outer(x, y, a, m, n, dtype=_ffi.F32):
     return make_cmd(_ffi.OP_OUTER, _ffi.flag_dtype(dtype), (x, y, a), (m, n))
 
 
+def _double_bits(v):
+    """A float64 scalar as the int64 a dim slot carries (gh_cmd.f is float32)."""
+    return int(np.array([v], dtype=np.float64).view(np.int64)[0])
+
+
 def cmd_conv2d(x, w, y, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dilation=(1, 1),
-               act=None, alpha=0.0, bn=None, eps=1e-5, pool2=False):
+               act=None, alpha=0.0, bn=None, eps=1e-5, pool2=False, dtype=_ffi.F32):
     """bn = (mean, var, gamma or 0, beta or 0) device pointers: BatchNorm (eval)
     on the result; pool2: 2x2 stride-2 MaxPool2D on the result (y is then
     B x F x oh/2 x ow/2).  Order: conv, bn, activation, pool."""
-    fl = {None: 0, "relu": _ffi.FLAG_ACT_RELU, "leaky": _ffi.FLAG_ACT_LEAKY}[act]
+    fl = {None: 0, "relu": _ffi.FLAG_ACT_RELU, "leaky": _ffi.FLAG_ACT_LEAKY}[act] | _ffi.flag_dtype(dtype)
     ptrs = [x, w, y]
     if bn is not None:
         mean, var, gamma, beta = bn
@@ -201,30 +206,30 @@ def cmd_conv2d(x, w, y, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dila
                      dilation[1]), (alpha, eps))
 
 
-def cmd_maxpool2d(x, y, B, Cn, H, W, kh, kw, pad, stride):
+def cmd_maxpool2d(x, y, B, Cn, H, W, kh, kw, pad, stride, dtype=_ffi.F32):
     """pad: 2 values (symmetric H, W) or 4 values (north, south, west, east) as in MaxPool2D."""
     if len(pad) == 4:
         p4, fl = tuple(pad), _ffi.FLAG_EXPLICIT_PAD
     else:
         p4, fl = (pad[0], pad[0], pad[1], pad[1]), 0
-    return make_cmd(_ffi.OP_MAXPOOL2D, fl, (x, y), (B, Cn, H, W, kh, kw) + p4 + tuple(stride))
+    return make_cmd(_ffi.OP_MAXPOOL2D, fl | _ffi.flag_dtype(dtype), (x, y), (B, Cn, H, W, kh, kw) + p4 + tuple(stride))
 
 
-def cmd_bn_infer(x, y, mean, var, B, Cn, S, eps, gamma=0, beta=0):
-    fl = (_ffi.FLAG_HAS_GAMMA if gamma else 0) | (_ffi.FLAG_HAS_BETA if beta else 0)
-    return make_cmd(_ffi.OP_BN_INFER, fl, (x, y, mean, var, gamma, beta), (B, Cn, S), (eps,))
+def cmd_bn_infer(x, y, mean, var, B, Cn, S, eps, gamma=0, beta=0, dtype=_ffi.F32):
+    fl = (_ffi.FLAG_HAS_GAMMA if gamma else 0) | (_ffi.FLAG_HAS_BETA if beta else 0) | _ffi.flag_dtype(dtype)
+    return make_cmd(_ffi.OP_BN_INFER, fl, (x, y, mean, var, gamma, beta), (B, Cn, S, _double_bits(eps)), (eps,))
 
 
-def cmd_relu(x, y, n):
-    return make_cmd(_ffi.OP_RELU, 0, (x, y), (n,))
+def cmd_relu(x, y, n, dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_RELU, _ffi.flag_dtype(dtype), (x, y), (n,))
 
 
-def cmd_leaky_relu(x, y, n, alpha):
-    return make_cmd(_ffi.OP_LEAKY_RELU, 0, (x, y), (n,), (alpha,))
+def cmd_leaky_relu(x, y, n, alpha, dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_LEAKY_RELU, _ffi.flag_dtype(dtype), (x, y), (n, _double_bits(alpha)), (alpha,))
 
 
-def cmd_softmax(x, y, rows, cols):
-    return make_cmd(_ffi.OP_SOFTMAX, 0, (x, y), (rows, cols))
+def cmd_softmax(x, y, rows, cols, dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_SOFTMAX, _ffi.flag_dtype(dtype), (x, y), (rows, cols))
 
 
 def cmd_maxpool2d_bwd(x, dy, dx, B, Cn, H, W, kh, kw, pad, stride):

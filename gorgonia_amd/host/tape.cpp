@@ -248,6 +248,15 @@ int OverwritesInput(const OpSpec& op) {
   return -1;
 }
 
+static uint32_t dtype_flag(Dtype dt) { return GH_FLAG_DTYPE(dt == Dtype::Float64 ? GH_F64 : GH_F32); }
+
+// float64 scalars ride in a dim slot as their bit pattern (gh_cmd.f is float32)
+static int64_t double_bits(double v) {
+  int64_t b;
+  std::memcpy(&b, &v, sizeof(b));
+  return b;
+}
+
 static std::string op_name(const OpSpec& op) {
   static const char* bins[] = {"add", "sub", "mul", "div", "pow", "lt", "lte", "gt", "gte", "eq", "ne", "mod"};
   switch (op.kind) {
@@ -331,10 +340,12 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     case OpKind::Conv2d: {
       const Tensor& x = *in[0];
       const Tensor& w = *in[1];
-      if (x.dt != Dtype::Float32) return bad("Conv2d: Unsupported Dtype");
+      if (x.dt == Dtype::Other || w.dt != x.dt) return bad("Conv2d: Unsupported Dtype");
+      if (x.dt == Dtype::Float64 && (op.fuse_bn || op.fuse_act_relu || op.fuse_act_leaky || op.fuse_pool2))
+        return bad("Conv2d: no epilogue operators for float64");
       gh_cmd c{};
       c.opcode = GH_OP_CONV2D;
-      c.flags = op.fuse_act_relu ? GH_FLAG_ACT_RELU : op.fuse_act_leaky ? GH_FLAG_ACT_LEAKY : 0;
+      c.flags = (op.fuse_act_relu ? GH_FLAG_ACT_RELU : op.fuse_act_leaky ? GH_FLAG_ACT_LEAKY : 0) | dtype_flag(x.dt);
       c.f[0] = (float)op.f0;
       c.ptr[0] = x.mem; c.ptr[1] = w.mem; c.ptr[2] = prealloc.mem;
       if (op.fuse_bn) {
@@ -356,12 +367,12 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     }
     case OpKind::MaxPool2D: {
       const Tensor& x = *in[0];
-      if (x.dt != Dtype::Float32) return bad("MaxPool2D: Unsupported Dtype");
+      if (x.dt == Dtype::Other) return bad("MaxPool2D: Unsupported Dtype");
       const auto& p = op.ints;
       const int64_t np = p[2];
       gh_cmd c{};
       c.opcode = GH_OP_MAXPOOL2D;
-      c.flags = np == 4 ? GH_FLAG_EXPLICIT_PAD : 0;
+      c.flags = (np == 4 ? GH_FLAG_EXPLICIT_PAD : 0) | dtype_flag(x.dt);
       c.ptr[0] = x.mem; c.ptr[1] = prealloc.mem;
       for (int i = 0; i < 4; i++) c.dim[i] = x.shape[i];
       c.dim[4] = p[0]; c.dim[5] = p[1];
@@ -373,14 +384,18 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     }
     case OpKind::BatchNorm: {
       const Tensor& x = *in[0];
-      if (x.dt != Dtype::Float32) return bad("BatchNorm: Unsupported Dtype");
+      if (x.dt == Dtype::Other) return bad("BatchNorm: Unsupported Dtype");
+      for (size_t i = 1; i < in.size(); i++)
+        if (in[i]->dt != x.dt) return bad("BatchNorm: statistics and input differ in dtype");
       gh_cmd c{};
       c.opcode = GH_OP_BN_INFER;
+      c.flags = dtype_flag(x.dt);
       c.ptr[0] = x.mem; c.ptr[1] = prealloc.mem; c.ptr[2] = in[1]->mem; c.ptr[3] = in[2]->mem;
       if (in.size() == 5) {
-        c.flags = GH_FLAG_HAS_GAMMA | GH_FLAG_HAS_BETA;
+        c.flags |= GH_FLAG_HAS_GAMMA | GH_FLAG_HAS_BETA;
         c.ptr[4] = in[3]->mem; c.ptr[5] = in[4]->mem;
       }
+      c.dim[3] = double_bits(op.f0);   // epsilon for the float64 kernel
       const int64_t B = x.shape[0], C = x.shape[1];
       c.dim[0] = B; c.dim[1] = C; c.dim[2] = x.shape.TotalSize() / (B * C);
       c.f[0] = (float)op.f0;
@@ -390,9 +405,12 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     case OpKind::Rectify:
     case OpKind::LeakyRelu: {
       gh_cmd c{};
+      if (in[0]->dt == Dtype::Other) return bad("Unsupported Dtype");
       c.opcode = op.kind == OpKind::Rectify ? GH_OP_RELU : GH_OP_LEAKY_RELU;
+      c.flags = dtype_flag(in[0]->dt);
       c.ptr[0] = in[0]->mem; c.ptr[1] = prealloc.mem;
       c.dim[0] = in[0]->DataSize();
+      c.dim[1] = double_bits(op.f0);   // alpha for the float64 kernel
       c.f[0] = (float)op.f0;
       e.Enqueue(c);
       return Status::OK();
@@ -400,7 +418,9 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     case OpKind::SoftMax: {
       const Tensor& x = *in[0];
       gh_cmd c{};
+      if (x.dt == Dtype::Other) return bad("SoftMax: Unsupported Dtype");
       c.opcode = GH_OP_SOFTMAX;
+      c.flags = dtype_flag(x.dt);
       c.ptr[0] = x.mem; c.ptr[1] = prealloc.mem;
       const int64_t cols = x.shape[x.shape.Dims() - 1];
       c.dim[0] = x.shape.TotalSize() / cols; c.dim[1] = cols;
@@ -569,6 +589,7 @@ int Graph::FuseActivations() {
     Node& p = nodes_[(size_t)n.inputs[0]];
     if (p.is_input || p.fused_away || p.read_into || uses[(size_t)p.id] != 1) continue;
     if (p.op.kind != OpKind::Conv2d && p.op.kind != OpKind::MatMul) continue;
+    if (p.dt != Dtype::Float32) continue;   // the epilogues exist for float32 only
     OpSpec op = p.op;
     std::vector<int> inputs = p.inputs;
     const bool has_act = op.fuse_act_relu || op.fuse_act_leaky;

@@ -74,17 +74,25 @@ def unary(fn, a):
     return A
 
 
+def _ft(x):
+    """float64 arrays keep their type (the *_f64 twins), everything else is float32."""
+    return np.float64 if np.asarray(x).dtype == np.float64 else np.float32
+
+
 def relu(x):
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    x = np.ascontiguousarray(x, dtype=_ft(x))
     y = np.empty_like(x)
-    lib().oracle_relu_f32(_p(y), _p(x), C.c_int64(x.size))
+    (lib().oracle_relu_f64 if x.dtype == np.float64 else lib().oracle_relu_f32)(_p(y), _p(x), C.c_int64(x.size))
     return y
 
 
 def leaky_relu(x, alpha):
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    x = np.ascontiguousarray(x, dtype=_ft(x))
     y = np.empty_like(x)
-    lib().oracle_leaky_relu_f32(_p(y), _p(x), C.c_float(alpha), C.c_int64(x.size))
+    if x.dtype == np.float64:
+        lib().oracle_leaky_relu_f64(_p(y), _p(x), C.c_double(alpha), C.c_int64(x.size))
+    else:
+        lib().oracle_leaky_relu_f32(_p(y), _p(x), C.c_float(alpha), C.c_int64(x.size))
     return y
 
 
@@ -147,6 +155,16 @@ def conv_out_hw(h, w, kh, kw, pad, stride, dil):
 
 
 def conv2d(x, w, pad=(0, 0), stride=(1, 1), dil=(1, 1)):
+    if _ft(x) == np.float64:
+        x = np.ascontiguousarray(x, dtype=np.float64)
+        w = np.ascontiguousarray(w, dtype=np.float64)
+        B, Cn, H, W = x.shape
+        F, _, kh, kw = w.shape
+        oh, ow = conv_out_hw(H, W, kh, kw, pad, stride, dil)
+        y = np.empty((B, F, oh, ow), dtype=np.float64)
+        lib().oracle_conv2d_f64(_p(x), _p(w), _p(y), *_i64(B, Cn, H, W, F, kh, kw, pad[0], pad[1],
+                                                           stride[0], stride[1], dil[0], dil[1]))
+        return y
     x = np.ascontiguousarray(x, dtype=np.float32)
     w = np.ascontiguousarray(w, dtype=np.float32)
     B, Cn, H, W = x.shape
@@ -187,27 +205,29 @@ def maxpool_out_hw(h, w, kh, kw, pad, stride):
 
 
 def maxpool2d(x, kernel, pad, stride):
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    x = np.ascontiguousarray(x, dtype=_ft(x))
     B, Cn, H, W = x.shape
     p4, explicit = _pad4(pad)
     oh, ow = maxpool_out_hw(H, W, kernel[0], kernel[1], pad, stride)
-    y = np.empty((B, Cn, oh, ow), dtype=np.float32)
-    lib().oracle_maxpool2d_f32(_p(x), _p(y), *_i64(B, Cn, H, W, kernel[0], kernel[1]), _p(p4),
+    y = np.empty((B, Cn, oh, ow), dtype=x.dtype)
+    (lib().oracle_maxpool2d_f64 if x.dtype == np.float64 else lib().oracle_maxpool2d_f32)(_p(x), _p(y), *_i64(B, Cn, H, W, kernel[0], kernel[1]), _p(p4),
                                C.c_int(explicit), *_i64(stride[0], stride[1]))
     return y
 
 
 def bn_infer(x, mean, var, eps, gamma=None, beta=None):
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    dt = _ft(x)
+    x = np.ascontiguousarray(x, dtype=dt)
     B, Cn = x.shape[:2]
     S = x.size // (B * Cn)
     y = np.empty_like(x)
-    mean = np.ascontiguousarray(mean, dtype=np.float32)
-    var = np.ascontiguousarray(var, dtype=np.float32)
-    g = np.ascontiguousarray(gamma, dtype=np.float32) if gamma is not None else None
-    b = np.ascontiguousarray(beta, dtype=np.float32) if beta is not None else None
-    lib().oracle_bn_infer_f32(_p(x), _p(y), _p(mean), _p(var), _p(g) if g is not None else None,
-                              _p(b) if b is not None else None, C.c_float(eps), *_i64(B, Cn, S))
+    mean = np.ascontiguousarray(mean, dtype=dt)
+    var = np.ascontiguousarray(var, dtype=dt)
+    g = np.ascontiguousarray(gamma, dtype=dt) if gamma is not None else None
+    b = np.ascontiguousarray(beta, dtype=dt) if beta is not None else None
+    f, e = (lib().oracle_bn_infer_f64, C.c_double(eps)) if dt == np.float64 else (lib().oracle_bn_infer_f32, C.c_float(eps))
+    f(_p(x), _p(y), _p(mean), _p(var), _p(g) if g is not None else None,
+      _p(b) if b is not None else None, e, *_i64(B, Cn, S))
     return y
 
 

@@ -1001,6 +1001,114 @@ EXPORT void oracle_softmax_f64(const double* x, double* y, int64_t rows, int64_t
 }
 
 /* HasNaN / HasInf predicates (cuda/engine.go:144-191, misc.cu:14-56). */
+/* ------------------------------------------------------------------ */
+/* float64 twins of the forward neural-network operators.  Each is the  */
+/* float32 function above with the element type changed (the CPU ops    */
+/* switch on the dtype and run the same loops, op_nn.go:909-957,        */
+/* 1559-1631; nn.go:83-163): no new algorithm, pinned through the        */
+/* float32 instance on data where both are exact, and by the float64    */
+/* rows of the reference's batch-norm table.  The convolution sums      */
+/* k = (c, kr, kc) in ascending order with a rounded multiply and a     */
+/* rounded add per step, like oracle_gemm_f32 does for the im2col form. */
+/* ------------------------------------------------------------------ */
+EXPORT void oracle_relu_f64(double* y, const double* x, int64_t n) {
+  int64_t i;
+  for (i = 0; i < n; i++) {
+    double m = x[i] >= 0.0 ? 1.0 : 0.0;
+    y[i] = x[i] * m;
+  }
+}
+
+EXPORT void oracle_leaky_relu_f64(double* y, const double* x, double alpha, int64_t n) {
+  int64_t i;
+  for (i = 0; i < n; i++) {
+    double ge = x[i] >= 0.0 ? 1.0 : 0.0;
+    double lt = x[i] < 0.0 ? 1.0 : 0.0;
+    double pos = x[i] * ge;
+    double neg = x[i] * lt;
+    double nega = neg * alpha;
+    y[i] = pos + nega;
+  }
+}
+
+EXPORT void oracle_conv2d_f64(const double* x, const double* w, double* y, int64_t B, int64_t C,
+                              int64_t H, int64_t W, int64_t F, int64_t kh, int64_t kw, int64_t padH,
+                              int64_t padW, int64_t strideH, int64_t strideW, int64_t dilH,
+                              int64_t dilW) {
+  int64_t oh, ow, bf;
+  oracle_conv_out_hw(H, W, kh, kw, padH, padW, strideH, strideW, dilH, dilW, &oh, &ow);
+#pragma omp parallel for if (g_threads > 1) schedule(static)
+  for (bf = 0; bf < B * F; bf++) {
+    int64_t b = bf / F, f = bf % F, orow, ocol, ch, kr, kc;
+    for (orow = 0; orow < oh; orow++)
+      for (ocol = 0; ocol < ow; ocol++) {
+        double acc = 0.0;
+        for (ch = 0; ch < C; ch++)
+          for (kr = 0; kr < kh; kr++) {
+            int64_t ir = -padH + kr * dilH + orow * strideH;
+            for (kc = 0; kc < kw; kc++) {
+              int64_t ic = -padW + kc * dilW + ocol * strideW;
+              double v = (ir < 0 || ir >= H || ic < 0 || ic >= W) ? 0.0 : x[((b * C + ch) * H + ir) * W + ic];
+              double p = v * w[((f * C + ch) * kh + kr) * kw + kc];
+              acc = acc + p;
+            }
+          }
+        y[(bf * oh + orow) * ow + ocol] = acc;
+      }
+  }
+}
+
+EXPORT void oracle_maxpool2d_f64(const double* x, double* y, int64_t B, int64_t C, int64_t H,
+                                 int64_t W, int64_t kh, int64_t kw, const int64_t* pad4,
+                                 int explicit_padding, int64_t strideH, int64_t strideW) {
+  int64_t oh, ow, bc;
+  oracle_maxpool_out_hw(H, W, kh, kw, pad4, strideH, strideW, &oh, &ow);
+  int64_t padH = explicit_padding ? pad4[1] : pad4[0];
+  int64_t padW = explicit_padding ? pad4[3] : pad4[2];
+#pragma omp parallel for if (g_threads > 1) schedule(static)
+  for (bc = 0; bc < B * C; bc++) {
+    const double* in = x + bc * H * W;
+    double* out = y + bc * oh * ow;
+    int64_t ph, pw, hi, wi;
+    for (ph = 0; ph < oh; ph++)
+      for (pw = 0; pw < ow; pw++) {
+        int64_t hs = ph * strideH - padH, ws = pw * strideW - padW;
+        int64_t he = hs + kh < H ? hs + kh : H;
+        int64_t we = ws + kw < W ? ws + kw : W;
+        if (hs < 0) hs = 0;
+        if (ws < 0) ws = 0;
+        double best = -DBL_MAX;   /* -maxFloat64, op_nn.go:916 */
+        for (hi = hs; hi < he; hi++)
+          for (wi = ws; wi < we; wi++)
+            if (in[hi * W + wi] > best) best = in[hi * W + wi];
+        out[ph * ow + pw] = best;
+      }
+  }
+}
+
+EXPORT void oracle_bn_infer_f64(const double* x, double* y, const double* run_mean,
+                                const double* run_var, const double* gamma, const double* beta_in,
+                                double eps, int64_t B, int64_t C, int64_t S) {
+  int64_t bc;
+#pragma omp parallel for if (g_threads > 1) schedule(static)
+  for (bc = 0; bc < B * C; bc++) {
+    int64_t c = bc % C, d;
+    double v = run_var[c] + eps;
+    double a = 1.0 / sqrt(v);
+    double nm = -run_mean[c];
+    double b = nm * a;
+    const double* in = x + bc * S;
+    double* out = y + bc * S;
+    for (d = 0; d < S; d++) {
+      double t = in[d] * a;
+      t = t + b;
+      if (gamma) t = gamma[c] * t;
+      if (beta_in) t = t + beta_in[c];
+      out[d] = t;
+    }
+  }
+}
+
 EXPORT int oracle_has_nan_f32(const float* a, int64_t n) {
   int64_t i;
   for (i = 0; i < n; i++) if (isnan(a[i])) return 1;

@@ -1,0 +1,144 @@
+"""GPU parity of the float64 forward neural-network operators (Conv2d, MaxPool2D,
+BatchNorm eval, Rectify, LeakyRelu, SoftMax) through the C ABI and the tape
+machine against the CPU oracle's float64 twins.  Bars: bit-exact for everything
+but SoftMax (same operation order, one rounding per step); SoftMax <= 4 float64
+ulp: the exponentials come from two libraries (each within 1 ulp), and their
+differences pass through the row sum and the quotient."""
+import numpy as np
+import pytest
+
+from gorgonia_amd import _ffi
+from gorgonia_amd import device as D
+from gorgonia_amd import graph as G
+from oracle import binding as O
+from tests.util import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+F64 = _ffi.F64
+
+
+def _rand(seed, shape, scale=1.0):
+    return np.random.default_rng(seed).standard_normal(shape) * scale
+
+
+def _ulp64(a, b):
+    ia = a.view(np.int64).astype(np.int64)
+    ib = b.view(np.int64).astype(np.int64)
+    ia = np.where(ia < 0, np.int64(-2**63) - ia, ia)
+    ib = np.where(ib < 0, np.int64(-2**63) - ib, ib)
+    return np.abs(ia - ib)
+
+
+CONV_CASES = [
+    # B, C, H, W, F, kh, kw, pad, stride, dil
+    (2, 3, 9, 8, 5, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (1, 8, 14, 14, 16, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (2, 4, 10, 11, 6, 1, 1, (0, 0), (1, 1), (1, 1)),
+    (2, 2, 12, 9, 3, 5, 3, (2, 1), (2, 1), (1, 1)),
+    (1, 3, 13, 13, 4, 3, 3, (2, 2), (1, 2), (2, 2)),
+]
+
+
+@pytest.mark.parametrize("cfg", CONV_CASES)
+def test_conv2d_float64_bit_exact(ctx, cfg):
+    B, C, H, W, F, kh, kw, pad, stride, dil = cfg
+    x, w = _rand(1, (B, C, H, W)), _rand(2, (F, C, kh, kw), 0.3)
+    want = O.conv2d(x, w, pad, stride, dil)
+    dx, dw, dy = ctx.upload(x), ctx.upload(w), ctx.malloc(want.size * 8)
+    ctx.run(D.cmd_conv2d(dx, dw, dy, B, C, H, W, F, kh, kw, pad, stride, dil, dtype=F64))
+    got = ctx.d2h(dy, want.shape, np.float64)
+    for p in (dx, dw, dy):
+        ctx.free(p)
+    assert_bits_equal(got, want, f"float64 conv {cfg}")
+    ref = O.conv2d(x.astype(np.float32), w.astype(np.float32), pad, stride, dil)
+    assert np.allclose(got, ref, rtol=1e-4, atol=1e-4)   # and it is the same convolution as the float32 one
+
+
+@pytest.mark.parametrize("cfg", [(2, 3, 8, 10, (2, 2), (0, 0), (2, 2)), (1, 2, 7, 8, (3, 2), (1, 1), (1, 2)),
+                                 (2, 4, 13, 13, (2, 2), (1, 0, 1, 0), (1, 1)), (2, 3, 9, 11, (2, 2), (0, 0), (2, 2))])
+def test_maxpool_float64_bit_exact(ctx, cfg):
+    B, C, H, W, kernel, pad, stride = cfg
+    x = _rand(3, (B, C, H, W))
+    x.reshape(-1)[::7] = 0.0
+    x.reshape(-1)[3::11] = -0.0
+    want = O.maxpool2d(x, kernel, pad, stride)
+    dx, dy = ctx.upload(x), ctx.malloc(want.size * 8)
+    ctx.run(D.cmd_maxpool2d(dx, dy, B, C, H, W, kernel[0], kernel[1], pad, stride, dtype=F64))
+    got = ctx.d2h(dy, want.shape, np.float64)
+    ctx.free(dx); ctx.free(dy)
+    assert_bits_equal(got, want, f"float64 maxpool {cfg}")
+
+
+@pytest.mark.parametrize("shape", [(4, 6), (2, 5, 7, 3)])
+@pytest.mark.parametrize("affine", [False, True])
+def test_batchnorm_float64_bit_exact(ctx, shape, affine):
+    x = _rand(4, shape)
+    Cn = shape[1]
+    mean, var = _rand(5, (Cn,)), np.random.default_rng(6).uniform(0.5, 2.0, Cn)
+    g, b = (_rand(7, (Cn,)), _rand(8, (Cn,))) if affine else (None, None)
+    want = O.bn_infer(x, mean, var, 1e-5, g, b)
+    held = [ctx.upload(a) for a in (x, mean, var)] + ([ctx.upload(g), ctx.upload(b)] if affine else [0, 0])
+    dy = ctx.malloc(x.size * 8)
+    B = shape[0]
+    ctx.run(D.cmd_bn_infer(held[0], dy, held[1], held[2], B, Cn, x.size // (B * Cn), 1e-5, held[3], held[4], dtype=F64))
+    got = ctx.d2h(dy, shape, np.float64)
+    for p in held + [dy]:
+        if p:
+            ctx.free(p)
+    assert_bits_equal(got, want, "float64 batchnorm")
+
+
+def test_activations_float64_bit_exact(ctx):
+    x = _rand(9, (100_003,))
+    x[:6] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-320]
+    dx, dy = ctx.upload(x), ctx.malloc(x.size * 8)
+    ctx.run(D.cmd_relu(dx, dy, x.size, dtype=F64))
+    assert_bits_equal(ctx.d2h(dy, x.shape, np.float64), O.relu(x), "float64 relu")
+    ctx.run(D.cmd_leaky_relu(dx, dy, x.size, 0.1, dtype=F64))   # 0.1 is not a float32: the full double must arrive
+    assert_bits_equal(ctx.d2h(dy, x.shape, np.float64), O.leaky_relu(x, 0.1), "float64 leaky relu")
+    ctx.free(dx); ctx.free(dy)
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (7, 10), (128, 10), (5, 64), (3, 65), (4, 1000)])
+def test_softmax_float64(ctx, shape):
+    x = _rand(10, shape, 3.0)
+    dx, dy = ctx.upload(x), ctx.malloc(x.size * 8)
+    ctx.run(D.cmd_softmax(dx, dy, shape[0], shape[1], dtype=F64))
+    got = ctx.d2h(dy, shape, np.float64)
+    ctx.free(dx); ctx.free(dy)
+    assert _ulp64(got, O.softmax(x)).max() <= 4
+    assert np.allclose(got.sum(axis=1), 1.0, atol=1e-14)
+
+
+def test_float64_commands_validate(ctx):
+    import ctypes as C
+    buf = C.create_string_buffer(256)
+    bad = D.cmd_conv2d(1, 2, 3, 1, 8, 8, 8, 8, 3, 3, (1, 1), act="relu", dtype=F64)
+    assert ctx.lib.gh_validate(C.byref(bad), 1, buf, 256) != 0 and b"float64" in buf.value
+    assert ctx.lib.gh_conv2d_can_pool(D.cmd_conv2d(1, 2, 3, 2, 8, 14, 14, 16, 3, 3, (1, 1), dtype=F64)) == 0
+    bwd = D.cmd_conv2d_bwd_data(1, 2, 3, 1, 8, 8, 8, 8, 3, 3, (1, 1))
+    bwd.flags |= _ffi.flag_dtype(F64)
+    assert ctx.lib.gh_validate(C.byref(bwd), 1, buf, 256) != 0
+
+
+def test_tape_float64_network(ctx):
+    """conv -> batchnorm -> leakyrelu -> maxpool -> reshape -> matmul -> softmax in float64 on the
+    tape machine, with activation folding requested (it must leave float64 nodes alone)."""
+    x, w = _rand(11, (2, 3, 8, 8)), _rand(12, (4, 3, 3, 3), 0.3)
+    mean, var = _rand(13, (4,)), np.random.default_rng(14).uniform(0.5, 2.0, 4)
+    gam, bet = _rand(15, (4,)), _rand(16, (4,))
+    w2 = _rand(17, (64, 5), 0.2)
+    g = G.NewGraph()
+    xn, wn = G.NewTensor(g, x), G.NewTensor(g, w)
+    h = G.Conv2d(xn, wn, (3, 3), (1, 1), (1, 1), (1, 1))
+    h = G.BatchNorm(h, G.NewTensor(g, gam), G.NewTensor(g, bet), G.NewTensor(g, mean), G.NewTensor(g, var), 1e-5)
+    h = G.MaxPool2D(G.LeakyRelu(h, 0.1), (2, 2), (0, 0), (2, 2))
+    out = G.Read(G.SoftMax(G.Mul(G.Reshape(h, (2, 64)), G.NewTensor(g, w2))), np.float64)
+    m = G.NewTapeMachine(g, fuse_activations=True)
+    assert m.fused == 0
+    m.RunAll()
+    ref = O.conv2d(x, w, (1, 1), (1, 1), (1, 1))
+    ref = O.maxpool2d(O.leaky_relu(O.bn_infer(ref, mean, var, 1e-5, gam, bet), 0.1).reshape(ref.shape), (2, 2), (0, 0), (2, 2))
+    want = O.softmax(ref.reshape(2, 64) @ w2)
+    assert np.allclose(out, want, rtol=1e-12, atol=1e-15)
+    m.Close()

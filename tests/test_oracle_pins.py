@@ -354,3 +354,51 @@ def test_mod_is_go_math_mod():
         r = O.binop("mod", "vv", (x * scale).astype(dt), (y * scale).astype(dt))
         exact = np.sign(x) * (np.abs(x) % np.abs(y)) * scale
         assert np.array_equal(r, exact.astype(dt))
+
+
+# ---- float64 twins of the forward neural-network operators -----------------------------
+
+def test_float64_nn_twins_equal_the_pinned_float32_functions_where_both_are_exact():
+    """Data on which float32 and float64 arithmetic are both exact (small integers, powers of
+    two): the float64 twins must reproduce the float32 functions pinned above."""
+    from oracle import binding as O
+    rng = np.random.default_rng(11)
+    x = rng.integers(-6, 7, (3, 4, 9, 8)).astype(np.float64)
+    w = rng.integers(-3, 4, (5, 4, 3, 3)).astype(np.float64)
+    f32 = lambda a: a.astype(np.float32)
+    for pad, stride, dil in [((1, 1), (1, 1), (1, 1)), ((0, 2), (2, 1), (1, 1)), ((2, 2), (1, 2), (2, 1))]:
+        a = O.conv2d(x, w, pad, stride, dil)
+        assert a.dtype == np.float64 and np.array_equal(a, O.conv2d(f32(x), f32(w), pad, stride, dil))
+    for kernel, pad, stride in [((2, 2), (0, 0), (2, 2)), ((3, 2), (1, 1), (1, 2)), ((2, 2), (1, 0, 1, 0), (1, 1))]:
+        a = O.maxpool2d(x, kernel, pad, stride)
+        assert a.dtype == np.float64 and np.array_equal(a, O.maxpool2d(f32(x), kernel, pad, stride))
+    assert np.array_equal(O.relu(x), O.relu(f32(x))) and np.array_equal(O.leaky_relu(x, 0.25), O.leaky_relu(f32(x), 0.25))
+    mean, var = np.array([1.0, -2.0, 0.5, 4.0]), np.array([3.0, 15.0, 0.0, 63.0])   # var + 1 is a square
+    g, b = np.array([2.0, -1.0, 0.5, 4.0]), np.array([1.0, 0.0, -3.0, 8.0])
+    assert np.array_equal(O.bn_infer(x, mean, var, 1.0, g, b), O.bn_infer(f32(x), mean, var, 1.0, g, b))
+
+
+def test_float64_nn_twins_against_their_definitions():
+    """General float64 data against independent numpy restatements: the documented per-step
+    roundings of batch norm and the activations, a sequential-order sum for the convolution."""
+    from oracle import binding as O
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((2, 3, 6, 5))
+    w = rng.standard_normal((4, 3, 3, 3))
+    got = O.conv2d(x, w, (1, 1), (1, 1), (1, 1))
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    want = np.zeros_like(got)
+    for c in range(3):
+        for kr in range(3):
+            for kc in range(3):   # k ascending, one rounded product and one rounded add per tap
+                want = want + xp[:, None, c, kr:kr + 6, kc:kc + 5] * w[None, :, c, kr, kc, None, None]
+    assert np.array_equal(got, want)
+    mean, var, g, b = rng.standard_normal(3), rng.uniform(0.5, 2, 3), rng.standard_normal(3), rng.standard_normal(3)
+    a = 1.0 / np.sqrt(var + 1e-5)
+    sh = (1, 3, 1, 1)
+    want = g.reshape(sh) * ((x * a.reshape(sh)) + (-mean * a).reshape(sh)) + b.reshape(sh)
+    assert np.array_equal(O.bn_infer(x, mean, var, 1e-5, g, b), want)
+    assert np.array_equal(O.relu(x), x * (x >= 0))
+    assert np.array_equal(O.leaky_relu(x, 0.1), x * (x >= 0) + (x * (x < 0)) * 0.1)
+    pooled = O.maxpool2d(x, (2, 2), (0, 0), (2, 2))
+    assert np.array_equal(pooled, x[:, :, :6, :4].reshape(2, 3, 3, 2, 2, 2).max(axis=(3, 5)))
