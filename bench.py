@@ -196,6 +196,44 @@ def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=Tr
     return dt / steps * 1e3, result, inp, launches
 
 
+def bench_convnet_machines(steps, warmup, count=2, batch=128):
+    """Throughput of `count` tape machines (each its own engine, stream and weights, each
+    running the same synchronous RunAll loop on its own batch) in as many host threads -
+    what goroutines with one VM each would do.  A step's launch and wait latency then
+    overlaps the other machines' kernels.  Returns (images/s, every machine's output)."""
+    import threading
+    from gorgonia_amd import configs, graph as G
+    inp = configs.convnet_inputs(batch)
+    machines = []
+    for _ in range(count):
+        g, outs = configs.build_convnet(inp, resident_input=True)
+        m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING, fuse_activations=True)
+        for _ in range(max(warmup, 3)):
+            m.RunAll()
+        machines.append((g, m, outs))
+    gate = threading.Barrier(count + 1)
+
+    def loop(m):
+        gate.wait()
+        for _ in range(steps):
+            m.RunAll()
+        gate.wait()
+
+    threads = [threading.Thread(target=loop, args=(m,)) for _, m, _ in machines]
+    for t in threads:
+        t.start()
+    gate.wait()
+    t0 = time.perf_counter()
+    gate.wait()
+    dt = time.perf_counter() - t0
+    for t in threads:
+        t.join()
+    results = [outs["out"].copy() for _, _, outs in machines]
+    for _, m, _ in machines:
+        m.Close()
+    return count * steps * batch / dt, results
+
+
 def bench_yolo(steps, warmup):
     """Config 5: Tiny-YOLO-v2-shaped forward, batch 8 x 3 x 416 x 416, on the tape
     machine with conv+BatchNorm+LeakyReLU(+MaxPool) folded, graph replay,
@@ -347,6 +385,9 @@ def main():
     ms_step, gpu_out, inp, launches = bench_convnet(a.steps, a.warmup, graph_replay=not a.eager_timing)
     images_s = 128 / ms_step * 1e3
     log(f"convnet: {ms_step:.4f} ms/step  {images_s:.0f} images/s  (graph launches {launches})")
+    two_images_s, two_out = bench_convnet_machines(a.steps, a.warmup, 2)
+    four_images_s, four_out = bench_convnet_machines(a.steps, a.warmup, 4)
+    log(f"convnet, machines in parallel host threads: two {two_images_s:.0f}, four {four_images_s:.0f} images/s")
     ms_h2d, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False)
     ms_eager, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, graph_replay=False)
 
@@ -436,6 +477,9 @@ def main():
             "convnet_ms_per_step_with_input_h2d": round(ms_h2d, 5),
             "convnet_images_s_with_input_h2d": round(128 / ms_h2d * 1e3, 1),
             "convnet_ms_per_step_eager_no_graph": round(ms_eager, 5),
+            "convnet_images_s_two_machines_two_host_threads": round(two_images_s, 1),
+            "convnet_images_s_four_machines_four_host_threads": round(four_images_s, 1),
+            "convnet_parallel_machines_outputs_equal_single": bool(all(np.array_equal(o, gpu_out) for o in two_out + four_out)),
             "yolo_shaped_forward": yolo, "convnet_training_step": train, "backward_kernels": bwd, "convnet_kernels": conv_k, "elementwise": elem, "linalg": lin, "parity": parity,
         },
     }

@@ -89,9 +89,9 @@ def build_elementwise(inp):
     return g, {"z": G.Read(z), "tanh": G.Read(t), "pow": G.Read(p)}
 
 
-def build_convnet(inp, resident=True):
+def build_convnet(inp, resident=True, resident_input=False):
     g = G.NewGraph()
-    h = G.NewTensor(g, inp["x"])
+    h = G.NewTensor(g, inp["x"], resident_input)
     for i in range(3):
         w = G.NewTensor(g, inp[f"w{i}"], resident)
         h = G.Conv2d(h, w, (3, 3), (1, 1), (1, 1), (1, 1))
