@@ -20,6 +20,7 @@
 // pass), so lanes run along output pixels for coalesced loads and stores.
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
 #include "gh_internal.h"
@@ -27,6 +28,8 @@
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+// the same four floats at any 4-byte aligned address (one 128-bit load all the same)
+typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kThreads = 256;
@@ -462,7 +465,7 @@ __global__ __launch_bounds__(256) void k_splitk_reduce4(const float* __restrict_
 // (Cutting K across workgroups as well, with the last one to arrive at a
 // per-tile counter adding the slices, was measured: the device-wide fences it
 // needs cost ~35 us per launch on this part, four times the whole kernel.)
-template <int WV, bool VEC>
+template <int WV, bool VEC, bool VECB>
 __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict__ A,
                                                          const float* __restrict__ B,
                                                          float* __restrict__ C, int M, int N, int K,
@@ -475,7 +478,10 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
   // a scalar branch, and a load in one arm does not look pending in the other
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 31, h = lane >> 5;
-  const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+  // VECB (N >= 32): the last column tile is moved left to end at column N, so
+  // every tile is whole; the columns it shares with its neighbour get the same
+  // bits from both (a column's sum does not depend on the tile it sits in).
+  const int m0 = blockIdx.y * 32, n0 = VECB ? min((int)blockIdx.x * 32, N - 32) : blockIdx.x * 32;
   const int m = m0 + r, n = n0 + r;
   const int nchunks = (K + 15) / 16;
 
@@ -487,10 +493,19 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
   // branch per lane: rows, columns and k past the matrix are clamped to the
   // last valid one and replaced by zero just before the MFMA, so nothing makes
   // the compiler wait for one load before it issues the next.
+  // The texture addresser takes a wavefront's load instruction at four lanes per
+  // clock whatever its width, so B read as eight one-float loads per chunk held
+  // a compute unit to ~16 bytes per clock; with VECB a chunk of B (16 k x 32
+  // columns) is two 128-bit loads per lane (lane = (k row, column quad)) and goes
+  // through a second wavefront-private LDS tile into the same MFMA order.
   constexpr int TP = 20;                     // pitch of the transposing tile: rows stay 16-byte aligned
   __shared__ __attribute__((aligned(16))) float tbuf[WV][32 * TP];
   __shared__ float sm_x[32 * 33], sm_e[32 * 33];   // the tile and its exponentials when a softmax follows
+  constexpr int TPB = 36;                    // pitch of the B tile: 16-byte aligned rows, conflict-free both ways
+  __shared__ __attribute__((aligned(16))) float tbufb[VECB ? WV : 1][16 * TPB];
   float* const T = tbuf[wave];
+  float* const TB = tbufb[VECB ? wave : 0];
+  const float* const b_vec = B + n0 + (lane & 7) * 4;   // row k0 + (lane >> 3), and 8 rows further down
   const int n_c = min(n, N - 1);
   const float* const a_vec = A + (int64_t)min(m0 + (lane >> 2), M - 1) * lda + (lane & 3) * 4;   // + 16 rows for the second load
   const int64_t a_vec_step = (int64_t)(min(m0 + 16 + (lane >> 2), M - 1) - min(m0 + (lane >> 2), M - 1)) * lda;
@@ -505,9 +520,17 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
 #pragma unroll
       for (int t = 0; t < 8; t++) a[t] = A[(int64_t)min(m0 + t * 4 + (lane >> 4), M - 1) * lda + kk];
     }
-    const int k0 = chunk * 16 + 8 * h;
+    if (VECB) {
+      const int kr = chunk * 16 + (lane >> 3);
+      const f32x4 lo = *reinterpret_cast<const f32x4_a4*>(b_vec + (int64_t)min(kr, K - 1) * ldb);
+      const f32x4 hi = *reinterpret_cast<const f32x4_a4*>(b_vec + (int64_t)min(kr + 8, K - 1) * ldb);
 #pragma unroll
-    for (int t = 0; t < 8; t++) b[t] = B[(int64_t)min(k0 + t, K - 1) * ldb + n_c];
+      for (int t = 0; t < 4; t++) { b[t] = lo[t]; b[4 + t] = hi[t]; }
+    } else {
+      const int k0 = chunk * 16 + 8 * h;
+#pragma unroll
+      for (int t = 0; t < 8; t++) b[t] = B[(int64_t)min(k0 + t, K - 1) * ldb + n_c];
+    }
   };
   // load order -> MFMA order, in place
   auto transpose_a = [&](int chunk, float (&a)[8]) {
@@ -524,6 +547,14 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
 #pragma unroll
     for (int t = 0; t < 4; t++) { a[t] = lo[t]; a[4 + t] = hi[t]; }
   };
+  auto transpose_b = [&](float (&b)[8]) {
+    if (!VECB) return;
+    f32x4 lo = {b[0], b[1], b[2], b[3]}, hi = {b[4], b[5], b[6], b[7]};
+    *reinterpret_cast<f32x4*>(TB + (lane >> 3) * TPB + (lane & 7) * 4) = lo;
+    *reinterpret_cast<f32x4*>(TB + (8 + (lane >> 3)) * TPB + (lane & 7) * 4) = hi;
+#pragma unroll
+    for (int t = 0; t < 8; t++) b[t] = TB[(8 * h + t) * TPB + r];
+  };
   // group = chunks c, c + WV, ... (G of them); the chunk order per wavefront is
   // fixed, so the sum is the same whatever the grouping
   auto load_group = [&](int c, float (&a)[G][8], float (&b)[G][8]) {
@@ -539,6 +570,7 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
     for (int g = 0; g < G; g++)
       if (c + g * WV < nchunks) {
         transpose_a(c + g * WV, a[g]);
+        transpose_b(b[g]);
         const int left = K - ((c + g * WV) * 16 + 8 * h);   // valid k of this lane's eight
 #pragma unroll
         for (int t = 0; t < 8; t++) {
@@ -606,6 +638,109 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
     for (int j = 0; j < N; j++) sum = sum + sm_e[il * 33 + j];
     const float inv = 1.0f / sum;
     if (m0 + il < M && jl < N) C[(int64_t)(m0 + il) * ldc + jl] = sm_e[il * 33 + jl] * inv;
+  }
+}
+
+// ---- small-output GEMM on 16-row tiles -----------------------------------------------
+// A compute unit keeps only so many cache lines in flight, which holds one
+// workgroup to ~40 GB/s of operand fill however its loads are written (measured
+// on the 32x32 kernel above), so a product whose 32x32 tiles cover a fraction of
+// the chip is bounded by the number of compute units it touches.  This kernel
+// cuts the output into tiles of 16 rows by 16*NT columns (two to four times as
+// many workgroups) on the 16x16x4 MFMA; the K split over the wavefronts of a
+// block and the fixed-order sum of their partial tiles are those of
+// k_gemm_skinny.  Lane l = (i = l % 16, q = l / 16) owns k = 16*chunk + 4*q + t
+// at MFMA step t: its four A values are one 128-bit load of row i, already in
+// MFMA order; of B it takes, per k, the NT adjacent columns n0 + NT*i + c (one
+// load of NT floats; with NT = 2 sixteen lanes cover one whole 128-byte line)
+// and column set c feeds accumulator c.  The last tile in each direction is
+// moved back to end at the matrix edge (M >= 16, N >= 16*NT), so no row or
+// column is ever masked; k past K is clamped in the address and zeroed before
+// the MFMA.
+template <int WV, int NT, bool VEC>
+__global__ __launch_bounds__(WV * 64) void k_gemm_skinny16(const float* __restrict__ A,
+                                                           const float* __restrict__ B,
+                                                           float* __restrict__ C, int M, int N, int K,
+                                                           int lda, int ldb, int ldc, int act, float alpha) {
+  constexpr int G = NT == 1 ? 5 : 4;
+  constexpr int BN = 16 * NT, TILE = 16 * BN;
+  typedef float bvec __attribute__((ext_vector_type(NT), aligned(4)));
+  __shared__ float part[WV * TILE];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int i = lane & 15, q = lane >> 4;
+  const int m0 = min((int)blockIdx.y * 16, M - 16), n0 = min((int)blockIdx.x * BN, N - BN);
+  const int nchunks = (K + 15) / 16;
+  const float* const a_row = A + (int64_t)(m0 + i) * lda;
+  const float* const b_col = B + n0 + NT * i;
+  auto load = [&](int chunk, float (&a)[4], float (&b)[4][NT]) {
+    const int k0 = chunk * 16 + 4 * q;
+    if (VEC) {   // K % 4 == 0: a quad is whole or entirely past K
+      const f32x4 v = *reinterpret_cast<const f32x4_a4*>(a_row + min(k0, K - 4));
+#pragma unroll
+      for (int t = 0; t < 4; t++) a[t] = v[t];
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; t++) a[t] = a_row[min(k0 + t, K - 1)];
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const float* src = b_col + (int64_t)min(k0 + t, K - 1) * ldb;
+      if constexpr (NT == 1) {
+        b[t][0] = *src;
+      } else {
+        const bvec v = *reinterpret_cast<const bvec*>(src);
+#pragma unroll
+        for (int c = 0; c < NT; c++) b[t][c] = v[c];
+      }
+    }
+  };
+  auto load_group = [&](int c, float (&a)[G][4], float (&b)[G][4][NT]) {
+#pragma unroll
+    for (int g = 0; g < G; g++)
+      if (c + g * WV < nchunks) load(c + g * WV, a[g], b[g]);
+  };
+  f32x4 acc[NT];
+#pragma unroll
+  for (int c = 0; c < NT; c++) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto mfma_group = [&](int c, float (&a)[G][4], float (&b)[G][4][NT]) {
+#pragma unroll
+    for (int g = 0; g < G; g++)
+      if (c + g * WV < nchunks) {
+        const int left = K - ((c + g * WV) * 16 + 4 * q);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          const float av = t < left ? a[g][t] : 0.f;
+#pragma unroll
+          for (int cs = 0; cs < NT; cs++) {
+            const float bv = t < left ? b[g][t][cs] : 0.f;
+            acc[cs] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[cs], 0, 0, 0);
+          }
+        }
+      }
+  };
+  float a0[G][4], b0[G][4][NT], a1[G][4], b1[G][4][NT];
+  int c0 = wave;
+  if (c0 < nchunks) load_group(c0, a0, b0);
+  while (c0 < nchunks) {
+    const int c1 = c0 + G * WV;
+    if (c1 < nchunks) load_group(c1, a1, b1);
+    mfma_group(c0, a0, b0);
+    if (c1 >= nchunks) break;
+    c0 = c1 + G * WV;
+    if (c0 < nchunks) load_group(c0, a0, b0);
+    mfma_group(c1, a1, b1);
+  }
+  // element v of accumulator c in lane (i, q) is C[m0 + 4*q + v][n0 + NT*i + c]
+#pragma unroll
+  for (int c = 0; c < NT; c++)
+#pragma unroll
+    for (int v = 0; v < 4; v++) part[wave * TILE + (4 * q + v) * BN + NT * i + c] = acc[c][v];
+  __syncthreads();
+  for (int e = threadIdx.x; e < TILE; e += WV * 64) {
+    float sum = part[e];
+#pragma unroll
+    for (int w = 1; w < WV; w++) sum = sum + part[w * TILE + e];
+    C[(int64_t)(m0 + e / BN) * ldc + n0 + e % BN] = act_apply(sum, act, alpha);
   }
 }
 
@@ -1765,12 +1900,35 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   const float* A = (const float*)(uintptr_t)c.ptr[0];
   const float* B = (const float*)(uintptr_t)c.ptr[1];
   float* C = (float*)(uintptr_t)c.ptr[2];
-  if (vec_a)
-    hipLaunchKernelGGL((k_gemm_skinny<WV, true>), grid, dim3(WV * 64), 0, ctx->stream, A, B, C, M, N, K, lda, ldb,
-                       ldc, act, c.f[0], softmax);
-  else
-    hipLaunchKernelGGL((k_gemm_skinny<WV, false>), grid, dim3(WV * 64), 0, ctx->stream, A, B, C, M, N, K, lda, ldb,
-                       ldc, act, c.f[0], softmax);
+  // Few 32x32 tiles: 16-row tiles reach two to four times as many compute units.
+  // Shapes that may carry the softmax epilogue (N <= 32) stay on one kernel, so
+  // the fused and the separate softmax see the same product bits.
+  const char* force = getenv("GORGONIA_HIP_SKINNY_TILE");   // "32", "16x32", "16x16": measurements
+  if (M >= 16 && N > 32 && tiles * 2 <= ctx->cu_count && !(force && !strcmp(force, "32"))) {
+    // 16x32 tiles read whole 128-byte lines of B; when even those leave half the
+    // chip without a tile, 16x16 (measured on MI355X, 8 wavefronts per block:
+    // 128x625x1152 11.0 us on 32x32, 8.4 on 16x32, 9.8 on 16x16; 64x1000x4096
+    // 33 / 21.8 / 19.5 us)
+    const int64_t blocks_wide = cdiv(M, 16) * cdiv(N, 32);
+    const bool narrow = force ? !strcmp(force, "16x16") : blocks_wide * 2 <= ctx->cu_count;
+    auto launch16 = [&](auto kernel, int bn) {
+      hipLaunchKernelGGL(kernel, dim3((N + bn - 1) / bn, (M + 15) / 16), dim3(WV * 64), 0, ctx->stream, A, B, C, M,
+                         N, K, lda, ldb, ldc, act, c.f[0]);
+    };
+    const bool vec = K % 4 == 0;
+    if (narrow) { if (vec) launch16(k_gemm_skinny16<WV, 1, true>, 16); else launch16(k_gemm_skinny16<WV, 1, false>, 16); }
+    else { if (vec) launch16(k_gemm_skinny16<WV, 2, true>, 32); else launch16(k_gemm_skinny16<WV, 2, false>, 32); }
+    return gh_check_hip(ctx, hipGetLastError(), "skinny gemm launch");
+  }
+  const bool vec_b = N >= 32;   // whole column tiles (the last one moved left)
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(WV * 64), 0, ctx->stream, A, B, C, M, N, K, lda, ldb, ldc, act, c.f[0],
+                       softmax);
+  };
+  if (vec_a && vec_b) launch(k_gemm_skinny<WV, true, true>);
+  else if (vec_a) launch(k_gemm_skinny<WV, true, false>);
+  else if (vec_b) launch(k_gemm_skinny<WV, false, true>);
+  else launch(k_gemm_skinny<WV, false, false>);
   return gh_check_hip(ctx, hipGetLastError(), "skinny gemm launch");
 }
 

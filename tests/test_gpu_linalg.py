@@ -30,7 +30,9 @@ def _run_gemm(ctx, A, B, ta=False, tb=False, act=None, alpha=0.0, softmax=False)
 
 SHAPES = [(1, 1, 1), (3, 5, 7), (32, 32, 2), (64, 64, 16), (65, 129, 33), (128, 128, 128),
           (256, 784, 300), (256, 300, 100), (256, 100, 10), (128, 1152, 625), (130, 10, 625),
-          (512, 512, 512), (1000, 37, 259)]  # (m, k, n)
+          (512, 512, 512), (1000, 37, 259),
+          # 16x16-tile small-output kernel: ragged edges, K not a multiple of 4 or 16
+          (100, 333, 37), (17, 1001, 48), (16, 35, 33), (64, 4096, 1000)]  # (m, k, n)
 
 
 @pytest.mark.parametrize("ta", [False, True])
@@ -50,7 +52,7 @@ def test_matmul_integer_exact(ctx):
     """Small-integer inputs: every partial sum is exactly representable, so any
     accumulation order must give the oracle's bits."""
     rng = np.random.default_rng(0)
-    for (m, k, n) in [(64, 64, 64), (100, 50, 30), (256, 300, 100), (7, 1, 5)]:
+    for (m, k, n) in [(64, 64, 64), (100, 50, 30), (256, 300, 100), (7, 1, 5), (100, 50, 36), (40, 77, 50)]:
         A = rng.integers(-8, 9, (m, k)).astype(np.float32)
         B = rng.integers(-8, 9, (k, n)).astype(np.float32)
         for ta, tb in [(False, False), (False, True), (True, False), (True, True)]:
