@@ -256,6 +256,28 @@ def bench_yolo(steps, warmup):
     return dt / steps * 1e3, result, inp
 
 
+def bench_mlp(steps, warmup):
+    """Config 1: MLP 256 x 784 -> 300 -> 100 -> 10 forward on the tape machine (three
+    dense layers, ReLU and SoftMax folded into the products' epilogues), graph replay,
+    weights and input resident."""
+    from gorgonia_amd import configs, graph as G
+    inp = configs.mlp_inputs(256)
+    g, outs = configs.build_mlp(inp, resident_input=True)
+    m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING, fuse_activations=True)
+    for _ in range(max(warmup, 3)):
+        m.RunAll()
+    eng = m.engine()
+    eng.DoWork()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        m.RunAll()
+    eng.DoWork()
+    dt = time.perf_counter() - t0
+    result = outs["out"].copy()
+    m.Close()
+    return dt / steps * 1e3, result, inp
+
+
 def bench_convnet_train(steps, warmup, batch=128):
     """Config 4 as a training step: forward, every layer's gradient, RMSProp
     update (examples/convnet/main.go:195) of the resident weights; only the
@@ -369,7 +391,7 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager-timing", action="store_true",
                     help="launch every kernel eagerly, no hipGraph (use under rocprofv3 --pmc)")
-    ap.add_argument("--only", default="", help="comma list of: convnet,elementwise,linalg,yolo,train")
+    ap.add_argument("--only", default="", help="comma list of: convnet,elementwise,linalg,mlp,yolo,train")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this engine runs on one GPU; --gpus must be 1 (no multi-GPU path is built)")
@@ -397,6 +419,12 @@ def main():
         yolo = {"ms_per_step": round(ms_yolo, 4), "images_s": round(8 / ms_yolo * 1e3, 1),
                 "TFLOPs": round(31_080_857_600 / ms_yolo / 1e9, 2), "flop_per_step": 31_080_857_600}
         log(f"yolo-shaped: {ms_yolo:.4f} ms/step  {8 / ms_yolo * 1e3:.0f} images/s")
+
+    mlp = None
+    if not only or "mlp" in only:
+        ms_mlp, mlp_out, mlp_inp = bench_mlp(a.steps, a.warmup)
+        mlp = {"ms_per_step": round(ms_mlp, 5), "images_s": round(256 / ms_mlp * 1e3, 1), "flop_per_step": 136_294_400}
+        log(f"mlp: {ms_mlp:.4f} ms/step  {256 / ms_mlp * 1e3:.0f} rows/s")
 
     train = None
     if not only or "train" in only:
@@ -445,6 +473,21 @@ def main():
             O.set_threads(1)
             cpu["convnet_train_images_s"] = round(128 * reps_t / tdt, 1)
             cpu["convnet_train_sample"] = f"{reps_t} training steps of the same 128-image batch, {threads} threads"
+        if mlp is not None:
+            from oracle import binding as O, forward as F
+            O.set_threads(threads)
+            t0 = time.perf_counter()
+            reps_m = 0
+            while reps_m < 200 and time.perf_counter() - t0 < 3.0:
+                mref = F.mlp(mlp_inp)
+                reps_m += 1
+            mdt = time.perf_counter() - t0
+            O.set_threads(1)
+            cpu["mlp_images_s"] = round(256 * reps_m / mdt, 1)
+            cpu["mlp_sample"] = f"{reps_m} forward passes of the same 256-row batch, {threads} threads"
+            merr = float(np.linalg.norm(mlp_out.astype(np.float64) - mref) / np.linalg.norm(mref))
+            parity["mlp_rel_frobenius_vs_oracle"] = merr
+            parity["ok"] = parity["ok"] and merr <= 1e-5
         if yolo is not None:
             from oracle import binding as O, forward as F
             O.set_threads(threads)
@@ -480,7 +523,7 @@ def main():
             "convnet_images_s_two_machines_two_host_threads": round(two_images_s, 1),
             "convnet_images_s_four_machines_four_host_threads": round(four_images_s, 1),
             "convnet_parallel_machines_outputs_equal_single": bool(all(np.array_equal(o, gpu_out) for o in two_out + four_out)),
-            "yolo_shaped_forward": yolo, "convnet_training_step": train, "backward_kernels": bwd, "convnet_kernels": conv_k, "elementwise": elem, "linalg": lin, "parity": parity,
+            "mlp_forward": mlp, "yolo_shaped_forward": yolo, "convnet_training_step": train, "backward_kernels": bwd, "convnet_kernels": conv_k, "elementwise": elem, "linalg": lin, "parity": parity,
         },
     }
     print(json.dumps(line), flush=True)

@@ -64,9 +64,9 @@ def yolo_inputs(batch=8, size=416):
 
 # ---- graphs -----------------------------------------------------------------------------
 
-def build_mlp(inp, resident=True):
+def build_mlp(inp, resident=True, resident_input=False):
     g = G.NewGraph()
-    x = G.NewTensor(g, inp["x"])
+    x = G.NewTensor(g, inp["x"], resident=resident_input)
     h = x
     for i in range(3):
         w = G.NewTensor(g, inp[f"w{i}"], resident)
