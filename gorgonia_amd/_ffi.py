@@ -42,6 +42,7 @@ FLAG_CONV_BN = 1 << 24
 FLAG_CONV_POOL2 = 1 << 25
 FLAG_BN_EVAL = 1 << 26
 FLAG_GEMM_SOFTMAX = 1 << 27
+FLAG_GEMM_BIAS = 1 << 28
 
 
 def flag_fn(f):

@@ -227,6 +227,8 @@ struct LoadIm2col {
 // ---- result writers ------------------------------------------------------------
 struct StoreRowMajor {
   float* C; int ldc;
+  const float* bias;   // optional row vector added to every row of the product, before the activation
+  __device__ __forceinline__ float pre(int j, float v) const { return bias ? v + bias[j] : v; }
   __device__ __forceinline__ void put(int i, int j, float v) const { C[(int64_t)i * ldc + j] = v; }
 };
 
@@ -234,6 +236,7 @@ struct StoreRowMajor {
 struct StoreNCHW {
   float* y; int F; int plane /* oh*ow */;
   ConvTail tail;
+  __device__ __forceinline__ float pre(int, float v) const { return v; }
   __device__ __forceinline__ void put(int i, int j, float v) const {
     const int b = j / plane, p = j - b * plane;
     y[((int64_t)b * F + i) * plane + p] = tail_apply(tail, i, v);
@@ -243,6 +246,7 @@ struct StoreNCHW {
 // Split-K partial sums: slab `split` of a [splits][M][N] workspace.
 struct StorePartial {
   float* ws; int N;
+  __device__ __forceinline__ float pre(int, float v) const { return v; }
   __device__ __forceinline__ void put(int i, int j, float v) const { ws[(int64_t)i * N + j] = v; }
 };
 
@@ -328,7 +332,7 @@ __device__ __forceinline__ void mfma_tile_loop(float* lds, LA& la, LB& lb, const
 #pragma unroll
       for (int b = 0; b < TN; b++) {
         const int j = n0 + wn + b * 32 + lr;
-        if (i < M && j < N) sc.put(i, j, act_apply(acc[a][b][v], act, alpha));
+        if (i < M && j < N) sc.put(i, j, act_apply(sc.pre(j, acc[a][b][v]), act, alpha));
       }
     }
 }
@@ -366,7 +370,8 @@ __global__ __launch_bounds__(kThreads) void k_sgemm(const float* __restrict__ A,
                                                     float* __restrict__ C, int M, int N, int K,
                                                     int lda, int ldb, int ldc, int64_t sA,
                                                     int64_t sB, int64_t sC, int act, float alpha,
-                                                    int splits, float* __restrict__ ws) {
+                                                    int splits, float* __restrict__ ws,
+                                                    const float* __restrict__ bias) {
   using LA = typename std::conditional<TA, LoadMnContig<BM, BK, VEC>, LoadKContig<BM, BK, VEC>>::type;
   using LB = typename std::conditional<TB, LoadKContig<BN, BK, VEC>, LoadMnContig<BN, BK, VEC>>::type;
   const int bz = blockIdx.z;
@@ -387,7 +392,7 @@ __global__ __launch_bounds__(kThreads) void k_sgemm(const float* __restrict__ A,
   } else {
     LA la; la.base = A + bz * sA; la.ld = lda; la.rmax = M; la.kmax = K;
     LB lb; lb.base = B + bz * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
-    StoreRowMajor sc{C + bz * sC, ldc};
+    StoreRowMajor sc{C + bz * sC, ldc, bias};
     mfma_tile_loop<BM, BN, BK, WAVES_M, LA, LB, StoreRowMajor>(lds, la, lb, sc, M, N, 0, nk, tile_m * BM,
                                                                tile_n * BN, act, alpha);
   }
@@ -430,7 +435,7 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(const float* __restrict__
     float acc = ws[e];
     for (int s = 1; s < splits; s++) acc = acc + ws[(int64_t)s * total + e];
     const int i = (int)(e / N), j = (int)(e - (int64_t)i * N);
-    sc.put(i, j, act_apply(acc, act, alpha));
+    sc.put(i, j, act_apply(sc.pre(j, acc), act, alpha));
   }
 }
 
@@ -450,7 +455,7 @@ __global__ __launch_bounds__(256) void k_splitk_reduce4(const float* __restrict_
   const float sum = pair + __shfl_xor(pair, 2, 64);
   if (e < total && q == 0) {
     const int i = (int)(e / N), j = (int)(e - (int64_t)i * N);
-    sc.put(i, j, act_apply(sum, act, alpha));
+    sc.put(i, j, act_apply(sc.pre(j, sum), act, alpha));
   }
 }
 
@@ -470,7 +475,8 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
                                                          const float* __restrict__ B,
                                                          float* __restrict__ C, int M, int N, int K,
                                                          int lda, int ldb, int ldc, int act,
-                                                         float alpha, int softmax) {
+                                                         float alpha, int softmax,
+                                                         const float* __restrict__ bias) {
   constexpr int G = 5;                       // k-chunks per group; two groups of loads are in flight
   constexpr int HALF = WV / 2;
   __shared__ float part[HALF * 1024];
@@ -617,6 +623,7 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
     const int v = e >> 6, l = e & 63;
     const int il = 8 * (v / 4) + 4 * (l >> 5) + (v % 4), jl = l & 31;
     const int i = m0 + il, j = n0 + jl;
+    if (bias && j < N) sum = sum + bias[j];
     if (softmax) sm_x[il * 33 + jl] = act_apply(sum, act, alpha);
     else if (i < M && j < N) C[(int64_t)i * ldc + j] = act_apply(sum, act, alpha);
   }
@@ -661,7 +668,8 @@ template <int WV, int NT, bool VEC>
 __global__ __launch_bounds__(WV * 64) void k_gemm_skinny16(const float* __restrict__ A,
                                                            const float* __restrict__ B,
                                                            float* __restrict__ C, int M, int N, int K,
-                                                           int lda, int ldb, int ldc, int act, float alpha) {
+                                                           int lda, int ldb, int ldc, int act, float alpha,
+                                                           const float* __restrict__ bias) {
   constexpr int G = NT == 1 ? 5 : 4;
   constexpr int BN = 16 * NT, TILE = 16 * BN;
   typedef float bvec __attribute__((ext_vector_type(NT), aligned(4)));
@@ -740,6 +748,7 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny16(const float* __restri
     float sum = part[e];
 #pragma unroll
     for (int w = 1; w < WV; w++) sum = sum + part[w * TILE + e];
+    if (bias) sum = sum + bias[n0 + e % BN];
     C[(int64_t)(m0 + e / BN) * ldc + n0 + e % BN] = act_apply(sum, act, alpha);
   }
 }
@@ -1632,13 +1641,14 @@ int launch_sgemm_cfg(gh_ctx* ctx, const gh_cmd& c, int splits) {
                    sA % 4 == 0 && sB % 4 == 0 && (ta ? M % 4 == 0 : K % 4 == 0) &&
                    (tb ? K % 4 == 0 : N % 4 == 0);
   const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
+  const float* bias = (c.flags & GH_FLAG_GEMM_BIAS) ? (const float*)(uintptr_t)c.ptr[3] : nullptr;
   float* ws = (float*)ctx->workspace;
   if (splits > 1 && (batch > 1 || (int64_t)splits * M * N * 4 > ctx->workspace_bytes))
     return gh_fail(ctx, GH_ESTATE, "sgemm: split-K slabs do not fit the workspace");
   const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, splits > 1 ? splits : batch);
 #define GH_GEMM_LAUNCH(TA_, TB_, V_)                                                                 \
   hipLaunchKernelGGL((k_sgemm<BM, BN, BK, WAVES_M, TA_, TB_, V_>), grid, dim3(kThreads), 0, ctx->stream, \
-                     A, B, C, M, N, K, lda, ldb, ldc, sA, sB, sC, act, c.f[0], splits, ws)
+                     A, B, C, M, N, K, lda, ldb, ldc, sA, sB, sC, act, c.f[0], splits, ws, bias)
   if (vec) {
     if (!ta && !tb) GH_GEMM_LAUNCH(false, false, true);
     else if (!ta && tb) GH_GEMM_LAUNCH(false, true, true);
@@ -1657,7 +1667,7 @@ int launch_sgemm_cfg(gh_ctx* ctx, const gh_cmd& c, int splits) {
   int64_t blocks = cdiv(total, 256);
   if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
   hipLaunchKernelGGL((k_splitk_reduce<StoreRowMajor>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws,
-                     splits, M, N, StoreRowMajor{C, ldc}, act, c.f[0]);
+                     splits, M, N, StoreRowMajor{C, ldc, bias}, act, c.f[0]);
   return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
 }
 
@@ -1906,6 +1916,7 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   const float* A = (const float*)(uintptr_t)c.ptr[0];
   const float* B = (const float*)(uintptr_t)c.ptr[1];
   float* C = (float*)(uintptr_t)c.ptr[2];
+  const float* bias = (c.flags & GH_FLAG_GEMM_BIAS) ? (const float*)(uintptr_t)c.ptr[3] : nullptr;
   // Few 32x32 tiles: 16-row tiles reach two to four times as many compute units.
   // Shapes that may carry the softmax epilogue (N <= 32) stay on one kernel, so
   // the fused and the separate softmax see the same product bits.
@@ -1919,7 +1930,7 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
     const bool narrow = force ? !strcmp(force, "16x16") : blocks_wide * 2 <= ctx->cu_count;
     auto launch16 = [&](auto kernel, int bn) {
       hipLaunchKernelGGL(kernel, dim3((N + bn - 1) / bn, (M + 15) / 16), dim3(WV * 64), 0, ctx->stream, A, B, C, M,
-                         N, K, lda, ldb, ldc, act, c.f[0]);
+                         N, K, lda, ldb, ldc, act, c.f[0], bias);
     };
     const bool vec = K % 4 == 0;
     if (narrow) { if (vec) launch16(k_gemm_skinny16<WV, 1, true>, 16); else launch16(k_gemm_skinny16<WV, 1, false>, 16); }
@@ -1929,7 +1940,7 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   const bool vec_b = N >= 32;   // whole column tiles (the last one moved left)
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, dim3(WV * 64), 0, ctx->stream, A, B, C, M, N, K, lda, ldb, ldc, act, c.f[0],
-                       softmax);
+                       softmax, bias);
   };
   if (vec_a && vec_b) launch(k_gemm_skinny<WV, true, true>);
   else if (vec_a) launch(k_gemm_skinny<WV, true, false>);
@@ -2066,7 +2077,7 @@ int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
     int rc = gh_check_hip(ctx, hipGetLastError(), "direct filter-gradient launch");
     if (rc) return rc;
     hipLaunchKernelGGL((k_splitk_reduce4<StoreRowMajor>), dim3((int)cdiv((int64_t)F * CKK * 4, 256)), dim3(256),
-                       0, ctx->stream, wsd, G, F, CKK, StoreRowMajor{(float*)(uintptr_t)c.ptr[2], CKK}, 0, 0.f);
+                       0, ctx->stream, wsd, G, F, CKK, StoreRowMajor{(float*)(uintptr_t)c.ptr[2], CKK, nullptr}, 0, 0.f);
     return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
   }
   constexpr int BM = 64, BN = 64, BK = 32;
@@ -2089,12 +2100,12 @@ int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
   if (rc || splits <= 1) return rc;
   if (splits >= 8) {
     hipLaunchKernelGGL((k_splitk_reduce4<StoreRowMajor>), dim3((int)cdiv((int64_t)F * CKK * 4, 256)), dim3(256),
-                       0, ctx->stream, ws, (int)splits, F, CKK, StoreRowMajor{dw, CKK}, 0, 0.f);
+                       0, ctx->stream, ws, (int)splits, F, CKK, StoreRowMajor{dw, CKK, nullptr}, 0, 0.f);
   } else {
     int64_t blocks = cdiv((int64_t)F * CKK, 256);
     if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
     hipLaunchKernelGGL((k_splitk_reduce<StoreRowMajor>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws,
-                       (int)splits, F, CKK, StoreRowMajor{dw, CKK}, 0, 0.f);
+                       (int)splits, F, CKK, StoreRowMajor{dw, CKK, nullptr}, 0, 0.f);
   }
   return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
 }

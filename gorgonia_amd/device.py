@@ -162,7 +162,8 @@ def cmd_copy(dst, src, nbytes):
 
 
 def cmd_gemm(a, b, c, m, n, k, lda=None, ldb=None, ldc=None, trans_a=False, trans_b=False,
-             batch=1, stride_a=0, stride_b=0, stride_c=0, act=None, alpha=0.0, dtype=_ffi.F32, softmax=False):
+             batch=1, stride_a=0, stride_b=0, stride_c=0, act=None, alpha=0.0, dtype=_ffi.F32, softmax=False,
+             bias=0):
     lda = lda if lda is not None else (m if trans_a else k)
     ldb = ldb if ldb is not None else (k if trans_b else n)
     ldc = ldc if ldc is not None else n
@@ -170,7 +171,9 @@ def cmd_gemm(a, b, c, m, n, k, lda=None, ldb=None, ldc=None, trans_a=False, tran
     fl |= {None: 0, "relu": _ffi.FLAG_ACT_RELU, "leaky": _ffi.FLAG_ACT_LEAKY}[act] | _ffi.flag_dtype(dtype)
     if softmax:
         fl |= _ffi.FLAG_GEMM_SOFTMAX
-    return make_cmd(_ffi.OP_GEMM, fl, (a, b, c), (m, n, k, lda, ldb, ldc, batch, stride_a, stride_b,
+    if bias:
+        fl |= _ffi.FLAG_GEMM_BIAS
+    return make_cmd(_ffi.OP_GEMM, fl, (a, b, c, bias), (m, n, k, lda, ldb, ldc, batch, stride_a, stride_b,
                                                   stride_c), (alpha,))
 
 

@@ -398,11 +398,13 @@ Status Engine::MatVecMul(Tensor& a, Tensor& b, Tensor& prealloc) {
   return Status::OK();
 }
 
-Status Engine::MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act, float alpha, bool softmax) {
+Status Engine::MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act, float alpha, bool softmax,
+                      uint64_t bias) {
   Status st = checkThreeFloat(a, b, prealloc);
   if (!st.ok()) return st.Wrap("MatMul failed pre check");
   if (a.dt == Dtype::Other) return Status::Err(GH_EINVAL, "Unsupported Dtype " + dtype_name(a.dt));
-  if (a.dt == Dtype::Float64 && act) return Status::Err(GH_EINVAL, "MatMul: no fused activation for float64");
+  if (a.dt == Dtype::Float64 && (act || bias))
+    return Status::Err(GH_EINVAL, "MatMul: no fused activation or bias for float64");
   if (a.shape.Dims() != 2 || b.shape.Dims() != 2 || prealloc.shape.Dims() != 2)
     return Status::Err(GH_EINVAL, "MatMul: operands must be matrices");
   const int64_t m = a.shape[0], k = a.shape[1], n = b.shape[1];
@@ -417,10 +419,10 @@ Status Engine::MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act, float alp
   c.opcode = GH_OP_GEMM;
   c.flags = (a.transposed ? GH_FLAG_TRANS_A : 0) | (b.transposed ? GH_FLAG_TRANS_B : 0) |
             (act == 1 ? GH_FLAG_ACT_RELU : act == 2 ? GH_FLAG_ACT_LEAKY : 0) |
-            (softmax ? GH_FLAG_GEMM_SOFTMAX : 0) |
+            (softmax ? GH_FLAG_GEMM_SOFTMAX : 0) | (bias ? GH_FLAG_GEMM_BIAS : 0) |
             GH_FLAG_DTYPE(a.dt == Dtype::Float64 ? GH_F64 : GH_F32);  // Dgemm / Sgemm, cuda/linalg.go:204-227
   c.f[0] = alpha;
-  c.ptr[0] = a.mem; c.ptr[1] = b.mem; c.ptr[2] = prealloc.mem;
+  c.ptr[0] = a.mem; c.ptr[1] = b.mem; c.ptr[2] = prealloc.mem; c.ptr[3] = bias;
   c.dim[0] = m; c.dim[1] = n; c.dim[2] = k;
   c.dim[3] = a.transposed ? m : k;
   c.dim[4] = b.transposed ? k : n;

@@ -151,7 +151,9 @@ class Engine {
   // ---- linalg (cuda/linalg.go:47-285) -----------------------------------------------------
   Status MatVecMul(Tensor& a, Tensor& b, Tensor& prealloc);
   // act: 0 none, 1 Rectify, 2 LeakyRelu(alpha) applied to the product (fused epilogue).
-  Status MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act = 0, float alpha = 0.f, bool softmax = false);
+  // bias (device address of n floats, 0 = none) is added to every row before the activation
+  Status MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act = 0, float alpha = 0.f, bool softmax = false,
+                uint64_t bias = 0);
   Status Outer(Tensor& a, Tensor& b, Tensor& prealloc);
   // batchedMatMul (operatorLinAlg.go:435-502): one strided-batched launch.
   Status BatchedMatMul(Tensor& a, Tensor& b, Tensor& c, bool transA, bool transB);

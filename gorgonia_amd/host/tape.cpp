@@ -264,7 +264,7 @@ static std::string op_name(const OpSpec& op) {
     case OpKind::ElemUnary: return "elemunary." + op.name;
     case OpKind::BroadcastBin: return std::string("broadcast.") + bins[op.fn];
     case OpKind::MatMul:
-      return std::string("matmul") + (op.fuse_act_relu ? "+rectify" : op.fuse_act_leaky ? "+leakyrelu" : "") +
+      return std::string("matmul") + (op.fuse_bias ? "+bias" : "") + (op.fuse_act_relu ? "+rectify" : op.fuse_act_leaky ? "+leakyrelu" : "") +
              (op.fuse_softmax ? "+softmax" : "");
     case OpKind::MatVecMul: return "matvecmul";
     case OpKind::Outer: return "outer";
@@ -326,7 +326,8 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       if (op.transA) { std::swap(a.shape.d[0], a.shape.d[1]); a.transposed = !a.transposed; }
       if (op.transB) { std::swap(b.shape.d[0], b.shape.d[1]); b.transposed = !b.transposed; }
       const int act = op.fuse_act_relu ? 1 : op.fuse_act_leaky ? 2 : 0;
-      return e.MatMul(a, b, prealloc, act, (float)op.f0, op.fuse_softmax);
+      if (op.fuse_bias && in.size() != 3) return bad("MatMul: fused bias needs a third input");
+      return e.MatMul(a, b, prealloc, act, (float)op.f0, op.fuse_softmax, op.fuse_bias ? in[2]->mem : 0);
     }
     case OpKind::MatVecMul: {
       Tensor a = *in[0];
@@ -584,9 +585,14 @@ int Graph::FuseActivations() {
     if (n.is_input || n.fused_away || n.inputs.empty()) continue;
     const OpKind k = n.op.kind;
     if (k != OpKind::Rectify && k != OpKind::LeakyRelu && k != OpKind::BatchNorm && k != OpKind::MaxPool2D &&
-        k != OpKind::SoftMax)
+        k != OpKind::SoftMax && !(k == OpKind::BroadcastBin && n.op.fn == GH_ADD))
       continue;
-    Node& p = nodes_[(size_t)n.inputs[0]];
+    // the producer: the first input, or for a broadcast add whichever input is the product
+    int pi = n.inputs[0];
+    if (k == OpKind::BroadcastBin && n.inputs.size() == 2 && nodes_[(size_t)n.inputs[1]].op.kind == OpKind::MatMul &&
+        !nodes_[(size_t)n.inputs[1]].is_input)
+      pi = n.inputs[1];
+    Node& p = nodes_[(size_t)pi];
     if (p.is_input || p.fused_away || p.read_into || uses[(size_t)p.id] != 1) continue;
     if (p.op.kind != OpKind::Conv2d && p.op.kind != OpKind::MatMul) continue;
     if (p.dt != Dtype::Float32) continue;   // the epilogues exist for float32 only
@@ -594,7 +600,16 @@ int Graph::FuseActivations() {
     std::vector<int> inputs = p.inputs;
     const bool has_act = op.fuse_act_relu || op.fuse_act_leaky;
     if (op.fuse_softmax) continue;   // nothing rides behind a softmax
-    if (k == OpKind::SoftMax) {
+    if (k == OpKind::BroadcastBin) {
+      // Add(Mul(x, w), b) with b one value per column: a + b and b + a are the same bits
+      if (op.kind != OpKind::MatMul || has_act || op.fuse_bias || n.inputs.size() != 2 || n.shape.Dims() != 2) continue;
+      const Node& small = nodes_[(size_t)(pi == n.inputs[0] ? n.inputs[1] : n.inputs[0])];
+      if (small.dt != Dtype::Float32 || small.shape.Dims() != 2 || small.shape[0] != 1 || small.shape[1] != n.shape[1] ||
+          n.shape[0] == 1)
+        continue;
+      op.fuse_bias = true;
+      inputs.push_back(small.id);
+    } else if (k == OpKind::SoftMax) {
       if (op.kind != OpKind::MatMul || op.transA || op.transB || n.shape.Dims() != 2) continue;
       gh_cmd c{};
       c.opcode = GH_OP_GEMM;
@@ -803,6 +818,11 @@ Status TapeMachine::flush() {
   const bool same = sc.cmds.size() == cur.size() &&
                     (cur.empty() || std::memcmp(sc.cmds.data(), cur.data(), cur.size() * sizeof(gh_cmd)) == 0);
   if (cur.empty()) return eng_.Sync();
+  // A graph launch has a higher fixed cost than a handful of plain launches
+  // (measured on MI355X: one small kernel per run 29 us replayed against 13 us
+  // eager, break-even at about five kernels), so short segments stay eager.
+  constexpr size_t kMinGraphCmds = 5;
+  if (cur.size() < kMinGraphCmds) return eng_.DoWork();
   if (sc.graph_id >= 0 && same) {
     eng_.DropSegment();
     Status st = eng_.GraphLaunch(sc.graph_id);

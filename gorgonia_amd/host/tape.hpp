@@ -76,6 +76,7 @@ struct OpSpec {
   bool fuse_act_relu = false;
   bool fuse_act_leaky = false;
   bool fuse_pool2 = false;
+  bool fuse_bias = false;     // MatMul only: the BroadcastAdd of a row vector that follows (last input)
   bool fuse_softmax = false;  // MatMul only: the SoftMax that follows, where gh_gemm_can_softmax allows
 };
 

@@ -132,6 +132,7 @@ enum gh_unaryfn {
 #define GH_FLAG_BN_EVAL      (1u << 26)   /* BN_BWD: eval-mode gradient dy/sqrt(var+eps)       */
 #define GH_FLAG_CONV_POOL2   (1u << 25)   /* CONV2D: 2x2 stride-2 unpadded MaxPool2D on the result */
 #define GH_FLAG_GEMM_SOFTMAX (1u << 27)   /* GEMM: row SoftMax on the result (after the activation) */
+#define GH_FLAG_GEMM_BIAS    (1u << 28)   /* GEMM: ptr[3] = N floats added to every row of the product (before the activation) */
 
 /*
  * One operator.  Field use per opcode:
@@ -149,6 +150,10 @@ enum gh_unaryfn {
  *             dim[6]=batch (0/1 = single)  dim[7..9]=strideA,strideB,strideC
  *             row-major; C(m x n) = op(A)(m x k) * op(B)(k x n)
  *             float64 with GH_FLAG_DTYPE(GH_F64) (no fused activation)
+ *             float32 epilogue, stored bits those of the separate commands, in
+ *             this order: GEMM_BIAS (ptr[3] = n floats, added to every row - the
+ *             BroadcastAdd of a dense layer's bias), ACT_RELU / ACT_LEAKY,
+ *             GEMM_SOFTMAX (see gh_gemm_can_softmax)
  * GEMV        ptr[0]=A ptr[1]=x ptr[2]=y   dim[0..2]=m,n,lda ; A is (m x n) row-major,
  *             y(m)=A x, or with TRANS_A y(n)=A^T x
  * OUTER       ptr[0]=x ptr[1]=y ptr[2]=A   dim[0..1]=m,n ; A(m x n) = x y^T

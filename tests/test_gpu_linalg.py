@@ -15,15 +15,17 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-5
 
 
-def _run_gemm(ctx, A, B, ta=False, tb=False, act=None, alpha=0.0, softmax=False):
+def _run_gemm(ctx, A, B, ta=False, tb=False, act=None, alpha=0.0, softmax=False, bias=None):
     m, k = (A.shape[1], A.shape[0]) if ta else A.shape
     n = B.shape[0] if tb else B.shape[1]
     dA, dB = ctx.upload(A), ctx.upload(B)
+    dbias = ctx.upload(bias) if bias is not None else 0
     dC = ctx.malloc(m * n * 4)
     ctx.run(D.cmd_fill(dC, m * n, np.nan))
-    ctx.run(D.cmd_gemm(dA, dB, dC, m, n, k, trans_a=ta, trans_b=tb, act=act, alpha=alpha, softmax=softmax))
+    ctx.run(D.cmd_gemm(dA, dB, dC, m, n, k, trans_a=ta, trans_b=tb, act=act, alpha=alpha, softmax=softmax,
+                       bias=dbias))
     out = ctx.d2h(dC, (m, n))
-    for p in (dA, dB, dC):
+    for p in (dA, dB, dC) + ((dbias,) if dbias else ()):
         ctx.free(p)
     return out
 
@@ -71,6 +73,38 @@ def test_matmul_fused_relu_epilogue(ctx):
     assert_bits_equal(fused, O.relu(plain).reshape(plain.shape), "gemm+relu epilogue")
     fusedl = _run_gemm(ctx, A, B, act="leaky", alpha=0.1)
     assert_bits_equal(fusedl, O.leaky_relu(plain, 0.1).reshape(plain.shape), "gemm+leaky epilogue")
+
+
+@pytest.mark.parametrize("m,k,n,ta,tb", [
+    (256, 784, 300, False, False),    # 16x32 tiles of the small-output kernel
+    (64, 512, 1000, False, False),    # 16x16 tiles
+    (256, 100, 10, False, False),     # 32x32 tiles
+    (512, 512, 512, False, False),    # tiled kernel
+    (300, 70, 200, True, True),       # tiled kernel, transposed views
+    (1024, 4096, 64, False, False),   # tiled kernel with a split K range and the reduction pass
+])
+def test_matmul_fused_bias_epilogue(ctx, m, k, n, ta, tb):
+    """Mul -> BroadcastAdd(row bias) [-> Rectify] as one command stores the bits of the separate commands."""
+    A = synth.normal(5, (k, m) if ta else (m, k))
+    B = synth.normal(6, (n, k) if tb else (k, n))
+    bias = synth.normal(7, (n,))
+    plain = _run_gemm(ctx, A, B, ta, tb)
+    want = O.bcast_binop("add", plain.reshape(-1), bias, m, n, 1).reshape(m, n)
+    assert_bits_equal(_run_gemm(ctx, A, B, ta, tb, bias=bias), want, "gemm+bias epilogue")
+    assert_bits_equal(_run_gemm(ctx, A, B, ta, tb, bias=bias, act="relu"), O.relu(want).reshape(m, n),
+                      "gemm+bias+relu epilogue")
+    if n <= 32 and not (ta or tb):
+        assert_bits_equal(_run_gemm(ctx, A, B, bias=bias, softmax=True), O.softmax(want), "gemm+bias+softmax epilogue")
+
+
+def test_matmul_bias_flag_checks(ctx):
+    import ctypes as C
+    buf = C.create_string_buffer(256)
+    for cmd in (D.cmd_gemm(1, 1, 1, 64, 64, 64, bias=1, dtype=1), ):
+        assert ctx.lib.gh_validate(C.byref(cmd), 1, buf, 256) != 0 and b"bias" in buf.value
+    cmd = D.cmd_gemm(1, 1, 1, 64, 64, 64, bias=1)
+    cmd.ptr[3] = 0
+    assert ctx.lib.gh_validate(C.byref(cmd), 1, buf, 256) != 0 and b"bias" in buf.value
 
 
 @pytest.mark.parametrize("m,k,n", [(128, 625, 10), (1, 32, 1), (33, 100, 32), (2048, 64, 7), (50, 48, 31)])

@@ -4,7 +4,7 @@ batching, hipGraph replay and Reset semantics."""
 import numpy as np
 import pytest
 
-from gorgonia_amd import configs, graph as G
+from gorgonia_amd import configs, graph as G, synth
 from oracle import forward as F
 from tests.util import assert_bits_equal, rel_frobenius, ulp_diff
 
@@ -27,6 +27,22 @@ def test_mlp_forward(ctx):
     assert np.allclose(res["out"].sum(axis=1), 1.0, atol=1e-5)
     assert m.segments() == 1
     m.Close()
+
+
+def test_mlp_dense_layers_fold_bias_activation_and_softmax(ctx):
+    """Mul -> BroadcastAdd(bias) -> Rectify / SoftMax of every dense layer becomes one product
+    command; the stored bits are those of the separate operators (non-zero biases here)."""
+    inp = configs.mlp_inputs(64)
+    for i, nb in enumerate((300, 100, 10)):
+        inp[f"b{i}"] = synth.normal(900 + i, (1, nb), 0.0, 0.5)
+    m1, _, r1 = run_once(configs.build_mlp, inp)
+    m2, _, r2 = run_once(configs.build_mlp, inp, fuse_activations=True)
+    assert rel_frobenius(r1["out"], F.mlp(inp)) <= 1e-5
+    assert_bits_equal(r1["out"], r2["out"], "fused dense layers change nothing")
+    assert m2.fused == 6  # three biases, two activations, the softmax
+    prog = m2.program()
+    assert prog.count("matmul+bias+rectify") == 2 and prog.count("matmul+bias+softmax") == 1
+    m1.Close(); m2.Close()
 
 
 def test_elementwise_chain_small_and_full(ctx):
