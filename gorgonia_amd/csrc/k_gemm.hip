@@ -920,7 +920,15 @@ __device__ __forceinline__ void conv3_tile(const float* __restrict__ x, const fl
   // between the MFMAs (a few percent slower); eight wavefronts per block with
   // the k-steps of a chunk split between two quads (MFMA phase at its ideal
   // length, but the wait for the next chunk's loads grows by as much; large
-  // layers 8-25 % slower); a per-block rotation of the chunk order (no change).
+  // layers 8-25 % slower); a per-block rotation of the chunk order (no change);
+  // a kernel of its own in which global_load_lds copies the operands straight
+  // into a ring of four LDS stages of four channels (filter rows as they lie in
+  // memory, pitch 36 floats, A fragments read along k; every thread issuing the
+  // same six copies per chunk so that "chunk landed" is s_waitcnt vmcnt(12), a
+  // bare s_barrier per chunk, copies written as asm because the compiler waits
+  // for every tracked LDS copy at each loop merge): bit-correct, loads three
+  // phases ahead and no LDS stores, yet 4-13 % slower on every layer it took -
+  // so load latency is not what holds this kernel back.
   auto stage_load = [&](int chunk) {
     const int c0 = chunk * CC;
     const float* xc = x + (int64_t)c0 * HW;
