@@ -252,6 +252,18 @@ int gh_submit(gh_ctx* ctx, const gh_cmd* cmds, int n) {
     std::string m;
     int rc = gh_validate_cmd(cmds[i], m);
     if (rc) return gh_fail(ctx, rc, "cmd " + std::to_string(i) + ": " + m);
+    // a run of solver steps with the same settings (a model's weight tensors) is one launch
+    const int run = gh_solver_run_length(cmds + i, n - i);
+    if (run > 1) {
+      for (int j = 1; j < run; j++) {
+        rc = gh_validate_cmd(cmds[i + j], m);
+        if (rc) return gh_fail(ctx, rc, "cmd " + std::to_string(i + j) + ": " + m);
+      }
+      rc = gh_launch_solver_steps(ctx, cmds + i, run);
+      if (rc) return rc;
+      i += run - 1;
+      continue;
+    }
     rc = dispatch(ctx, cmds[i]);
     if (rc) return rc;
   }

@@ -58,6 +58,8 @@ int gh_launch_bn_train(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_bn_bwd(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_softmax_bwd(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_solver_step(gh_ctx* ctx, const gh_cmd& c);
+int gh_solver_run_length(const gh_cmd* cmds, int n);
+int gh_launch_solver_steps(gh_ctx* ctx, const gh_cmd* cmds, int count);
 int gh_launch_rand_uniform(gh_ctx* ctx, const gh_cmd& c);
 // float64 twins of the forward neural-network operators (k_nn64.hip)
 int gh_launch_relu_f64(gh_ctx* ctx, const gh_cmd& c, bool leaky);

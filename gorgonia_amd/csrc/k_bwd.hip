@@ -7,6 +7,7 @@
 // (op_nn.go:1834-1943) and softmaxDiffOp (op_softmax.go:266-279); the
 // arithmetic follows the CPU engine.  All of them are HBM-bound.
 #include <cfloat>
+#include <cstring>
 
 #include "gh_internal.h"
 
@@ -354,12 +355,31 @@ __device__ __forceinline__ float prep_grad(float g, float w, int use, const Solv
   return g;
 }
 
+// Up to kSolverBatch weight tensors per launch: a model's solver steps are many
+// small tensors, and one launch per tensor costs more than the arithmetic.
+// Tensor t owns workgroups [first[t], first[t + 1]).
+constexpr int kSolverBatch = 8;
+struct SolverBatch {
+  float* w[kSolverBatch]; const float* g[kSolverBatch]; float* c1[kSolverBatch]; float* c2[kSolverBatch];
+  int64_t n[kSolverBatch];
+  int first[kSolverBatch + 1];
+  int count;
+};
+
 template <int KIND>
-__global__ __launch_bounds__(kBlock) void k_solver_step(float* __restrict__ w, const float* __restrict__ g,
-                                                        float* __restrict__ c1, float* __restrict__ c2,
-                                                        int64_t n, int use, SolverPar p) {
+__global__ __launch_bounds__(kBlock) void k_solver_step(SolverBatch sb, int use, SolverPar p) {
+  int t = 0;
+#pragma unroll
+  for (int q = 1; q < kSolverBatch; q++)
+    if (q < sb.count && (int)blockIdx.x >= sb.first[q]) t = q;
+  float* __restrict__ w = sb.w[t];
+  const float* __restrict__ g = sb.g[t];
+  float* __restrict__ c1 = sb.c1[t];
+  float* __restrict__ c2 = sb.c2[t];
+  const int64_t n = sb.n[t];
+  const int64_t nblk = sb.first[t + 1] - sb.first[t];
   const float neg_eta = -p.eta;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+  for (int64_t i = (int64_t)(blockIdx.x - sb.first[t]) * kBlock + threadIdx.x; i < n; i += nblk * kBlock) {
     if (KIND == GH_SOLVER_VANILLA) {
       float gi = prep_grad(g[i], w[i], use, p);
       gi = gi * neg_eta;
@@ -537,26 +557,57 @@ int gh_launch_softmax_bwd(gh_ctx* ctx, const gh_cmd& c) {
   return gh_check_hip(ctx, hipGetLastError(), "softmax backward launch");
 }
 
-int gh_launch_solver_step(gh_ctx* ctx, const gh_cmd& c) {
-  const int64_t n = c.dim[0];
-  if (n == 0) return GH_OK;
+// How many of the commands cmds[0..n) form one solver launch: consecutive
+// SOLVER_STEP commands with the same solver, options and hyper-parameters.
+int gh_solver_run_length(const gh_cmd* cmds, int n) {
+  if (n <= 0 || cmds[0].opcode != GH_OP_SOLVER_STEP) return 0;
+  int len = 1;
+  while (len < n && len < kSolverBatch && cmds[len].opcode == GH_OP_SOLVER_STEP && cmds[len].flags == cmds[0].flags &&
+         memcmp(cmds[len].f, cmds[0].f, sizeof(cmds[0].f)) == 0) {
+    // a tensor stepped twice keeps its two steps in order: the run ends before the repeat
+    bool repeat = false;
+    for (int j = 0; j < len; j++) repeat = repeat || cmds[j].ptr[0] == cmds[len].ptr[0];
+    if (repeat) break;
+    len++;
+  }
+  return len;
+}
+
+// One launch for cmds[0..count) (count from gh_solver_run_length).
+int gh_launch_solver_steps(gh_ctx* ctx, const gh_cmd* cmds, int count) {
+  const gh_cmd& c = cmds[0];
   const int kind = (int)gh_fn(c.flags), use = (int)gh_mode(c.flags);
   SolverPar p{c.f[0], c.f[1], c.f[2], c.f[3], c.f[4], c.f[5], c.f[6], c.f[7], c.f[8], c.f[9]};
-  float* w = (float*)(uintptr_t)c.ptr[0];
-  const float* g = (const float*)(uintptr_t)c.ptr[1];
-  float* c1 = (float*)(uintptr_t)c.ptr[2];
-  float* c2 = (float*)(uintptr_t)c.ptr[3];
-  int64_t blocks = (n + kBlock - 1) / kBlock;
-  if (blocks > (int64_t)ctx->cu_count * 32) blocks = (int64_t)ctx->cu_count * 32;
-  const dim3 grid((int)blocks), block(kBlock);
+  SolverBatch sb{};
+  int nt = 0, blocks_total = 0;
+  for (int i = 0; i < count; i++) {
+    const int64_t n = cmds[i].dim[0];
+    if (n == 0) continue;
+    sb.w[nt] = (float*)(uintptr_t)cmds[i].ptr[0];
+    sb.g[nt] = (const float*)(uintptr_t)cmds[i].ptr[1];
+    sb.c1[nt] = (float*)(uintptr_t)cmds[i].ptr[2];
+    sb.c2[nt] = (float*)(uintptr_t)cmds[i].ptr[3];
+    sb.n[nt] = n;
+    int64_t blocks = (n + kBlock - 1) / kBlock;
+    if (blocks > (int64_t)ctx->cu_count * 32) blocks = (int64_t)ctx->cu_count * 32;
+    sb.first[nt] = blocks_total;
+    blocks_total += (int)blocks;
+    nt++;
+  }
+  if (nt == 0) return GH_OK;
+  for (int i = nt; i <= kSolverBatch; i++) sb.first[i] = blocks_total;
+  sb.count = nt;
+  const dim3 grid(blocks_total), block(kBlock);
   if (kind == GH_SOLVER_VANILLA)
-    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_VANILLA>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p);
+    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_VANILLA>), grid, block, 0, ctx->stream, sb, use, p);
   else if (kind == GH_SOLVER_RMSPROP)
-    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_RMSPROP>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p);
+    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_RMSPROP>), grid, block, 0, ctx->stream, sb, use, p);
   else
-    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_ADAM>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p);
+    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_ADAM>), grid, block, 0, ctx->stream, sb, use, p);
   return gh_check_hip(ctx, hipGetLastError(), "solver step launch");
 }
+
+int gh_launch_solver_step(gh_ctx* ctx, const gh_cmd& c) { return gh_launch_solver_steps(ctx, &c, 1); }
 
 static int stream_blocks(gh_ctx* ctx, int64_t n) {
   int64_t blocks = (n + kBlock - 1) / kBlock;

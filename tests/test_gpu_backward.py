@@ -180,6 +180,44 @@ def test_solver_steps_bit_exact(ctx, kind, kw):
         ctx.free(p)
 
 
+@pytest.mark.parametrize("kind,kw", [("rmsprop", dict(eta=0.01, clip=2.0)), ("adam", dict(eta=0.001, iteration=3))])
+def test_solver_steps_of_many_tensors_in_one_submit(ctx, kind, kw):
+    """A run of solver steps with the same settings handed over in one submit is executed as
+    one launch; weights and caches are those of one submit per tensor (eleven tensors: more
+    than one launch holds; ragged and empty sizes; the first tensor stepped twice, in order)."""
+    sizes = [1, 255, 256, 257, 1000, 0, 70001, 33, 4096, 5, 12345]
+    par, use = O.solver_params(kind=kind, **kw)
+    ws = [synth.normal(50 + i, (max(n, 1),))[:n] for i, n in enumerate(sizes)]
+    gs = [synth.normal(80 + i, (max(n, 1),), 0.0, 3.0)[:n] for i, n in enumerate(sizes)]
+    results = []
+    for batched in (False, True):
+        bufs = []
+        cmds = []
+        for w, g in zip(ws, gs):
+            n = w.size
+            pw, pg = ctx.upload(w if n else np.zeros(1, np.float32)), ctx.upload(g if n else np.zeros(1, np.float32))
+            pc1, pc2 = ctx.upload(np.zeros(max(n, 1), np.float32)), ctx.upload(np.zeros(max(n, 1), np.float32))
+            bufs.append((pw, pg, pc1, pc2, n))
+            cmds.append(D.cmd_solver_step(kind, pw, pg, n, par, use, pc1, pc2))
+        cmds.append(D.cmd_solver_step(kind, bufs[0][0], bufs[0][1], sizes[0], par, use, bufs[0][2], bufs[0][3]))
+        if batched:
+            ctx.run(cmds)
+        else:
+            for c in cmds:
+                ctx.run(c)
+        results.append([(ctx.d2h(pw, (max(n, 1),))[:n], ctx.d2h(pc1, (max(n, 1),))[:n], ctx.d2h(pc2, (max(n, 1),))[:n])
+                        for pw, pg, pc1, pc2, n in bufs])
+        for b in bufs:
+            for q in b[:4]:
+                ctx.free(q)
+    for (w1, a1, b1), (w2, a2, b2) in zip(*results):
+        assert_bits_equal(w1, w2, "weights: one submit == one submit per tensor")
+        assert_bits_equal(a1, a2, "cache")
+        assert_bits_equal(b1, b2, "second cache")
+    w_ref, _, c_ref, v_ref = O.solver_step(kind, ws[4], gs[4], np.zeros(1000, np.float32), np.zeros(1000, np.float32), **kw)
+    assert_bits_equal(results[1][4][0], w_ref, "batched step vs oracle")
+
+
 def test_backward_commands_validate(ctx):
     import ctypes as C
     buf = C.create_string_buffer(256)
