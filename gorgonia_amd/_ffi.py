@@ -20,7 +20,7 @@ ERR_NAMES = {0: "GH_OK", 1: "GH_EINVAL", 2: "GH_EDEVICE", 3: "GH_EOOM", 4: "GH_E
 (OP_NOP, OP_ELEM_BIN, OP_ELEM_UNARY, OP_BCAST_BIN, OP_MEMCPY_D2D, OP_GEMM, OP_GEMV, OP_OUTER,
  OP_CONV2D, OP_MAXPOOL2D, OP_BN_INFER, OP_RELU, OP_LEAKY_RELU, OP_SOFTMAX, OP_HAS_NAN, OP_HAS_INF,
  OP_FILL, OP_MAXPOOL2D_BWD, OP_CONV2D_BWD_DATA, OP_CONV2D_BWD_FILTER, OP_BN_TRAIN, OP_BN_BWD,
- OP_SOFTMAX_BWD, OP_SOLVER_STEP, OP_RAND_UNIFORM, OP_DROPOUT, OP_DROPOUT_BWD) = range(27)
+ OP_SOFTMAX_BWD, OP_SOLVER_STEP, OP_RAND_UNIFORM, OP_DROPOUT, OP_DROPOUT_BWD, OP_RELU_BWD) = range(28)
 
 BIN_FN = {"mod": 11, "add": 0, "sub": 1, "mul": 2, "div": 3, "pow": 4, "lt": 5, "lte": 6, "gt": 7, "gte": 8,
           "eq": 9, "ne": 10}

@@ -115,7 +115,6 @@ def build_convnet_train(inp, onehot, lr, read_grads=True, solver="set"):
     x = G.NewTensor(g, inp["x"], True)
     y = G.NewTensor(g, onehot, True)
     w = [G.NewTensor(g, inp[f"w{i}"], True) for i in range(5)]
-    zero = G.NewScalar(g, 0.0)
     lr_s = G.NewScalar(g, lr)
     scale = G.NewScalar(g, -1.0 / onehot.size)
     conv = dict(kernelShape=(3, 3), pad=(1, 1), stride=(1, 1), dilation=(1, 1))
@@ -133,12 +132,12 @@ def build_convnet_train(inp, onehot, lr, read_grads=True, solver="set"):
     # backward
     g4 = G.SoftMaxDiff(out, G.HadamardProd(y, scale))
     dw = {4: G.Mul(a3, g4, transA=True)}
-    dz3 = G.HadamardProd(G.Mul(g4, w[4], transB=True), G.Gte(z3, zero))
+    dz3 = G.RectifyDiff(z3, G.Mul(g4, w[4], transB=True))
     dw[3] = G.Mul(r, dz3, transA=True)
     grad = G.Reshape(G.Mul(dz3, w[3], transB=True), h.Shape())
     for i in (2, 1, 0):
         x_in, z, a = acts[i]
-        dz = G.HadamardProd(G.MaxPool2DDiff(a, grad, (2, 2), (0, 0), (2, 2)), G.Gte(z, zero))
+        dz = G.RectifyDiff(z, G.MaxPool2DDiff(a, grad, (2, 2), (0, 0), (2, 2)))
         dw[i] = G.Conv2dDiffFilter(x_in, dz, **conv)
         if i:
             grad = G.Conv2dDiffImage(dz, w[i], x_in.Shape(), **conv)

@@ -227,6 +227,7 @@ static int dispatch(gh_ctx* ctx, const gh_cmd& c) {
     case GH_OP_RAND_UNIFORM: return gh_launch_rand_uniform(ctx, c);
     case GH_OP_DROPOUT: return gh_launch_dropout(ctx, c);
     case GH_OP_DROPOUT_BWD: return gh_launch_dropout_bwd(ctx, c);
+    case GH_OP_RELU_BWD: return gh_launch_relu_bwd(ctx, c);
   }
   return GH_ENOFUNC;
 }

@@ -41,6 +41,7 @@ int gh_launch_elem_bin(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_elem_unary(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_bcast_bin(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_relu(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_relu_bwd(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_leaky_relu(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_fill(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_has_nan_inf(gh_ctx* ctx, const gh_cmd& c);

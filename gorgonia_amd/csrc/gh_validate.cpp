@@ -163,6 +163,11 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (c.dim[0] < 0) return bad("negative size");
       if (c.ptr[1] & 7) return bad("rand: state must be 8-byte aligned");
       return GH_OK;
+    case GH_OP_RELU_BWD:
+      if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
+      if (c.dim[0] < 0) return bad("negative size");
+      if (dt != GH_F32) return bad("relu backward: float32 only");
+      return GH_OK;
     case GH_OP_DROPOUT:
     case GH_OP_DROPOUT_BWD:
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");

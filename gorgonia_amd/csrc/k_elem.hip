@@ -474,6 +474,33 @@ __global__ __launch_bounds__(kBlock) void k_relu(const float* __restrict__ x, fl
   }
 }
 
+// Rectify's gradient as the CPU engine spells it: Gte(x, 0) written as 1.0 / 0.0,
+// then HadamardProd with the incoming gradient (one multiplication, so a masked
+// element is dy * 0.0 with dy's sign, and a NaN gradient stays NaN).
+__global__ __launch_bounds__(kBlock) void k_relu_bwd(const float* __restrict__ x, const float* dy, float* dx,
+                                                     int64_t n, int vec) {
+  typedef float V __attribute__((ext_vector_type(4)));
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (vec) {
+    const int64_t nv = n / 4;
+    const V* xv = reinterpret_cast<const V*>(x);
+    const V* gv = reinterpret_cast<const V*>(dy);
+    V* ov = reinterpret_cast<V*>(dx);
+    for (; i < nv; i += stride) {
+      const V a = xv[i], g = gv[i];
+      V r;
+#pragma unroll
+      for (int e = 0; e < 4; e++) r[e] = g[e] * (a[e] >= 0.0f ? 1.0f : 0.0f);
+      ov[i] = r;
+    }
+    const int64_t t = nv * 4 + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t < n) dx[t] = dy[t] * (x[t] >= 0.0f ? 1.0f : 0.0f);
+  } else {
+    for (; i < n; i += stride) dx[i] = dy[i] * (x[i] >= 0.0f ? 1.0f : 0.0f);
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void k_fill(float* A, int64_t n, float v) {
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) A[i] = v;
@@ -663,6 +690,16 @@ int gh_launch_relu(gh_ctx* ctx, const gh_cmd& c) {
                      ctx->stream, (const float*)(uintptr_t)c.ptr[0], (float*)(uintptr_t)c.ptr[1], n,
                      0.0f, vec);
   return gh_check_hip(ctx, hipGetLastError(), "relu launch");
+}
+
+int gh_launch_relu_bwd(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t n = c.dim[0];
+  if (n == 0) return GH_OK;
+  const int vec = aligned16(c.ptr[0]) && aligned16(c.ptr[1]) && aligned16(c.ptr[2]) && n >= 4;
+  hipLaunchKernelGGL(k_relu_bwd, dim3(grid_for(ctx, vec ? n / 4 + 4 : n, 2)), dim3(kBlock), 0, ctx->stream,
+                     (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                     (float*)(uintptr_t)c.ptr[2], n, vec);
+  return gh_check_hip(ctx, hipGetLastError(), "relu backward launch");
 }
 
 int gh_launch_leaky_relu(gh_ctx* ctx, const gh_cmd& c) {

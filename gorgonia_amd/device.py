@@ -289,6 +289,10 @@ def cmd_dropout_bwd(y, dy, dx, n, prob):
     return make_cmd(_ffi.OP_DROPOUT_BWD, 0, (y, dy, dx), (n,), (prob,))
 
 
+def cmd_relu_bwd(x, dy, dx, n):
+    return make_cmd(_ffi.OP_RELU_BWD, 0, (x, dy, dx), (n,))
+
+
 def cmd_has(kind, a, flag, n, dtype=_ffi.F32):
     op = _ffi.OP_HAS_NAN if kind == "nan" else _ffi.OP_HAS_INF
     return make_cmd(op, _ffi.flag_dtype(dtype), (a, flag), (n,))

@@ -14,7 +14,7 @@ from .engine import Engine, EngineError, GhhOp, load_host
 
 (K_ELEMBIN, K_ELEMUNARY, K_BCAST, K_MATMUL, K_MATVEC, K_OUTER, K_BMM, K_CONV2D, K_MAXPOOL, K_BN,
  K_RECTIFY, K_LEAKY, K_SOFTMAX, K_RESHAPE, K_MAXPOOL_DIFF, K_CONV_DIFF_DATA, K_CONV_DIFF_FILTER, K_BN_TRAIN,
- K_BN_DIFF, K_SOFTMAX_DIFF, K_SET, K_SOLVER, K_RAND_UNIFORM, K_DROPOUT, K_DROPOUT_DIFF) = range(25)
+ K_BN_DIFF, K_SOFTMAX_DIFF, K_SET, K_SOLVER, K_RAND_UNIFORM, K_DROPOUT, K_DROPOUT_DIFF, K_RECTIFY_DIFF) = range(26)
 
 
 class Node:
@@ -263,6 +263,13 @@ def Dropout(x, prob, rand=None, seed=0, training=True):
 def DropoutDiff(y, grad, prob):
     """dropoutDiffOp (op_dropout.go:205-238): dx = dy/p where y is non-zero, else 0."""
     return y.g.apply(K_DROPOUT_DIFF, [y, grad], f0=float(prob))
+
+
+def RectifyDiff(x, grad):
+    """The gradient of Rectify(x) as one operator, where the reference's device build calls the
+    activation backward of ops/nn/activation_cuda.go:130-153: grad * (x >= 0), the bits of
+    HadamardProd(grad, Gte(x, 0))."""
+    return x.g.apply(K_RECTIFY_DIFF, [x, grad])
 
 
 class TapeMachine:

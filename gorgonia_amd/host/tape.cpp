@@ -223,6 +223,11 @@ Status InferShape(const OpSpec& op, const std::vector<const Shape*>& in, Shape* 
       *out = s;
       return Status::OK();
     }
+    case OpKind::RectifyDiff:
+      if (!need(2) || !in[0]->Eq(*in[1]))
+        return bad("RectifyDiff: Shape mismatch. Expected " + in[0]->String() + ". Got " + (need(2) ? in[1]->String() : "nothing"));
+      *out = *in[0];
+      return Status::OK();
     case OpKind::Dropout:
     case OpKind::DropoutDiff:
       if (!need(2) || in[0]->TotalSize() != in[1]->TotalSize()) return bad("Dropout: operand sizes differ");
@@ -245,6 +250,7 @@ int OverwritesInput(const OpSpec& op) {
   // 476-481); everything else writes a fresh value
   if (op.kind == OpKind::ElemUnary) return 0;
   if (op.kind == OpKind::ElemBin) return 0;
+  if (op.kind == OpKind::RectifyDiff) return 1;   // the gradient is masked in place
   return -1;
 }
 
@@ -289,6 +295,7 @@ static std::string op_name(const OpSpec& op) {
     case OpKind::RandUniform: return "rand.uniform";
     case OpKind::Dropout: return "dropout";
     case OpKind::DropoutDiff: return "dropoutDiff";
+    case OpKind::RectifyDiff: return "rectifyDiff";
     case OpKind::SolverStep: return op.fn == GH_SOLVER_ADAM ? "solver.adam" : op.fn == GH_SOLVER_RMSPROP ? "solver.rmsprop" : "solver.vanilla";
   }
   return "?";
@@ -507,6 +514,15 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       c.ptr[0] = prealloc.mem;
       c.ptr[1] = in.empty() ? 0 : in[0]->mem;
       c.dim[0] = prealloc.shape.TotalSize(); c.dim[1] = op.ints[0]; c.dim[2] = op.ints[1];
+      e.Enqueue(c);
+      return Status::OK();
+    }
+    case OpKind::RectifyDiff: {
+      if (in[0]->dt != Dtype::Float32 || in[1]->dt != Dtype::Float32) return bad("RectifyDiff: Unsupported Dtype");
+      gh_cmd c{};
+      c.opcode = GH_OP_RELU_BWD;
+      c.ptr[0] = in[0]->mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
+      c.dim[0] = in[0]->shape.TotalSize();
       e.Enqueue(c);
       return Status::OK();
     }

@@ -57,7 +57,8 @@ enum class OpKind : int32_t {
                          // (a Float64 scalar used as raw bits) read as the offset and advanced by the size
   Dropout = 23,          // dropoutOp (op_dropout.go:107-132): inputs x, uniform numbers; f0 = probability,
                          // fn = 1 while training, 0 for the identity of evaluation
-  DropoutDiff = 24       // dropoutDiffOp (op_dropout.go:205-238): inputs y, grad; f0 = probability
+  DropoutDiff = 24,      // dropoutDiffOp (op_dropout.go:205-238): inputs y, grad; f0 = probability
+  RectifyDiff = 25       // activation backward (ops/nn/activation_cuda.go:130-153): inputs x, grad; grad * (x >= 0)
 };
 
 struct OpSpec {

@@ -91,6 +91,7 @@ enum gh_opcode {
   GH_OP_RAND_UNIFORM = 24,      /* the random source of Dropout (nn.go:71-77), generated on the device */
   GH_OP_DROPOUT = 25,           /* dropoutOp.do, op_dropout.go:107-132; ops/nn/dropout_cuda.go    */
   GH_OP_DROPOUT_BWD = 26,       /* dropoutDiffOp, op_dropout.go:205-238                            */
+  GH_OP_RELU_BWD = 27,          /* activation backward, ops/nn/activation_cuda.go:130-153; CPU: dy * (x >= 0) */
   GH_OP__COUNT
 };
 
@@ -196,6 +197,8 @@ enum gh_unaryfn {
  * DROPOUT     ptr[0]=x ptr[1]=y ptr[2]=r (uniform numbers, one per element)  dim[0]=n
  *             f[0]=drop probability ; y = r < 1-p ? x/(1-p) : 0 ; BN_EVAL or p == 0: y = x
  * DROPOUT_BWD ptr[0]=y ptr[1]=dy ptr[2]=dx         dim[0]=n f[0]=drop probability
+ * RELU_BWD    ptr[0]=x ptr[1]=dy ptr[2]=dx         dim[0]=n ; dx = dy * (x >= 0 ? 1 : 0), the bits of
+ *             Gte(x, 0) followed by HadamardProd; dx may be dy (in place)
  *             dx = (p != 0 && y != 0) ? dy/p : 0   (the reference divides by p)
  * SOLVER_STEP ptr[0]=weights ptr[1]=grad [ptr[2]=cache (RMSProp cache / Adam m) ptr[3]=Adam v]
  *             dim[0]=n ; flags: FN = gh_solver, MODE = use mask (1 l1reg, 2 l2reg, 4 clip,

@@ -218,6 +218,27 @@ def test_solver_steps_of_many_tensors_in_one_submit(ctx, kind, kw):
     assert_bits_equal(results[1][4][0], w_ref, "batched step vs oracle")
 
 
+@pytest.mark.parametrize("n", [1, 3, 4, 1000, 262147])
+def test_relu_backward_is_gte_then_hadamard(ctx, n):
+    """RELU_BWD stores the bits of Gte(x, 0) followed by HadamardProd with the gradient
+    (special values included), also in place on the gradient."""
+    x = synth.normal(61, (n,))
+    dy = synth.normal(62, (n,))
+    special = np.array([0.0, -0.0, np.nan, np.inf, -np.inf, 1e-45, -1e-45], np.float32)
+    k = min(n, special.size)
+    x[:k] = special[:k]
+    dy[n - k:] = special[:k]
+    mask = O.binop("gte", "vs", x, np.zeros(1, np.float32))
+    want = O.binop("mul", "vv", dy, mask)
+    px, pdy, pdx = ctx.upload(x), ctx.upload(dy), ctx.malloc(n * 4)
+    ctx.run(D.cmd_relu_bwd(px, pdy, pdx, n))
+    assert_bits_equal(ctx.d2h(pdx, (n,)), want, "relu backward")
+    ctx.run(D.cmd_relu_bwd(px, pdy, pdy, n))
+    assert_bits_equal(ctx.d2h(pdy, (n,)), want, "relu backward in place")
+    for p in (px, pdy, pdx):
+        ctx.free(p)
+
+
 def test_backward_commands_validate(ctx):
     import ctypes as C
     buf = C.create_string_buffer(256)
