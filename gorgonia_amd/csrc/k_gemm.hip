@@ -664,7 +664,12 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny(const float* __restrict
 // moved back to end at the matrix edge (M >= 16, N >= 16*NT), so no row or
 // column is ever masked; k past K is clamped in the address and zeroed before
 // the MFMA.
-template <int WV, int NT, bool VEC>
+// TA / TB: the operand is a transposed view (A stored k x m, B stored n x k, as
+// for k_sgemm); the lane's four k-values are then four loads for A and one
+// 128-bit load for B instead of the other way round.  N < 16 (NT = 1 only;
+// transposed views alone reach here with so few columns): one column tile,
+// column indices clamped in the loads and masked in the store.
+template <int WV, int NT, bool TA, bool TB>
 __global__ __launch_bounds__(WV * 64) void k_gemm_skinny16(const float* __restrict__ A,
                                                            const float* __restrict__ B,
                                                            float* __restrict__ C, int M, int N, int K,
@@ -676,29 +681,53 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny16(const float* __restri
   __shared__ float part[WV * TILE];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 15, q = lane >> 4;
-  const int m0 = min((int)blockIdx.y * 16, M - 16), n0 = min((int)blockIdx.x * BN, N - BN);
+  const bool ragged_n = N < BN;
+  const int m0 = min((int)blockIdx.y * 16, M - 16), n0 = ragged_n ? 0 : min((int)blockIdx.x * BN, N - BN);
   const int nchunks = (K + 15) / 16;
-  const float* const a_row = A + (int64_t)(m0 + i) * lda;
-  const float* const b_col = B + n0 + NT * i;
-  auto load = [&](int chunk, float (&a)[4], float (&b)[4][NT]) {
-    const int k0 = chunk * 16 + 4 * q;
-    if (VEC) {   // K % 4 == 0: a quad is whole or entirely past K
-      const f32x4 v = *reinterpret_cast<const f32x4_a4*>(a_row + min(k0, K - 4));
+  int ncol[NT];   // this lane's columns (clamped when the tile is wider than the matrix)
 #pragma unroll
-      for (int t = 0; t < 4; t++) a[t] = v[t];
+  for (int c = 0; c < NT; c++) ncol[c] = min(n0 + NT * i + c, N - 1);
+  // k runs along the row of an untransposed A and of a transposed B
+  const float* const a_base = TA ? A + m0 + i : A + (int64_t)(m0 + i) * lda;
+  // The lane's quad of chunk `chunk` starts at k0 = 16*chunk + 4*q; a quad that
+  // would stick out past K starts at K-4 instead, and its elements below k0
+  // (which the quad before it already covers) are zeroed before the MFMA.  So
+  // element t always stands for k = kb + t with kb = min(k0, K-4): every load is
+  // unconditional, k-contiguous operands are one 128-bit load at any 4-byte
+  // aligned address, and no loaded value is touched under a branch (which would
+  // make each load wait for the one before it).
+  auto load_k4 = [&](const float* row, int kb, float (&dst)[4]) {
+    const f32x4 v = *reinterpret_cast<const f32x4_a4*>(row + kb);
+#pragma unroll
+    for (int t = 0; t < 4; t++) dst[t] = v[t];
+  };
+  auto load = [&](int chunk, float (&a)[4], float (&b)[4][NT]) {
+    const int kb = min(chunk * 16 + 4 * q, K - 4);
+    if constexpr (TA) {
+#pragma unroll
+      for (int t = 0; t < 4; t++) a[t] = a_base[(int64_t)(kb + t) * lda];
+    } else {
+      load_k4(a_base, kb, a);
+    }
+    if constexpr (TB) {
+#pragma unroll
+      for (int c = 0; c < NT; c++) {
+        float col[4];
+        load_k4(B + (int64_t)ncol[c] * ldb, kb, col);
+#pragma unroll
+        for (int t = 0; t < 4; t++) b[t][c] = col[t];
+      }
     } else {
 #pragma unroll
-      for (int t = 0; t < 4; t++) a[t] = a_row[min(k0 + t, K - 1)];
-    }
+      for (int t = 0; t < 4; t++) {
+        const float* src = B + (int64_t)(kb + t) * ldb;
+        if constexpr (NT == 1) {
+          b[t][0] = src[ncol[0]];
+        } else {
+          const bvec v = *reinterpret_cast<const bvec*>(src + ncol[0]);
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
-      const float* src = b_col + (int64_t)min(k0 + t, K - 1) * ldb;
-      if constexpr (NT == 1) {
-        b[t][0] = *src;
-      } else {
-        const bvec v = *reinterpret_cast<const bvec*>(src);
-#pragma unroll
-        for (int c = 0; c < NT; c++) b[t][c] = v[c];
+          for (int c = 0; c < NT; c++) b[t][c] = v[c];
+        }
       }
     }
   };
@@ -714,13 +743,14 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny16(const float* __restri
 #pragma unroll
     for (int g = 0; g < G; g++)
       if (c + g * WV < nchunks) {
-        const int left = K - ((c + g * WV) * 16 + 4 * q);
+        const int k0 = (c + g * WV) * 16 + 4 * q;
+        const int first = k0 - min(k0, K - 4);   // elements below this index belong to the quad before
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-          const float av = t < left ? a[g][t] : 0.f;
+          const float av = t >= first ? a[g][t] : 0.f;
 #pragma unroll
           for (int cs = 0; cs < NT; cs++) {
-            const float bv = t < left ? b[g][t][cs] : 0.f;
+            const float bv = t >= first ? b[g][t][cs] : 0.f;
             acc[cs] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[cs], 0, 0, 0);
           }
         }
@@ -748,8 +778,10 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny16(const float* __restri
     float sum = part[e];
 #pragma unroll
     for (int w = 1; w < WV; w++) sum = sum + part[w * TILE + e];
-    if (bias) sum = sum + bias[n0 + e % BN];
-    C[(int64_t)(m0 + e / BN) * ldc + n0 + e % BN] = act_apply(sum, act, alpha);
+    const int col = n0 + e % BN;
+    if (col >= N) continue;
+    if (bias) sum = sum + bias[col];
+    C[(int64_t)(m0 + e / BN) * ldc + col] = act_apply(sum, act, alpha);
   }
 }
 
@@ -1910,41 +1942,52 @@ static const char* force_tile() { return getenv("GORGONIA_HIP_SKINNY_TILE"); }
 // shape belongs to the tiled kernel.
 static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   const int64_t batch = c.dim[6] <= 0 ? 1 : c.dim[6];
-  if (batch != 1 || (c.flags & (GH_FLAG_TRANS_A | GH_FLAG_TRANS_B))) return -1;
+  const bool ta = c.flags & GH_FLAG_TRANS_A, tb = c.flags & GH_FLAG_TRANS_B;
+  if (batch != 1 || (ta && tb)) return -1;
   const int M = (int)c.dim[0], N = (int)c.dim[1], K = (int)c.dim[2];
   const int64_t tiles = cdiv(M, 32) * cdiv(N, 32);
   if (tiles > ctx->cu_count || K < 32) return -1;
   if (getenv("GORGONIA_HIP_GEMM_PLAN")) return -1;  // a forced tile plan means the tiled kernel
   const int lda = (int)c.dim[3], ldb = (int)c.dim[4], ldc = (int)c.dim[5];
   const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
-  const bool vec_a = al16(c.ptr[0]) && lda % 4 == 0 && K % 16 == 0;
   constexpr int WV = 8;  // 512 threads leave each wavefront 256 registers for the grouped loads
-  const dim3 grid((N + 31) / 32, (M + 31) / 32);
   const int softmax = (c.flags & GH_FLAG_GEMM_SOFTMAX) ? 1 : 0;
   const float* A = (const float*)(uintptr_t)c.ptr[0];
   const float* B = (const float*)(uintptr_t)c.ptr[1];
   float* C = (float*)(uintptr_t)c.ptr[2];
   const float* bias = (c.flags & GH_FLAG_GEMM_BIAS) ? (const float*)(uintptr_t)c.ptr[3] : nullptr;
   // Few 32x32 tiles: 16-row tiles reach two to four times as many compute units.
-  // Shapes that may carry the softmax epilogue (N <= 32) stay on one kernel, so
-  // the fused and the separate softmax see the same product bits.
+  // Untransposed shapes that may carry the softmax epilogue (N <= 32) stay on
+  // one kernel, so the fused and the separate softmax see the same product bits;
+  // transposed views (the weight and input gradients of a dense layer) only
+  // have the 16-row kernel.
   const char* force = force_tile();
-  if (M >= 16 && N > 32 && tiles * 2 <= ctx->cu_count && !(force && !strcmp(force, "32"))) {
+  const bool transposed = ta || tb;
+  if (transposed && (M < 16 || softmax)) return -1;
+  if (transposed || (M >= 16 && N > 32 && tiles * 2 <= ctx->cu_count && !(force && !strcmp(force, "32")))) {
     // 16x32 tiles read whole 128-byte lines of B; when even those leave half the
     // chip without a tile, 16x16 (measured on MI355X, 8 wavefronts per block:
     // 128x625x1152 11.0 us on 32x32, 8.4 on 16x32, 9.8 on 16x16; 64x1000x4096
     // 33 / 21.8 / 19.5 us)
     const int64_t blocks_wide = cdiv(M, 16) * cdiv(N, 32);
-    const bool narrow = force ? !strcmp(force, "16x16") : blocks_wide * 2 <= ctx->cu_count;
+    const bool narrow = N < 32 || (force ? !strcmp(force, "16x16") : blocks_wide * 2 <= ctx->cu_count);
     auto launch16 = [&](auto kernel, int bn) {
       hipLaunchKernelGGL(kernel, dim3((N + bn - 1) / bn, (M + 15) / 16), dim3(WV * 64), 0, ctx->stream, A, B, C, M,
                          N, K, lda, ldb, ldc, act, c.f[0], bias);
     };
-    const bool vec = K % 4 == 0;
-    if (narrow) { if (vec) launch16(k_gemm_skinny16<WV, 1, true>, 16); else launch16(k_gemm_skinny16<WV, 1, false>, 16); }
-    else { if (vec) launch16(k_gemm_skinny16<WV, 2, true>, 32); else launch16(k_gemm_skinny16<WV, 2, false>, 32); }
+#define GH_SKINNY16(TA_, TB_)                                                               \
+  do {                                                                                      \
+    if (narrow) launch16(k_gemm_skinny16<WV, 1, TA_, TB_>, 16);                             \
+    else launch16(k_gemm_skinny16<WV, 2, TA_, TB_>, 32);                                    \
+  } while (0)
+    if (ta) GH_SKINNY16(true, false);
+    else if (tb) GH_SKINNY16(false, true);
+    else GH_SKINNY16(false, false);
+#undef GH_SKINNY16
     return gh_check_hip(ctx, hipGetLastError(), "skinny gemm launch");
   }
+  const bool vec_a = al16(c.ptr[0]) && lda % 4 == 0 && K % 16 == 0;
+  const dim3 grid((N + 31) / 32, (M + 31) / 32);
   const bool vec_b = N >= 32;   // whole column tiles (the last one moved left)
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, dim3(WV * 64), 0, ctx->stream, A, B, C, M, N, K, lda, ldb, ldc, act, c.f[0],
