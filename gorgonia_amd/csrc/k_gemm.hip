@@ -674,7 +674,7 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny16(const float* __restri
                                                            const float* __restrict__ B,
                                                            float* __restrict__ C, int M, int N, int K,
                                                            int lda, int ldb, int ldc, int act, float alpha,
-                                                           const float* __restrict__ bias) {
+                                                           const float* __restrict__ bias, int softmax) {
   constexpr int G = NT == 1 ? 5 : 4;
   constexpr int BN = 16 * NT, TILE = 16 * BN;
   typedef float bvec __attribute__((ext_vector_type(NT), aligned(4)));
@@ -774,6 +774,34 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny16(const float* __restri
 #pragma unroll
     for (int v = 0; v < 4; v++) part[wave * TILE + (4 * q + v) * BN + NT * i + c] = acc[c][v];
   __syncthreads();
+  if (NT == 1 && softmax) {
+    // Row softmax (N <= 16: the one column tile holds whole rows) with the
+    // arithmetic of the softmax kernel: max, exp(x - max) in float64 rounded
+    // once, the sum taken in column order, one rounded reciprocal.
+    __shared__ float sm_x[16 * 17], sm_e[16 * 17];
+    const int e = threadIdx.x, row = (e >> 4) & 15, col = e & 15;
+    if (e < TILE) {
+      float sum = part[e];
+#pragma unroll
+      for (int w = 1; w < WV; w++) sum = sum + part[w * TILE + e];
+      if (bias && col < N) sum = sum + bias[col];
+      sm_x[row * 17 + col] = act_apply(sum, act, alpha);
+    }
+    __syncthreads();
+    if (e < TILE) {
+      float mx = -INFINITY;
+      for (int j = 0; j < N; j++) mx = fmaxf(mx, sm_x[row * 17 + j]);
+      sm_e[row * 17 + col] = col < N ? (float)exp((double)(sm_x[row * 17 + col] - mx)) : 0.f;
+    }
+    __syncthreads();
+    if (e < TILE && col < N) {
+      float sum = 0.f;
+      for (int j = 0; j < N; j++) sum = sum + sm_e[row * 17 + j];
+      const float inv = 1.0f / sum;
+      C[(int64_t)(m0 + row) * ldc + col] = sm_e[row * 17 + col] * inv;
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < TILE; e += WV * 64) {
     float sum = part[e];
 #pragma unroll
@@ -1957,14 +1985,16 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   float* C = (float*)(uintptr_t)c.ptr[2];
   const float* bias = (c.flags & GH_FLAG_GEMM_BIAS) ? (const float*)(uintptr_t)c.ptr[3] : nullptr;
   // Few 32x32 tiles: 16-row tiles reach two to four times as many compute units.
-  // Untransposed shapes that may carry the softmax epilogue (N <= 32) stay on
-  // one kernel, so the fused and the separate softmax see the same product bits;
-  // transposed views (the weight and input gradients of a dense layer) only
-  // have the 16-row kernel.
+  // Which kernel takes a product depends on its shape only, never on the
+  // softmax flag, so the fused and the separate softmax see the same product
+  // bits: N <= 16 goes to the 16x16 tiles (softmax in their epilogue), 16 < N <=
+  // 32 stays on the 32x32 tile.  Transposed views (the weight and input
+  // gradients of a dense layer) only have the 16-row kernel.
   const char* force = force_tile();
   const bool transposed = ta || tb;
   if (transposed && (M < 16 || softmax)) return -1;
-  if (transposed || (M >= 16 && N > 32 && tiles * 2 <= ctx->cu_count && !(force && !strcmp(force, "32")))) {
+  const bool tiles16 = N <= 16 || (N > 32 && tiles * 2 <= ctx->cu_count);
+  if (transposed || (M >= 16 && tiles16 && !(force && !strcmp(force, "32")))) {
     // 16x32 tiles read whole 128-byte lines of B; when even those leave half the
     // chip without a tile, 16x16 (measured on MI355X, 8 wavefronts per block:
     // 128x625x1152 11.0 us on 32x32, 8.4 on 16x32, 9.8 on 16x16; 64x1000x4096
@@ -1973,7 +2003,7 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
     const bool narrow = N < 32 || (force ? !strcmp(force, "16x16") : blocks_wide * 2 <= ctx->cu_count);
     auto launch16 = [&](auto kernel, int bn) {
       hipLaunchKernelGGL(kernel, dim3((N + bn - 1) / bn, (M + 15) / 16), dim3(WV * 64), 0, ctx->stream, A, B, C, M,
-                         N, K, lda, ldb, ldc, act, c.f[0], bias);
+                         N, K, lda, ldb, ldc, act, c.f[0], bias, softmax);
     };
 #define GH_SKINNY16(TA_, TB_)                                                               \
   do {                                                                                      \
