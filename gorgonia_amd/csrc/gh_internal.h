@@ -42,6 +42,13 @@ int gh_launch_elem_unary(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_bcast_bin(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_relu(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_relu_bwd(gh_ctx* ctx, const gh_cmd& c);
+// float64 twins of the backward operators (k_bwd64.hip)
+int gh_launch_relu_bwd_f64(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_dropout_f64(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_dropout_bwd_f64(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_softmax_bwd_f64(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_maxpool2d_bwd_f64(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_solver_step_f64(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_leaky_relu(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_fill(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_has_nan_inf(gh_ctx* ctx, const gh_cmd& c);

@@ -9,6 +9,11 @@
 #include "gh_internal.h"
 
 static bool pos(int64_t v) { return v > 0; }
+static double dim_double(int64_t bits) {   // a float64 scalar carried in a dim slot
+  double v;
+  memcpy(&v, &bits, sizeof(v));
+  return v;
+}
 
 int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
   auto bad = [&](const char* m) { msg = m; return (int)GH_EINVAL; };
@@ -140,16 +145,19 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (!pos(c.dim[0]) || !pos(c.dim[1]) || !pos(c.dim[2])) return bad("bn: B,C,S must be positive");
       if (c.dim[1] > 65535) return bad("bn: more than 65535 channels");
       if (c.dim[0] * c.dim[2] < 2) return bad("bn: training statistics need at least two values per channel");
+      if (dt != GH_F32) return bad("bn training: float32 only");
       return GH_OK;
     case GH_OP_BN_BWD:
       for (int i = 0; i < 5; i++)
         if (!c.ptr[i]) return bad("null operand");
       if (!pos(c.dim[0]) || !pos(c.dim[1]) || !pos(c.dim[2])) return bad("bn: B,C,S must be positive");
       if (c.dim[1] > 65535) return bad("bn: more than 65535 channels");
+      if (dt != GH_F32) return bad("bn backward: float32 only");
       return GH_OK;
     case GH_OP_SOFTMAX_BWD:
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
       if (c.dim[0] < 0 || !pos(c.dim[1])) return bad("softmax: bad shape");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     case GH_OP_SOLVER_STEP:
       if (fn >= GH_SOLVER__COUNT) { msg = "unknown solver"; return GH_ENOFUNC; }
@@ -157,22 +165,26 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (fn >= GH_SOLVER_RMSPROP && !c.ptr[2]) return bad("solver cache is null");
       if (fn == GH_SOLVER_ADAM && !c.ptr[3]) return bad("Adam second-moment cache is null");
       if (c.dim[0] < 0) return bad("negative size");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     case GH_OP_RAND_UNIFORM:
       if (!c.ptr[0]) return bad("null operand");
       if (c.dim[0] < 0) return bad("negative size");
       if (c.ptr[1] & 7) return bad("rand: state must be 8-byte aligned");
+      if (dt != GH_F32) return bad("rand: float32 only");
       return GH_OK;
     case GH_OP_RELU_BWD:
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
       if (c.dim[0] < 0) return bad("negative size");
-      if (dt != GH_F32) return bad("relu backward: float32 only");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     case GH_OP_DROPOUT:
     case GH_OP_DROPOUT_BWD:
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
       if (c.dim[0] < 0) return bad("negative size");
-      if (!(c.f[0] >= 0.0f && c.f[0] < 1.0f)) return bad("dropout: probability must be in [0, 1)");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
+      if (dt == GH_F64 ? !(dim_double(c.dim[1]) >= 0.0 && dim_double(c.dim[1]) < 1.0) : !(c.f[0] >= 0.0f && c.f[0] < 1.0f))
+        return bad("dropout: probability must be in [0, 1)");
       return GH_OK;
     case GH_OP_RELU:
     case GH_OP_LEAKY_RELU:

@@ -464,6 +464,7 @@ int bn_groups(int64_t n, int64_t S) {
 }  // namespace
 
 int gh_launch_maxpool2d_bwd(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_maxpool2d_bwd_f64(ctx, c);
   const int64_t B = c.dim[0], C = c.dim[1];
   PoolGeom g;
   g.H = (int)c.dim[2]; g.W = (int)c.dim[3]; g.kh = (int)c.dim[4]; g.kw = (int)c.dim[5];
@@ -547,6 +548,7 @@ int gh_launch_bn_bwd(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_softmax_bwd(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_softmax_bwd_f64(ctx, c);
   const int64_t rows = c.dim[0];
   const int cols = (int)c.dim[1];
   if (rows == 0) return GH_OK;
@@ -561,6 +563,7 @@ int gh_launch_softmax_bwd(gh_ctx* ctx, const gh_cmd& c) {
 // SOLVER_STEP commands with the same solver, options and hyper-parameters.
 int gh_solver_run_length(const gh_cmd* cmds, int n) {
   if (n <= 0 || cmds[0].opcode != GH_OP_SOLVER_STEP) return 0;
+  if (gh_dtype_of(cmds[0].flags) == GH_F64) return 1;   // float64 steps go one tensor per launch
   int len = 1;
   while (len < n && len < kSolverBatch && cmds[len].opcode == GH_OP_SOLVER_STEP && cmds[len].flags == cmds[0].flags &&
          memcmp(cmds[len].f, cmds[0].f, sizeof(cmds[0].f)) == 0) {
@@ -607,7 +610,10 @@ int gh_launch_solver_steps(gh_ctx* ctx, const gh_cmd* cmds, int count) {
   return gh_check_hip(ctx, hipGetLastError(), "solver step launch");
 }
 
-int gh_launch_solver_step(gh_ctx* ctx, const gh_cmd& c) { return gh_launch_solver_steps(ctx, &c, 1); }
+int gh_launch_solver_step(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_solver_step_f64(ctx, c);
+  return gh_launch_solver_steps(ctx, &c, 1);
+}
 
 static int stream_blocks(gh_ctx* ctx, int64_t n) {
   int64_t blocks = (n + kBlock - 1) / kBlock;
@@ -626,6 +632,7 @@ int gh_launch_rand_uniform(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_dropout(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_dropout_f64(ctx, c);
   const int64_t n = c.dim[0];
   if (n == 0) return GH_OK;
   const int identity = (c.flags & GH_FLAG_BN_EVAL) || c.f[0] == 0.0f;
@@ -637,6 +644,7 @@ int gh_launch_dropout(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_dropout_bwd(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_dropout_bwd_f64(ctx, c);
   const int64_t n = c.dim[0];
   if (n == 0) return GH_OK;
   hipLaunchKernelGGL(k_dropout_bwd, dim3(stream_blocks(ctx, n)), dim3(kBlock), 0, ctx->stream,

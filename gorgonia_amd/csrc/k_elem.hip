@@ -693,6 +693,7 @@ int gh_launch_relu(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_relu_bwd(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_relu_bwd_f64(ctx, c);
   const int64_t n = c.dim[0];
   if (n == 0) return GH_OK;
   const int vec = aligned16(c.ptr[0]) && aligned16(c.ptr[1]) && aligned16(c.ptr[2]) && n >= 4;

@@ -235,8 +235,8 @@ def cmd_softmax(x, y, rows, cols, dtype=_ffi.F32):
     return make_cmd(_ffi.OP_SOFTMAX, _ffi.flag_dtype(dtype), (x, y), (rows, cols))
 
 
-def cmd_maxpool2d_bwd(x, dy, dx, B, Cn, H, W, kh, kw, pad, stride):
-    c = cmd_maxpool2d(x, dy, B, Cn, H, W, kh, kw, pad, stride)
+def cmd_maxpool2d_bwd(x, dy, dx, B, Cn, H, W, kh, kw, pad, stride, dtype=_ffi.F32):
+    c = cmd_maxpool2d(x, dy, B, Cn, H, W, kh, kw, pad, stride, dtype=dtype)
     c.opcode = _ffi.OP_MAXPOOL2D_BWD
     c.ptr[2] = int(dx)
     return c
@@ -264,16 +264,19 @@ def cmd_bn_bwd(x, dy, dx, save_mean, save_var, B, Cn, S, eps, training=True):
                     (B, Cn, S), (eps,))
 
 
-def cmd_softmax_bwd(y, dy, dx, rows, cols):
-    return make_cmd(_ffi.OP_SOFTMAX_BWD, 0, (y, dy, dx), (rows, cols))
+def cmd_softmax_bwd(y, dy, dx, rows, cols, dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_SOFTMAX_BWD, _ffi.flag_dtype(dtype), (y, dy, dx), (rows, cols))
 
 
 SOLVER = {"vanilla": 0, "rmsprop": 1, "adam": 2}
 
 
-def cmd_solver_step(kind, w, g, n, par, use, cache=0, cache2=0):
-    """par: the ten float32 constants of gorgonia_hip.h's SOLVER_STEP row; use: option mask."""
-    fl = _ffi.flag_fn(SOLVER[kind]) | _ffi.flag_mode(use)
+def cmd_solver_step(kind, w, g, n, par, use, cache=0, cache2=0, dtype=_ffi.F32):
+    """par: the ten constants of gorgonia_hip.h's SOLVER_STEP row (float32 in f[], or for float64
+    tensors as double bit patterns in dim[1..10]); use: option mask."""
+    fl = _ffi.flag_fn(SOLVER[kind]) | _ffi.flag_mode(use) | _ffi.flag_dtype(dtype)
+    if dtype == _ffi.F64:
+        return make_cmd(_ffi.OP_SOLVER_STEP, fl, (w, g, cache, cache2), (n,) + tuple(_double_bits(v) for v in par))
     return make_cmd(_ffi.OP_SOLVER_STEP, fl, (w, g, cache, cache2), (n,), tuple(float(v) for v in par))
 
 
@@ -281,16 +284,17 @@ def cmd_rand_uniform(out, n, seed, offset=0, state=0):
     return make_cmd(_ffi.OP_RAND_UNIFORM, 0, (out, state), (n, seed, offset))
 
 
-def cmd_dropout(x, y, r, n, prob, training=True):
-    return make_cmd(_ffi.OP_DROPOUT, 0 if training else _ffi.FLAG_BN_EVAL, (x, y, r), (n,), (prob,))
+def cmd_dropout(x, y, r, n, prob, training=True, dtype=_ffi.F32):
+    fl = (0 if training else _ffi.FLAG_BN_EVAL) | _ffi.flag_dtype(dtype)
+    return make_cmd(_ffi.OP_DROPOUT, fl, (x, y, r), (n, _double_bits(prob)), (prob,))
 
 
-def cmd_dropout_bwd(y, dy, dx, n, prob):
-    return make_cmd(_ffi.OP_DROPOUT_BWD, 0, (y, dy, dx), (n,), (prob,))
+def cmd_dropout_bwd(y, dy, dx, n, prob, dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_DROPOUT_BWD, _ffi.flag_dtype(dtype), (y, dy, dx), (n, _double_bits(prob)), (prob,))
 
 
-def cmd_relu_bwd(x, dy, dx, n):
-    return make_cmd(_ffi.OP_RELU_BWD, 0, (x, dy, dx), (n,))
+def cmd_relu_bwd(x, dy, dx, n, dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_RELU_BWD, _ffi.flag_dtype(dtype), (x, dy, dx), (n,))
 
 
 def cmd_has(kind, a, flag, n, dtype=_ffi.F32):

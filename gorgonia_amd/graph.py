@@ -78,7 +78,9 @@ def NewTensor(g, value, resident=False):
     dt = {np.dtype(np.float32): 0, np.dtype(np.float64): 1}.get(value.dtype, 2)
     nid = g.lib.ghh_graph_new_tensor(g.h, shp, value.ndim, dt, value.ctypes.data_as(C.c_void_p),
                                      int(resident))
-    return Node(g, nid)
+    node = Node(g, nid)
+    node.dtype = value.dtype
+    return node
 
 
 def NewScalar(g, value, dtype=np.float32, resident=True):
@@ -225,9 +227,10 @@ def SolverStep(kind, weights, grad, caches=(), eta=0.001, eps=1e-8, l1reg=0.0, l
     """One Step of NewVanillaSolver / NewRMSPropSolver / NewAdamSolver (solvers.go) on one
     weight tensor, on the device: the weights (a resident input) and the solver's caches
     (resident inputs, zero at the start) are updated in place.  The constants are
-    rounded to float32 the way the reference rounds them; Adam's bias corrections
-    depend on `iteration`, so an Adam step is a new command every run."""
-    f = np.float32
+    rounded to the weights' type the way the reference rounds them (float64 weights keep
+    them in double); Adam's bias corrections depend on `iteration`, so an Adam step is a
+    new command every run."""
+    f = np.float64 if getattr(weights, "dtype", None) == np.float64 else np.float32
     a, b = (f(decay), f(1.0 - decay)) if kind == "rmsprop" else (f(beta1), f(beta2))
     fs = [f(eta), f(eps), f(l1reg), f(l2reg), f(clip), f(1) / f(batch), a, b,
           f(1) / f(1 - beta1 ** iteration), f(1) / f(1 - beta2 ** iteration)]

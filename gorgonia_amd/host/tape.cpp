@@ -441,9 +441,10 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       const Tensor& x = *in[0];
       const auto& p = op.ints;
       const int64_t np = p[2];
+      if (x.dt == Dtype::Other || in[1]->dt != x.dt) return bad("MaxPool2DDiff: Unsupported Dtype");
       gh_cmd c{};
       c.opcode = GH_OP_MAXPOOL2D_BWD;
-      c.flags = np == 4 ? GH_FLAG_EXPLICIT_PAD : 0;
+      c.flags = (np == 4 ? GH_FLAG_EXPLICIT_PAD : 0) | dtype_flag(x.dt);
       c.ptr[0] = x.mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
       for (int i = 0; i < 4; i++) c.dim[i] = x.shape[i];
       c.dim[4] = p[0]; c.dim[5] = p[1];
@@ -456,6 +457,7 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     case OpKind::Conv2dDiffData:
     case OpKind::Conv2dDiffFilter: {
       const bool data = op.kind == OpKind::Conv2dDiffData;
+      if (in[0]->dt != Dtype::Float32 || in[1]->dt != Dtype::Float32) return bad("Conv2d gradients: float32 only");
       gh_cmd c{};
       c.opcode = data ? GH_OP_CONV2D_BWD_DATA : GH_OP_CONV2D_BWD_FILTER;
       c.ptr[0] = in[0]->mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
@@ -489,8 +491,10 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     }
     case OpKind::SoftMaxDiff: {
       const Tensor& y = *in[0];
+      if (y.dt == Dtype::Other || in[1]->dt != y.dt) return bad("SoftMaxDiff: Unsupported Dtype");
       gh_cmd c{};
       c.opcode = GH_OP_SOFTMAX_BWD;
+      c.flags = dtype_flag(y.dt);
       c.ptr[0] = y.mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
       const int64_t cols = y.shape[y.shape.Dims() - 1];
       c.dim[0] = y.shape.TotalSize() / cols; c.dim[1] = cols;
@@ -500,10 +504,14 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     case OpKind::SolverStep: {
       gh_cmd c{};
       c.opcode = GH_OP_SOLVER_STEP;
-      c.flags = GH_FLAG_FN(op.fn) | GH_FLAG_MODE(op.ints[0]);
+      for (size_t i = 0; i < in.size(); i++)
+        if (in[i]->dt == Dtype::Other || in[i]->dt != in[0]->dt) return bad("SolverStep: Unsupported Dtype");
+      c.flags = GH_FLAG_FN(op.fn) | GH_FLAG_MODE(op.ints[0]) | dtype_flag(in[0]->dt);
       for (size_t i = 0; i < in.size(); i++) c.ptr[i] = in[i]->mem;
       c.dim[0] = in[0]->DataSize();
       for (int i = 0; i < 10; i++) c.f[i] = (float)op.fs[(size_t)i];
+      if (in[0]->dt == Dtype::Float64)   // float64 tensors take the constants as doubles
+        for (int i = 0; i < 10; i++) c.dim[1 + i] = double_bits(op.fs[(size_t)i]);
       e.Enqueue(c);
       return Status::OK();
     }
@@ -518,9 +526,10 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       return Status::OK();
     }
     case OpKind::RectifyDiff: {
-      if (in[0]->dt != Dtype::Float32 || in[1]->dt != Dtype::Float32) return bad("RectifyDiff: Unsupported Dtype");
+      if (in[0]->dt == Dtype::Other || in[1]->dt != in[0]->dt) return bad("RectifyDiff: Unsupported Dtype");
       gh_cmd c{};
       c.opcode = GH_OP_RELU_BWD;
+      c.flags = dtype_flag(in[0]->dt);
       c.ptr[0] = in[0]->mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
       c.dim[0] = in[0]->shape.TotalSize();
       e.Enqueue(c);
@@ -528,11 +537,13 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     }
     case OpKind::Dropout:
     case OpKind::DropoutDiff: {
-      if (in[0]->dt != Dtype::Float32 || in[1]->dt != Dtype::Float32) return bad("Dropout: Unsupported Dtype");
+      if (in[0]->dt == Dtype::Other || in[1]->dt != in[0]->dt) return bad("Dropout: Unsupported Dtype");
       gh_cmd c{};
       c.opcode = op.kind == OpKind::Dropout ? GH_OP_DROPOUT : GH_OP_DROPOUT_BWD;
+      c.flags = dtype_flag(in[0]->dt);
+      c.dim[1] = double_bits(op.f0);
       if (op.kind == OpKind::Dropout) {
-        if (!op.fn) c.flags = GH_FLAG_BN_EVAL;
+        if (!op.fn) c.flags |= GH_FLAG_BN_EVAL;
         c.ptr[0] = in[0]->mem; c.ptr[1] = prealloc.mem; c.ptr[2] = in[1]->mem;
       } else {
         c.ptr[0] = in[0]->mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;

@@ -186,9 +186,12 @@ enum gh_unaryfn {
  * BN_BWD      ptr[0]=x ptr[1]=dy ptr[2]=dx ptr[3]=save_mean ptr[4]=save_var
  *             dim[0..2]=B,C,S  f[0]=eps ; BN_EVAL selects dx = dy/sqrt(save_var/n + eps)
  * SOFTMAX_BWD ptr[0]=y ptr[1]=dy ptr[2]=dx        dim[0]=rows dim[1]=cols
- * float64: CONV2D (no epilogue flags), MAXPOOL2D, BN_INFER, RELU, LEAKY_RELU and SOFTMAX take
+ * float64: CONV2D (no epilogue flags), MAXPOOL2D, BN_INFER, RELU, LEAKY_RELU, SOFTMAX,
+ *             MAXPOOL2D_BWD, SOFTMAX_BWD, RELU_BWD, DROPOUT, DROPOUT_BWD and SOLVER_STEP take
  *             GH_FLAG_DTYPE(GH_F64); their scalars then travel as the bit pattern of a double
- *             in a dim slot (LEAKY_RELU alpha: dim[1]; BN_INFER epsilon: dim[3])
+ *             in a dim slot (LEAKY_RELU alpha: dim[1]; BN_INFER epsilon: dim[3]; DROPOUT and
+ *             DROPOUT_BWD probability: dim[1]; SOLVER_STEP's ten constants: dim[1..10]).
+ *             CONV2D_BWD_*, BN_TRAIN, BN_BWD and RAND_UNIFORM are float32 only
  * RAND_UNIFORM ptr[0]=out [ptr[1]=state]          dim[0]=n dim[1]=seed dim[2]=offset
  *             float32 in [0,1) with 24 random bits, element i = SplitMix64 output function
  *             of seed*0xD1342543DE82EF95 + (offset + i + 1)*0x9E3779B97F4A7C15.  With a
@@ -197,9 +200,9 @@ enum gh_unaryfn {
  * DROPOUT     ptr[0]=x ptr[1]=y ptr[2]=r (uniform numbers, one per element)  dim[0]=n
  *             f[0]=drop probability ; y = r < 1-p ? x/(1-p) : 0 ; BN_EVAL or p == 0: y = x
  * DROPOUT_BWD ptr[0]=y ptr[1]=dy ptr[2]=dx         dim[0]=n f[0]=drop probability
+ *             dx = (p != 0 && y != 0) ? dy/p : 0   (the reference divides by p)
  * RELU_BWD    ptr[0]=x ptr[1]=dy ptr[2]=dx         dim[0]=n ; dx = dy * (x >= 0 ? 1 : 0), the bits of
  *             Gte(x, 0) followed by HadamardProd; dx may be dy (in place)
- *             dx = (p != 0 && y != 0) ? dy/p : 0   (the reference divides by p)
  * SOLVER_STEP ptr[0]=weights ptr[1]=grad [ptr[2]=cache (RMSProp cache / Adam m) ptr[3]=Adam v]
  *             dim[0]=n ; flags: FN = gh_solver, MODE = use mask (1 l1reg, 2 l2reg, 4 clip,
  *             8 batch) ; f[0]=eta f[1]=eps f[2]=l1reg f[3]=l2reg f[4]=clip f[5]=1/batch

@@ -254,13 +254,14 @@ def softmax(x):
 
 
 def maxpool2d_bwd(x, dy, kernel, pad, stride):
-    x = np.ascontiguousarray(x, dtype=np.float32)
-    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    x = np.ascontiguousarray(x, dtype=_ft(x))
+    dy = np.ascontiguousarray(dy, dtype=x.dtype)
     B, Cn, H, W = x.shape
     p4, explicit = _pad4(pad)
     dx = np.empty_like(x)
-    lib().oracle_maxpool2d_bwd_f32(_p(x), _p(dy), _p(dx), *_i64(B, Cn, H, W, kernel[0], kernel[1]), _p(p4),
-                                   C.c_int(explicit), *_i64(stride[0], stride[1]))
+    f = lib().oracle_maxpool2d_bwd_f64 if x.dtype == np.float64 else lib().oracle_maxpool2d_bwd_f32
+    f(_p(x), _p(dy), _p(dx), *_i64(B, Cn, H, W, kernel[0], kernel[1]), _p(p4), C.c_int(explicit),
+      *_i64(stride[0], stride[1]))
     return dx
 
 
@@ -321,11 +322,12 @@ def bn_bwd(x, dy, save_mean, save_var, eps, training=True):
 
 
 def softmax_bwd(y, dy):
-    y = np.ascontiguousarray(y, dtype=np.float32)
-    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    y = np.ascontiguousarray(y, dtype=_ft(y))
+    dy = np.ascontiguousarray(dy, dtype=y.dtype)
     rows, cols = int(np.prod(y.shape[:-1])), y.shape[-1]
     dx = np.empty_like(y)
-    lib().oracle_softmax_bwd_f32(_p(y), _p(dy), _p(dx), *_i64(rows, cols))
+    (lib().oracle_softmax_bwd_f64 if y.dtype == np.float64 else lib().oracle_softmax_bwd_f32)(
+        _p(y), _p(dy), _p(dx), *_i64(rows, cols))
     return dx
 
 
@@ -333,46 +335,50 @@ SOLVER = {"vanilla": 0, "rmsprop": 1, "adam": 2}
 
 
 def solver_params(eta, eps=1e-8, l1reg=0.0, l2reg=0.0, clip=0.0, batch=1.0, decay=0.999, beta1=0.9, beta2=0.999,
-                  kind="vanilla", iteration=1):
-    """The float32 constants a solver step uses, computed the way the reference does
-    (float64 first, then one cast; solvers.go:307-314, 492-525, 793-806), and its use mask."""
-    f = np.float32
+                  kind="vanilla", iteration=1, dtype=np.float32):
+    """The constants a solver step uses in the tensors' type, computed the way the reference does
+    (float64 first, then one cast for float32 tensors; solvers.go:307-314, 492-525, 793-806), and
+    its use mask."""
+    f = np.dtype(dtype).type
     if kind == "rmsprop":
         a, b = f(decay), f(1.0 - decay)
     else:
         a, b = f(beta1), f(beta2)
     c1 = f(1) / f(1 - beta1 ** iteration)
     c2 = f(1) / f(1 - beta2 ** iteration)
-    par = np.array([f(eta), f(eps), f(l1reg), f(l2reg), f(clip), f(1) / f(batch), a, b, c1, c2], dtype=np.float32)
+    par = np.array([f(eta), f(eps), f(l1reg), f(l2reg), f(clip), f(1) / f(batch), a, b, c1, c2], dtype=dtype)
     use = (1 if l1reg else 0) | (2 if l2reg else 0) | (4 if clip else 0) | (8 if batch > 1 else 0)
     return par, use
 
 
 def solver_step(kind, w, g, c1=None, c2=None, **kw):
-    """One solver step in place on copies; returns (w, g, c1, c2)."""
-    par, use = solver_params(kind=kind, **kw)
-    w = np.array(w, dtype=np.float32, copy=True)
-    g = np.array(g, dtype=np.float32, copy=True)
-    c1 = np.zeros_like(w) if c1 is None else np.array(c1, dtype=np.float32, copy=True)
-    c2 = np.zeros_like(w) if c2 is None else np.array(c2, dtype=np.float32, copy=True)
-    lib().oracle_solver_step_f32(C.c_int(SOLVER[kind]), _p(w), _p(g), _p(c1), _p(c2), C.c_int64(w.size),
-                                 C.c_int(use), _p(par))
+    """One solver step in place on copies, in w's type (float32 or float64); returns (w, g, c1, c2)."""
+    dt = _ft(np.asarray(w))
+    par, use = solver_params(kind=kind, dtype=dt, **kw)
+    w = np.array(w, dtype=dt, copy=True)
+    g = np.array(g, dtype=dt, copy=True)
+    c1 = np.zeros_like(w) if c1 is None else np.array(c1, dtype=dt, copy=True)
+    c2 = np.zeros_like(w) if c2 is None else np.array(c2, dtype=dt, copy=True)
+    (lib().oracle_solver_step_f64 if dt == np.float64 else lib().oracle_solver_step_f32)(
+        C.c_int(SOLVER[kind]), _p(w), _p(g), _p(c1), _p(c2), C.c_int64(w.size), C.c_int(use), _p(par))
     return w, g, c1, c2
 
 
 def dropout(x, r, prob, training=True):
-    x = np.ascontiguousarray(x, dtype=np.float32)
-    r = np.ascontiguousarray(r, dtype=np.float32)
+    x = np.ascontiguousarray(x, dtype=_ft(x))
+    r = np.ascontiguousarray(r, dtype=x.dtype)
     y = np.empty_like(x)
-    lib().oracle_dropout_f32(_p(x), _p(r), _p(y), C.c_int64(x.size), C.c_double(prob), C.c_int(int(training)))
+    (lib().oracle_dropout_f64 if x.dtype == np.float64 else lib().oracle_dropout_f32)(
+        _p(x), _p(r), _p(y), C.c_int64(x.size), C.c_double(prob), C.c_int(int(training)))
     return y
 
 
 def dropout_bwd(y, dy, prob):
-    y = np.ascontiguousarray(y, dtype=np.float32)
-    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    y = np.ascontiguousarray(y, dtype=_ft(y))
+    dy = np.ascontiguousarray(dy, dtype=y.dtype)
     dx = np.empty_like(y)
-    lib().oracle_dropout_bwd_f32(_p(y), _p(dy), _p(dx), C.c_int64(y.size), C.c_double(prob))
+    (lib().oracle_dropout_bwd_f64 if y.dtype == np.float64 else lib().oracle_dropout_bwd_f32)(
+        _p(y), _p(dy), _p(dx), C.c_int64(y.size), C.c_double(prob))
     return dx
 
 

@@ -55,6 +55,12 @@
  *                                            forward pass.  tensor.SoftMaxB
  *                                            itself is not vendored: PARITY
  *                                            UNPINNED bit-for-bit.
+ *   float64 twins (forward NN operators,   - each against its pinned float32
+ *   max-pool / softmax backward, dropout,    counterpart: equal on inputs whose
+ *   solver steps)                            float32 arithmetic is exact, within
+ *                                            float32 rounding elsewhere; the
+ *                                            reference's float64 goldens where it
+ *                                            has them (max pool, softmax)
  */
 #include <math.h>
 #include <stdint.h>
@@ -1107,6 +1113,130 @@ EXPORT void oracle_bn_infer_f64(const double* x, double* y, const double* run_me
       out[d] = t;
     }
   }
+}
+
+/* ================================================================== */
+/* float64 twins of the backward operators, dropout and the solver     */
+/* steps: the reference's Float64 branches (maxPoolDiffOp.f64s         */
+/* op_nn.go:1095-1120, softmaxDiffOp op_softmax.go:266-279, dropout    */
+/* op_dropout.go:118-132,215-238, the Float64 cases of the solvers'    */
+/* Step solvers.go:299,496,793) - the float32 restatements above with  */
+/* every operation in double.                                          */
+/* ================================================================== */
+EXPORT void oracle_maxpool2d_bwd_f64(const double* x, const double* dy, double* dx, int64_t B,
+                                     int64_t C, int64_t H, int64_t W, int64_t kh, int64_t kw,
+                                     const int64_t* pad4, int explicit_padding, int64_t strideH,
+                                     int64_t strideW) {
+  int64_t oh, ow, bc;
+  oracle_maxpool_out_hw(H, W, kh, kw, pad4, strideH, strideW, &oh, &ow);
+  int64_t padH = explicit_padding ? pad4[1] : pad4[0];
+  int64_t padW = explicit_padding ? pad4[3] : pad4[2];
+  for (bc = 0; bc < B * C; bc++) {
+    const double* in = x + bc * H * W;
+    const double* g = dy + bc * oh * ow;
+    double* out = dx + bc * H * W;
+    int64_t ph, pw, hi, wi, i;
+    for (i = 0; i < H * W; i++) out[i] = 0.0;
+    for (ph = 0; ph < oh; ph++)
+      for (pw = 0; pw < ow; pw++) {
+        int64_t hs = ph * strideH - padH, ws = pw * strideW - padW;
+        int64_t he = hs + kh < H ? hs + kh : H;
+        int64_t we = ws + kw < W ? ws + kw : W;
+        if (hs < 0) hs = 0;
+        if (ws < 0) ws = 0;
+        double best = -DBL_MAX;
+        int64_t arg = -1;
+        for (hi = hs; hi < he; hi++)
+          for (wi = ws; wi < we; wi++)
+            if (in[hi * W + wi] > best) { best = in[hi * W + wi]; arg = hi * W + wi; }
+        if (arg >= 0) out[arg] = out[arg] + g[ph * ow + pw];
+      }
+  }
+}
+
+EXPORT void oracle_softmax_bwd_f64(const double* y, const double* dy, double* dx, int64_t rows,
+                                   int64_t cols) {
+  int64_t r, j;
+  for (r = 0; r < rows; r++) {
+    const double* yy = y + r * cols;
+    const double* g = dy + r * cols;
+    double dot = 0.0;
+    for (j = 0; j < cols; j++) { double t = g[j] * yy[j]; dot = dot + t; }
+    for (j = 0; j < cols; j++) { double t = g[j] - dot; dx[r * cols + j] = yy[j] * t; }
+  }
+}
+
+static double clampd(double v, double lo, double hi) { return v < lo ? lo : (v > hi ? hi : v); }
+static double signd(double v) { return v > 0.0 ? 1.0 : (v < 0.0 ? -1.0 : 0.0); }
+
+static double prep_grad_f64(double g, double w, int use, const double* par) {
+  if (use & 1) { double t = par[2] * signd(w); g = g + t; }
+  if (use & 2) { double t = w * par[3]; g = g + t; }
+  if (use & 8) g = g * par[5];
+  if ((use & 4) && par[4] > 0.0) g = clampd(g, -par[4], par[4]);
+  return g;
+}
+
+EXPORT void oracle_solver_step_f64(int kind, double* w, double* g, double* c1, double* c2, int64_t n,
+                                   int use, const double* par) {
+  int64_t i;
+  const double neg_eta = -par[0];
+  for (i = 0; i < n; i++) {
+    if (kind == 0) {            /* vanilla */
+      double gi = prep_grad_f64(g[i], w[i], use, par);
+      gi = gi * neg_eta;
+      w[i] = w[i] + gi;
+      g[i] = gi;
+    } else if (kind == 1) {     /* RMSProp */
+      double gi = g[i];
+      double gt2 = gi * gi;
+      double cw = c1[i] * par[6];
+      gt2 = gt2 * par[7];
+      cw = cw + gt2;
+      c1[i] = cw;
+      if (use & 4) gi = clampd(gi, -par[4], par[4]);
+      double upd = cw + par[1];
+      upd = 1.0 / sqrt(upd);
+      gi = gi * neg_eta;
+      upd = upd * gi;
+      if (use & 2) { double reg = w[i] * par[3]; upd = upd - reg; }
+      w[i] = w[i] + upd;
+      g[i] = gi;
+    } else {                    /* Adam */
+      double gi = prep_grad_f64(g[i], w[i], use, par);
+      double omb1 = 1.0 - par[6], omb2 = 1.0 - par[7];
+      double t1 = gi * omb1;
+      double g2 = gi * gi;
+      g2 = g2 * omb2;
+      double mb = c1[i] * par[6];
+      t1 = t1 + mb;
+      double vb = c2[i] * par[7];
+      g2 = g2 + vb;
+      c1[i] = t1;
+      c2[i] = g2;
+      double mh = t1 * par[8];
+      double vh = g2 * par[9];
+      vh = sqrt(vh);
+      vh = vh + par[1];
+      mh = mh * neg_eta;
+      mh = mh / vh;
+      w[i] = w[i] + mh;
+      g[i] = g2;
+    }
+  }
+}
+
+EXPORT void oracle_dropout_f64(const double* x, const double* r, double* y, int64_t n, double prob,
+                               int training) {
+  int64_t i;
+  if (prob == 0.0 || !training) { for (i = 0; i < n; i++) y[i] = x[i]; return; }
+  const double keep = 1.0 - prob;
+  for (i = 0; i < n; i++) y[i] = r[i] < keep ? x[i] / keep : 0.0;
+}
+
+EXPORT void oracle_dropout_bwd_f64(const double* y, const double* dy, double* dx, int64_t n, double prob) {
+  int64_t i;
+  for (i = 0; i < n; i++) dx[i] = (prob != 0.0 && y[i] != 0.0) ? dy[i] / prob : 0.0;
 }
 
 EXPORT int oracle_has_nan_f32(const float* a, int64_t n) {

@@ -1,0 +1,164 @@
+"""GPU parity of the float64 backward operators, dropout and solver steps (max-pool, softmax
+and activation gradients, dropout forward/backward, Vanilla / RMSProp / Adam steps) through
+the C ABI against the CPU oracle's float64 twins.  Bar: bit-exact (same operation order, one
+IEEE rounding per step; division and square root are correctly rounded on both sides)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from gorgonia_amd import _ffi
+from gorgonia_amd import device as D
+from oracle import binding as O
+from tests.util import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+F64 = _ffi.F64
+
+
+def _rand(seed, shape, scale=1.0):
+    return np.random.default_rng(seed).standard_normal(shape) * scale
+
+
+def _up(ctx, a):
+    return ctx.upload(np.ascontiguousarray(a, dtype=np.float64))
+
+
+@pytest.mark.parametrize("kernel,pad,stride,shape", [
+    ((2, 2), (0, 0), (2, 2), (3, 4, 14, 14)),
+    ((2, 2), (0, 0), (2, 2), (2, 3, 7, 7)),
+    ((3, 3), (1, 1), (2, 2), (2, 2, 9, 11)),
+    ((2, 2), (1, 0, 1, 0), (1, 1), (1, 3, 13, 13)),
+    ((3, 2), (1, 1), (1, 1), (2, 2, 6, 5)),
+])
+def test_maxpool_backward_float64(ctx, kernel, pad, stride, shape):
+    x = _rand(1, shape)
+    x[0, 0, :2, :2] = 0.5   # a tie: the first element of the window wins
+    oh, ow = O.maxpool2d(x, kernel, pad, stride).shape[2:]
+    dy = _rand(2, shape[:2] + (oh, ow))
+    want = O.maxpool2d_bwd(x, dy, kernel, pad, stride)
+    px, pdy, pdx = _up(ctx, x), _up(ctx, dy), ctx.malloc(x.size * 8)
+    ctx.run(D.cmd_maxpool2d_bwd(px, pdy, pdx, *shape, kernel[0], kernel[1], pad, stride, dtype=F64))
+    assert_bits_equal(ctx.d2h(pdx, shape, np.float64), want, "max-pool backward float64")
+    for p in (px, pdy, pdx):
+        ctx.free(p)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (128, 10), (37, 129), (1000, 3)])
+def test_softmax_backward_float64(ctx, rows, cols):
+    y = O.softmax(_rand(3, (rows, cols)))
+    dy = _rand(4, (rows, cols))
+    want = O.softmax_bwd(y, dy)
+    py, pdy, pdx = _up(ctx, y), _up(ctx, dy), ctx.malloc(rows * cols * 8)
+    ctx.run(D.cmd_softmax_bwd(py, pdy, pdx, rows, cols, dtype=F64))
+    assert_bits_equal(ctx.d2h(pdx, (rows, cols), np.float64), want, "softmax backward float64")
+    for p in (py, pdy, pdx):
+        ctx.free(p)
+
+
+@pytest.mark.parametrize("n", [1, 5, 1000, 70001])
+def test_relu_backward_and_dropout_float64(ctx, n):
+    x = _rand(5, (n,))
+    dy = _rand(6, (n,))
+    special = np.array([0.0, -0.0, np.nan, np.inf, -np.inf], np.float64)
+    k = min(n, special.size)
+    x[:k] = special[:k]
+    mask = O.binop("gte", "vs", x, np.zeros(1))
+    want = O.binop("mul", "vv", dy, mask)
+    px, pdy, pdx = _up(ctx, x), _up(ctx, dy), ctx.malloc(n * 8)
+    ctx.run(D.cmd_relu_bwd(px, pdy, pdx, n, dtype=F64))
+    assert_bits_equal(ctx.d2h(pdx, (n,), np.float64), want, "relu backward float64")
+    # dropout forward (training and not) and backward
+    r = np.random.default_rng(7).random(n)
+    pr, py = _up(ctx, r), ctx.malloc(n * 8)
+    for prob in (0.3, 0.0):
+        ctx.run(D.cmd_dropout(px, py, pr, n, prob, dtype=F64))
+        y = ctx.d2h(py, (n,), np.float64)
+        assert_bits_equal(y, O.dropout(x, r, prob), f"dropout float64 p={prob}")
+        ctx.run(D.cmd_dropout_bwd(py, pdy, pdx, n, prob, dtype=F64))
+        assert_bits_equal(ctx.d2h(pdx, (n,), np.float64), O.dropout_bwd(y, dy, prob), f"dropout backward float64 p={prob}")
+    ctx.run(D.cmd_dropout(px, py, pr, n, 0.3, training=False, dtype=F64))
+    assert_bits_equal(ctx.d2h(py, (n,), np.float64), x, "dropout float64 outside training")
+    for p in (px, pdy, pdx, pr, py):
+        ctx.free(p)
+
+
+@pytest.mark.parametrize("kind,kw", [
+    ("vanilla", dict(eta=0.1, l1reg=0.01, l2reg=0.02, clip=1.5, batch=4.0)),
+    ("rmsprop", dict(eta=0.01, clip=2.0, l2reg=0.001, decay=0.9)),
+    ("adam", dict(eta=0.001, iteration=1, l2reg=0.01, clip=3.0)),
+])
+def test_solver_steps_float64(ctx, kind, kw):
+    n = 50021
+    w, c1, c2 = _rand(8, (n,)), np.zeros(n), np.zeros(n)
+    pw, pc1, pc2 = _up(ctx, w), _up(ctx, c1), _up(ctx, c2)
+    for step in range(3):
+        g = _rand(9 + step, (n,), 3.0)
+        if kind == "adam":
+            kw = dict(kw, iteration=kw["iteration"] + (1 if step else 0))
+        par, use = O.solver_params(kind=kind, dtype=np.float64, **kw)
+        pg = _up(ctx, g)
+        ctx.run(D.cmd_solver_step(kind, pw, pg, n, par, use, pc1, pc2, dtype=F64))
+        ctx.free(pg)
+        w, _, c1, c2 = O.solver_step(kind, w, g, c1, c2, **kw)
+        assert_bits_equal(ctx.d2h(pw, (n,), np.float64), w, f"{kind} float64 weights, step {step}")
+        if kind != "vanilla":
+            assert_bits_equal(ctx.d2h(pc1, (n,), np.float64), c1, f"{kind} float64 cache, step {step}")
+        if kind == "adam":
+            assert_bits_equal(ctx.d2h(pc2, (n,), np.float64), c2, f"adam float64 v, step {step}")
+    for p in (pw, pc1, pc2):
+        ctx.free(p)
+
+
+def test_float64_flags_validate(ctx):
+    buf = C.create_string_buffer(256)
+    ok = D.cmd_dropout(1, 2, 3, 10, 0.25, dtype=F64)
+    assert ctx.lib.gh_validate(C.byref(ok), 1, buf, 256) == 0
+    bad = D.cmd_dropout(1, 2, 3, 10, 1.5, dtype=F64)
+    assert ctx.lib.gh_validate(C.byref(bad), 1, buf, 256) != 0 and b"probability" in buf.value
+    for cmd in (D.cmd_bn_train(1, 2, 3, 4, 5, 6, 2, 4, 4, 1e-5, 0.9),):
+        cmd.flags |= _ffi.flag_dtype(F64)
+        assert ctx.lib.gh_validate(C.byref(cmd), 1, buf, 256) != 0 and b"float32 only" in buf.value
+
+
+def test_float64_training_ops_on_the_tape(ctx):
+    """A float64 dense layer trained on the tape machine: MatMul, SoftMax, SoftMaxDiff,
+    RectifyDiff, MaxPool2DDiff-free path, RMSProp step - every command carries the float64
+    flag and the solver's constants stay doubles; two steps against the oracle's twins."""
+    from gorgonia_amd import graph as G
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((16, 12))
+    w0 = rng.standard_normal((12, 5)) * 0.3
+    onehot = np.zeros((16, 5))
+    onehot[np.arange(16), np.arange(16) % 5] = 1.0
+    g = G.NewGraph()
+    xn = G.NewTensor(g, x)
+    wn = G.NewTensor(g, w0.copy(), resident=True)
+    cache = G.NewTensor(g, np.zeros_like(w0), resident=True)
+    yn = G.NewTensor(g, onehot)
+    scale = G.NewScalar(g, -1.0 / onehot.size, dtype=np.float64)
+    z = G.Mul(xn, wn)
+    a = G.Rectify(z)
+    out = G.SoftMax(a)
+    gout = G.SoftMaxDiff(out, G.HadamardProd(yn, scale))
+    dz = G.RectifyDiff(z, gout)
+    dw = G.Mul(xn, dz, transA=True)
+    res = {"out": G.Read(out, dtype=np.float64), "dw": G.Read(dw, dtype=np.float64)}
+    G.SolverStep("rmsprop", wn, dw, [cache], eta=0.01, decay=0.9)
+    res["w"] = G.Read(wn, dtype=np.float64)
+    m = G.NewTapeMachine(g)
+    w, c = w0.copy(), np.zeros_like(w0)
+    for step in range(2):
+        m.RunAll()
+        zz = x @ w
+        aa = O.relu(zz).reshape(zz.shape)
+        oo = O.softmax(aa)
+        go = O.softmax_bwd(oo, O.binop("mul", "vs", onehot.reshape(-1), np.array([-1.0 / onehot.size])).reshape(onehot.shape))
+        dzz = O.binop("mul", "vv", go.reshape(-1), O.binop("gte", "vs", zz.reshape(-1), np.zeros(1))).reshape(zz.shape)
+        dww = x.T @ dzz
+        assert np.allclose(res["out"], oo, rtol=0, atol=1e-12), f"step {step}"
+        assert np.allclose(res["dw"], dww, rtol=0, atol=1e-12), f"step {step}"
+        w_new, _, c, _ = O.solver_step("rmsprop", w.reshape(-1), res["dw"].reshape(-1), c.reshape(-1), eta=0.01, decay=0.9)
+        assert_bits_equal(res["w"].reshape(-1), w_new, f"float64 RMSProp step {step} on the device's own gradient")
+        w = w_new.reshape(w0.shape)
+    m.Close()

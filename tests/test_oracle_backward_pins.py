@@ -302,3 +302,56 @@ def test_uniform_source_is_the_synthetic_stream():
     a = O.uniform01(1 << 16, 5)
     assert np.array_equal(O.uniform01(100, 5, offset=1000), a[1000:1100])
     assert 0.0 <= a.min() and a.max() < 1.0 and abs(a.mean() - 0.5) < 0.01
+
+
+# ---- float64 twins of the backward operators ---------------------------------------------
+
+def test_float64_backward_twins_against_the_float32_oracle():
+    """Each float64 twin equals its pinned float32 counterpart where float32 arithmetic is
+    exact (small integers, divisions by powers of two) and stays within float32 rounding of
+    it on random data - a dropped term or a wrong index in a twin fails both."""
+    rng = np.random.default_rng(5)
+    # max-pool backward: integer gradients (every sum exact); ties and padding included
+    x = rng.integers(-3, 4, (2, 3, 7, 9)).astype(np.float32)
+    for kernel, pad, stride in [((2, 2), (0, 0), (2, 2)), ((3, 3), (1, 1), (2, 2)), ((2, 2), (1, 0, 1, 0), (1, 1))]:
+        oh, ow = O.maxpool2d(x, kernel, pad, stride).shape[2:]
+        dy = rng.integers(-5, 6, (2, 3, oh, ow)).astype(np.float32)
+        d32 = O.maxpool2d_bwd(x, dy, kernel, pad, stride)
+        d64 = O.maxpool2d_bwd(x.astype(np.float64), dy.astype(np.float64), kernel, pad, stride)
+        assert d64.dtype == np.float64 and np.array_equal(d64, d32.astype(np.float64))
+    # softmax backward: integer y and dy (exact), then random (within float32 rounding)
+    y = rng.integers(-3, 4, (5, 7)).astype(np.float32)
+    dy = rng.integers(-3, 4, (5, 7)).astype(np.float32)
+    assert np.array_equal(O.softmax_bwd(y.astype(np.float64), dy.astype(np.float64)), O.softmax_bwd(y, dy).astype(np.float64))
+    y = O.softmax(rng.standard_normal((6, 10)).astype(np.float32))
+    dy = rng.standard_normal((6, 10)).astype(np.float32)
+    np.testing.assert_allclose(O.softmax_bwd(y.astype(np.float64), dy.astype(np.float64)), O.softmax_bwd(y, dy), rtol=0, atol=1e-6)
+    # dropout: keep = 0.5 divides exactly
+    xd = rng.integers(-8, 9, 64).astype(np.float32)
+    r = rng.random(64).astype(np.float32)
+    y32 = O.dropout(xd, r, 0.5)
+    y64 = O.dropout(xd.astype(np.float64), r.astype(np.float64), 0.5)
+    assert np.array_equal(y64, y32.astype(np.float64))
+    assert np.array_equal(O.dropout(xd.astype(np.float64), r.astype(np.float64), 0.5, training=False), xd)
+    g = rng.integers(-8, 9, 64).astype(np.float32)
+    assert np.array_equal(O.dropout_bwd(y64, g.astype(np.float64), 0.5), O.dropout_bwd(y32, g, 0.5).astype(np.float64))
+    # solver steps: three steps of each kind within float32 rounding of the float32 oracle
+    for kind, kw in [("vanilla", dict(eta=0.1, l2reg=0.01, clip=1.5, batch=4.0)), ("rmsprop", dict(eta=0.01, clip=2.0, l2reg=0.001)),
+                     ("adam", dict(eta=0.001, iteration=2, l1reg=0.01))]:
+        w32 = rng.standard_normal(500).astype(np.float32)
+        w64 = w32.astype(np.float64)
+        c32 = [None, None]
+        c64 = [None, None]
+        for step in range(3):
+            g32 = (rng.standard_normal(500) * 3).astype(np.float32)
+            w32, _, c32[0], c32[1] = O.solver_step(kind, w32, g32, c32[0], c32[1], **kw)
+            w64, _, c64[0], c64[1] = O.solver_step(kind, w64, g32.astype(np.float64), c64[0], c64[1], **kw)
+        assert w64.dtype == np.float64
+        np.testing.assert_allclose(w64, w32, rtol=2e-5, atol=2e-6)
+        if kind != "vanilla":
+            np.testing.assert_allclose(c64[0], c32[0], rtol=2e-5, atol=1e-7)
+    # vanilla without options is w - eta*g exactly
+    w = rng.standard_normal(100)
+    g = rng.standard_normal(100)
+    got, _, _, _ = O.solver_step("vanilla", w, g, eta=0.25)
+    assert np.array_equal(got, w + g * -0.25)
