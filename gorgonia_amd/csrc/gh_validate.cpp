@@ -106,7 +106,6 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
         if ((c.flags & GH_FLAG_HAS_BETA) && !c.ptr[6]) return bad("conv2d: fused BatchNorm beta is null");
       }
       if (dt > GH_F64) return bad("Unsupported Dtype");
-      if (dt == GH_F64 && c.opcode != GH_OP_CONV2D) return bad("conv2d backward: float32 only");
       if (dt == GH_F64 && (c.flags & (GH_FLAG_CONV_BN | GH_FLAG_CONV_POOL2 | GH_FLAG_ACT_RELU | GH_FLAG_ACT_LEAKY)))
         return bad("conv2d: no epilogue operators for float64");
       if ((c.flags & GH_FLAG_CONV_POOL2) && !gh_conv2d_can_pool(&c))

@@ -2135,6 +2135,7 @@ static ConvGeom conv_geom(const gh_cmd& c) {
 
 // dW = dY2d^T . col  (ptr[0] = x, ptr[1] = dy, ptr[2] = dw)
 int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_conv2d_bwd_filter_f64(ctx, c);
   const ConvGeom g = conv_geom(c);
   const int F = (int)c.dim[4], CKK = g.C * g.kh * g.kw;
   if (conv_direct_shape(c) && F <= 65535) {
@@ -2193,6 +2194,7 @@ int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
 
 // dX = col2im(dY2d . Wflat)  (ptr[0] = dy, ptr[1] = w, ptr[2] = dx)
 int gh_launch_conv2d_bwd_data(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_conv2d_bwd_data_f64(ctx, c);
   const ConvGeom g = conv_geom(c);
   const int B = (int)c.dim[0], F = (int)c.dim[4];
   const float* dy = (const float*)(uintptr_t)c.ptr[0];

@@ -148,6 +148,74 @@ __global__ __launch_bounds__(kBlock) void k_conv2d_f64(const double* __restrict_
   }
 }
 
+// Conv2d gradients in float64 (the reference differentiates the im2col form,
+// nn.go:211-305, op_nn.go:267-291, 605-640; these sum the same products per
+// element): one thread per gradient element, plain loops, not tuned.
+// Image gradient: dx[b,c,iy,ix] = sum over f, kr, kc of dy[b,f,oy,ox] * w[f,c,kr,kc]
+// where oy*stride - pad + kr*dil = iy (and the same for columns).
+__global__ __launch_bounds__(kBlock) void k_conv2d_bwd_data_f64(const double* __restrict__ dy,
+                                                                const double* __restrict__ w,
+                                                                double* __restrict__ dx, Conv64 g, int64_t total) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  const int plane = g.H * g.W;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += stride) {
+    const int64_t bc = i / plane;
+    const int rem = (int)(i - bc * plane);
+    const int iy = rem / g.W, ix = rem - iy * g.W;
+    const int b = (int)(bc / g.C), c = (int)(bc - (int64_t)b * g.C);
+    double acc = 0.0;
+    for (int f = 0; f < g.F; f++) {
+      const double* gy = dy + ((int64_t)b * g.F + f) * g.oh * g.ow;
+      const double* wf = w + ((int64_t)f * g.C + c) * g.kh * g.kw;
+      for (int kr = 0; kr < g.kh; kr++) {
+        const int ty = iy + g.padH - kr * g.dilH;
+        if (ty < 0 || ty % g.strideH) continue;
+        const int oy = ty / g.strideH;
+        if (oy >= g.oh) continue;
+        for (int kc = 0; kc < g.kw; kc++) {
+          const int tx = ix + g.padW - kc * g.dilW;
+          if (tx < 0 || tx % g.strideW) continue;
+          const int ox = tx / g.strideW;
+          if (ox >= g.ow) continue;
+          const double p = gy[oy * g.ow + ox] * wf[kr * g.kw + kc];
+          acc = acc + p;
+        }
+      }
+    }
+    dx[i] = acc;
+  }
+}
+
+// Filter gradient: dw[f,c,kr,kc] = sum over b, oy, ox of dy[b,f,oy,ox] * x[b,c,iy,ix].
+__global__ __launch_bounds__(kBlock) void k_conv2d_bwd_filter_f64(const double* __restrict__ x,
+                                                                  const double* __restrict__ dy,
+                                                                  double* __restrict__ dw, Conv64 g, int64_t total) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  const int kk = g.kh * g.kw;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += stride) {
+    const int64_t fc = i / kk;
+    const int tap = (int)(i - fc * kk);
+    const int kr = tap / g.kw, kc = tap - kr * g.kw;
+    const int f = (int)(fc / g.C), c = (int)(fc - (int64_t)f * g.C);
+    double acc = 0.0;
+    for (int b = 0; b < g.B; b++) {
+      const double* gy = dy + ((int64_t)b * g.F + f) * g.oh * g.ow;
+      const double* xc = x + ((int64_t)b * g.C + c) * g.H * g.W;
+      for (int oy = 0; oy < g.oh; oy++) {
+        const int iy = oy * g.strideH - g.padH + kr * g.dilH;
+        if (iy < 0 || iy >= g.H) continue;
+        for (int ox = 0; ox < g.ow; ox++) {
+          const int ix = ox * g.strideW - g.padW + kc * g.dilW;
+          if (ix < 0 || ix >= g.W) continue;
+          const double p = gy[oy * g.ow + ox] * xc[iy * g.W + ix];
+          acc = acc + p;
+        }
+      }
+    }
+    dw[i] = acc;
+  }
+}
+
 int blocks_for(gh_ctx* ctx, int64_t n) {
   int64_t blocks = (n + kBlock - 1) / kBlock;
   if (blocks > (int64_t)ctx->cu_count * 32) blocks = (int64_t)ctx->cu_count * 32;
@@ -205,13 +273,38 @@ int gh_launch_softmax_f64(gh_ctx* ctx, const gh_cmd& c) {
   return gh_check_hip(ctx, hipGetLastError(), "softmax launch");
 }
 
-int gh_launch_conv2d_f64(gh_ctx* ctx, const gh_cmd& c) {
+static Conv64 conv64_geom(const gh_cmd& c) {
   Conv64 g;
   g.B = (int)c.dim[0]; g.C = (int)c.dim[1]; g.H = (int)c.dim[2]; g.W = (int)c.dim[3]; g.F = (int)c.dim[4];
   g.kh = (int)c.dim[5]; g.kw = (int)c.dim[6]; g.padH = (int)c.dim[7]; g.padW = (int)c.dim[8];
   g.strideH = (int)c.dim[9]; g.strideW = (int)c.dim[10]; g.dilH = (int)c.dim[11]; g.dilW = (int)c.dim[12];
   g.oh = (int)gh_conv_out(g.H, g.kh, g.padH, g.strideH, g.dilH);
   g.ow = (int)gh_conv_out(g.W, g.kw, g.padW, g.strideW, g.dilW);
+  return g;
+}
+
+int gh_launch_conv2d_bwd_data_f64(gh_ctx* ctx, const gh_cmd& c) {
+  const Conv64 g = conv64_geom(c);
+  const int64_t total = (int64_t)g.B * g.C * g.H * g.W;
+  if (total <= 0) return GH_OK;
+  hipLaunchKernelGGL(k_conv2d_bwd_data_f64, dim3(blocks_for(ctx, total)), dim3(kBlock), 0, ctx->stream,
+                     (const double*)(uintptr_t)c.ptr[0], (const double*)(uintptr_t)c.ptr[1],
+                     (double*)(uintptr_t)c.ptr[2], g, total);
+  return gh_check_hip(ctx, hipGetLastError(), "conv2d image gradient launch");
+}
+
+int gh_launch_conv2d_bwd_filter_f64(gh_ctx* ctx, const gh_cmd& c) {
+  const Conv64 g = conv64_geom(c);
+  const int64_t total = (int64_t)g.F * g.C * g.kh * g.kw;
+  if (total <= 0) return GH_OK;
+  hipLaunchKernelGGL(k_conv2d_bwd_filter_f64, dim3(blocks_for(ctx, total)), dim3(kBlock), 0, ctx->stream,
+                     (const double*)(uintptr_t)c.ptr[0], (const double*)(uintptr_t)c.ptr[1],
+                     (double*)(uintptr_t)c.ptr[2], g, total);
+  return gh_check_hip(ctx, hipGetLastError(), "conv2d filter gradient launch");
+}
+
+int gh_launch_conv2d_f64(gh_ctx* ctx, const gh_cmd& c) {
+  const Conv64 g = conv64_geom(c);
   const int64_t total = (int64_t)g.B * g.F * g.oh * g.ow;
   if (total <= 0) return GH_OK;
   hipLaunchKernelGGL(k_conv2d_f64, dim3(blocks_for(ctx, total)), dim3(kBlock), 0, ctx->stream,

@@ -246,13 +246,17 @@ def _conv_dims(B, Cin, H, W, F, kh, kw, pad, stride, dilation):
     return (B, Cin, H, W, F, kh, kw, pad[0], pad[1], stride[0], stride[1], dilation[0], dilation[1])
 
 
-def cmd_conv2d_bwd_data(dy, w, dx, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dilation=(1, 1)):
+def cmd_conv2d_bwd_data(dy, w, dx, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dilation=(1, 1),
+                        dtype=_ffi.F32):
     """dx of Conv2d; B, Cin, H, W describe x (and dx)."""
-    return make_cmd(_ffi.OP_CONV2D_BWD_DATA, 0, (dy, w, dx), _conv_dims(B, Cin, H, W, F, kh, kw, pad, stride, dilation))
+    return make_cmd(_ffi.OP_CONV2D_BWD_DATA, _ffi.flag_dtype(dtype), (dy, w, dx),
+                    _conv_dims(B, Cin, H, W, F, kh, kw, pad, stride, dilation))
 
 
-def cmd_conv2d_bwd_filter(x, dy, dw, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dilation=(1, 1)):
-    return make_cmd(_ffi.OP_CONV2D_BWD_FILTER, 0, (x, dy, dw), _conv_dims(B, Cin, H, W, F, kh, kw, pad, stride, dilation))
+def cmd_conv2d_bwd_filter(x, dy, dw, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dilation=(1, 1),
+                          dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_CONV2D_BWD_FILTER, _ffi.flag_dtype(dtype), (x, dy, dw),
+                    _conv_dims(B, Cin, H, W, F, kh, kw, pad, stride, dilation))
 
 
 def cmd_bn_train(x, y, run_mean, run_var, save_mean, save_var, B, Cn, S, eps, momentum):

@@ -457,9 +457,10 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     case OpKind::Conv2dDiffData:
     case OpKind::Conv2dDiffFilter: {
       const bool data = op.kind == OpKind::Conv2dDiffData;
-      if (in[0]->dt != Dtype::Float32 || in[1]->dt != Dtype::Float32) return bad("Conv2d gradients: float32 only");
+      if (in[0]->dt == Dtype::Other || in[1]->dt != in[0]->dt) return bad("Conv2d gradients: Unsupported Dtype");
       gh_cmd c{};
       c.opcode = data ? GH_OP_CONV2D_BWD_DATA : GH_OP_CONV2D_BWD_FILTER;
+      c.flags = dtype_flag(in[0]->dt);
       c.ptr[0] = in[0]->mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
       const Shape& xs = data ? prealloc.shape : in[0]->shape;
       for (int i = 0; i < 4; i++) c.dim[i] = xs[i];

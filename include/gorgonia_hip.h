@@ -187,11 +187,12 @@ enum gh_unaryfn {
  *             dim[0..2]=B,C,S  f[0]=eps ; BN_EVAL selects dx = dy/sqrt(save_var/n + eps)
  * SOFTMAX_BWD ptr[0]=y ptr[1]=dy ptr[2]=dx        dim[0]=rows dim[1]=cols
  * float64: CONV2D (no epilogue flags), MAXPOOL2D, BN_INFER, RELU, LEAKY_RELU, SOFTMAX,
- *             MAXPOOL2D_BWD, SOFTMAX_BWD, RELU_BWD, DROPOUT, DROPOUT_BWD and SOLVER_STEP take
+ *             CONV2D_BWD_DATA, CONV2D_BWD_FILTER, MAXPOOL2D_BWD, SOFTMAX_BWD, RELU_BWD, DROPOUT,
+ *             DROPOUT_BWD and SOLVER_STEP take
  *             GH_FLAG_DTYPE(GH_F64); their scalars then travel as the bit pattern of a double
  *             in a dim slot (LEAKY_RELU alpha: dim[1]; BN_INFER epsilon: dim[3]; DROPOUT and
  *             DROPOUT_BWD probability: dim[1]; SOLVER_STEP's ten constants: dim[1..10]).
- *             CONV2D_BWD_*, BN_TRAIN, BN_BWD and RAND_UNIFORM are float32 only
+ *             BN_TRAIN, BN_BWD and RAND_UNIFORM are float32 only
  * RAND_UNIFORM ptr[0]=out [ptr[1]=state]          dim[0]=n dim[1]=seed dim[2]=offset
  *             float32 in [0,1) with 24 random bits, element i = SplitMix64 output function
  *             of seed*0xD1342543DE82EF95 + (offset + i + 1)*0x9E3779B97F4A7C15.  With a

@@ -266,7 +266,19 @@ def maxpool2d_bwd(x, dy, kernel, pad, stride):
 
 
 def conv2d_bwd(x, w, dy, pad=(0, 0), stride=(1, 1), dil=(1, 1)):
-    """(dx, dw) of Conv2d as the reference's graph differentiates it, float32."""
+    """(dx, dw) of Conv2d as the reference's graph differentiates it (float32), or for float64
+    operands from the definition in float64."""
+    if np.asarray(x).dtype == np.float64:
+        x = np.ascontiguousarray(x, dtype=np.float64)
+        w = np.ascontiguousarray(w, dtype=np.float64)
+        dy = np.ascontiguousarray(dy, dtype=np.float64)
+        B, Cn, H, W = x.shape
+        F, _, kh, kw = w.shape
+        dx, dw = np.empty_like(x), np.empty_like(w)
+        lib().oracle_conv2d_bwd_f64(_p(x), _p(w), _p(dy), _p(dx), _p(dw),
+                                    *_i64(B, Cn, H, W, F, kh, kw, pad[0], pad[1], stride[0], stride[1],
+                                          dil[0], dil[1]))
+        return dx, dw
     x = np.ascontiguousarray(x, dtype=np.float32)
     w = np.ascontiguousarray(w, dtype=np.float32)
     dy = np.ascontiguousarray(dy, dtype=np.float32)

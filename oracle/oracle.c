@@ -1154,6 +1154,36 @@ EXPORT void oracle_maxpool2d_bwd_f64(const double* x, const double* dy, double* 
   }
 }
 
+/* Conv2d gradients from the definition with float64 operands: the float64 twin
+ * of oracle_conv2d_bwd_f32 (same products; float64 sums make the order moot at
+ * the conv tolerance, and on integer-valued data every order is exact). */
+EXPORT void oracle_conv2d_bwd_f64(const double* x, const double* w, const double* dy, double* dx,
+                                  double* dw, int64_t B, int64_t C, int64_t H, int64_t W, int64_t F,
+                                  int64_t kh, int64_t kw, int64_t padH, int64_t padW,
+                                  int64_t strideH, int64_t strideW, int64_t dilH, int64_t dilW) {
+  int64_t oh, ow, b, f, r, c, ch, kr, kc, i;
+  oracle_conv_out_hw(H, W, kh, kw, padH, padW, strideH, strideW, dilH, dilW, &oh, &ow);
+  for (i = 0; i < B * C * H * W; i++) dx[i] = 0.0;
+  for (i = 0; i < F * C * kh * kw; i++) dw[i] = 0.0;
+  for (b = 0; b < B; b++)
+    for (f = 0; f < F; f++)
+      for (r = 0; r < oh; r++)
+        for (c = 0; c < ow; c++) {
+          const double g = dy[((b * F + f) * oh + r) * ow + c];
+          for (ch = 0; ch < C; ch++)
+            for (kr = 0; kr < kh; kr++)
+              for (kc = 0; kc < kw; kc++) {
+                int64_t ir = r * strideH - padH + kr * dilH;
+                int64_t ic = c * strideW - padW + kc * dilW;
+                if (ir < 0 || ir >= H || ic < 0 || ic >= W) continue;
+                int64_t xi = ((b * C + ch) * H + ir) * W + ic;
+                int64_t wi = ((f * C + ch) * kh + kr) * kw + kc;
+                dx[xi] += g * w[wi];
+                dw[wi] += g * x[xi];
+              }
+        }
+}
+
 EXPORT void oracle_softmax_bwd_f64(const double* y, const double* dy, double* dx, int64_t rows,
                                    int64_t cols) {
   int64_t r, j;

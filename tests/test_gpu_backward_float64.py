@@ -162,3 +162,35 @@ def test_float64_training_ops_on_the_tape(ctx):
         assert_bits_equal(res["w"].reshape(-1), w_new, f"float64 RMSProp step {step} on the device's own gradient")
         w = w_new.reshape(w0.shape)
     m.Close()
+
+
+@pytest.mark.parametrize("cfg", [
+    (2, 3, 9, 8, 5, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (1, 8, 14, 14, 16, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (2, 4, 10, 11, 6, 1, 1, (0, 0), (1, 1), (1, 1)),
+    (2, 2, 12, 9, 3, 5, 3, (2, 1), (2, 1), (1, 1)),
+    (1, 3, 13, 13, 4, 3, 3, (2, 2), (1, 2), (2, 2)),
+])
+def test_conv_gradients_float64(ctx, cfg):
+    """Image and filter gradients of Conv2d in float64: relative Frobenius error <= 1e-12
+    against the oracle's float64 definition, and equal on integer-valued operands."""
+    B, Cn, H, W, F, kh, kw, pad, stride, dil = cfg
+    for integer in (False, True):
+        rng = np.random.default_rng(21)
+        gen = (lambda s: rng.integers(-3, 4, s).astype(np.float64)) if integer else (lambda s: rng.standard_normal(s))
+        x, w = gen((B, Cn, H, W)), gen((F, Cn, kh, kw))
+        oh, ow = O.conv2d(x, w, pad, stride, dil).shape[2:]
+        dy = gen((B, F, oh, ow))
+        dx_ref, dw_ref = O.conv2d_bwd(x, w, dy, pad, stride, dil)
+        px, pw, pdy = _up(ctx, x), _up(ctx, w), _up(ctx, dy)
+        pdx, pdw = ctx.malloc(x.size * 8), ctx.malloc(w.size * 8)
+        ctx.run([D.cmd_conv2d_bwd_data(pdy, pw, pdx, B, Cn, H, W, F, kh, kw, pad, stride, dil, dtype=F64),
+                 D.cmd_conv2d_bwd_filter(px, pdy, pdw, B, Cn, H, W, F, kh, kw, pad, stride, dil, dtype=F64)])
+        dx, dw = ctx.d2h(pdx, x.shape, np.float64), ctx.d2h(pdw, w.shape, np.float64)
+        if integer:
+            assert np.array_equal(dx, dx_ref) and np.array_equal(dw, dw_ref)
+        else:
+            assert np.linalg.norm(dx - dx_ref) <= 1e-12 * np.linalg.norm(dx_ref)
+            assert np.linalg.norm(dw - dw_ref) <= 1e-12 * np.linalg.norm(dw_ref)
+        for p in (px, pw, pdy, pdx, pdw):
+            ctx.free(p)

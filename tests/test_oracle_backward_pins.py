@@ -355,3 +355,23 @@ def test_float64_backward_twins_against_the_float32_oracle():
     g = rng.standard_normal(100)
     got, _, _, _ = O.solver_step("vanilla", w, g, eta=0.25)
     assert np.array_equal(got, w + g * -0.25)
+
+
+def test_float64_conv_gradients_against_the_float32_oracle():
+    """The float64 conv gradients equal the pinned float32 ones on integer-valued operands
+    (every order of summation exact) and agree within float32 rounding on random ones."""
+    rng = np.random.default_rng(6)
+    for (B, C, H, W, F, kh, kw, pad, stride, dil) in [(2, 3, 7, 6, 4, 3, 3, (1, 1), (1, 1), (1, 1)),
+                                                      (1, 2, 9, 9, 3, 3, 2, (2, 0), (2, 1), (1, 2))]:
+        x = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+        w = rng.integers(-3, 4, (F, C, kh, kw)).astype(np.float32)
+        oh, ow = O.conv2d(x, w, pad, stride, dil).shape[2:]
+        dy = rng.integers(-3, 4, (B, F, oh, ow)).astype(np.float32)
+        dx32, dw32 = O.conv2d_bwd(x, w, dy, pad, stride, dil)
+        dx64, dw64 = O.conv2d_bwd(x.astype(np.float64), w.astype(np.float64), dy.astype(np.float64), pad, stride, dil)
+        assert dx64.dtype == np.float64 and np.array_equal(dx64, dx32) and np.array_equal(dw64, dw32)
+        xr, wr, dyr = (rng.standard_normal(a.shape).astype(np.float32) for a in (x, w, dy))
+        dx32, dw32 = O.conv2d_bwd(xr, wr, dyr, pad, stride, dil)
+        dx64, dw64 = O.conv2d_bwd(xr.astype(np.float64), wr.astype(np.float64), dyr.astype(np.float64), pad, stride, dil)
+        assert np.linalg.norm(dx64 - dx32) <= 1e-5 * np.linalg.norm(dx64)
+        assert np.linalg.norm(dw64 - dw32) <= 1e-5 * np.linalg.norm(dw64)
