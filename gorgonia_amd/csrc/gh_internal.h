@@ -49,6 +49,8 @@ int gh_launch_dropout_bwd_f64(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_softmax_bwd_f64(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_maxpool2d_bwd_f64(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_solver_step_f64(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_bn_train_f64(gh_ctx* ctx, const gh_cmd& c);
+int gh_launch_bn_bwd_f64(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_conv2d_bwd_data_f64(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_conv2d_bwd_filter_f64(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_leaky_relu(gh_ctx* ctx, const gh_cmd& c);

@@ -144,14 +144,14 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (!pos(c.dim[0]) || !pos(c.dim[1]) || !pos(c.dim[2])) return bad("bn: B,C,S must be positive");
       if (c.dim[1] > 65535) return bad("bn: more than 65535 channels");
       if (c.dim[0] * c.dim[2] < 2) return bad("bn: training statistics need at least two values per channel");
-      if (dt != GH_F32) return bad("bn training: float32 only");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     case GH_OP_BN_BWD:
       for (int i = 0; i < 5; i++)
         if (!c.ptr[i]) return bad("null operand");
       if (!pos(c.dim[0]) || !pos(c.dim[1]) || !pos(c.dim[2])) return bad("bn: B,C,S must be positive");
       if (c.dim[1] > 65535) return bad("bn: more than 65535 channels");
-      if (dt != GH_F32) return bad("bn backward: float32 only");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     case GH_OP_SOFTMAX_BWD:
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
@@ -170,7 +170,7 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (!c.ptr[0]) return bad("null operand");
       if (c.dim[0] < 0) return bad("negative size");
       if (c.ptr[1] & 7) return bad("rand: state must be 8-byte aligned");
-      if (dt != GH_F32) return bad("rand: float32 only");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;
     case GH_OP_RELU_BWD:
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");

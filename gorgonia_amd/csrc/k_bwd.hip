@@ -424,7 +424,9 @@ __global__ __launch_bounds__(kBlock) void k_solver_step(SolverBatch sb, int use,
 // ---- dropout and its random source -------------------------------------------------------
 // Counter-based: element i is a pure function of (seed, offset + i), so the
 // numbers do not depend on the launch shape and a CPU twin can reproduce them.
-__global__ __launch_bounds__(kBlock) void k_rand_uniform(float* __restrict__ out, int64_t n, uint64_t seed,
+// T = float: the top 24 bits; T = double: the top 53 bits of the same 64-bit value.
+template <class T>
+__global__ __launch_bounds__(kBlock) void k_rand_uniform(T* __restrict__ out, int64_t n, uint64_t seed,
                                                          uint64_t offset, const uint64_t* __restrict__ state) {
   if (state) offset = *state;
   const uint64_t base = seed * 0xD1342543DE82EF95ull;
@@ -433,7 +435,8 @@ __global__ __launch_bounds__(kBlock) void k_rand_uniform(float* __restrict__ out
     z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
     z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
     z = z ^ (z >> 31);
-    out[i] = (float)(uint32_t)(z >> 40) * 5.9604644775390625e-08f;
+    if constexpr (sizeof(T) == 8) out[i] = (double)(z >> 11) * 1.1102230246251565e-16;   // 2^-53
+    else out[i] = (float)(uint32_t)(z >> 40) * 5.9604644775390625e-08f;                    // 2^-24
   }
 }
 
@@ -496,6 +499,7 @@ int gh_launch_maxpool2d_bwd(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_bn_train(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_bn_train_f64(ctx, c);
   const int64_t B = c.dim[0], C = c.dim[1], S = c.dim[2], n = B * S;
   const int G = bn_groups(n, S);
   // scratch: [C][G] sums, [C][G] squared deviations, [C] batch variance
@@ -524,6 +528,7 @@ int gh_launch_bn_train(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_bn_bwd(gh_ctx* ctx, const gh_cmd& c) {
+  if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_bn_bwd_f64(ctx, c);
   const int64_t B = c.dim[0], C = c.dim[1], S = c.dim[2], n = B * S;
   const int G = bn_groups(n, S);
   if (2 * C * G * 4 > ctx->workspace_bytes) return gh_fail(ctx, GH_ESTATE, "batchnorm: reduction scratch does not fit the workspace");
@@ -624,8 +629,11 @@ static int stream_blocks(gh_ctx* ctx, int64_t n) {
 int gh_launch_rand_uniform(gh_ctx* ctx, const gh_cmd& c) {
   const int64_t n = c.dim[0];
   uint64_t* state = (uint64_t*)(uintptr_t)c.ptr[1];
-  if (n > 0)
-    hipLaunchKernelGGL(k_rand_uniform, dim3(stream_blocks(ctx, n)), dim3(kBlock), 0, ctx->stream,
+  if (n > 0 && gh_dtype_of(c.flags) == GH_F64)
+    hipLaunchKernelGGL(k_rand_uniform<double>, dim3(stream_blocks(ctx, n)), dim3(kBlock), 0, ctx->stream,
+                       (double*)(uintptr_t)c.ptr[0], n, (uint64_t)c.dim[1], (uint64_t)c.dim[2], state);
+  else if (n > 0)
+    hipLaunchKernelGGL(k_rand_uniform<float>, dim3(stream_blocks(ctx, n)), dim3(kBlock), 0, ctx->stream,
                        (float*)(uintptr_t)c.ptr[0], n, (uint64_t)c.dim[1], (uint64_t)c.dim[2], state);
   if (state && n > 0) hipLaunchKernelGGL(k_rand_advance, dim3(1), dim3(1), 0, ctx->stream, state, (uint64_t)n);
   return gh_check_hip(ctx, hipGetLastError(), "uniform generator launch");

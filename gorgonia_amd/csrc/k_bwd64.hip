@@ -7,7 +7,7 @@
 // operation in double.  Plain one-thread-per-element kernels, not tuned.
 // Scalars ride in dim slots as the bit pattern of a double (gh_cmd.f is float32):
 // DROPOUT / DROPOUT_BWD probability in dim[1]; SOLVER_STEP's ten constants in
-// dim[1..10].
+// dim[1..10]; BN_TRAIN epsilon and momentum in dim[3], dim[4]; BN_BWD epsilon in dim[3].
 #include <cfloat>
 #include <cstring>
 
@@ -104,6 +104,110 @@ __global__ __launch_bounds__(kBlock) void k_maxpool2d_bwd_f64(const double* __re
         if (arg == me) acc = acc + gy[ph * g.ow + pw];
       }
     dx[idx] = acc;
+  }
+}
+
+// ---- BatchNorm training forward and gradient (op_nn.go:1489-1635, 1834-1943) -------------
+// One workgroup per channel: the channel's n = B*S values are summed by a fixed
+// tree (thread-strided partial sums, then a tree over the 256 threads), so
+// results repeat run to run; against the reference's sequential sums the
+// difference is float64 rounding.
+__device__ __forceinline__ double block_sum_f64(double v, double* sh) {
+  sh[threadIdx.x] = v;
+  __syncthreads();
+  for (int off = kBlock / 2; off > 0; off >>= 1) {
+    if ((int)threadIdx.x < off) sh[threadIdx.x] = sh[threadIdx.x] + sh[threadIdx.x + off];
+    __syncthreads();
+  }
+  const double r = sh[0];
+  __syncthreads();
+  return r;
+}
+
+__global__ __launch_bounds__(kBlock) void k_bn_train_f64(const double* __restrict__ x, double* __restrict__ y,
+                                                         double* __restrict__ run_mean,
+                                                         double* __restrict__ run_var,
+                                                         double* __restrict__ save_mean,
+                                                         double* __restrict__ save_var, int64_t B, int C,
+                                                         int64_t S, double eps, double momentum) {
+  __shared__ double sh[kBlock];
+  const int c = blockIdx.x;
+  const int64_t n = B * S;
+  auto at = [&](int64_t e) { return ((e / S) * C + c) * S + e % S; };
+  double acc = 0.0;
+  for (int64_t e = threadIdx.x; e < n; e += kBlock) acc = acc + x[at(e)];
+  const double mean = block_sum_f64(acc, sh) / (double)n;
+  acc = 0.0;
+  for (int64_t e = threadIdx.x; e < n; e += kBlock) {
+    const double t = x[at(e)] - mean;
+    const double t2 = t * t;
+    acc = acc + t2;
+  }
+  const double var = block_sum_f64(acc, sh);   // the SUM of squared deviations, as the reference keeps it
+  if (threadIdx.x == 0) {
+    save_mean[c] = mean;
+    save_var[c] = var;
+    const double m1 = momentum * mean, m2 = (1.0 - momentum) * run_mean[c];
+    run_mean[c] = m1 + m2;
+    const double unb = var / (double)(n - 1);
+    const double v1 = momentum * unb, v2 = (1.0 - momentum) * run_var[c];
+    run_var[c] = v1 + v2;
+  }
+  const double vb = var / (double)n;
+  const double a = 1.0 / sqrt(vb + eps);
+  const double b = -mean * a;
+  for (int64_t e = threadIdx.x; e < n; e += kBlock) {
+    const double t = x[at(e)] * a;
+    y[at(e)] = t + b;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void k_bn_bwd_f64(const double* __restrict__ x, const double* __restrict__ dy,
+                                                       double* __restrict__ dx,
+                                                       const double* __restrict__ save_mean,
+                                                       const double* __restrict__ save_var, int64_t B, int C,
+                                                       int64_t S, double eps, int training) {
+  __shared__ double sh[kBlock];
+  const int c = blockIdx.x;
+  const int64_t n = B * S;
+  auto at = [&](int64_t e) { return ((e / S) * C + c) * S + e % S; };
+  const double mean = save_mean[c];
+  double s = 0.0, dot = 0.0;
+  for (int64_t e = threadIdx.x; e < n; e += kBlock) {
+    const double xv = x[at(e)], g = dy[at(e)];
+    s = s + g;
+    double p;
+    if (S == 1) {
+      const double t = xv - mean;
+      p = t * g;
+    } else {
+      const double t1 = xv * g, t2 = mean * g;
+      p = t1 - t2;
+    }
+    dot = dot + p;
+  }
+  const double sum = block_sum_f64(s, sh);
+  const double dotp = block_sum_f64(dot, sh);
+  const double vb = save_var[c] / (double)n;
+  const double invstd = 1.0 / sqrt(vb + eps);
+  double k = dotp * invstd;
+  k = k * invstd;
+  k = k / (double)n;
+  const double grad_mean = sum / (double)n;
+  for (int64_t e = threadIdx.x; e < n; e += kBlock) {
+    const double xv = x[at(e)], g = dy[at(e)];
+    double out;
+    if (!training) {
+      out = g * invstd;
+    } else {
+      double t = xv - mean;
+      t = t * k;
+      double u;
+      if (S == 1) { u = g - t; u = u - grad_mean; }
+      else { u = g - grad_mean; u = u - t; }
+      out = u * invstd;
+    }
+    dx[at(e)] = out;
   }
 }
 
@@ -223,6 +327,25 @@ int gh_launch_maxpool2d_bwd_f64(gh_ctx* ctx, const gh_cmd& c) {
                      (const double*)(uintptr_t)c.ptr[0], (const double*)(uintptr_t)c.ptr[1],
                      (double*)(uintptr_t)c.ptr[2], g, total);
   return gh_check_hip(ctx, hipGetLastError(), "maxpool backward launch");
+}
+
+int gh_launch_bn_train_f64(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t B = c.dim[0], C = c.dim[1], S = c.dim[2];
+  hipLaunchKernelGGL(k_bn_train_f64, dim3((unsigned)C), dim3(kBlock), 0, ctx->stream,
+                     (const double*)(uintptr_t)c.ptr[0], (double*)(uintptr_t)c.ptr[1],
+                     (double*)(uintptr_t)c.ptr[2], (double*)(uintptr_t)c.ptr[3], (double*)(uintptr_t)c.ptr[4],
+                     (double*)(uintptr_t)c.ptr[5], B, (int)C, S, bits_to_double(c.dim[3]), bits_to_double(c.dim[4]));
+  return gh_check_hip(ctx, hipGetLastError(), "batchnorm training launch");
+}
+
+int gh_launch_bn_bwd_f64(gh_ctx* ctx, const gh_cmd& c) {
+  const int64_t B = c.dim[0], C = c.dim[1], S = c.dim[2];
+  hipLaunchKernelGGL(k_bn_bwd_f64, dim3((unsigned)C), dim3(kBlock), 0, ctx->stream,
+                     (const double*)(uintptr_t)c.ptr[0], (const double*)(uintptr_t)c.ptr[1],
+                     (double*)(uintptr_t)c.ptr[2], (const double*)(uintptr_t)c.ptr[3],
+                     (const double*)(uintptr_t)c.ptr[4], B, (int)C, S, bits_to_double(c.dim[3]),
+                     (c.flags & GH_FLAG_BN_EVAL) ? 0 : 1);
+  return gh_check_hip(ctx, hipGetLastError(), "batchnorm backward launch");
 }
 
 int gh_launch_solver_step_f64(gh_ctx* ctx, const gh_cmd& c) {

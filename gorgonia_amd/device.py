@@ -259,13 +259,14 @@ def cmd_conv2d_bwd_filter(x, dy, dw, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride
                     _conv_dims(B, Cin, H, W, F, kh, kw, pad, stride, dilation))
 
 
-def cmd_bn_train(x, y, run_mean, run_var, save_mean, save_var, B, Cn, S, eps, momentum):
-    return make_cmd(_ffi.OP_BN_TRAIN, 0, (x, y, run_mean, run_var, save_mean, save_var), (B, Cn, S), (eps, momentum))
+def cmd_bn_train(x, y, run_mean, run_var, save_mean, save_var, B, Cn, S, eps, momentum, dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_BN_TRAIN, _ffi.flag_dtype(dtype), (x, y, run_mean, run_var, save_mean, save_var),
+                    (B, Cn, S, _double_bits(eps), _double_bits(momentum)), (eps, momentum))
 
 
-def cmd_bn_bwd(x, dy, dx, save_mean, save_var, B, Cn, S, eps, training=True):
-    return make_cmd(_ffi.OP_BN_BWD, 0 if training else _ffi.FLAG_BN_EVAL, (x, dy, dx, save_mean, save_var),
-                    (B, Cn, S), (eps,))
+def cmd_bn_bwd(x, dy, dx, save_mean, save_var, B, Cn, S, eps, training=True, dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_BN_BWD, (0 if training else _ffi.FLAG_BN_EVAL) | _ffi.flag_dtype(dtype),
+                    (x, dy, dx, save_mean, save_var), (B, Cn, S, _double_bits(eps)), (eps,))
 
 
 def cmd_softmax_bwd(y, dy, dx, rows, cols, dtype=_ffi.F32):
@@ -284,8 +285,8 @@ def cmd_solver_step(kind, w, g, n, par, use, cache=0, cache2=0, dtype=_ffi.F32):
     return make_cmd(_ffi.OP_SOLVER_STEP, fl, (w, g, cache, cache2), (n,), tuple(float(v) for v in par))
 
 
-def cmd_rand_uniform(out, n, seed, offset=0, state=0):
-    return make_cmd(_ffi.OP_RAND_UNIFORM, 0, (out, state), (n, seed, offset))
+def cmd_rand_uniform(out, n, seed, offset=0, state=0, dtype=_ffi.F32):
+    return make_cmd(_ffi.OP_RAND_UNIFORM, _ffi.flag_dtype(dtype), (out, state), (n, seed, offset))
 
 
 def cmd_dropout(x, y, r, n, prob, training=True, dtype=_ffi.F32):

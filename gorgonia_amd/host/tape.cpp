@@ -472,16 +472,21 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     case OpKind::BatchNormTrain:
     case OpKind::BatchNormDiff: {
       const Tensor& x = *in[0];
-      if (x.dt != Dtype::Float32) return bad("BatchNorm: Unsupported Dtype");
+      if (x.dt == Dtype::Other) return bad("BatchNorm: Unsupported Dtype");
+      for (size_t i = 1; i < in.size(); i++)
+        if (in[i]->dt != x.dt) return bad("BatchNorm: Unsupported Dtype");
       gh_cmd c{};
       const int64_t B = x.shape[0], C = x.shape[1];
+      c.flags = dtype_flag(x.dt);
       c.dim[0] = B; c.dim[1] = C; c.dim[2] = x.shape.TotalSize() / (B * C);
       c.f[0] = (float)op.f0;
+      c.dim[3] = double_bits(op.f0);   // float64: epsilon (and momentum below) as doubles
       if (op.kind == OpKind::BatchNormTrain) {
         c.opcode = GH_OP_BN_TRAIN;
         c.ptr[0] = x.mem; c.ptr[1] = prealloc.mem;
         for (int i = 0; i < 4; i++) c.ptr[2 + i] = in[(size_t)(1 + i)]->mem;
         c.f[1] = (float)op.f1;
+        c.dim[4] = double_bits(op.f1);
       } else {
         c.opcode = GH_OP_BN_BWD;
         c.ptr[0] = x.mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;

@@ -192,7 +192,8 @@ enum gh_unaryfn {
  *             GH_FLAG_DTYPE(GH_F64); their scalars then travel as the bit pattern of a double
  *             in a dim slot (LEAKY_RELU alpha: dim[1]; BN_INFER epsilon: dim[3]; DROPOUT and
  *             DROPOUT_BWD probability: dim[1]; SOLVER_STEP's ten constants: dim[1..10]).
- *             BN_TRAIN, BN_BWD and RAND_UNIFORM are float32 only
+ *             BN_TRAIN (epsilon dim[3], momentum dim[4]), BN_BWD (epsilon dim[3]) and
+ *             RAND_UNIFORM (53 random bits: the top 53 of the same 64-bit value) likewise
  * RAND_UNIFORM ptr[0]=out [ptr[1]=state]          dim[0]=n dim[1]=seed dim[2]=offset
  *             float32 in [0,1) with 24 random bits, element i = SplitMix64 output function
  *             of seed*0xD1342543DE82EF95 + (offset + i + 1)*0x9E3779B97F4A7C15.  With a

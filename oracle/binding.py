@@ -308,28 +308,38 @@ def conv2d_bwd_direct_f64(x, w, dy, pad=(0, 0), stride=(1, 1), dil=(1, 1)):
 
 def bn_train_stats(x, run_mean, run_var, momentum, eps):
     """Training-mode forward; returns (y, running_mean, running_var, save_mean, save_var_sum)."""
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    dt = _ft(x)
+    x = np.ascontiguousarray(x, dtype=dt)
     B, Cn = x.shape[:2]
     S = x.size // (B * Cn)
     y = np.empty_like(x)
-    rm = np.array(run_mean, dtype=np.float32, copy=True)
-    rv = np.array(run_var, dtype=np.float32, copy=True)
-    sm, sv = np.empty(Cn, np.float32), np.empty(Cn, np.float32)
-    lib().oracle_bn_train_stats_f32(_p(x), _p(y), _p(rm), _p(rv), _p(sm), _p(sv), C.c_float(momentum),
-                                    C.c_float(eps), *_i64(B, Cn, S))
+    rm = np.array(run_mean, dtype=dt, copy=True)
+    rv = np.array(run_var, dtype=dt, copy=True)
+    sm, sv = np.empty(Cn, dt), np.empty(Cn, dt)
+    if dt == np.float64:
+        lib().oracle_bn_train_stats_f64(_p(x), _p(y), _p(rm), _p(rv), _p(sm), _p(sv), C.c_double(momentum),
+                                        C.c_double(eps), *_i64(B, Cn, S))
+    else:
+        lib().oracle_bn_train_stats_f32(_p(x), _p(y), _p(rm), _p(rv), _p(sm), _p(sv), C.c_float(momentum),
+                                        C.c_float(eps), *_i64(B, Cn, S))
     return y, rm, rv, sm, sv
 
 
 def bn_bwd(x, dy, save_mean, save_var, eps, training=True):
-    x = np.ascontiguousarray(x, dtype=np.float32)
-    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    dt = _ft(x)
+    x = np.ascontiguousarray(x, dtype=dt)
+    dy = np.ascontiguousarray(dy, dtype=dt)
     B, Cn = x.shape[:2]
     S = x.size // (B * Cn)
     dx = np.empty_like(x)
-    sm = np.ascontiguousarray(save_mean, dtype=np.float32)
-    sv = np.ascontiguousarray(save_var, dtype=np.float32)
-    lib().oracle_bn_bwd_f32(_p(x), _p(dy), _p(dx), _p(sm), _p(sv), C.c_float(eps), C.c_int(int(training)),
-                            *_i64(B, Cn, S))
+    sm = np.ascontiguousarray(save_mean, dtype=dt)
+    sv = np.ascontiguousarray(save_var, dtype=dt)
+    if dt == np.float64:
+        lib().oracle_bn_bwd_f64(_p(x), _p(dy), _p(dx), _p(sm), _p(sv), C.c_double(eps), C.c_int(int(training)),
+                                *_i64(B, Cn, S))
+    else:
+        lib().oracle_bn_bwd_f32(_p(x), _p(dy), _p(dx), _p(sm), _p(sv), C.c_float(eps), C.c_int(int(training)),
+                                *_i64(B, Cn, S))
     return dx
 
 
@@ -394,9 +404,10 @@ def dropout_bwd(y, dy, prob):
     return dx
 
 
-def uniform01(n, seed, offset=0):
-    out = np.empty(n, np.float32)
-    lib().oracle_uniform01_f32(_p(out), C.c_int64(n), C.c_uint64(seed), C.c_uint64(offset))
+def uniform01(n, seed, offset=0, dtype=np.float32):
+    out = np.empty(n, dtype)
+    (lib().oracle_uniform01_f64 if out.dtype == np.float64 else lib().oracle_uniform01_f32)(
+        _p(out), C.c_int64(n), C.c_uint64(seed), C.c_uint64(offset))
     return out
 
 

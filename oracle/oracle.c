@@ -973,6 +973,18 @@ EXPORT void oracle_uniform01_f32(float* out, int64_t n, uint64_t seed, uint64_t 
   }
 }
 
+/* The float64 form keeps the top 53 bits of the same 64-bit value. */
+EXPORT void oracle_uniform01_f64(double* out, int64_t n, uint64_t seed, uint64_t offset) {
+  int64_t i;
+  for (i = 0; i < n; i++) {
+    uint64_t z = seed * 0xD1342543DE82EF95ull + (offset + (uint64_t)i + 1) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z = z ^ (z >> 31);
+    out[i] = (double)(z >> 11) * 1.1102230246251565e-16;
+  }
+}
+
 /* ------------------------------------------------------------------ */
 EXPORT void oracle_softmax_f32(const float* x, float* y, int64_t rows, int64_t cols) {
   int64_t r, j;
@@ -1150,6 +1162,91 @@ EXPORT void oracle_maxpool2d_bwd_f64(const double* x, const double* dy, double* 
           for (wi = ws; wi < we; wi++)
             if (in[hi * W + wi] > best) { best = in[hi * W + wi]; arg = hi * W + wi; }
         if (arg >= 0) out[arg] = out[arg] + g[ph * ow + pw];
+      }
+  }
+}
+
+EXPORT void oracle_bn_train_stats_f64(const double* x, double* y, double* run_mean, double* run_var,
+                                      double* save_mean, double* save_var, double momentum,
+                                      double eps, int64_t B, int64_t C, int64_t S) {
+  int64_t n = B * S, c;
+  for (c = 0; c < C; c++) {
+    double mean = 0.0, var = 0.0;
+    int64_t s, d;
+    for (s = 0; s < B; s++)
+      for (d = 0; d < S; d++) mean = mean + x[(s * C + c) * S + d];
+    mean = mean / (double)n;
+    for (s = 0; s < B; s++)
+      for (d = 0; d < S; d++) {
+        double t = x[(s * C + c) * S + d] - mean;
+        double t2 = t * t;
+        var = var + t2;
+      }
+    save_mean[c] = mean;
+    save_var[c] = var;
+    {
+      double m1 = momentum * mean;
+      double m2 = (1.0 - momentum) * run_mean[c];
+      run_mean[c] = m1 + m2;
+      double unb = var / (double)(n - 1);
+      double v1 = momentum * unb;
+      double v2 = (1.0 - momentum) * run_var[c];
+      run_var[c] = v1 + v2;
+    }
+    double vb = var / (double)n;
+    double a = 1.0 / sqrt(vb + eps);
+    double b = -mean * a;
+    for (s = 0; s < B; s++)
+      for (d = 0; d < S; d++) {
+        int64_t i = (s * C + c) * S + d;
+        double t = x[i] * a;
+        y[i] = t + b;
+      }
+  }
+}
+
+EXPORT void oracle_bn_bwd_f64(const double* x, const double* dy, double* dx, const double* save_mean,
+                              const double* save_var, double eps, int training, int64_t B,
+                              int64_t C, int64_t S) {
+  int64_t n = B * S, c;
+  for (c = 0; c < C; c++) {
+    double dotp = 0.0, sum = 0.0;
+    int64_t s, d;
+    const double mean = save_mean[c];
+    for (s = 0; s < B; s++)
+      for (d = 0; d < S; d++) {
+        int64_t i = (s * C + c) * S + d;
+        sum = sum + dy[i];
+        double partial;
+        if (S == 1) {
+          double t = x[i] - mean;
+          partial = t * dy[i];
+        } else {
+          double t1 = x[i] * dy[i];
+          double t2 = mean * dy[i];
+          partial = t1 - t2;
+        }
+        dotp = dotp + partial;
+      }
+    double vb = save_var[c] / (double)n;
+    double invstd = 1.0 / sqrt(vb + eps);
+    double kk = dotp * invstd;
+    kk = kk * invstd;
+    kk = kk / (double)n;
+    double gradMean = sum / (double)n;
+    for (s = 0; s < B; s++)
+      for (d = 0; d < S; d++) {
+        int64_t i = (s * C + c) * S + d;
+        if (training) {
+          double t = x[i] - mean;
+          t = t * kk;
+          double u;
+          if (S == 1) { u = dy[i] - t; u = u - gradMean; }
+          else { u = dy[i] - gradMean; u = u - t; }
+          dx[i] = u * invstd;
+        } else {
+          dx[i] = dy[i] * invstd;
+        }
       }
   }
 }

@@ -116,9 +116,24 @@ def test_float64_flags_validate(ctx):
     assert ctx.lib.gh_validate(C.byref(ok), 1, buf, 256) == 0
     bad = D.cmd_dropout(1, 2, 3, 10, 1.5, dtype=F64)
     assert ctx.lib.gh_validate(C.byref(bad), 1, buf, 256) != 0 and b"probability" in buf.value
-    for cmd in (D.cmd_bn_train(1, 2, 3, 4, 5, 6, 2, 4, 4, 1e-5, 0.9),):
-        cmd.flags |= _ffi.flag_dtype(F64)
-        assert ctx.lib.gh_validate(C.byref(cmd), 1, buf, 256) != 0 and b"float32 only" in buf.value
+    assert ctx.lib.gh_validate(C.byref(D.cmd_rand_uniform(1, 10, 3, dtype=F64)), 1, buf, 256) == 0
+
+
+def test_uniform_source_float64(ctx):
+    """53-bit uniform numbers: bit-identical to the oracle's twin, the float32 stream's values
+    are their top 24 bits, and a device-side counter moves the stream on."""
+    n = 10007
+    out = ctx.malloc(n * 8)
+    ctx.run(D.cmd_rand_uniform(out, n, 12345, 77, dtype=F64))
+    got = ctx.d2h(out, (n,), np.float64)
+    assert_bits_equal(got, O.uniform01(n, 12345, 77, dtype=np.float64), "float64 uniform stream")
+    assert np.all((got >= 0) & (got < 1)) and abs(got.mean() - 0.5) < 0.02
+    assert np.array_equal(np.floor(got * 2**24) / 2**24, O.uniform01(n, 12345, 77).astype(np.float64))
+    state = ctx.upload(np.array([5], np.uint64).view(np.float64))
+    ctx.run(D.cmd_rand_uniform(out, 100, 9, state=state, dtype=F64))
+    ctx.run(D.cmd_rand_uniform(out, 100, 9, state=state, dtype=F64))
+    assert_bits_equal(ctx.d2h(out, (100,), np.float64), O.uniform01(100, 9, 105, dtype=np.float64), "second draw")
+    ctx.free(out); ctx.free(state)
 
 
 def test_float64_training_ops_on_the_tape(ctx):
@@ -194,3 +209,30 @@ def test_conv_gradients_float64(ctx, cfg):
             assert np.linalg.norm(dw - dw_ref) <= 1e-12 * np.linalg.norm(dw_ref)
         for p in (px, pw, pdy, pdx, pdw):
             ctx.free(p)
+
+
+@pytest.mark.parametrize("shape", [(8, 5, 6, 7), (4, 16, 14, 14), (64, 10), (3, 2, 1, 1)])
+def test_batchnorm_training_and_gradient_float64(ctx, shape):
+    """BN_TRAIN and BN_BWD in float64 against the oracle's twins: relative error <= 1e-12
+    (the device sums a channel by a tree, the oracle in sequence)."""
+    B, Cn = shape[:2]
+    S = int(np.prod(shape[2:])) if len(shape) > 2 else 1
+    x, dy = _rand(31, shape), _rand(32, shape)
+    rm, rv = _rand(33, (Cn,)), np.random.default_rng(34).random(Cn) + 0.5
+    y_ref, rm_ref, rv_ref, sm_ref, sv_ref = O.bn_train_stats(x, rm, rv, 0.9, 1e-5)
+    px, py, prm, prv = _up(ctx, x), ctx.malloc(x.size * 8), _up(ctx, rm), _up(ctx, rv)
+    psm, psv = ctx.malloc(Cn * 8), ctx.malloc(Cn * 8)
+    ctx.run(D.cmd_bn_train(px, py, prm, prv, psm, psv, B, Cn, S, 1e-5, 0.9, dtype=F64))
+    close = lambda a, b: np.linalg.norm(a - b) <= 1e-12 * max(np.linalg.norm(b), 1e-300)
+    assert close(ctx.d2h(py, shape, np.float64), y_ref)
+    assert close(ctx.d2h(prm, (Cn,), np.float64), rm_ref) and close(ctx.d2h(prv, (Cn,), np.float64), rv_ref)
+    sm, sv = ctx.d2h(psm, (Cn,), np.float64), ctx.d2h(psv, (Cn,), np.float64)
+    assert close(sm, sm_ref) and close(sv, sv_ref)
+    pdy, pdx = _up(ctx, dy), ctx.malloc(x.size * 8)
+    for training in (True, False):
+        ctx.run(D.cmd_bn_bwd(px, pdy, pdx, psm, psv, B, Cn, S, 1e-5, training, dtype=F64))
+        want = O.bn_bwd(x, dy, sm, sv, 1e-5, training)
+        got = ctx.d2h(pdx, shape, np.float64)
+        assert np.linalg.norm(got - want) <= 1e-10 * max(np.linalg.norm(want), 1e-300), (training, shape)
+    for p in (px, py, prm, prv, psm, psv, pdy, pdx):
+        ctx.free(p)

@@ -375,3 +375,34 @@ def test_float64_conv_gradients_against_the_float32_oracle():
         dx64, dw64 = O.conv2d_bwd(xr.astype(np.float64), wr.astype(np.float64), dyr.astype(np.float64), pad, stride, dil)
         assert np.linalg.norm(dx64 - dx32) <= 1e-5 * np.linalg.norm(dx64)
         assert np.linalg.norm(dw64 - dw32) <= 1e-5 * np.linalg.norm(dw64)
+
+
+def test_float64_batchnorm_training_twins_against_the_float32_oracle():
+    """The float64 BatchNorm training forward and gradient agree with the pinned float32 oracle
+    within float32 rounding, and the gradient is the derivative of the training forward."""
+    rng = np.random.default_rng(8)
+    for shape in [(6, 3, 4, 5), (16, 7)]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        dy = rng.standard_normal(shape).astype(np.float32)
+        Cn = shape[1]
+        rm, rv = rng.standard_normal(Cn).astype(np.float32), (rng.random(Cn) + 0.5).astype(np.float32)
+        out32 = O.bn_train_stats(x, rm, rv, 0.9, 1e-5)
+        out64 = O.bn_train_stats(x.astype(np.float64), rm.astype(np.float64), rv.astype(np.float64), 0.9, 1e-5)
+        for a, b in zip(out64, out32):
+            assert a.dtype == np.float64
+            np.testing.assert_allclose(a, b, rtol=2e-5, atol=2e-5)
+        for training in (True, False):
+            d32 = O.bn_bwd(x, dy, out32[3], out32[4], 1e-5, training)
+            d64 = O.bn_bwd(x.astype(np.float64), dy.astype(np.float64), out64[3], out64[4], 1e-5, training)
+            np.testing.assert_allclose(d64, d32, rtol=1e-4, atol=2e-5)
+        # finite differences of the float64 training forward: d/dx sum(y * dy)
+        x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+        grad = O.bn_bwd(x64, dy64, out64[3], out64[4], 1e-5, True)
+        idx = tuple(int(v) // 2 for v in shape)
+        h = 1e-6
+        xp, xm = x64.copy(), x64.copy()
+        xp[idx] += h
+        xm[idx] -= h
+        fp = (O.bn_train_stats(xp, rm, rv, 0.9, 1e-5)[0] * dy64).sum()
+        fm = (O.bn_train_stats(xm, rm, rv, 0.9, 1e-5)[0] * dy64).sum()
+        assert abs((fp - fm) / (2 * h) - grad[idx]) <= 1e-6 * max(1.0, abs(grad[idx]))
