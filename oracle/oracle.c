@@ -56,11 +56,13 @@
  *                                            itself is not vendored: PARITY
  *                                            UNPINNED bit-for-bit.
  *   float64 twins (forward NN operators,   - each against its pinned float32
- *   max-pool / softmax backward, dropout,    counterpart: equal on inputs whose
- *   solver steps)                            float32 arithmetic is exact, within
- *                                            float32 rounding elsewhere; the
- *                                            reference's float64 goldens where it
- *                                            has them (max pool, softmax)
+ *   conv / max-pool / batch-norm / softmax   counterpart: equal on inputs whose
+ *   gradients, dropout, solver steps)        float32 arithmetic is exact, within
+ *                                            float32 rounding elsewhere (plus
+ *                                            finite differences for batch norm);
+ *                                            the reference's float64 goldens where
+ *                                            it has them (max pool, softmax)
+ *   uniform01 float64                      - its top 24 bits are the float32 stream
  */
 #include <math.h>
 #include <stdint.h>

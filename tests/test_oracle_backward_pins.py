@@ -406,3 +406,13 @@ def test_float64_batchnorm_training_twins_against_the_float32_oracle():
         fp = (O.bn_train_stats(xp, rm, rv, 0.9, 1e-5)[0] * dy64).sum()
         fm = (O.bn_train_stats(xm, rm, rv, 0.9, 1e-5)[0] * dy64).sum()
         assert abs((fp - fm) / (2 * h) - grad[idx]) <= 1e-6 * max(1.0, abs(grad[idx]))
+
+
+def test_uniform_source_float64_extends_the_float32_stream():
+    """The 53-bit numbers are the same stream at a finer grain: their top 24 bits are the float32
+    values (which are pinned to the synthetic-input generator)."""
+    u64 = O.uniform01(5000, 42, 7, dtype=np.float64)
+    u32 = O.uniform01(5000, 42, 7)
+    assert u64.dtype == np.float64 and np.all((u64 >= 0) & (u64 < 1))
+    assert np.array_equal(np.floor(u64 * 2**24) / 2**24, u32.astype(np.float64))
+    assert len(np.unique(u64)) == 5000
