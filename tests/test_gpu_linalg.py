@@ -50,6 +50,32 @@ def test_matmul_vs_oracle(ctx, ta, tb):
         assert rel_frobenius(O.gemm(A, B, ta, tb), ref) <= TOL
 
 
+def test_matmul_small_output_shapes_sweep(ctx):
+    """Seeded sweep over the shapes the small-output kernels take (few output tiles, K from 32
+    up, ragged everything, transposed views): every product against the float64 one, and on
+    integer-valued operands exactly."""
+    rng = np.random.default_rng(2024)
+    for case in range(60):
+        m = int(rng.integers(1, 200))
+        n = int(rng.integers(1, 200))
+        k = int(rng.integers(32, 700))
+        ta, tb = [(False, False), (True, False), (False, True), (True, True)][case % 4]
+        integer = case % 3 == 0
+        if integer:
+            A = rng.integers(-4, 5, (k, m) if ta else (m, k)).astype(np.float32)
+            B = rng.integers(-4, 5, (n, k) if tb else (k, n)).astype(np.float32)
+        else:
+            A = synth.normal(1000 + case, (k, m) if ta else (m, k))
+            B = synth.normal(2000 + case, (n, k) if tb else (k, n))
+        got = _run_gemm(ctx, A, B, ta, tb)
+        ref = O.gemm_f64acc(A, B, ta, tb)
+        if integer:
+            assert np.array_equal(got, ref.astype(np.float32)), f"case {case}: {m}x{k}x{n} ta={ta} tb={tb}"
+        else:
+            err = rel_frobenius(got, ref)
+            assert err <= TOL, f"case {case}: {m}x{k}x{n} ta={ta} tb={tb}: {err:.3e}"
+
+
 def test_matmul_integer_exact(ctx):
     """Small-integer inputs: every partial sum is exactly representable, so any
     accumulation order must give the oracle's bits."""
