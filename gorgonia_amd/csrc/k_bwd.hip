@@ -103,6 +103,43 @@ __global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2_bwd(const float* __res
   }
 }
 
+// 2x2 / stride 2 / no padding at any H, W (odd sizes, rows that are no multiple of
+// four): one thread per window with scalar accesses; the thread of the last
+// window column / row also zeroes the column / row an odd size leaves outside
+// every window.  Same scan order, strict > and "0 + dy" as above.
+__global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2_bwd_any(const float* __restrict__ x,
+                                                                  const float* __restrict__ dy,
+                                                                  float* __restrict__ dx, int H, int W,
+                                                                  int64_t windows) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  const int oh = H / 2, ow = W / 2;
+  for (int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x; idx < windows; idx += stride) {
+    const int pw = (int)(idx % ow);
+    const int64_t row = idx / ow;
+    const int ph = (int)(row % oh);
+    const int64_t bc = row / oh;
+    const int64_t at = (bc * H + 2 * ph) * (int64_t)W + 2 * pw;
+    const float v00 = x[at], v01 = x[at + 1], v10 = x[at + W], v11 = x[at + W + 1];
+    float best = -FLT_MAX;
+    int arg = -1;
+    if (v00 > best) { best = v00; arg = 0; }
+    if (v01 > best) { best = v01; arg = 1; }
+    if (v10 > best) { best = v10; arg = 2; }
+    if (v11 > best) { best = v11; arg = 3; }
+    const float v = 0.0f + dy[idx];
+    dx[at] = arg == 0 ? v : 0.0f;
+    dx[at + 1] = arg == 1 ? v : 0.0f;
+    dx[at + W] = arg == 2 ? v : 0.0f;
+    dx[at + W + 1] = arg == 3 ? v : 0.0f;
+    if ((W & 1) && pw == ow - 1) { dx[at + 2] = 0.0f; dx[at + W + 2] = 0.0f; }
+    if ((H & 1) && ph == oh - 1) {
+      dx[at + 2 * (int64_t)W] = 0.0f;
+      dx[at + 2 * (int64_t)W + 1] = 0.0f;
+      if ((W & 1) && pw == ow - 1) dx[at + 2 * (int64_t)W + 2] = 0.0f;
+    }
+  }
+}
+
 // ---- BatchNorm: per-channel reductions ----------------------------------------------
 // A channel's n = B*S values are split over G workgroups; each reduces its share
 // with a fixed tree (so results repeat run to run), the consumers add the G
@@ -488,6 +525,16 @@ int gh_launch_maxpool2d_bwd(gh_ctx* ctx, const gh_cmd& c) {
     hipLaunchKernelGGL(k_maxpool_2x2s2_bwd, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
                        (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
                        (float*)(uintptr_t)c.ptr[2], g.H, g.W, pairs);
+    return gh_check_hip(ctx, hipGetLastError(), "maxpool backward launch");
+  }
+  if (g.kh == 2 && g.kw == 2 && g.strideH == 2 && g.strideW == 2 && g.padH == 0 && g.padW == 0 && !explicit_pad &&
+      padS == 0 && padE == 0 && g.H >= 2 && g.W >= 2) {
+    const int64_t windows = B * C * (int64_t)g.oh * g.ow;
+    int64_t blocks = (windows + kBlock - 1) / kBlock;
+    if (blocks > (int64_t)ctx->cu_count * 64) blocks = (int64_t)ctx->cu_count * 64;
+    hipLaunchKernelGGL(k_maxpool_2x2s2_bwd_any, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
+                       (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                       (float*)(uintptr_t)c.ptr[2], g.H, g.W, windows);
     return gh_check_hip(ctx, hipGetLastError(), "maxpool backward launch");
   }
   int64_t blocks = (total + kBlock - 1) / kBlock;

@@ -25,6 +25,11 @@ POOL_CASES = [
     (2, 3, 12, 9, (3, 3), (1, 1), (2, 2)),
     (1, 2, 7, 8, (3, 2), (1, 1), (1, 2)),
     (16, 32, 28, 28, (2, 2), (0, 0), (2, 2)),        # convnet pool 0 (batch trimmed)
+    (8, 16, 14, 14, (2, 2), (0, 0), (2, 2)),         # convnet pool 1: rows of 14 (no multiple of four)
+    (8, 16, 7, 7, (2, 2), (0, 0), (2, 2)),           # convnet pool 2: odd size, last row and column unpooled
+    (1, 1, 2, 3, (2, 2), (0, 0), (2, 2)),
+    (1, 2, 3, 2, (2, 2), (0, 0), (2, 2)),
+    (1, 1, 2, 2, (2, 2), (0, 0, 0, 0), (2, 2)),      # explicit four-value padding of zero
 ]
 
 
