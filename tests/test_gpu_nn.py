@@ -191,6 +191,37 @@ def test_conv_epilogue_pool_bit_exact(ctx, cfg):
                                     pool2=True), chain, f"conv+bn+leaky+pool {cfg}")
 
 
+def test_conv_random_geometry_sweep(ctx):
+    """Seeded sweep over 3x3 and other geometries (all three convolution kernels, ragged sizes,
+    batch boundaries inside blocks): the plain convolution against the oracle, and wherever the
+    pool may ride in the epilogue, conv+ReLU+pool against the separate commands bit for bit."""
+    rng = np.random.default_rng(77)
+    pooled = 0
+    for case in range(36):
+        B = int(rng.integers(1, 7))
+        C = int(rng.choice([1, 3, 4, 8, 16, 24, 40]))
+        H, W = int(rng.integers(3, 34)), int(rng.integers(3, 34))
+        F = int(rng.integers(1, 90))
+        k = 3 if case % 5 else int(rng.choice([1, 2, 5]))
+        pad = int(rng.integers(0, 2)) if k == 3 else int(rng.integers(0, k))
+        if H + 2 * pad < k or W + 2 * pad < k:
+            continue
+        x = synth.uniform(3000 + case, (B, C, H, W), -1, 1)
+        w = synth.he_normal(4000 + case, (F, C, k, k))
+        got = gpu_conv(ctx, x, w, (pad, pad), (1, 1), (1, 1))
+        ref = O.conv2d(x, w, (pad, pad), (1, 1), (1, 1))
+        err = rel_frobenius(got, ref)
+        assert err <= TOL, f"case {case}: B{B} C{C} {H}x{W} F{F} k{k} pad{pad}: {err:.3e}"
+        cmd = D.cmd_conv2d(1, 1, 1, B, C, H, W, F, k, k, (pad, pad))
+        if k == 3 and ctx.lib.gh_conv2d_can_pool(cmd) == 1:
+            pooled += 1
+            act = gpu_conv(ctx, x, w, (pad, pad), (1, 1), (1, 1), act="relu")
+            want = gpu_pool(ctx, act, (2, 2), (0, 0), (2, 2))
+            assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), act="relu", pool2=True), want,
+                              f"case {case}: conv+relu+pool B{B} C{C} {H}x{W} F{F} pad{pad}")
+    assert pooled >= 8
+
+
 def test_conv_pool_flag_needs_a_pooling_kernel(ctx):
     # 13 rows of 13: no block of at most 128 pixels holds a whole image
     cmd = D.cmd_conv2d(0x1000, 0x2000, 0x3000, 2, 8, 13, 13, 16, 3, 3, (1, 1), pool2=True)
