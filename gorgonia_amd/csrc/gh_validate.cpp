@@ -62,8 +62,8 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (dt == GH_F64 && (c.flags & (GH_FLAG_ACT_RELU | GH_FLAG_ACT_LEAKY)))
         return bad("gemm: no fused activation for float64");
       if (dt == GH_F64 && batch > 65535) return bad("gemm: batch too large");
-      if ((c.flags & GH_FLAG_GEMM_BIAS) && (dt != GH_F32 || !c.ptr[3]))
-        return bad("gemm: the fused row bias is float32 only and needs ptr[3]");
+      if ((c.flags & GH_FLAG_GEMM_BIAS) && (dt != GH_F32 || !c.ptr[3] || ta || tb))
+        return bad("gemm: the fused row bias is float32 only, takes untransposed operands and needs ptr[3]");
       if ((c.flags & GH_FLAG_GEMM_SOFTMAX) && !gh_gemm_can_softmax(&c))
         return bad("gemm: no fused softmax for this shape (see gh_gemm_can_softmax)");
       return GH_OK;

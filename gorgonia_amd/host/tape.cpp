@@ -639,6 +639,7 @@ int Graph::FuseActivations() {
     if (k == OpKind::BroadcastBin) {
       // Add(Mul(x, w), b) with b one value per column: a + b and b + a are the same bits
       if (op.kind != OpKind::MatMul || has_act || op.fuse_bias || n.inputs.size() != 2 || n.shape.Dims() != 2) continue;
+      if (op.transA || op.transB) continue;   // the bias epilogue exists for untransposed products
       const Node& small = nodes_[(size_t)(pi == n.inputs[0] ? n.inputs[1] : n.inputs[0])];
       if (small.dt != Dtype::Float32 || small.shape.Dims() != 2 || small.shape[0] != 1 || small.shape[1] != n.shape[1] ||
           n.shape[0] == 1)

@@ -133,7 +133,7 @@ enum gh_unaryfn {
 #define GH_FLAG_BN_EVAL      (1u << 26)   /* BN_BWD: eval-mode gradient dy/sqrt(var+eps)       */
 #define GH_FLAG_CONV_POOL2   (1u << 25)   /* CONV2D: 2x2 stride-2 unpadded MaxPool2D on the result */
 #define GH_FLAG_GEMM_SOFTMAX (1u << 27)   /* GEMM: row SoftMax on the result (after the activation) */
-#define GH_FLAG_GEMM_BIAS    (1u << 28)   /* GEMM: ptr[3] = N floats added to every row of the product (before the activation) */
+#define GH_FLAG_GEMM_BIAS    (1u << 28)   /* GEMM (untransposed): ptr[3] = N floats added to every row of the product (before the activation) */
 
 /*
  * One operator.  Field use per opcode:
