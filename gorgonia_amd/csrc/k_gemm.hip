@@ -1198,6 +1198,10 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_lds(const float* __restric
 // the epilogue.  With WS == 2 the stored pixel is the 2x2/stride-2 max-pool
 // window of four convolution results (scan order and strict > of the pooling
 // kernel), which cuts the bytes written by four.
+// (The same shapes on the 16x16x4 MFMA - one wavefront per 16 stored pixels,
+// each lane fetching its own tap per step from x - were measured slower: 59 us
+// against 41 on 8x3x416x416 -> 16; the per-tap address arithmetic and bounds
+// tests cost more than the matrix cores save at K = 27.)
 template <int C, int WS>
 __global__ __launch_bounds__(256) void k_conv3x3_direct(const float* __restrict__ x,
                                                         const float* __restrict__ w,
