@@ -136,9 +136,9 @@ def bench_linalg(ctx, iters):
 # WRITE_SIZE runs of this script (KiB per dispatch; FETCH_SIZE scaled by 2.0,
 # WRITE_SIZE by 1.0, the factors a 64 MiB device copy in the same runs gives).
 MEASURED_TRAFFIC_BYTES = {
-    "conv0": (2 * 931.8 + 3232.0) * 1024,
-    "conv1": (2 * 4352.7 + 2464.0) * 1024,
-    "conv2": (2 * 2110.9 + 576.0) * 1024,
+    "conv0": (2 * 935.4 + 3232.0) * 1024,
+    "conv1": (2 * 4350.2 + 2464.0) * 1024,
+    "conv2": (2 * 2108.9 + 576.0) * 1024,
 }
 
 CONVNET_LAYERS = [  # (name, B-relative shape) of configuration 4
