@@ -234,13 +234,13 @@ def bench_convnet_machines(steps, warmup, count=2, batch=128):
     return count * steps * batch / dt, results
 
 
-def bench_yolo(steps, warmup):
+def bench_yolo(steps, warmup, resident_input=True):
     """Config 5: Tiny-YOLO-v2-shaped forward, batch 8 x 3 x 416 x 416, on the tape
     machine with conv+BatchNorm+LeakyReLU(+MaxPool) folded, graph replay,
     weights and input resident."""
     from gorgonia_amd import configs, graph as G
     inp = configs.yolo_inputs(8, 416)
-    g, outs = configs.build_yolo(inp, resident_input=True)
+    g, outs = configs.build_yolo(inp, resident_input=resident_input)
     m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING, fuse_activations=True)
     for _ in range(max(warmup, 3)):
         m.RunAll()
@@ -256,13 +256,13 @@ def bench_yolo(steps, warmup):
     return dt / steps * 1e3, result, inp
 
 
-def bench_mlp(steps, warmup):
+def bench_mlp(steps, warmup, resident_input=True):
     """Config 1: MLP 256 x 784 -> 300 -> 100 -> 10 forward on the tape machine (three
     dense layers, ReLU and SoftMax folded into the products' epilogues), graph replay,
     weights and input resident."""
     from gorgonia_amd import configs, graph as G
     inp = configs.mlp_inputs(256)
-    g, outs = configs.build_mlp(inp, resident_input=True)
+    g, outs = configs.build_mlp(inp, resident_input=resident_input)
     m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING, fuse_activations=True)
     for _ in range(max(warmup, 3)):
         m.RunAll()
@@ -422,14 +422,18 @@ def main():
     yolo = None
     if not only or "yolo" in only:
         ms_yolo, yolo_out, yolo_inp = bench_yolo(max(20, a.steps // 4), a.warmup)
+        ms_yolo_h2d, _, _ = bench_yolo(max(10, a.steps // 8), a.warmup, resident_input=False)
         yolo = {"ms_per_step": round(ms_yolo, 4), "images_s": round(8 / ms_yolo * 1e3, 1),
-                "TFLOPs": round(31_080_857_600 / ms_yolo / 1e9, 2), "flop_per_step": 31_080_857_600}
+                "TFLOPs": round(31_080_857_600 / ms_yolo / 1e9, 2), "flop_per_step": 31_080_857_600,
+                "ms_per_step_with_input_h2d": round(ms_yolo_h2d, 4)}
         log(f"yolo-shaped: {ms_yolo:.4f} ms/step  {8 / ms_yolo * 1e3:.0f} images/s")
 
     mlp = None
     if not only or "mlp" in only:
         ms_mlp, mlp_out, mlp_inp = bench_mlp(a.steps, a.warmup)
-        mlp = {"ms_per_step": round(ms_mlp, 5), "images_s": round(256 / ms_mlp * 1e3, 1), "flop_per_step": 136_294_400}
+        ms_mlp_h2d, _, _ = bench_mlp(max(20, a.steps // 4), a.warmup, resident_input=False)
+        mlp = {"ms_per_step": round(ms_mlp, 5), "images_s": round(256 / ms_mlp * 1e3, 1), "flop_per_step": 136_294_400,
+               "ms_per_step_with_input_h2d": round(ms_mlp_h2d, 5)}
         log(f"mlp: {ms_mlp:.4f} ms/step  {256 / ms_mlp * 1e3:.0f} rows/s")
 
     train = None
