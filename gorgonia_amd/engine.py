@@ -53,6 +53,10 @@ HOST_SYMBOLS = {
     "ghh_engine_put": (C.c_int, [_P, C.c_uint64, C.c_int64]),
     "ghh_engine_reset_allocator": (C.c_int, [_P]),
     "ghh_engine_alloc_accessible": (C.c_int, [_P]),
+    "ghh_engine_memset": (C.c_int, [_P, C.c_uint64, _P]),
+    "ghh_engine_memclr": (C.c_int, [_P, C.c_uint64]),
+    "ghh_engine_accessible": (C.c_int, [_P, C.c_uint64, _P]),
+    "ghh_engine_alloc_flags": (C.c_int, [_P, _P]),
     "ghh_engine_memcpy": (C.c_int, [_P, C.c_uint64, C.c_int64, C.c_uint64, C.c_int64]),
     "ghh_engine_h2d": (C.c_int, [_P, C.c_uint64, _P, C.c_int64]),
     "ghh_engine_d2h": (C.c_int, [_P, _P, C.c_uint64, C.c_int64]),
@@ -205,6 +209,29 @@ class Engine:
 
     def AllocAccessible(self):
         return bool(self.lib.ghh_engine_alloc_accessible(self.h))
+
+    def AllocFlags(self):
+        """(manually managed, column-major tag): cuda/engine.go:81-83."""
+        out = (C.c_int32 * 2)()
+        self.lib.ghh_engine_alloc_flags(self.h, C.byref(out))
+        return bool(out[0]), bool(out[1])
+
+    def Memset(self, mem, val=None):
+        self._check(self.lib.ghh_engine_memset(self.h, int(mem), None))
+
+    def Memclr(self, mem):
+        self._check(self.lib.ghh_engine_memclr(self.h, int(mem)))
+
+    def Accessible(self, mem):
+        out = C.c_uint64(0)
+        self._check(self.lib.ghh_engine_accessible(self.h, int(mem), C.byref(out)))
+        return out.value
+
+    def NonStdAlloc(self):
+        pass
+
+    def WorksWith(self, order=None):
+        return True
 
     def pending(self):
         return self.lib.ghh_engine_pending(self.h)

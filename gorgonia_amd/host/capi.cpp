@@ -76,6 +76,15 @@ int ghh_engine_get(ghh_engine* e, int64_t size, uint64_t* mem) { return ret(e, e
 int ghh_engine_put(ghh_engine* e, uint64_t mem, int64_t size) { e->e->Put(mem, size); return 0; }
 int ghh_engine_reset_allocator(ghh_engine* e) { e->e->ResetAllocator(); return 0; }
 int ghh_engine_alloc_accessible(ghh_engine* e) { return e->e->AllocAccessible() ? 1 : 0; }
+int ghh_engine_memset(ghh_engine* e, uint64_t mem, const void* val) { return ret(e, e->e->Memset(mem, val)); }
+int ghh_engine_memclr(ghh_engine* e, uint64_t mem) { return ret(e, e->e->Memclr(mem)); }
+int ghh_engine_accessible(ghh_engine* e, uint64_t mem, uint64_t* out) { return ret(e, e->e->Accessible(mem, out)); }
+int ghh_engine_alloc_flags(ghh_engine* e, int32_t out[2]) {
+  bool mm, cm;
+  e->e->AllocFlags(&mm, &cm);
+  out[0] = mm; out[1] = cm;
+  return 0;
+}
 int ghh_engine_memcpy(ghh_engine* e, uint64_t dst, int64_t dsize, uint64_t src, int64_t ssize) {
   return ret(e, e->e->Memcpy(dst, dsize, src, ssize));
 }

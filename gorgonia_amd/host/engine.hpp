@@ -102,6 +102,14 @@ class Engine {
   Status Free(uint64_t mem, int64_t size) { Put(mem, size); return Status::OK(); }
   Status Memcpy(uint64_t dst, int64_t dsize, uint64_t src, int64_t ssize);  // eager, min size
   bool WorksWith() const { return true; }
+  // The reference leaves these three unimplemented and panics (cuda/engine.go:93-99,
+  // 130-132); here they report the same words as an error instead of aborting.
+  Status Memset(uint64_t, const void*) { return Status::Err(GH_ENOFUNC, "not implemented"); }
+  Status Memclr(uint64_t) { return Status::Err(GH_ENOFUNC, "not implemented"); }
+  Status Accessible(uint64_t, uint64_t*) { return Status::Err(GH_ENOFUNC, "not implemented"); }
+  // AllocFlags (cuda/engine.go:81-83): manually managed memory, column-major tag.
+  void AllocFlags(bool* manually_managed, bool* col_major) const { *manually_managed = true; *col_major = true; }
+  void NonStdAlloc() {}                            // cuda/engine.go:138
 
   // Host <-> device transfers (ExternMetadata.Transfer, cuda.go:179-215); queued
   // behind the segment recorded so far.  `synchronous` flushes like Signal().

@@ -63,6 +63,13 @@ GH_API int ghh_engine_get(ghh_engine* e, int64_t size, uint64_t* mem);   /* Aren
 GH_API int ghh_engine_put(ghh_engine* e, uint64_t mem, int64_t size);    /* Arena.Put */
 GH_API int ghh_engine_reset_allocator(ghh_engine* e);
 GH_API int ghh_engine_alloc_accessible(ghh_engine* e);                   /* AllocAccessible */
+/* Memset, Memclr, Accessible: "not implemented" in the reference (cuda/engine.go:93-99,
+ * 130-132, a panic there); GH_ENOFUNC with that message here. */
+GH_API int ghh_engine_memset(ghh_engine* e, uint64_t mem, const void* val);
+GH_API int ghh_engine_memclr(ghh_engine* e, uint64_t mem);
+GH_API int ghh_engine_accessible(ghh_engine* e, uint64_t mem, uint64_t* out);
+/* AllocFlags (cuda/engine.go:81-83): out[0] = manually managed, out[1] = column-major tag */
+GH_API int ghh_engine_alloc_flags(ghh_engine* e, int32_t out[2]);
 GH_API int ghh_engine_memcpy(ghh_engine* e, uint64_t dst, int64_t dsize, uint64_t src, int64_t ssize);
 GH_API int ghh_engine_h2d(ghh_engine* e, uint64_t dst, const void* src, int64_t bytes);
 GH_API int ghh_engine_d2h(ghh_engine* e, void* dst, uint64_t src, int64_t bytes);

@@ -91,6 +91,15 @@ def test_has_func_and_unknown_unary(eng):
     assert eng.AllocAccessible() is False
 
 
+def test_unimplemented_engine_methods_say_so(eng):
+    """cuda/engine.go:93-99,130-132 panic with these words; here they are errors."""
+    for call in (lambda: eng.Memset(0), lambda: eng.Memclr(0), lambda: eng.Accessible(0)):
+        with pytest.raises(EngineError, match="not implemented"):
+            call()
+    assert eng.AllocFlags() == (True, True) and eng.WorksWith() is True
+    eng.NonStdAlloc()
+
+
 def test_elem_grid_size_matches_reference_rule(eng):
     """cuda/external.go:52-85 with the device limits defaulted (1024 threads)."""
     assert eng.ElemGridSize(100) == (1, 1, 1, 100, 1, 1)
