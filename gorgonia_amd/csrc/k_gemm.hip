@@ -1265,71 +1265,181 @@ __global__ __launch_bounds__(256) void k_conv3x3_direct(const float* __restrict_
 // ---- float64 GEMM -----------------------------------------------------------------
 // C = op(A) op(B) in float64 on the matrix cores (v_mfma_f64_16x16x4f64: lane l
 // feeds A[l%16][l/16] and B[l/16][l%16]; accumulator register v of lane l is
-// C[4*v + l/16][l%16]).  64x64 block tile, four wavefronts of 32x32, operands
-// staged k-major through LDS with plain bounds-checked loads (any transpose, any
-// leading dimension).  Present for the float64 engine path; not tuned.
+// C[4*v + l/16][l%16]), any transpose, extents and leading dimensions.
+// Global loads are pairs of doubles along the operand's contiguous axis: VEC
+// when every pair is whole and 16-byte aligned (even extents, leading
+// dimensions and batch strides, aligned bases), otherwise 8-byte aligned pairs
+// with a single at an odd end (the extra tests cost about 9 % at 2048^3).  LDS tiles are
+// k-pair-major: element (r, k) of a tile sits at (k/2)*S2 + 2*r + (k&1).  The
+// four k-rows a 16x16x4 MFMA reads are then two pair rows: lanes 0-31 of a
+// ds_read_b64 (k and k+1 of rows r..r+15) cover 32 consecutive doubles, lanes
+// 32-63 the next pair row - no bank conflict for any S2 - and an operand whose
+// k axis is contiguous in memory goes to LDS with one 16-byte store per pair
+// (S2*8 = 64 mod 256 keeps the k-pairs of a row apart).  BM x BN block, 2x2
+// wavefronts of (BM/2) x (BN/2), register-staged double buffering with one
+// barrier per k-tile.
 typedef double f64x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+typedef double f64x2_a8 __attribute__((ext_vector_type(2), aligned(8)));
 
-__global__ __launch_bounds__(kThreads) void k_dgemm(const double* __restrict__ A,
-                                                    const double* __restrict__ B,
-                                                    double* __restrict__ C, int M, int N, int K,
-                                                    int lda, int ldb, int ldc, int64_t sA, int64_t sB,
-                                                    int64_t sC, int ta, int tb) {
-  constexpr int BM = 64, BN = 64, BK = 16, S = 66;
-  __shared__ double As[BK * S], Bs[BK * S];
-  A += blockIdx.z * sA;
-  B += blockIdx.z * sB;
-  C += blockIdx.z * sC;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
-  const int lr = lane & 15, lk = lane >> 4;
-  f64x4 acc[2][2];
+// Operand stored [r][k] with k contiguous (A not transposed; B transposed).
+template <int R, int BK, bool VEC>
+struct LoadKContig64 {
+  static constexpr int S2 = 2 * R + 8;
+  static constexpr int SIZE = (BK / 2) * S2;
+  static constexpr int TOTAL = R * BK / 2;   // pairs per tile
+  static constexpr int NV = (TOTAL + kThreads - 1) / kThreads;
+  const double* base; int ld; int rmax; int kmax;
+  f64x2 reg[NV];
+  __device__ __forceinline__ void load(int r0, int k0) {
 #pragma unroll
-  for (int a = 0; a < 2; a++)
-#pragma unroll
-    for (int b = 0; b < 2; b++) acc[a][b] = f64x4{0.0, 0.0, 0.0, 0.0};
-  for (int k0 = 0; k0 < K; k0 += BK) {
-    // 64 x 16 elements per operand, 4 per thread; consecutive threads walk the
-    // operand's contiguous axis
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      const int f = threadIdx.x + e * kThreads;
-      {
-        const int r = ta ? f % BM : f / BK, k = ta ? f / BM : f % BK;
-        const int i = m0 + r, kk = k0 + k;
-        double v = 0.0;
-        if (i < M && kk < K) v = ta ? A[(int64_t)kk * lda + i] : A[(int64_t)i * lda + kk];
-        As[k * S + r] = v;
+    for (int j = 0; j < NV; j++) {
+      const int f = threadIdx.x + j * kThreads;
+      const int r = r0 + f / (BK / 2);
+      const int k = k0 + (f % (BK / 2)) * 2;
+      f64x2 v = {0.0, 0.0};
+      if ((TOTAL % kThreads == 0 || f < TOTAL) && r < rmax) {
+        const double* p = base + (int64_t)r * ld + k;
+        if (VEC) {
+          if (k < kmax) v = *reinterpret_cast<const f64x2*>(p);
+        } else {
+          if (k + 1 < kmax) v = *reinterpret_cast<const f64x2_a8*>(p);
+          else if (k < kmax) v[0] = p[0];
+        }
       }
-      {
-        const int c = tb ? f / BK : f % BN, k = tb ? f % BK : f / BN;
-        const int j = n0 + c, kk = k0 + k;
-        double v = 0.0;
-        if (j < N && kk < K) v = tb ? B[(int64_t)j * ldb + kk] : B[(int64_t)kk * ldb + j];
-        Bs[k * S + c] = v;
-      }
+      reg[j] = v;
     }
-    __syncthreads();
+  }
+  __device__ __forceinline__ void store(double* lds) const {
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 4) {
-      double af[2], bf[2];
+    for (int j = 0; j < NV; j++) {
+      const int f = threadIdx.x + j * kThreads;
+      if (TOTAL % kThreads != 0 && f >= TOTAL) continue;
+      *reinterpret_cast<f64x2*>(&lds[(f % (BK / 2)) * S2 + 2 * (f / (BK / 2))]) = reg[j];
+    }
+  }
+};
+
+// Operand stored [k][c] with c contiguous (B not transposed; A transposed): a
+// thread takes columns c, c+1 of rows k, k+1 and writes the two k-pairs.
+template <int R, int BK, bool VEC>
+struct LoadMnContig64 {
+  static constexpr int S2 = 2 * R + 8;
+  static constexpr int SIZE = (BK / 2) * S2;
+  static constexpr int TOTAL = (R / 2) * (BK / 2);   // 2x2 cells per tile
+  static constexpr int NV = (TOTAL + kThreads - 1) / kThreads;
+  const double* base; int ld; int rmax; int kmax;
+  f64x2 reg[NV][2];
+  __device__ __forceinline__ void load(int c0, int k0) {
 #pragma unroll
-      for (int a = 0; a < 2; a++) af[a] = As[(kk + lk) * S + wm + a * 16 + lr];
+    for (int j = 0; j < NV; j++) {
+      const int f = threadIdx.x + j * kThreads;
+      const int c = c0 + (f % (R / 2)) * 2;
+      const int k = k0 + (f / (R / 2)) * 2;
+      f64x2 v0 = {0.0, 0.0}, v1 = {0.0, 0.0};
+      if ((TOTAL % kThreads == 0 || f < TOTAL) && c < rmax) {
+        const double* p = base + (int64_t)k * ld + c;
+        if (VEC) {
+          if (k < kmax) v0 = *reinterpret_cast<const f64x2*>(p);
+          if (k + 1 < kmax) v1 = *reinterpret_cast<const f64x2*>(p + ld);
+        } else if (c + 1 < rmax) {
+          if (k < kmax) v0 = *reinterpret_cast<const f64x2_a8*>(p);
+          if (k + 1 < kmax) v1 = *reinterpret_cast<const f64x2_a8*>(p + ld);
+        } else {
+          if (k < kmax) v0[0] = p[0];
+          if (k + 1 < kmax) v1[0] = p[ld];
+        }
+      }
+      reg[j][0] = v0;
+      reg[j][1] = v1;
+    }
+  }
+  __device__ __forceinline__ void store(double* lds) const {
 #pragma unroll
-      for (int b = 0; b < 2; b++) bf[b] = Bs[(kk + lk) * S + wn + b * 16 + lr];
+    for (int j = 0; j < NV; j++) {
+      const int f = threadIdx.x + j * kThreads;
+      if (TOTAL % kThreads != 0 && f >= TOTAL) continue;
+      double* d = &lds[(f / (R / 2)) * S2 + 4 * (f % (R / 2))];
+      *reinterpret_cast<f64x2*>(d) = f64x2{reg[j][0][0], reg[j][1][0]};
+      *reinterpret_cast<f64x2*>(d + 2) = f64x2{reg[j][0][1], reg[j][1][1]};
+    }
+  }
+};
+
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC>
+__global__ __launch_bounds__(kThreads) void k_dgemm(const double* __restrict__ A,
+                                                          const double* __restrict__ B,
+                                                          double* __restrict__ C, int M, int N, int K,
+                                                          int lda, int ldb, int ldc, int64_t sA,
+                                                          int64_t sB, int64_t sC) {
+  using LA = typename std::conditional<TA, LoadMnContig64<BM, BK, VEC>, LoadKContig64<BM, BK, VEC>>::type;
+  using LB = typename std::conditional<TB, LoadKContig64<BN, BK, VEC>, LoadMnContig64<BN, BK, VEC>>::type;
+  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
+  static_assert(TM >= 1 && TN >= 1 && WM % 16 == 0 && WN % 16 == 0, "bad wave tiling");
+  __shared__ double lds[2 * (LA::SIZE + LB::SIZE)];
+  double* const As = lds;
+  double* const Bs = lds + 2 * LA::SIZE;
+
+  int tile_m, tile_n;
+  tile_coords(&tile_m, &tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+  const int lr = lane & 15, lk = lane >> 4;
+
+  LA la; la.base = A + blockIdx.z * sA; la.ld = lda; la.rmax = M; la.kmax = K;
+  LB lb; lb.base = B + blockIdx.z * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
+  C += blockIdx.z * sC;
+
+  f64x4 acc[TM][TN];
 #pragma unroll
-      for (int a = 0; a < 2; a++)
+  for (int a = 0; a < TM; a++)
 #pragma unroll
-        for (int b = 0; b < 2; b++)
-          acc[a][b] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[a], bf[b], acc[a][b], 0, 0, 0);
+    for (int b = 0; b < TN; b++) acc[a][b] = f64x4{0.0, 0.0, 0.0, 0.0};
+
+  const int nk = (K + BK - 1) / BK;
+  la.load(m0, 0);
+  lb.load(n0, 0);
+  la.store(As);
+  lb.store(Bs);
+  __syncthreads();
+  // this lane's element of MFMA k-step 0: pair row lk/2, parity lk&1
+  const int a_off = (lk >> 1) * LA::S2 + 2 * (wm + lr) + (lk & 1);
+  const int b_off = (lk >> 1) * LB::S2 + 2 * (wn + lr) + (lk & 1);
+  for (int kt = 0; kt < nk; kt++) {
+    const int cur = kt & 1;
+    const bool more = kt + 1 < nk;
+    if (more) {
+      la.load(m0, (kt + 1) * BK);
+      lb.load(n0, (kt + 1) * BK);
+    }
+    const double* a_s = As + cur * LA::SIZE + a_off;
+    const double* b_s = Bs + cur * LB::SIZE + b_off;
+    double af[BK / 4][TM], bf[BK / 4][TN];
+#pragma unroll
+    for (int st = 0; st < BK / 4; st++) {
+#pragma unroll
+      for (int a = 0; a < TM; a++) af[st][a] = a_s[st * 2 * LA::S2 + a * 32];
+#pragma unroll
+      for (int b = 0; b < TN; b++) bf[st][b] = b_s[st * 2 * LB::S2 + b * 32];
+    }
+#pragma unroll
+    for (int st = 0; st < BK / 4; st++)
+#pragma unroll
+      for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int b = 0; b < TN; b++)
+          acc[a][b] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[st][a], bf[st][b], acc[a][b], 0, 0, 0);
+    if (more) {
+      la.store(As + (cur ^ 1) * LA::SIZE);
+      lb.store(Bs + (cur ^ 1) * LB::SIZE);
     }
     __syncthreads();
   }
 #pragma unroll
-  for (int a = 0; a < 2; a++)
+  for (int a = 0; a < TM; a++)
 #pragma unroll
-    for (int b = 0; b < 2; b++)
+    for (int b = 0; b < TN; b++)
 #pragma unroll
       for (int v = 0; v < 4; v++) {
         const int i = m0 + wm + a * 16 + 4 * v + lk, j = n0 + wn + b * 16 + lr;
@@ -2061,16 +2171,42 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   return gh_check_hip(ctx, hipGetLastError(), "skinny gemm launch");
 }
 
+template <int BM, int BN, int BK>
+static void launch_dgemm_cfg(gh_ctx* ctx, const gh_cmd& c, int M, int N, int K, int64_t batch) {
+  const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, (unsigned)batch);
+  const double* A = (const double*)(uintptr_t)c.ptr[0];
+  const double* B = (const double*)(uintptr_t)c.ptr[1];
+  double* C = (double*)(uintptr_t)c.ptr[2];
+  const int lda = (int)c.dim[3], ldb = (int)c.dim[4], ldc = (int)c.dim[5];
+  const int64_t sA = batch > 1 ? c.dim[7] : 0, sB = batch > 1 ? c.dim[8] : 0, sC = batch > 1 ? c.dim[9] : 0;
+  const bool ta = c.flags & GH_FLAG_TRANS_A, tb = c.flags & GH_FLAG_TRANS_B;
+  const auto even = [](int64_t v) { return (v & 1) == 0; };
+  const bool vec = even(M) && even(N) && even(K) && even(lda) && even(ldb) && even(sA) && even(sB) &&
+                   ((c.ptr[0] | c.ptr[1]) & 15) == 0;
+#define GH_DGEMM_GO(TA, TB)                                                                                    \
+  do {                                                                                                         \
+    if (vec)                                                                                                   \
+      hipLaunchKernelGGL((k_dgemm<BM, BN, BK, TA, TB, true>), grid, dim3(kThreads), 0, ctx->stream, A, B, C, M, \
+                         N, K, lda, ldb, ldc, sA, sB, sC);                                                     \
+    else                                                                                                       \
+      hipLaunchKernelGGL((k_dgemm<BM, BN, BK, TA, TB, false>), grid, dim3(kThreads), 0, ctx->stream, A, B, C,  \
+                         M, N, K, lda, ldb, ldc, sA, sB, sC);                                                  \
+  } while (0)
+  if (ta && tb) GH_DGEMM_GO(true, true);
+  else if (ta) GH_DGEMM_GO(true, false);
+  else if (tb) GH_DGEMM_GO(false, true);
+  else GH_DGEMM_GO(false, false);
+#undef GH_DGEMM_GO
+}
+
 int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
   if (gh_dtype_of(c.flags) == GH_F64) {
     const int M = (int)c.dim[0], N = (int)c.dim[1], K = (int)c.dim[2];
     const int64_t batch = c.dim[6] <= 0 ? 1 : c.dim[6];
-    const dim3 grid((N + 63) / 64, (M + 63) / 64, (unsigned)batch);
-    hipLaunchKernelGGL(k_dgemm, grid, dim3(kThreads), 0, ctx->stream, (const double*)(uintptr_t)c.ptr[0],
-                       (const double*)(uintptr_t)c.ptr[1], (double*)(uintptr_t)c.ptr[2], M, N, K, (int)c.dim[3],
-                       (int)c.dim[4], (int)c.dim[5], batch > 1 ? c.dim[7] : 0, batch > 1 ? c.dim[8] : 0,
-                       batch > 1 ? c.dim[9] : 0, (c.flags & GH_FLAG_TRANS_A) ? 1 : 0,
-                       (c.flags & GH_FLAG_TRANS_B) ? 1 : 0);
+    // 128x128 tiles once they fill the device, 64x64 with a longer k-tile below that
+    const int64_t tiles128 = (int64_t)((M + 127) / 128) * ((N + 127) / 128) * batch;
+    if (tiles128 >= ctx->cu_count) launch_dgemm_cfg<128, 128, 8>(ctx, c, M, N, K, batch);
+    else launch_dgemm_cfg<64, 64, 16>(ctx, c, M, N, K, batch);
     return gh_check_hip(ctx, hipGetLastError(), "dgemm launch");
   }
   const int rs = try_launch_gemm_skinny(ctx, c);

@@ -269,7 +269,8 @@ def test_matmul_float64(ctx, ta, tb):
     against numpy's float64 product (1e-13 relative) and exactly on integer data."""
     from gorgonia_amd import _ffi
     rng = np.random.default_rng(17)
-    for (m, k, n) in [(1, 1, 1), (3, 5, 7), (16, 4, 16), (65, 129, 33), (128, 128, 128), (256, 300, 100), (100, 37, 259)]:
+    for (m, k, n) in [(1, 1, 1), (3, 5, 7), (16, 4, 16), (65, 129, 33), (128, 128, 128), (256, 300, 100), (100, 37, 259),
+                      (66, 130, 34), (32, 2, 32), (2050, 70, 2046), (1024, 24, 4100)]:
         for integer in (False, True):
             A = rng.integers(-8, 9, (k, m) if ta else (m, k)).astype(np.float64) if integer else \
                 rng.standard_normal((k, m) if ta else (m, k))
@@ -299,3 +300,22 @@ def test_batched_matmul_float64(ctx):
     for p in (dA, dB, dC):
         ctx.free(p)
     assert rel_frobenius(got, A @ B) <= 1e-13
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False)])
+def test_batched_matmul_float64_large_tiles(ctx, ta, tb):
+    """Enough even-sized batches that the float64 product takes its 128x128 tiles, with
+    ragged edges in every extent; integer data, so the result is exact."""
+    from gorgonia_amd import _ffi
+    rng = np.random.default_rng(19)
+    bt, m, k, n = 70, 130, 36, 258
+    A = rng.integers(-8, 9, (bt, k, m) if ta else (bt, m, k)).astype(np.float64)
+    B = rng.integers(-8, 9, (bt, n, k) if tb else (bt, k, n)).astype(np.float64)
+    dA, dB, dC = ctx.upload(A), ctx.upload(B), ctx.malloc(bt * m * n * 8)
+    ctx.run(D.cmd_gemm(dA, dB, dC, m, n, k, trans_a=ta, trans_b=tb, batch=bt, stride_a=m * k, stride_b=k * n,
+                       stride_c=m * n, dtype=_ffi.F64))
+    got = ctx.d2h(dC, (bt, m, n), dtype=np.float64)
+    for p in (dA, dB, dC):
+        ctx.free(p)
+    want = (A.transpose(0, 2, 1) if ta else A) @ (B.transpose(0, 2, 1) if tb else B)
+    assert np.array_equal(got, want)
