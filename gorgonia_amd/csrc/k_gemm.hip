@@ -359,6 +359,9 @@ __device__ __forceinline__ void split_range(int nk, int splits, int s, int* kt0,
 // every XCD one contiguous range of tiles; inside a range, tiles are walked in
 // groups of 8 tile-rows so that co-resident workgroups share A rows and B
 // columns (a plain row-major walk re-read A and B ~6x from HBM at 4096^3).
+// (For a batch of products the same regrouping over the whole launch, so that
+// an XCD works through whole matrices, was measured: no gain on 64 x 512^3, and
+// the extra branch cost the register-tight 128x128 kernel 9 % at 4096^3.)
 __device__ __forceinline__ void tile_coords(int* tm, int* tn) {
   const int gx = gridDim.x, gy = gridDim.y;  // tiles along N, along M
   const int total = gx * gy;

@@ -82,6 +82,7 @@ HOST_SYMBOLS = {
     "ghh_graph_let": (C.c_int, [_P, C.c_int, _P]),
     "ghh_graph_read": (C.c_int, [_P, C.c_int, _P]),
     "ghh_graph_node_shape": (C.c_int, [_P, C.c_int, C.POINTER(C.c_int64), C.c_int]),
+    "ghh_graph_node_dtype": (C.c_int, [_P, C.c_int]),
     "ghh_graph_fuse_activations": (C.c_int, [_P]),
     "ghh_tape_new": (_P, [_P, C.c_int, C.c_int]),
     "ghh_tape_destroy": (None, [_P]),

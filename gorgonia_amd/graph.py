@@ -24,6 +24,13 @@ class Node:
     def Shape(self):
         return self.g.shape_of(self.id)
 
+    def Dtype(self):
+        """numpy dtype of the node's value (float32 or float64)."""
+        code = self.g.lib.ghh_graph_node_dtype(self.g.h, self.id)
+        if code not in (0, 1):
+            raise EngineError(1, f"node {self.id}: the device path holds float32 and float64 values only")
+        return np.dtype(np.float64 if code == 1 else np.float32)
+
 
 class ExprGraph:
     def __init__(self):
@@ -93,9 +100,14 @@ def Let(node, value):
     node.g._check(node.g.lib.ghh_graph_let(node.g.h, node.id, value.ctypes.data_as(C.c_void_p)))
 
 
-def Read(node, dtype=np.float32):
-    """gorgonia.Read: returns the host array the value lands in after RunAll."""
-    out = np.empty(node.Shape(), dtype=dtype)
+def Read(node, dtype=None):
+    """gorgonia.Read: returns the host array the value lands in after RunAll.  The array
+    has the node's own dtype; asking for another one is an error (the machine copies the
+    value's bytes, it does not convert)."""
+    want = node.Dtype()
+    if dtype is not None and np.dtype(dtype) != want:
+        raise EngineError(1, f"Read: node {node.id} holds {want}, not {np.dtype(dtype)}")
+    out = np.empty(node.Shape(), dtype=want)
     node.g._keep.append(out)
     node.g._check(node.g.lib.ghh_graph_read(node.g.h, node.id, out.ctypes.data_as(C.c_void_p)))
     return out

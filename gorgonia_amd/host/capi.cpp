@@ -206,6 +206,10 @@ int ghh_graph_node_shape(ghh_graph* g, int node, int64_t* shape, int cap) {
   for (int i = 0; i < s.Dims() && i < cap; i++) shape[i] = s[i];
   return s.Dims();
 }
+int ghh_graph_node_dtype(ghh_graph* g, int node) {
+  if (node < 0 || node >= (int)g->g.Nodes().size()) return -1;
+  return (int)g->g.Nodes()[(size_t)node].dt;
+}
 int ghh_graph_fuse_activations(ghh_graph* g) { return g->g.FuseActivations(); }
 
 ghh_tape* ghh_tape_new(ghh_graph* g, int graph_replay, int reupload_resident) {

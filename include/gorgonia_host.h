@@ -119,6 +119,8 @@ GH_API int ghh_graph_apply(ghh_graph* g, const ghh_op* op, const int* inputs, in
 GH_API int ghh_graph_let(ghh_graph* g, int node, const void* host);
 GH_API int ghh_graph_read(ghh_graph* g, int node, void* host_out);
 GH_API int ghh_graph_node_shape(ghh_graph* g, int node, int64_t* shape, int cap);
+/* Node.Dtype(): 0 float32, 1 float64, 2 other; -1 for a bad node id */
+GH_API int ghh_graph_node_dtype(ghh_graph* g, int node);
 GH_API int ghh_graph_fuse_activations(ghh_graph* g);
 
 GH_API ghh_tape* ghh_tape_new(ghh_graph* g, int graph_replay, int reupload_resident);

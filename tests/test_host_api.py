@@ -108,6 +108,20 @@ def test_elem_grid_size_matches_reference_rule(eng):
     assert eng.ElemGridSize(1 << 24) == (16384, 1, 1, 1024, 1, 1)
 
 
+def test_read_takes_the_node_dtype():
+    """A float64 value lands in a float64 host array; a mismatched request is refused
+    (the machine copies bytes, so a float32 array would be overrun)."""
+    g = G.NewGraph()
+    x = G.NewTensor(g, np.zeros((4, 6), np.float64))
+    w = G.NewTensor(g, np.zeros((6, 3), np.float64))
+    y = G.Mul(x, w)
+    assert y.Dtype() == np.float64 and G.Read(y).dtype == np.float64
+    with pytest.raises(EngineError, match="holds float64"):
+        G.Read(y, dtype=np.float32)
+    z = G.Rectify(G.NewTensor(g, np.zeros((2, 2), np.float32)))
+    assert G.Read(z).dtype == np.float32 and G.Read(z, np.float32).shape == (2, 2)
+
+
 def test_shape_inference_and_errors():
     g = G.NewGraph()
     x = G.NewTensor(g, np.zeros((2, 3, 8, 8), np.float32))
