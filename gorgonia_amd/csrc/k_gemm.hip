@@ -1369,38 +1369,22 @@ struct LoadMnContig64 {
   }
 };
 
-template <int BM, int BN, int BK, bool TA, bool TB, bool VEC>
-__global__ __launch_bounds__(kThreads) void k_dgemm(const double* __restrict__ A,
-                                                          const double* __restrict__ B,
-                                                          double* __restrict__ C, int M, int N, int K,
-                                                          int lda, int ldb, int ldc, int64_t sA,
-                                                          int64_t sB, int64_t sC) {
-  using LA = typename std::conditional<TA, LoadMnContig64<BM, BK, VEC>, LoadKContig64<BM, BK, VEC>>::type;
-  using LB = typename std::conditional<TB, LoadKContig64<BN, BK, VEC>, LoadMnContig64<BN, BK, VEC>>::type;
+// The float64 MFMA core: 2x2 wavefronts over a BM x BN block, k-tiles [0, nk).
+template <int BM, int BN, int BK, class LA, class LB>
+__device__ __forceinline__ void dmfma_tile_loop(double* lds, LA& la, LB& lb, int m0, int n0, int nk,
+                                                f64x4 (&acc)[BM / 32][BN / 32]) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
   static_assert(TM >= 1 && TN >= 1 && WM % 16 == 0 && WN % 16 == 0, "bad wave tiling");
-  __shared__ double lds[2 * (LA::SIZE + LB::SIZE)];
   double* const As = lds;
   double* const Bs = lds + 2 * LA::SIZE;
-
-  int tile_m, tile_n;
-  tile_coords(&tile_m, &tile_n);
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
   const int lr = lane & 15, lk = lane >> 4;
-
-  LA la; la.base = A + blockIdx.z * sA; la.ld = lda; la.rmax = M; la.kmax = K;
-  LB lb; lb.base = B + blockIdx.z * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
-  C += blockIdx.z * sC;
-
-  f64x4 acc[TM][TN];
 #pragma unroll
   for (int a = 0; a < TM; a++)
 #pragma unroll
     for (int b = 0; b < TN; b++) acc[a][b] = f64x4{0.0, 0.0, 0.0, 0.0};
 
-  const int nk = (K + BK - 1) / BK;
   la.load(m0, 0);
   lb.load(n0, 0);
   la.store(As);
@@ -1439,6 +1423,29 @@ __global__ __launch_bounds__(kThreads) void k_dgemm(const double* __restrict__ A
     }
     __syncthreads();
   }
+}
+
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC>
+__global__ __launch_bounds__(kThreads) void k_dgemm(const double* __restrict__ A,
+                                                    const double* __restrict__ B,
+                                                    double* __restrict__ C, int M, int N, int K,
+                                                    int lda, int ldb, int ldc, int64_t sA,
+                                                    int64_t sB, int64_t sC) {
+  using LA = typename std::conditional<TA, LoadMnContig64<BM, BK, VEC>, LoadKContig64<BM, BK, VEC>>::type;
+  using LB = typename std::conditional<TB, LoadKContig64<BN, BK, VEC>, LoadMnContig64<BN, BK, VEC>>::type;
+  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
+  __shared__ double lds[2 * (LA::SIZE + LB::SIZE)];
+  int tile_m, tile_n;
+  tile_coords(&tile_m, &tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  LA la; la.base = A + blockIdx.z * sA; la.ld = lda; la.rmax = M; la.kmax = K;
+  LB lb; lb.base = B + blockIdx.z * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
+  C += blockIdx.z * sC;
+  f64x4 acc[TM][TN];
+  dmfma_tile_loop<BM, BN, BK, LA, LB>(lds, la, lb, m0, n0, (K + BK - 1) / BK, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+  const int lr = lane & 15, lk = lane >> 4;
 #pragma unroll
   for (int a = 0; a < TM; a++)
 #pragma unroll
@@ -1448,6 +1455,111 @@ __global__ __launch_bounds__(kThreads) void k_dgemm(const double* __restrict__ A
         const int i = m0 + wm + a * 16 + 4 * v + lk, j = n0 + wn + b * 16 + lr;
         if (i < M && j < N) C[(int64_t)i * ldc + j] = acc[a][b][v];
       }
+}
+
+// ---- float64 Conv2d as an implicit GEMM on the matrix cores ---------------------------
+// y(F x P) = w(F x C*kh*kw) . col(C*kh*kw x P), P = B*oh*ow, with the same tile
+// loop as the float64 product.  The filter matrix is the k-contiguous operand;
+// the col operand is gathered from NCHW x: a thread keeps one output pixel for
+// the whole kernel (its image offset and first input row / column are decoded
+// once) and fetches pairs of consecutive k = (c, kr, kc) for it, padding taps as
+// zeros.  Any kernel size, stride, dilation and padding.
+struct ConvGeom64 {
+  int C, H, W, F, oh, ow, kh, kw, padH, padW, strideH, strideW, dilH, dilW;
+  int P, K;           // B*oh*ow, C*kh*kw
+  unsigned mKK, mkw;  // division magics for kh*kw and kw (see div_magic)
+};
+
+template <int R, int BK>
+struct LoadIm2col64 {
+  static constexpr int S2 = 2 * R + 8;
+  static constexpr int SIZE = (BK / 2) * S2;
+  static constexpr int KP_STEP = kThreads / R;            // k-pairs covered per pass
+  static constexpr int NV = (BK / 2 + KP_STEP - 1) / KP_STEP;
+  static_assert(kThreads % R == 0, "pixel columns must divide the block");
+  const double* xp;   // x at (image, first input row, first input column) of this thread's pixel
+  const ConvGeom64* g;
+  int iy0, ix0;
+  bool pvalid;
+  f64x2 reg[NV];
+  __device__ __forceinline__ void init(const double* x, const ConvGeom64* geom, int n0) {
+    g = geom;
+    const int p = n0 + (int)(threadIdx.x % R);
+    pvalid = p < g->P;
+    const int plane = g->oh * g->ow;
+    const int pp = pvalid ? p : 0;
+    const int b = pp / plane, rem = pp - b * plane;
+    const int oy = rem / g->ow, ox = rem - oy * g->ow;
+    iy0 = oy * g->strideH - g->padH;
+    ix0 = ox * g->strideW - g->padW;
+    xp = x + ((int64_t)b * g->C * g->H + iy0) * g->W + ix0;
+  }
+  __device__ __forceinline__ void load(int, int k0) {
+    const int KK = g->kh * g->kw;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int kp = (int)(threadIdx.x / R) + j * KP_STEP;
+      f64x2 v = {0.0, 0.0};
+      if ((BK / 2) % KP_STEP == 0 || kp < BK / 2) {
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+          const int k = k0 + 2 * kp + e;
+          if (pvalid && k < g->K) {
+            const int c = div_magic(k, g->mKK), tap = k - c * KK;
+            const int kr = div_magic(tap, g->mkw), kc = tap - kr * g->kw;
+            const int dy = kr * g->dilH, dx = kc * g->dilW;
+            const int iy = iy0 + dy, ix = ix0 + dx;
+            if (iy >= 0 && iy < g->H && ix >= 0 && ix < g->W) v[e] = xp[((int64_t)c * g->H + dy) * g->W + dx];
+          }
+        }
+      }
+      reg[j] = v;
+    }
+  }
+  __device__ __forceinline__ void store(double* lds) const {
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int kp = (int)(threadIdx.x / R) + j * KP_STEP;
+      if ((BK / 2) % KP_STEP != 0 && kp >= BK / 2) continue;
+      *reinterpret_cast<f64x2*>(&lds[kp * S2 + 2 * (int)(threadIdx.x % R)]) = reg[j];
+    }
+  }
+};
+
+template <int BM, int BN, bool VEC>
+__global__ __launch_bounds__(kThreads) void k_conv2d_f64_mfma(const double* __restrict__ x,
+                                                              const double* __restrict__ w,
+                                                              double* __restrict__ y, ConvGeom64 g) {
+  constexpr int BK = 8;
+  using LA = LoadKContig64<BM, BK, VEC>;
+  using LB = LoadIm2col64<BN, BK>;
+  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
+  __shared__ double lds[2 * (LA::SIZE + LB::SIZE)];
+  int tile_m, tile_n;
+  tile_coords(&tile_m, &tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  LA la; la.base = w; la.ld = g.K; la.rmax = g.F; la.kmax = g.K;
+  LB lb; lb.init(x, &g, n0);
+  f64x4 acc[TM][TN];
+  dmfma_tile_loop<BM, BN, BK, LA, LB>(lds, la, lb, m0, n0, (g.K + BK - 1) / BK, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+  const int lr = lane & 15, lk = lane >> 4;
+  const int plane = g.oh * g.ow;
+#pragma unroll
+  for (int b = 0; b < TN; b++) {
+    const int j = n0 + wn + b * 16 + lr;
+    if (j >= g.P) continue;
+    const int bb = j / plane, pix = j - bb * plane;
+    double* yb = y + (int64_t)bb * g.F * plane + pix;
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        const int i = m0 + wm + a * 16 + 4 * v + lk;
+        if (i < g.F) yb[(int64_t)i * plane] = acc[a][b][v];
+      }
+  }
 }
 
 // ---- Conv2d backward ---------------------------------------------------------------
@@ -2172,6 +2284,42 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   else if (vec_b) launch(k_gemm_skinny<WV, false, true>);
   else launch(k_gemm_skinny<WV, false, false>);
   return gh_check_hip(ctx, hipGetLastError(), "skinny gemm launch");
+}
+
+template <int BM, int BN>
+static void launch_conv64_cfg(gh_ctx* ctx, const gh_cmd& c, const ConvGeom64& g) {
+  const dim3 grid((g.P + BN - 1) / BN, (g.F + BM - 1) / BM, 1);
+  const double* x = (const double*)(uintptr_t)c.ptr[0];
+  const double* w = (const double*)(uintptr_t)c.ptr[1];
+  double* y = (double*)(uintptr_t)c.ptr[2];
+  if ((g.K & 1) == 0 && (c.ptr[1] & 15) == 0)
+    hipLaunchKernelGGL((k_conv2d_f64_mfma<BM, BN, true>), grid, dim3(kThreads), 0, ctx->stream, x, w, y, g);
+  else
+    hipLaunchKernelGGL((k_conv2d_f64_mfma<BM, BN, false>), grid, dim3(kThreads), 0, ctx->stream, x, w, y, g);
+}
+
+// Float64 Conv2d on the matrix cores; false = not taken (few filters or a tiny
+// problem: the one-thread-per-result kernel stays).
+bool gh_try_launch_conv2d_f64_mfma(gh_ctx* ctx, const gh_cmd& c) {
+  ConvGeom64 g;
+  const int64_t B = c.dim[0];
+  g.C = (int)c.dim[1]; g.H = (int)c.dim[2]; g.W = (int)c.dim[3]; g.F = (int)c.dim[4];
+  g.kh = (int)c.dim[5]; g.kw = (int)c.dim[6]; g.padH = (int)c.dim[7]; g.padW = (int)c.dim[8];
+  g.strideH = (int)c.dim[9]; g.strideW = (int)c.dim[10]; g.dilH = (int)c.dim[11]; g.dilW = (int)c.dim[12];
+  g.oh = (int)gh_conv_out(g.H, g.kh, g.padH, g.strideH, g.dilH);
+  g.ow = (int)gh_conv_out(g.W, g.kw, g.padW, g.strideW, g.dilW);
+  const int64_t P = B * g.oh * g.ow, K = (int64_t)g.C * g.kh * g.kw;
+  if (g.F < 16 || P < 256 || K < 8 || P * g.F * K < (int64_t)1 << 22) return false;
+  if (P > 0x7fffffff || K * (int64_t)(g.kh * g.kw) >= ((int64_t)1 << 32)) return false;
+  g.P = (int)P;
+  g.K = (int)K;
+  g.mKK = div_magic_of((unsigned)(g.kh * g.kw));
+  g.mkw = div_magic_of((unsigned)g.kw);
+  const int64_t tiles128 = (int64_t)((g.F + 127) / 128) * ((P + 127) / 128);
+  if (g.F <= 32) launch_conv64_cfg<32, 128>(ctx, c, g);
+  else if (tiles128 >= ctx->cu_count) launch_conv64_cfg<128, 128>(ctx, c, g);
+  else launch_conv64_cfg<64, 64>(ctx, c, g);
+  return true;
 }
 
 template <int BM, int BN, int BK>

@@ -54,6 +54,42 @@ def test_conv2d_float64_bit_exact(ctx, cfg):
     assert np.allclose(got, ref, rtol=1e-4, atol=1e-4)   # and it is the same convolution as the float32 one
 
 
+CONV_MFMA_CASES = [
+    # enough filters and pixels for the matrix-core kernel: each of its three tile shapes, odd and even
+    # C*kh*kw, ragged edges in filters and pixels, stride / dilation / rectangular kernels
+    (4, 1, 28, 28, 32, 3, 3, (1, 1), (1, 1), (1, 1)),      # 32-filter tiles, K = 9
+    (3, 5, 17, 19, 24, 3, 3, (1, 1), (1, 1), (1, 1)),      # 32-filter tiles, ragged, K = 45
+    (8, 32, 14, 14, 64, 3, 3, (1, 1), (1, 1), (1, 1)),     # 64x64 tiles
+    (2, 7, 21, 20, 70, 5, 3, (2, 1), (2, 1), (1, 1)),      # 64x64 tiles, ragged, strided
+    (2, 6, 23, 23, 40, 3, 3, (2, 2), (1, 2), (2, 2)),      # dilated
+    (40, 8, 30, 30, 130, 3, 3, (1, 1), (1, 1), (1, 1)),    # 128x128 tiles, ragged filters
+    (36, 16, 30, 31, 128, 1, 1, (0, 0), (1, 1), (1, 1)),   # 128x128 tiles, 1x1
+]
+
+
+@pytest.mark.parametrize("cfg", CONV_MFMA_CASES)
+def test_conv2d_float64_matrix_cores(ctx, cfg):
+    """The float64 implicit-GEMM kernel: the matrix cores sum each group of four products in
+    their own order, so against the oracle's sequential float64 sum the bar is 1e-13 relative
+    (far inside the 1e-5 of the float32 path), and equality on small-integer data, where
+    every partial sum is exact."""
+    B, C, H, W, F, kh, kw, pad, stride, dil = cfg
+    rng = np.random.default_rng(5)
+    for integer in (False, True):
+        x = rng.integers(-4, 5, (B, C, H, W)).astype(np.float64) if integer else rng.standard_normal((B, C, H, W))
+        w = rng.integers(-4, 5, (F, C, kh, kw)).astype(np.float64) if integer else rng.standard_normal((F, C, kh, kw)) * 0.3
+        want = O.conv2d(x, w, pad, stride, dil)
+        dx, dw, dy = ctx.upload(x), ctx.upload(w), ctx.malloc(want.size * 8)
+        ctx.run(D.cmd_conv2d(dx, dw, dy, B, C, H, W, F, kh, kw, pad, stride, dil, dtype=F64))
+        got = ctx.d2h(dy, want.shape, np.float64)
+        for p in (dx, dw, dy):
+            ctx.free(p)
+        if integer:
+            assert np.array_equal(got, want), f"integer float64 conv {cfg}"
+        else:
+            assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-13, f"float64 conv {cfg}"
+
+
 @pytest.mark.parametrize("cfg", [(2, 3, 8, 10, (2, 2), (0, 0), (2, 2)), (1, 2, 7, 8, (3, 2), (1, 1), (1, 2)),
                                  (2, 4, 13, 13, (2, 2), (1, 0, 1, 0), (1, 1)), (2, 3, 9, 11, (2, 2), (0, 0), (2, 2))])
 def test_maxpool_float64_bit_exact(ctx, cfg):
