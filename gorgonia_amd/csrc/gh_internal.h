@@ -80,6 +80,8 @@ int gh_launch_bn_infer_f64(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_softmax_f64(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_conv2d_f64(gh_ctx* ctx, const gh_cmd& c);
 bool gh_try_launch_conv2d_f64_mfma(gh_ctx* ctx, const gh_cmd& c);
+bool gh_try_launch_conv2d_bwd_data_f64_mfma(gh_ctx* ctx, const gh_cmd& c);
+bool gh_try_launch_conv2d_bwd_filter_f64_mfma(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_dropout(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_dropout_bwd(gh_ctx* ctx, const gh_cmd& c);
 

@@ -1369,9 +1369,9 @@ struct LoadMnContig64 {
   }
 };
 
-// The float64 MFMA core: 2x2 wavefronts over a BM x BN block, k-tiles [0, nk).
+// The float64 MFMA core: 2x2 wavefronts over a BM x BN block, k-tiles [kt0, kt1).
 template <int BM, int BN, int BK, class LA, class LB>
-__device__ __forceinline__ void dmfma_tile_loop(double* lds, LA& la, LB& lb, int m0, int n0, int nk,
+__device__ __forceinline__ void dmfma_tile_loop(double* lds, LA& la, LB& lb, int m0, int n0, int kt0, int kt1,
                                                 f64x4 (&acc)[BM / 32][BN / 32]) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
   static_assert(TM >= 1 && TN >= 1 && WM % 16 == 0 && WN % 16 == 0, "bad wave tiling");
@@ -1385,17 +1385,17 @@ __device__ __forceinline__ void dmfma_tile_loop(double* lds, LA& la, LB& lb, int
 #pragma unroll
     for (int b = 0; b < TN; b++) acc[a][b] = f64x4{0.0, 0.0, 0.0, 0.0};
 
-  la.load(m0, 0);
-  lb.load(n0, 0);
+  la.load(m0, kt0 * BK);
+  lb.load(n0, kt0 * BK);
   la.store(As);
   lb.store(Bs);
   __syncthreads();
   // this lane's element of MFMA k-step 0: pair row lk/2, parity lk&1
   const int a_off = (lk >> 1) * LA::S2 + 2 * (wm + lr) + (lk & 1);
   const int b_off = (lk >> 1) * LB::S2 + 2 * (wn + lr) + (lk & 1);
-  for (int kt = 0; kt < nk; kt++) {
-    const int cur = kt & 1;
-    const bool more = kt + 1 < nk;
+  for (int kt = kt0; kt < kt1; kt++) {
+    const int cur = (kt - kt0) & 1;
+    const bool more = kt + 1 < kt1;
     if (more) {
       la.load(m0, (kt + 1) * BK);
       lb.load(n0, (kt + 1) * BK);
@@ -1442,7 +1442,7 @@ __global__ __launch_bounds__(kThreads) void k_dgemm(const double* __restrict__ A
   LB lb; lb.base = B + blockIdx.z * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
   C += blockIdx.z * sC;
   f64x4 acc[TM][TN];
-  dmfma_tile_loop<BM, BN, BK, LA, LB>(lds, la, lb, m0, n0, (K + BK - 1) / BK, acc);
+  dmfma_tile_loop<BM, BN, BK, LA, LB>(lds, la, lb, m0, n0, 0, (K + BK - 1) / BK, acc);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
   const int lr = lane & 15, lk = lane >> 4;
@@ -1455,6 +1455,60 @@ __global__ __launch_bounds__(kThreads) void k_dgemm(const double* __restrict__ A
         const int i = m0 + wm + a * 16 + 4 * v + lk, j = n0 + wn + b * 16 + lr;
         if (i < M && j < N) C[(int64_t)i * ldc + j] = acc[a][b][v];
       }
+}
+
+// Float64 product with a small result (a dense layer on a batch: too few 64x64
+// tiles to occupy the device, and a k loop of a thousand steps behind each).
+// One workgroup per 16x16 tile of C, its WV wavefronts each summing a slice of
+// K straight from global memory into one MFMA accumulator (element (i, k) of
+// op(A) at A[i*sai + k*sak], (k, j) of op(B) at B[k*sbk + j*sbj], so every
+// transpose is the same code); loads are unconditional at clamped addresses and
+// masked afterwards, so they all stay in flight.  The slices are added in LDS in
+// wavefront order: the result does not depend on scheduling.
+template <int WV>
+__global__ __launch_bounds__(WV * 64) void k_dgemm_skinny(const double* __restrict__ A,
+                                                          const double* __restrict__ B,
+                                                          double* __restrict__ C, int M, int N, int K,
+                                                          int64_t sai, int64_t sak, int64_t sbk,
+                                                          int64_t sbj, int ldc) {
+  __shared__ double part[WV][256];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lr = lane & 15, lk = lane >> 4;
+  const int m0 = blockIdx.y * 16, n0 = blockIdx.x * 16;
+  const double* ap = A + (int64_t)min(m0 + lr, M - 1) * sai;
+  const double* bp = B + (int64_t)min(n0 + lr, N - 1) * sbj;
+  const int kper = (((K + WV - 1) / WV) + 3) & ~3;
+  const int k0 = wave * kper, k1 = min(K, k0 + kper);
+  f64x4 acc = {0.0, 0.0, 0.0, 0.0};
+  for (int k = k0; k < k1; k += 16) {
+    double a[4], b[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int kc = min(k + 4 * u + lk, K - 1);
+      a[u] = ap[kc * sak];
+      b[u] = bp[kc * sbk];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const bool ok = k + 4 * u + lk < k1;
+      a[u] = ok ? a[u] : 0.0;
+      b[u] = ok ? b[u] : 0.0;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) acc = __builtin_amdgcn_mfma_f64_16x16x4f64(a[u], b[u], acc, 0, 0, 0);
+  }
+#pragma unroll
+  for (int v = 0; v < 4; v++) part[wave][v * 64 + lane] = acc[v];
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      double sum = part[0][v * 64 + lane];
+      for (int w = 1; w < WV; w++) sum = sum + part[w][v * 64 + lane];
+      const int i = m0 + 4 * v + lk, j = n0 + lr;
+      if (i < M && j < N) C[(int64_t)i * ldc + j] = sum;
+    }
+  }
 }
 
 // ---- float64 Conv2d as an implicit GEMM on the matrix cores ---------------------------
@@ -1480,6 +1534,7 @@ struct LoadIm2col64 {
   const double* xp;   // x at (image, first input row, first input column) of this thread's pixel
   const ConvGeom64* g;
   int iy0, ix0;
+  int safe;           // offset from xp of an element that is always readable (the image's first)
   bool pvalid;
   f64x2 reg[NV];
   __device__ __forceinline__ void init(const double* x, const ConvGeom64* geom, int n0) {
@@ -1493,28 +1548,35 @@ struct LoadIm2col64 {
     iy0 = oy * g->strideH - g->padH;
     ix0 = ox * g->strideW - g->padW;
     xp = x + ((int64_t)b * g->C * g->H + iy0) * g->W + ix0;
+    safe = -(iy0 * g->W + ix0);
   }
+  // Every load is issued, at a clamped address (the image base for a padding tap
+  // or a k past the end), and masked afterwards: a load inside a branch would make
+  // the wavefront wait for it before the next one is issued.
   __device__ __forceinline__ void load(int, int k0) {
     const int KK = g->kh * g->kw;
+    unsigned okbits = 0;
 #pragma unroll
     for (int j = 0; j < NV; j++) {
       const int kp = (int)(threadIdx.x / R) + j * KP_STEP;
-      f64x2 v = {0.0, 0.0};
-      if ((BK / 2) % KP_STEP == 0 || kp < BK / 2) {
 #pragma unroll
-        for (int e = 0; e < 2; e++) {
-          const int k = k0 + 2 * kp + e;
-          if (pvalid && k < g->K) {
-            const int c = div_magic(k, g->mKK), tap = k - c * KK;
-            const int kr = div_magic(tap, g->mkw), kc = tap - kr * g->kw;
-            const int dy = kr * g->dilH, dx = kc * g->dilW;
-            const int iy = iy0 + dy, ix = ix0 + dx;
-            if (iy >= 0 && iy < g->H && ix >= 0 && ix < g->W) v[e] = xp[((int64_t)c * g->H + dy) * g->W + dx];
-          }
-        }
+      for (int e = 0; e < 2; e++) {
+        const int k = k0 + 2 * kp + e;
+        const int kk = min(k, g->K - 1);
+        const int c = div_magic(kk, g->mKK), tap = kk - c * KK;
+        const int kr = div_magic(tap, g->mkw), kc = tap - kr * g->kw;
+        const int dy = kr * g->dilH, dx = kc * g->dilW;
+        const int iy = iy0 + dy, ix = ix0 + dx;
+        const bool ok = pvalid && k < g->K && iy >= 0 && iy < g->H && ix >= 0 && ix < g->W;
+        const int off = ok ? (c * g->H + dy) * g->W + dx : safe;
+        reg[j][e] = xp[off];
+        okbits |= (ok ? 1u : 0u) << (2 * j + e);
       }
-      reg[j] = v;
     }
+#pragma unroll
+    for (int j = 0; j < NV; j++)
+#pragma unroll
+      for (int e = 0; e < 2; e++) reg[j][e] = ((okbits >> (2 * j + e)) & 1u) ? reg[j][e] : 0.0;
   }
   __device__ __forceinline__ void store(double* lds) const {
 #pragma unroll
@@ -1526,11 +1588,10 @@ struct LoadIm2col64 {
   }
 };
 
-template <int BM, int BN, bool VEC>
+template <int BM, int BN, int BK, bool VEC>
 __global__ __launch_bounds__(kThreads) void k_conv2d_f64_mfma(const double* __restrict__ x,
                                                               const double* __restrict__ w,
                                                               double* __restrict__ y, ConvGeom64 g) {
-  constexpr int BK = 8;
   using LA = LoadKContig64<BM, BK, VEC>;
   using LB = LoadIm2col64<BN, BK>;
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
@@ -1541,7 +1602,7 @@ __global__ __launch_bounds__(kThreads) void k_conv2d_f64_mfma(const double* __re
   LA la; la.base = w; la.ld = g.K; la.rmax = g.F; la.kmax = g.K;
   LB lb; lb.init(x, &g, n0);
   f64x4 acc[TM][TN];
-  dmfma_tile_loop<BM, BN, BK, LA, LB>(lds, la, lb, m0, n0, (g.K + BK - 1) / BK, acc);
+  dmfma_tile_loop<BM, BN, BK, LA, LB>(lds, la, lb, m0, n0, 0, (g.K + BK - 1) / BK, acc);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
   const int lr = lane & 15, lk = lane >> 4;
@@ -1559,6 +1620,152 @@ __global__ __launch_bounds__(kThreads) void k_conv2d_f64_mfma(const double* __re
         const int i = m0 + wm + a * 16 + 4 * v + lk;
         if (i < g.F) yb[(int64_t)i * plane] = acc[a][b][v];
       }
+  }
+}
+
+// ---- float64 Conv2d filter gradient on the matrix cores ------------------------------
+// dW(F x C*kh*kw) = sum over pixels p = (b, oy, ox) of dy[b][f][oy][ox] * col[k][p]
+// (the reference's dY2d^T . col, op_nn.go:267-291): the same tile loop with the
+// pixel axis as the contraction, cut into slices (blockIdx.z) whose partial
+// sums are added in slice order by k_splitk_reduce_f64.  Both operands are
+// gathered; every load is issued at a clamped address and masked afterwards.
+
+// A operand: row f, k = pixel, from NCHW dy.
+template <int R, int BK>
+struct LoadDyRows64 {
+  static constexpr int S2 = 2 * R + 8;
+  static constexpr int SIZE = (BK / 2) * S2;
+  static constexpr int TOTAL = R * BK / 2;
+  static constexpr int NV = TOTAL / kThreads;
+  static_assert(TOTAL % kThreads == 0, "tile must divide over the block");
+  const double* dy; int F, plane, P;
+  f64x2 reg[NV];
+  __device__ __forceinline__ void load(int r0, int k0) {
+    unsigned okbits = 0;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int f = threadIdx.x + j * kThreads;
+      const int r = r0 + f / (BK / 2);
+      const int rc = min(r, F - 1);
+#pragma unroll
+      for (int e = 0; e < 2; e++) {
+        const int p = k0 + (f % (BK / 2)) * 2 + e;
+        const unsigned pc = (unsigned)min(p, P - 1);
+        const unsigned b = pc / (unsigned)plane, pix = pc - b * (unsigned)plane;
+        reg[j][e] = dy[((int64_t)b * F + rc) * plane + pix];
+        okbits |= ((r < F && p < P) ? 1u : 0u) << (2 * j + e);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NV; j++)
+#pragma unroll
+      for (int e = 0; e < 2; e++) reg[j][e] = ((okbits >> (2 * j + e)) & 1u) ? reg[j][e] : 0.0;
+  }
+  __device__ __forceinline__ void store(double* lds) const {
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int f = threadIdx.x + j * kThreads;
+      *reinterpret_cast<f64x2*>(&lds[(f % (BK / 2)) * S2 + 2 * (f / (BK / 2))]) = reg[j];
+    }
+  }
+};
+
+// B operand: column n = (c, kr, kc) kept by the thread, k = pixel, gathered from NCHW x.
+template <int R, int BK>
+struct LoadColT64 {
+  static constexpr int S2 = 2 * R + 8;
+  static constexpr int SIZE = (BK / 2) * S2;
+  static constexpr int KP_STEP = kThreads / R;
+  static constexpr int NV = (BK / 2) / KP_STEP;
+  static_assert(kThreads % R == 0 && (BK / 2) % KP_STEP == 0, "columns and k-pairs must divide the block");
+  const double* xc;   // x at channel c of image 0
+  const ConvGeom64* g;
+  int dy0, dx0;       // input row / column of output pixel (0, 0) for this tap
+  bool nvalid;
+  f64x2 reg[NV];
+  __device__ __forceinline__ void init(const double* x, const ConvGeom64* geom, int n0) {
+    g = geom;
+    const int n = n0 + (int)(threadIdx.x % R);
+    nvalid = n < g->K;
+    const int nn = nvalid ? n : 0;
+    const int KK = g->kh * g->kw;
+    const int c = nn / KK, tap = nn - c * KK;
+    const int kr = tap / g->kw, kc = tap - kr * g->kw;
+    dy0 = kr * g->dilH - g->padH;
+    dx0 = kc * g->dilW - g->padW;
+    xc = x + (int64_t)c * g->H * g->W;
+  }
+  __device__ __forceinline__ void load(int, int k0) {
+    const unsigned plane = (unsigned)(g->oh * g->ow);
+    unsigned okbits = 0;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int kp = (int)(threadIdx.x / R) + j * KP_STEP;
+#pragma unroll
+      for (int e = 0; e < 2; e++) {
+        const int p = k0 + 2 * kp + e;
+        const unsigned pc = (unsigned)min(p, g->P - 1);
+        const unsigned b = pc / plane, rem = pc - b * plane;
+        const unsigned oy = rem / (unsigned)g->ow, ox = rem - oy * (unsigned)g->ow;
+        const int iy = (int)oy * g->strideH + dy0, ix = (int)ox * g->strideW + dx0;
+        const bool ok = nvalid && p < g->P && iy >= 0 && iy < g->H && ix >= 0 && ix < g->W;
+        const int64_t off = ok ? ((int64_t)b * g->C * g->H + iy) * g->W + ix : 0;
+        reg[j][e] = xc[off];
+        okbits |= (ok ? 1u : 0u) << (2 * j + e);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NV; j++)
+#pragma unroll
+      for (int e = 0; e < 2; e++) reg[j][e] = ((okbits >> (2 * j + e)) & 1u) ? reg[j][e] : 0.0;
+  }
+  __device__ __forceinline__ void store(double* lds) const {
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int kp = (int)(threadIdx.x / R) + j * KP_STEP;
+      *reinterpret_cast<f64x2*>(&lds[kp * S2 + 2 * (int)(threadIdx.x % R)]) = reg[j];
+    }
+  }
+};
+
+template <int BM, int BN, int BK>
+__global__ __launch_bounds__(kThreads) void k_conv2d_wgrad_f64(const double* __restrict__ x,
+                                                               const double* __restrict__ dy,
+                                                               double* __restrict__ dw, ConvGeom64 g,
+                                                               int splits, double* __restrict__ ws) {
+  using LA = LoadDyRows64<BM, BK>;
+  using LB = LoadColT64<BN, BK>;
+  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
+  __shared__ double lds[2 * (LA::SIZE + LB::SIZE)];
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int nk = (g.P + BK - 1) / BK;
+  const int per = (nk + splits - 1) / splits;
+  const int kt0 = blockIdx.z * per, kt1 = min(nk, kt0 + per);
+  LA la; la.dy = dy; la.F = g.F; la.plane = g.oh * g.ow; la.P = g.P;
+  LB lb; lb.init(x, &g, n0);
+  f64x4 acc[TM][TN];
+  dmfma_tile_loop<BM, BN, BK, LA, LB>(lds, la, lb, m0, n0, kt0, kt1, acc);
+  double* out = splits > 1 ? ws + (int64_t)blockIdx.z * g.F * g.K : dw;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+  const int lr = lane & 15, lk = lane >> 4;
+#pragma unroll
+  for (int a = 0; a < TM; a++)
+#pragma unroll
+    for (int b = 0; b < TN; b++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        const int i = m0 + wm + a * 16 + 4 * v + lk, j = n0 + wn + b * 16 + lr;
+        if (i < g.F && j < g.K) out[(int64_t)i * g.K + j] = acc[a][b][v];
+      }
+}
+
+__global__ __launch_bounds__(256) void k_splitk_reduce_f64(const double* __restrict__ ws, int splits,
+                                                           int64_t total, double* __restrict__ out) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    double s = ws[i];
+    for (int z = 1; z < splits; z++) s = s + ws[(int64_t)z * total + i];
+    out[i] = s;
   }
 }
 
@@ -1747,9 +1954,9 @@ __global__ __launch_bounds__(256) void k_conv3x3_wgrad_direct(const float* __res
 // filters mirrored and their channel axes swapped, under padding
 // dil*(k-1) - pad, so the forward kernels compute it.  This writes those filters:
 // wt[c][f][kr][kc] = w[f][c][kh-1-kr][kw-1-kc].
-__global__ __launch_bounds__(256) void k_flip_filters(const float* __restrict__ w,
-                                                      float* __restrict__ wt, int F, int C, int kh,
-                                                      int kw) {
+template <class T>
+__global__ __launch_bounds__(256) void k_flip_filters(const T* __restrict__ w, T* __restrict__ wt, int F,
+                                                      int C, int kh, int kw) {
   const int64_t total = (int64_t)F * C * kh * kw;
   const int kk = kh * kw;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
@@ -2286,22 +2493,22 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   return gh_check_hip(ctx, hipGetLastError(), "skinny gemm launch");
 }
 
-template <int BM, int BN>
+template <int BM, int BN, int BK>
 static void launch_conv64_cfg(gh_ctx* ctx, const gh_cmd& c, const ConvGeom64& g) {
   const dim3 grid((g.P + BN - 1) / BN, (g.F + BM - 1) / BM, 1);
   const double* x = (const double*)(uintptr_t)c.ptr[0];
   const double* w = (const double*)(uintptr_t)c.ptr[1];
   double* y = (double*)(uintptr_t)c.ptr[2];
   if ((g.K & 1) == 0 && (c.ptr[1] & 15) == 0)
-    hipLaunchKernelGGL((k_conv2d_f64_mfma<BM, BN, true>), grid, dim3(kThreads), 0, ctx->stream, x, w, y, g);
+    hipLaunchKernelGGL((k_conv2d_f64_mfma<BM, BN, BK, true>), grid, dim3(kThreads), 0, ctx->stream, x, w, y, g);
   else
-    hipLaunchKernelGGL((k_conv2d_f64_mfma<BM, BN, false>), grid, dim3(kThreads), 0, ctx->stream, x, w, y, g);
+    hipLaunchKernelGGL((k_conv2d_f64_mfma<BM, BN, BK, false>), grid, dim3(kThreads), 0, ctx->stream, x, w, y, g);
 }
 
-// Float64 Conv2d on the matrix cores; false = not taken (few filters or a tiny
-// problem: the one-thread-per-result kernel stays).
-bool gh_try_launch_conv2d_f64_mfma(gh_ctx* ctx, const gh_cmd& c) {
-  ConvGeom64 g;
+// Geometry of a float64 convolution command; false when an extent leaves the
+// 32-bit index arithmetic of the matrix-core kernels.
+static bool conv64_fill(const gh_cmd& c, ConvGeom64* out) {
+  ConvGeom64& g = *out;
   const int64_t B = c.dim[0];
   g.C = (int)c.dim[1]; g.H = (int)c.dim[2]; g.W = (int)c.dim[3]; g.F = (int)c.dim[4];
   g.kh = (int)c.dim[5]; g.kw = (int)c.dim[6]; g.padH = (int)c.dim[7]; g.padW = (int)c.dim[8];
@@ -2309,16 +2516,84 @@ bool gh_try_launch_conv2d_f64_mfma(gh_ctx* ctx, const gh_cmd& c) {
   g.oh = (int)gh_conv_out(g.H, g.kh, g.padH, g.strideH, g.dilH);
   g.ow = (int)gh_conv_out(g.W, g.kw, g.padW, g.strideW, g.dilW);
   const int64_t P = B * g.oh * g.ow, K = (int64_t)g.C * g.kh * g.kw;
-  if (g.F < 16 || P < 256 || K < 8 || P * g.F * K < (int64_t)1 << 22) return false;
-  if (P > 0x7fffffff || K * (int64_t)(g.kh * g.kw) >= ((int64_t)1 << 32)) return false;
+  if (P <= 0 || K <= 0 || P > 0x7fffffff || K * (int64_t)(g.kh * g.kw) >= ((int64_t)1 << 32)) return false;
+  if ((int64_t)g.C * g.H * g.W + (int64_t)(g.padH + 1) * g.W + g.padW >= 0x7fffffff) return false;  // 32-bit offsets inside an image
   g.P = (int)P;
   g.K = (int)K;
   g.mKK = div_magic_of((unsigned)(g.kh * g.kw));
   g.mkw = div_magic_of((unsigned)g.kw);
+  return true;
+}
+
+// Float64 Conv2d on the matrix cores; false = not taken (few filters or a tiny
+// problem: the one-thread-per-result kernel stays).
+bool gh_try_launch_conv2d_f64_mfma(gh_ctx* ctx, const gh_cmd& c) {
+  ConvGeom64 g;
+  if (!conv64_fill(c, &g)) return false;
+  const int64_t P = g.P, K = g.K;
+  if (g.F < 16 || P < 256 || K < 8 || P * g.F * K < (int64_t)1 << 22) return false;
   const int64_t tiles128 = (int64_t)((g.F + 127) / 128) * ((P + 127) / 128);
-  if (g.F <= 32) launch_conv64_cfg<32, 128>(ctx, c, g);
-  else if (tiles128 >= ctx->cu_count) launch_conv64_cfg<128, 128>(ctx, c, g);
-  else launch_conv64_cfg<64, 64>(ctx, c, g);
+  // the smaller tiles do less per k-tile, so they take twice the k range per barrier
+  if (g.F <= 32) launch_conv64_cfg<32, 128, 16>(ctx, c, g);
+  else if (tiles128 >= ctx->cu_count) launch_conv64_cfg<128, 128, 8>(ctx, c, g);
+  else launch_conv64_cfg<64, 64, 16>(ctx, c, g);
+  return true;
+}
+
+// Float64 image gradient of a stride-1 convolution: the forward kernel over dy
+// with mirrored, transposed filters (held at the top of the workspace).
+bool gh_try_launch_conv2d_bwd_data_f64_mfma(gh_ctx* ctx, const gh_cmd& c) {
+  ConvGeom64 g;
+  if (!conv64_fill(c, &g)) return false;
+  const int padH = g.dilH * (g.kh - 1) - g.padH, padW = g.dilW * (g.kw - 1) - g.padW;
+  const int64_t wcount = (int64_t)g.F * g.K;
+  const int64_t wbytes = (wcount * 8 + 255) / 256 * 256;
+  if (g.strideH != 1 || g.strideW != 1 || padH < 0 || padW < 0 || wbytes > ctx->workspace_bytes) return false;
+  gh_cmd f{};
+  f.opcode = GH_OP_CONV2D;
+  f.flags = c.flags;
+  double* wt = (double*)((char*)ctx->workspace + ctx->workspace_bytes - wbytes);
+  f.ptr[0] = c.ptr[0]; f.ptr[1] = (uint64_t)(uintptr_t)wt; f.ptr[2] = c.ptr[2];
+  f.dim[0] = c.dim[0]; f.dim[1] = g.F; f.dim[2] = g.oh; f.dim[3] = g.ow; f.dim[4] = g.C;
+  f.dim[5] = g.kh; f.dim[6] = g.kw; f.dim[7] = padH; f.dim[8] = padW;
+  f.dim[9] = 1; f.dim[10] = 1; f.dim[11] = g.dilH; f.dim[12] = g.dilW;
+  // decide before mirroring whether the forward kernel takes the shape (same tests as above)
+  ConvGeom64 gf;
+  if (!conv64_fill(f, &gf)) return false;
+  if (gf.F < 16 || gf.P < 256 || gf.K < 8 || (int64_t)gf.P * gf.F * gf.K < (int64_t)1 << 22) return false;
+  int64_t blocks = cdiv(wcount, 256);
+  if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
+  hipLaunchKernelGGL(k_flip_filters<double>, dim3((int)blocks), dim3(256), 0, ctx->stream,
+                     (const double*)(uintptr_t)c.ptr[1], wt, g.F, g.C, g.kh, g.kw);
+  return gh_try_launch_conv2d_f64_mfma(ctx, f);
+}
+
+// Float64 filter gradient on the matrix cores, pixel axis cut into slices.
+bool gh_try_launch_conv2d_bwd_filter_f64_mfma(gh_ctx* ctx, const gh_cmd& c) {
+  ConvGeom64 g;
+  if (!conv64_fill(c, &g)) return false;
+  if ((int64_t)g.P * g.F * g.K < (int64_t)1 << 22 || g.P < 64) return false;
+  constexpr int BM = 64, BN = 64, BK = 16;
+  const int64_t tiles = cdiv(g.F, BM) * cdiv(g.K, BN);
+  const int64_t nk = cdiv(g.P, BK);
+  int64_t splits = cdiv(5 * (int64_t)ctx->cu_count / 2, tiles);   // ~2.5 workgroups per CU
+  if (splits > nk / 4) splits = nk / 4;
+  if (splits > 128) splits = 128;
+  const int64_t slab = (int64_t)g.F * g.K * 8;
+  if (ctx->workspace_bytes / slab < splits) splits = ctx->workspace_bytes / slab;
+  if (splits < 1) splits = 1;
+  double* dw = (double*)(uintptr_t)c.ptr[2];
+  const dim3 grid((unsigned)cdiv(g.K, BN), (unsigned)cdiv(g.F, BM), (unsigned)splits);
+  hipLaunchKernelGGL((k_conv2d_wgrad_f64<BM, BN, BK>), grid, dim3(kThreads), 0, ctx->stream,
+                     (const double*)(uintptr_t)c.ptr[0], (const double*)(uintptr_t)c.ptr[1], dw, g, (int)splits,
+                     (double*)ctx->workspace);
+  if (splits > 1) {
+    const int64_t total = (int64_t)g.F * g.K;
+    int64_t blocks = cdiv(total, 256);
+    if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
+    hipLaunchKernelGGL(k_splitk_reduce_f64, dim3((int)blocks), dim3(256), 0, ctx->stream,
+                       (const double*)ctx->workspace, (int)splits, total, dw);
+  }
   return true;
 }
 
@@ -2354,6 +2629,22 @@ int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
   if (gh_dtype_of(c.flags) == GH_F64) {
     const int M = (int)c.dim[0], N = (int)c.dim[1], K = (int)c.dim[2];
     const int64_t batch = c.dim[6] <= 0 ? 1 : c.dim[6];
+    const int64_t tiles64 = (int64_t)((M + 63) / 64) * ((N + 63) / 64);
+    if (batch == 1 && K >= 64 && tiles64 * 4 <= ctx->cu_count && M >= 1 && N >= 1) {
+      const bool ta = c.flags & GH_FLAG_TRANS_A, tb = c.flags & GH_FLAG_TRANS_B;
+      const int64_t lda = c.dim[3], ldb = c.dim[4];
+      const dim3 grid((N + 15) / 16, (M + 15) / 16, 1);
+      const double* A = (const double*)(uintptr_t)c.ptr[0];
+      const double* B = (const double*)(uintptr_t)c.ptr[1];
+      double* C = (double*)(uintptr_t)c.ptr[2];
+      if (K >= 256)
+        hipLaunchKernelGGL((k_dgemm_skinny<8>), grid, dim3(512), 0, ctx->stream, A, B, C, M, N, K, ta ? 1 : lda,
+                           ta ? lda : 1, tb ? 1 : ldb, tb ? ldb : 1, (int)c.dim[5]);
+      else
+        hipLaunchKernelGGL((k_dgemm_skinny<4>), grid, dim3(256), 0, ctx->stream, A, B, C, M, N, K, ta ? 1 : lda,
+                           ta ? lda : 1, tb ? 1 : ldb, tb ? ldb : 1, (int)c.dim[5]);
+      return gh_check_hip(ctx, hipGetLastError(), "dgemm launch");
+    }
     // 128x128 tiles once they fill the device, 64x64 with a longer k-tile below that
     const int64_t tiles128 = (int64_t)((M + 127) / 128) * ((N + 127) / 128) * batch;
     if (tiles128 >= ctx->cu_count) launch_dgemm_cfg<128, 128, 8>(ctx, c, M, N, K, batch);
@@ -2526,7 +2817,7 @@ int gh_launch_conv2d_bwd_data(gh_ctx* ctx, const gh_cmd& c) {
     float* wt = (float*)((char*)ctx->workspace + ctx->workspace_bytes - wbytes);
     int64_t blocks = cdiv((int64_t)F * g.C * g.kh * g.kw, 256);
     if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
-    hipLaunchKernelGGL(k_flip_filters, dim3((int)blocks), dim3(256), 0, ctx->stream, w, wt, F, g.C, g.kh, g.kw);
+    hipLaunchKernelGGL(k_flip_filters<float>, dim3((int)blocks), dim3(256), 0, ctx->stream, w, wt, F, g.C, g.kh, g.kw);
     int rc = gh_check_hip(ctx, hipGetLastError(), "filter mirror launch");
     if (rc) return rc;
     gh_cmd f{};

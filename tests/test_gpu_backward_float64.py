@@ -185,6 +185,13 @@ def test_float64_training_ops_on_the_tape(ctx):
     (2, 4, 10, 11, 6, 1, 1, (0, 0), (1, 1), (1, 1)),
     (2, 2, 12, 9, 3, 5, 3, (2, 1), (2, 1), (1, 1)),
     (1, 3, 13, 13, 4, 3, 3, (2, 2), (1, 2), (2, 2)),
+    # large enough for the matrix-core kernels (filter gradient cut into slices over the pixels,
+    # image gradient as a convolution with mirrored filters)
+    (8, 32, 14, 14, 64, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (32, 1, 28, 28, 32, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (3, 16, 21, 20, 40, 3, 3, (1, 1), (2, 2), (1, 1)),
+    (2, 20, 23, 23, 24, 5, 3, (4, 2), (1, 1), (2, 2)),
+    (5, 70, 7, 7, 130, 3, 3, (1, 1), (1, 1), (1, 1)),
 ])
 def test_conv_gradients_float64(ctx, cfg):
     """Image and filter gradients of Conv2d in float64: relative Frobenius error <= 1e-12
