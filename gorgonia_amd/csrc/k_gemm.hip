@@ -1763,8 +1763,18 @@ __global__ __launch_bounds__(kThreads) void k_conv2d_wgrad_f64(const double* __r
 __global__ __launch_bounds__(256) void k_splitk_reduce_f64(const double* __restrict__ ws, int splits,
                                                            int64_t total, double* __restrict__ out) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    double s = ws[i];
-    for (int z = 1; z < splits; z++) s = s + ws[(int64_t)z * total + i];
+    // slices are added in order; eight loads are issued before their adds so the
+    // chain of additions does not wait for one memory round trip per slice
+    double s = 0.0;
+    int z = 0;
+    for (; z + 8 <= splits; z += 8) {
+      double v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = ws[(int64_t)(z + u) * total + i];
+#pragma unroll
+      for (int u = 0; u < 8; u++) s = s + v[u];
+    }
+    for (; z < splits; z++) s = s + ws[(int64_t)z * total + i];
     out[i] = s;
   }
 }
@@ -2578,7 +2588,7 @@ bool gh_try_launch_conv2d_bwd_filter_f64_mfma(gh_ctx* ctx, const gh_cmd& c) {
   const int64_t nk = cdiv(g.P, BK);
   int64_t splits = cdiv(5 * (int64_t)ctx->cu_count / 2, tiles);   // ~2.5 workgroups per CU
   if (splits > nk / 4) splits = nk / 4;
-  if (splits > 128) splits = 128;
+  if (splits > 512) splits = 512;
   const int64_t slab = (int64_t)g.F * g.K * 8;
   if (ctx->workspace_bytes / slab < splits) splits = ctx->workspace_bytes / slab;
   if (splits < 1) splits = 1;
