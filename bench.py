@@ -168,9 +168,9 @@ def bench_convnet_kernels(ctx, batch, iters):
     return out
 
 
-def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=True):
+def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=True, dtype=np.float32):
     from gorgonia_amd import configs, graph as G
-    inp = configs.convnet_inputs(batch)
+    inp = {k: v.astype(dtype) for k, v in configs.convnet_inputs(batch).items()}
     g = G.NewGraph()
     # same graph as configs.build_convnet, with the input batch optionally resident
     h = G.NewTensor(g, inp["x"], resident=resident_input)
@@ -278,13 +278,13 @@ def bench_mlp(steps, warmup, resident_input=True):
     return dt / steps * 1e3, result, inp
 
 
-def bench_convnet_train(steps, warmup, batch=128):
+def bench_convnet_train(steps, warmup, batch=128, dtype=np.float32):
     """Config 4 as a training step: forward, every layer's gradient, RMSProp
     update (examples/convnet/main.go:195) of the resident weights; only the
     128x10 output leaves the device."""
     from gorgonia_amd import configs, graph as G
-    inp = configs.convnet_inputs(batch)
-    onehot = np.zeros((batch, 10), np.float32)
+    inp = {k: v.astype(dtype) for k, v in configs.convnet_inputs(batch).items()}
+    onehot = np.zeros((batch, 10), dtype)
     onehot[np.arange(batch), np.arange(batch) % 10] = 1.0
     g, outs = configs.build_convnet_train(inp, onehot, 0.01, read_grads=False, solver="rmsprop")
     m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING)
@@ -442,6 +442,28 @@ def main():
         train = {"ms_per_step": round(ms_train, 4), "images_s": round(128 / ms_train * 1e3, 1)}
         log(f"convnet training step: {ms_train:.4f} ms/step  {128 / ms_train * 1e3:.0f} images/s")
 
+    # the same network in float64, the default dtype of the reference's example
+    # (examples/convnet/main.go:28): forward and training step on the fp64 matrix cores
+    f64 = None
+    if not only or "float64" in only:
+        n64 = max(20, a.steps // 4)
+        ms64, out64, inp64, _ = bench_convnet(n64, a.warmup, graph_replay=not a.eager_timing, dtype=np.float64)
+        ms64t, _, _ = bench_convnet_train(n64, a.warmup, dtype=np.float64)
+        f64 = {"forward_ms_per_step": round(ms64, 4), "forward_images_s": round(128 / ms64 * 1e3, 1),
+               "training_ms_per_step": round(ms64t, 4), "training_images_s": round(128 / ms64t * 1e3, 1)}
+        if not a.skip_cpu:
+            from oracle import binding as O
+            O.set_threads(min(16, os.cpu_count() or 1))
+            h = inp64["x"]
+            for i in range(3):
+                h = O.conv2d(h, inp64[f"w{i}"], (1, 1), (1, 1), (1, 1))
+                h = O.maxpool2d(O.relu(h).reshape(h.shape), (2, 2), (0, 0), (2, 2))
+            h = O.relu(h.reshape(128, -1) @ inp64["w3"]).reshape(128, -1)
+            ref64 = O.softmax(h @ inp64["w4"])
+            O.set_threads(1)
+            f64["forward_rel_frobenius_vs_oracle"] = float(np.linalg.norm(out64 - ref64) / np.linalg.norm(ref64))
+        log(f"float64 convnet: forward {ms64:.4f} ms/step, training {ms64t:.4f} ms/step")
+
     iters = 30
     conv_k = bench_convnet_kernels(ctx, 128, iters) if not only or "convnet" in only else {}
     elem = bench_elementwise(ctx, iters) if not only or "elementwise" in only else {}
@@ -534,7 +556,7 @@ def main():
             "convnet_images_s_four_machines_four_host_threads": four_images_s and round(four_images_s, 1),
             "convnet_parallel_machines_outputs_equal_single": (bool(all(np.array_equal(o, gpu_out) for o in two_out + four_out))
                                                                if two_out else None),
-            "mlp_forward": mlp, "yolo_shaped_forward": yolo, "convnet_training_step": train, "backward_kernels": bwd, "convnet_kernels": conv_k, "elementwise": elem, "linalg": lin, "parity": parity,
+            "mlp_forward": mlp, "yolo_shaped_forward": yolo, "convnet_training_step": train, "convnet_float64": f64, "backward_kernels": bwd, "convnet_kernels": conv_k, "elementwise": elem, "linalg": lin, "parity": parity,
         },
     }
     print(json.dumps(line), flush=True)
