@@ -2544,9 +2544,12 @@ bool gh_try_launch_conv2d_f64_mfma(gh_ctx* ctx, const gh_cmd& c) {
   if (g.F < 16 || P < 256 || K < 8 || P * g.F * K < (int64_t)1 << 22) return false;
   const int64_t tiles128 = (int64_t)((g.F + 127) / 128) * ((P + 127) / 128);
   // the smaller tiles do less per k-tile, so they take twice the k range per barrier
+  const int64_t tiles64 = (int64_t)((g.F + 63) / 64) * ((P + 63) / 64);
   if (g.F <= 32) launch_conv64_cfg<32, 128, 16>(ctx, c, g);
   else if (tiles128 >= ctx->cu_count) launch_conv64_cfg<128, 128, 8>(ctx, c, g);
-  else launch_conv64_cfg<64, 64, 16>(ctx, c, g);
+  else if (tiles64 >= ctx->cu_count) launch_conv64_cfg<64, 64, 16>(ctx, c, g);
+  else launch_conv64_cfg<32, 64, 16>(ctx, c, g);   // too few 64x64 tiles for the device (measured: 97 against 108 us on
+                                                   // 128x128x7x7 -> 64 filters, no gain once every CU has a 64x64 tile)
   return true;
 }
 
