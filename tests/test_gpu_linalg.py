@@ -319,3 +319,37 @@ def test_batched_matmul_float64_large_tiles(ctx, ta, tb):
         ctx.free(p)
     want = (A.transpose(0, 2, 1) if ta else A) @ (B.transpose(0, 2, 1) if tb else B)
     assert np.array_equal(got, want)
+
+
+def test_matmul_float64_views_sweep(ctx):
+    """Seeded sweep of the float64 product over all three kernels (small-output, 64x64 and
+    128x128 tiles): every transpose, odd and even extents, operands that are windows of
+    larger buffers (leading dimension beyond the row, base 8 bytes off a 16-byte boundary)
+    and a strided output.  Integer data: every result must be exact, and the output's
+    padding columns must stay untouched."""
+    from gorgonia_amd import _ffi
+    rng = np.random.default_rng(23)
+    shapes = [(70, 96, 33), (130, 200, 64), (17, 300, 9), (200, 66, 140), (512, 40, 512), (1100, 16, 1300),
+              (257, 129, 1027), (64, 1024, 48)]
+    for idx, (m, k, n) in enumerate(shapes):
+        for ta in (False, True):
+            for tb in (False, True):
+                pa, pb, pc = int(rng.integers(0, 4)), int(rng.integers(0, 4)), int(rng.integers(0, 3))
+                oa, ob = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+                ra, ca = (k, m) if ta else (m, k)
+                rb, cb = (n, k) if tb else (k, n)
+                bufA = rng.integers(-6, 7, ra * (ca + pa) + oa).astype(np.float64)
+                bufB = rng.integers(-6, 7, rb * (cb + pb) + ob).astype(np.float64)
+                A = bufA[oa:].reshape(ra, ca + pa)[:, :ca]
+                B = bufB[ob:].reshape(rb, cb + pb)[:, :cb]
+                want = (A.T if ta else A) @ (B.T if tb else B)
+                Cbuf = np.full((m, n + pc), -77.0)
+                dA, dB, dC = ctx.upload(bufA), ctx.upload(bufB), ctx.upload(Cbuf)
+                ctx.run(D.cmd_gemm(dA + 8 * oa, dB + 8 * ob, dC, m, n, k, lda=ca + pa, ldb=cb + pb, ldc=n + pc,
+                                   trans_a=ta, trans_b=tb, dtype=_ffi.F64))
+                got = ctx.d2h(dC, (m, n + pc), dtype=np.float64)
+                for p in (dA, dB, dC):
+                    ctx.free(p)
+                tag = f"case {idx} {m}x{k}x{n} ta={ta} tb={tb} pads {pa},{pb},{pc} offs {oa},{ob}"
+                assert np.array_equal(got[:, :n], want), tag
+                assert np.all(got[:, n:] == -77.0), tag + ": padding written"

@@ -177,3 +177,39 @@ def test_tape_float64_network(ctx):
     want = O.softmax(ref.reshape(2, 64) @ w2)
     assert np.allclose(out, want, rtol=1e-12, atol=1e-15)
     m.Close()
+
+
+def test_conv2d_float64_seeded_geometry_sweep(ctx):
+    """Forward, image gradient and filter gradient in float64 over seeded geometries large
+    enough for the matrix-core kernels (kernel 1..5, stride 1..2, dilation 1..2, any padding
+    that keeps the output non-empty), integer data: all three must be exact."""
+    rng = np.random.default_rng(31)
+    done = 0
+    while done < 12:
+        B, C, F = int(rng.integers(2, 7)), int(rng.integers(1, 40)), int(rng.integers(16, 90))
+        H, W = int(rng.integers(9, 26)), int(rng.integers(9, 26))
+        kh, kw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        stride = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        dil = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        pad = (int(rng.integers(0, dil[0] * (kh - 1) + 1)), int(rng.integers(0, dil[1] * (kw - 1) + 1)))
+        if dil[0] * (kh - 1) + 1 > H + 2 * pad[0] or dil[1] * (kw - 1) + 1 > W + 2 * pad[1]:
+            continue
+        x = rng.integers(-3, 4, (B, C, H, W)).astype(np.float64)
+        w = rng.integers(-3, 4, (F, C, kh, kw)).astype(np.float64)
+        want = O.conv2d(x, w, pad, stride, dil)
+        dyv = rng.integers(-3, 4, want.shape).astype(np.float64)
+        dx_ref, dw_ref = O.conv2d_bwd(x, w, dyv, pad, stride, dil)
+        px, pw, pdy = ctx.upload(x), ctx.upload(w), ctx.upload(dyv)
+        py, pdx, pdw = ctx.malloc(want.size * 8), ctx.malloc(x.size * 8), ctx.malloc(w.size * 8)
+        ctx.run([D.cmd_conv2d(px, pw, py, B, C, H, W, F, kh, kw, pad, stride, dil, dtype=F64),
+                 D.cmd_conv2d_bwd_data(pdy, pw, pdx, B, C, H, W, F, kh, kw, pad, stride, dil, dtype=F64),
+                 D.cmd_conv2d_bwd_filter(px, pdy, pdw, B, C, H, W, F, kh, kw, pad, stride, dil, dtype=F64)])
+        got = ctx.d2h(py, want.shape, np.float64)
+        dx, dw = ctx.d2h(pdx, x.shape, np.float64), ctx.d2h(pdw, w.shape, np.float64)
+        for p in (px, pw, pdy, py, pdx, pdw):
+            ctx.free(p)
+        tag = f"B{B} C{C} F{F} {H}x{W} k{kh}x{kw} pad{pad} stride{stride} dil{dil}"
+        assert np.array_equal(got, want), "forward " + tag
+        assert np.array_equal(dx, dx_ref), "image gradient " + tag
+        assert np.array_equal(dw, dw_ref), "filter gradient " + tag
+        done += 1
