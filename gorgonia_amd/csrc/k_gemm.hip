@@ -1502,9 +1502,10 @@ __device__ __forceinline__ void dmfma_tile_loop_deep(double* lds, LA& la0, LB& l
 // there are at least three k-tiles (measured on the float64 convnet's layers:
 // 13-21 % faster on 32x64 tiles, 3-7 % on 64x64 and 32x128); with one or two
 // k-tiles the second register set only fetches a tile twice (a 9-tap first layer
-// ran 30 % slower), and 128-wide tiles have MFMA phases long enough to cover a
-// single tile in flight.  The filter-gradient kernel keeps the plain loop: its
-// gathers gained nothing from the second set.
+// ran 30 % slower), and the 128x128 tiles lose with the second set (2048^3
+// product 358 -> 399 us): their MFMA phase already covers one tile in flight.
+// The filter-gradient kernel keeps the plain loop: its gathers gained nothing
+// from the second set.
 template <int BM, int BN, int BK, class LA, class LB>
 __device__ __forceinline__ void dmfma_tile_loop_auto(double* lds, LA& la, LB& lb, int m0, int n0, int nkt,
                                                      f64x4 (&acc)[BM / 32][BN / 32]) {
