@@ -87,6 +87,7 @@ SYMBOLS = {
     "gh_memcpy_d2h": (C.c_int, [_P, _P, C.c_uint64, C.c_int64]),
     "gh_memcpy_d2d": (C.c_int, [_P, C.c_uint64, C.c_uint64, C.c_int64]),
     "gh_submit": (C.c_int, [_P, C.POINTER(GhCmd), C.c_int]),
+    "gh_submit_noalloc": (C.c_int, [_P, C.POINTER(GhCmd), C.c_int]),
     "gh_validate": (C.c_int, [C.POINTER(GhCmd), C.c_int, C.c_char_p, C.c_int]),
     "gh_conv2d_can_pool": (C.c_int, [C.POINTER(GhCmd)]),
     "gh_gemm_can_softmax": (C.c_int, [C.POINTER(GhCmd)]),

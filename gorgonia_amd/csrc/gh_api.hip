@@ -15,6 +15,38 @@ int gh_fail(gh_ctx* ctx, int code, const std::string& msg) {
   return code;
 }
 
+// Scratch of gh_submit_noalloc: part of the library's device image, so it exists
+// on every GPU the library runs on from load time to process exit and no call
+// has to allocate it.  In host code this name only stands for the symbol; the
+// per-device address comes from hipGetSymbolAddress (static_scratch below) and
+// is the only thing ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[GH_NOALLOC_SCRATCH_BYTES];
+
+static constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices] = {};   // address of `scratch` on device i; filled by gh_init
+
+// Address of the static scratch on `device`, which must be current.  Resolved
+// once per device (every GPU holds its own copy at its own address).
+static hipError_t static_scratch(int device, void** out) {
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_scratch_ptr[device] = p;
+  }
+  *out = g_scratch_ptr[device];
+  return hipSuccess;
+}
+
+int gh_ws_short(gh_ctx* ctx, int64_t need) {
+  if (!ctx->ws_strict) return GH_OK;
+  return gh_fail(ctx, GH_EINVAL,
+                 "gh_submit_noalloc: operator needs " + std::to_string(need) + " bytes of scratch, the fixed scratch holds " +
+                     std::to_string((int64_t)GH_NOALLOC_SCRATCH_BYTES) + " (use gh_submit)");
+}
+
 int gh_check_hip(gh_ctx* ctx, hipError_t e, const char* what) {
   if (e == hipSuccess) return GH_OK;
   std::string m = std::string(what) + ": " + hipGetErrorString(e);
@@ -65,12 +97,18 @@ int gh_init(int device, int64_t arena_bytes, gh_ctx** out) {
     }
     ctx->arena_bytes = arena_bytes;
   }
-  // Context-owned scratch: split-K partial sums and reduction flags.
+  // Context-owned scratch: split-K partial sums, reduction partials, mirrored
+  // filters.  Mandatory: the launchers index it without asking again.
   ctx->workspace_bytes = 64ll << 20;
-  if (hipMalloc(&ctx->workspace, (size_t)ctx->workspace_bytes) != hipSuccess) {
+  void* fixed = nullptr;
+  if (hipMalloc(&ctx->workspace, (size_t)ctx->workspace_bytes) != hipSuccess ||
+      static_scratch(device, &fixed) != hipSuccess) {
     (void)hipGetLastError();
-    ctx->workspace = nullptr;
-    ctx->workspace_bytes = 0;
+    if (ctx->workspace) hipFree(ctx->workspace);
+    if (ctx->arena) hipFree(ctx->arena);
+    hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return GH_EOOM;
   }
   *out = ctx;
   return GH_OK;
@@ -246,9 +284,7 @@ int gh_validate(const gh_cmd* cmds, int n, char* msg, int msg_len) {
   return GH_OK;
 }
 
-int gh_submit(gh_ctx* ctx, const gh_cmd* cmds, int n) {
-  if (!ctx || n < 0 || (n > 0 && !cmds)) return GH_EINVAL;
-  if (ctx->err) return ctx->err;
+static int submit_cmds(gh_ctx* ctx, const gh_cmd* cmds, int n) {
   for (int i = 0; i < n; i++) {
     std::string m;
     int rc = gh_validate_cmd(cmds[i], m);
@@ -269,6 +305,33 @@ int gh_submit(gh_ctx* ctx, const gh_cmd* cmds, int n) {
     if (rc) return rc;
   }
   return GH_OK;
+}
+
+int gh_submit(gh_ctx* ctx, const gh_cmd* cmds, int n) {
+  if (!ctx || n < 0 || (n > 0 && !cmds)) return GH_EINVAL;
+  if (ctx->err) return ctx->err;
+  return submit_cmds(ctx, cmds, n);
+}
+
+int gh_submit_noalloc(gh_ctx* ctx, const gh_cmd* cmds, int n) {
+  if (!ctx || n < 0 || (n > 0 && !cmds)) return GH_EINVAL;
+  if (ctx->err) return ctx->err;
+  void* fixed = ctx->device >= 0 && ctx->device < kMaxDevices ? g_scratch_ptr[ctx->device] : nullptr;
+  if (!fixed) return gh_fail(ctx, GH_ESTATE, "gh_submit_noalloc: the fixed scratch was not resolved on this device");
+  // Same launchers, same plans: only the scratch they index changes, and a plan
+  // that would not fit it is refused instead of shrunk (gh_ws_short).  Nothing
+  // in the scratch has to start at zero: every slab and partial is written
+  // before it is read.
+  void* const keep = ctx->workspace;
+  const int64_t keep_bytes = ctx->workspace_bytes;
+  ctx->workspace = fixed;
+  ctx->workspace_bytes = GH_NOALLOC_SCRATCH_BYTES;
+  ctx->ws_strict = true;
+  const int rc = submit_cmds(ctx, cmds, n);
+  ctx->ws_strict = false;
+  ctx->workspace = keep;
+  ctx->workspace_bytes = keep_bytes;
+  return rc;
 }
 
 int gh_sync(gh_ctx* ctx) {

@@ -27,7 +27,16 @@ struct gh_ctx {
   // scratch owned by the context (split-K partials, reduction flags)
   void* workspace = nullptr;
   int64_t workspace_bytes = 0;
+  // set while gh_submit_noalloc runs: the scratch is the library's fixed array and a
+  // plan may not shrink to fit it (results must not depend on the scratch size)
+  bool ws_strict = false;
 };
+
+// A launcher calls this where `need` bytes of scratch do not fit the workspace,
+// before it shrinks its plan (fewer split-K slices, a kernel without scratch).
+// Returns GH_OK to go on shrinking; under gh_submit_noalloc it records the
+// sticky error instead and returns its code, which the launcher passes on.
+int gh_ws_short(gh_ctx* ctx, int64_t need);
 
 // Record a sticky error on the context and return its code.
 int gh_fail(gh_ctx* ctx, int code, const std::string& msg);

@@ -2217,7 +2217,10 @@ inline int clamp_splits(gh_ctx* ctx, int64_t splits, int64_t M, int64_t N, int64
   const int64_t slab = M * N * 4;
   if (slab <= 0 || !ctx->workspace) return 1;
   const int64_t fit = ctx->workspace_bytes / slab;
-  if (splits > fit) splits = fit;
+  if (splits > fit) {
+    if (gh_ws_short(ctx, splits * slab)) return 1;   // the caller returns ctx->err
+    splits = fit;
+  }
   return splits < 1 ? 1 : (int)splits;
 }
 
@@ -2501,12 +2504,18 @@ int try_launch_conv3_cc(gh_ctx* ctx, const gh_cmd& c) {
       }
       if (vs > g.nchunks) vs = g.nchunks;
       if (vs < 1) vs = 1;
-      while (vs > 1 && (int64_t)vs * F * g.P * 4 > ctx->workspace_bytes) vs--;
+      if (vs > 1 && (int64_t)vs * F * g.P * 4 > ctx->workspace_bytes) {
+        if (int rc = gh_ws_short(ctx, (int64_t)vs * F * g.P * 4)) return rc;
+        while (vs > 1 && (int64_t)vs * F * g.P * 4 > ctx->workspace_bytes) vs--;
+      }
     }
     g.vsplits = vs;
     splits = 1;
   }
-  while (splits > 1 && (int64_t)splits * F * g.P * 4 > ctx->workspace_bytes) splits--;
+  if (splits > 1 && (int64_t)splits * F * g.P * 4 > ctx->workspace_bytes) {
+    if (int rc = gh_ws_short(ctx, (int64_t)splits * F * g.P * 4)) return rc;
+    while (splits > 1 && (int64_t)splits * F * g.P * 4 > ctx->workspace_bytes) splits--;
+  }
 #define GH_CONV3(BM_, BN_)                                                                        \
   (per_thread <= 8 ? launch_conv3_cfg<BM_, BN_, CC, 2, 8>(ctx, c, g, splits, lds)                 \
                    : launch_conv3_cfg<BM_, BN_, CC, 2, 16>(ctx, c, g, splits, lds))
@@ -2654,7 +2663,8 @@ bool gh_try_launch_conv2d_bwd_data_f64_mfma(gh_ctx* ctx, const gh_cmd& c) {
   const int padH = g.dilH * (g.kh - 1) - g.padH, padW = g.dilW * (g.kw - 1) - g.padW;
   const int64_t wcount = (int64_t)g.F * g.K;
   const int64_t wbytes = (wcount * 8 + 255) / 256 * 256;
-  if (g.strideH != 1 || g.strideW != 1 || padH < 0 || padW < 0 || wbytes > ctx->workspace_bytes) return false;
+  if (g.strideH != 1 || g.strideW != 1 || padH < 0 || padW < 0) return false;
+  if (wbytes > ctx->workspace_bytes) return gh_ws_short(ctx, wbytes) != GH_OK;   // true: the caller returns ctx->err
   gh_cmd f{};
   f.opcode = GH_OP_CONV2D;
   f.flags = c.flags;
@@ -2686,7 +2696,10 @@ bool gh_try_launch_conv2d_bwd_filter_f64_mfma(gh_ctx* ctx, const gh_cmd& c) {
   if (splits > nk / 4) splits = nk / 4;
   if (splits > 512) splits = 512;
   const int64_t slab = (int64_t)g.F * g.K * 8;
-  if (ctx->workspace_bytes / slab < splits) splits = ctx->workspace_bytes / slab;
+  if (splits > 1 && ctx->workspace_bytes / slab < splits) {
+    if (gh_ws_short(ctx, splits * slab)) return true;   // the caller returns ctx->err
+    splits = ctx->workspace_bytes / slab;
+  }
   if (splits < 1) splits = 1;
   double* dw = (double*)(uintptr_t)c.ptr[2];
   const dim3 grid((unsigned)cdiv(g.K, BN), (unsigned)cdiv(g.F, BM), (unsigned)splits);
@@ -2763,6 +2776,7 @@ int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
     return gh_fail(ctx, GH_EINVAL, "gemm: no fused softmax for this shape (see gh_gemm_can_softmax)");
   const int64_t batch = c.dim[6] <= 0 ? 1 : c.dim[6];
   const TilePlan p = plan_tiles(ctx, c.dim[0], c.dim[1], c.dim[2], batch, false);
+  if (ctx->err) return ctx->err;
   if (p.tile == kTile128) return launch_sgemm_cfg<128, 128, 2>(ctx, c, p.splits);
   return launch_sgemm_cfg<64, 64, 2>(ctx, c, p.splits);
 }
@@ -2830,6 +2844,7 @@ int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
   g.P = (int)c.dim[0] * g.oh * g.ow;
   const int F = (int)c.dim[4], K = g.C * g.kh * g.kw;
   const TilePlan p = plan_tiles(ctx, F, g.P, K, 1, true);
+  if (ctx->err) return ctx->err;
   if (p.tile == kTile128) return launch_conv_k<128, 128, 2>(ctx, c, g, F, K, p.splits);
   if (p.tile == kTile32x256) return launch_conv_k<32, 256, 1>(ctx, c, g, F, K, p.splits);
   return launch_conv_k<64, 64, 2>(ctx, c, g, F, K, p.splits);
@@ -2856,7 +2871,12 @@ int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
   if (conv_direct_shape(c) && F <= 65535) {
     const int B = (int)c.dim[0];
     int G = B < 64 ? B : 64;
-    while (G > 1 && (int64_t)G * F * CKK * 4 > ctx->workspace_bytes) G--;
+    if ((int64_t)G * F * CKK * 4 > ctx->workspace_bytes) {
+      if (int rc = gh_ws_short(ctx, (int64_t)G * F * CKK * 4)) return rc;
+      while (G > 1 && (int64_t)G * F * CKK * 4 > ctx->workspace_bytes) G--;
+      if ((int64_t)G * F * CKK * 4 > ctx->workspace_bytes)
+        return gh_fail(ctx, GH_ESTATE, "conv2d filter gradient: partial sums do not fit the workspace");
+    }
     float* wsd = (float*)ctx->workspace;
     const float* xd = (const float*)(uintptr_t)c.ptr[0];
     const float* dyd = (const float*)(uintptr_t)c.ptr[1];
@@ -2884,7 +2904,10 @@ int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
   if (splits > nk / 4) splits = nk / 4;
   if (splits > 64) splits = 64;
   const int64_t slab = (int64_t)F * CKK * 4;
-  if (ctx->workspace_bytes / slab < splits) splits = ctx->workspace_bytes / slab;
+  if (splits > 1 && ctx->workspace_bytes / slab < splits) {
+    if (int rc = gh_ws_short(ctx, splits * slab)) return rc;
+    splits = ctx->workspace_bytes / slab;
+  }
   if (splits < 1) splits = 1;
   const float* x = (const float*)(uintptr_t)c.ptr[0];
   const float* dy = (const float*)(uintptr_t)c.ptr[1];
@@ -2917,7 +2940,10 @@ int gh_launch_conv2d_bwd_data(gh_ctx* ctx, const gh_cmd& c) {
   float* dx = (float*)(uintptr_t)c.ptr[2];
   const int64_t wbytes = ((int64_t)F * g.C * g.kh * g.kw * 4 + 255) / 256 * 256;
   const int padH = g.dilH * (g.kh - 1) - g.padH, padW = g.dilW * (g.kw - 1) - g.padW;
-  if (g.strideH == 1 && g.strideW == 1 && padH >= 0 && padW >= 0 && wbytes <= ctx->workspace_bytes / 2) {
+  const bool mirror_shape = g.strideH == 1 && g.strideW == 1 && padH >= 0 && padW >= 0;
+  if (mirror_shape && wbytes > ctx->workspace_bytes / 2)
+    if (int rc = gh_ws_short(ctx, 2 * wbytes)) return rc;
+  if (mirror_shape && wbytes <= ctx->workspace_bytes / 2) {
     // mirrored filters live at the top of the workspace; the forward launch
     // below may use what is left of it for its own split-K slabs
     float* wt = (float*)((char*)ctx->workspace + ctx->workspace_bytes - wbytes);

@@ -288,7 +288,7 @@ int gh_launch_conv2d_bwd_data_f64(gh_ctx* ctx, const gh_cmd& c) {
   const int64_t total = (int64_t)g.B * g.C * g.H * g.W;
   if (total <= 0) return GH_OK;
   if (gh_try_launch_conv2d_bwd_data_f64_mfma(ctx, c))
-    return gh_check_hip(ctx, hipGetLastError(), "conv2d image gradient launch");
+    return ctx->err ? ctx->err : gh_check_hip(ctx, hipGetLastError(), "conv2d image gradient launch");
   hipLaunchKernelGGL(k_conv2d_bwd_data_f64, dim3(blocks_for(ctx, total)), dim3(kBlock), 0, ctx->stream,
                      (const double*)(uintptr_t)c.ptr[0], (const double*)(uintptr_t)c.ptr[1],
                      (double*)(uintptr_t)c.ptr[2], g, total);
@@ -300,7 +300,7 @@ int gh_launch_conv2d_bwd_filter_f64(gh_ctx* ctx, const gh_cmd& c) {
   const int64_t total = (int64_t)g.F * g.C * g.kh * g.kw;
   if (total <= 0) return GH_OK;
   if (gh_try_launch_conv2d_bwd_filter_f64_mfma(ctx, c))
-    return gh_check_hip(ctx, hipGetLastError(), "conv2d filter gradient launch");
+    return ctx->err ? ctx->err : gh_check_hip(ctx, hipGetLastError(), "conv2d filter gradient launch");
   hipLaunchKernelGGL(k_conv2d_bwd_filter_f64, dim3(blocks_for(ctx, total)), dim3(kBlock), 0, ctx->stream,
                      (const double*)(uintptr_t)c.ptr[0], (const double*)(uintptr_t)c.ptr[1],
                      (double*)(uintptr_t)c.ptr[2], g, total);
@@ -311,7 +311,7 @@ int gh_launch_conv2d_f64(gh_ctx* ctx, const gh_cmd& c) {
   const Conv64 g = conv64_geom(c);
   const int64_t total = (int64_t)g.B * g.F * g.oh * g.ow;
   if (total <= 0) return GH_OK;
-  if (gh_try_launch_conv2d_f64_mfma(ctx, c)) return gh_check_hip(ctx, hipGetLastError(), "conv2d launch");
+  if (gh_try_launch_conv2d_f64_mfma(ctx, c)) return ctx->err ? ctx->err : gh_check_hip(ctx, hipGetLastError(), "conv2d launch");
   hipLaunchKernelGGL(k_conv2d_f64, dim3(blocks_for(ctx, total)), dim3(kBlock), 0, ctx->stream,
                      (const double*)(uintptr_t)c.ptr[0], (const double*)(uintptr_t)c.ptr[1],
                      (double*)(uintptr_t)c.ptr[2], g, total);

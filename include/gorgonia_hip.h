@@ -263,6 +263,20 @@ GH_API int gh_memcpy_d2d(gh_ctx* ctx, gh_devptr dst, gh_devptr src, int64_t byte
  * A command that fails validation enqueues nothing from that command on and
  * returns GH_EINVAL/GH_ENOFUNC with the index in gh_last_error(). */
 GH_API int gh_submit(gh_ctx* ctx, const gh_cmd* cmds, int n);
+/* No counterpart in the reference.  For callers that cannot allocate device
+ * memory around a submit - code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc: gh_submit with the same commands, kernels and
+ * results, except that the operators' scratch (split-K partial sums, reduction
+ * partials, mirrored filters for the image gradient) is a fixed array of
+ * GH_NOALLOC_SCRATCH_BYTES inside the library's device image instead of the
+ * context's workspace, and the call itself allocates and frees nothing.  An
+ * operator whose plan needs more scratch than that is refused with GH_EINVAL
+ * (message names the need) and nothing from it on is enqueued; plans never
+ * shrink to fit, so accepted commands store the bits gh_submit stores.  All
+ * contexts on one GPU share the array: calls whose work overlaps in time on one
+ * GPU (two contexts, two threads) race on it. */
+#define GH_NOALLOC_SCRATCH_BYTES (16 << 20)
+GH_API int gh_submit_noalloc(gh_ctx* ctx, const gh_cmd* cmds, int n);
 /* Validate only: same checks as gh_submit, touches no device. */
 GH_API int gh_validate(const gh_cmd* cmds, int n, char* msg, int msg_len);
 /* 1 when this CONV2D command may carry GH_FLAG_CONV_POOL2 (a convolution whose
