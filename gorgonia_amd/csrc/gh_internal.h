@@ -69,6 +69,10 @@ int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_gemv(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_outer(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c);
+// small-image 3x3 convolution (k_conv_small.hip): -1 when the shape is not one it takes
+int gh_try_launch_conv_small(gh_ctx* ctx, const gh_cmd& c);
+bool gh_conv_small_takes(const gh_cmd& c);
+bool gh_conv_small_can_pool(const gh_cmd& c);
 int gh_launch_maxpool2d(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_bn_infer(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_softmax(gh_ctx* ctx, const gh_cmd& c);

@@ -24,6 +24,7 @@
 #include <type_traits>
 
 #include "gh_internal.h"
+#include "gh_conv_common.h"
 
 namespace {
 
@@ -33,39 +34,6 @@ typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kThreads = 256;
-
-// Epilogue activations in the reference's arithmetic form (nn.go:83-163).
-__device__ __forceinline__ float act_apply(float v, int act, float alpha) {
-  if (act == 1) return v * (v >= 0.0f ? 1.0f : 0.0f);
-  if (act == 2) {
-    const float pos = v * (v >= 0.0f ? 1.0f : 0.0f);
-    const float neg = v * (v < 0.0f ? 1.0f : 0.0f);
-    const float na = neg * alpha;
-    return pos + na;
-  }
-  return v;
-}
-
-// Operators riding in a convolution's epilogue, applied per stored value in this
-// order: BatchNorm in eval mode with BN_INFER's arithmetic (op_nn.go:1559-1584:
-// a = 1/sqrt(var+eps), b = -mean*a, y = x*a + b, then gamma*y, then + beta, each
-// step rounded), then the activation.  Null mean: no BatchNorm.
-struct ConvTail {
-  const float* mean; const float* var; const float* gamma; const float* beta;
-  float eps; int act; float alpha;
-};
-
-__device__ __forceinline__ float tail_apply(const ConvTail& t, int f, float v) {
-  if (t.mean) {
-    const float a = 1.0f / sqrtf(t.var[f] + t.eps);
-    const float b = -t.mean[f] * a;
-    v = v * a;
-    v = v + b;
-    if (t.gamma) v = t.gamma[f] * v;
-    if (t.beta) v = v + t.beta[f];
-  }
-  return act_apply(v, t.act, t.alpha);
-}
 
 // ---- operand loaders ---------------------------------------------------------
 // A loader moves one R x BK (or BK x R) operand tile: load() global->registers,
@@ -2192,20 +2160,6 @@ inline bool al16(uint64_t p) { return (p & 15u) == 0; }
 enum { kTile128 = 0, kTile64 = 1, kTile32x256 = 2 };
 struct TilePlan { int tile; int splits; };
 
-inline ConvTail conv_tail(const gh_cmd& c) {
-  ConvTail t{};
-  if (c.flags & GH_FLAG_CONV_BN) {
-    t.mean = (const float*)(uintptr_t)c.ptr[3];
-    t.var = (const float*)(uintptr_t)c.ptr[4];
-    t.gamma = (c.flags & GH_FLAG_HAS_GAMMA) ? (const float*)(uintptr_t)c.ptr[5] : nullptr;
-    t.beta = (c.flags & GH_FLAG_HAS_BETA) ? (const float*)(uintptr_t)c.ptr[6] : nullptr;
-    t.eps = c.f[1];
-  }
-  t.act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
-  t.alpha = c.f[0];
-  return t;
-}
-
 inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Largest split count whose [splits][M][N] slabs fit the context workspace.
@@ -2829,6 +2783,8 @@ static int launch_conv_direct(gh_ctx* ctx, const gh_cmd& c) {
 int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
   if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_conv2d_f64(ctx, c);
   if (conv_direct_shape(c) && !getenv("GORGONIA_HIP_CONV_NO_DIRECT")) return launch_conv_direct(ctx, c);
+  const int rcs = gh_try_launch_conv_small(ctx, c);
+  if (rcs >= 0) return rcs;
   const int rc3 = try_launch_conv3(ctx, c);
   if (rc3 >= 0) return rc3;
   if (c.flags & GH_FLAG_CONV_POOL2)
@@ -3027,6 +2983,9 @@ extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {
     return oh >= 2 && ow >= 2;
   }
   if (getenv("GORGONIA_HIP_CONV_NO_POOL")) return 0;  // tuning switch: keep MaxPool2D a kernel of its own
+  // a shape the small-image kernel takes is pooled there or not at all (the plain and the
+  // pooled command must sum in the same order)
+  if (gh_conv_small_takes(*c)) return gh_conv_small_can_pool(*c) ? 1 : 0;
   Conv3Geom g;
   int BM, BN, per_thread;
   size_t lds;

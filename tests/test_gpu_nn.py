@@ -191,6 +191,46 @@ def test_conv_epilogue_pool_bit_exact(ctx, cfg):
                                     pool2=True), chain, f"conv+bn+leaky+pool {cfg}")
 
 
+# shapes the small-image kernel takes (3x3, images up to 16x16, 16/32/64/128 channels): ragged filter
+# tiles, batches that do not fill the last workgroup, no padding, odd and even extents, H != W
+SMALL_IMAGE_CASES = [(7, 16, 7, 7, 10, 1), (5, 32, 14, 14, 50, 1), (9, 64, 7, 7, 33, 1), (3, 128, 5, 6, 20, 1),
+                     (6, 32, 16, 16, 16, 0), (2, 64, 9, 13, 17, 0), (1, 16, 4, 4, 5, 1), (11, 32, 6, 11, 64, 1),
+                     (130, 64, 7, 7, 8, 1)]
+
+
+@pytest.mark.parametrize("cfg", SMALL_IMAGE_CASES)
+def test_conv_small_images(ctx, cfg):
+    """The small-image convolution kernel against the oracle (<= 1e-5, exact on integers), and every
+    epilogue it can carry against the separate commands bit for bit."""
+    B, C, H, W, F, pad = cfg
+    x = synth.uniform(31, (B, C, H, W), -1, 1)
+    w = synth.he_normal(32, (F, C, 3, 3))
+    plain = gpu_conv(ctx, x, w, (pad, pad), (1, 1), (1, 1))
+    ref = O.conv2d_direct_f64(x, w, (pad, pad), (1, 1), (1, 1))
+    err = rel_frobenius(plain, ref)
+    assert err <= TOL, f"small conv {cfg}: rel frobenius {err:.3e}"
+    rng = np.random.default_rng(9)
+    xi = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+    wi = rng.integers(-3, 4, (F, C, 3, 3)).astype(np.float32)
+    assert_bits_equal(gpu_conv(ctx, xi, wi, (pad, pad), (1, 1), (1, 1)), O.conv2d(xi, wi, (pad, pad), (1, 1), (1, 1)),
+                      f"integer small conv {cfg}")
+    mean, var = synth.normal(33, (F,), 0.0, 0.1), synth.uniform(34, (F,), 0.5, 1.5)
+    gamma, beta = synth.uniform(35, (F,), 0.5, 1.5), synth.normal(36, (F,), 0.0, 0.1)
+    bn = O.bn_infer(plain, mean, var, 1e-5, gamma, beta)
+    leaky = O.leaky_relu(bn, 0.1).reshape(bn.shape)
+    assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, gamma, beta), act="leaky", alpha=0.1), leaky,
+                      f"small conv+bn+leaky {cfg}")
+    cmd = D.cmd_conv2d(1, 1, 1, B, C, H, W, F, 3, 3, (pad, pad))
+    if plain.shape[2] >= 2 and plain.shape[3] >= 2:
+        assert ctx.lib.gh_conv2d_can_pool(cmd) == 1
+        relu = O.relu(plain).reshape(plain.shape)
+        assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), act="relu", pool2=True),
+                          O.maxpool2d(relu, (2, 2), (0, 0), (2, 2)), f"small conv+relu+pool {cfg}")
+        assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, gamma, beta), act="leaky", alpha=0.1,
+                                        pool2=True),
+                          O.maxpool2d(leaky, (2, 2), (0, 0), (2, 2)), f"small conv+bn+leaky+pool {cfg}")
+
+
 def test_conv_random_geometry_sweep(ctx):
     """Seeded sweep over 3x3 and other geometries (all three convolution kernels, ragged sizes,
     batch boundaries inside blocks): the plain convolution against the oracle, and wherever the
