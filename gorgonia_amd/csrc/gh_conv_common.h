@@ -37,6 +37,27 @@ __device__ __forceinline__ float tail_apply(const ConvTail& t, int f, float v) {
   return act_apply(v, t.act, t.alpha);
 }
 
+// The same arithmetic with the per-filter BatchNorm constants taken from a table a
+// workgroup fills once (conv_tail_table): a and b are rounded exactly as above, so the
+// stored bits are those of tail_apply.  tab = [4][n]: a, b, gamma, beta.
+__device__ __forceinline__ void conv_tail_table(const ConvTail& t, float* tab, int n, int i, int f) {
+  if (!t.mean) return;
+  const float a = 1.0f / sqrtf(t.var[f] + t.eps);
+  tab[i] = a;
+  tab[n + i] = -t.mean[f] * a;
+  if (t.gamma) tab[2 * n + i] = t.gamma[f];
+  if (t.beta) tab[3 * n + i] = t.beta[f];
+}
+__device__ __forceinline__ float tail_apply_table(const ConvTail& t, const float* tab, int n, int i, float v) {
+  if (t.mean) {
+    v = v * tab[i];
+    v = v + tab[n + i];
+    if (t.gamma) v = tab[2 * n + i] * v;
+    if (t.beta) v = v + tab[3 * n + i];
+  }
+  return act_apply(v, t.act, t.alpha);
+}
+
 inline ConvTail conv_tail(const gh_cmd& c) {
   ConvTail t{};
   if (c.flags & GH_FLAG_CONV_BN) {

@@ -73,6 +73,10 @@ int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c);
 int gh_try_launch_conv_small(gh_ctx* ctx, const gh_cmd& c);
 bool gh_conv_small_takes(const gh_cmd& c);
 bool gh_conv_small_can_pool(const gh_cmd& c);
+// 3x3 convolution over patches with K split across wavefronts (k_conv_patch.hip), same conventions
+int gh_try_launch_conv_patch(gh_ctx* ctx, const gh_cmd& c);
+bool gh_conv_patch_takes(const gh_cmd& c);
+bool gh_conv_patch_can_pool(const gh_cmd& c);
 int gh_launch_maxpool2d(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_bn_infer(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_softmax(gh_ctx* ctx, const gh_cmd& c);

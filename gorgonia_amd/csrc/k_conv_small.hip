@@ -59,6 +59,7 @@ struct SmallGeom {
   int IPP;           // load items per plane: H * CH (<= 64)
   int lpg_shift;     // lanes per plane group = 1 << lpg_shift >= IPP
   int nout;          // result columns per workgroup: pool ? IPB * ph * pw : IPB * oh * ow
+  int epi_off;       // float offset in LDS of the per-filter epilogue table (past every other use)
   unsigned mPPI, mOW, mPW, mPQ, mNOUT, mCH;   // magics: ppi, ow, pw, ph*pw, nout, CH
 };
 
@@ -87,6 +88,8 @@ __global__ __launch_bounds__(WV * 64) void k_conv3x3_small(const float* __restri
   const int m0 = blockIdx.y * BM, b0 = blockIdx.x * g.IPB;
   const int nimg = min(g.IPB, g.B - b0);
   const int c0 = wave * g.CW;            // this wavefront's first channel
+  float* const ftab = lds + g.epi_off;   // [4][BM] BatchNorm constants of this workgroup's filters
+  if (tid < BM) conv_tail_table(tail, ftab, BM, tid, min(m0 + tid, g.F - 1));
 
   // ---- all global loads of this wavefront, quad by quad; slots past the end repeat the last one
   f32x4 wv[NQ][NWQ], xv[NQ][kSlotsX];
@@ -264,7 +267,7 @@ __global__ __launch_bounds__(WV * 64) void k_conv3x3_small(const float* __restri
 #pragma unroll
         for (int j = 0; j < 4; j++) {
           if (mf + j < g.F) {
-            const float v = tail_apply(tail, mf + j, s[j]);
+            const float v = tail_apply_table(tail, ftab, BM, 4 * mg + j, s[j]);
             if (v > best[j]) best[j] = v;
           }
         }
@@ -286,7 +289,7 @@ __global__ __launch_bounds__(WV * 64) void k_conv3x3_small(const float* __restri
       float* yp = y + ((int64_t)(b0 + img) * g.F + mf) * plane + r;
 #pragma unroll
       for (int j = 0; j < 4; j++)
-        if (mf + j < g.F) yp[j * plane] = tail_apply(tail, mf + j, s[j]);
+        if (mf + j < g.F) yp[j * plane] = tail_apply_table(tail, ftab, BM, 4 * mg + j, s[j]);
     }
   }
 }
@@ -349,7 +352,7 @@ bool small_plan(const gh_cmd& c, bool pool, SmallPlan* out) {
       if (!TN) continue;
       const size_t stage = ((size_t)g.K * 16 * TM + (size_t)IPB * g.C * g.PL + 8 + 16 * TN) * 4;
       const size_t red = (size_t)4 * 16 * TN * (16 * TM + 4) * 4;
-      const size_t lds = stage > red ? stage : red;
+      const size_t lds = (stage > red ? stage : red) + (size_t)4 * 16 * TM * 4;   // + the epilogue table
       if (lds > kLdsBudget) continue;
       const int64_t blocks = ((F + 16 * TM - 1) / (16 * TM)) * ((B + IPB - 1) / IPB);
       const int coresident = lds <= 75 * 1024 ? 2 : 1;
@@ -361,6 +364,7 @@ bool small_plan(const gh_cmd& c, bool pool, SmallPlan* out) {
   }
   if (!bestTM) return false;
   g.IPB = bestIPB;
+  g.epi_off = (int)(best_lds / 4) - 4 * 16 * bestTM;
   g.nout = pool ? g.IPB * g.ph * g.pw : g.IPB * g.oh * g.ow;
   g.mPPI = magic_of(g.ppi); g.mOW = magic_of(g.ow); g.mPW = magic_of(g.pw); g.mPQ = magic_of(g.ph * g.pw);
   g.mNOUT = magic_of(g.nout); g.mCH = magic_of(g.CH);

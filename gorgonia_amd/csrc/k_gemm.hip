@@ -2785,6 +2785,8 @@ int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
   if (conv_direct_shape(c) && !getenv("GORGONIA_HIP_CONV_NO_DIRECT")) return launch_conv_direct(ctx, c);
   const int rcs = gh_try_launch_conv_small(ctx, c);
   if (rcs >= 0) return rcs;
+  const int rcp = gh_try_launch_conv_patch(ctx, c);
+  if (rcp >= 0) return rcp;
   const int rc3 = try_launch_conv3(ctx, c);
   if (rc3 >= 0) return rc3;
   if (c.flags & GH_FLAG_CONV_POOL2)
@@ -2983,9 +2985,10 @@ extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {
     return oh >= 2 && ow >= 2;
   }
   if (getenv("GORGONIA_HIP_CONV_NO_POOL")) return 0;  // tuning switch: keep MaxPool2D a kernel of its own
-  // a shape the small-image kernel takes is pooled there or not at all (the plain and the
+  // a shape the small-image or the patch kernel takes is pooled there or not at all (the plain and the
   // pooled command must sum in the same order)
   if (gh_conv_small_takes(*c)) return gh_conv_small_can_pool(*c) ? 1 : 0;
+  if (gh_conv_patch_takes(*c)) return gh_conv_patch_can_pool(*c) ? 1 : 0;
   Conv3Geom g;
   int BM, BN, per_thread;
   size_t lds;

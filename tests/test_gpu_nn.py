@@ -231,6 +231,40 @@ def test_conv_small_images(ctx, cfg):
                           O.maxpool2d(leaky, (2, 2), (0, 0), (2, 2)), f"small conv+bn+leaky+pool {cfg}")
 
 
+# shapes the patch kernel takes (3x3, 64 channels or more, K split over eight wavefronts): partial
+# patches on both axes, ragged filter tiles, no padding, pooled extents odd and even
+PATCH_CASES = [(2, 64, 20, 17, 40, 1), (2, 64, 28, 28, 32, 1), (1, 64, 24, 14, 20, 0), (1, 96, 26, 26, 48, 1), (3, 128, 13, 13, 70, 1), (1, 64, 31, 18, 16, 0),
+               (2, 256, 13, 13, 33, 1), (1, 64, 52, 52, 32, 1), (2, 64, 9, 40, 24, 1)]
+
+
+@pytest.mark.parametrize("cfg", PATCH_CASES)
+def test_conv_patch_kernel(ctx, cfg):
+    """The patch convolution kernel against the oracle (<= 1e-5, exact on integers), and every epilogue
+    it can carry against the oracle's operators applied to its own plain result, bit for bit."""
+    B, C, H, W, F, pad = cfg
+    x = synth.uniform(41, (B, C, H, W), -1, 1)
+    w = synth.he_normal(42, (F, C, 3, 3))
+    plain = gpu_conv(ctx, x, w, (pad, pad), (1, 1), (1, 1))
+    ref = O.conv2d_direct_f64(x, w, (pad, pad), (1, 1), (1, 1))
+    err = rel_frobenius(plain, ref)
+    assert err <= TOL, f"patch conv {cfg}: rel frobenius {err:.3e}"
+    rng = np.random.default_rng(10)
+    xi = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+    wi = rng.integers(-3, 4, (F, C, 3, 3)).astype(np.float32)
+    assert_bits_equal(gpu_conv(ctx, xi, wi, (pad, pad), (1, 1), (1, 1)), O.conv2d(xi, wi, (pad, pad), (1, 1), (1, 1)),
+                      f"integer patch conv {cfg}")
+    mean, var = synth.normal(43, (F,), 0.0, 0.1), synth.uniform(44, (F,), 0.5, 1.5)
+    gamma, beta = synth.uniform(45, (F,), 0.5, 1.5), synth.normal(46, (F,), 0.0, 0.1)
+    leaky = O.leaky_relu(O.bn_infer(plain, mean, var, 1e-5, gamma, beta), 0.1).reshape(plain.shape)
+    assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, gamma, beta), act="leaky", alpha=0.1), leaky,
+                      f"patch conv+bn+leaky {cfg}")
+    cmd = D.cmd_conv2d(1, 1, 1, B, C, H, W, F, 3, 3, (pad, pad))
+    if ctx.lib.gh_conv2d_can_pool(cmd) == 1:
+        assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, gamma, beta), act="leaky", alpha=0.1,
+                                        pool2=True),
+                          O.maxpool2d(leaky, (2, 2), (0, 0), (2, 2)), f"patch conv+bn+leaky+pool {cfg}")
+
+
 def test_conv_random_geometry_sweep(ctx):
     """Seeded sweep over 3x3 and other geometries (all three convolution kernels, ragged sizes,
     batch boundaries inside blocks): the plain convolution against the oracle, and wherever the
