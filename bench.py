@@ -59,38 +59,87 @@ def time_cmds(ctx, cmds, iters, warm=3):
     return ms
 
 
+ELEMENTWISE_SETS = 8   # operand sets a timed kernel rotates over: 8 x (2..3) x 64 MiB >= 1 GiB, four times the last-level cache
+
+
 def bench_elementwise(ctx, iters):
-    """Config 2: z = Sigmoid(x*y + b); Tanh(z); Pow(z, 2) on 4096x4096 float32."""
+    """Config 2: z = Sigmoid(x*y + b); Tanh(z); Pow(z, 2) on 4096x4096 float32.
+
+    Every kernel is timed twice.  `cold`: consecutive launches walk over ELEMENTWISE_SETS
+    distinct operand sets (1-1.5 GiB in all), so no launch finds its operands in the 256 MB
+    last-level cache and the bytes really cross the HBM interface - that is the figure
+    reported as frac_hbm.  `warm`: the same launch on one operand set over and over (128-192
+    MiB, cache-assisted), kept next to it as frac_llc_assisted."""
     from gorgonia_amd import configs, device as D
     inp = configs.elementwise_inputs(4096)
     N = 4096 * 4096
-    x, y, b = ctx.upload(inp["x"]), ctx.upload(inp["y"]), ctx.upload(inp["b"])
-    z, t, p = ctx.malloc(4 * N), ctx.malloc(4 * N), ctx.malloc(4 * N)
+    S = ELEMENTWISE_SETS
+    x0, y0, b = ctx.upload(inp["x"]), ctx.upload(inp["y"]), ctx.upload(inp["b"])
     two = ctx.upload(np.array([2.0], np.float32))
-    ctx.run([D.cmd_bin("mul", "vv", x, y, N, dst=z), D.cmd_bcast("add", z, z, b, 4096, 4096, 1),
-             D.cmd_unary("sigmoid", z, N)])
-    kernels = [
-        ("HadamardProd", D.cmd_bin("mul", "vv", x, y, N, dst=p), 3 * 4 * N),
-        ("BroadcastAdd", D.cmd_bcast("add", p, p, b, 4096, 4096, 1), 2 * 4 * N + 4 * 4096),
-        ("Sigmoid", D.cmd_unary("sigmoid", p, N, dst=t), 2 * 4 * N),
-        ("Tanh", D.cmd_unary("tanh", z, N, dst=t), 2 * 4 * N),
-        ("Pow2", D.cmd_bin("pow", "vs", z, two, N, dst=p), 2 * 4 * N),
-    ]
-    out, total_ms, total_bytes = {}, 0.0, 0
-    for name, cmd, nbytes in kernels:
-        ms = time_cmds(ctx, [cmd], iters)
-        out[name] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1),
-                     "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "bytes": nbytes}
-        total_ms += ms
+    xs, ys, ps = [x0], [y0], [ctx.malloc(4 * N)]
+    for _ in range(S - 1):   # the other sets are device-side copies of the first
+        xs.append(ctx.malloc(4 * N)); ys.append(ctx.malloc(4 * N)); ps.append(ctx.malloc(4 * N))
+        ctx.run([D.cmd_copy(xs[-1], x0, 4 * N), D.cmd_copy(ys[-1], y0, 4 * N)])
+    # z = Sigmoid(x*y + b) per set, written into ys (the chain's intermediate value)
+    zs = ys
+
+    def build(name, i):
+        x, p, z = xs[i], ps[i], zs[i]
+        if name == "HadamardProd":
+            return D.cmd_bin("mul", "vv", x, zs[i], N, dst=p)
+        if name == "BroadcastAdd":
+            return D.cmd_bcast("add", p, x, b, 4096, 4096, 1)
+        if name == "Sigmoid":
+            return D.cmd_unary("sigmoid", x, N, dst=p)
+        if name == "Tanh":
+            return D.cmd_unary("tanh", z, N, dst=p)
+        return D.cmd_bin("pow", "vs", z, two, N, dst=p)
+
+    sizes = {"HadamardProd": 3 * 4 * N, "BroadcastAdd": 2 * 4 * N + 4 * 4096, "Sigmoid": 2 * 4 * N,
+             "Tanh": 2 * 4 * N, "Pow2": 2 * 4 * N}
+    out, total_ms, total_ms_warm, total_bytes = {}, 0.0, 0.0, 0
+    passes = max(2, iters // S)
+    for name, nbytes in sizes.items():
+        ms_cold = time_cmds(ctx, [build(name, i) for i in range(S)], passes) / S
+        ms_warm = time_cmds(ctx, [build(name, 0)], iters)
+        out[name] = {"us": round(ms_cold * 1e3, 2), "GBps": round(nbytes / ms_cold / 1e6, 1),
+                     "frac_hbm": round(nbytes / ms_cold / 1e6 / HBM_PEAK_GBPS, 4), "bytes": nbytes,
+                     "us_llc_assisted": round(ms_warm * 1e3, 2),
+                     "frac_llc_assisted": round(nbytes / ms_warm / 1e6 / HBM_PEAK_GBPS, 4)}
+        total_ms += ms_cold
+        total_ms_warm += ms_warm
         total_bytes += nbytes
-    # device copy of the same size as a measured ceiling next to the nominal one
-    ms = time_cmds(ctx, [D.cmd_copy(t, x, 4 * N)], iters)
+    # the chain as configuration 2 issues it - five launches in order on one set of tensors
+    # (x, y, z, t, p: 320 MiB, intermediates re-read straight after they were written)
+    z, t, p = ys[1], ps[0], ps[1]
+    seq = [D.cmd_bin("mul", "vv", xs[0], ys[0], N, dst=z), D.cmd_bcast("add", z, z, b, 4096, 4096, 1),
+           D.cmd_unary("sigmoid", z, N), D.cmd_unary("tanh", z, N, dst=t), D.cmd_bin("pow", "vs", z, two, N, dst=p)]
+    ms_seq = time_cmds(ctx, seq, max(4, iters // 3))
+    # tensors no cache can hold (8192 x 8192, 256 MiB each): the kernels' streaming form
+    big = [ctx.malloc(16 * N) for _ in range(3)]
+    ctx.run([D.cmd_fill(q, 4 * N, 1.5) for q in big[:2]])
+    streaming = {}
+    for name, cmd, nbytes in (("Neg_8192", D.cmd_unary("neg", big[0], 4 * N, dst=big[2]), 2 * 16 * N),
+                              ("HadamardProd_8192", D.cmd_bin("mul", "vv", big[0], big[1], 4 * N, dst=big[2]), 3 * 16 * N)):
+        ms = time_cmds(ctx, [cmd], max(4, iters // 4))
+        streaming[name] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1),
+                           "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "bytes": nbytes}
+    for q in big:
+        ctx.free(q)
+    # device copy of the same size as a measured ceiling next to the nominal one, cold and warm
+    ms = time_cmds(ctx, [D.cmd_copy(ps[i], xs[i], 4 * N) for i in range(S)], passes) / S
     copy_gbps = 2 * 4 * N / ms / 1e6
-    for q in (x, y, b, z, t, p, two):
+    ms = time_cmds(ctx, [D.cmd_copy(ps[0], xs[0], 4 * N)], iters)
+    copy_gbps_warm = 2 * 4 * N / ms / 1e6
+    for q in xs + ys + ps + [b, two]:
         ctx.free(q)
     return {"chain_GBps": round(total_bytes / total_ms / 1e6, 1), "chain_bytes": total_bytes,
             "chain_us": round(total_ms * 1e3, 1), "frac_hbm": round(total_bytes / total_ms / 1e6 / HBM_PEAK_GBPS, 4),
-            "device_copy_GBps": round(copy_gbps, 1), "kernels": out}
+            "frac_llc_assisted": round(total_bytes / total_ms_warm / 1e6 / HBM_PEAK_GBPS, 4),
+            "chain_in_sequence_us": round(ms_seq * 1e3, 1), "chain_in_sequence_GBps": round(total_bytes / ms_seq / 1e6, 1),
+            "streaming_8192": streaming, "operand_sets": S, "footprint_bytes": 3 * S * 4 * N,
+            "device_copy_GBps": round(copy_gbps, 1), "device_copy_GBps_llc_assisted": round(copy_gbps_warm, 1),
+            "kernels": out}
 
 
 def bench_linalg(ctx, iters):
