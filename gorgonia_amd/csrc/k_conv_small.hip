@@ -358,7 +358,8 @@ bool small_plan(const gh_cmd& c, bool pool, SmallPlan* out) {
       const int coresident = lds <= 75 * 1024 ? 2 : 1;
       const int64_t rounds = (blocks + 256 * coresident - 1) / (256 * coresident);
       const double mfma_us = (WV / 4) * (double)(NQ * 9 * TM * TN) * 32.0 / 2100.0;
-      const double est = rounds * (4.5 + coresident * mfma_us);
+      // (two workgroups sharing a compute unit overlap each other's fixed cost only in part)
+      const double est = rounds * (4.5 + coresident * mfma_us * 1.1);
       if (!bestTM || est < best) { best = est; bestTM = TM; bestIPB = IPB; bestTN = TN; best_lds = lds; }
     }
   }
