@@ -33,6 +33,14 @@ def log(*a):
 
 
 EAGER_TIMING = False  # --eager-timing: no hipGraph anywhere (for hardware-counter runs)
+# A tape machine in "measured" mode runs a segment plainly three times, captures it, replays it twice
+# and then keeps the quicker way: the timed loops start after that.
+WARM_RUNS = 8
+VERDICTS = {}  # workload -> how its segment ended up being run ("plain" / "replay")
+
+
+def replay_mode():
+    return False if EAGER_TIMING else "measured"
 
 
 def time_cmds(ctx, cmds, iters, warm=3):
@@ -217,7 +225,8 @@ def bench_convnet_kernels(ctx, batch, iters):
     return out
 
 
-def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=True, dtype=np.float32):
+def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=True, dtype=np.float32,
+                  reupload_all=False):
     from gorgonia_amd import configs, graph as G
     inp = {k: v.astype(dtype) for k, v in configs.convnet_inputs(batch).items()}
     g = G.NewGraph()
@@ -229,8 +238,10 @@ def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=Tr
     h = G.Reshape(h, (batch, 128 * 3 * 3))
     h = G.Rectify(G.Mul(h, G.NewTensor(g, inp["w3"], True)))
     out = G.Read(G.SoftMax(G.Mul(h, G.NewTensor(g, inp["w4"], True))))
-    m = G.NewTapeMachine(g, graph_replay=graph_replay, fuse_activations=True)
-    for _ in range(max(warmup, 3)):  # first run eager, second captures, third replays
+    # reupload_all: every input, weights too, crosses the bus on every run as the
+    # reference's tape machine does it (vm_tape_cuda.go:220-243)
+    m = G.NewTapeMachine(g, graph_replay=graph_replay, fuse_activations=True, reupload_resident=reupload_all)
+    for _ in range(max(warmup, WARM_RUNS)):
         m.RunAll()
     eng = m.engine()
     eng.DoWork()
@@ -241,6 +252,8 @@ def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=Tr
     dt = time.perf_counter() - t0
     result = out.copy()
     launches = m.graph_launches()
+    VERDICTS[f"convnet{'_f64' if dtype == np.float64 else ''}{'' if resident_input else '_input_h2d'}"
+             f"{'_all_h2d' if reupload_all else ''}{'' if graph_replay == 'measured' else '_' + str(graph_replay)}"] = m.segment_verdict()
     m.Close()
     return dt / steps * 1e3, result, inp, launches
 
@@ -256,8 +269,8 @@ def bench_convnet_machines(steps, warmup, count=2, batch=128):
     machines = []
     for _ in range(count):
         g, outs = configs.build_convnet(inp, resident_input=True)
-        m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING, fuse_activations=True)
-        for _ in range(max(warmup, 3)):
+        m = G.NewTapeMachine(g, graph_replay=replay_mode(), fuse_activations=True)
+        for _ in range(max(warmup, WARM_RUNS)):
             m.RunAll()
         machines.append((g, m, outs))
     gate = threading.Barrier(count + 1)
@@ -290,8 +303,8 @@ def bench_yolo(steps, warmup, resident_input=True):
     from gorgonia_amd import configs, graph as G
     inp = configs.yolo_inputs(8, 416)
     g, outs = configs.build_yolo(inp, resident_input=resident_input)
-    m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING, fuse_activations=True)
-    for _ in range(max(warmup, 3)):
+    m = G.NewTapeMachine(g, graph_replay=replay_mode(), fuse_activations=True)
+    for _ in range(max(warmup, WARM_RUNS)):
         m.RunAll()
     eng = m.engine()
     eng.DoWork()
@@ -301,6 +314,7 @@ def bench_yolo(steps, warmup, resident_input=True):
     eng.DoWork()
     dt = time.perf_counter() - t0
     result = outs["out"].copy()
+    VERDICTS["yolo" if resident_input else "yolo_input_h2d"] = m.segment_verdict()
     m.Close()
     return dt / steps * 1e3, result, inp
 
@@ -312,8 +326,8 @@ def bench_mlp(steps, warmup, resident_input=True):
     from gorgonia_amd import configs, graph as G
     inp = configs.mlp_inputs(256)
     g, outs = configs.build_mlp(inp, resident_input=resident_input)
-    m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING, fuse_activations=True)
-    for _ in range(max(warmup, 3)):
+    m = G.NewTapeMachine(g, graph_replay=replay_mode(), fuse_activations=True)
+    for _ in range(max(warmup, WARM_RUNS)):
         m.RunAll()
     eng = m.engine()
     eng.DoWork()
@@ -323,6 +337,7 @@ def bench_mlp(steps, warmup, resident_input=True):
     eng.DoWork()
     dt = time.perf_counter() - t0
     result = outs["out"].copy()
+    VERDICTS["mlp" if resident_input else "mlp_input_h2d"] = m.segment_verdict()
     m.Close()
     return dt / steps * 1e3, result, inp
 
@@ -336,8 +351,8 @@ def bench_convnet_train(steps, warmup, batch=128, dtype=np.float32):
     onehot = np.zeros((batch, 10), dtype)
     onehot[np.arange(batch), np.arange(batch) % 10] = 1.0
     g, outs = configs.build_convnet_train(inp, onehot, 0.01, read_grads=False, solver="rmsprop")
-    m = G.NewTapeMachine(g, graph_replay=not EAGER_TIMING)
-    for _ in range(max(warmup, 3)):
+    m = G.NewTapeMachine(g, graph_replay=replay_mode())
+    for _ in range(max(warmup, WARM_RUNS)):
         m.RunAll()
     eng = m.engine()
     eng.DoWork()
@@ -346,6 +361,7 @@ def bench_convnet_train(steps, warmup, batch=128, dtype=np.float32):
         m.RunAll()
     eng.DoWork()
     dt = time.perf_counter() - t0
+    VERDICTS["convnet_train" + ("_f64" if dtype == np.float64 else "")] = m.segment_verdict()
     m.Close()
     return dt / steps * 1e3, inp, onehot
 
@@ -456,7 +472,7 @@ def main():
     info = ctx.info()
     log(f"device {info.arch.decode()} CUs={info.compute_units}")
 
-    ms_step, gpu_out, inp, launches = bench_convnet(a.steps, a.warmup, graph_replay=not a.eager_timing)
+    ms_step, gpu_out, inp, launches = bench_convnet(a.steps, a.warmup, graph_replay=replay_mode())
     images_s = 128 / ms_step * 1e3
     log(f"convnet: {ms_step:.4f} ms/step  {images_s:.0f} images/s  (graph launches {launches})")
     two_images_s = four_images_s = None
@@ -466,7 +482,10 @@ def main():
         four_images_s, four_out = bench_convnet_machines(a.steps, a.warmup, 4)
         log(f"convnet, machines in parallel host threads: two {two_images_s:.0f}, four {four_images_s:.0f} images/s")
     ms_h2d, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False)
+    ms_h2d_all, out_h2d_all, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False,
+                                                  reupload_all=True)
     ms_eager, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, graph_replay=False)
+    ms_replay, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, graph_replay=not EAGER_TIMING)
 
     yolo = None
     if not only or "yolo" in only:
@@ -496,7 +515,7 @@ def main():
     f64 = None
     if not only or "float64" in only:
         n64 = max(20, a.steps // 4)
-        ms64, out64, inp64, _ = bench_convnet(n64, a.warmup, graph_replay=not a.eager_timing, dtype=np.float64)
+        ms64, out64, inp64, _ = bench_convnet(n64, a.warmup, graph_replay=replay_mode(), dtype=np.float64)
         ms64t, _, _ = bench_convnet_train(n64, a.warmup, dtype=np.float64)
         f64 = {"forward_ms_per_step": round(ms64, 4), "forward_images_s": round(128 / ms64 * 1e3, 1),
                "training_ms_per_step": round(ms64t, 4), "training_images_s": round(128 / ms64t * 1e3, 1)}
@@ -590,7 +609,8 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "convnet forward, float32 NCHW batch 128x1x28x28 (config 4): "
                                "3x[Conv2d 3x3 pad1 + ReLU + MaxPool 2x2] -> Dense 625 ReLU -> Dense 10 SoftMax; "
-                               "tape machine, one segment, hipGraph replay, weights and input resident",
+                               "tape machine, one segment, run the quicker of plain submits and hipGraph replay "
+                               "(timed by the machine on its first runs), weights and input resident",
                    "batch": 128, "flop_per_step": 2_093_410_816},
         "roofline": roofline,
         "cpu_baseline": cpu,
@@ -600,7 +620,13 @@ def main():
             "sgemm_frac_mfma": lin.get("sgemm_4096", {}).get("frac_mfma"),
             "convnet_ms_per_step_with_input_h2d": round(ms_h2d, 5),
             "convnet_images_s_with_input_h2d": round(128 / ms_h2d * 1e3, 1),
+            "convnet_ms_per_step_all_inputs_reuploaded": round(ms_h2d_all, 5),
+            "convnet_images_s_all_inputs_reuploaded": round(128 / ms_h2d_all * 1e3, 1),
+            "convnet_all_inputs_reuploaded_bytes_per_step": int(sum(v.nbytes for v in inp.values())),
+            "convnet_reuploaded_output_equals_resident": bool(np.array_equal(out_h2d_all, gpu_out)),
             "convnet_ms_per_step_eager_no_graph": round(ms_eager, 5),
+            "convnet_ms_per_step_graph_replay_always": round(ms_replay, 5),
+            "segment_run_as": dict(VERDICTS),
             "convnet_images_s_two_machines_two_host_threads": two_images_s and round(two_images_s, 1),
             "convnet_images_s_four_machines_four_host_threads": four_images_s and round(four_images_s, 1),
             "convnet_parallel_machines_outputs_equal_single": (bool(all(np.array_equal(o, gpu_out) for o in two_out + four_out))

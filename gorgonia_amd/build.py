@@ -109,8 +109,27 @@ def build_host(force=False):
     return out
 
 
+C_CONSUMER_DIR = os.path.join(ROOT, "tests", "c_consumer")
+# The device header is meant for C callers (cgo compiles it as C): the consumer
+# is built as strict C99 so anything that is not C in the header stops the build.
+C_CONSUMER_FLAGS = ["-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-O1", "-I", INCLUDE]
+
+
+def build_c_consumer(force=False):
+    """The plain-C program of tests/c_consumer: links the device library only."""
+    src = os.path.join(C_CONSUMER_DIR, "consumer.c")
+    if not os.path.exists(src):
+        return None
+    out = os.path.join(C_CONSUMER_DIR, "consumer.bin")
+    if force or _newer([src] + _headers(INCLUDE), out):
+        cc = shutil.which("gcc") or "gcc"
+        _run([cc] + C_CONSUMER_FLAGS + [src, "-o", out, "-L", LIBDIR, "-lgorgonia_hip",
+                                        "-Wl,-rpath,$ORIGIN/../../gorgonia_amd/lib"])
+    return out
+
+
 def build_all(force=False):
-    return [p for p in (build_device(force), build_host(force)) if p]
+    return [p for p in (build_device(force), build_host(force), build_c_consumer(force)) if p]
 
 
 def main():

@@ -81,6 +81,7 @@ int gh_init(int device, int64_t arena_bytes, gh_ctx** out) {
   }
   hipDeviceProp_t prop;
   if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->cu_count = prop.multiProcessorCount;
+  if (const char* sm = getenv("GORGONIA_HIP_SYNC")) ctx->sync_spin = strcmp(sm, "spin") == 0;
   if (arena_bytes > 0) {
     size_t free_b = 0, total_b = 0;
     hipMemGetInfo(&free_b, &total_b);
@@ -210,24 +211,49 @@ int gh_memcpy_d2h(gh_ctx* ctx, void* dst, gh_devptr src, int64_t bytes) {
                       "hipMemcpyAsync(D2H)");
 }
 
-// Word copy for small transfers: a kernel node costs less inside a captured
-// graph than a copy-engine node, and it can write pinned host memory too.
+// Copies done by a kernel: a kernel node costs less inside a captured graph than
+// a copy-engine node, and either side may be pinned host memory (results staged
+// out to the host, inputs staged in from it over PCIe).
 __global__ __launch_bounds__(256) void k_copy_words(uint32_t* __restrict__ dst,
                                                     const uint32_t* __restrict__ src, int64_t n) {
   const int64_t stride = (int64_t)gridDim.x * 256;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) dst[i] = src[i];
 }
+// 16 bytes per lane, two in flight; the tail (< 16 bytes, a multiple of 4) goes word by word.
+__global__ __launch_bounds__(256) void k_copy_vec(uint4* __restrict__ dst, const uint4* __restrict__ src,
+                                                  int64_t n16, int64_t tail_words) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + stride < n16; i += 2 * stride) {
+    const uint4 a = src[i], b = src[i + stride];
+    dst[i] = a;
+    dst[i + stride] = b;
+  }
+  if (i < n16) dst[i] = src[i];
+  if (blockIdx.x == 0 && (int64_t)threadIdx.x < tail_words)
+    ((uint32_t*)(dst + n16))[threadIdx.x] = ((const uint32_t*)(src + n16))[threadIdx.x];
+}
+
+static constexpr int64_t kKernelCopyLimit = 16 << 20;
 
 int gh_memcpy_d2d(gh_ctx* ctx, gh_devptr dst, gh_devptr src, int64_t bytes) {
   if (!ctx || bytes < 0 || (bytes > 0 && (!dst || !src))) return GH_EINVAL;
   if (ctx->err) return ctx->err;
   if (bytes == 0) return GH_OK;
-  if (bytes <= (1 << 20) && ((dst | src | (uint64_t)bytes) & 3) == 0) {
-    const int64_t n = bytes / 4;
-    int64_t blocks = (n + 255) / 256;
-    if (blocks > 256) blocks = 256;
-    hipLaunchKernelGGL(k_copy_words, dim3((int)blocks), dim3(256), 0, ctx->stream,
-                       (uint32_t*)(uintptr_t)dst, (const uint32_t*)(uintptr_t)src, n);
+  if (bytes <= kKernelCopyLimit && ((dst | src | (uint64_t)bytes) & 3) == 0) {
+    if (((dst | src) & 15) == 0 && bytes >= 4096) {
+      const int64_t n16 = bytes / 16;
+      int64_t blocks = (n16 + 511) / 512;
+      if (blocks > 1024) blocks = 1024;
+      hipLaunchKernelGGL(k_copy_vec, dim3((int)blocks), dim3(256), 0, ctx->stream, (uint4*)(uintptr_t)dst,
+                         (const uint4*)(uintptr_t)src, n16, (bytes % 16) / 4);
+    } else {
+      const int64_t n = bytes / 4;
+      int64_t blocks = (n + 255) / 256;
+      if (blocks > 1024) blocks = 1024;
+      hipLaunchKernelGGL(k_copy_words, dim3((int)blocks), dim3(256), 0, ctx->stream,
+                         (uint32_t*)(uintptr_t)dst, (const uint32_t*)(uintptr_t)src, n);
+    }
     return gh_check_hip(ctx, hipGetLastError(), "copy launch");
   }
   return gh_check_hip(ctx,
@@ -337,7 +363,14 @@ int gh_submit_noalloc(gh_ctx* ctx, const gh_cmd* cmds, int n) {
 int gh_sync(gh_ctx* ctx) {
   if (!ctx) return GH_EINVAL;
   if (ctx->capturing) return gh_fail(ctx, GH_ESTATE, "gh_sync during graph capture");
-  hipError_t e = hipStreamSynchronize(ctx->stream);
+  hipError_t e;
+  if (ctx->sync_spin) {
+    // poll the stream from this thread instead of blocking in the runtime's wait
+    while ((e = hipStreamQuery(ctx->stream)) == hipErrorNotReady) {
+    }
+  } else {
+    e = hipStreamSynchronize(ctx->stream);
+  }
   if (e != hipSuccess) gh_check_hip(ctx, e, "hipStreamSynchronize");
   return ctx->err;
 }

@@ -30,6 +30,7 @@ struct gh_ctx {
   // set while gh_submit_noalloc runs: the scratch is the library's fixed array and a
   // plan may not shrink to fit it (results must not depend on the scratch size)
   bool ws_strict = false;
+  bool sync_spin = false;  // gh_sync polls the stream instead of blocking in the runtime
 };
 
 // A launcher calls this where `need` bytes of scratch do not fit the workspace,

@@ -85,6 +85,7 @@ HOST_SYMBOLS = {
     "ghh_graph_node_dtype": (C.c_int, [_P, C.c_int]),
     "ghh_graph_fuse_activations": (C.c_int, [_P]),
     "ghh_tape_new": (_P, [_P, C.c_int, C.c_int]),
+    "ghh_tape_new_with_engine": (_P, [_P, _P, C.c_int, C.c_int]),
     "ghh_tape_destroy": (None, [_P]),
     "ghh_tape_last_error": (C.c_char_p, [_P]),
     "ghh_tape_init": (C.c_int, [_P, C.c_int]),
@@ -99,6 +100,8 @@ HOST_SYMBOLS = {
     "ghh_tape_register_address": (C.c_uint64, [_P, C.c_int]),
     "ghh_tape_program_string": (C.c_int, [_P, C.c_char_p, C.c_int]),
     "ghh_tape_engine": (_P, [_P]),
+    "ghh_tape_segment_verdict": (C.c_int, [_P, C.c_int]),
+    "ghh_tape_phase_ns": (None, [_P, C.POINTER(C.c_int64)]),
 }
 
 _hlib = None

@@ -165,6 +165,12 @@ def Conv2d(im, filter, kernelShape, pad=None, stride=(1, 1), dilation=None):
     return im.g.apply(K_CONV2D, [im, filter], ints=list(kernelShape) + list(pad) + list(stride) + list(dilation))
 
 
+def Conv1d(im, filter, kernel, pad, stride, dilation):
+    """nnops.Conv1d (ops/nn/api_cuda.go:18-20; nn.go:308-310): a Conv2d over (B, C, 1, W) with
+    kernel {1, kernel}, pad {0, pad}, stride {1, stride}, dilation {1, dilation}."""
+    return Conv2d(im, filter, (1, kernel), [0, pad], [1, stride], [1, dilation])
+
+
 def MaxPool2D(x, kernel, pad, stride):
     """nnops.MaxPool2D (nn.go:322-375): pad has 2 values (symmetric) or 4 (N, S, W, E)."""
     return x.g.apply(K_MAXPOOL, [x], ints=list(kernel) + [len(pad)] + list(pad) + list(stride))
@@ -291,11 +297,18 @@ class TapeMachine:
     """NewTapeMachine(g, ...) / RunAll / Reset / Close (vm_tape.go:45-249)."""
 
     def __init__(self, g, graph_replay=False, reupload_resident=False, fuse_activations=False,
-                 device=0, compile_only=False):
+                 device=0, compile_only=False, engine=None):
         self.g = g
         self.lib = g.lib
         self.fused = self.lib.ghh_graph_fuse_activations(g.h) if fuse_activations else 0
-        self.h = self.lib.ghh_tape_new(g.h, int(graph_replay), int(reupload_resident))
+        self._shared_engine = engine  # WithEngine(e) (vm.go:318-329): kept alive, never closed here
+        # graph_replay: False, True (capture on the second run, replay from then on) or
+        # "measured" (time plain submits against replays first, keep the quicker)
+        mode = 2 if graph_replay == "measured" else int(bool(graph_replay))
+        if engine is not None:
+            self.h = self.lib.ghh_tape_new_with_engine(g.h, engine.h, mode, int(reupload_resident))
+        else:
+            self.h = self.lib.ghh_tape_new(g.h, mode, int(reupload_resident))
         if compile_only:
             self._check(self.lib.ghh_tape_compile_only(self.h))
         else:
@@ -329,6 +342,16 @@ class TapeMachine:
     def graph_launches(self):
         return self.lib.ghh_tape_graph_launches(self.h)
 
+    def segment_verdict(self, segment=0):
+        """'measuring', 'plain' or 'replay' for a segment of the last run (graph_replay="measured")."""
+        return ("measuring", "plain", "replay")[self.lib.ghh_tape_segment_verdict(self.h, segment)]
+
+    def phase_ns(self):
+        """Host nanoseconds of the last RunAll: (whole call, launching, waiting for the device)."""
+        out = (C.c_int64 * 3)()
+        self.lib.ghh_tape_phase_ns(self.h, out)
+        return tuple(out)
+
     def submit_calls(self):
         return self.lib.ghh_tape_submit_calls(self.h)
 
@@ -342,5 +365,12 @@ class TapeMachine:
         return buf.value.decode()
 
 
-def NewTapeMachine(g, **kw):
+def WithEngine(e):
+    """VMOpt of the reference (vm.go:318-329): NewTapeMachine(g, WithEngine(e))."""
+    return {"engine": e}
+
+
+def NewTapeMachine(g, *opts, **kw):
+    for o in opts:
+        kw.update(o)
     return TapeMachine(g, **kw)

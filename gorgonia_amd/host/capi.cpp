@@ -215,10 +215,23 @@ int ghh_graph_fuse_activations(ghh_graph* g) { return g->g.FuseActivations(); }
 ghh_tape* ghh_tape_new(ghh_graph* g, int graph_replay, int reupload_resident) {
   TapeOptions o;
   o.graph_replay = graph_replay != 0;
+  o.replay_measured = graph_replay == 2;
   o.reupload_resident = reupload_resident != 0;
   ghh_tape* t = new ghh_tape();
   t->t = new TapeMachine(&g->g, o);
   t->eng.e = &t->t->Eng();
+  t->eng.owned = false;
+  return t;
+}
+ghh_tape* ghh_tape_new_with_engine(ghh_graph* g, ghh_engine* e, int graph_replay, int reupload_resident) {
+  if (!g || !e || !e->e) return nullptr;
+  TapeOptions o;
+  o.graph_replay = graph_replay != 0;
+  o.replay_measured = graph_replay == 2;
+  o.reupload_resident = reupload_resident != 0;
+  ghh_tape* t = new ghh_tape();
+  t->t = new TapeMachine(&g->g, o, e->e);
+  t->eng.e = e->e;
   t->eng.owned = false;
   return t;
 }
@@ -244,5 +257,7 @@ int ghh_tape_program_string(ghh_tape* t, char* buf, int cap) {
   return (int)s.size();
 }
 ghh_engine* ghh_tape_engine(ghh_tape* t) { return &t->eng; }
+int ghh_tape_segment_verdict(ghh_tape* t, int segment) { return t->t->SegmentVerdict(segment); }
+void ghh_tape_phase_ns(ghh_tape* t, int64_t* out3) { t->t->PhaseNs(out3); }
 
 }  // extern "C"

@@ -362,6 +362,11 @@ Status Engine::GraphLaunch(int id) {
   int rc = gh_graph_launch(ctx_, id);
   return rc == GH_OK ? Status::OK() : fail(rc, "gh_graph_launch");
 }
+Status Engine::GraphDestroy(int id) {
+  if (!ctx_ || id < 0) return Status::OK();
+  int rc = gh_graph_destroy(ctx_, id);
+  return rc == GH_OK ? Status::OK() : fail(rc, "gh_graph_destroy");
+}
 
 // ---- linalg -------------------------------------------------------------------------
 static Status checkThreeFloat(const Tensor& a, const Tensor& b, const Tensor& ret) {

@@ -182,6 +182,7 @@ class Engine {
   Status GraphBegin();
   Status GraphEnd(int* id);
   Status GraphLaunch(int id);
+  Status GraphDestroy(int id);
 
  private:
   Status fail(int rc, const std::string& what);

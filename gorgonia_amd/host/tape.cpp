@@ -1,6 +1,7 @@
 #include "tape.hpp"
 
 #include <algorithm>
+#include <chrono>
 #include <cstring>
 #include <sstream>
 
@@ -11,6 +12,9 @@ namespace gorgonia {
 // yolo-shaped stack written by its last kernel costs ~57 us of PCIe time; the
 // explicit copy behind the segment it replaces cost ~85 us.)
 static constexpr int64_t kStageLimit = 8 << 20;
+// inputs re-uploaded on every run are staged through pinned memory up to these sizes
+static constexpr int64_t kStageInLimit = 16 << 20;    // per input (what one copy kernel moves)
+static constexpr int64_t kStageInTotal = 512ll << 20; // per machine
 
 static Status bad(const std::string& m) { return Status::Err(GH_EINVAL, m); }
 
@@ -309,7 +313,9 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
     case OpKind::ElemBin: {
       Tensor& a = *in[0];
       Tensor& b = *in[1];
-      static const char* names[] = {"Add", "Sub", "Mul", "Div", "Pow", "Lt", "Lte", "Gt", "Gte", "ElEq", "ElNe"};
+      static const char* names[GH_BINFN__COUNT] = {"Add", "Sub", "Mul", "Div", "Pow", "Lt",
+                                                   "Lte", "Gt",  "Gte", "ElEq", "ElNe", "Mod"};
+      if (op.fn < 0 || op.fn >= GH_BINFN__COUNT) return Status::Err(GH_ENOFUNC, "no binary function " + std::to_string(op.fn));
       const bool as = a.shape.IsScalar(), bs = b.shape.IsScalar();
       if (as != bs) {  // tensor-scalar: the *Scalar methods (operatorPointwise_binary.go:359-426)
         Tensor& t = as ? b : a;
@@ -583,6 +589,14 @@ int Graph::NewTensor(const Shape& s, Dtype dt, const void* host, bool resident) 
 }
 
 Status Graph::Apply(const OpSpec& op, const std::vector<int>& inputs, int* out) {
+  // an operator the engine has no function for is refused here, before any
+  // table is indexed with it (the reference's HasFunc check, op_math_cuda.go:34-36)
+  if ((int)op.kind < 0 || (int)op.kind > (int)OpKind::RectifyDiff)
+    return Status::Err(GH_ENOFUNC, "Apply: no operator of kind " + std::to_string((int)op.kind));
+  if ((op.kind == OpKind::ElemBin || op.kind == OpKind::BroadcastBin) && (op.fn < 0 || op.fn >= GH_BINFN__COUNT))
+    return Status::Err(GH_ENOFUNC, "Apply: no binary function " + std::to_string(op.fn));
+  if (op.kind == OpKind::SolverStep && (op.fn < 0 || op.fn >= GH_SOLVER__COUNT))
+    return Status::Err(GH_ENOFUNC, "Apply: no solver " + std::to_string(op.fn));
   std::vector<const Shape*> shapes;
   for (int i : inputs) {
     if (i < 0 || i >= (int)nodes_.size()) return bad("Apply: unknown input node");
@@ -762,12 +776,18 @@ Status TapeMachine::Compile() {
   regs_.assign((size_t)nreg, Tensor());
   reg_live_.assign((size_t)nreg, 0);
   resident_done_.assign((size_t)N, 0);
-  std::vector<int64_t> reg_bytes((size_t)nreg, 0);
+  reg_bytes_.assign((size_t)nreg, 0);
+  std::vector<int64_t>& reg_bytes = reg_bytes_;
   gpumem_ = 0;
 
+  // Inputs first, operators after: every upload sits at the head of the program
+  // (the reference interleaves them, compile.go:16-60; the values an operator
+  // sees are the same), so the operators of a run form one uninterrupted segment.
+  for (int pass = 0; pass < 2; pass++)
   for (int i = 0; i < N; i++) {
     Node& n = nodes[(size_t)i];
     if (n.fused_away) continue;
+    if ((pass == 0) != (n.is_input && n.alias_of < 0)) continue;
     if (n.alias_of >= 0 && n.op.kind != OpKind::Set && n.op.kind != OpKind::SolverStep) continue;  // a view: nothing to run
     const int r = node_reg_[(size_t)i];
     const int64_t bytes = bytes_of(n);
@@ -829,14 +849,39 @@ Status TapeMachine::Init(int device) {
   int64_t need = 0;
   for (auto& in : prog_)
     if (in.kind == InstrKind::Alloc) need += (in.size + 31) / 32 * 32;
-  st = eng_.Init(device, need > gpumem_ ? need : gpumem_);
-  if (!st.ok()) return st;
+  if (borrowed_) {
+    if (!eng_.Initialized()) return Status::Err(GH_ESTATE, "WithEngine: the engine is not initialised");
+    int64_t room = 0;
+    for (auto& hole : eng_.Allocator().freelist()) room += hole.second;
+    if (need > room)
+      return Status::Err(GH_EOOM, "WithEngine: the program needs " + std::to_string(need) +
+                                      " bytes of registers, the engine's arena has " + std::to_string(room) + " free");
+  } else {
+    st = eng_.Init(device, need > gpumem_ ? need : gpumem_);
+    if (!st.ok()) return st;
+  }
+  open_ = true;
   stage_.assign(g_->Nodes().size(), nullptr);
-  for (auto& in : prog_)
+  stage_in_.assign(g_->Nodes().size(), nullptr);
+  int64_t staged_in = 0;
+  for (auto& in : prog_) {
     if (in.kind == InstrKind::StageOut || in.kind == InstrKind::AllocHost) {
       st = eng_.HostAlloc(in.size, &stage_[(size_t)in.node]);
       if (!st.ok()) return st;
     }
+    // an input uploaded on every run goes through a pinned buffer of its own
+    // (RunAll waits for the device before it returns, so one buffer per input
+    // is the whole ring); inputs past the cap fall back to a direct copy
+    if (in.kind == InstrKind::Transport) {
+      const Node& n = g_->Nodes()[(size_t)in.node];
+      if ((n.resident && !opt_.reupload_resident) || in.size % 4 != 0 || in.size > kStageInLimit ||
+          staged_in + in.size > kStageInTotal)
+        continue;
+      st = eng_.HostAlloc(in.size, &stage_in_[(size_t)in.node]);
+      if (!st.ok()) return st;
+      staged_in += in.size;
+    }
+  }
   return Status::OK();
 }
 
@@ -845,9 +890,25 @@ uint64_t TapeMachine::RegisterAddress(int node) const {
   return regs_[(size_t)node_reg_[(size_t)node]].mem;
 }
 
+static inline int64_t now_ns() {
+  return std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
 Status TapeMachine::flush() {
   segments_++;
-  if (!opt_.graph_replay) return eng_.DoWork();
+  // launch, then wait, with the host time of each kept for PhaseNs()
+  auto launch_and_wait = [&](auto&& launch) -> Status {
+    const int64_t t0 = now_ns();
+    Status st = launch();
+    const int64_t t1 = now_ns();
+    ns_launch_ += t1 - t0;
+    if (!st.ok()) return st;
+    st = eng_.Sync();
+    ns_wait_ += now_ns() - t1;
+    return st;
+  };
+  auto eager = [&]() { return launch_and_wait([&]() { return eng_.SubmitPending(); }); };
+  if (!opt_.graph_replay) return eager();
   const size_t idx = (size_t)seg_index_++;
   if (seg_cache_.size() <= idx) seg_cache_.resize(idx + 1);
   SegCache& sc = seg_cache_[idx];
@@ -859,16 +920,47 @@ Status TapeMachine::flush() {
   // (measured on MI355X: one small kernel per run 29 us replayed against 13 us
   // eager, break-even at about five kernels), so short segments stay eager.
   constexpr size_t kMinGraphCmds = 5;
-  if (cur.size() < kMinGraphCmds) return eng_.DoWork();
+  if (cur.size() < kMinGraphCmds) {
+    sc.verdict = SegCache::Plain;
+    return eager();
+  }
+  if (opt_.replay_measured && same && sc.verdict != SegCache::Replay) {
+    // two timed plain runs, a capture, two timed replays, then the verdict
+    constexpr int kTimed = 2;
+    if (sc.verdict == SegCache::Plain) return eager();
+    if (sc.plain_timed < kTimed) {
+      const int64_t l0 = ns_launch_, w0 = ns_wait_;
+      Status st = eager();
+      sc.plain_ns = std::min(sc.plain_ns, (ns_launch_ - l0) + (ns_wait_ - w0));
+      sc.plain_timed++;
+      return st;
+    }
+    if (sc.graph_id >= 0 && sc.replay_timed < kTimed) {
+      eng_.DropSegment();
+      graph_launches_++;
+      const int64_t l0 = ns_launch_, w0 = ns_wait_;
+      Status st = launch_and_wait([&]() { return eng_.GraphLaunch(sc.graph_id); });
+      sc.replay_ns = std::min(sc.replay_ns, (ns_launch_ - l0) + (ns_wait_ - w0));
+      if (++sc.replay_timed == kTimed) {
+        if (sc.replay_ns < sc.plain_ns) {
+          sc.verdict = SegCache::Replay;
+        } else {
+          sc.verdict = SegCache::Plain;
+          eng_.GraphDestroy(sc.graph_id);
+          sc.graph_id = -1;
+        }
+      }
+      return st;
+    }
+    // falls through to the capture below
+  }
   if (sc.graph_id >= 0 && same) {
     eng_.DropSegment();
-    Status st = eng_.GraphLaunch(sc.graph_id);
-    if (!st.ok()) return st;
     graph_launches_++;
-    return eng_.Sync();
+    return launch_and_wait([&]() { return eng_.GraphLaunch(sc.graph_id); });
   }
   if (same && runs_ >= 1) {
-    // second identical run of this segment: capture it, then launch the capture
+    // an identical run of this segment: capture it, then launch the capture
     Status st = eng_.GraphBegin();
     if (!st.ok()) return st;
     st = eng_.SubmitPending();
@@ -877,14 +969,16 @@ Status TapeMachine::flush() {
     if (!st.ok()) return st;
     if (!st2.ok()) return st2;
     sc.graph_id = id;
-    st = eng_.GraphLaunch(id);
-    if (!st.ok()) return st;
     graph_launches_++;
-    return eng_.Sync();
+    return launch_and_wait([&]() { return eng_.GraphLaunch(id); });
   }
   sc.cmds = cur;  // first sight (or the pointer set changed): run eagerly, remember
+  if (sc.graph_id >= 0) eng_.GraphDestroy(sc.graph_id);  // the capture of the old pointer set is dead
   sc.graph_id = -1;
-  return eng_.DoWork();
+  sc.plain_timed = sc.replay_timed = 0;
+  sc.plain_ns = sc.replay_ns = INT64_MAX;
+  sc.verdict = SegCache::Measuring;
+  return eager();
 }
 
 Status TapeMachine::RunAll() {
@@ -892,6 +986,8 @@ Status TapeMachine::RunAll() {
   auto& nodes = g_->Nodes();
   segments_ = 0;
   seg_index_ = 0;
+  const int64_t t_run = now_ns();
+  ns_launch_ = ns_wait_ = 0;
   for (size_t pc = 0; pc < prog_.size(); pc++) {
     const Instr& in = prog_[pc];
     Status st;
@@ -913,6 +1009,14 @@ Status TapeMachine::RunAll() {
       case InstrKind::Transport: {
         Node& n = nodes[(size_t)in.node];
         if (n.resident && resident_done_[(size_t)in.node] && !opt_.reupload_resident) break;
+        if (void* pinned = stage_in_[(size_t)in.node]) {
+          // host value -> pinned buffer now, pinned buffer -> register as a command of
+          // the segment: the upload is captured and replayed with the operators
+          std::memcpy(pinned, n.host, (size_t)in.size);
+          eng_.RecordCopy(regs_[(size_t)in.reg].mem, (uint64_t)(uintptr_t)pinned, in.size);
+          resident_done_[(size_t)in.node] = 1;
+          break;
+        }
         st = eng_.MemcpyHtoD(regs_[(size_t)in.reg].mem, n.host, in.size);
         if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": devTrans");
         resident_done_[(size_t)in.node] = 1;
@@ -979,24 +1083,56 @@ Status TapeMachine::RunAll() {
   // segment stays replayable.
   eng_.Allocator().coalesce();
   eng_.Allocator().reset_stats();
+  ns_total_ = now_ns() - t_run;
   return st;
 }
 
+void TapeMachine::drop_graphs() {
+  for (SegCache& sc : seg_cache_) {
+    if (sc.graph_id >= 0) eng_.GraphDestroy(sc.graph_id);
+    sc.graph_id = -1;
+    sc.cmds.clear();
+  }
+}
+
+// Give back what this machine holds in the arena (a shared engine's other
+// users keep theirs).
+void TapeMachine::release_registers() {
+  for (size_t r = 0; r < reg_live_.size(); r++)
+    if (reg_live_[r]) {
+      eng_.Put(regs_[r].mem, reg_bytes_[r]);
+      reg_live_[r] = 0;
+    }
+}
+
 Status TapeMachine::Reset() {
-  if (!eng_.Initialized()) return Status::OK();
+  if (!open_ || !eng_.Initialized()) return Status::OK();
   eng_.DropSegment();
-  eng_.ResetAllocator();
+  if (borrowed_) release_registers();
+  else eng_.ResetAllocator();
   std::fill(reg_live_.begin(), reg_live_.end(), 0);
   std::fill(resident_done_.begin(), resident_done_.end(), 0);
   return Status::OK();
 }
 
 Status TapeMachine::Close() {
-  for (void*& p : stage_) {
-    eng_.HostFree(p);
-    p = nullptr;
+  if (!open_) return Status::OK();
+  open_ = false;
+  if (eng_.Initialized()) {
+    drop_graphs();
+    for (auto* v : {&stage_, &stage_in_})
+      for (void*& p : *v) {
+        eng_.HostFree(p);
+        p = nullptr;
+      }
   }
-  return eng_.Close();
+  if (!borrowed_) return eng_.Close();
+  if (eng_.Initialized()) {
+    eng_.DropSegment();
+    release_registers();
+    eng_.Allocator().coalesce();
+  }
+  return Status::OK();
 }
 
 std::string TapeMachine::ProgramString() const {

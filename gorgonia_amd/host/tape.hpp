@@ -135,15 +135,28 @@ struct Instr {
 
 struct TapeOptions {
   bool graph_replay = false;      // capture each segment into a hipGraph and replay it
+  // With graph_replay: time a segment's plain submits and its replays over its
+  // first runs and keep whichever finishes sooner.  A replayed graph saves the
+  // per-kernel launch calls but starts later than the first plain launch does,
+  // so it only pays for segments of many short kernels.
+  bool replay_measured = false;
   bool reupload_resident = false; // treat resident inputs like the reference does (H2D every run)
 };
 
 class TapeMachine {
  public:
-  TapeMachine(Graph* g, const TapeOptions& o) : g_(g), opt_(o) {}
+  TapeMachine(Graph* g, const TapeOptions& o) : g_(g), opt_(o), eng_(own_) {}
+  // WithEngine(e) (vm.go:318-329): the machine computes on an engine its caller
+  // created and initialised, takes its registers from that engine's arena and
+  // leaves the engine open when it closes.  Machines that share an engine run
+  // one after the other, never at the same time.
+  TapeMachine(Graph* g, const TapeOptions& o, Engine* shared)
+      : g_(g), opt_(o), eng_(shared ? *shared : own_), borrowed_(shared != nullptr) {}
   ~TapeMachine();
   // Compile (compile.go:16-60 for forward graphs), size the arena from the
   // program (compile.go:148-216) and create the engine (vm_tape_cuda.go:17-41).
+  // With a shared engine nothing is created: the engine must be initialised
+  // already and its arena must still have room for the program's registers.
   Status Init(int device);
   Status Compile();  // program only, no device
   Status RunAll();
@@ -153,28 +166,51 @@ class TapeMachine {
   const std::vector<Instr>& Program() const { return prog_; }
   int64_t GpuMem() const { return gpumem_; }
   int Segments() const { return segments_; }      // flush points in the last run
+  // How segment `i` of the last run is executed: 0 still measuring, 1 plain submits, 2 graph replay.
+  int SegmentVerdict(int i) const { return i >= 0 && i < (int)seg_cache_.size() ? (int)seg_cache_[(size_t)i].verdict : 0; }
   int GraphLaunches() const { return graph_launches_; }
+  // Host time of the last RunAll in nanoseconds: [0] the whole call, [1] inside
+  // graph launches and submits, [2] waiting for the device.
+  void PhaseNs(int64_t out[3]) const { out[0] = ns_total_; out[1] = ns_launch_; out[2] = ns_wait_; }
   uint64_t RegisterAddress(int node) const;
   std::string ProgramString() const;              // program.String() (vm_tape.go:493-522)
 
  private:
   Status flush();
+  void drop_graphs();   // destroy every captured segment graph
+  void release_registers();
   Graph* g_;
   TapeOptions opt_;
-  Engine eng_;
+  Engine own_;
+  Engine& eng_;          // own_, or the caller's engine
+  bool borrowed_ = false;
+  bool open_ = false;    // Init done, Close not yet
   std::vector<Instr> prog_;
   std::vector<Tensor> regs_;       // one per register
   std::vector<int> node_reg_;      // node -> register
   std::vector<char> reg_live_;     // register currently holds arena memory
+  std::vector<int64_t> reg_bytes_; // register -> bytes it was allocated with
   std::vector<char> resident_done_;
   // Small outputs leave through pinned host buffers written by a copy at the
   // end of the segment, so a replayed run is one graph launch and one wait;
   // node -> buffer (null: the output is read with a D2H copy after the flush).
   std::vector<void*> stage_;
+  // Inputs uploaded on every run enter through pinned host buffers read by a
+  // copy at the head of the segment; node -> buffer (null: direct H2D copy).
+  std::vector<void*> stage_in_;
   int64_t gpumem_ = 0;
   int runs_ = 0, segments_ = 0, graph_launches_ = 0;
+  int64_t ns_total_ = 0, ns_launch_ = 0, ns_wait_ = 0;
   // per-segment replay cache
-  struct SegCache { std::vector<gh_cmd> cmds; int graph_id = -1; };
+  struct SegCache {
+    std::vector<gh_cmd> cmds;
+    int graph_id = -1;
+    // replay_measured bookkeeping: host nanoseconds (launch + wait) of the best
+    // plain and the best replayed run so far, and the verdict
+    int plain_timed = 0, replay_timed = 0;
+    int64_t plain_ns = INT64_MAX, replay_ns = INT64_MAX;
+    enum { Measuring, Plain, Replay } verdict = Measuring;
+  };
   std::vector<SegCache> seg_cache_;
   int seg_index_ = 0;
 };

@@ -147,6 +147,9 @@ enum gh_unaryfn {
  *             dim[0]=outer dim[1]=mid dim[2]=inner; small has `mid` elements,
  *             element (o,m,i) pairs big[o,m,i] with small[m]
  * MEMCPY_D2D  ptr[0]=dst ptr[1]=src        dim[0]=bytes
+ *             either side may be pinned host memory from gh_host_alloc (the
+ *             device reads or writes it over the bus): this is how a segment
+ *             carries its own input uploads and result downloads
  * GEMM        ptr[0]=A ptr[1]=B ptr[2]=C   dim[0..2]=m,n,k  dim[3..5]=lda,ldb,ldc
  *             dim[6]=batch (0/1 = single)  dim[7..9]=strideA,strideB,strideC
  *             row-major; C(m x n) = op(A)(m x k) * op(B)(k x n)

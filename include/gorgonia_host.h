@@ -123,7 +123,22 @@ GH_API int ghh_graph_node_shape(ghh_graph* g, int node, int64_t* shape, int cap)
 GH_API int ghh_graph_node_dtype(ghh_graph* g, int node);
 GH_API int ghh_graph_fuse_activations(ghh_graph* g);
 
+/* graph_replay: 0 every segment is submitted command by command on every run;
+ * 1 a segment whose commands repeat is captured into a hipGraph on its second
+ * run and replayed from then on; 2 as 1, but the machine first times two plain
+ * runs and two replays of the segment and keeps the quicker way
+ * (ghh_tape_segment_verdict tells which).  reupload_resident: resident inputs
+ * are uploaded on every run like all others (vm_tape_cuda.go:220-243). */
 GH_API ghh_tape* ghh_tape_new(ghh_graph* g, int graph_replay, int reupload_resident);
+/* NewTapeMachine(g, WithEngine(e)) (vm.go:318-329): the machine runs on the
+ * caller's engine, which must be initialised (ghh_engine_init) before
+ * ghh_tape_init and must outlive the machine.  Registers come out of that
+ * engine's arena and go back to it on ghh_tape_reset / ghh_tape_close; the
+ * engine itself stays open.  ghh_tape_init's device argument is ignored, and
+ * it returns GH_ESTATE for an engine that is not initialised, GH_EOOM when the
+ * arena has less free space than the program's registers need.  Machines on
+ * one engine run one after the other. */
+GH_API ghh_tape* ghh_tape_new_with_engine(ghh_graph* g, ghh_engine* e, int graph_replay, int reupload_resident);
 GH_API void ghh_tape_destroy(ghh_tape* t);
 GH_API const char* ghh_tape_last_error(ghh_tape* t);
 GH_API int ghh_tape_init(ghh_tape* t, int device);   /* compile + engine init */
@@ -137,6 +152,12 @@ GH_API int64_t ghh_tape_submit_calls(ghh_tape* t);
 GH_API uint64_t ghh_tape_register_address(ghh_tape* t, int node);
 GH_API int ghh_tape_program_string(ghh_tape* t, char* buf, int cap);
 GH_API ghh_engine* ghh_tape_engine(ghh_tape* t);     /* borrowed: do not destroy */
+/* How segment `segment` of the last run executes: 0 undecided (still being timed, or graph_replay
+ * is not 2), 1 plain submits, 2 graph replay. */
+GH_API int ghh_tape_segment_verdict(ghh_tape* t, int segment);
+/* Host time of the last RunAll in nanoseconds: out3[0] the whole call, out3[1]
+ * inside gh_submit / gh_graph_launch, out3[2] waiting for the device. */
+GH_API void ghh_tape_phase_ns(ghh_tape* t, int64_t* out3);
 /* compile only (no device): lets CPU tests inspect the instruction stream */
 GH_API int ghh_tape_compile_only(ghh_tape* t);
 

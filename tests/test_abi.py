@@ -79,3 +79,21 @@ def test_validation_rejects_bad_commands():
 
 def test_version_string():
     assert b"gfx950" in _ffi.load().gh_version()
+
+
+def test_headers_are_plain_c99(tmp_path):
+    """cgo compiles the header as C: both headers, and the plain-C consumer that fills a gh_cmd[]
+    and calls gh_submit, must pass gcc -std=c99 -pedantic -Werror (no C++-isms, no extensions)."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    assert gcc, "gcc is part of the image"
+    tu = tmp_path / "both.c"
+    tu.write_text('#include "gorgonia_hip.h"\n#include "gorgonia_host.h"\n'
+                  "int main(void) { gh_cmd c; ghh_tensor t; (void)c; (void)t; return (int)sizeof(gh_cmd) - 248; }\n")
+    flags = ["-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include")]
+    p = subprocess.run([gcc] + flags + ["-fsyntax-only", str(tu)], capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr
+    src = os.path.join(ROOT, "tests", "c_consumer", "consumer.c")
+    p = subprocess.run([gcc] + flags + ["-c", src, "-o", str(tmp_path / "consumer.o")], capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr

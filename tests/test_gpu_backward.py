@@ -77,6 +77,10 @@ CONV_BWD_CASES = [
     (16, 64, 7, 7, 128, 3, 3, (1, 1), (1, 1), (1, 1)),
     (2, 16, 52, 52, 32, 3, 3, (1, 1), (1, 1), (1, 1)),
     (2, 256, 13, 13, 512, 3, 3, (1, 1), (1, 1), (1, 1)),
+    # Conv1d shapes (ops/nn/api_cuda.go:18-20): H = 1, kernel {1,k}
+    (3, 4, 1, 37, 6, 1, 3, (0, 1), (1, 1), (1, 1)),
+    (2, 8, 1, 64, 16, 1, 5, (0, 2), (1, 2), (1, 1)),
+    (2, 3, 1, 50, 5, 1, 3, (0, 2), (1, 1), (1, 2)),
 ]
 
 

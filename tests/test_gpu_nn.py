@@ -69,6 +69,11 @@ CONV_CASES = [
     (2, 16, 66, 68, 40, 3, 3, (0, 0), (1, 1), (1, 1)),
     (1, 8, 104, 104, 64, 3, 3, (1, 1), (1, 1), (1, 1)),
     (1, 16, 70, 130, 96, 3, 3, (1, 1), (1, 1), (1, 1)),
+    # Conv1d (ops/nn/api_cuda.go:18-20): H = 1, kernel {1,k}, pad {0,p}, stride {1,s}, dilation {1,d}
+    (3, 4, 1, 37, 6, 1, 3, (0, 1), (1, 1), (1, 1)),
+    (2, 8, 1, 64, 16, 1, 5, (0, 2), (1, 2), (1, 1)),
+    (2, 3, 1, 50, 5, 1, 3, (0, 2), (1, 1), (1, 2)),
+    (4, 16, 1, 128, 32, 1, 7, (0, 0), (1, 3), (1, 2)),
 ]
 
 

@@ -143,10 +143,134 @@ def test_one_submit_per_segment(ctx):
 
 
 def test_reupload_mode_matches_resident(ctx):
+    """Inputs uploaded on every run (what the reference does with every input,
+    vm_tape_cuda.go:220-243) travel inside the segment: all uploads sit at the head of the
+    program, go through pinned buffers, and a run stays one gh_submit (eager) or one graph
+    launch (replayed) - whatever the number of inputs."""
     inp = configs.convnet_inputs(8)
     m1, _, r1 = run_once(configs.build_convnet, inp)
-    g, outs = configs.build_convnet(inp, resident=False)
-    m2 = G.NewTapeMachine(g)
-    m2.RunAll(); m2.RunAll()
-    assert_bits_equal(outs["out"], r1["out"], "re-uploaded weights")
-    m1.Close(); m2.Close()
+    for kw in (dict(), dict(reupload_resident=True), dict(graph_replay=True, fuse_activations=True),
+               dict(graph_replay=True, fuse_activations=True, reupload_resident=True)):
+        g, outs = configs.build_convnet(inp, resident=False)
+        m2 = G.NewTapeMachine(g, **kw)
+        prog = [l.split()[1] for l in m2.program().splitlines()[1:] if "\t" in l]
+        first_op = prog.index("execOp")
+        assert "devTrans" not in prog[first_op:], "an upload after the first operator splits the segment"
+        assert prog.count("devTrans") == 6
+        for it in range(4):
+            outs["out"][...] = -1.0
+            s0, l0 = m2.submit_calls(), m2.graph_launches()
+            m2.RunAll()
+            crossings = (m2.submit_calls() - s0) + (m2.graph_launches() - l0)
+            assert crossings <= 2, f"{kw} run {it}: {crossings} submits/launches"
+            assert m2.segments() == 1
+            assert_bits_equal(outs["out"], r1["out"], f"re-uploaded inputs {kw} run {it}")
+        if kw.get("graph_replay"):
+            assert m2.graph_launches() >= 2 and m2.submit_calls() - s0 == 0
+        # a new value bound to an input reaches the device on the next run
+        x2 = inp["x"][::-1].copy()
+        G.Let(G.Node(g, 0), x2)
+        m2.RunAll()
+        m3, _, r3 = run_once(configs.build_convnet, dict(inp, x=x2))
+        assert_bits_equal(outs["out"], r3["out"], f"rebound input {kw}")
+        m3.Close()
+        m2.Close()
+    m1.Close()
+
+
+def test_with_engine_machines_share_one_arena(ctx):
+    """NewTapeMachine(g, WithEngine(e)) (vm.go:318-329): two machines run one after the
+    other on the caller's engine, give the results of machines with engines of their
+    own, hand their registers back on Close and leave the engine open."""
+    from gorgonia_amd.engine import Engine, EngineError
+    inp_a = configs.convnet_inputs(8)
+    inp_b = configs.mlp_inputs(64)
+    ma, _, want_a = run_once(configs.build_convnet, inp_a)
+    ma.Close()
+    mb, _, want_b = run_once(configs.build_mlp, inp_b)
+    mb.Close()
+
+    e = Engine()
+    ga, outs_a = configs.build_convnet(inp_a)
+    with pytest.raises(EngineError, match="not initialised"):
+        G.NewTapeMachine(ga, G.WithEngine(e))
+    e.Init(0, 256 << 20)
+    m1 = G.NewTapeMachine(ga, G.WithEngine(e), graph_replay=True)
+    gb, outs_b = configs.build_mlp(inp_b)
+    m2 = G.NewTapeMachine(gb, G.WithEngine(e))
+    for it in range(3):
+        outs_a["out"][...] = -1.0
+        m1.RunAll()
+        assert_bits_equal(outs_a["out"], want_a["out"], f"shared engine, convnet run {it}")
+        outs_b["out"][...] = -1.0
+        m2.RunAll()
+        assert_bits_equal(outs_b["out"], want_b["out"], f"shared engine, mlp run {it}")
+    # the two machines hold different arena memory for their resident inputs (the weights)
+    held_a = {m1.register_address(G.Node(ga, i)) for i in (1, 5, 9, 14, 17)}
+    held_b = {m2.register_address(G.Node(gb, i)) for i in (1, 2)}
+    assert 0 not in held_a | held_b and not (held_a & held_b)
+    m1.Reset()
+    m1.RunAll()
+    assert_bits_equal(outs_a["out"], want_a["out"], "shared engine, after Reset")
+    m1.Close()
+    m2.RunAll()   # the other machine is untouched by the first one's Close
+    assert_bits_equal(outs_b["out"], want_b["out"], "shared engine, after the other machine closed")
+    m2.Close()
+    # the engine is still open and its arena is whole again: a machine that needs most of it fits
+    gc, outs_c = configs.build_convnet(inp_a)
+    m3 = G.NewTapeMachine(gc, G.WithEngine(e))
+    m3.RunAll()
+    assert_bits_equal(outs_c["out"], want_a["out"], "shared engine, third machine")
+    m3.Close()
+    # an arena too small for the program is refused at init with the allocator's error code
+    small = Engine()
+    small.Init(0, 4096)
+    gd, _ = configs.build_convnet(inp_a)
+    with pytest.raises(EngineError, match="arena has"):
+        G.NewTapeMachine(gd, G.WithEngine(small))
+    small.Close(); small.destroy()
+    e.Close(); e.destroy()
+
+
+def test_conv1d_on_the_tape(ctx):
+    """nnops.Conv1d (ops/nn/api_cuda.go:18-20) is Conv2d over a height-1 image."""
+    from oracle import binding as O
+    x = synth.uniform(11, (4, 8, 1, 96), -1, 1)
+    w = synth.he_normal(12, (12, 8, 1, 5))
+    for pad, stride, dil in ((2, 1, 1), (0, 2, 1), (4, 1, 2), (3, 3, 2)):
+        g = G.NewGraph()
+        y = G.Conv1d(G.NewTensor(g, x), G.NewTensor(g, w, resident=True), 5, pad, stride, dil)
+        out = G.Read(y)
+        m = G.NewTapeMachine(g)
+        m.RunAll()
+        want = O.conv2d_direct_f64(x, w, (0, pad), (1, stride), (1, dil))
+        assert out.shape == want.shape == (4, 12, 1, (96 + 2 * pad - (dil * 4 + 1)) // stride + 1)
+        assert rel_frobenius(out, want) <= 1e-5, (pad, stride, dil)
+        m.Close()
+
+
+def test_measured_replay_keeps_results_and_settles(ctx):
+    """graph_replay="measured": the machine times plain submits against replays of a segment on
+    its first runs and keeps the quicker; every run along the way, and after the verdict, stores
+    the bits of the plain run."""
+    for build, inp in ((configs.build_convnet, configs.convnet_inputs(16)),
+                       (configs.build_mlp, configs.mlp_inputs(64))):
+        m0, _, want = run_once(build, inp, fuse_activations=True)
+        m0.Close()
+        g, outs = build(inp)
+        m = G.NewTapeMachine(g, graph_replay="measured", fuse_activations=True)
+        assert m.segment_verdict() == "measuring"
+        for it in range(12):
+            outs["out"][...] = -1.0
+            m.RunAll()
+            assert_bits_equal(outs["out"], want["out"], f"measured replay, run {it}")
+            if it < 3 and build is configs.build_convnet:
+                assert m.segment_verdict() == "measuring"
+        assert m.segment_verdict() in ("plain", "replay")
+        if build is configs.build_mlp:
+            assert m.segment_verdict() == "plain"   # three commands: too short to be worth a graph
+        # launches: the capture and two timed replays, more only if replay won
+        assert m.graph_launches() in (0, 3) or m.segment_verdict() == "replay"
+        total, launch, wait = m.phase_ns()
+        assert total >= launch + wait > 0
+        m.Close()

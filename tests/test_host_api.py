@@ -184,3 +184,33 @@ def test_tape_program_convnet_fusion():
     m2 = G.NewTapeMachine(g2, compile_only=True)
     assert m2.program().count(" rectify") == 4
     m2.Close()
+
+
+def test_apply_refuses_functions_the_engine_does_not_have():
+    """Operator kind, binary function and solver numbers are range-checked when the
+    node is made (no name table is ever indexed with them); Mod is a real entry."""
+    from gorgonia_amd import _ffi
+    g = G.NewGraph()
+    a = G.NewTensor(g, np.zeros((4, 6), np.float32))
+    b = G.NewTensor(g, np.zeros((4, 6), np.float32))
+    for kind, fn in ((G.K_ELEMBIN, 12), (G.K_ELEMBIN, -1), (G.K_BCAST, 99), (G.K_SOLVER, 3), (26, 0), (-1, 0)):
+        with pytest.raises(EngineError) as ei:
+            g.apply(kind, [a, b], fn=fn)
+        assert ei.value.code == _ffi.GH_ENOFUNC, (kind, fn, str(ei.value))
+    y = g.apply(G.K_ELEMBIN, [a, b], fn=_ffi.BIN_FN["mod"])
+    G.Read(y)
+    m = G.NewTapeMachine(g, compile_only=True)
+    assert "elembin.mod" in m.program()
+    m.Close()
+
+
+def test_conv1d_is_conv2d_with_unit_height():
+    g = G.NewGraph()
+    x = G.NewTensor(g, np.zeros((2, 3, 1, 40), np.float32))
+    w = G.NewTensor(g, np.zeros((5, 3, 1, 3), np.float32))
+    assert G.Conv1d(x, w, 3, 1, 1, 1).Shape() == (2, 5, 1, 40)
+    assert G.Conv1d(x, w, 3, 0, 2, 1).Shape() == (2, 5, 1, 19)
+    assert G.Conv1d(x, w, 3, 2, 1, 2).Shape() == (2, 5, 1, 40)
+    m = G.NewTapeMachine(g, compile_only=True)
+    assert "conv2d" in m.program()
+    m.Close()
