@@ -43,17 +43,28 @@ def replay_mode():
     return False if EAGER_TIMING else "measured"
 
 
+SUSTAIN_MS = 40.0   # a kernel is timed after this much back-to-back work of its own, over this much more
+
+
 def time_cmds(ctx, cmds, iters, warm=3):
-    """Average milliseconds per pass over `cmds`: `iters` passes are captured
-    into one hipGraph (so host enqueue time is out of the picture) and the
-    replay is bracketed by HIP events on the engine's stream."""
+    """Average milliseconds per pass over `cmds`: `iters` passes are captured into one hipGraph
+    (so host enqueue time is out of the picture) and replays are bracketed by HIP events on the
+    engine's stream.
+
+    The GPU raises its clocks only under load that lasts: the same kernel measured over a 5 ms
+    burst after idle time runs 15-20 % slower than in a loop that has been busy for tens of
+    milliseconds (64 x 512^3 products: 178 us against 151 us).  A production loop is the second
+    case, so the graph is first replayed for SUSTAIN_MS, then timed over at least SUSTAIN_MS.
+    The first replay after the capture - the short-burst figure - is kept in
+    time_cmds.last_burst_ms."""
     ctx.submit(list(cmds) * warm)
     ctx.sync()
     if EAGER_TIMING:
         ctx.event(0)
         ctx.submit(list(cmds) * iters)
         ctx.event(1)
-        return ctx.elapsed_ms(0, 1) / iters
+        time_cmds.last_burst_ms = ctx.elapsed_ms(0, 1) / iters
+        return time_cmds.last_burst_ms
     ctx.graph_begin()
     ctx.submit(list(cmds) * iters)
     gid = ctx.graph_end()
@@ -62,9 +73,21 @@ def time_cmds(ctx, cmds, iters, warm=3):
     ctx.event(0)
     ctx.graph_launch(gid)
     ctx.event(1)
-    ms = ctx.elapsed_ms(0, 1) / iters
+    one = ctx.elapsed_ms(0, 1)
+    time_cmds.last_burst_ms = one / iters
+    reps = max(1, min(4000, int(SUSTAIN_MS / max(one, 1e-3)) + 1))
+    for _ in range(reps):
+        ctx.graph_launch(gid)
+    ctx.event(0)
+    for _ in range(reps):
+        ctx.graph_launch(gid)
+    ctx.event(1)
+    ms = ctx.elapsed_ms(0, 1) / (iters * reps)
     ctx.graph_destroy(gid)
     return ms
+
+
+time_cmds.last_burst_ms = None
 
 
 ELEMENTWISE_SETS = 8   # operand sets a timed kernel rotates over: 8 x (2..3) x 64 MiB >= 1 GiB, four times the last-level cache
@@ -162,7 +185,8 @@ def bench_linalg(ctx, iters):
         ms = time_cmds(ctx, [cmd], max(5, iters // 2))
         fl = 2.0 * m * n * k * batch
         res[name] = {"us": round(ms * 1e3, 1), "TFLOPs": round(fl / ms / 1e9, 2),
-                     "frac_mfma": round(fl / ms / 1e9 / MFMA_F32_PEAK_TFLOPS, 4), "flop": fl}
+                     "frac_mfma": round(fl / ms / 1e9 / MFMA_F32_PEAK_TFLOPS, 4), "flop": fl,
+                     "us_short_burst": round(time_cmds.last_burst_ms * 1e3, 1)}
         for q in (A, B, Cm):
             ctx.free(q)
     # float64 product (Dgemm path), against the fp64 matrix peak of 78.6 TFLOP/s
@@ -183,7 +207,12 @@ def bench_linalg(ctx, iters):
     nb = 4 * (m * n + m + n)
     res["gemv_8192"] = {"us": round(ms * 1e3, 1), "GBps": round(nb / ms / 1e6, 1),
                         "frac_hbm": round(nb / ms / 1e6 / HBM_PEAK_GBPS, 4), "bytes": nb}
-    for q in (A, xv, yv):
+    # the transposed product (x^T A): the same bytes, columns summed over rows
+    xt, yt = ctx.upload(synth.normal(5, (m,))), ctx.malloc(4 * n)
+    ms = time_cmds(ctx, [D.cmd_gemv(A, xt, yt, m, n, trans=True)], iters)
+    res["gemv_t_8192"] = {"us": round(ms * 1e3, 1), "GBps": round(nb / ms / 1e6, 1),
+                          "frac_hbm": round(nb / ms / 1e6 / HBM_PEAK_GBPS, 4), "bytes": nb}
+    for q in (A, xv, yv, xt, yt):
         ctx.free(q)
     return res
 
@@ -219,7 +248,8 @@ def bench_convnet_kernels(ctx, batch, iters):
         out_hw = (hw // 2) if pool else hw
         nb = 4 * (batch * cin * hw * hw + f * cin * 9 + batch * f * out_hw * out_hw)
         out[name] = {"us": round(ms * 1e3, 2), "TFLOPs": round(fl / ms / 1e9, 2), "flop": fl,
-                     "GBps": round(nb / ms / 1e6, 1), "bytes": nb, "pool_fused": pool}
+                     "GBps": round(nb / ms / 1e6, 1), "bytes": nb, "pool_fused": pool,
+                     "us_short_burst": round(time_cmds.last_burst_ms * 1e3, 2)}
         for q in (x, w, y):
             ctx.free(q)
     return out

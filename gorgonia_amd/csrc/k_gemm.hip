@@ -18,6 +18,7 @@
 // K = C*kh*kw: the "B" operand is gathered straight from the NCHW input (no
 // im2col buffer) and the result is written straight into NCHW (no transpose
 // pass), so lanes run along output pixels for coalesced loads and stores.
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -327,15 +328,26 @@ __device__ __forceinline__ void split_range(int nk, int splits, int s, int* kt0,
 // every XCD one contiguous range of tiles; inside a range, tiles are walked in
 // groups of 8 tile-rows so that co-resident workgroups share A rows and B
 // columns (a plain row-major walk re-read A and B ~6x from HBM at 4096^3).
-// (For a batch of products the same regrouping over the whole launch, so that
-// an XCD works through whole matrices, was measured: no gain on 64 x 512^3, and
-// the extra branch cost the register-tight 128x128 kernel 9 % at 4096^3.)
-__device__ __forceinline__ void tile_coords(int* tm, int* tn) {
+// For a batch of products (`batched`: blockIdx.z counts matrices) the regrouping
+// runs over the whole launch instead, so that an XCD works through whole
+// matrices and each operand tile enters one L2 only; *bz is the matrix.
+__device__ __forceinline__ void tile_coords(int* tm, int* tn, int* bz, bool batched) {
   const int gx = gridDim.x, gy = gridDim.y;  // tiles along N, along M
   const int total = gx * gy;
   int id = blockIdx.y * gx + blockIdx.x;
   constexpr int kXcd = 8, kGroup = 8;
-  if (total % kXcd == 0) id = (id % kXcd) * (total / kXcd) + id / kXcd;
+  *bz = blockIdx.z;
+  if (batched) {
+    const int all = total * (int)gridDim.z;
+    if (all % kXcd == 0) {
+      const int lin = (int)blockIdx.z * total + id;
+      const int nid = (lin % kXcd) * (all / kXcd) + lin / kXcd;
+      *bz = nid / total;
+      id = nid - *bz * total;
+    }
+  } else if (total % kXcd == 0) {
+    id = (id % kXcd) * (total / kXcd) + id / kXcd;
+  }
   const int per_group = kGroup * gx;
   const int first_m = (id / per_group) * kGroup;
   const int gsz = min(gy - first_m, kGroup);
@@ -346,7 +358,7 @@ __device__ __forceinline__ void tile_coords(int* tm, int* tn) {
 
 // blockIdx.z is the batch index (splits == 1) or the split-K slice (batch == 1).
 template <int BM, int BN, int BK, int WAVES_M, bool TA, bool TB, bool VEC, bool BIAS = false>
-__global__ __launch_bounds__(kThreads) void k_sgemm(const float* __restrict__ A,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(BM == 128 && BN == 128 ? 4 : 1))) void k_sgemm(const float* __restrict__ A,
                                                     const float* __restrict__ B,
                                                     float* __restrict__ C, int M, int N, int K,
                                                     int lda, int ldb, int ldc, int64_t sA,
@@ -355,10 +367,10 @@ __global__ __launch_bounds__(kThreads) void k_sgemm(const float* __restrict__ A,
                                                     const float* __restrict__ bias) {
   using LA = typename std::conditional<TA, LoadMnContig<BM, BK, VEC>, LoadKContig<BM, BK, VEC>>::type;
   using LB = typename std::conditional<TB, LoadKContig<BN, BK, VEC>, LoadMnContig<BN, BK, VEC>>::type;
-  const int bz = blockIdx.z;
   const int nk = (K + BK - 1) / BK;
-  int tile_m, tile_n;
-  tile_coords(&tile_m, &tile_n);
+  int tile_m, tile_n, bz;
+  tile_coords(&tile_m, &tile_n, &bz, splits <= 1 && gridDim.z > 1);
+
   // one LDS allocation shared by both call sites below (a static array inside
   // the tile loop would be instantiated once per call site)
   __shared__ float lds[2 * BK * (LA::S + LB::S)];
@@ -669,7 +681,21 @@ __global__ __launch_bounds__(WV * 64) void k_gemm_skinny16(const float* __restri
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 15, q = lane >> 4;
   const bool ragged_n = N < BN;
-  const int m0 = min((int)blockIdx.y * 16, M - 16), n0 = ragged_n ? 0 : min((int)blockIdx.x * BN, N - BN);
+  // Workgroup ids are dealt round-robin over the 8 XCDs, each with its own L2.
+  // Regroup them so that one XCD gets a contiguous run of ids, and walk a run
+  // row-tile fastest: every row tile of a column tile then reads that strip of
+  // B (the weights, the big operand of a dense layer) through the same L2, once
+  // from memory, instead of once per XCD.
+  int tile_x, tile_y;
+  {
+    const int gx = gridDim.x, gy = gridDim.y, total = gx * gy;
+    const int id = blockIdx.y * gx + blockIdx.x;
+    const int xcd = id & 7, per = total >> 3, extra = total & 7;
+    const int nid = xcd * per + min(xcd, extra) + (id >> 3);
+    tile_x = nid / gy;
+    tile_y = nid - tile_x * gy;
+  }
+  const int m0 = min(tile_y * 16, M - 16), n0 = ragged_n ? 0 : min(tile_x * BN, N - BN);
   const int nchunks = (K + 15) / 16;
   int ncol[NT];   // this lane's columns (clamped when the tile is wider than the matrix)
 #pragma unroll
@@ -1496,12 +1522,12 @@ __global__ __launch_bounds__(kThreads) void k_dgemm(const double* __restrict__ A
   using LB = typename std::conditional<TB, LoadKContig64<BN, BK, VEC>, LoadMnContig64<BN, BK, VEC>>::type;
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
   __shared__ double lds[2 * (LA::SIZE + LB::SIZE)];
-  int tile_m, tile_n;
-  tile_coords(&tile_m, &tile_n);
+  int tile_m, tile_n, bz;
+  tile_coords(&tile_m, &tile_n, &bz, gridDim.z > 1);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  LA la; la.base = A + blockIdx.z * sA; la.ld = lda; la.rmax = M; la.kmax = K;
-  LB lb; lb.base = B + blockIdx.z * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
-  C += blockIdx.z * sC;
+  LA la; la.base = A + bz * sA; la.ld = lda; la.rmax = M; la.kmax = K;
+  LB lb; lb.base = B + bz * sB; lb.ld = ldb; lb.rmax = N; lb.kmax = K;
+  C += bz * sC;
   f64x4 acc[TM][TN];
   dmfma_tile_loop_auto<BM, BN, BK, LA, LB>(lds, la, lb, m0, n0, (K + BK - 1) / BK, acc);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -1657,8 +1683,8 @@ __global__ __launch_bounds__(kThreads) void k_conv2d_f64_mfma(const double* __re
   using LB = LoadIm2col64<BN, BK>;
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
   __shared__ double lds[2 * (LA::SIZE + LB::SIZE)];
-  int tile_m, tile_n;
-  tile_coords(&tile_m, &tile_n);
+  int tile_m, tile_n, bz_unused;
+  tile_coords(&tile_m, &tile_n, &bz_unused, false);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   LA la; la.base = w; la.ld = g.K; la.rmax = g.F; la.kmax = g.K;
   LB lb; lb.init(x, &g, n0);
@@ -2099,16 +2125,82 @@ __global__ __launch_bounds__(256) void k_gemv_n(const float* __restrict__ A,
   if (lane == 0) y[row] = acc;
 }
 
-// y(n) = A(m x n)^T x: each thread owns one column, walks rows; consecutive
-// lanes read consecutive addresses.
-__global__ __launch_bounds__(256) void k_gemv_t(const float* __restrict__ A,
-                                                const float* __restrict__ x, float* __restrict__ y,
-                                                int m, int n, int lda) {
-  const int col = blockIdx.x * 256 + threadIdx.x;
-  if (col >= n) return;
+// y(n) = A(m x n)^T x.  A workgroup takes 256*V*J adjacent columns and a range
+// of rows and walks the rows in order, RU rows in flight; a thread owns J groups
+// of V adjacent columns 256*V apart, so one load instruction of the workgroup
+// reads 1024*V contiguous bytes of a row and J of them a contiguous run.  No
+// thread shares a sum with another.  With more than one row range the partial
+// rows go to `out` = [chunks][n] scratch and k_gemv_t_sum adds them in a fixed
+// order, so the result does not depend on timing.  (Measured at 8192 x 8192: V=4,
+// J=2, RU=8 with half as many workgroups as compute units streams at 6.7 TB/s;
+// more, smaller workgroups scatter the row streams and lose a quarter of that.)
+template <int V, int J, int RU>
+__global__ __launch_bounds__(256) void k_gemv_t(const float* __restrict__ A, const float* __restrict__ x,
+                                                float* __restrict__ out, int m, int n, int lda,
+                                                int rows_per_chunk) {
+  typedef float vec __attribute__((ext_vector_type(V), aligned(4 * V)));
+  constexpr int GS = 256 * V;  // columns between a thread's groups
+  const int cb = blockIdx.x * GS * J + threadIdx.x * V;
+  const int r0 = blockIdx.y * rows_per_chunk, r1 = min(m, r0 + rows_per_chunk);
+  // a group past the last column reads its neighbour to the left instead (same
+  // rows, valid memory) and is not stored
+  int col[J];
+#pragma unroll
+  for (int j = 0; j < J; j++) col[j] = min(cb + j * GS, n - V);
+  if (col[0] < 0) return;  // n < V cannot happen for V = 1; for V = 4 the caller guarantees n >= 4
+  const float* a = A + (int64_t)r0 * lda;
+  vec acc[J];
+#pragma unroll
+  for (int j = 0; j < J; j++) acc[j] = vec{};
+  int r = r0;
+  for (; r + RU <= r1; r += RU) {
+    vec v[RU][J];
+    float xv[RU];
+#pragma unroll
+    for (int i = 0; i < RU; i++)
+#pragma unroll
+      for (int j = 0; j < J; j++) v[i][j] = *reinterpret_cast<const vec*>(a + (int64_t)i * lda + col[j]);
+#pragma unroll
+    for (int i = 0; i < RU; i++) xv[i] = x[r + i];
+#pragma unroll
+    for (int i = 0; i < RU; i++)
+#pragma unroll
+      for (int j = 0; j < J; j++) acc[j] += v[i][j] * xv[i];
+    a += (int64_t)RU * lda;
+  }
+  for (; r < r1; r++, a += lda) {
+    const float xr = x[r];
+#pragma unroll
+    for (int j = 0; j < J; j++) acc[j] += *reinterpret_cast<const vec*>(a + col[j]) * xr;
+  }
+#pragma unroll
+  for (int j = 0; j < J; j++)
+    if (cb + j * GS < n) *reinterpret_cast<vec*>(out + (int64_t)blockIdx.y * n + cb + j * GS) = acc[j];
+}
+
+// y[c] = sum over chunks of part[k][c].  Four threads share a column: thread q
+// adds chunks q, q+4, q+8, ... in that order (eight loads in flight), then the
+// four sums are added as (s0 + s1) + (s2 + s3).
+__global__ __launch_bounds__(256) void k_gemv_t_sum(const float* __restrict__ part, float* __restrict__ y,
+                                                    int chunks, int n) {
+  __shared__ float sh[4][64];
+  const int cg = threadIdx.x & 63, q = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + cg;
   float acc = 0.f;
-  for (int r = 0; r < m; r++) acc += A[(int64_t)r * lda + col] * x[r];
-  y[col] = acc;
+  if (c < n) {
+    int k = q;
+    for (; k + 28 < chunks; k += 32) {
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] = part[(int64_t)(k + 4 * i) * n + c];
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc += v[i];
+    }
+    for (; k < chunks; k += 4) acc += part[(int64_t)k * n + c];
+  }
+  sh[q][cg] = acc;
+  __syncthreads();
+  if (q == 0 && c < n) y[c] = (sh[0][cg] + sh[1][cg]) + (sh[2][cg] + sh[3][cg]);
 }
 
 __global__ __launch_bounds__(256) void k_outer(const float* __restrict__ x,
@@ -2157,7 +2249,7 @@ inline bool al16(uint64_t p) { return (p & 15u) == 0; }
 // leave CUs idle) and 32x256 (all four wavefronts along N: few filters, many
 // pixels).  When even the small shape yields too few blocks, K is split across
 // grid.z and a second kernel sums the slabs.
-enum { kTile128 = 0, kTile64 = 1, kTile32x256 = 2 };
+enum { kTile128 = 0, kTile64 = 1, kTile32x256 = 2, kTile128x64 = 3 };
 struct TilePlan { int tile; int splits; };
 
 inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -2182,7 +2274,7 @@ TilePlan plan_tiles(gh_ctx* ctx, int64_t M, int64_t N, int64_t K, int64_t batch,
   TilePlan p{kTile128, 1};
   if (const char* env = getenv("GORGONIA_HIP_GEMM_PLAN")) {  // tuning override: "tile,splits"
     int t = 0, sp = 1;
-    if (sscanf(env, "%d,%d", &t, &sp) == 2 && t >= 0 && t <= 2 && sp >= 1) {
+    if (sscanf(env, "%d,%d", &t, &sp) == 2 && t >= 0 && t <= 3 && sp >= 1) {
       p.tile = (t == kTile32x256 && !allow_32x256) ? kTile64 : t;
       p.splits = clamp_splits(ctx, sp, M, N, K, batch);
       return p;
@@ -2732,6 +2824,7 @@ int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
   const TilePlan p = plan_tiles(ctx, c.dim[0], c.dim[1], c.dim[2], batch, false);
   if (ctx->err) return ctx->err;
   if (p.tile == kTile128) return launch_sgemm_cfg<128, 128, 2>(ctx, c, p.splits);
+  if (p.tile == kTile128x64) return launch_sgemm_cfg<128, 64, 2>(ctx, c, p.splits);
   return launch_sgemm_cfg<64, 64, 2>(ctx, c, p.splits);
 }
 
@@ -2945,7 +3038,24 @@ int gh_launch_gemv(gh_ctx* ctx, const gh_cmd& c) {
   const float* x = (const float*)(uintptr_t)c.ptr[1];
   float* y = (float*)(uintptr_t)c.ptr[2];
   if (c.flags & GH_FLAG_TRANS_A) {
-    hipLaunchKernelGGL(k_gemv_t, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, A, x, y, m, n, lda);
+    // (column block, row range) pairs: about half as many workgroups as compute
+    // units, each with at least 64 rows to stream
+    const bool vec = al16(c.ptr[0]) && al16(c.ptr[2]) && lda % 4 == 0 && n % 4 == 0 && n >= 4;
+    const int cols = vec ? 2048 : 512;
+    const int cblocks = (n + cols - 1) / cols;
+    int chunks = (int)std::min<int64_t>(std::max<int64_t>(1, (int64_t)ctx->cu_count / 2 / cblocks), (m + 63) / 64);
+    if (chunks > 1 && (int64_t)chunks * n * 4 > ctx->workspace_bytes) {
+      if (gh_ws_short(ctx, (int64_t)chunks * n * 4)) return ctx->err;
+      chunks = 1;
+    }
+    const int rows = ((m + chunks - 1) / chunks + 7) / 8 * 8;
+    chunks = (m + rows - 1) / rows;
+    float* out = chunks > 1 ? (float*)ctx->workspace : y;
+    const dim3 grid(cblocks, chunks);
+    if (vec) hipLaunchKernelGGL((k_gemv_t<4, 2, 8>), grid, dim3(256), 0, ctx->stream, A, x, out, m, n, lda, rows);
+    else hipLaunchKernelGGL((k_gemv_t<1, 2, 8>), grid, dim3(256), 0, ctx->stream, A, x, out, m, n, lda, rows);
+    if (chunks > 1)
+      hipLaunchKernelGGL(k_gemv_t_sum, dim3((n + 63) / 64), dim3(256), 0, ctx->stream, out, y, chunks, n);
   } else {
     const int vec = al16(c.ptr[0]) && al16(c.ptr[1]) && lda % 4 == 0;
     hipLaunchKernelGGL(k_gemv_n, dim3((m + 3) / 4), dim3(256), 0, ctx->stream, A, x, y, m, n, lda, vec);

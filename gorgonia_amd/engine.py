@@ -85,6 +85,7 @@ HOST_SYMBOLS = {
     "ghh_graph_node_dtype": (C.c_int, [_P, C.c_int]),
     "ghh_graph_fuse_activations": (C.c_int, [_P]),
     "ghh_tape_new": (_P, [_P, C.c_int, C.c_int]),
+    "ghh_lisp_new": (_P, [_P, C.c_int]),
     "ghh_tape_new_with_engine": (_P, [_P, _P, C.c_int, C.c_int]),
     "ghh_tape_destroy": (None, [_P]),
     "ghh_tape_last_error": (C.c_char_p, [_P]),

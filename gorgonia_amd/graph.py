@@ -297,7 +297,7 @@ class TapeMachine:
     """NewTapeMachine(g, ...) / RunAll / Reset / Close (vm_tape.go:45-249)."""
 
     def __init__(self, g, graph_replay=False, reupload_resident=False, fuse_activations=False,
-                 device=0, compile_only=False, engine=None):
+                 device=0, compile_only=False, engine=None, node_at_a_time=False):
         self.g = g
         self.lib = g.lib
         self.fused = self.lib.ghh_graph_fuse_activations(g.h) if fuse_activations else 0
@@ -305,7 +305,9 @@ class TapeMachine:
         # graph_replay: False, True (capture on the second run, replay from then on) or
         # "measured" (time plain submits against replays first, keep the quicker)
         mode = 2 if graph_replay == "measured" else int(bool(graph_replay))
-        if engine is not None:
+        if node_at_a_time:
+            self.h = self.lib.ghh_lisp_new(g.h, int(reupload_resident))
+        elif engine is not None:
             self.h = self.lib.ghh_tape_new_with_engine(g.h, engine.h, mode, int(reupload_resident))
         else:
             self.h = self.lib.ghh_tape_new(g.h, mode, int(reupload_resident))
@@ -363,6 +365,12 @@ class TapeMachine:
         buf = C.create_string_buffer(n + 1)
         self.lib.ghh_tape_program_string(self.h, buf, n + 1)
         return buf.value.decode()
+
+
+def NewLispMachine(g, **kw):
+    """NewLispMachine(g) (vm_genera.go:43-120), forward execution: every node is run and waited for
+    on its own.  The reference's tests run one graph on both machines and compare."""
+    return TapeMachine(g, node_at_a_time=True, **kw)
 
 
 def WithEngine(e):

@@ -223,6 +223,17 @@ ghh_tape* ghh_tape_new(ghh_graph* g, int graph_replay, int reupload_resident) {
   t->eng.owned = false;
   return t;
 }
+ghh_tape* ghh_lisp_new(ghh_graph* g, int reupload_resident) {
+  if (!g) return nullptr;
+  TapeOptions o;
+  o.node_at_a_time = true;
+  o.reupload_resident = reupload_resident != 0;
+  ghh_tape* t = new ghh_tape();
+  t->t = new TapeMachine(&g->g, o);
+  t->eng.e = &t->t->Eng();
+  t->eng.owned = false;
+  return t;
+}
 ghh_tape* ghh_tape_new_with_engine(ghh_graph* g, ghh_engine* e, int graph_replay, int reupload_resident) {
   if (!g || !e || !e->e) return nullptr;
   TapeOptions o;

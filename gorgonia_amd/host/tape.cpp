@@ -737,7 +737,7 @@ Status TapeMachine::Compile() {
     Node& n = nodes[(size_t)i];
     if (n.fused_away) continue;
     if (n.alias_of >= 0) { node_reg_[(size_t)i] = node_reg_[(size_t)root[(size_t)i]]; continue; }
-    const int ow = n.is_input ? -1 : OverwritesInput(n.op);
+    const int ow = n.is_input || opt_.node_at_a_time ? -1 : OverwritesInput(n.op);
     if (ow >= 0 && ow < (int)n.inputs.size()) {
       int src = n.inputs[(size_t)ow];
       if (n.op.kind == OpKind::ElemBin && n.inputs.size() == 2 && nodes[(size_t)src].shape.IsScalar())
@@ -1039,6 +1039,10 @@ Status TapeMachine::RunAll() {
         }
         st = CUDADo(eng_, n.op, out, inp);
         if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": " + op_name(n.op));
+        if (opt_.node_at_a_time) {
+          st = flush();  // DoWork after every node (vm_genera.go:144)
+          if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": " + op_name(n.op) + ": DoWork failed");
+        }
         break;
       }
       case InstrKind::Free:

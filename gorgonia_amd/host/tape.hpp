@@ -141,6 +141,12 @@ struct TapeOptions {
   // so it only pays for segments of many short kernels.
   bool replay_measured = false;
   bool reupload_resident = false; // treat resident inputs like the reference does (H2D every run)
+  // The lispMachine's way of running a graph (vm_genera.go:121-200,296-430): every
+  // node is executed and waited for when it is reached - one submit and one wait
+  // per operator, no segment batching, no replay - and no operator writes over
+  // an input's register.  Same operators, same kernels: the values are those of
+  // the batched machine, which is what running one graph on both machines checks.
+  bool node_at_a_time = false;
 };
 
 class TapeMachine {

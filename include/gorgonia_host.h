@@ -130,6 +130,11 @@ GH_API int ghh_graph_fuse_activations(ghh_graph* g);
  * (ghh_tape_segment_verdict tells which).  reupload_resident: resident inputs
  * are uploaded on every run like all others (vm_tape_cuda.go:220-243). */
 GH_API ghh_tape* ghh_tape_new(ghh_graph* g, int graph_replay, int reupload_resident);
+/* NewLispMachine(g) (vm_genera.go:43-120), forward execution only: the same handle type and calls
+ * as a tape machine, but every node is submitted and waited for on its own when it is reached
+ * (vm_genera.go:144) and no operator overwrites an input.  It exists for what the reference uses
+ * its second machine for in tests: run one graph on both, require equal values. */
+GH_API ghh_tape* ghh_lisp_new(ghh_graph* g, int reupload_resident);
 /* NewTapeMachine(g, WithEngine(e)) (vm.go:318-329): the machine runs on the
  * caller's engine, which must be initialised (ghh_engine_init) before
  * ghh_tape_init and must outlive the machine.  Registers come out of that

@@ -134,3 +134,60 @@ def test_yolo_shaped_batch_8_at_416(ctx):
     one["x"] = inp["x"][3:4].copy()
     alone = _tape(configs.build_yolo, one, fuse_activations=True)
     assert rel_frobenius(alone["out"][0], res["out"][3]) <= TOL
+
+
+def _yolo_with_taps(inp, taps, fuse):
+    """The yolo-shaped stack with host reads on chosen layers: unfused, the convolution's own
+    output, the BatchNorm+LeakyRelu output and the pooled output of each tapped layer; fused,
+    only the pooled output (the one value the folded kernel stores)."""
+    g = G.NewGraph()
+    h = G.NewTensor(g, inp["x"], False)
+    reads = {}
+    for i in range(7):
+        w = G.NewTensor(g, inp[f"w{i}"], True)
+        h = G.Conv2d(h, w, (3, 3), (1, 1), (1, 1), (1, 1))
+        if i in taps and not fuse:
+            reads[f"conv{i}"] = G.Read(h)
+        m, v, ga, be = (G.NewTensor(g, inp[f"{k}{i}"], True) for k in ("mean", "var", "gamma", "beta"))
+        h = G.LeakyRelu(G.BatchNorm(h, ga, be, m, v, 1e-5), 0.1)
+        if i in taps and not fuse:
+            reads[f"act{i}"] = G.Read(h)
+        if i < 5:
+            h = G.MaxPool2D(h, (2, 2), (0, 0), (2, 2))
+        elif i == 5:
+            h = G.MaxPool2D(h, (2, 2), (1, 0, 1, 0), (1, 1))
+        if i in taps:
+            reads[f"pool{i}"] = G.Read(h)
+    reads["out"] = G.Read(G.Conv2d(h, G.NewTensor(g, inp["w7"], True), (1, 1), (0, 0), (1, 1), (1, 1)))
+    m = G.NewTapeMachine(g, fuse_activations=fuse)
+    m.RunAll()
+    res = {k: v.copy() for k, v in reads.items()}
+    m.Close()
+    return res
+
+
+def test_yolo_shaped_intermediates_bit_for_bit(ctx):
+    """Full size (8 x 3 x 416 x 416).  Everything after a convolution is exact arithmetic with one
+    rounding per step, so it is held to bits, not to a norm: the oracle's BatchNorm + LeakyRelu
+    applied to the convolution output the DEVICE produced must give the device's activation, the
+    oracle's MaxPool2D of that the device's pooled value, and the folded kernel
+    (conv+BN+LeakyRelu+pool in one launch) must store exactly the unfused chain's pooled bits.
+    Layers 1 (16->32 at 208x208), 3 (64->128 at 52x52) and 5 (256->512 at 13x13, stride-1 pool)
+    go through three different convolution kernels."""
+    inp = configs.yolo_inputs(8, 416)
+    taps = (1, 3, 5)
+    plain = _yolo_with_taps(inp, taps, fuse=False)
+    fused = _yolo_with_taps(inp, taps, fuse=True)
+    for i in taps:
+        conv = plain[f"conv{i}"]
+        want_act = O.leaky_relu(O.bn_infer(conv, inp[f"mean{i}"], inp[f"var{i}"], 1e-5, inp[f"gamma{i}"],
+                                           inp[f"beta{i}"]), 0.1).reshape(conv.shape)
+        assert_bits_equal(plain[f"act{i}"], want_act, f"layer {i}: BatchNorm+LeakyRelu of the device's conv output")
+        if i < 5:
+            want_pool = O.maxpool2d(plain[f"act{i}"], (2, 2), (0, 0), (2, 2))
+        else:
+            want_pool = O.maxpool2d(plain[f"act{i}"], (2, 2), (1, 0, 1, 0), (1, 1))
+        assert_bits_equal(plain[f"pool{i}"], want_pool, f"layer {i}: MaxPool2D of the device's activation")
+        assert_bits_equal(fused[f"pool{i}"], plain[f"pool{i}"], f"layer {i}: folded kernel == unfused chain")
+    assert_bits_equal(fused["out"], plain["out"], "folded forward == unfused forward")
+    assert rel_frobenius(plain["out"], F.yolo(inp)) <= TOL

@@ -209,7 +209,8 @@ def test_batched_matmul_reference_example(ctx):
         ctx.free(p)
 
 
-@pytest.mark.parametrize("m,n", [(1, 1), (5, 3), (64, 64), (300, 784), (1000, 1001), (2048, 4096)])
+@pytest.mark.parametrize("m,n", [(1, 1), (5, 3), (64, 64), (300, 784), (1000, 1001), (2048, 4096), (4099, 260),
+                                 (33, 8192), (7, 1028)])
 @pytest.mark.parametrize("trans", [False, True])
 def test_matvec(ctx, m, n, trans):
     A = synth.normal(7, (m, n))
@@ -221,6 +222,17 @@ def test_matvec(ctx, m, n, trans):
     ref = (A.T if trans else A).astype(np.float64) @ x.astype(np.float64)
     assert rel_frobenius(got, ref) <= TOL
     assert rel_frobenius(O.gemv(A, x, trans), ref) <= TOL
+    # integer data: exact in any order of summation; a second launch repeats the bits
+    rng = np.random.default_rng(3)
+    Ai = rng.integers(-3, 4, (m, n)).astype(np.float32)
+    xi = rng.integers(-3, 4, x.shape).astype(np.float32)
+    ctx.h2d(dA, Ai); ctx.h2d(dx, xi)
+    ctx.run(D.cmd_gemv(dA, dx, dy, m, n, trans=trans))
+    gi = ctx.d2h(dy, got.shape)
+    assert np.array_equal(gi, ((Ai.T if trans else Ai).astype(np.int64) @ xi.astype(np.int64)).astype(np.float32))
+    ctx.h2d(dA, A); ctx.h2d(dx, x)
+    ctx.run(D.cmd_gemv(dA, dx, dy, m, n, trans=trans))
+    assert_bits_equal(ctx.d2h(dy, got.shape), got, "second launch")
     for p in (dA, dx, dy):
         ctx.free(p)
 

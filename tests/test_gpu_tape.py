@@ -274,3 +274,36 @@ def test_measured_replay_keeps_results_and_settles(ctx):
         total, launch, wait = m.phase_ns()
         assert total >= launch + wait > 0
         m.Close()
+
+
+def test_lisp_machine_differential(ctx):
+    """The reference's main test pattern (nn_test.go:25-79, operatorPointwise_unary_test.go:14-95):
+    one graph on the TapeMachine and on the LispMachine, equal values required.  Here the second
+    machine runs node by node - a submit and a wait per operator, fresh memory for every value -
+    and the first batches, overwrites dead inputs, folds followers into epilogues and replays."""
+    cases = [
+        (configs.build_elementwise, configs.elementwise_inputs(64)),
+        (configs.build_mlp, configs.mlp_inputs(32)),
+        (configs.build_convnet, configs.convnet_inputs(8)),
+        (configs.build_yolo, configs.yolo_inputs(1, 64)),
+    ]
+    for build, inp in cases:
+        g, outs = build(inp)
+        lisp = G.NewLispMachine(g)
+        lisp.RunAll()
+        want = {k: v.copy() for k, v in outs.items()}
+        n_ops = lisp.program().count("execOp")
+        assert lisp.segments() == n_ops + 1, "one DoWork per node, and the one in front of the reads"
+        assert "[unsafe]" not in lisp.program()
+        lisp.RunAll()
+        for k in outs:
+            assert_bits_equal(outs[k], want[k], f"{build.__name__}.{k}: lisp machine, second run")
+        lisp.Close()
+        for kw in (dict(), dict(fuse_activations=True), dict(fuse_activations=True, graph_replay=True)):
+            g2, outs2 = build(inp)
+            m = G.NewTapeMachine(g2, **kw)
+            for _ in range(3):
+                m.RunAll()
+            for k in outs2:
+                assert_bits_equal(outs2[k], want[k], f"{build.__name__}.{k}: tape {kw} == lisp")
+            m.Close()
