@@ -78,6 +78,10 @@ bool gh_conv_small_can_pool(const gh_cmd& c);
 int gh_try_launch_conv_patch(gh_ctx* ctx, const gh_cmd& c);
 bool gh_conv_patch_takes(const gh_cmd& c);
 bool gh_conv_patch_can_pool(const gh_cmd& c);
+// k_conv_wide.hip: 3x3 stride-1 convolution over large images with up to 64 channels
+int gh_try_launch_conv_wide(gh_ctx* ctx, const gh_cmd& c);
+bool gh_conv_wide_takes(const gh_cmd& c);
+bool gh_conv_wide_can_pool(const gh_cmd& c);
 int gh_launch_maxpool2d(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_bn_infer(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_softmax(gh_ctx* ctx, const gh_cmd& c);

@@ -1,0 +1,471 @@
+// Conv2d 3x3 / stride 1 over large images with few input channels (up to 64), float32,
+// on the 16x16x4 MFMA: one workgroup = 16 TM filters x one TH x TW patch of one image,
+// the patch's pixels split over its eight wavefronts, each of which runs the whole K.
+//
+// Replaces cuDNN ConvolutionForward (ops/nn/convolution_cuda.go:111-117) for the first
+// layers of an image network: many output pixels, a short contraction.  With K = C * 9 of
+// a few hundred at most, the whole filter tile and every channel of the padded patch fit
+// in LDS at once, so there is one staging phase, one barrier, and then nothing but
+// operand fetches and MFMAs; the results leave from the accumulators, no partial sums
+// cross wavefronts.  Same GEMM view as the other convolution kernels (M = filters, N =
+// output pixels, K in the reference's (c, kr, kc) order, op_nn.go:418-437), results
+// written straight into NCHW.
+//
+//   * One output is one accumulator chain over K, channel quad by channel quad, tap by
+//     tap, whatever the patch shape and whether or not the pooling below is fused: the
+//     stored bits depend on the operands only.
+//   * A channel count that is not a multiple of four is padded with zero planes and zero
+//     filter columns in LDS (a first layer's 3 channels or 1).
+//   * With GH_FLAG_CONV_POOL2 the patch has even extents and the N axis enumerates (pooled
+//     pixel, position in the 2x2 window), so a window is four adjacent lanes of one
+//     accumulator register: the maximum is taken across them in scan order with strict >
+//     (the pooling kernel's rule, op_nn.go:860-907) and one lane stores it.
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <mutex>
+
+#include "gh_conv_common.h"
+#include "gh_internal.h"
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+inline unsigned magic_of(unsigned d) { return d <= 1 ? 0u : (unsigned)((0x100000000ull + d - 1) / d); }
+// n / d with magic = magic_of(d), exact while n * d < 2^32; branch-free (magic 0 stands for d = 1)
+__device__ __forceinline__ int mdiv(int n, unsigned magic) {
+  const unsigned q = __umulhi((unsigned)n, magic);
+  return (int)(q | ((unsigned)n & (0u - (unsigned)(magic == 0))));
+}
+
+struct WideGeom {
+  int B, C, H, W, F, pad, oh, ow, HW, K;
+  int NQ, KP;                     // channel quads ceil(C / 4); padded contraction 36 NQ
+  int TH, TW, tiles_x, tiles_y;   // output patch, patches per image
+  int PW, PP, PL;                 // padded patch: row length TW + 2, size (TH + 2) * PW, plane pitch in LDS
+  int npix;                       // TH * TW
+  int pool, ph, pw, HTW;          // fused 2x2 / stride-2 max-pool: pooled extents of y, TW / 2
+  unsigned mTXY, mTX, mPP, mPW, mTW, mHTW;   // magics: tiles_x*tiles_y, tiles_x, PP, PW, TW, HTW
+};
+
+constexpr int kWaves = 8;
+constexpr int kThreads = kWaves * 64;
+
+// value of lane (l & ~3) + I, for every lane l: a 2x2 window's position I
+template <int I>
+__device__ __forceinline__ float quad_bcast(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), I * 0x55, 0xf, 0xf, true));
+}
+
+// XS: patch cells each thread stages per tile (4 NQ PP <= XS * kThreads); DB: two patch buffers.
+// The 12-slot kernels are held to 128 registers so that two workgroups share a compute unit
+// where their LDS allows: one's staging, epilogue and barriers then run under the other's MFMAs.
+template <int TM, int TN, int XS, bool DB>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 12 && TM * TN <= 4 ? 4 : 2))) void k_conv3x3_wide(const float* __restrict__ x, const float* __restrict__ w,
+                                                           float* __restrict__ y, WideGeom g, ConvTail tail) {
+  constexpr int BM = 16 * TM;
+  constexpr int NB = kWaves * 16 * TN;   // N entries of the workgroup
+  extern __shared__ float lds[];
+  const int plane_floats = 4 * g.NQ * g.PL + 8;    // one patch buffer; its last 8 floats take idle slots' writes
+  float* const As = lds;                           // [TM][KP][16]: filter tile, k-major, 16 filters a row
+  float* const P0 = lds + TM * g.KP * 16;          // [DB ? 2 : 1][4 NQ][PL]: padded patch, one plane per channel
+  int* const tab = reinterpret_cast<int*>(P0 + (DB ? 2 : 1) * plane_floats);   // [NB] cell of N entry n in the patch
+  float* const ftab = reinterpret_cast<float*>(tab + NB);                      // [4][BM] BatchNorm constants
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int li = lane & 15, lk = lane >> 4;
+  const int m0 = blockIdx.y * BM;
+  if (tid < BM) conv_tail_table(tail, ftab, BM, tid, min(m0 + tid, g.F - 1));
+
+  // ---- the filter tile, once: As[a][k][f] = w[m0 + 16 a + f][k], zero for k >= K
+  {
+    const int f = tid & (BM - 1), j0 = tid / BM;
+    const float* const wrow = w + (int64_t)min(m0 + f, g.F - 1) * g.K;
+    float* const ad = As + (f >> 4) * g.KP * 16 + (f & 15);
+    constexpr int JS = kThreads / BM;    // 128-bit columns in flight per pass
+    const int ncol = g.KP / 4;
+    if ((g.K & 3) == 0) {
+      for (int j = j0; j < ncol; j += 4 * JS) {
+        f32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const f32x4_a4*>(wrow + 4 * min(j + u * JS, ncol - 1));
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          const int jj = min(j + u * JS, ncol - 1);   // passes past the end rewrite the last column
+#pragma unroll
+          for (int e = 0; e < 4; e++) ad[(4 * jj + e) * 16] = v[u][e];
+        }
+      }
+    } else {
+      for (int k = j0; k < g.KP; k += JS) ad[k * 16] = k < g.K ? wrow[k] : 0.f;
+    }
+  }
+  // ---- per-thread patch cells, the same for every tile: source offset relative to the patch
+  // origin, row and column inside the padded patch, destination in the buffer.  Cells of padded
+  // channels are flagged and written as zero; slots past the last cell are flagged too and
+  // write the spare floats at the end of the buffer.
+  int xrel[XS], xpk[XS];   // xpk = zero-cell flag << 31 | row << 24 | column << 16 | destination
+  {
+    const int cells = 4 * g.NQ * g.PP;
+#pragma unroll
+    for (int u = 0; u < XS; u++) {
+      const int id = tid + u * kThreads;
+      const int idc = min(id, cells - 1);
+      const int pl = mdiv(idc, g.mPP), rem = idc - pl * g.PP;
+      const int r = mdiv(rem, g.mPW), cc = rem - r * g.PW;
+      const bool real = id < cells && pl < g.C;
+      xrel[u] = min(pl, g.C - 1) * g.HW + r * g.W + cc;
+      const int dst = id < cells ? pl * g.PL + rem : 4 * g.NQ * g.PL + (lane & 7);
+      xpk[u] = (real ? 0 : (int)0x80000000) | (r << 24) | (cc << 16) | dst;
+    }
+  }
+  // ---- table of patch cells of the N entries
+  for (int n = tid; n < NB; n += kThreads) {
+    const int nn = n < g.npix ? n : 0;   // idle column: any valid cell
+    int ty, tx;
+    if (g.pool) {
+      const int q = nn >> 2, wpos = nn & 3;
+      const int py = mdiv(q, g.mHTW), px = q - py * g.HTW;
+      ty = 2 * py + (wpos >> 1);
+      tx = 2 * px + (wpos & 1);
+    } else {
+      ty = mdiv(nn, g.mTW);
+      tx = nn - ty * g.TW;
+    }
+    tab[n] = ty * g.PW + tx;
+  }
+
+  float xv[XS];
+  // global loads of one tile's patch into registers (cells outside the image: zero, no load)
+  auto load_patch = [&](int tile) {
+    const int bimg = mdiv(tile, g.mTXY);
+    const int trem = tile - bimg * (g.tiles_x * g.tiles_y);
+    const int tyi = mdiv(trem, g.mTX), txi = trem - tyi * g.tiles_x;
+    const int py0 = tyi * g.TH - g.pad, px0 = txi * g.TW - g.pad;
+    const float* const xo = x + (int64_t)bimg * g.C * g.HW + py0 * g.W + px0;
+#pragma unroll
+    for (int u = 0; u < XS; u++) {
+      const int iy = py0 + ((xpk[u] >> 24) & 0x7f), ix = px0 + ((xpk[u] >> 16) & 0xff);
+      xv[u] = 0.f;
+      if (xpk[u] >= 0 && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) xv[u] = xo[xrel[u]];
+    }
+  };
+  auto store_patch = [&](float* buf) {
+#pragma unroll
+    for (int u = 0; u < XS; u++) buf[xpk[u] & 0xffff] = xv[u];
+  };
+
+  const int ntiles = g.B * g.tiles_x * g.tiles_y;
+  int tile = blockIdx.x;                 // the launch has no more workgroups than tiles
+  load_patch(tile);
+  store_patch(P0);
+  __syncthreads();
+
+  const int n0 = wave * 16 * TN;         // this wavefront's first N entry
+  int pb[TN][3];   // one base per kernel row, so the column tap is an immediate offset
+#pragma unroll
+  for (int t = 0; t < TN; t++) {
+    const int p = tab[n0 + t * 16 + li] + lk * g.PL;
+#pragma unroll
+    for (int kr = 0; kr < 3; kr++) pb[t][kr] = p + kr * g.PW;
+  }
+  const float* const abase0 = As + lk * 9 * 16 + li;
+  const int astride = g.KP * 16;         // between the 16-filter halves of the tile
+  int cur = 0;
+
+  for (;;) {
+    const int next = tile + gridDim.x;
+    const bool more = next < ntiles;
+    if (more) load_patch(next);          // in flight during this tile's MFMAs
+
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+      for (int t = 0; t < TN; t++) acc[a][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // ---- MFMA: step = (channel quad, tap); lane group lk takes channel 4 quad + lk.  Operands
+    // of step s + 2 are fetched while step s runs (three register sets), across quad
+    // boundaries too; one LDS read is placed after each MFMA.
+    float af[3][TM], bf[3][TN];
+    const float* abase = abase0;
+    const float* pq = P0 + cur * plane_floats;   // plane base of the current quad
+    auto fetch = [&](int set, int tap, int aoff, int poff) {
+      const int kr = tap / 3, kc = tap % 3;
+#pragma unroll
+      for (int a = 0; a < TM; a++) af[set][a] = abase[aoff + tap * 16 + a * astride];
+#pragma unroll
+      for (int t = 0; t < TN; t++) bf[set][t] = pq[poff + pb[t][kr] + kc];
+    };
+    fetch(0, 0, 0, 0);
+    fetch(1, 1, 0, 0);
+    for (int qd = 0; qd < g.NQ; qd++) {
+      // the two fetches that reach into the next quad; the last quad repeats its own (unused)
+      const int na = qd + 1 < g.NQ ? 36 * 16 : 0, np = qd + 1 < g.NQ ? 4 * g.PL : 0;
+#pragma unroll
+      for (int tap = 0; tap < 9; tap++) {
+        if (tap + 2 < 9) fetch((tap + 2) % 3, tap + 2, 0, 0);
+        else fetch((tap + 2) % 3, tap + 2 - 9, na, np);
+#pragma unroll
+        for (int a = 0; a < TM; a++)
+#pragma unroll
+          for (int t = 0; t < TN; t++)
+            acc[a][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[tap % 3][a], bf[tap % 3][t], acc[a][t], 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < TM * TN; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // DS read
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      abase += 36 * 16;
+      pq += 4 * g.PL;
+    }
+
+    // ---- epilogue from the accumulators: register v of acc[a][t] is filter m0 + 16 a + 4 lk + v
+    // at N entry n0 + 16 t + li
+    {
+      const int bimg = mdiv(tile, g.mTXY);
+      const int trem = tile - bimg * (g.tiles_x * g.tiles_y);
+      const int tyi = mdiv(trem, g.mTX), txi = trem - tyi * g.tiles_x;
+      const int oy0 = tyi * g.TH, ox0 = txi * g.TW;
+      // where each N tile's value goes (element offset inside a filter's plane), -1: nowhere
+      int yoff[TN];
+      const int plane = g.pool ? g.ph * g.pw : g.oh * g.ow;
+#pragma unroll
+      for (int t = 0; t < TN; t++) {
+        const int n = n0 + 16 * t + li;
+        if (g.pool) {
+          const int q = n >> 2;
+          const int py = mdiv(q, g.mHTW), px = q - py * g.HTW;
+          const int oy = (oy0 >> 1) + py, ox = (ox0 >> 1) + px;
+          yoff[t] = ((n & 3) == 0 && n < g.npix && oy < g.ph && ox < g.pw) ? oy * g.pw + ox : -1;
+        } else {
+          const int ty = mdiv(n, g.mTW), tx = n - ty * g.TW;
+          const int oy = oy0 + ty, ox = ox0 + tx;
+          yoff[t] = (n < g.npix && oy < g.oh && ox < g.ow) ? oy * g.ow + ox : -1;
+        }
+      }
+#pragma unroll
+      for (int a = 0; a < TM; a++) {
+        // BatchNorm constants of this lane's filters 16 a + 4 lk + (0..3): one 128-bit read each
+        const float* const fp = ftab + 16 * a + 4 * lk;
+        f32x4 ca = {0.f, 0.f, 0.f, 0.f}, cb = ca, cg = ca, ce = ca;
+        if (tail.mean) {
+          ca = *reinterpret_cast<const f32x4*>(fp);
+          cb = *reinterpret_cast<const f32x4*>(fp + BM);
+          if (tail.gamma) cg = *reinterpret_cast<const f32x4*>(fp + 2 * BM);
+          if (tail.beta) ce = *reinterpret_cast<const f32x4*>(fp + 3 * BM);
+        }
+        const int f0 = m0 + 16 * a + 4 * lk;
+        float* const yf = y + ((int64_t)bimg * g.F + f0) * plane;
+#pragma unroll
+        for (int t = 0; t < TN; t++) {
+#pragma unroll
+          for (int v = 0; v < 4; v++) {
+            float val = acc[a][t][v];
+            if (tail.mean) {
+              val = val * ca[v];
+              val = val + cb[v];
+              if (tail.gamma) val = cg[v] * val;
+              if (tail.beta) val = val + ce[v];
+            }
+            val = act_apply(val, tail.act, tail.alpha);
+            if (g.pool) {
+              float best = -3.402823466e+38f;
+              const float v0 = quad_bcast<0>(val), v1 = quad_bcast<1>(val), v2 = quad_bcast<2>(val), v3 = quad_bcast<3>(val);
+              if (v0 > best) best = v0;   // window positions in scan order
+              if (v1 > best) best = v1;
+              if (v2 > best) best = v2;
+              if (v3 > best) best = v3;
+              val = best;
+            }
+            if (yoff[t] >= 0 && f0 + v < g.F) yf[(int64_t)v * plane + yoff[t]] = val;
+          }
+        }
+      }
+    }
+    if (!more) break;
+    if constexpr (DB) {
+      cur ^= 1;
+      store_patch(P0 + cur * plane_floats);   // the buffer nobody reads during this tile
+      __syncthreads();
+    } else {
+      __syncthreads();                        // every wavefront is done reading the patch
+      store_patch(P0);
+      __syncthreads();
+    }
+    tile = next;
+  }
+}
+
+struct WidePlan {
+  WideGeom g;
+  int TM, TN, XS;
+  bool DB;
+  size_t lds;
+};
+
+constexpr size_t kLdsBudget = 156 * 1024;   // of the 160 KB a workgroup may hold
+constexpr int kMaxSlots = 24;               // patch cells per thread the kernel is built for
+constexpr int kDeviceCUs = 256;             // the plan is a function of the command alone: MI355X
+
+inline size_t wide_lds(const WideGeom& g, int TM, int TN, int PL, bool db) {
+  return ((size_t)TM * g.KP * 16 + (size_t)(db ? 2 : 1) * (4 * g.NQ * PL + 8) + kWaves * 16 * TN + 4 * 16 * TM) * 4;
+}
+
+// Geometry and workgroup shape for one command, a function of its shape and of `pool`
+// only; false when the kernel does not take the shape.
+bool wide_plan(const gh_cmd& c, bool pool, WidePlan* out) {
+  if (gh_dtype_of(c.flags) != GH_F32) return false;
+  const int64_t B = c.dim[0], C = c.dim[1], H = c.dim[2], W = c.dim[3], F = c.dim[4];
+  const int64_t pad = c.dim[7];
+  if (c.dim[5] != 3 || c.dim[6] != 3 || c.dim[9] != 1 || c.dim[10] != 1 || c.dim[11] != 1 || c.dim[12] != 1 ||
+      c.dim[8] != pad || pad < 0 || pad > 1)
+    return false;
+  if (B < 1 || F < 1 || C < 5 || C > 64 || H < 3 || W < 3 || H > 8192 || W > 8192) return false;
+  if (B * C * H * W >= (1ll << 31) || B * F * H * W >= (1ll << 31) || F > (1 << 20)) return false;
+  if (getenv("GORGONIA_HIP_CONV_NO_WIDE")) return false;   // tuning switch: the other kernels only
+  WideGeom g{};
+  g.B = (int)B; g.C = (int)C; g.H = (int)H; g.W = (int)W; g.F = (int)F; g.pad = (int)pad;
+  g.oh = g.H + 2 * g.pad - 2; g.ow = g.W + 2 * g.pad - 2;
+  if (g.oh <= 0 || g.ow <= 0) return false;
+  g.pool = pool ? 1 : 0; g.ph = g.oh / 2; g.pw = g.ow / 2;
+  if (pool && (g.ph == 0 || g.pw == 0)) return false;
+  g.HW = g.H * g.W; g.K = g.C * 9; g.NQ = (g.C + 3) / 4; g.KP = 36 * g.NQ;
+  // enough pixels that patches alone fill the device: this kernel does not split K
+  const int need_h = pool ? 2 * g.ph : g.oh, need_w = pool ? 2 * g.pw : g.ow;
+  if ((int64_t)B * need_h * need_w < 128 * 256) return false;
+  // Candidates: 16, 32 or 64 filters per workgroup, one or two patch buffers; for each the patch
+  // shape with the least padded MFMA work (then the smallest halo) among those whose staging
+  // fits the kernel's slots and LDS.  The candidate with the shortest estimated run wins:
+  // rounds of tiles over the workgroups the device holds at once (two per compute unit when
+  // LDS and registers allow; a lone workgroup's staging and epilogue are not hidden).
+  int tm_hi = F > 32 ? 4 : F > 16 ? 2 : 1, tm_lo = 1;
+  int menu_lo = 1, menu_hi = 2;
+  if (const char* env = getenv("GORGONIA_HIP_CONV_WIDE_PLAN")) {   // tuning override: "TM,TN"
+    int tm = 0, tn = 0;
+    if (sscanf(env, "%d,%d", &tm, &tn) == 2 && (tm == 1 || tm == 2 || tm == 4) && (tn == 1 || tn == 2)) {
+      tm_hi = tm_lo = tm; menu_lo = menu_hi = tn;
+    }
+  }
+  const int step = pool ? 2 : 1;
+  double best_est = 0;
+  bool found = false;
+  for (int TM = tm_hi; TM >= tm_lo; TM >>= 1)
+    for (int db = 1; db >= 0; db--)
+    for (int TN = menu_lo; TN <= menu_hi; TN++) {
+      int64_t best_work = 0, best_halo = 0;
+      int bTH = 0, bTW = 0, bTN = 0;
+      for (int TH = step; TH <= 64 && TH <= need_h + step - 1; TH += step)
+        for (int TW = step; TW <= 128 && TW <= need_w + step - 1; TW += step) {
+          const int npix = TH * TW;
+          if (npix > kWaves * 16 * TN || npix <= kWaves * 16 * (TN - 1)) continue;
+          const int PP = (TH + 2) * (TW + 2);
+          if (4 * g.NQ * PP > kMaxSlots * kThreads) continue;
+          if (wide_lds(g, TM, TN, PP | 1, db != 0) > kLdsBudget) continue;
+          const int64_t tiles = (int64_t)((need_h + TH - 1) / TH) * ((need_w + TW - 1) / TW);
+          const int64_t work = tiles * TN, halo = tiles * PP;
+          if (!bTN || work < best_work || (work == best_work && halo < best_halo)) {
+            best_work = work; best_halo = halo; bTH = TH; bTW = TW; bTN = TN;
+          }
+        }
+      if (!bTN) continue;
+      WideGeom h = g;
+      h.TH = bTH; h.TW = bTW; h.HTW = bTW / 2;
+      h.tiles_x = (need_w + bTW - 1) / bTW; h.tiles_y = (need_h + bTH - 1) / bTH;
+      h.PW = bTW + 2; h.PP = (bTH + 2) * h.PW;
+      h.PL = h.PP | 1;   // odd pitch: the four channel planes of a fetch start in different banks
+      h.npix = bTH * bTW;
+      const int64_t ntiles = (int64_t)h.B * h.tiles_x * h.tiles_y;
+      if (ntiles > (1ll << 30)) continue;
+      const int XS = 4 * h.NQ * h.PP <= 12 * kThreads ? 12 : kMaxSlots;
+      const size_t lds = wide_lds(h, TM, bTN, h.PL, db != 0);
+      const int occ = (XS == 12 && TM * bTN <= 4 && 2 * lds <= 158 * 1024) ? 2 : 1;
+      const int ft = (h.F + 16 * TM - 1) / (16 * TM);
+      const int64_t groups = std::max<int64_t>(1, (int64_t)kDeviceCUs * occ / ft);
+      const int64_t rounds = (ntiles + groups - 1) / groups;
+      // a tile's MFMA time in units of one 16x16 tile over K, shared by `occ` workgroups
+      const double est = (double)rounds * TM * bTN * occ * (occ == 2 ? 1.0 : db ? 1.35 : 1.45);
+      if (!found || est < best_est) {
+        found = true; best_est = est;
+        h.mTXY = magic_of(h.tiles_x * h.tiles_y); h.mTX = magic_of(h.tiles_x); h.mPP = magic_of(h.PP);
+        h.mPW = magic_of(h.PW); h.mTW = magic_of(h.TW); h.mHTW = magic_of(h.HTW);
+        out->g = h; out->TM = TM; out->TN = bTN; out->XS = XS; out->DB = db != 0; out->lds = lds;
+      }
+    }
+  return found;
+}
+
+template <int TM, int TN, int XS, bool DB>
+int launch_wide(gh_ctx* ctx, const gh_cmd& c, const WidePlan& p) {
+  // more than 64 KB of dynamic LDS has to be allowed per kernel, once
+  static std::once_flag once;
+  static hipError_t attr_rc = hipSuccess;
+  std::call_once(once, [] {
+    attr_rc = hipFuncSetAttribute((const void*)k_conv3x3_wide<TM, TN, XS, DB>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  });
+  if (attr_rc != hipSuccess) return gh_check_hip(ctx, attr_rc, "hipFuncSetAttribute(conv3x3 wide)");
+  // Persistent workgroups: as many as the device holds at once (two per compute unit where
+  // their LDS allows), shared among the filter tiles; each walks its tiles id, id + G, ...
+  // G is then lowered to the fewest workgroups that need no more rounds.
+  const int64_t ntiles = (int64_t)p.g.B * p.g.tiles_x * p.g.tiles_y;
+  const int ft = (p.g.F + 16 * TM - 1) / (16 * TM);
+  const int per_cu = (XS == 12 && TM * TN <= 4 && 2 * p.lds <= 158 * 1024) ? 2 : 1;
+  int64_t G = std::max<int64_t>(1, (int64_t)ctx->cu_count * per_cu / ft);
+  if (G > ntiles) G = ntiles;
+  const int64_t rounds = (ntiles + G - 1) / G;
+  G = (ntiles + rounds - 1) / rounds;
+  const dim3 grid((unsigned)G, (unsigned)ft);
+  if (getenv("GORGONIA_HIP_CONV_WIDE_DEBUG"))
+    fprintf(stderr, "wide conv: TM=%d TN=%d XS=%d DB=%d patch %dx%d tiles %lld G=%lld ft=%d lds=%zu\n", TM, TN, XS, (int)DB,
+            p.g.TH, p.g.TW, (long long)ntiles, (long long)G, ft, p.lds);
+  hipLaunchKernelGGL((k_conv3x3_wide<TM, TN, XS, DB>), grid, dim3(kThreads), p.lds, ctx->stream,
+                     (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                     (float*)(uintptr_t)c.ptr[2], p.g, conv_tail(c));
+  return gh_check_hip(ctx, hipGetLastError(), "conv3x3 wide launch");
+}
+
+template <int TM, int TN>
+int launch_wide_tile(gh_ctx* ctx, const gh_cmd& c, const WidePlan& p) {
+  if (p.XS == 12) return p.DB ? launch_wide<TM, TN, 12, true>(ctx, c, p) : launch_wide<TM, TN, 12, false>(ctx, c, p);
+  return p.DB ? launch_wide<TM, TN, kMaxSlots, true>(ctx, c, p) : launch_wide<TM, TN, kMaxSlots, false>(ctx, c, p);
+}
+
+}  // namespace
+
+bool gh_conv_wide_takes(const gh_cmd& c) {
+  WidePlan p;
+  return wide_plan(c, false, &p);
+}
+
+// Pooling rides in the epilogue where the even-sized patches it needs cost about the same
+// matrix work as the best plain patch grid.
+bool gh_conv_wide_can_pool(const gh_cmd& c) {
+  WidePlan p, q;
+  if (!wide_plan(c, false, &p) || !wide_plan(c, true, &q)) return false;
+  auto work = [](const WidePlan& a) {
+    return (int64_t)a.g.tiles_x * a.g.tiles_y * a.TN * a.TM * ((a.g.F + 16 * a.TM - 1) / (16 * a.TM));
+  };
+  return work(q) * 100 <= work(p) * 110;
+}
+
+// Returns -1 when the shape is not one this kernel takes.
+int gh_try_launch_conv_wide(gh_ctx* ctx, const gh_cmd& c) {
+  WidePlan p;
+  const bool pool = c.flags & GH_FLAG_CONV_POOL2;
+  // a pooled command only rides here when the plain one would too
+  if (!wide_plan(c, false, &p)) return -1;
+  if (pool && (!gh_conv_wide_can_pool(c) || !wide_plan(c, true, &p)))
+    return gh_fail(ctx, GH_EINVAL, "conv2d: no fused pooling for this shape (see gh_conv2d_can_pool)");
+#define GH_WIDE_TN(TM_)                                       \
+  if (p.TN == 1) return launch_wide_tile<TM_, 1>(ctx, c, p);  \
+  return launch_wide_tile<TM_, 2>(ctx, c, p);
+  if (p.TM == 1) { GH_WIDE_TN(1) }
+  if (p.TM == 2) { GH_WIDE_TN(2) }
+  GH_WIDE_TN(4)
+#undef GH_WIDE_TN
+}

@@ -2880,6 +2880,8 @@ int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
   if (rcs >= 0) return rcs;
   const int rcp = gh_try_launch_conv_patch(ctx, c);
   if (rcp >= 0) return rcp;
+  const int rcw = gh_try_launch_conv_wide(ctx, c);
+  if (rcw >= 0) return rcw;
   const int rc3 = try_launch_conv3(ctx, c);
   if (rc3 >= 0) return rc3;
   if (c.flags & GH_FLAG_CONV_POOL2)
@@ -3095,10 +3097,11 @@ extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {
     return oh >= 2 && ow >= 2;
   }
   if (getenv("GORGONIA_HIP_CONV_NO_POOL")) return 0;  // tuning switch: keep MaxPool2D a kernel of its own
-  // a shape the small-image or the patch kernel takes is pooled there or not at all (the plain and the
+  // a shape the small-image, the patch or the wide-image kernel takes is pooled there or not at all (the plain and the
   // pooled command must sum in the same order)
   if (gh_conv_small_takes(*c)) return gh_conv_small_can_pool(*c) ? 1 : 0;
   if (gh_conv_patch_takes(*c)) return gh_conv_patch_can_pool(*c) ? 1 : 0;
+  if (gh_conv_wide_takes(*c)) return gh_conv_wide_can_pool(*c) ? 1 : 0;
   Conv3Geom g;
   int BM, BN, per_thread;
   size_t lds;

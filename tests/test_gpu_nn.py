@@ -270,6 +270,46 @@ def test_conv_patch_kernel(ctx, cfg):
                           O.maxpool2d(leaky, (2, 2), (0, 0), (2, 2)), f"patch conv+bn+leaky+pool {cfg}")
 
 
+# shapes the wide-image kernel takes (3x3, at most 64 channels, enough pixels that patches alone fill the
+# device; whole K per wavefront): channel counts that are not multiples of four, ragged filter tiles,
+# partial patches on both axes, no padding, pooled extents odd and even
+WIDE_CASES = [(2, 16, 130, 131, 32, 1), (1, 32, 104, 104, 64, 1), (3, 3, 120, 96, 16, 1), (40, 1, 28, 28, 32, 1),
+              (2, 8, 129, 140, 5, 0), (1, 24, 181, 190, 40, 1), (1, 64, 190, 181, 21, 1), (2, 12, 150, 111, 70, 0),
+              (1, 6, 200, 170, 33, 1)]
+
+
+@pytest.mark.parametrize("cfg", WIDE_CASES)
+def test_conv_wide_kernel(ctx, cfg):
+    """The wide-image convolution kernel against the oracle (<= 1e-5, exact on integers), and every
+    epilogue it can carry against the oracle's operators applied to its own plain result, bit for bit."""
+    B, C, H, W, F, pad = cfg
+    x = synth.uniform(51, (B, C, H, W), -1, 1)
+    w = synth.he_normal(52, (F, C, 3, 3))
+    plain = gpu_conv(ctx, x, w, (pad, pad), (1, 1), (1, 1))
+    ref = O.conv2d_direct_f64(x, w, (pad, pad), (1, 1), (1, 1))
+    err = rel_frobenius(plain, ref)
+    assert err <= TOL, f"wide conv {cfg}: rel frobenius {err:.3e}"
+    rng = np.random.default_rng(11)
+    xi = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+    wi = rng.integers(-3, 4, (F, C, 3, 3)).astype(np.float32)
+    assert_bits_equal(gpu_conv(ctx, xi, wi, (pad, pad), (1, 1), (1, 1)), O.conv2d(xi, wi, (pad, pad), (1, 1), (1, 1)),
+                      f"integer wide conv {cfg}")
+    mean, var = synth.normal(53, (F,), 0.0, 0.1), synth.uniform(54, (F,), 0.5, 1.5)
+    gamma, beta = synth.uniform(55, (F,), 0.5, 1.5), synth.normal(56, (F,), 0.0, 0.1)
+    leaky = O.leaky_relu(O.bn_infer(plain, mean, var, 1e-5, gamma, beta), 0.1).reshape(plain.shape)
+    assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, gamma, beta), act="leaky", alpha=0.1), leaky,
+                      f"wide conv+bn+leaky {cfg}")
+    relu = O.relu(plain).reshape(plain.shape)
+    assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), act="relu"), relu, f"wide conv+relu {cfg}")
+    cmd = D.cmd_conv2d(1, 1, 1, B, C, H, W, F, 3, 3, (pad, pad))
+    if ctx.lib.gh_conv2d_can_pool(cmd) == 1:
+        assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, gamma, beta), act="leaky", alpha=0.1,
+                                        pool2=True),
+                          O.maxpool2d(leaky, (2, 2), (0, 0), (2, 2)), f"wide conv+bn+leaky+pool {cfg}")
+        assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), act="relu", pool2=True),
+                          O.maxpool2d(relu, (2, 2), (0, 0), (2, 2)), f"wide conv+relu+pool {cfg}")
+
+
 def test_conv_random_geometry_sweep(ctx):
     """Seeded sweep over 3x3 and other geometries (all three convolution kernels, ragged sizes,
     batch boundaries inside blocks): the plain convolution against the oracle, and wherever the
