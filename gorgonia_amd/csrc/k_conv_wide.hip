@@ -87,15 +87,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
     constexpr int JS = kThreads / BM;    // 128-bit columns in flight per pass
     const int ncol = g.KP / 4;
     if ((g.K & 3) == 0) {
+      // every workgroup reads the same filter rows at the same moment: each starts at a column
+      // of its own (and wraps), so that their loads spread over the cache channels
+      const int rot = (int)((blockIdx.x * 5u) % (unsigned)ncol);
       for (int j = j0; j < ncol; j += 4 * JS) {
         f32x4 v[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const f32x4_a4*>(wrow + 4 * min(j + u * JS, ncol - 1));
+        int jj[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-          const int jj = min(j + u * JS, ncol - 1);   // passes past the end rewrite the last column
+          const int jc = min(j + u * JS, ncol - 1) + rot;   // passes past the end rewrite the last column
+          jj[u] = jc >= ncol ? jc - ncol : jc;
+          v[u] = *reinterpret_cast<const f32x4_a4*>(wrow + 4 * jj[u]);
+        }
 #pragma unroll
-          for (int e = 0; e < 4; e++) ad[(4 * jj + e) * 16] = v[u][e];
+        for (int u = 0; u < 4; u++) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) ad[(4 * jj[u] + e) * 16] = v[u][e];
         }
       }
     } else {
@@ -103,10 +110,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
     }
   }
   // ---- per-thread patch cells, the same for every tile: source offset relative to the patch
-  // origin, row and column inside the padded patch, destination in the buffer.  Cells of padded
-  // channels are flagged and written as zero; slots past the last cell are flagged too and
-  // write the spare floats at the end of the buffer.
-  int xrel[XS], xpk[XS];   // xpk = zero-cell flag << 31 | row << 24 | column << 16 | destination
+  // origin, row and column inside the padded patch, destination in the buffer.  Slots past the
+  // last cell and cells of padded channels are flagged: they load nothing that matters and
+  // write the spare floats at the end of the buffer; the padded planes are zeroed here, once.
+  int xrel[XS], xpk[XS];   // xpk = flag << 31 | row << 24 | column << 16 | destination
   {
     const int cells = 4 * g.NQ * g.PP;
 #pragma unroll
@@ -117,9 +124,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
       const int r = mdiv(rem, g.mPW), cc = rem - r * g.PW;
       const bool real = id < cells && pl < g.C;
       xrel[u] = min(pl, g.C - 1) * g.HW + r * g.W + cc;
-      const int dst = id < cells ? pl * g.PL + rem : 4 * g.NQ * g.PL + (lane & 7);
+      const int dst = real ? pl * g.PL + rem : 4 * g.NQ * g.PL + (lane & 7);
       xpk[u] = (real ? 0 : (int)0x80000000) | (r << 24) | (cc << 16) | dst;
     }
+    const int zero0 = g.C * g.PL, zero1 = 4 * g.NQ * g.PL;
+    for (int bsel = 0; bsel < (DB ? 2 : 1); bsel++)
+      for (int i = zero0 + tid; i < zero1; i += kThreads) P0[bsel * plane_floats + i] = 0.f;
   }
   // ---- table of patch cells of the N entries
   for (int n = tid; n < NB; n += kThreads) {
@@ -138,18 +148,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
   }
 
   float xv[XS];
-  // global loads of one tile's patch into registers (cells outside the image: zero, no load)
+  // global loads of one tile's patch into registers.  A patch that lies inside the image, halo
+  // and all, needs no test: every load is base + per-thread offset.  At the image border each
+  // cell is tested and cells outside are zero.
   auto load_patch = [&](int tile) {
     const int bimg = mdiv(tile, g.mTXY);
     const int trem = tile - bimg * (g.tiles_x * g.tiles_y);
     const int tyi = mdiv(trem, g.mTX), txi = trem - tyi * g.tiles_x;
     const int py0 = tyi * g.TH - g.pad, px0 = txi * g.TW - g.pad;
     const float* const xo = x + (int64_t)bimg * g.C * g.HW + py0 * g.W + px0;
+    if (py0 >= 0 && px0 >= 0 && py0 + g.TH + 2 <= g.H && px0 + g.TW + 2 <= g.W) {
 #pragma unroll
-    for (int u = 0; u < XS; u++) {
-      const int iy = py0 + ((xpk[u] >> 24) & 0x7f), ix = px0 + ((xpk[u] >> 16) & 0xff);
-      xv[u] = 0.f;
-      if (xpk[u] >= 0 && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) xv[u] = xo[xrel[u]];
+      for (int u = 0; u < XS; u++) xv[u] = xo[xrel[u]];
+    } else {
+#pragma unroll
+      for (int u = 0; u < XS; u++) {
+        const int iy = py0 + ((xpk[u] >> 24) & 0x7f), ix = px0 + ((xpk[u] >> 16) & 0xff);
+        xv[u] = 0.f;
+        if (xpk[u] >= 0 && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) xv[u] = xo[xrel[u]];
+      }
     }
   };
   auto store_patch = [&](float* buf) {
@@ -171,8 +188,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
 #pragma unroll
     for (int kr = 0; kr < 3; kr++) pb[t][kr] = p + kr * g.PW;
   }
-  const float* const abase0 = As + lk * 9 * 16 + li;
-  const int astride = g.KP * 16;         // between the 16-filter halves of the tile
   int cur = 0;
 
   for (;;) {
@@ -188,26 +203,43 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
 
     // ---- MFMA: step = (channel quad, tap); lane group lk takes channel 4 quad + lk.  Operands
     // of step s + 2 are fetched while step s runs (three register sets), across quad
-    // boundaries too; one LDS read is placed after each MFMA.
+    // boundaries too; one LDS read is placed after each MFMA.  The fetch stream has its own
+    // pointers, moved once per quad just before it enters the next one (taps are immediate
+    // offsets), so the loop carries TM + 3 TN vector adds per 9 TM TN MFMAs and no other
+    // vector instruction: the SIMD runs vector and matrix instructions one after the other,
+    // never at once, so each one outside the matrix pipe is time the matrix pipe stands idle.
     float af[3][TM], bf[3][TN];
-    const float* abase = abase0;
-    const float* pq = P0 + cur * plane_floats;   // plane base of the current quad
-    auto fetch = [&](int set, int tap, int aoff, int poff) {
+    const float* fa[TM];
+    const float* fb[TN][3];
+#pragma unroll
+    for (int a = 0; a < TM; a++) fa[a] = As + a * (g.KP * 16) + lk * 9 * 16 + li;
+#pragma unroll
+    for (int t = 0; t < TN; t++)
+#pragma unroll
+      for (int kr = 0; kr < 3; kr++) fb[t][kr] = P0 + cur * plane_floats + pb[t][kr];
+    auto fetch = [&](int set, int tap) {
       const int kr = tap / 3, kc = tap % 3;
 #pragma unroll
-      for (int a = 0; a < TM; a++) af[set][a] = abase[aoff + tap * 16 + a * astride];
+      for (int a = 0; a < TM; a++) af[set][a] = fa[a][tap * 16];
 #pragma unroll
-      for (int t = 0; t < TN; t++) bf[set][t] = pq[poff + pb[t][kr] + kc];
+      for (int t = 0; t < TN; t++) bf[set][t] = fb[t][kr][kc];
     };
-    fetch(0, 0, 0, 0);
-    fetch(1, 1, 0, 0);
+    fetch(0, 0);
+    fetch(1, 1);
     for (int qd = 0; qd < g.NQ; qd++) {
-      // the two fetches that reach into the next quad; the last quad repeats its own (unused)
+      // the last quad's look-ahead fetches repeat its own first taps (unused)
       const int na = qd + 1 < g.NQ ? 36 * 16 : 0, np = qd + 1 < g.NQ ? 4 * g.PL : 0;
 #pragma unroll
       for (int tap = 0; tap < 9; tap++) {
-        if (tap + 2 < 9) fetch((tap + 2) % 3, tap + 2, 0, 0);
-        else fetch((tap + 2) % 3, tap + 2 - 9, na, np);
+        if (tap == 7) {
+#pragma unroll
+          for (int a = 0; a < TM; a++) fa[a] += na;
+#pragma unroll
+          for (int t = 0; t < TN; t++)
+#pragma unroll
+            for (int kr = 0; kr < 3; kr++) fb[t][kr] += np;
+        }
+        fetch((tap + 2) % 3, (tap + 2) % 9);
 #pragma unroll
         for (int a = 0; a < TM; a++)
 #pragma unroll
@@ -220,8 +252,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-      abase += 36 * 16;
-      pq += 4 * g.PL;
     }
 
     // ---- epilogue from the accumulators: register v of acc[a][t] is filter m0 + 16 a + 4 lk + v
@@ -248,6 +278,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
           yoff[t] = (n < g.npix && oy < g.oh && ox < g.ow) ? oy * g.ow + ox : -1;
         }
       }
+      // one 64-bit base per tile, 32-bit byte offsets per lane (a filter tile's planes span < 2 GB)
+      char* const ytile = reinterpret_cast<char*>(y + ((int64_t)bimg * g.F + m0) * plane);
+      const unsigned pbytes = 4u * (unsigned)plane;
+      const bool all4 = (g.F & 3) == 0;   // then a lane's four filters exist or not together
 #pragma unroll
       for (int a = 0; a < TM; a++) {
         // BatchNorm constants of this lane's filters 16 a + 4 lk + (0..3): one 128-bit read each
@@ -259,10 +293,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
           if (tail.gamma) cg = *reinterpret_cast<const f32x4*>(fp + 2 * BM);
           if (tail.beta) ce = *reinterpret_cast<const f32x4*>(fp + 3 * BM);
         }
-        const int f0 = m0 + 16 * a + 4 * lk;
-        float* const yf = y + ((int64_t)bimg * g.F + f0) * plane;
+        const int fl = 16 * a + 4 * lk;              // first of the lane's four filters, inside the tile
+        const int nf = min(max(g.F - (m0 + fl), 0), 4);   // how many of them exist
 #pragma unroll
         for (int t = 0; t < TN; t++) {
+          unsigned off = (unsigned)fl * pbytes + 4u * (unsigned)max(yoff[t], 0);
+          const bool live = yoff[t] >= 0 && nf > 0;
+          float res[4];
 #pragma unroll
           for (int v = 0; v < 4; v++) {
             float val = acc[a][t][v];
@@ -282,7 +319,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
               if (v3 > best) best = v3;
               val = best;
             }
-            if (yoff[t] >= 0 && f0 + v < g.F) yf[(int64_t)v * plane + yoff[t]] = val;
+            res[v] = val;
+          }
+          if (all4) {
+            if (live) {   // one test for the four stores
+#pragma unroll
+              for (int v = 0; v < 4; v++) *reinterpret_cast<float*>(ytile + (off + v * pbytes)) = res[v];
+            }
+          } else {
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+              if (live && v < nf) *reinterpret_cast<float*>(ytile + (off + v * pbytes)) = res[v];
           }
         }
       }
@@ -331,7 +378,7 @@ bool wide_plan(const gh_cmd& c, bool pool, WidePlan* out) {
   WideGeom g{};
   g.B = (int)B; g.C = (int)C; g.H = (int)H; g.W = (int)W; g.F = (int)F; g.pad = (int)pad;
   g.oh = g.H + 2 * g.pad - 2; g.ow = g.W + 2 * g.pad - 2;
-  if (g.oh <= 0 || g.ow <= 0) return false;
+  if (g.oh <= 0 || g.ow <= 0 || (int64_t)g.oh * g.ow > (1 << 22)) return false;   // 64 planes of results within 32-bit byte offsets
   g.pool = pool ? 1 : 0; g.ph = g.oh / 2; g.pw = g.ow / 2;
   if (pool && (g.ph == 0 || g.pw == 0)) return false;
   g.HW = g.H * g.W; g.K = g.C * 9; g.NQ = (g.C + 3) / 4; g.KP = 36 * g.NQ;
@@ -388,7 +435,9 @@ bool wide_plan(const gh_cmd& c, bool pool, WidePlan* out) {
       const int64_t groups = std::max<int64_t>(1, (int64_t)kDeviceCUs * occ / ft);
       const int64_t rounds = (ntiles + groups - 1) / groups;
       // a tile's MFMA time in units of one 16x16 tile over K, shared by `occ` workgroups
-      const double est = (double)rounds * TM * bTN * occ * (occ == 2 ? 1.0 : db ? 1.35 : 1.45);
+      // (operand fetches per MFMA grow as the wavefront's tile shrinks: TM + TN reads feed TM TN MFMAs)
+      const double est = (double)rounds * TM * bTN * occ * (occ == 2 ? 1.0 : db ? 1.35 : 1.45) *
+                         (1.0 + 0.12 * (TM + bTN) / (TM * bTN));
       if (!found || est < best_est) {
         found = true; best_est = est;
         h.mTXY = magic_of(h.tiles_x * h.tiles_y); h.mTX = magic_of(h.tiles_x); h.mPP = magic_of(h.PP);
