@@ -75,6 +75,9 @@ def time_cmds(ctx, cmds, iters, warm=3):
     ctx.event(1)
     one = ctx.elapsed_ms(0, 1)
     time_cmds.last_burst_ms = one / iters
+    if SUSTAIN_MS <= 0:
+        ctx.graph_destroy(gid)
+        return time_cmds.last_burst_ms
     reps = max(1, min(4000, int(SUSTAIN_MS / max(one, 1e-3)) + 1))
     for _ in range(reps):
         ctx.graph_launch(gid)
@@ -222,10 +225,14 @@ def bench_linalg(ctx, iters):
 # WRITE_SIZE runs of this script (KiB per dispatch; FETCH_SIZE scaled by 2.0,
 # WRITE_SIZE by 1.0, the factors a 64 MiB device copy in the same runs gives).
 MEASURED_TRAFFIC_BYTES = {
-    "conv0": (2 * 935.4 + 3232.0) * 1024,
-    "conv1": (2 * 4350.2 + 2464.0) * 1024,
-    "conv2": (2 * 2108.9 + 576.0) * 1024,
+    "conv0": (2 * 936.1 + 3232.0) * 1024,
+    "conv1": (2 * 1959.8 + 1568.0) * 1024,
+    "conv2": (2 * 2039.0 + 576.0) * 1024,
 }
+# SQ_VALU_MFMA_BUSY_CYCLES / (128 * GRBM_GUI_ACTIVE) of the same kernels in a rocprofv3 --pmc run of this
+# script (eager launches, one at a time: launch and drain are inside GUI_ACTIVE, clocks are not sustained)
+MEASURED_MFMA_BUSY = {"conv0": 0.0, "conv1": 0.277, "conv2": 0.219}
+CONV_KERNEL_NAME = {"conv0": "k_conv3x3_direct<1,2>", "conv1": "k_conv3x3_small<8,1,13,1>", "conv2": "k_conv3x3_small<8,1,9,2>"}
 
 CONVNET_LAYERS = [  # (name, B-relative shape) of configuration 4
     ("conv0", 1, 28, 32), ("conv1", 32, 14, 64), ("conv2", 64, 7, 128),
@@ -282,8 +289,9 @@ def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=Tr
     dt = time.perf_counter() - t0
     result = out.copy()
     launches = m.graph_launches()
-    VERDICTS[f"convnet{'_f64' if dtype == np.float64 else ''}{'' if resident_input else '_input_h2d'}"
-             f"{'_all_h2d' if reupload_all else ''}{'' if graph_replay == 'measured' else '_' + str(graph_replay)}"] = m.segment_verdict()
+    if graph_replay == "measured":
+        VERDICTS[f"convnet{'_f64' if dtype == np.float64 else ''}{'' if resident_input else '_input_h2d'}"
+                 f"{'_all_h2d' if reupload_all else ''}"] = m.segment_verdict()
     m.Close()
     return dt / steps * 1e3, result, inp, launches
 
@@ -489,13 +497,18 @@ def main():
                          "overlapping kernels stretch each other's durations)")
     ap.add_argument("--eager-timing", action="store_true",
                     help="launch every kernel eagerly, no hipGraph (use under rocprofv3 --pmc)")
+    ap.add_argument("--short-timing", action="store_true",
+                    help="time each kernel over one graph replay only (no sustained-clock loop): for runs under a "
+                         "tracing profiler, which records every launch")
     ap.add_argument("--only", default="", help="comma list of: convnet,elementwise,linalg,mlp,yolo,train")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this engine runs on one GPU; --gpus must be 1 (no multi-GPU path is built)")
     only = set(filter(None, a.only.split(",")))
-    global EAGER_TIMING
+    global EAGER_TIMING, SUSTAIN_MS
     EAGER_TIMING = a.eager_timing
+    if a.short_timing:
+        SUSTAIN_MS = 0.0
 
     from gorgonia_amd.device import Context
     ctx = Context(0, 0)
@@ -511,9 +524,9 @@ def main():
         two_images_s, two_out = bench_convnet_machines(a.steps, a.warmup, 2)
         four_images_s, four_out = bench_convnet_machines(a.steps, a.warmup, 4)
         log(f"convnet, machines in parallel host threads: two {two_images_s:.0f}, four {four_images_s:.0f} images/s")
-    ms_h2d, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False)
+    ms_h2d, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False, graph_replay=replay_mode())
     ms_h2d_all, out_h2d_all, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False,
-                                                  reupload_all=True)
+                                                  reupload_all=True, graph_replay=replay_mode())
     ms_eager, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, graph_replay=False)
     ms_replay, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, graph_replay=not EAGER_TIMING)
 
@@ -574,13 +587,14 @@ def main():
     if conv_k:
         name = max(conv_k, key=lambda k: conv_k[k]["us"])
         r = conv_k[name]
-        kname = "k_conv3x3_direct" if name == "conv0" else "k_conv3x3_lds"
+        kname = CONV_KERNEL_NAME[name]
         tail = "ReLU and the 2x2 max-pool in the epilogue" if r["pool_fused"] else "ReLU in the epilogue"
         roofline = {"kernel": f"{kname}: {name} of the convnet step with {tail}", "bound": "mfma",
                     "achieved": r["TFLOPs"], "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(r["TFLOPs"] / MFMA_F32_PEAK_TFLOPS, 4),
-                    "traffic": int(MEASURED_TRAFFIC_BYTES[name]),
-                    "launch_us": r["us"], "algorithmic_flop": r["flop"]}
+                    "traffic": int(MEASURED_TRAFFIC_BYTES[name]), "mfma_busy": MEASURED_MFMA_BUSY[name],
+                    "launch_us": r["us"], "launch_us_short_burst": r.get("us_short_burst"),
+                    "algorithmic_flop": r["flop"]}
 
     cpu = None
     parity = None
