@@ -14,8 +14,9 @@
 //     results repeat bit for bit and do not depend on the patch shape or on fused pooling.
 //   * A wavefront stages its own operands in its own LDS region - 36 filter columns
 //     k-major and the four channel planes of the padded patch, halo cells outside the
-//     image written as zero - so the main loop has no workgroup barrier; the next quad's
-//     global loads are in flight while the current one is multiplied.
+//     image written as zero - so the main loop has no workgroup barrier (there is one in
+//     front of it, behind the shared table of patch cells); the next quad's global loads are
+//     in flight while the current one is multiplied.
 //   * With GH_FLAG_CONV_POOL2 the patch has even extents and the N axis enumerates
 //     (pooled pixel, position in the 2x2 window); the epilogue reads a window as four
 //     adjacent columns (scan order and strict > of the pooling kernel, op_nn.go:860-907).
@@ -119,10 +120,11 @@ __global__ __launch_bounds__(kWaves * 64) void k_conv3x3_patch(const float* __re
   };
   load_quad();
 
-  // ---- table of patch cells (every wavefront writes the same values), operand bases
-#pragma unroll
-  for (int i = 0; i < (16 * TN + 63) / 64; i++) {
-    const int n = min(lane + 64 * i, 16 * TN - 1);
+  // ---- table of patch cells, one entry per thread, then the only barrier in front of the MFMAs
+  // (reached with the first quad's loads in flight); operand bases
+  static_assert(NTH >= 16 * TN, "one table entry per thread");
+  if (tid < 16 * TN) {
+    const int n = tid;
     const int nn = n < g.npix ? n : 0;   // idle column: any valid cell
     int ty, tx;
     if (g.pool) {
@@ -136,6 +138,7 @@ __global__ __launch_bounds__(kWaves * 64) void k_conv3x3_patch(const float* __re
     }
     tab[n] = ty * g.PW + tx;
   }
+  __syncthreads();
   int pb[TN][3];   // one base per kernel row, so the column tap is an immediate offset
 #pragma unroll
   for (int t = 0; t < TN; t++) {

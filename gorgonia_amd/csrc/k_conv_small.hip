@@ -17,8 +17,9 @@
 //     on whether the pooling below is fused: per output it is always the same WV partial
 //     sums, each over the same channels in the same order.
 //   * Each wavefront stages only its own channels (filter columns and image planes), so
-//     nothing before that sum needs a workgroup barrier, and the loads of channel quad
-//     q + 1 are in flight while quad q is multiplied.
+//     between the start (one barrier, behind the shared table of pixel offsets, with every
+//     load already in flight) and that sum nothing needs a workgroup barrier, and the loads
+//     of channel quad q + 1 are in flight while quad q is multiplied.
 //   * With GH_FLAG_CONV_POOL2 the N axis enumerates (image, pooled pixel, position in the
 //     2x2 window): the row and column a 2x2/stride-2 pool discards on an odd extent are
 //     never computed, and the epilogue reads a window as four adjacent columns (scan order
@@ -123,9 +124,13 @@ __global__ __launch_bounds__(WV * 64) void k_conv3x3_small(const float* __restri
       for (int i = lane; i < per; i += 64) p4[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
   }
-#pragma unroll
-  for (int i = 0; i < (16 * TN + 63) / 64; i++) {
-    const int n = min(lane + 64 * i, 16 * TN - 1);
+  // one entry per thread (the workgroup has more threads than N entries), then the only barrier
+  // in front of the MFMAs - every wavefront reaches it with its loads still in flight.  (Each
+  // wavefront building the whole table for itself cost 4 x 25 vector instructions per wavefront,
+  // and vector instructions are time the matrix pipe stands idle.)
+  static_assert(NTH >= 16 * TN, "one table entry per thread");
+  if (tid < 16 * TN) {
+    const int n = tid;
     int img = mdiv(n, g.mPPI);
     const int r = n - img * g.ppi;
     int oy, ox;
@@ -139,8 +144,9 @@ __global__ __launch_bounds__(WV * 64) void k_conv3x3_small(const float* __restri
       ox = r - oy * g.ow;
     }
     if (img >= g.IPB) { img = 0; oy = 0; ox = 0; }   // idle column: any valid address
-    tab[n] = img * g.C * g.PL + oy * g.Wp + ox;      // every wavefront writes the same values
+    tab[n] = img * g.C * g.PL + oy * g.Wp + ox;
   }
+  __syncthreads();
   // per-lane operand bases: one per kernel row, so the column tap is an immediate offset
   int pb[TN][3];
   {

@@ -40,42 +40,52 @@ constexpr int kThreads = 256;
 // A loader moves one R x BK (or BK x R) operand tile: load() global->registers,
 // store() registers->LDS in k-major order with row stride S.
 
+// What a thread's slots have in common - its row inside the tile, its k offset, the address of
+// its first element - is computed once per tile in prep(); a load then costs two compares and
+// one 64-bit add of a wavefront-uniform offset per slot.  (Vector instructions in this loop are
+// time the matrix pipe stands idle; recomputing row, column, address and LDS index per slot and
+// k-tile was 1.9 of them per MFMA.)
+
 // Operand stored [r][k] with k contiguous (A not transposed; B transposed).
 template <int R, int BK, bool VEC>
 struct LoadKContig {
   static constexpr int S = R + 2;  // S % 32 == 2 keeps the transposing writes conflict-free
   static constexpr int TOTAL = R * BK / 4;  // float4 slots in a tile
   static constexpr int NV = (TOTAL + kThreads - 1) / kThreads;
+  static constexpr int RS = kThreads / (BK / 4);   // rows between a thread's slots
+  static_assert(kThreads % (BK / 4) == 0, "a thread's slots share their k offset");
   const float* base; int ld; int rmax; int kmax;
+  const float* p0;   // first slot's element at k = 0
+  int rrel, kq;      // first slot's row (absolute), k offset inside a tile
   f32x4 reg[NV];
-  __device__ __forceinline__ void load(int r0, int k0) {
+  __device__ __forceinline__ void prep(int r0) {
+    rrel = r0 + (int)threadIdx.x / (BK / 4);
+    kq = ((int)threadIdx.x % (BK / 4)) * 4;
+    p0 = base + (int64_t)rrel * ld + kq;
+  }
+  __device__ __forceinline__ void load(int, int k0) {
 #pragma unroll
     for (int j = 0; j < NV; j++) {
-      const int f = threadIdx.x + j * kThreads;
-      const int r = r0 + f / (BK / 4);
-      const int k = k0 + (f % (BK / 4)) * 4;
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
-      if ((TOTAL % kThreads == 0 || f < TOTAL) && r < rmax) {
-        const float* p = base + (int64_t)r * ld + k;
+      if ((TOTAL % kThreads == 0 || (int)threadIdx.x + j * kThreads < TOTAL) && rrel < rmax - j * RS) {
+        const float* p = p0 + ((int64_t)(j * RS) * ld + k0);
         if (VEC) {
-          if (k < kmax) v = *reinterpret_cast<const f32x4*>(p);
+          if (kq < kmax - k0) v = *reinterpret_cast<const f32x4*>(p);
         } else {
 #pragma unroll
-          for (int e = 0; e < 4; e++) if (k + e < kmax) v[e] = p[e];
+          for (int e = 0; e < 4; e++) if (kq + e < kmax - k0) v[e] = p[e];
         }
       }
       reg[j] = v;
     }
   }
   __device__ __forceinline__ void store(float* lds) const {
+    float* const d = lds + kq * S + (int)threadIdx.x / (BK / 4);
 #pragma unroll
     for (int j = 0; j < NV; j++) {
-      const int f = threadIdx.x + j * kThreads;
-      if (TOTAL % kThreads != 0 && f >= TOTAL) continue;
-      const int r = f / (BK / 4);
-      const int kq = (f % (BK / 4)) * 4;
+      if (TOTAL % kThreads != 0 && (int)threadIdx.x + j * kThreads >= TOTAL) continue;
 #pragma unroll
-      for (int e = 0; e < 4; e++) lds[(kq + e) * S + r] = reg[j][e];
+      for (int e = 0; e < 4; e++) d[e * S + j * RS] = reg[j][e];
     }
   }
 };
@@ -86,17 +96,23 @@ struct LoadMnContig {
   static constexpr int S = R;
   static constexpr int TOTAL = R * BK / 4;
   static constexpr int NV = (TOTAL + kThreads - 1) / kThreads;
+  static constexpr int KS = kThreads / (R / 4);    // k rows between a thread's slots
+  static_assert(kThreads % (R / 4) == 0, "a thread's slots share their column");
   const float* base; int ld; int rmax; int kmax;
+  const float* p0;   // first slot's element at k0 = 0
+  int c, kl;         // the thread's first column (absolute), first slot's k row inside a tile
   f32x4 reg[NV];
-  __device__ __forceinline__ void load(int c0, int k0) {
+  __device__ __forceinline__ void prep(int c0) {
+    kl = (int)threadIdx.x / (R / 4);
+    c = c0 + ((int)threadIdx.x % (R / 4)) * 4;
+    p0 = base + (int64_t)kl * ld + c;
+  }
+  __device__ __forceinline__ void load(int, int k0) {
 #pragma unroll
     for (int j = 0; j < NV; j++) {
-      const int f = threadIdx.x + j * kThreads;
-      const int k = k0 + f / (R / 4);
-      const int c = c0 + (f % (R / 4)) * 4;
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
-      if ((TOTAL % kThreads == 0 || f < TOTAL) && k < kmax) {
-        const float* p = base + (int64_t)k * ld + c;
+      if ((TOTAL % kThreads == 0 || (int)threadIdx.x + j * kThreads < TOTAL) && kl < kmax - k0 - j * KS) {
+        const float* p = p0 + (int64_t)(k0 + j * KS) * ld;
         if (VEC) {
           if (c < rmax) v = *reinterpret_cast<const f32x4*>(p);
         } else {
@@ -108,13 +124,11 @@ struct LoadMnContig {
     }
   }
   __device__ __forceinline__ void store(float* lds) const {
+    float* const d = lds + ((int)threadIdx.x / (R / 4)) * S + ((int)threadIdx.x % (R / 4)) * 4;
 #pragma unroll
     for (int j = 0; j < NV; j++) {
-      const int f = threadIdx.x + j * kThreads;
-      if (TOTAL % kThreads != 0 && f >= TOTAL) continue;
-      const int k = f / (R / 4);
-      const int c = (f % (R / 4)) * 4;
-      *reinterpret_cast<f32x4*>(&lds[k * S + c]) = reg[j];
+      if (TOTAL % kThreads != 0 && (int)threadIdx.x + j * kThreads >= TOTAL) continue;
+      *reinterpret_cast<f32x4*>(&d[j * KS * S]) = reg[j];
     }
   }
 };
@@ -140,6 +154,7 @@ struct LoadIm2col {
   uint64_t tap_mask;    // bit r set: tap r = kr*kw + kc lies inside the image
   const float* xb;
   float reg[KPT];
+  __device__ __forceinline__ void prep(int) {}
   __device__ __forceinline__ void init(int p0) {
     const int kh = KH ? KH : g.kh, kw = KW ? KW : g.kw;
     const int p = p0 + (threadIdx.x % R);
@@ -255,6 +270,8 @@ __device__ __forceinline__ void mfma_tile_loop(float* lds, LA& la, LB& lb, const
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
 
+  la.prep(m0);
+  lb.prep(n0);
   la.load(m0, kt0 * BK);
   lb.load(n0, kt0 * BK);
   la.store(As);
@@ -1887,6 +1904,7 @@ struct LoadDyRows {
   const float* dy; int F; int plane; int kmax /* B*plane */;
   int next_k = -1, b = 0, p = 0;
   float reg[RPT];
+  __device__ __forceinline__ void prep(int) {}
   __device__ __forceinline__ void load(int r0, int k0) {
     const int kk = threadIdx.x % BK, rb = threadIdx.x / BK;
     const int j = k0 + kk;
@@ -1925,6 +1943,7 @@ struct LoadIm2colT {
   int dyo[RPT], dxo[RPT];
   int next_k = -1, b = 0, oy = 0, ox = 0;
   float reg[RPT];
+  __device__ __forceinline__ void prep(int) {}
   __device__ __forceinline__ void init(int n0) {
     const int rb = threadIdx.x / BK;
     const int kk = g.kh * g.kw;
