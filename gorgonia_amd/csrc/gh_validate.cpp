@@ -163,6 +163,8 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (!c.ptr[0] || !c.ptr[1]) return bad("null operand");
       if (fn >= GH_SOLVER_RMSPROP && !c.ptr[2]) return bad("solver cache is null");
       if (fn == GH_SOLVER_ADAM && !c.ptr[3]) return bad("Adam second-moment cache is null");
+      if (c.ptr[4] && fn != GH_SOLVER_ADAM) return bad("only Adam takes bias corrections");
+      if (c.ptr[4] & (dt == GH_F64 ? 7 : 3)) return bad("Adam bias corrections must be aligned to their type");
       if (c.dim[0] < 0) return bad("negative size");
       if (dt > GH_F64) return bad("Unsupported Dtype");
       return GH_OK;

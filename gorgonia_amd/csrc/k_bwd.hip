@@ -404,7 +404,11 @@ struct SolverBatch {
 };
 
 template <int KIND>
-__global__ __launch_bounds__(kBlock) void k_solver_step(SolverBatch sb, int use, SolverPar p) {
+__global__ __launch_bounds__(kBlock) void k_solver_step(SolverBatch sb, int use, SolverPar p,
+                                                        const float* __restrict__ corr) {
+  // Adam's two bias corrections from device memory when the command names it: they change
+  // every step, and as command constants they would make every step a new command
+  if (KIND == GH_SOLVER_ADAM && corr) { p.corr1 = corr[0]; p.corr2 = corr[1]; }
   int t = 0;
 #pragma unroll
   for (int q = 1; q < kSolverBatch; q++)
@@ -618,7 +622,7 @@ int gh_solver_run_length(const gh_cmd* cmds, int n) {
   if (gh_dtype_of(cmds[0].flags) == GH_F64) return 1;   // float64 steps go one tensor per launch
   int len = 1;
   while (len < n && len < kSolverBatch && cmds[len].opcode == GH_OP_SOLVER_STEP && cmds[len].flags == cmds[0].flags &&
-         memcmp(cmds[len].f, cmds[0].f, sizeof(cmds[0].f)) == 0) {
+         cmds[len].ptr[4] == cmds[0].ptr[4] && memcmp(cmds[len].f, cmds[0].f, sizeof(cmds[0].f)) == 0) {
     // a tensor stepped twice keeps its two steps in order: the run ends before the repeat
     bool repeat = false;
     for (int j = 0; j < len; j++) repeat = repeat || cmds[j].ptr[0] == cmds[len].ptr[0];
@@ -653,12 +657,13 @@ int gh_launch_solver_steps(gh_ctx* ctx, const gh_cmd* cmds, int count) {
   for (int i = nt; i <= kSolverBatch; i++) sb.first[i] = blocks_total;
   sb.count = nt;
   const dim3 grid(blocks_total), block(kBlock);
+  const float* corr = (const float*)(uintptr_t)c.ptr[4];
   if (kind == GH_SOLVER_VANILLA)
-    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_VANILLA>), grid, block, 0, ctx->stream, sb, use, p);
+    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_VANILLA>), grid, block, 0, ctx->stream, sb, use, p, corr);
   else if (kind == GH_SOLVER_RMSPROP)
-    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_RMSPROP>), grid, block, 0, ctx->stream, sb, use, p);
+    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_RMSPROP>), grid, block, 0, ctx->stream, sb, use, p, corr);
   else
-    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_ADAM>), grid, block, 0, ctx->stream, sb, use, p);
+    hipLaunchKernelGGL((k_solver_step<GH_SOLVER_ADAM>), grid, block, 0, ctx->stream, sb, use, p, corr);
   return gh_check_hip(ctx, hipGetLastError(), "solver step launch");
 }
 

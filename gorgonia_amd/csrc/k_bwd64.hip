@@ -226,7 +226,9 @@ __device__ __forceinline__ double prep_grad(double g, double w, int use, const S
 template <int KIND>
 __global__ __launch_bounds__(kBlock) void k_solver_step_f64(double* __restrict__ w, const double* __restrict__ g,
                                                             double* __restrict__ c1, double* __restrict__ c2,
-                                                            int64_t n, int use, SolverPar64 p) {
+                                                            int64_t n, int use, SolverPar64 p,
+                                                            const double* __restrict__ corr) {
+  if (KIND == GH_SOLVER_ADAM && corr) { p.corr1 = corr[0]; p.corr2 = corr[1]; }   // see k_solver_step
   const double neg_eta = -p.eta;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
     if (KIND == GH_SOLVER_VANILLA) {
@@ -361,11 +363,12 @@ int gh_launch_solver_step_f64(gh_ctx* ctx, const gh_cmd& c) {
   double* c1 = (double*)(uintptr_t)c.ptr[2];
   double* c2 = (double*)(uintptr_t)c.ptr[3];
   const dim3 grid(blocks_for(ctx, n)), block(kBlock);
+  const double* corr = (const double*)(uintptr_t)c.ptr[4];
   if (kind == GH_SOLVER_VANILLA)
-    hipLaunchKernelGGL((k_solver_step_f64<GH_SOLVER_VANILLA>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p);
+    hipLaunchKernelGGL((k_solver_step_f64<GH_SOLVER_VANILLA>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p, corr);
   else if (kind == GH_SOLVER_RMSPROP)
-    hipLaunchKernelGGL((k_solver_step_f64<GH_SOLVER_RMSPROP>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p);
+    hipLaunchKernelGGL((k_solver_step_f64<GH_SOLVER_RMSPROP>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p, corr);
   else
-    hipLaunchKernelGGL((k_solver_step_f64<GH_SOLVER_ADAM>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p);
+    hipLaunchKernelGGL((k_solver_step_f64<GH_SOLVER_ADAM>), grid, block, 0, ctx->stream, w, g, c1, c2, n, use, p, corr);
   return gh_check_hip(ctx, hipGetLastError(), "solver step launch");
 }

@@ -240,21 +240,34 @@ def Set(a, b):
     return a.g.apply(K_SET, [a, b])
 
 
+def AdamCorrections(iteration, beta1=0.9, beta2=0.999, dtype=np.float32):
+    """The two bias corrections of an Adam step, 1/(1 - beta^t), rounded to the weights' type the
+    way the reference rounds them (solvers.go:780-870): the value to bind (Let) before each run
+    to the `corrections` input of SolverStep("adam", ...)."""
+    f = np.dtype(dtype).type
+    return np.array([f(1) / f(1 - beta1 ** iteration), f(1) / f(1 - beta2 ** iteration)], dtype=dtype)
+
+
 def SolverStep(kind, weights, grad, caches=(), eta=0.001, eps=1e-8, l1reg=0.0, l2reg=0.0, clip=0.0, batch=1.0,
-               decay=0.999, beta1=0.9, beta2=0.999, iteration=1):
+               decay=0.999, beta1=0.9, beta2=0.999, iteration=1, corrections=None):
     """One Step of NewVanillaSolver / NewRMSPropSolver / NewAdamSolver (solvers.go) on one
     weight tensor, on the device: the weights (a resident input) and the solver's caches
     (resident inputs, zero at the start) are updated in place.  The constants are
     rounded to the weights' type the way the reference rounds them (float64 weights keep
-    them in double); Adam's bias corrections depend on `iteration`, so an Adam step is a
-    new command every run."""
+    them in double).  Adam's bias corrections depend on the iteration: given as `iteration`
+    they are constants of the command (one graph per step); given as `corrections` - an input
+    node holding AdamCorrections(t), rebound before each run - they are read from memory and
+    the same command, and the same captured segment, serves every step."""
     f = np.float64 if getattr(weights, "dtype", None) == np.float64 else np.float32
     a, b = (f(decay), f(1.0 - decay)) if kind == "rmsprop" else (f(beta1), f(beta2))
     fs = [f(eta), f(eps), f(l1reg), f(l2reg), f(clip), f(1) / f(batch), a, b,
           f(1) / f(1 - beta1 ** iteration), f(1) / f(1 - beta2 ** iteration)]
     use = (1 if l1reg else 0) | (2 if l2reg else 0) | (4 if clip else 0) | (8 if batch > 1 else 0)
     fn = {"vanilla": 0, "rmsprop": 1, "adam": 2}[kind]
-    return weights.g.apply(K_SOLVER, [weights, grad] + list(caches), fn=fn, ints=[use], fs=fs)
+    extra = [corrections] if corrections is not None else []
+    if extra and kind != "adam":
+        raise EngineError(1, "only Adam takes bias corrections")
+    return weights.g.apply(K_SOLVER, [weights, grad] + list(caches) + extra, fn=fn, ints=[use], fs=fs)
 
 
 def RandUniform(g, shape, seed, offset=0, counter=None):

@@ -215,9 +215,12 @@ Status InferShape(const OpSpec& op, const std::vector<const Shape*>& in, Shape* 
       return Status::OK();
     case OpKind::SolverStep: {
       if (op.fn < 0 || op.fn >= GH_SOLVER__COUNT) return bad("SolverStep: unknown solver");
-      if (in.size() != (size_t)(2 + op.fn)) return bad("SolverStep: weights, grad and the solver's caches expected");
-      for (size_t i = 1; i < in.size(); i++)
+      // Adam may take one more input: its two bias corrections as a tensor (a new value every step)
+      const bool corr = op.fn == GH_SOLVER_ADAM && in.size() == 5;
+      if (in.size() != (size_t)(2 + op.fn) && !corr) return bad("SolverStep: weights, grad and the solver's caches expected");
+      for (size_t i = 1; i < (size_t)(2 + op.fn); i++)
         if (in[i]->TotalSize() != in[0]->TotalSize()) return bad("SolverStep: sizes differ");
+      if (corr && in[4]->TotalSize() != 2) return bad("SolverStep: the bias corrections are two values");
       if (op.fs.size() < 10 || op.ints.empty()) return bad("SolverStep: constants missing");
       *out = *in[0];
       return Status::OK();
@@ -522,7 +525,7 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       for (size_t i = 0; i < in.size(); i++)
         if (in[i]->dt == Dtype::Other || in[i]->dt != in[0]->dt) return bad("SolverStep: Unsupported Dtype");
       c.flags = GH_FLAG_FN(op.fn) | GH_FLAG_MODE(op.ints[0]) | dtype_flag(in[0]->dt);
-      for (size_t i = 0; i < in.size(); i++) c.ptr[i] = in[i]->mem;
+      for (size_t i = 0; i < in.size(); i++) c.ptr[i] = in[i]->mem;   // Adam: in[4] = bias corrections in memory
       c.dim[0] = in[0]->DataSize();
       for (int i = 0; i < 10; i++) c.f[i] = (float)op.fs[(size_t)i];
       if (in[0]->dt == Dtype::Float64)   // float64 tensors take the constants as doubles

@@ -212,6 +212,10 @@ enum gh_unaryfn {
  *             dim[0]=n ; flags: FN = gh_solver, MODE = use mask (1 l1reg, 2 l2reg, 4 clip,
  *             8 batch) ; f[0]=eta f[1]=eps f[2]=l1reg f[3]=l2reg f[4]=clip f[5]=1/batch
  *             f[6]=decay|beta1 f[7]=(1-decay)|beta2 f[8]=1/(1-beta1^t) f[9]=1/(1-beta2^t).
+ *             Adam only: [ptr[4]=two values of the weights' type in device memory (or pinned
+ *             host memory) that replace f[8], f[9] when the step runs] - the bias corrections
+ *             change every iteration, and read from memory they leave the command, and with
+ *             it a captured segment, unchanged from step to step.
  *             Weights and caches are updated in place with the reference's sequence of
  *             tensor ops, one rounding each; grad is left untouched (the reference zeroes it)
  */

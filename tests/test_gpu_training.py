@@ -5,7 +5,7 @@ gradient; every kernel on the way has its own tighter test)."""
 import numpy as np
 import pytest
 
-from gorgonia_amd import configs, graph as G
+from gorgonia_amd import configs, graph as G, synth
 from oracle import forward as F
 from tests.util import assert_bits_equal, rel_frobenius
 
@@ -102,4 +102,40 @@ def test_set_updates_a_resident_input_in_place(ctx):
     for k in range(1, 4):
         m.RunAll()
         assert_bits_equal(out, np.arange(8, dtype=np.float32) + k, f"after {k} runs")
+    m.Close()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_adam_steps_replay_with_corrections_from_memory(ctx, dtype):
+    """Adam's bias corrections change every iteration.  Bound as an input that the host rebinds
+    before each run they are read from memory, so the step is the same command every time: the
+    segment is captured once and replayed, and weights and both caches follow the oracle's
+    iterations bit for bit (as command constants every step would be a new command)."""
+    from oracle import binding as O
+    n = 5000
+    w0 = synth.normal(61, (n,)).astype(dtype)
+    grads = [synth.normal(70 + t, (n,), 0.0, 2.0).astype(dtype) for t in range(6)]
+    g = G.NewGraph()
+    w = G.NewTensor(g, w0.copy(), resident=True)
+    m1 = G.NewTensor(g, np.zeros(n, dtype), resident=True)
+    m2 = G.NewTensor(g, np.zeros(n, dtype), resident=True)
+    grad = G.NewTensor(g, grads[0])
+    corr = G.NewTensor(g, G.AdamCorrections(1, dtype=dtype))
+    # enough small operators in front of the step that the segment is worth a graph
+    gg = grad
+    for _ in range(4):
+        gg = G.Neg(G.Neg(gg))
+    out = G.Read(G.SolverStep("adam", w, gg, (m1, m2), eta=0.01, l2reg=1e-4, clip=3.0, corrections=corr))
+    r1, r2 = G.Read(m1), G.Read(m2)
+    m = G.NewTapeMachine(g, graph_replay=True)
+    want_w, c1, c2 = w0.copy(), np.zeros(n, dtype), np.zeros(n, dtype)
+    for t in range(6):
+        G.Let(grad, grads[t])
+        G.Let(corr, G.AdamCorrections(t + 1, dtype=dtype))
+        m.RunAll()
+        want_w, _, c1, c2 = O.solver_step("adam", want_w, grads[t], c1, c2, eta=0.01, l2reg=1e-4, clip=3.0, iteration=t + 1)
+        assert_bits_equal(out, want_w, f"adam weights, iteration {t + 1}")
+        assert_bits_equal(r1, c1, f"adam m, iteration {t + 1}")
+        assert_bits_equal(r2, c2, f"adam v, iteration {t + 1}")
+    assert m.graph_launches() >= 4, "the step did not stay the same command"
     m.Close()
