@@ -2,11 +2,21 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "gh_internal.h"
 
 // Epilogue activations in the reference's arithmetic form (nn.go:83-163).
+// act 3 is LeakyRelu for a finite alpha >= 0 in four instructions instead of eight, with the
+// same bits: for v < 0 the reference's sum is -0 + v alpha = v alpha, for v >= 0 it is v + 0 = v,
+// and the v * 0 that fmaf adds is a zero of v's sign (which changes neither) unless v is
+// infinite or NaN, where it makes the NaN the reference's inf * 0 makes.
 __device__ __forceinline__ float act_apply(float v, int act, float alpha) {
   if (act == 1) return v * (v >= 0.0f ? 1.0f : 0.0f);
+  if (act == 3) {
+    const float na = v * alpha;
+    return __builtin_fmaf(v, 0.0f, v < 0.0f ? na : v);
+  }
   if (act == 2) {
     const float pos = v * (v >= 0.0f ? 1.0f : 0.0f);
     const float neg = v * (v < 0.0f ? 1.0f : 0.0f);
@@ -40,13 +50,16 @@ __device__ __forceinline__ float tail_apply(const ConvTail& t, int f, float v) {
 // The same arithmetic with the per-filter BatchNorm constants taken from a table a
 // workgroup fills once (conv_tail_table): a and b are rounded exactly as above, so the
 // stored bits are those of tail_apply.  tab = [4][n]: a, b, gamma, beta.
+// An absent gamma is stored as 1 and an absent beta as -0: multiplying by 1 and adding -0
+// leave every float32 as it is (+0 + -0 = +0, -0 + -0 = -0), so a kernel may apply all four
+// steps without asking which exist (tail_apply_fixed) and still store tail_apply's bits.
 __device__ __forceinline__ void conv_tail_table(const ConvTail& t, float* tab, int n, int i, int f) {
   if (!t.mean) return;
   const float a = 1.0f / sqrtf(t.var[f] + t.eps);
   tab[i] = a;
   tab[n + i] = -t.mean[f] * a;
-  if (t.gamma) tab[2 * n + i] = t.gamma[f];
-  if (t.beta) tab[3 * n + i] = t.beta[f];
+  tab[2 * n + i] = t.gamma ? t.gamma[f] : 1.0f;
+  tab[3 * n + i] = t.beta ? t.beta[f] : -0.0f;
 }
 __device__ __forceinline__ float tail_apply_table(const ConvTail& t, const float* tab, int n, int i, float v) {
   if (t.mean) {
@@ -56,6 +69,33 @@ __device__ __forceinline__ float tail_apply_table(const ConvTail& t, const float
     if (t.beta) v = v + tab[3 * n + i];
   }
   return act_apply(v, t.act, t.alpha);
+}
+
+// The epilogue with what it consists of fixed at compile time (BN: BatchNorm from a
+// conv_tail_table; ACT: 0 none, 1 Rectify, 2 LeakyRelu, 3 its short form): no branch per stored value.  Scalar
+// branches inside an epilogue's value loops were a fifth of a small convolution's run.
+template <bool BN, int ACT>
+__device__ __forceinline__ float tail_apply_fixed(const float* tab, int n, int i, float v, float alpha) {
+  if constexpr (BN) {
+    v = v * tab[i];
+    v = v + tab[n + i];
+    v = tab[2 * n + i] * v;
+    v = v + tab[3 * n + i];
+  }
+  return act_apply(v, ACT, alpha);
+}
+// Calls body(bool_constant<BN>, integral_constant<int, ACT>) for the tail's combination.
+template <class Body>
+__device__ __forceinline__ void conv_tail_dispatch(const ConvTail& t, Body&& body) {
+  using T = std::true_type; using F = std::false_type;
+  using A0 = std::integral_constant<int, 0>; using A1 = std::integral_constant<int, 1>;
+  using A2 = std::integral_constant<int, 2>; using A3 = std::integral_constant<int, 3>;
+  const bool quick_leaky = t.act == 2 && t.alpha >= 0.0f && t.alpha <= 3.402823466e+38f;
+  if (t.mean) {
+    if (t.act == 1) body(T{}, A1{}); else if (quick_leaky) body(T{}, A3{}); else if (t.act == 2) body(T{}, A2{}); else body(T{}, A0{});
+  } else {
+    if (t.act == 1) body(F{}, A1{}); else if (quick_leaky) body(F{}, A3{}); else if (t.act == 2) body(F{}, A2{}); else body(F{}, A0{});
+  }
 }
 
 inline ConvTail conv_tail(const gh_cmd& c) {

@@ -207,60 +207,71 @@ __global__ __launch_bounds__(kWaves * 64) void k_conv3x3_patch(const float* __re
   }
   __syncthreads();
 
-  // ---- sum the four slots in order, epilogue, store: an item is four filters of one result column
-  if (g.pool) {
-    const int npool = g.npix >> 2;
-    const int nitems = (BM / 4) * npool;
-    const int pplane = g.ph * g.pw;
-    for (int it = tid; it < nitems; it += NTH) {
-      const int mg = mdiv(it, g.mNPOOL), q = it - mg * npool;
-      const int py = mdiv(q, g.mHTW), px = q - py * g.HTW;
-      const int oy = (oy0 >> 1) + py, ox = (ox0 >> 1) + px;
-      if (oy >= g.ph || ox >= g.pw) continue;
-      const int mf = m0 + 4 * mg;
-      const float* rp = R + (4 * q) * MP + 4 * mg;
-      f32x4 best = {-3.402823466e+38f, -3.402823466e+38f, -3.402823466e+38f, -3.402823466e+38f};
+  // ---- sum the four slots in order, epilogue, store: an item is four filters of one result
+  // column.  What the epilogue consists of is uniform over the launch, so the item loops are
+  // compiled once per combination and the combination chosen once, outside them.
+  const float alpha = tail.alpha;
+  auto items = [&](auto bn_c, auto act_c, auto all_c) {
+    constexpr bool BN = decltype(bn_c)::value;
+    constexpr int ACT = decltype(act_c)::value;
+    constexpr bool ALL4 = decltype(all_c)::value;   // every item's four filters exist
+    if (g.pool) {
+      const int npool = g.npix >> 2;
+      const int nitems = (BM / 4) * npool;
+      const int pplane = g.ph * g.pw;
+      for (int it = tid; it < nitems; it += NTH) {
+        const int mg = mdiv(it, g.mNPOOL), q = it - mg * npool;
+        const int py = mdiv(q, g.mHTW), px = q - py * g.HTW;
+        const int oy = (oy0 >> 1) + py, ox = (ox0 >> 1) + px;
+        if (oy >= g.ph || ox >= g.pw) continue;
+        const int mf = m0 + 4 * mg;
+        const float* rp = R + (4 * q) * MP + 4 * mg;
+        f32x4 best = {-3.402823466e+38f, -3.402823466e+38f, -3.402823466e+38f, -3.402823466e+38f};
 #pragma unroll
-      for (int i = 0; i < 4; i++) {   // window positions in scan order
-        const f32x4 s0 = *reinterpret_cast<const f32x4*>(rp + i * MP);
-        const f32x4 s1 = *reinterpret_cast<const f32x4*>(rp + i * MP + RW);
-        const f32x4 s2 = *reinterpret_cast<const f32x4*>(rp + i * MP + 2 * RW);
-        const f32x4 s3 = *reinterpret_cast<const f32x4*>(rp + i * MP + 3 * RW);
-        const f32x4 s = ((s0 + s1) + s2) + s3;
+        for (int i = 0; i < 4; i++) {   // window positions in scan order
+          const f32x4 s0 = *reinterpret_cast<const f32x4*>(rp + i * MP);
+          const f32x4 s1 = *reinterpret_cast<const f32x4*>(rp + i * MP + RW);
+          const f32x4 s2 = *reinterpret_cast<const f32x4*>(rp + i * MP + 2 * RW);
+          const f32x4 s3 = *reinterpret_cast<const f32x4*>(rp + i * MP + 3 * RW);
+          const f32x4 s = ((s0 + s1) + s2) + s3;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-          if (mf + j < g.F) {
-            const float v = tail_apply_table(tail, ftab, BM, 4 * mg + j, s[j]);
+          for (int j = 0; j < 4; j++) {
+            // a filter beyond F reads the last filter's table row and is never stored
+            const float v = tail_apply_fixed<BN, ACT>(ftab, BM, 4 * mg + j, s[j], alpha);
             if (v > best[j]) best[j] = v;
           }
         }
+        float* yp = y + ((int64_t)bimg * g.F + mf) * pplane + oy * g.pw + ox;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          if (ALL4 || mf + j < g.F) yp[(int64_t)j * pplane] = best[j];
       }
-      float* yp = y + ((int64_t)bimg * g.F + mf) * pplane + oy * g.pw + ox;
+    } else {
+      const int nitems = (BM / 4) * g.npix;
+      const int plane = g.oh * g.ow;
+      for (int it = tid; it < nitems; it += NTH) {
+        const int mg = mdiv(it, g.mNPIX), q = it - mg * g.npix;
+        const int ty = mdiv(q, g.mTW), tx = q - ty * g.TW;
+        const int oy = oy0 + ty, ox = ox0 + tx;
+        if (oy >= g.oh || ox >= g.ow) continue;
+        const int mf = m0 + 4 * mg;
+        const float* rp = R + q * MP + 4 * mg;
+        const f32x4 s0 = *reinterpret_cast<const f32x4*>(rp);
+        const f32x4 s1 = *reinterpret_cast<const f32x4*>(rp + RW);
+        const f32x4 s2 = *reinterpret_cast<const f32x4*>(rp + 2 * RW);
+        const f32x4 s3 = *reinterpret_cast<const f32x4*>(rp + 3 * RW);
+        const f32x4 s = ((s0 + s1) + s2) + s3;
+        float* yp = y + ((int64_t)bimg * g.F + mf) * plane + oy * g.ow + ox;
 #pragma unroll
-      for (int j = 0; j < 4; j++)
-        if (mf + j < g.F) yp[(int64_t)j * pplane] = best[j];
+        for (int j = 0; j < 4; j++)
+          if (ALL4 || mf + j < g.F) yp[(int64_t)j * plane] = tail_apply_fixed<BN, ACT>(ftab, BM, 4 * mg + j, s[j], alpha);
+      }
     }
-  } else {
-    const int nitems = (BM / 4) * g.npix;
-    const int plane = g.oh * g.ow;
-    for (int it = tid; it < nitems; it += NTH) {
-      const int mg = mdiv(it, g.mNPIX), q = it - mg * g.npix;
-      const int ty = mdiv(q, g.mTW), tx = q - ty * g.TW;
-      const int oy = oy0 + ty, ox = ox0 + tx;
-      if (oy >= g.oh || ox >= g.ow) continue;
-      const int mf = m0 + 4 * mg;
-      const float* rp = R + q * MP + 4 * mg;
-      const f32x4 s0 = *reinterpret_cast<const f32x4*>(rp);
-      const f32x4 s1 = *reinterpret_cast<const f32x4*>(rp + RW);
-      const f32x4 s2 = *reinterpret_cast<const f32x4*>(rp + 2 * RW);
-      const f32x4 s3 = *reinterpret_cast<const f32x4*>(rp + 3 * RW);
-      const f32x4 s = ((s0 + s1) + s2) + s3;
-      float* yp = y + ((int64_t)bimg * g.F + mf) * plane + oy * g.ow + ox;
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        if (mf + j < g.F) yp[(int64_t)j * plane] = tail_apply_table(tail, ftab, BM, 4 * mg + j, s[j]);
-    }
-  }
+  };
+  const bool all4 = m0 + BM <= g.F;
+  conv_tail_dispatch(tail, [&](auto bn_c, auto act_c) {
+    if (all4) items(bn_c, act_c, std::true_type{}); else items(bn_c, act_c, std::false_type{});
+  });
 }
 
 struct PatchPlan {

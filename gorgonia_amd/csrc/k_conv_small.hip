@@ -252,52 +252,64 @@ __global__ __launch_bounds__(WV * 64) void k_conv3x3_small(const float* __restri
   }
   __syncthreads();
 
-  // ---- sum the four slots in order, epilogue, store: an item is four filters of one result column
+  // ---- sum the four slots in order, epilogue, store: an item is four filters of one result
+  // column.  What the epilogue consists of is uniform over the launch, so the item loop is
+  // compiled once per combination and the combination chosen once, outside the loop.
   const int nitems = (BM / 4) * g.nout;
-  for (int it = tid; it < nitems; it += NTH) {
-    const int mg = mdiv(it, g.mNOUT), q = it - mg * g.nout;
-    const int mf = m0 + 4 * mg;
-    if (g.pool) {
-      const int pq = g.ph * g.pw;
-      const int img = mdiv(q, g.mPQ), qq = q - img * pq;
-      if (img >= nimg) continue;
-      const float* rp = R + (4 * q) * MP + 4 * mg;
-      f32x4 best = {-3.402823466e+38f, -3.402823466e+38f, -3.402823466e+38f, -3.402823466e+38f};
+  const float alpha = tail.alpha;
+  auto items = [&](auto bn_c, auto act_c, auto all_c) {
+    constexpr bool BN = decltype(bn_c)::value;
+    constexpr int ACT = decltype(act_c)::value;
+    constexpr bool ALL4 = decltype(all_c)::value;   // every item's four filters exist
+    for (int it = tid; it < nitems; it += NTH) {
+      const int mg = mdiv(it, g.mNOUT), q = it - mg * g.nout;
+      const int mf = m0 + 4 * mg;
+      const int nf = ALL4 ? 4 : g.F - mf;
+      if (g.pool) {
+        const int pq = g.ph * g.pw;
+        const int img = mdiv(q, g.mPQ), qq = q - img * pq;
+        if (img >= nimg) continue;
+        const float* rp = R + (4 * q) * MP + 4 * mg;
+        f32x4 best = {-3.402823466e+38f, -3.402823466e+38f, -3.402823466e+38f, -3.402823466e+38f};
 #pragma unroll
-      for (int i = 0; i < 4; i++) {   // window positions in scan order
-        const f32x4 s0 = *reinterpret_cast<const f32x4*>(rp + i * MP);
-        const f32x4 s1 = *reinterpret_cast<const f32x4*>(rp + i * MP + RW);
-        const f32x4 s2 = *reinterpret_cast<const f32x4*>(rp + i * MP + 2 * RW);
-        const f32x4 s3 = *reinterpret_cast<const f32x4*>(rp + i * MP + 3 * RW);
-        const f32x4 s = ((s0 + s1) + s2) + s3;
+        for (int i = 0; i < 4; i++) {   // window positions in scan order
+          const f32x4 s0 = *reinterpret_cast<const f32x4*>(rp + i * MP);
+          const f32x4 s1 = *reinterpret_cast<const f32x4*>(rp + i * MP + RW);
+          const f32x4 s2 = *reinterpret_cast<const f32x4*>(rp + i * MP + 2 * RW);
+          const f32x4 s3 = *reinterpret_cast<const f32x4*>(rp + i * MP + 3 * RW);
+          const f32x4 s = ((s0 + s1) + s2) + s3;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-          if (mf + j < g.F) {
-            const float v = tail_apply_table(tail, ftab, BM, 4 * mg + j, s[j]);
+          for (int j = 0; j < 4; j++) {
+            // a filter beyond F reads a table row of the last filter and is never stored
+            const float v = tail_apply_fixed<BN, ACT>(ftab, BM, 4 * mg + j, s[j], alpha);
             if (v > best[j]) best[j] = v;
           }
         }
+        float* yp = y + ((int64_t)(b0 + img) * g.F + mf) * pq + qq;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          if (ALL4 || j < nf) yp[j * pq] = best[j];
+      } else {
+        const int plane = g.oh * g.ow;
+        const int img = mdiv(q, g.mPPI), r = q - img * plane;
+        if (img >= nimg) continue;
+        const float* rp = R + q * MP + 4 * mg;
+        const f32x4 s0 = *reinterpret_cast<const f32x4*>(rp);
+        const f32x4 s1 = *reinterpret_cast<const f32x4*>(rp + RW);
+        const f32x4 s2 = *reinterpret_cast<const f32x4*>(rp + 2 * RW);
+        const f32x4 s3 = *reinterpret_cast<const f32x4*>(rp + 3 * RW);
+        const f32x4 s = ((s0 + s1) + s2) + s3;
+        float* yp = y + ((int64_t)(b0 + img) * g.F + mf) * plane + r;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          if (ALL4 || j < nf) yp[j * plane] = tail_apply_fixed<BN, ACT>(ftab, BM, 4 * mg + j, s[j], alpha);
       }
-      float* yp = y + ((int64_t)(b0 + img) * g.F + mf) * pq + qq;
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        if (mf + j < g.F) yp[j * pq] = best[j];
-    } else {
-      const int plane = g.oh * g.ow;
-      const int img = mdiv(q, g.mPPI), r = q - img * plane;
-      if (img >= nimg) continue;
-      const float* rp = R + q * MP + 4 * mg;
-      const f32x4 s0 = *reinterpret_cast<const f32x4*>(rp);
-      const f32x4 s1 = *reinterpret_cast<const f32x4*>(rp + RW);
-      const f32x4 s2 = *reinterpret_cast<const f32x4*>(rp + 2 * RW);
-      const f32x4 s3 = *reinterpret_cast<const f32x4*>(rp + 3 * RW);
-      const f32x4 s = ((s0 + s1) + s2) + s3;
-      float* yp = y + ((int64_t)(b0 + img) * g.F + mf) * plane + r;
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        if (mf + j < g.F) yp[j * plane] = tail_apply_table(tail, ftab, BM, 4 * mg + j, s[j]);
     }
-  }
+  };
+  const bool all4 = m0 + BM <= g.F;
+  conv_tail_dispatch(tail, [&](auto bn_c, auto act_c) {
+    if (all4) items(bn_c, act_c, std::true_type{}); else items(bn_c, act_c, std::false_type{});
+  });
 }
 
 struct SmallPlan {

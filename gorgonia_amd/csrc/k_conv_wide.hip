@@ -53,10 +53,10 @@ struct WideGeom {
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
 
-// value of lane (l & ~3) + I, for every lane l: a 2x2 window's position I
-template <int I>
-__device__ __forceinline__ float quad_bcast(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), I * 0x55, 0xf, 0xf, true));
+// A 2x2 window's four positions sit in the four lanes of a quad, in scan order.
+template <int A, int B, int C, int D>
+__device__ __forceinline__ float quad_perm(float v) {   // lane i of each quad reads lane (A,B,C,D)[i] of it
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), A | (B << 2) | (C << 4) | (D << 6), 0xf, 0xf, true));
 }
 
 // XS: patch cells each thread stages per tile (4 NQ PP <= XS * kThreads); DB: two patch buffers.
@@ -257,6 +257,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
     // ---- epilogue from the accumulators: register v of acc[a][t] is filter m0 + 16 a + 4 lk + v
     // at N entry n0 + 16 t + li
     {
+      // The lane's coordinates pass through an empty asm here, so that what the epilogue derives
+      // from them is computed per tile and does not sit in registers through the MFMA loop.
+      int eli = li, elk = lk;
+      asm volatile("" : "+v"(eli), "+v"(elk));
       const int bimg = mdiv(tile, g.mTXY);
       const int trem = tile - bimg * (g.tiles_x * g.tiles_y);
       const int tyi = mdiv(trem, g.mTX), txi = trem - tyi * g.tiles_x;
@@ -266,7 +270,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
       const int plane = g.pool ? g.ph * g.pw : g.oh * g.ow;
 #pragma unroll
       for (int t = 0; t < TN; t++) {
-        const int n = n0 + 16 * t + li;
+        const int n = n0 + 16 * t + eli;
         if (g.pool) {
           const int q = n >> 2;
           const int py = mdiv(q, g.mHTW), px = q - py * g.HTW;
@@ -282,57 +286,78 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
       char* const ytile = reinterpret_cast<char*>(y + ((int64_t)bimg * g.F + m0) * plane);
       const unsigned pbytes = 4u * (unsigned)plane;
       const bool all4 = (g.F & 3) == 0;   // then a lane's four filters exist or not together
+      const float alpha = tail.alpha;
+      // What the epilogue consists of is uniform over the launch: the value loops are compiled
+      // once per combination and the combination is chosen once per tile, not once per value.
+      auto values = [&](auto bn_c, auto act_c, auto pool_c) {
+        constexpr bool BN = decltype(bn_c)::value;
+        constexpr int ACT = decltype(act_c)::value;
+        constexpr bool POOL = decltype(pool_c)::value;
 #pragma unroll
-      for (int a = 0; a < TM; a++) {
-        // BatchNorm constants of this lane's filters 16 a + 4 lk + (0..3): one 128-bit read each
-        const float* const fp = ftab + 16 * a + 4 * lk;
-        f32x4 ca = {0.f, 0.f, 0.f, 0.f}, cb = ca, cg = ca, ce = ca;
-        if (tail.mean) {
-          ca = *reinterpret_cast<const f32x4*>(fp);
-          cb = *reinterpret_cast<const f32x4*>(fp + BM);
-          if (tail.gamma) cg = *reinterpret_cast<const f32x4*>(fp + 2 * BM);
-          if (tail.beta) ce = *reinterpret_cast<const f32x4*>(fp + 3 * BM);
-        }
-        const int fl = 16 * a + 4 * lk;              // first of the lane's four filters, inside the tile
-        const int nf = min(max(g.F - (m0 + fl), 0), 4);   // how many of them exist
+        for (int a = 0; a < TM; a++) {
+          // BatchNorm constants of this lane's filters 16 a + 4 lk + (0..3): one 128-bit read
+          // each; an absent gamma is 1 and an absent beta -0 in the table, which change no bits
+          const float* const fp = ftab + 16 * a + 4 * elk;
+          if constexpr (BN) {   // two constants at a time, so that eight registers hold them, not sixteen
+            const f32x4 ca = *reinterpret_cast<const f32x4*>(fp);
+            const f32x4 cb = *reinterpret_cast<const f32x4*>(fp + BM);
 #pragma unroll
-        for (int t = 0; t < TN; t++) {
-          unsigned off = (unsigned)fl * pbytes + 4u * (unsigned)max(yoff[t], 0);
-          const bool live = yoff[t] >= 0 && nf > 0;
-          float res[4];
+            for (int t = 0; t < TN; t++)
 #pragma unroll
-          for (int v = 0; v < 4; v++) {
-            float val = acc[a][t][v];
-            if (tail.mean) {
-              val = val * ca[v];
-              val = val + cb[v];
-              if (tail.gamma) val = cg[v] * val;
-              if (tail.beta) val = val + ce[v];
-            }
-            val = act_apply(val, tail.act, tail.alpha);
-            if (g.pool) {
-              float best = -3.402823466e+38f;
-              const float v0 = quad_bcast<0>(val), v1 = quad_bcast<1>(val), v2 = quad_bcast<2>(val), v3 = quad_bcast<3>(val);
-              if (v0 > best) best = v0;   // window positions in scan order
-              if (v1 > best) best = v1;
-              if (v2 > best) best = v2;
-              if (v3 > best) best = v3;
-              val = best;
-            }
-            res[v] = val;
+              for (int v = 0; v < 4; v++) {
+                acc[a][t][v] = acc[a][t][v] * ca[v];
+                acc[a][t][v] = acc[a][t][v] + cb[v];
+              }
+            const f32x4 cg = *reinterpret_cast<const f32x4*>(fp + 2 * BM);
+            const f32x4 ce = *reinterpret_cast<const f32x4*>(fp + 3 * BM);
+#pragma unroll
+            for (int t = 0; t < TN; t++)
+#pragma unroll
+              for (int v = 0; v < 4; v++) {
+                acc[a][t][v] = cg[v] * acc[a][t][v];
+                acc[a][t][v] = acc[a][t][v] + ce[v];
+              }
           }
-          if (all4) {
-            if (live) {   // one test for the four stores
+          const int fl = 16 * a + 4 * elk;             // first of the lane's four filters, inside the tile
+          const int nf = min(max(g.F - (m0 + fl), 0), 4);   // how many of them exist
 #pragma unroll
-              for (int v = 0; v < 4; v++) *reinterpret_cast<float*>(ytile + (off + v * pbytes)) = res[v];
+          for (int t = 0; t < TN; t++) {
+            unsigned off = (unsigned)fl * pbytes + 4u * (unsigned)max(yoff[t], 0);
+            const bool live = yoff[t] >= 0 && nf > 0;
+            float res[4];
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+              float val = act_apply(acc[a][t][v], ACT, alpha);
+              if constexpr (POOL) {
+                // The reference scans the window in order from -FLT_MAX, taking a value only if it
+                // is greater.  The same in three steps: each lane clamps its own value the way the
+                // scan would (NaN and anything <= -FLT_MAX never enter), then a tree over the quad
+                // in which the earlier position keeps a tie (it matters between +0 and -0).  Lane
+                // 0 of the quad ends with the window's value; the others are not stored.
+                val = val > -3.402823466e+38f ? val : -3.402823466e+38f;
+                const float nb = quad_perm<1, 0, 3, 2>(val);
+                val = nb > val ? nb : val;          // lanes 0 and 2: pairs (0,1) and (2,3)
+                const float far = quad_perm<2, 3, 0, 1>(val);
+                val = far > val ? far : val;        // lane 0: the whole window
+              }
+              res[v] = val;
             }
-          } else {
+            if (all4) {
+              if (live) {   // one test for the four stores
 #pragma unroll
-            for (int v = 0; v < 4; v++)
-              if (live && v < nf) *reinterpret_cast<float*>(ytile + (off + v * pbytes)) = res[v];
+                for (int v = 0; v < 4; v++) *reinterpret_cast<float*>(ytile + (off + v * pbytes)) = res[v];
+              }
+            } else {
+#pragma unroll
+              for (int v = 0; v < 4; v++)
+                if (live && v < nf) *reinterpret_cast<float*>(ytile + (off + v * pbytes)) = res[v];
+            }
           }
         }
-      }
+      };
+      conv_tail_dispatch(tail, [&](auto bn_c, auto act_c) {
+        if (g.pool) values(bn_c, act_c, std::true_type{}); else values(bn_c, act_c, std::false_type{});
+      });
     }
     if (!more) break;
     if constexpr (DB) {
@@ -434,10 +459,12 @@ bool wide_plan(const gh_cmd& c, bool pool, WidePlan* out) {
       const int ft = (h.F + 16 * TM - 1) / (16 * TM);
       const int64_t groups = std::max<int64_t>(1, (int64_t)kDeviceCUs * occ / ft);
       const int64_t rounds = (ntiles + groups - 1) / groups;
-      // a tile's MFMA time in units of one 16x16 tile over K, shared by `occ` workgroups
-      // (operand fetches per MFMA grow as the wavefront's tile shrinks: TM + TN reads feed TM TN MFMAs)
-      const double est = (double)rounds * TM * bTN * occ * (occ == 2 ? 1.0 : db ? 1.35 : 1.45) *
-                         (1.0 + 0.12 * (TM + bTN) / (TM * bTN));
+      // A round costs a workgroup, per 16 pixels of its patch, one unit per 16 filters (MFMAs and
+      // epilogue) plus 0.85 of a unit for staging the patch, whatever the filter count: measured
+      // on 16 -> 32 channels at 208 x 208 (6.3 us a round for 32 filters, 4.1 for 16).  `occ`
+      // workgroups share a compute unit's time; alone, a workgroup's staging is not hidden.
+      const double est = (double)rounds * occ * bTN * (TM + 0.85) * (occ == 2 ? 1.0 : db ? 1.35 : 1.45) *
+                         (bTN == 2 ? 0.98 : 1.0);
       if (!found || est < best_est) {
         found = true; best_est = est;
         h.mTXY = magic_of(h.tiles_x * h.tiles_y); h.mTX = magic_of(h.tiles_x); h.mPP = magic_of(h.PP);
