@@ -196,6 +196,59 @@ def test_conv_epilogue_pool_bit_exact(ctx, cfg):
                                     pool2=True), chain, f"conv+bn+leaky+pool {cfg}")
 
 
+# one shape per convolution kernel that carries an epilogue: direct (C <= 4), small images, patches of
+# deep layers, wide images, the LDS-tiled 3x3 one, and the gather kernel (1x1)
+SPECIAL_VALUE_CASES = [(3, 1, 28, 28, 32, 3, 1), (5, 32, 14, 14, 64, 3, 1), (2, 256, 13, 13, 64, 3, 1),
+                       (2, 16, 130, 131, 32, 3, 1), (1, 64, 52, 80, 72, 3, 1), (2, 64, 13, 13, 40, 1, 0)]
+
+
+@pytest.mark.parametrize("cfg", SPECIAL_VALUE_CASES)
+def test_conv_epilogue_special_values_bit_exact(ctx, cfg):
+    """Epilogues on results that are +0, -0, infinite, NaN, tiny and huge: images with blank (+0) and -0
+    regions, a few infinities and NaNs, values near overflow, filters with zeroed taps.  The activations'
+    short forms must store what the reference's arithmetic (pos + neg * alpha on the plain result) stores
+    for every such value and every alpha sign, and pooling must keep the first of a tie between zeros."""
+    B, C, H, W, F, k, pad = cfg
+    rng = np.random.default_rng(77)
+    x = synth.uniform(71, (B, C, H, W), -1, 1)
+    x[:, :, : H // 3, :] = 0.0                       # blank rows: results exactly +0
+    x[:, :, H // 3: H // 2, : W // 2] = -0.0
+    x[0, 0, H - 2, W - 2] = np.inf
+    x[B - 1, C - 1, H // 2 + 1, 1] = -np.inf
+    x[0, C // 2, H - 3, W // 2] = np.nan
+    x[B - 1, 0, H - 1, :] *= 3e38                    # products overflow for some filters
+    x[0, 0, H // 2 + 2, :] *= 1e-38                  # denormal products
+    w = synth.he_normal(72, (F, C, k, k))
+    w[rng.integers(0, F, 8), rng.integers(0, C, 8)] = 0.0
+    w[1 % F] = -np.abs(w[1 % F])
+    plain = gpu_conv(ctx, x, w, (pad, pad), (1, 1), (1, 1))
+    assert np.isnan(plain).any() and np.isinf(plain).any() and (plain == 0).any()
+    mean, var = synth.normal(73, (F,), 0.0, 0.1), synth.uniform(74, (F,), 0.5, 1.5)
+    gamma, beta = synth.uniform(75, (F,), 0.5, 1.5), synth.normal(76, (F,), 0.0, 0.1)
+    cmd = D.cmd_conv2d(1, 1, 1, B, C, H, W, F, k, k, (pad, pad))
+    can_pool = ctx.lib.gh_conv2d_can_pool(cmd) == 1
+    relu = O.relu(plain).reshape(plain.shape)
+    assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), act="relu"), relu, f"conv+relu {cfg}")
+    if can_pool:
+        assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), act="relu", pool2=True),
+                          O.maxpool2d(relu, (2, 2), (0, 0), (2, 2)), f"conv+relu+pool {cfg}")
+        assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), pool2=True),
+                          O.maxpool2d(plain, (2, 2), (0, 0), (2, 2)), f"conv+pool {cfg}")
+    for alpha in (0.1, 0.0, -0.5, 2.0, np.inf):
+        leaky = O.leaky_relu(plain, alpha).reshape(plain.shape)
+        assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), act="leaky", alpha=alpha), leaky,
+                          f"conv+leaky({alpha}) {cfg}")
+        for g, b in ((gamma, beta), (None, beta), (gamma, None), (None, None)):
+            bn = O.bn_infer(plain, mean, var, 1e-5, g, b)
+            want = O.leaky_relu(bn, alpha).reshape(plain.shape)
+            assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, g, b), act="leaky", alpha=alpha),
+                              want, f"conv+bn+leaky({alpha}) gamma={g is not None} beta={b is not None} {cfg}")
+            if can_pool and alpha in (0.1, -0.5):
+                assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), bn=(mean, var, g, b), act="leaky",
+                                                alpha=alpha, pool2=True),
+                                  O.maxpool2d(want, (2, 2), (0, 0), (2, 2)), f"conv+bn+leaky({alpha})+pool {cfg}")
+
+
 # shapes the small-image kernel takes (3x3, images up to 16x16, 16/32/64/128 channels): ragged filter
 # tiles, batches that do not fill the last workgroup, no padding, odd and even extents, H != W
 SMALL_IMAGE_CASES = [(7, 16, 7, 7, 10, 1), (5, 32, 14, 14, 50, 1), (9, 64, 7, 7, 33, 1), (3, 128, 5, 6, 20, 1),
