@@ -397,7 +397,7 @@ bool wide_plan(const gh_cmd& c, bool pool, WidePlan* out) {
   if (c.dim[5] != 3 || c.dim[6] != 3 || c.dim[9] != 1 || c.dim[10] != 1 || c.dim[11] != 1 || c.dim[12] != 1 ||
       c.dim[8] != pad || pad < 0 || pad > 1)
     return false;
-  if (B < 1 || F < 1 || C < 5 || C > 64 || H < 3 || W < 3 || H > 8192 || W > 8192) return false;
+  if (B < 1 || F < 1 || C < 3 || C > 64 || H < 3 || W < 3 || H > 8192 || W > 8192) return false;
   if (B * C * H * W >= (1ll << 31) || B * F * H * W >= (1ll << 31) || F > (1 << 20)) return false;
   if (getenv("GORGONIA_HIP_CONV_NO_WIDE")) return false;   // tuning switch: the other kernels only
   WideGeom g{};

@@ -2854,6 +2854,17 @@ static bool conv_direct_shape(const gh_cmd& c) {
          c.dim[12] == 1 && c.dim[7] == c.dim[8] && c.dim[1] >= 1 && c.dim[1] <= 4;
 }
 
+// The direct kernel's shapes, less those the wide-image kernel runs quicker: three or four
+// channels fill most of a quad of its K steps, and on images with enough pixels its matrix
+// cores then beat the vector units (3 -> 16 at 416 x 416: 42 us against 53).  Only where it can
+// also pool, so that a shape's plain and pooled commands stay with one kernel and one summing
+// order.
+static bool conv_direct_takes(const gh_cmd& c) {
+  if (!conv_direct_shape(c) || getenv("GORGONIA_HIP_CONV_NO_DIRECT")) return false;
+  if (c.dim[1] >= 3 && gh_conv_wide_takes(c) && gh_conv_wide_can_pool(c)) return false;
+  return true;
+}
+
 static int launch_conv_direct(gh_ctx* ctx, const gh_cmd& c) {
   const int B = (int)c.dim[0], C = (int)c.dim[1], H = (int)c.dim[2], W = (int)c.dim[3], F = (int)c.dim[4];
   const int pad = (int)c.dim[7];
@@ -2894,7 +2905,7 @@ static int launch_conv_direct(gh_ctx* ctx, const gh_cmd& c) {
 
 int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
   if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_conv2d_f64(ctx, c);
-  if (conv_direct_shape(c) && !getenv("GORGONIA_HIP_CONV_NO_DIRECT")) return launch_conv_direct(ctx, c);
+  if (conv_direct_takes(c)) return launch_conv_direct(ctx, c);
   const int rcs = gh_try_launch_conv_small(ctx, c);
   if (rcs >= 0) return rcs;
   const int rcp = gh_try_launch_conv_patch(ctx, c);
@@ -3111,7 +3122,7 @@ extern "C" int gh_gemm_can_softmax(const gh_cmd* c) {
 
 extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {
   if (!c || c->opcode != GH_OP_CONV2D || gh_dtype_of(c->flags) != GH_F32) return 0;
-  if (conv_direct_shape(*c) && !getenv("GORGONIA_HIP_CONV_NO_DIRECT")) {
+  if (conv_direct_takes(*c)) {
     const int64_t oh = c->dim[2] + 2 * c->dim[7] - 2, ow = c->dim[3] + 2 * c->dim[7] - 2;
     return oh >= 2 && ow >= 2;
   }
