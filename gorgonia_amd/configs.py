@@ -156,7 +156,7 @@ def build_convnet_train(inp, onehot, lr, read_grads=True, solver="set"):
     return g, outs
 
 
-def build_yolo(inp, resident=True, resident_input=False):
+def build_yolo(inp, resident=True, resident_input=False, borrow_output=False):
     g = G.NewGraph()
     h = G.NewTensor(g, inp["x"], resident_input)
     for i in range(7):
@@ -170,7 +170,8 @@ def build_yolo(inp, resident=True, resident_input=False):
         elif i == 5:
             h = G.MaxPool2D(h, (2, 2), (1, 0, 1, 0), (1, 1))  # darknet stride-1 pool
     out = G.Conv2d(h, G.NewTensor(g, inp["w7"], resident), (1, 1), (0, 0), (1, 1), (1, 1))
-    return g, {"out": G.Read(out)}
+    # borrow_output: the 2.3 MB result stays in the machine's pinned buffer (TapeMachine.value)
+    return g, {"out": G.ReadBorrowed(out) if borrow_output else G.Read(out)}
 
 
 FLOPS = {  # algorithmic flop per forward pass at the configured batch sizes

@@ -113,6 +113,20 @@ def Read(node, dtype=None):
     return out
 
 
+class BorrowedRead:
+    """A Read whose value stays in the machine's own pinned host buffer: TapeMachine.value(r)
+    is a numpy view of it, valid after RunAll and overwritten by the next one."""
+
+    def __init__(self, node):
+        self.node = node
+
+
+def ReadBorrowed(node):
+    """gorgonia.Read without the final host-to-host copy: the machine lends its buffer."""
+    node.g._check(node.g.lib.ghh_graph_read_borrowed(node.g.h, node.id))
+    return BorrowedRead(node)
+
+
 def _bin(fn):
     return lambda a, b: a.g.apply(K_ELEMBIN, [a, b], fn=_ffi.BIN_FN[fn])
 
@@ -360,6 +374,17 @@ class TapeMachine:
     def segment_verdict(self, segment=0):
         """'measuring', 'plain' or 'replay' for a segment of the last run (graph_replay="measured")."""
         return ("measuring", "plain", "replay")[self.lib.ghh_tape_segment_verdict(self.h, segment)]
+
+    def value(self, borrowed):
+        """The numpy view of a ReadBorrowed value (no copy; the next RunAll overwrites it)."""
+        node = borrowed.node
+        ptr = self.lib.ghh_tape_read_buffer(self.h, node.id)
+        if not ptr:
+            raise EngineError(1, f"value: node {node.id} is not a borrowed read of this machine")
+        shape = node.Shape()
+        n = int(np.prod(shape)) if len(shape) else 1
+        ctype = C.c_double if node.Dtype() == np.float64 else C.c_float
+        return np.ctypeslib.as_array((ctype * n).from_address(ptr)).reshape(shape)
 
     def phase_ns(self):
         """Host nanoseconds of the last RunAll: (whole call, launching, waiting for the device)."""

@@ -627,6 +627,16 @@ Status Graph::Let(int node, const void* host) {
 Status Graph::Read(int node, void* host_out) {
   if (node < 0 || node >= (int)nodes_.size()) return bad("Read: unknown node");
   nodes_[(size_t)node].read_into = host_out;
+  nodes_[(size_t)node].read_borrowed = false;
+  return Status::OK();
+}
+
+Status Graph::ReadBorrowed(int node) {
+  static char marker;   // read_into only has to be non-null: nothing is ever copied there
+  if (node < 0 || node >= (int)nodes_.size()) return bad("ReadBorrowed: unknown node");
+  Node& n = nodes_[(size_t)node];
+  n.read_into = &marker;
+  n.read_borrowed = true;
   return Status::OK();
 }
 
@@ -770,7 +780,7 @@ Status TapeMachine::Compile() {
   for (int i = 0; i < N; i++) {
     const Node& n = nodes[(size_t)i];
     if (!n.read_into || n.is_input || n.fused_away || n.alias_of >= 0 || inplace[(size_t)i]) continue;
-    if (bytes_of(n) > kStageLimit || bytes_of(n) % 4 != 0 || last_reader[(size_t)i] >= 0) continue;
+    if ((bytes_of(n) > kStageLimit && !n.read_borrowed) || bytes_of(n) % 4 != 0 || last_reader[(size_t)i] >= 0) continue;
     bool shared = false;
     for (int j = 0; j < N; j++)
       if (j != i && (root[(size_t)j] == i || node_reg_[(size_t)j] == node_reg_[(size_t)i])) shared = true;
@@ -821,8 +831,8 @@ Status TapeMachine::Compile() {
   // host reads: one flush, then the copies (compile.go:437-462 puts a flush in
   // front of every consumer that needs a finished value)
   for (int i = 0; i < N; i++)
-    if (nodes[(size_t)i].read_into && !host_out[(size_t)i] && bytes_of(nodes[(size_t)i]) <= kStageLimit &&
-        bytes_of(nodes[(size_t)i]) % 4 == 0)
+    if (nodes[(size_t)i].read_into && !host_out[(size_t)i] &&
+        (bytes_of(nodes[(size_t)i]) <= kStageLimit || nodes[(size_t)i].read_borrowed) && bytes_of(nodes[(size_t)i]) % 4 == 0)
       prog_.push_back({InstrKind::StageOut, i, node_reg_[(size_t)i], bytes_of(nodes[(size_t)i]), false});
   prog_.push_back({InstrKind::Flush, -1, -1, 0, false});
   std::vector<int> freed;
@@ -886,6 +896,11 @@ Status TapeMachine::Init(int device) {
     }
   }
   return Status::OK();
+}
+
+const void* TapeMachine::ReadBuffer(int node) const {
+  if (node < 0 || node >= (int)stage_.size() || !g_->Nodes()[(size_t)node].read_borrowed) return nullptr;
+  return stage_[(size_t)node];
 }
 
 uint64_t TapeMachine::RegisterAddress(int node) const {
@@ -1067,8 +1082,9 @@ Status TapeMachine::RunAll() {
       case InstrKind::Read: {
         Node& n = nodes[(size_t)in.node];
         if (in.node < (int)stage_.size() && stage_[(size_t)in.node]) {
-          // the flush in front of the reads has waited for the staging copy
-          std::memcpy(n.read_into, stage_[(size_t)in.node], (size_t)in.size);
+          // the flush in front of the reads has waited for the staging copy; a borrowed
+          // read is finished with that
+          if (!n.read_borrowed) std::memcpy(n.read_into, stage_[(size_t)in.node], (size_t)in.size);
           break;
         }
         st = eng_.MemcpyDtoH(n.read_into, regs_[(size_t)in.reg].mem, in.size, false);

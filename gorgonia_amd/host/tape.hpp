@@ -100,6 +100,7 @@ struct Node {
   OpSpec op;
   std::vector<int> inputs;
   void* read_into = nullptr;      // Read(node, &host) target
+  bool read_borrowed = false;     // ReadBorrowed: the value stays in the machine's own pinned buffer
   bool fused_away = false;        // absorbed into the follower that now computes both: no register, no instruction
   int alias_of = -1;              // Reshape shares its input's register
 };
@@ -110,6 +111,10 @@ class Graph {
   Status Apply(const OpSpec& op, const std::vector<int>& inputs, int* out);
   Status Let(int node, const void* host);              // rebind an input value
   Status Read(int node, void* host_out);               // gorgonia.Read
+  // Read without the last host copy: the machine keeps the value in pinned host memory of its
+  // own (TapeMachine::ReadBuffer) and overwrites it on every run, as the reference rebinds
+  // the Value a Read points at (op.go readOp.Do).
+  Status ReadBorrowed(int node);
   // Fold BatchNorm (eval), Rectify/LeakyRelu and a 2x2/2 MaxPool2D into the
   // Conv2d that feeds them (activations into MatMul too) when nothing else reads
   // the intermediate value.  The follower takes over the producer's operator
@@ -179,6 +184,7 @@ class TapeMachine {
   // graph launches and submits, [2] waiting for the device.
   void PhaseNs(int64_t out[3]) const { out[0] = ns_total_; out[1] = ns_launch_; out[2] = ns_wait_; }
   uint64_t RegisterAddress(int node) const;
+  const void* ReadBuffer(int node) const;   // where a ReadBorrowed node's value is after RunAll (null: not such a node)
   std::string ProgramString() const;              // program.String() (vm_tape.go:493-522)
 
  private:

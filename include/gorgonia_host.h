@@ -118,6 +118,12 @@ GH_API int ghh_graph_new_tensor(ghh_graph* g, const int64_t* shape, int ndim, in
 GH_API int ghh_graph_apply(ghh_graph* g, const ghh_op* op, const int* inputs, int n_inputs, int* out);
 GH_API int ghh_graph_let(ghh_graph* g, int node, const void* host);
 GH_API int ghh_graph_read(ghh_graph* g, int node, void* host_out);
+/* Read without the last host copy (op.go:readOp rebinds the Value a Read points at; here the
+ * caller borrows the machine's buffer instead): after every RunAll the node's value is in
+ * pinned host memory the machine owns, at ghh_tape_read_buffer(t, node) - the same address for
+ * the machine's lifetime, overwritten by the next run, freed by ghh_tape_close.  The producing
+ * kernel or a staging copy inside the segment writes it there; nothing is copied afterwards. */
+GH_API int ghh_graph_read_borrowed(ghh_graph* g, int node);
 GH_API int ghh_graph_node_shape(ghh_graph* g, int node, int64_t* shape, int cap);
 /* Node.Dtype(): 0 float32, 1 float64, 2 other; -1 for a bad node id */
 GH_API int ghh_graph_node_dtype(ghh_graph* g, int node);
@@ -155,6 +161,8 @@ GH_API int ghh_tape_segments(ghh_tape* t);
 GH_API int ghh_tape_graph_launches(ghh_tape* t);
 GH_API int64_t ghh_tape_submit_calls(ghh_tape* t);
 GH_API uint64_t ghh_tape_register_address(ghh_tape* t, int node);
+/* Where a ghh_graph_read_borrowed node's value lies after RunAll; NULL for any other node. */
+GH_API const void* ghh_tape_read_buffer(ghh_tape* t, int node);
 GH_API int ghh_tape_program_string(ghh_tape* t, char* buf, int cap);
 GH_API ghh_engine* ghh_tape_engine(ghh_tape* t);     /* borrowed: do not destroy */
 /* How segment `segment` of the last run executes: 0 undecided (still being timed, or graph_replay

@@ -249,6 +249,47 @@ def test_conv1d_on_the_tape(ctx):
         m.Close()
 
 
+def test_borrowed_reads_hold_what_read_copies(ctx):
+    """ReadBorrowed leaves a value in the machine's pinned buffer; Read copies it out.  Same bits,
+    for a value only the host reads (written there by its kernel), one that other nodes also
+    read (staged by a copy in the segment), a reshaped view and one past the staging limit of
+    ordinary reads; on plain runs, replayed runs and after the input changes."""
+    a0 = synth.uniform(31, (3, 1024, 1024), -1, 1)      # 12 MB: beyond the 8 MB of a staged Read
+    b0 = synth.uniform(32, (3, 1024, 1024), -1, 1)
+
+    def build(borrow):
+        g = G.NewGraph()
+        a, b = G.NewTensor(g, a0.copy()), G.NewTensor(g, b0, resident=True)
+        s = G.Add(a, b)            # read by the host and by the next two nodes
+        t = G.HadamardProd(s, b)   # only the host reads it: 12 MB
+        u = G.Reshape(G.Tanh(s), (3 * 1024, 1024))
+        small = G.Neg(G.NewTensor(g, synth.uniform(33, (7, 5), -1, 1)))   # 140 bytes
+        rd = G.ReadBorrowed if borrow else G.Read
+        return g, a, {"s": rd(s), "t": rd(t), "u": rd(u), "small": rd(small)}
+
+    for mode in (False, True):
+        g0, in0, want = build(False)
+        m0 = G.NewTapeMachine(g0, graph_replay=mode)
+        g1, in1, got = build(True)
+        m1 = G.NewTapeMachine(g1, graph_replay=mode)
+        addr = None
+        for it in range(4):
+            if it == 2:   # a new input value: both graphs see it
+                fresh = synth.uniform(40, a0.shape, -2, 2)
+                G.Let(in0, fresh); G.Let(in1, fresh)
+            m0.RunAll(); m1.RunAll()
+            views = {k: m1.value(v) for k, v in got.items()}
+            for k in want:
+                assert views[k].shape == want[k].shape
+                assert_bits_equal(views[k], want[k], f"borrowed read {k}, replay={mode}, run {it}")
+            here = {k: v.ctypes.data for k, v in views.items()}
+            assert addr is None or addr == here   # one buffer per value for the machine's life
+            addr = here
+        with pytest.raises(Exception):
+            m0.value(G.BorrowedRead(in0))          # not a borrowed read of that machine
+        m0.Close(); m1.Close()
+
+
 def test_measured_replay_keeps_results_and_settles(ctx):
     """graph_replay="measured": the machine times plain submits against replays of a segment on
     its first runs and keeps the quicker; every run along the way, and after the verdict, stores

@@ -214,3 +214,31 @@ def test_conv1d_is_conv2d_with_unit_height():
     m = G.NewTapeMachine(g, compile_only=True)
     assert "conv2d" in m.program()
     m.Close()
+
+
+def test_borrowed_reads_in_the_program():
+    """ReadBorrowed: a value only the host reads is written by its kernel into the machine's
+    pinned buffer (allocHost), one with other readers is staged by a copy inside the segment
+    (stageOut), both whatever their size; an ordinary Read past 8 MB is copied after the flush
+    instead.  Nothing but a borrowed read has a buffer to lend."""
+    def build(read):
+        g = G.NewGraph()
+        a = G.NewTensor(g, np.zeros((3, 1024, 1024), np.float32))
+        b = G.NewTensor(g, np.zeros((3, 1024, 1024), np.float32))
+        s = G.Add(a, b)
+        t = G.HadamardProd(s, b)
+        return g, a, read(s), read(t)
+    g, a, rs, rt = build(G.ReadBorrowed)
+    m = G.NewTapeMachine(g, compile_only=True)
+    prog = m.program()
+    assert "allocHost node 3" in prog and "stageOut node 2" in prog
+    assert prog.index("stageOut") < prog.index("flush") < prog.index("read node 2")
+    with pytest.raises(EngineError):
+        m.value(G.BorrowedRead(a))
+    m.Close()
+    g2, _, _, _ = build(G.Read)
+    m2 = G.NewTapeMachine(g2, compile_only=True)
+    assert "allocHost" not in m2.program() and "stageOut" not in m2.program()
+    m2.Close()
+    with pytest.raises(EngineError):
+        g.lib.ghh_graph_read_borrowed(g.h, 99) and g._check(g.lib.ghh_graph_read_borrowed(g.h, 99))
