@@ -455,20 +455,30 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(const float* __restrict__
   }
 }
 
-// Many slabs, few results (filter gradients): four lanes share one result.
-// Lane q adds slabs q, q+4, q+8, ... in that order, then the four sums are
-// combined as (s0 + s1) + (s2 + s3): a fixed order, so results repeat.
-template <class SC>
-__global__ __launch_bounds__(256) void k_splitk_reduce4(const float* __restrict__ ws, int splits, int M,
+// Many slabs, few results (filter gradients): L lanes share one result (4, or 16 from 64
+// slabs up).  Lane q adds slabs q, q+L, q+2L, ... in that order, then the L sums are
+// combined pairwise, neighbours first: (s0 + s1) + (s2 + s3), ... - a fixed order, so
+// results repeat.
+template <class SC, int L>
+__global__ __launch_bounds__(256) void k_splitk_reduce_lanes(const float* __restrict__ ws, int splits, int M,
                                                         int N, SC sc, int act, float alpha) {
   const int64_t total = (int64_t)M * N;
-  const int q = threadIdx.x & 3;
-  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 2;
+  const int q = threadIdx.x & (L - 1);
+  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) / L;
   float acc = 0.f;
-  if (e < total)
-    for (int s = q; s < splits; s += 4) acc = acc + ws[(int64_t)s * total + e];
-  const float pair = acc + __shfl_xor(acc, 1, 64);      // lanes 0,1 -> s0+s1 ; lanes 2,3 -> s2+s3 (commutative)
-  const float sum = pair + __shfl_xor(pair, 2, 64);
+  if (e < total) {
+    const float* p = ws + (int64_t)q * total + e;
+    int s = q;
+    for (; s + 3 * L < splits; s += 4 * L) {   // four loads in flight
+      const float v0 = p[0], v1 = p[(int64_t)L * total], v2 = p[2 * (int64_t)L * total], v3 = p[3 * (int64_t)L * total];
+      acc = acc + v0; acc = acc + v1; acc = acc + v2; acc = acc + v3;
+      p += 4 * (int64_t)L * total;
+    }
+    for (; s < splits; s += L) { acc = acc + p[0]; p += (int64_t)L * total; }
+  }
+  float sum = acc;
+#pragma unroll
+  for (int d = 1; d < L; d <<= 1) sum = sum + __shfl_xor(sum, d, 64);   // commutative per level: every lane ends with the total
   if (e < total && q == 0) {
     const int i = (int)(e / N), j = (int)(e - (int64_t)i * N);
     sc.put(i, j, act_apply(sc.pre(j, sum), act, alpha));
@@ -2946,6 +2956,24 @@ static ConvGeom conv_geom(const gh_cmd& c) {
   return g;
 }
 
+// Sum `splits` slabs of F x CKK partial filter gradients from the workspace into dw, in slab order.
+static int launch_slab_reduce(gh_ctx* ctx, const float* ws, int splits, int F, int CKK, float* dw) {
+  const int64_t total = (int64_t)F * CKK;
+  if (splits >= 64) {
+    hipLaunchKernelGGL((k_splitk_reduce_lanes<StoreRowMajor, 16>), dim3((int)cdiv(total * 16, 256)), dim3(256), 0,
+                       ctx->stream, ws, splits, F, CKK, StoreRowMajor{dw, CKK}, 0, 0.f);
+  } else if (splits >= 8) {
+    hipLaunchKernelGGL((k_splitk_reduce_lanes<StoreRowMajor, 4>), dim3((int)cdiv(total * 4, 256)), dim3(256), 0,
+                       ctx->stream, ws, splits, F, CKK, StoreRowMajor{dw, CKK}, 0, 0.f);
+  } else {
+    int64_t blocks = cdiv(total, 256);
+    if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
+    hipLaunchKernelGGL((k_splitk_reduce<StoreRowMajor>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws, splits, F,
+                       CKK, StoreRowMajor{dw, CKK}, 0, 0.f);
+  }
+  return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
+}
+
 // dW = dY2d^T . col  (ptr[0] = x, ptr[1] = dy, ptr[2] = dw)
 int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
   if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_conv2d_bwd_filter_f64(ctx, c);
@@ -2976,9 +3004,16 @@ int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
 #undef GH_WGRAD_DIRECT
     int rc = gh_check_hip(ctx, hipGetLastError(), "direct filter-gradient launch");
     if (rc) return rc;
-    hipLaunchKernelGGL((k_splitk_reduce4<StoreRowMajor>), dim3((int)cdiv((int64_t)F * CKK * 4, 256)), dim3(256),
+    hipLaunchKernelGGL((k_splitk_reduce_lanes<StoreRowMajor, 4>), dim3((int)cdiv((int64_t)F * CKK * 4, 256)), dim3(256),
                        0, ctx->stream, wsd, G, F, CKK, StoreRowMajor{(float*)(uintptr_t)c.ptr[2], CKK}, 0, 0.f);
     return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
+  }
+  {
+    // small images: the kernel that keeps dy and x of a few images in LDS; slabs summed as below
+    int sp = 0;
+    const int rcs = gh_try_launch_conv_wgrad_small(ctx, c, &sp);
+    if (rcs > 0 || (rcs == 0 && sp <= 1)) return rcs;
+    if (rcs == 0) return launch_slab_reduce(ctx, (const float*)ctx->workspace, sp, F, CKK, (float*)(uintptr_t)c.ptr[2]);
   }
   constexpr int BM = 64, BN = 64, BK = 32;
   const int64_t tiles = cdiv(F, BM) * cdiv(CKK, BN);
@@ -3001,16 +3036,7 @@ int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
                      CKK, (int)splits, ws);
   int rc = gh_check_hip(ctx, hipGetLastError(), "conv filter-gradient launch");
   if (rc || splits <= 1) return rc;
-  if (splits >= 8) {
-    hipLaunchKernelGGL((k_splitk_reduce4<StoreRowMajor>), dim3((int)cdiv((int64_t)F * CKK * 4, 256)), dim3(256),
-                       0, ctx->stream, ws, (int)splits, F, CKK, StoreRowMajor{dw, CKK}, 0, 0.f);
-  } else {
-    int64_t blocks = cdiv((int64_t)F * CKK, 256);
-    if (blocks > (int64_t)ctx->cu_count * 8) blocks = (int64_t)ctx->cu_count * 8;
-    hipLaunchKernelGGL((k_splitk_reduce<StoreRowMajor>), dim3((int)blocks), dim3(256), 0, ctx->stream, ws,
-                       (int)splits, F, CKK, StoreRowMajor{dw, CKK}, 0, 0.f);
-  }
-  return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
+  return launch_slab_reduce(ctx, ws, (int)splits, F, CKK, dw);
 }
 
 // dX = col2im(dY2d . Wflat)  (ptr[0] = dy, ptr[1] = w, ptr[2] = dx)

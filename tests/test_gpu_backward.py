@@ -77,6 +77,15 @@ CONV_BWD_CASES = [
     (16, 64, 7, 7, 128, 3, 3, (1, 1), (1, 1), (1, 1)),
     (2, 16, 52, 52, 32, 3, 3, (1, 1), (1, 1), (1, 1)),
     (2, 256, 13, 13, 512, 3, 3, (1, 1), (1, 1), (1, 1)),
+    # the small-image filter-gradient kernel (3x3, images up to 16x16, channels in sixteens, >= 16 filters):
+    # a ragged filter tile, image groups that do not divide the batch, no padding, H != W, one slab with
+    # many groups per workgroup (the tiles alone fill the device), the 16x16 limit, three-pixel images
+    (7, 16, 7, 7, 40, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (9, 32, 6, 11, 80, 3, 3, (0, 0), (1, 1), (1, 1)),
+    (5, 48, 16, 16, 17, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (3, 512, 5, 4, 1024, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (33, 16, 3, 3, 16, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (130, 16, 14, 14, 64, 3, 3, (1, 1), (1, 1), (1, 1)),
     # Conv1d shapes (ops/nn/api_cuda.go:18-20): H = 1, kernel {1,k}
     (3, 4, 1, 37, 6, 1, 3, (0, 1), (1, 1), (1, 1)),
     (2, 8, 1, 64, 16, 1, 5, (0, 2), (1, 2), (1, 1)),
