@@ -263,12 +263,14 @@ def bench_convnet_kernels(ctx, batch, iters):
 
 
 def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=True, dtype=np.float32,
-                  reupload_all=False):
+                  reupload_all=False, borrow_input=False):
     from gorgonia_amd import configs, graph as G
     inp = {k: v.astype(dtype) for k, v in configs.convnet_inputs(batch).items()}
     g = G.NewGraph()
     # same graph as configs.build_convnet, with the input batch optionally resident
-    h = G.NewTensor(g, inp["x"], resident=resident_input)
+    h = xin = G.NewTensor(g, inp["x"], resident=resident_input)
+    if borrow_input:   # the batch is written into the machine's pinned buffer (a loader's job), not copied there
+        G.LetBorrowed(xin)
     for i in range(3):
         w = G.NewTensor(g, inp[f"w{i}"], True)
         h = G.MaxPool2D(G.Rectify(G.Conv2d(h, w, (3, 3), (1, 1), (1, 1), (1, 1))), (2, 2), (0, 0), (2, 2))
@@ -278,6 +280,8 @@ def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=Tr
     # reupload_all: every input, weights too, crosses the bus on every run as the
     # reference's tape machine does it (vm_tape_cuda.go:220-243)
     m = G.NewTapeMachine(g, graph_replay=graph_replay, fuse_activations=True, reupload_resident=reupload_all)
+    if borrow_input:
+        m.input(xin)[...] = inp["x"]
     for _ in range(max(warmup, WARM_RUNS)):
         m.RunAll()
     eng = m.engine()
@@ -291,7 +295,7 @@ def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=Tr
     launches = m.graph_launches()
     if graph_replay == "measured":
         VERDICTS[f"convnet{'_f64' if dtype == np.float64 else ''}{'' if resident_input else '_input_h2d'}"
-                 f"{'_all_h2d' if reupload_all else ''}"] = m.segment_verdict()
+                 f"{'_all_h2d' if reupload_all else ''}{'_borrowed' if borrow_input else ''}"] = m.segment_verdict()
     m.Close()
     return dt / steps * 1e3, result, inp, launches
 
@@ -527,6 +531,8 @@ def main():
         four_images_s, four_out = bench_convnet_machines(a.steps, a.warmup, 4)
         log(f"convnet, machines in parallel host threads: two {two_images_s:.0f}, four {four_images_s:.0f} images/s")
     ms_h2d, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False, graph_replay=replay_mode())
+    ms_h2d_b, out_h2d_b, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False,
+                                              graph_replay=replay_mode(), borrow_input=True)
     ms_h2d_all, out_h2d_all, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, resident_input=False,
                                                   reupload_all=True, graph_replay=replay_mode())
     ms_eager, _, _, _ = bench_convnet(max(20, a.steps // 4), a.warmup, graph_replay=False)
@@ -670,6 +676,8 @@ def main():
             "sgemm_frac_mfma": lin.get("sgemm_4096", {}).get("frac_mfma"),
             "convnet_ms_per_step_with_input_h2d": round(ms_h2d, 5),
             "convnet_images_s_with_input_h2d": round(128 / ms_h2d * 1e3, 1),
+            "convnet_ms_per_step_with_input_h2d_from_borrowed_pinned_buffer": round(ms_h2d_b, 5),
+            "convnet_borrowed_input_output_equals_resident": bool(np.array_equal(out_h2d_b, gpu_out)),
             "convnet_ms_per_step_all_inputs_reuploaded": round(ms_h2d_all, 5),
             "convnet_images_s_all_inputs_reuploaded": round(128 / ms_h2d_all * 1e3, 1),
             "convnet_all_inputs_reuploaded_bytes_per_step": int(sum(v.nbytes for v in inp.values())),

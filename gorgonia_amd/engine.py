@@ -82,6 +82,7 @@ HOST_SYMBOLS = {
     "ghh_graph_let": (C.c_int, [_P, C.c_int, _P]),
     "ghh_graph_read": (C.c_int, [_P, C.c_int, _P]),
     "ghh_graph_read_borrowed": (C.c_int, [_P, C.c_int]),
+    "ghh_graph_let_borrowed": (C.c_int, [_P, C.c_int]),
     "ghh_graph_node_shape": (C.c_int, [_P, C.c_int, C.POINTER(C.c_int64), C.c_int]),
     "ghh_graph_node_dtype": (C.c_int, [_P, C.c_int]),
     "ghh_graph_fuse_activations": (C.c_int, [_P]),
@@ -101,6 +102,7 @@ HOST_SYMBOLS = {
     "ghh_tape_submit_calls": (C.c_int64, [_P]),
     "ghh_tape_register_address": (C.c_uint64, [_P, C.c_int]),
     "ghh_tape_read_buffer": (_P, [_P, C.c_int]),
+    "ghh_tape_input_buffer": (_P, [_P, C.c_int]),
     "ghh_tape_program_string": (C.c_int, [_P, C.c_char_p, C.c_int]),
     "ghh_tape_engine": (_P, [_P]),
     "ghh_tape_segment_verdict": (C.c_int, [_P, C.c_int]),

@@ -121,6 +121,13 @@ class BorrowedRead:
         self.node = node
 
 
+def LetBorrowed(node):
+    """Let without the host-to-host copy: the input's value is what the caller writes into
+    TapeMachine.input(node), the machine's pinned buffer for it."""
+    node.g._check(node.g.lib.ghh_graph_let_borrowed(node.g.h, node.id))
+    return node
+
+
 def ReadBorrowed(node):
     """gorgonia.Read without the final host-to-host copy: the machine lends its buffer."""
     node.g._check(node.g.lib.ghh_graph_read_borrowed(node.g.h, node.id))
@@ -375,16 +382,26 @@ class TapeMachine:
         """'measuring', 'plain' or 'replay' for a segment of the last run (graph_replay="measured")."""
         return ("measuring", "plain", "replay")[self.lib.ghh_tape_segment_verdict(self.h, segment)]
 
+    def _view(self, ptr, node):
+        shape = node.Shape()
+        n = int(np.prod(shape)) if len(shape) else 1
+        ctype = C.c_double if node.Dtype() == np.float64 else C.c_float
+        return np.ctypeslib.as_array((ctype * n).from_address(ptr)).reshape(shape)
+
+    def input(self, node):
+        """The numpy view of a LetBorrowed input's pinned buffer: write the next value there."""
+        ptr = self.lib.ghh_tape_input_buffer(self.h, node.id)
+        if not ptr:
+            raise EngineError(1, f"input: node {node.id} is not a borrowed input of this machine")
+        return self._view(ptr, node)
+
     def value(self, borrowed):
         """The numpy view of a ReadBorrowed value (no copy; the next RunAll overwrites it)."""
         node = borrowed.node
         ptr = self.lib.ghh_tape_read_buffer(self.h, node.id)
         if not ptr:
             raise EngineError(1, f"value: node {node.id} is not a borrowed read of this machine")
-        shape = node.Shape()
-        n = int(np.prod(shape)) if len(shape) else 1
-        ctype = C.c_double if node.Dtype() == np.float64 else C.c_float
-        return np.ctypeslib.as_array((ctype * n).from_address(ptr)).reshape(shape)
+        return self._view(ptr, node)
 
     def phase_ns(self):
         """Host nanoseconds of the last RunAll: (whole call, launching, waiting for the device)."""

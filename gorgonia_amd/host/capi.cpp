@@ -201,6 +201,7 @@ int ghh_graph_apply(ghh_graph* g, const ghh_op* op, const int* inputs, int n_inp
 int ghh_graph_let(ghh_graph* g, int node, const void* host) { return ret(g, g->g.Let(node, host)); }
 int ghh_graph_read(ghh_graph* g, int node, void* host_out) { return ret(g, g->g.Read(node, host_out)); }
 int ghh_graph_read_borrowed(ghh_graph* g, int node) { return ret(g, g->g.ReadBorrowed(node)); }
+int ghh_graph_let_borrowed(ghh_graph* g, int node) { return ret(g, g->g.LetBorrowed(node)); }
 int ghh_graph_node_shape(ghh_graph* g, int node, int64_t* shape, int cap) {
   if (node < 0 || node >= (int)g->g.Nodes().size()) return -1;
   const Shape& s = g->g.Nodes()[(size_t)node].shape;
@@ -264,6 +265,7 @@ int ghh_tape_graph_launches(ghh_tape* t) { return t->t->GraphLaunches(); }
 int64_t ghh_tape_submit_calls(ghh_tape* t) { return t->t->Eng().SubmitCalls(); }
 uint64_t ghh_tape_register_address(ghh_tape* t, int node) { return t->t->RegisterAddress(node); }
 const void* ghh_tape_read_buffer(ghh_tape* t, int node) { return t->t->ReadBuffer(node); }
+void* ghh_tape_input_buffer(ghh_tape* t, int node) { return t->t->InputBuffer(node); }
 int ghh_tape_program_string(ghh_tape* t, char* buf, int cap) {
   std::string s = t->t->ProgramString();
   if (buf && cap > 0) snprintf(buf, (size_t)cap, "%s", s.c_str());

@@ -621,6 +621,15 @@ Status Graph::Apply(const OpSpec& op, const std::vector<int>& inputs, int* out) 
 Status Graph::Let(int node, const void* host) {
   if (node < 0 || node >= (int)nodes_.size() || !nodes_[(size_t)node].is_input) return bad("Let: not an input node");
   nodes_[(size_t)node].host = host;
+  nodes_[(size_t)node].host_borrowed = false;
+  return Status::OK();
+}
+
+Status Graph::LetBorrowed(int node) {
+  static const char marker = 0;   // host only has to be non-null: nothing is ever read through it
+  if (node < 0 || node >= (int)nodes_.size() || !nodes_[(size_t)node].is_input) return bad("LetBorrowed: not an input node");
+  nodes_[(size_t)node].host = &marker;
+  nodes_[(size_t)node].host_borrowed = true;
   return Status::OK();
 }
 
@@ -887,6 +896,13 @@ Status TapeMachine::Init(int device) {
     // is the whole ring); inputs past the cap fall back to a direct copy
     if (in.kind == InstrKind::Transport) {
       const Node& n = g_->Nodes()[(size_t)in.node];
+      if (n.host_borrowed) {   // the caller fills this buffer itself: it exists whatever the size
+        if (in.size % 4 != 0)
+          return Status::Err(GH_EINVAL, "LetBorrowed: input node " + std::to_string(in.node) + " is not a multiple of 4 bytes");
+        st = eng_.HostAlloc(in.size, &stage_in_[(size_t)in.node]);
+        if (!st.ok()) return st;
+        continue;
+      }
       if ((n.resident && !opt_.reupload_resident) || in.size % 4 != 0 || in.size > kStageInLimit ||
           staged_in + in.size > kStageInTotal)
         continue;
@@ -896,6 +912,11 @@ Status TapeMachine::Init(int device) {
     }
   }
   return Status::OK();
+}
+
+void* TapeMachine::InputBuffer(int node) const {
+  if (node < 0 || node >= (int)stage_in_.size() || !g_->Nodes()[(size_t)node].host_borrowed) return nullptr;
+  return stage_in_[(size_t)node];
 }
 
 const void* TapeMachine::ReadBuffer(int node) const {
@@ -1030,7 +1051,7 @@ Status TapeMachine::RunAll() {
         if (void* pinned = stage_in_[(size_t)in.node]) {
           // host value -> pinned buffer now, pinned buffer -> register as a command of
           // the segment: the upload is captured and replayed with the operators
-          std::memcpy(pinned, n.host, (size_t)in.size);
+          if (!n.host_borrowed) std::memcpy(pinned, n.host, (size_t)in.size);
           eng_.RecordCopy(regs_[(size_t)in.reg].mem, (uint64_t)(uintptr_t)pinned, in.size);
           resident_done_[(size_t)in.node] = 1;
           break;

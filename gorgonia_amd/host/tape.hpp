@@ -97,6 +97,7 @@ struct Node {
   bool is_input = false;
   bool resident = false;          // uploaded once and kept (weights); else re-uploaded per run
   const void* host = nullptr;     // bound host value (Let / WithValue)
+  bool host_borrowed = false;     // LetBorrowed: the caller writes the value into the machine's pinned buffer
   OpSpec op;
   std::vector<int> inputs;
   void* read_into = nullptr;      // Read(node, &host) target
@@ -110,6 +111,9 @@ class Graph {
   int NewTensor(const Shape& s, Dtype dt, const void* host, bool resident);
   Status Apply(const OpSpec& op, const std::vector<int>& inputs, int* out);
   Status Let(int node, const void* host);              // rebind an input value
+  // The input's value is whatever the caller has written into the machine's pinned buffer for
+  // it (TapeMachine::InputBuffer) when a run uploads it: Let without the host-to-host copy.
+  Status LetBorrowed(int node);
   Status Read(int node, void* host_out);               // gorgonia.Read
   // Read without the last host copy: the machine keeps the value in pinned host memory of its
   // own (TapeMachine::ReadBuffer) and overwrites it on every run, as the reference rebinds
@@ -184,6 +188,7 @@ class TapeMachine {
   // graph launches and submits, [2] waiting for the device.
   void PhaseNs(int64_t out[3]) const { out[0] = ns_total_; out[1] = ns_launch_; out[2] = ns_wait_; }
   uint64_t RegisterAddress(int node) const;
+  void* InputBuffer(int node) const;        // where a LetBorrowed input's next value goes (null: not such a node)
   const void* ReadBuffer(int node) const;   // where a ReadBorrowed node's value is after RunAll (null: not such a node)
   std::string ProgramString() const;              // program.String() (vm_tape.go:493-522)
 

@@ -124,6 +124,11 @@ GH_API int ghh_graph_read(ghh_graph* g, int node, void* host_out);
  * the machine's lifetime, overwritten by the next run, freed by ghh_tape_close.  The producing
  * kernel or a staging copy inside the segment writes it there; nothing is copied afterwards. */
 GH_API int ghh_graph_read_borrowed(ghh_graph* g, int node);
+/* Let without the host-to-host copy (the counterpart of ghh_graph_read_borrowed for inputs): the
+ * input's value is what the caller has written to ghh_tape_input_buffer(t, node) - pinned host
+ * memory the machine owns, one address for its life - when a run uploads it.  A data loader
+ * that decodes a batch straight into that buffer saves the copy ghh_graph_let's value takes. */
+GH_API int ghh_graph_let_borrowed(ghh_graph* g, int node);
 GH_API int ghh_graph_node_shape(ghh_graph* g, int node, int64_t* shape, int cap);
 /* Node.Dtype(): 0 float32, 1 float64, 2 other; -1 for a bad node id */
 GH_API int ghh_graph_node_dtype(ghh_graph* g, int node);
@@ -163,6 +168,8 @@ GH_API int64_t ghh_tape_submit_calls(ghh_tape* t);
 GH_API uint64_t ghh_tape_register_address(ghh_tape* t, int node);
 /* Where a ghh_graph_read_borrowed node's value lies after RunAll; NULL for any other node. */
 GH_API const void* ghh_tape_read_buffer(ghh_tape* t, int node);
+/* Where a ghh_graph_let_borrowed input's next value is to be written; NULL for any other node. */
+GH_API void* ghh_tape_input_buffer(ghh_tape* t, int node);
 GH_API int ghh_tape_program_string(ghh_tape* t, char* buf, int cap);
 GH_API ghh_engine* ghh_tape_engine(ghh_tape* t);     /* borrowed: do not destroy */
 /* How segment `segment` of the last run executes: 0 undecided (still being timed, or graph_replay

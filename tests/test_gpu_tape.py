@@ -290,6 +290,44 @@ def test_borrowed_reads_hold_what_read_copies(ctx):
         m0.Close(); m1.Close()
 
 
+def test_borrowed_inputs_upload_what_the_caller_wrote(ctx):
+    """LetBorrowed: the caller writes an input's value into the machine's pinned buffer and the run
+    uploads it from there; same results as Let with a host array, on plain and replayed runs, with the
+    value changed between runs, for a per-run input and for one that is resident (uploaded once)."""
+    inp = configs.convnet_inputs(16)
+    for mode in (False, True):
+        m0, outs0, want = run_once(configs.build_convnet, inp, fuse_activations=True)
+        m0.Close()
+        g = G.NewGraph()
+        x = G.LetBorrowed(G.NewTensor(g, inp["x"]))
+        ws = [G.NewTensor(g, inp[f"w{i}"], resident=True) for i in range(5)]
+        G.LetBorrowed(ws[4])                      # resident: taken from its buffer on the first run only
+        h = x
+        for i in range(3):
+            h = G.MaxPool2D(G.Rectify(G.Conv2d(h, ws[i], (3, 3), (1, 1), (1, 1), (1, 1))), (2, 2), (0, 0), (2, 2))
+        h = G.Rectify(G.Mul(G.Reshape(h, (16, 128 * 3 * 3)), ws[3]))
+        out = G.Read(G.SoftMax(G.Mul(h, ws[4])))
+        m = G.NewTapeMachine(g, graph_replay=mode, fuse_activations=True)
+        m.input(x)[...] = inp["x"]
+        m.input(ws[4])[...] = inp["w4"]
+        addr = m.input(x).ctypes.data
+        for it in range(3):
+            m.RunAll()
+            assert_bits_equal(out, want["out"], f"borrowed input, replay={mode}, run {it}")
+            m.input(ws[4])[...] = 0.0             # resident and uploaded: ignored from now on
+        assert m.input(x).ctypes.data == addr
+        # a new batch: both ways of binding see it
+        fresh = dict(inp, x=synth.uniform(99, inp["x"].shape, 0, 1))
+        m1, _, want1 = run_once(configs.build_convnet, fresh, fuse_activations=True)
+        m1.Close()
+        m.input(x)[...] = fresh["x"]
+        m.RunAll()
+        assert_bits_equal(out, want1["out"], f"borrowed input, new batch, replay={mode}")
+        with pytest.raises(Exception):
+            m.input(ws[0])                        # bound with a host array, nothing to lend
+        m.Close()
+
+
 def test_measured_replay_keeps_results_and_settles(ctx):
     """graph_replay="measured": the machine times plain submits against replays of a segment on
     its first runs and keeps the quicker; every run along the way, and after the verdict, stores
