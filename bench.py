@@ -395,7 +395,7 @@ def bench_convnet_train(steps, warmup, batch=128, dtype=np.float32):
     onehot = np.zeros((batch, 10), dtype)
     onehot[np.arange(batch), np.arange(batch) % 10] = 1.0
     g, outs = configs.build_convnet_train(inp, onehot, 0.01, read_grads=False, solver="rmsprop")
-    m = G.NewTapeMachine(g, graph_replay=replay_mode())
+    m = G.NewTapeMachine(g, graph_replay=replay_mode(), fuse_activations=True)
     for _ in range(max(warmup, WARM_RUNS)):
         m.RunAll()
     eng = m.engine()

@@ -24,6 +24,16 @@ struct PoolGeom {
 // element in row-major window order that beats everything before it, from
 // -FLT_MAX).  Gathering the same contributions per element in the same window
 // order gives the same bits without atomics, overlapping windows included.
+//
+// RELU (GH_FLAG_ACT_RELU): x is the value before a Rectify whose result was pooled.  The windows
+// are scanned over x * (x >= 0) and the gathered sum is multiplied by (x >= 0): the gradient
+// of MaxPool2D(Rectify(x)) with the bits of MaxPool2DDiff followed by the activation's own
+// gradient (dy times the 1.0 / 0.0 of Gte), without the Rectify result or the pooling gradient
+// ever being stored.
+__device__ __forceinline__ float relu_of(float v) { return v * (v >= 0.0f ? 1.0f : 0.0f); }
+__device__ __forceinline__ float relu_mask(float v) { return v >= 0.0f ? 1.0f : 0.0f; }
+
+template <bool RELU>
 __global__ __launch_bounds__(kBlock) void k_maxpool2d_bwd(const float* __restrict__ x,
                                                           const float* __restrict__ dy,
                                                           float* __restrict__ dx, PoolGeom g,
@@ -53,12 +63,13 @@ __global__ __launch_bounds__(kBlock) void k_maxpool2d_bwd(const float* __restric
         int arg = -1;
         for (int hi = hs; hi < he; hi++)
           for (int wi = ws; wi < we; wi++) {
-            const float v = in[hi * g.W + wi];
+            float v = in[hi * g.W + wi];
+            if (RELU) v = relu_of(v);
             if (v > best) { best = v; arg = hi * g.W + wi; }
           }
         if (arg == me) acc = acc + gy[ph * g.ow + pw];
       }
-    dx[idx] = acc;
+    dx[idx] = RELU ? acc * relu_mask(in[me]) : acc;
   }
 }
 
@@ -66,6 +77,7 @@ __global__ __launch_bounds__(kBlock) void k_maxpool2d_bwd(const float* __restric
 // overlap, so one thread owns two adjacent windows - two float4 row loads, one
 // float2 of dy, two float4 stores - with the generic kernel's scan order
 // (r0c0, r0c1, r1c0, r1c1), strict >, and its "0 + dy" for the winner.
+template <bool RELU>
 __global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2_bwd(const float* __restrict__ x,
                                                               const float* __restrict__ dy,
                                                               float* __restrict__ dx, int H, int W,
@@ -80,8 +92,16 @@ __global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2_bwd(const float* __res
     const int64_t bc = row / oh;
     const int ph = (int)(row - bc * oh);
     const int64_t at = (bc * H + 2 * ph) * (int64_t)W + 4 * pp;
-    const f4 r0 = *reinterpret_cast<const f4*>(x + at);
-    const f4 r1 = *reinterpret_cast<const f4*>(x + at + W);
+    f4 r0 = *reinterpret_cast<const f4*>(x + at);
+    f4 r1 = *reinterpret_cast<const f4*>(x + at + W);
+    f4 m0 = {1.f, 1.f, 1.f, 1.f}, m1 = m0;
+    if (RELU) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        m0[j] = relu_mask(r0[j]); m1[j] = relu_mask(r1[j]);
+        r0[j] = relu_of(r0[j]); r1[j] = relu_of(r1[j]);
+      }
+    }
     const f2 g = *reinterpret_cast<const f2*>(dy + (bc * oh + ph) * (int64_t)ow + 2 * pp);
     f4 o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -98,6 +118,7 @@ __global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2_bwd(const float* __res
       o1[2 * e] = arg == 2 ? v : 0.0f;
       o1[2 * e + 1] = arg == 3 ? v : 0.0f;
     }
+    if (RELU) { o0 = o0 * m0; o1 = o1 * m1; }
     *reinterpret_cast<f4*>(dx + at) = o0;
     *reinterpret_cast<f4*>(dx + at + W) = o1;
   }
@@ -107,6 +128,7 @@ __global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2_bwd(const float* __res
 // four): one thread per window with scalar accesses; the thread of the last
 // window column / row also zeroes the column / row an odd size leaves outside
 // every window.  Same scan order, strict > and "0 + dy" as above.
+template <bool RELU>
 __global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2_bwd_any(const float* __restrict__ x,
                                                                   const float* __restrict__ dy,
                                                                   float* __restrict__ dx, int H, int W,
@@ -119,7 +141,12 @@ __global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2_bwd_any(const float* _
     const int ph = (int)(row % oh);
     const int64_t bc = row / oh;
     const int64_t at = (bc * H + 2 * ph) * (int64_t)W + 2 * pw;
-    const float v00 = x[at], v01 = x[at + 1], v10 = x[at + W], v11 = x[at + W + 1];
+    float v00 = x[at], v01 = x[at + 1], v10 = x[at + W], v11 = x[at + W + 1];
+    float k00 = 1.f, k01 = 1.f, k10 = 1.f, k11 = 1.f;
+    if (RELU) {
+      k00 = relu_mask(v00); k01 = relu_mask(v01); k10 = relu_mask(v10); k11 = relu_mask(v11);
+      v00 = relu_of(v00); v01 = relu_of(v01); v10 = relu_of(v10); v11 = relu_of(v11);
+    }
     float best = -FLT_MAX;
     int arg = -1;
     if (v00 > best) { best = v00; arg = 0; }
@@ -127,10 +154,10 @@ __global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2_bwd_any(const float* _
     if (v10 > best) { best = v10; arg = 2; }
     if (v11 > best) { best = v11; arg = 3; }
     const float v = 0.0f + dy[idx];
-    dx[at] = arg == 0 ? v : 0.0f;
-    dx[at + 1] = arg == 1 ? v : 0.0f;
-    dx[at + W] = arg == 2 ? v : 0.0f;
-    dx[at + W + 1] = arg == 3 ? v : 0.0f;
+    dx[at] = (arg == 0 ? v : 0.0f) * k00;   // k.. is 1 without RELU: v * 1 is v
+    dx[at + 1] = (arg == 1 ? v : 0.0f) * k01;
+    dx[at + W] = (arg == 2 ? v : 0.0f) * k10;
+    dx[at + W + 1] = (arg == 3 ? v : 0.0f) * k11;
     if ((W & 1) && pw == ow - 1) { dx[at + 2] = 0.0f; dx[at + W + 2] = 0.0f; }
     if ((H & 1) && ph == oh - 1) {
       dx[at + 2 * (int64_t)W] = 0.0f;
@@ -521,14 +548,20 @@ int gh_launch_maxpool2d_bwd(gh_ctx* ctx, const gh_cmd& c) {
   g.padW = (int)(explicit_pad ? padE : padW);
   const int64_t total = B * C * g.H * g.W;
   if (total == 0) return GH_OK;
+  const bool relu = c.flags & GH_FLAG_ACT_RELU;   // gradient of MaxPool2D(Rectify(x)) with respect to x
   if (g.kh == 2 && g.kw == 2 && g.strideH == 2 && g.strideW == 2 && g.padH == 0 && g.padW == 0 &&
       g.H % 2 == 0 && g.W % 4 == 0 && ((c.ptr[0] | c.ptr[2]) & 15) == 0 && (c.ptr[1] & 7) == 0) {
     const int64_t pairs = total / 8;
     int64_t blocks = (pairs + kBlock - 1) / kBlock;
     if (blocks > (int64_t)ctx->cu_count * 64) blocks = (int64_t)ctx->cu_count * 64;
-    hipLaunchKernelGGL(k_maxpool_2x2s2_bwd, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
-                       (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
-                       (float*)(uintptr_t)c.ptr[2], g.H, g.W, pairs);
+    if (relu)
+      hipLaunchKernelGGL(k_maxpool_2x2s2_bwd<true>, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
+                         (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                         (float*)(uintptr_t)c.ptr[2], g.H, g.W, pairs);
+    else
+      hipLaunchKernelGGL(k_maxpool_2x2s2_bwd<false>, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
+                         (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                         (float*)(uintptr_t)c.ptr[2], g.H, g.W, pairs);
     return gh_check_hip(ctx, hipGetLastError(), "maxpool backward launch");
   }
   if (g.kh == 2 && g.kw == 2 && g.strideH == 2 && g.strideW == 2 && g.padH == 0 && g.padW == 0 && !explicit_pad &&
@@ -536,16 +569,26 @@ int gh_launch_maxpool2d_bwd(gh_ctx* ctx, const gh_cmd& c) {
     const int64_t windows = B * C * (int64_t)g.oh * g.ow;
     int64_t blocks = (windows + kBlock - 1) / kBlock;
     if (blocks > (int64_t)ctx->cu_count * 64) blocks = (int64_t)ctx->cu_count * 64;
-    hipLaunchKernelGGL(k_maxpool_2x2s2_bwd_any, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
-                       (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
-                       (float*)(uintptr_t)c.ptr[2], g.H, g.W, windows);
+    if (relu)
+      hipLaunchKernelGGL(k_maxpool_2x2s2_bwd_any<true>, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
+                         (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                         (float*)(uintptr_t)c.ptr[2], g.H, g.W, windows);
+    else
+      hipLaunchKernelGGL(k_maxpool_2x2s2_bwd_any<false>, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
+                         (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                         (float*)(uintptr_t)c.ptr[2], g.H, g.W, windows);
     return gh_check_hip(ctx, hipGetLastError(), "maxpool backward launch");
   }
   int64_t blocks = (total + kBlock - 1) / kBlock;
   if (blocks > (int64_t)ctx->cu_count * 64) blocks = (int64_t)ctx->cu_count * 64;
-  hipLaunchKernelGGL(k_maxpool2d_bwd, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
-                     (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
-                     (float*)(uintptr_t)c.ptr[2], g, total);
+  if (relu)
+    hipLaunchKernelGGL(k_maxpool2d_bwd<true>, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
+                       (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                       (float*)(uintptr_t)c.ptr[2], g, total);
+  else
+    hipLaunchKernelGGL(k_maxpool2d_bwd<false>, dim3((int)blocks), dim3(kBlock), 0, ctx->stream,
+                       (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
+                       (float*)(uintptr_t)c.ptr[2], g, total);
   return gh_check_hip(ctx, hipGetLastError(), "maxpool backward launch");
 }
 

@@ -18,6 +18,11 @@ struct PoolGeom {
   int H, W, oh, ow, kh, kw, padH, padW, strideH, strideW;
 };
 
+// Rectify in the reference's arithmetic (nn.go:136-163), for pooling kernels that take their
+// input through it (GH_FLAG_ACT_RELU on MAXPOOL2D: the activation's result is never stored).
+__device__ __forceinline__ float relu_of(float v) { return v * (v >= 0.0f ? 1.0f : 0.0f); }
+
+template <bool RELU>
 __global__ __launch_bounds__(kBlock) void k_maxpool2d(const float* __restrict__ x,
                                                       float* __restrict__ y, PoolGeom g,
                                                       int64_t total) {
@@ -35,7 +40,8 @@ __global__ __launch_bounds__(kBlock) void k_maxpool2d(const float* __restrict__ 
     float best = -FLT_MAX;
     for (int hi = hs; hi < he; hi++)
       for (int wi = ws; wi < we; wi++) {
-        const float v = in[hi * g.W + wi];
+        float v = in[hi * g.W + wi];
+        if (RELU) v = relu_of(v);
         if (v > best) best = v;
       }
     y[idx] = best;
@@ -45,6 +51,7 @@ __global__ __launch_bounds__(kBlock) void k_maxpool2d(const float* __restrict__ 
 // 2x2 / stride 2 / no padding, even W: each thread produces two adjacent
 // outputs from two float4 loads (rows hi, hi+1), same compare order as the
 // generic kernel: (r0,c0), (r0,c1), (r1,c0), (r1,c1).
+template <bool RELU>
 __global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2(const float* __restrict__ x,
                                                           float* __restrict__ y, int H, int W,
                                                           int oh, int ow, int64_t pairs) {
@@ -58,8 +65,12 @@ __global__ __launch_bounds__(kBlock) void k_maxpool_2x2s2(const float* __restric
     const int64_t bc = row / oh;
     const int ph = (int)(row - bc * oh);
     const float* in = x + (bc * H + 2 * ph) * (int64_t)W + 4 * pp;
-    const f4 r0 = *(reinterpret_cast<const f4*>(in));
-    const f4 r1 = *(reinterpret_cast<const f4*>(in + W));
+    f4 r0 = *(reinterpret_cast<const f4*>(in));
+    f4 r1 = *(reinterpret_cast<const f4*>(in + W));
+    if (RELU) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) { r0[j] = relu_of(r0[j]); r1[j] = relu_of(r1[j]); }
+    }
     f2 o;
 #pragma unroll
     for (int e = 0; e < 2; e++) {
@@ -178,6 +189,7 @@ int gh_launch_maxpool2d(gh_ctx* ctx, const gh_cmd& c) {
   if (total <= 0) return GH_OK;
   const float* x = (const float*)(uintptr_t)c.ptr[0];
   float* y = (float*)(uintptr_t)c.ptr[1];
+  const bool relu = c.flags & GH_FLAG_ACT_RELU;   // y = pool(x * (x >= 0))
   const bool fast = g.kh == 2 && g.kw == 2 && g.strideH == 2 && g.strideW == 2 && padN == 0 &&
                     padS == 0 && padW == 0 && padE == 0 && g.W % 4 == 0 && g.H % 2 == 0 &&
                     al16(c.ptr[0]) && (c.ptr[1] & 7u) == 0;
@@ -185,12 +197,17 @@ int gh_launch_maxpool2d(gh_ctx* ctx, const gh_cmd& c) {
     const int64_t pairs = total / 2;
     int64_t blocks = (pairs + kBlock - 1) / kBlock;
     if (blocks > (int64_t)ctx->cu_count * 16) blocks = (int64_t)ctx->cu_count * 16;
-    hipLaunchKernelGGL(k_maxpool_2x2s2, dim3((int)blocks), dim3(kBlock), 0, ctx->stream, x, y, g.H, g.W,
-                       g.oh, g.ow, pairs);
+    if (relu)
+      hipLaunchKernelGGL(k_maxpool_2x2s2<true>, dim3((int)blocks), dim3(kBlock), 0, ctx->stream, x, y, g.H, g.W,
+                         g.oh, g.ow, pairs);
+    else
+      hipLaunchKernelGGL(k_maxpool_2x2s2<false>, dim3((int)blocks), dim3(kBlock), 0, ctx->stream, x, y, g.H, g.W,
+                         g.oh, g.ow, pairs);
   } else {
     int64_t blocks = (total + kBlock - 1) / kBlock;
     if (blocks > (int64_t)ctx->cu_count * 16) blocks = (int64_t)ctx->cu_count * 16;
-    hipLaunchKernelGGL(k_maxpool2d, dim3((int)blocks), dim3(kBlock), 0, ctx->stream, x, y, g, total);
+    if (relu) hipLaunchKernelGGL(k_maxpool2d<true>, dim3((int)blocks), dim3(kBlock), 0, ctx->stream, x, y, g, total);
+    else hipLaunchKernelGGL(k_maxpool2d<false>, dim3((int)blocks), dim3(kBlock), 0, ctx->stream, x, y, g, total);
   }
   return gh_check_hip(ctx, hipGetLastError(), "maxpool2d launch");
 }

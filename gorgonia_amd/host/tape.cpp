@@ -289,13 +289,13 @@ static std::string op_name(const OpSpec& op) {
       return std::string("conv2d") + (op.fuse_bn ? "+batchnorm(eval)" : "") +
              (op.fuse_act_relu ? "+rectify" : op.fuse_act_leaky ? "+leakyrelu" : "") +
              (op.fuse_pool2 ? "+maxpool2d" : "");
-    case OpKind::MaxPool2D: return "maxpool2d";
+    case OpKind::MaxPool2D: return op.relu_input ? "rectify+maxpool2d" : "maxpool2d";
     case OpKind::BatchNorm: return "batchnorm(eval)";
     case OpKind::Rectify: return "rectify";
     case OpKind::LeakyRelu: return "leakyrelu";
     case OpKind::SoftMax: return "softmax";
     case OpKind::Reshape: return "reshape";
-    case OpKind::MaxPool2DDiff: return "maxpool2d.diff";
+    case OpKind::MaxPool2DDiff: return op.relu_input ? "rectify+maxpool2d.diff" : "maxpool2d.diff";
     case OpKind::Conv2dDiffData: return "conv2d.diff.image";
     case OpKind::Conv2dDiffFilter: return "conv2d.diff.filter";
     case OpKind::BatchNormTrain: return "batchnorm(train)";
@@ -392,7 +392,7 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       const int64_t np = p[2];
       gh_cmd c{};
       c.opcode = GH_OP_MAXPOOL2D;
-      c.flags = (np == 4 ? GH_FLAG_EXPLICIT_PAD : 0) | dtype_flag(x.dt);
+      c.flags = (np == 4 ? GH_FLAG_EXPLICIT_PAD : 0) | (op.relu_input ? GH_FLAG_ACT_RELU : 0) | dtype_flag(x.dt);
       c.ptr[0] = x.mem; c.ptr[1] = prealloc.mem;
       for (int i = 0; i < 4; i++) c.dim[i] = x.shape[i];
       c.dim[4] = p[0]; c.dim[5] = p[1];
@@ -456,7 +456,7 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       if (x.dt == Dtype::Other || in[1]->dt != x.dt) return bad("MaxPool2DDiff: Unsupported Dtype");
       gh_cmd c{};
       c.opcode = GH_OP_MAXPOOL2D_BWD;
-      c.flags = (np == 4 ? GH_FLAG_EXPLICIT_PAD : 0) | dtype_flag(x.dt);
+      c.flags = (np == 4 ? GH_FLAG_EXPLICIT_PAD : 0) | (op.relu_input ? GH_FLAG_ACT_RELU : 0) | dtype_flag(x.dt);
       c.ptr[0] = x.mem; c.ptr[1] = in[1]->mem; c.ptr[2] = prealloc.mem;
       for (int i = 0; i < 4; i++) c.dim[i] = x.shape[i];
       c.dim[4] = p[0]; c.dim[5] = p[1];
@@ -721,6 +721,50 @@ int Graph::FuseActivations() {
     n.inputs = inputs;
     p.fused_away = true;
     fused++;
+  }
+  fused += fuse_pooled_rectify();
+  return fused;
+}
+
+// The training pattern around a pooled activation:
+//   a = Rectify(z); p = MaxPool2D(a); ...; da = MaxPool2DDiff(a, g); dz = RectifyDiff(z, da)
+// with a read by nothing but the pool and its gradient, and da by nothing but dz.  The pool then
+// reads z through the activation, and dz becomes one operator that scans the windows over
+// z * (z >= 0) and masks the result with (z >= 0): a and da are never stored, and every value
+// that is stored has the bits the four operators would have given it.
+int Graph::fuse_pooled_rectify() {
+  int fused = 0;
+  const size_t N = nodes_.size();
+  std::vector<std::vector<int>> users(N);
+  for (auto& n : nodes_)
+    if (!n.fused_away)
+      for (int i : n.inputs) users[(size_t)i].push_back(n.id);
+  for (auto& a : nodes_) {
+    if (a.fused_away || a.is_input || a.read_into || a.op.kind != OpKind::Rectify || a.dt != Dtype::Float32) continue;
+    if (a.inputs.size() != 1 || users[(size_t)a.id].size() != 2) continue;
+    const int z = a.inputs[0];
+    Node* pool = nullptr;
+    Node* diff = nullptr;
+    for (int u : users[(size_t)a.id]) {
+      Node& n = nodes_[(size_t)u];
+      if (n.op.kind == OpKind::MaxPool2D && n.inputs.size() == 1 && !n.op.relu_input) pool = &n;
+      if (n.op.kind == OpKind::MaxPool2DDiff && n.inputs.size() == 2 && n.inputs[0] == a.id && n.inputs[1] != a.id &&
+          !n.op.relu_input)
+        diff = &n;
+    }
+    if (!pool || !diff || diff->read_into || diff->op.ints != pool->op.ints) continue;
+    if (users[(size_t)diff->id].size() != 1) continue;
+    Node& dz = nodes_[(size_t)users[(size_t)diff->id][0]];
+    if (dz.op.kind != OpKind::RectifyDiff || dz.inputs.size() != 2 || dz.inputs[0] != z || dz.inputs[1] != diff->id) continue;
+    if (nodes_[(size_t)z].dt != Dtype::Float32 || nodes_[(size_t)z].fused_away) continue;
+    pool->op.relu_input = true;
+    pool->inputs[0] = z;
+    dz.op = diff->op;
+    dz.op.relu_input = true;
+    dz.inputs = {z, diff->inputs[1]};
+    a.fused_away = true;
+    diff->fused_away = true;
+    fused += 2;
   }
   return fused;
 }

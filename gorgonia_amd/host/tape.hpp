@@ -79,6 +79,9 @@ struct OpSpec {
   bool fuse_pool2 = false;
   bool fuse_bias = false;     // MatMul only: the BroadcastAdd of a row vector that follows (last input)
   bool fuse_softmax = false;  // MatMul only: the SoftMax that follows, where gh_gemm_can_softmax allows
+  // MaxPool2D / MaxPool2DDiff: input 0 is the value before a Rectify and is read through it; the
+  // diff also applies the Rectify's own gradient (it stands for RectifyDiff(z, MaxPool2DDiff(Rectify(z), g)))
+  bool relu_input = false;
 };
 
 // Output shape of an op (InferShape of each reference op); error if the inputs
@@ -125,6 +128,7 @@ class Graph {
   // and inputs; the values it stores are bit-identical to the unfused chain's.
   // Returns the number of operators folded away.
   int FuseActivations();
+  int fuse_pooled_rectify();   // part of FuseActivations: the Rectify between a pool and both gradients
   const std::vector<Node>& Nodes() const { return nodes_; }
   std::vector<Node>& Nodes() { return nodes_; }
 

@@ -171,6 +171,8 @@ enum gh_unaryfn {
  *             shape B,F,oh/2,ow/2; only where gh_conv2d_can_pool says so)
  * MAXPOOL2D   ptr[0]=x ptr[1]=y            dim[0..3]=B,C,H,W dim[4..5]=kh,kw
  *             dim[6..9]=padN,padS,padW,padE dim[10..11]=strideH,strideW
+ *             GH_FLAG_ACT_RELU (float32): x is read through Rectify, y = pool(x*(x>=0));
+ *             the activation's result is never stored
  * BN_INFER    ptr[0]=x ptr[1]=y ptr[2]=mean ptr[3]=var [ptr[4]=gamma ptr[5]=beta]
  *             dim[0..2]=B,C,S  f[0]=eps
  * RELU        ptr[0]=x ptr[1]=y            dim[0]=n
@@ -181,6 +183,9 @@ enum gh_unaryfn {
  * FILL        ptr[0]=A                     dim[0]=n f[0]=value
  * MAXPOOL2D_BWD     ptr[0]=x ptr[1]=dy ptr[2]=dx ; dims as MAXPOOL2D.  dx gets, per element,
  *             the dy of every window whose argmax it is (first maximum in scan order)
+ *             GH_FLAG_ACT_RELU (float32): x is the value before a Rectify whose result was
+ *             pooled; dx = (x>=0) * that gradient taken over x*(x>=0) - MaxPool2DDiff then the
+ *             activation's gradient, with their bits, in one pass
  * CONV2D_BWD_DATA   ptr[0]=dy ptr[1]=w ptr[2]=dx ; dims as CONV2D (B,C,H,W describe x / dx)
  * CONV2D_BWD_FILTER ptr[0]=x ptr[1]=dy ptr[2]=dw ; dims as CONV2D
  * BN_TRAIN    ptr[0]=x ptr[1]=y ptr[2]=running_mean ptr[3]=running_var (both updated)

@@ -7,6 +7,7 @@ reduction order differs from the CPU's sequential sums)."""
 import numpy as np
 import pytest
 
+from gorgonia_amd import _ffi
 from gorgonia_amd import device as D
 from gorgonia_amd import synth
 from oracle import binding as O
@@ -47,6 +48,37 @@ def test_maxpool_backward_bit_exact(ctx, cfg):
         for p in (dx_, dy_, dd):
             ctx.free(p)
         assert_bits_equal(got, O.maxpool2d_bwd(x, dy, kernel, pad, stride), f"maxpool backward {cfg}")
+
+
+@pytest.mark.parametrize("cfg", POOL_CASES)
+def test_maxpool_through_rectify_bit_exact(ctx, cfg):
+    """GH_FLAG_ACT_RELU on the pooling commands: y = MaxPool2D(Rectify(z)) and its gradient with respect
+    to z, each in one pass, with the bits of the separate operators (oracle: relu, pool, pool gradient,
+    then dy * (z >= 0)).  Inputs with zeros of both signs and exact ties inside windows."""
+    B, C, H, W, kernel, pad, stride = cfg
+    rng = np.random.default_rng(2)
+    zs = [synth.normal(17, (B, C, H, W)), rng.integers(-2, 3, (B, C, H, W)).astype(np.float32)]
+    zs.append(np.where(rng.random((B, C, H, W)) < 0.3, np.float32(-0.0), zs[1]).astype(np.float32))
+    for z in zs:
+        oh, ow = O.maxpool_out_hw(H, W, kernel[0], kernel[1], pad, stride)
+        dy = synth.normal(18, (B, C, oh, ow))
+        a = O.relu(z).reshape(z.shape)
+        want_y = O.maxpool2d(a, kernel, pad, stride)
+        da = O.maxpool2d_bwd(a, dy, kernel, pad, stride)
+        want_dz = (da * (z >= 0).astype(np.float32)).astype(np.float32)
+        pz, pdy = ctx.upload(z), ctx.upload(dy)
+        py, pdz = ctx.malloc(want_y.size * 4), ctx.malloc(z.size * 4)
+        ctx.run([D.cmd_fill(py, want_y.size, np.nan), D.cmd_fill(pdz, z.size, np.nan)])
+        fwd = D.cmd_maxpool2d(pz, py, B, C, H, W, kernel[0], kernel[1], pad, stride)
+        bwd = D.cmd_maxpool2d_bwd(pz, pdy, pdz, B, C, H, W, kernel[0], kernel[1], pad, stride)
+        fwd.flags |= _ffi.FLAG_ACT_RELU
+        bwd.flags |= _ffi.FLAG_ACT_RELU
+        ctx.run([fwd, bwd])
+        got_y, got_dz = ctx.d2h(py, want_y.shape), ctx.d2h(pdz, z.shape)
+        for p in (pz, pdy, py, pdz):
+            ctx.free(p)
+        assert_bits_equal(got_y, want_y, f"pool(relu(z)) {cfg}")
+        assert_bits_equal(got_dz, want_dz, f"gradient of pool(relu(z)) {cfg}")
 
 
 @pytest.mark.parametrize("shape", [(1, 1), (7, 10), (128, 10), (5, 64), (3, 65), (4, 1000)])

@@ -41,6 +41,31 @@ def test_convnet_training_step_gradients(ctx):
     m.Close()
 
 
+def test_training_step_with_folded_operators_keeps_every_bit(ctx):
+    """FuseActivations on the training graph: the Rectify between each convolution's pool and the two
+    gradients is read through by both (its result and the pooling gradient are never stored) and the last
+    product carries its SoftMax.  Output and every weight gradient equal the unfolded machine's bit for bit,
+    on the first step and on the second (weights updated on the device), plainly run and replayed."""
+    inp = configs.convnet_inputs(24)
+    y = _onehot(24)
+    for replay in (False, True):
+        g0, outs0 = configs.build_convnet_train(inp, y, 0.05)
+        m0 = G.NewTapeMachine(g0)
+        g1, outs1 = configs.build_convnet_train(inp, y, 0.05)
+        m1 = G.NewTapeMachine(g1, fuse_activations=True, graph_replay=replay)
+        assert m1.fused == 7           # 3 x (Rectify, MaxPool2DDiff) + the SoftMax
+        prog = m1.program()
+        assert prog.count("rectify+maxpool2d.diff") == 3 and prog.count("rectify+maxpool2d") == 6
+        assert prog.count("rectifyDiff") == 1       # the dense layer's activation is not pooled
+        ops = lambda m: len([l for l in m.program().splitlines() if "execOp" in l])
+        assert ops(m1) == ops(m0) - 7
+        for step in range(3):
+            m0.RunAll(); m1.RunAll()
+            for k in outs0:
+                assert_bits_equal(outs1[k], outs0[k], f"{k}, step {step}, replay={replay}")
+        m0.Close(); m1.Close()
+
+
 def test_training_steps_replayed_from_a_graph(ctx):
     """Steps 2.. run as hipGraph replays; the in-place weight updates persist
     between replays and the cost goes down."""
