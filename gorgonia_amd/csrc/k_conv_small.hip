@@ -387,6 +387,10 @@ bool small_plan(const gh_cmd& c, bool pool, SmallPlan* out) {
   g.nout = pool ? g.IPB * g.ph * g.pw : g.IPB * g.oh * g.ow;
   g.mPPI = magic_of(g.ppi); g.mOW = magic_of(g.ow); g.mPW = magic_of(g.pw); g.mPQ = magic_of(g.ph * g.pw);
   g.mNOUT = magic_of(g.nout); g.mCH = magic_of(g.CH);
+  // 128 channels and more leave LDS for only 16 filter rows of all of K: half the B-operand reuse.
+  // The patch kernel stages K quad by quad and keeps 32 (128 -> 64 at 7 x 7, batch 128: 16.7 us
+  // against 21.3 here); where it takes the shape, it has it.
+  if (bestTM == 1 && F >= 32 && C >= 128 && gh_conv_patch_takes(c)) return false;
   out->g = g; out->WV = WV; out->TM = bestTM; out->TN = bestTN; out->NQ = NQ; out->lds = best_lds;
   return true;
 }
