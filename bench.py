@@ -338,7 +338,7 @@ def bench_convnet_machines(steps, warmup, count=2, batch=128):
     return count * steps * batch / dt, results
 
 
-def bench_yolo(steps, warmup, resident_input=True, borrow_output=True):
+def bench_yolo(steps, warmup, resident_input=True, borrow_output=True, borrow_input=False):
     """Config 5: Tiny-YOLO-v2-shaped forward, batch 8 x 3 x 416 x 416, on the tape
     machine with conv+BatchNorm+LeakyReLU(+MaxPool) folded, graph replay,
     weights and input resident.  borrow_output: the 8 x 425 x 13 x 13 result (2.3 MB) is read
@@ -346,8 +346,11 @@ def bench_yolo(steps, warmup, resident_input=True, borrow_output=True):
     otherwise Read copies it from there into the caller's array on every step."""
     from gorgonia_amd import configs, graph as G
     inp = configs.yolo_inputs(8, 416)
-    g, outs = configs.build_yolo(inp, resident_input=resident_input, borrow_output=borrow_output)
+    g, outs = configs.build_yolo(inp, resident_input=resident_input, borrow_output=borrow_output,
+                                 borrow_input=borrow_input)
     m = G.NewTapeMachine(g, graph_replay=replay_mode(), fuse_activations=True)
+    if borrow_input:
+        m.input(g.x_node)[...] = inp["x"]
     for _ in range(max(warmup, WARM_RUNS)):
         m.RunAll()
     eng = m.engine()
@@ -543,9 +546,12 @@ def main():
         ms_yolo, yolo_out, yolo_inp = bench_yolo(max(20, a.steps // 4), a.warmup)
         ms_yolo_h2d, _, _ = bench_yolo(max(10, a.steps // 8), a.warmup, resident_input=False)
         ms_yolo_copy, yolo_out_copy, _ = bench_yolo(max(10, a.steps // 8), a.warmup, borrow_output=False)
+        ms_yolo_h2d_b, yolo_out_b, _ = bench_yolo(max(10, a.steps // 8), a.warmup, resident_input=False, borrow_input=True)
         yolo = {"ms_per_step": round(ms_yolo, 4), "images_s": round(8 / ms_yolo * 1e3, 1),
                 "TFLOPs": round(31_080_857_600 / ms_yolo / 1e9, 2), "flop_per_step": 31_080_857_600,
                 "ms_per_step_with_input_h2d": round(ms_yolo_h2d, 4),
+                "ms_per_step_with_input_h2d_from_borrowed_pinned_buffer": round(ms_yolo_h2d_b, 4),
+                "borrowed_input_output_equals_resident": bool(np.array_equal(yolo_out, yolo_out_b)),
                 "output": "read in the machine's pinned buffer (ReadBorrowed), 2298400 bytes",
                 "ms_per_step_output_copied_to_caller": round(ms_yolo_copy, 4),
                 "copied_output_equals_borrowed": bool(np.array_equal(yolo_out, yolo_out_copy))}

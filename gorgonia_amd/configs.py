@@ -156,9 +156,12 @@ def build_convnet_train(inp, onehot, lr, read_grads=True, solver="set"):
     return g, outs
 
 
-def build_yolo(inp, resident=True, resident_input=False, borrow_output=False):
+def build_yolo(inp, resident=True, resident_input=False, borrow_output=False, borrow_input=False):
     g = G.NewGraph()
     h = G.NewTensor(g, inp["x"], resident_input)
+    if borrow_input:   # the batch is written into TapeMachine.input(g.x_node), the machine's pinned buffer
+        G.LetBorrowed(h)
+    g.x_node = h
     for i in range(7):
         w = G.NewTensor(g, inp[f"w{i}"], resident)
         h = G.Conv2d(h, w, (3, 3), (1, 1), (1, 1), (1, 1))
