@@ -242,3 +242,36 @@ def test_borrowed_reads_in_the_program():
     m2.Close()
     with pytest.raises(EngineError):
         g.lib.ghh_graph_read_borrowed(g.h, 99) and g._check(g.lib.ghh_graph_read_borrowed(g.h, 99))
+
+
+def test_pooled_rectify_is_folded_only_when_nothing_else_reads_it():
+    """FuseActivations folds Rectify into the pool and both gradients (a = Rectify(z); MaxPool2D(a);
+    RectifyDiff(z, MaxPool2DDiff(a, g))) only when a and the pooling gradient have no other reader, the
+    two pooling operators agree on their geometry and both gradients hang off the same z."""
+    def build(read_a=False, other_geometry=False, read_da=False, other_z=False):
+        g = G.NewGraph()
+        x = G.NewTensor(g, np.zeros((2, 3, 8, 8), np.float32))
+        w = G.NewTensor(g, np.zeros((4, 3, 3, 3), np.float32), resident=True)
+        z = G.Conv2d(x, w, (3, 3), (1, 1), (1, 1), (1, 1))
+        a = G.Rectify(z)
+        p = G.MaxPool2D(a, (2, 2), (0, 0), (2, 2))
+        G.Read(p)
+        grad = G.NewTensor(g, np.zeros((2, 4, 4, 4), np.float32))
+        da = G.MaxPool2DDiff(a, grad, (2, 2), (0, 0), (1, 1) if other_geometry else (2, 2)) if not other_geometry else \
+            G.MaxPool2DDiff(a, G.NewTensor(g, np.zeros((2, 4, 7, 7), np.float32)), (2, 2), (0, 0), (1, 1))
+        z2 = G.Conv2d(x, w, (3, 3), (1, 1), (1, 1), (1, 1)) if other_z else z
+        G.Read(G.RectifyDiff(z2, da))
+        if read_a:
+            G.Read(a)
+        if read_da:
+            G.Read(da)
+        return g
+    m = G.NewTapeMachine(build(), compile_only=True, fuse_activations=True)
+    assert m.fused == 2 and m.program().count("rectify+maxpool2d") == 2 and "rectifyDiff" not in m.program()
+    m.Close()
+    for kw in (dict(read_a=True), dict(other_geometry=True), dict(read_da=True), dict(other_z=True)):
+        m = G.NewTapeMachine(build(**kw), compile_only=True, fuse_activations=True)
+        # (with a z of its own the activation folds into its convolution instead, the ordinary way)
+        assert m.fused == (1 if "other_z" in kw else 0) and ("conv2d+rectify" in m.program()) == ("other_z" in kw), kw
+        assert "rectify+maxpool2d" not in m.program() and "rectifyDiff" in m.program(), kw
+        m.Close()
