@@ -225,13 +225,13 @@ def bench_linalg(ctx, iters):
 # WRITE_SIZE runs of this script (KiB per dispatch; FETCH_SIZE scaled by 2.0,
 # WRITE_SIZE by 1.0, the factors a 64 MiB device copy in the same runs gives).
 MEASURED_TRAFFIC_BYTES = {
-    "conv0": (2 * 937.6 + 3232.0) * 1024,
-    "conv1": (2 * 1953.3 + 1568.0) * 1024,
-    "conv2": (2 * 2033.0 + 576.0) * 1024,
+    "conv0": (2 * 937.5 + 3232.0) * 1024,
+    "conv1": (2 * 1953.6 + 1568.0) * 1024,
+    "conv2": (2 * 2033.1 + 576.0) * 1024,
 }
 # SQ_VALU_MFMA_BUSY_CYCLES / (128 * GRBM_GUI_ACTIVE) of the same kernels in a rocprofv3 --pmc run of this
 # script (eager launches, one at a time: launch and drain are inside GUI_ACTIVE, clocks are not sustained)
-MEASURED_MFMA_BUSY = {"conv0": 0.0, "conv1": 0.285, "conv2": 0.225}
+MEASURED_MFMA_BUSY = {"conv0": 0.0, "conv1": 0.288, "conv2": 0.226}
 CONV_KERNEL_NAME = {"conv0": "k_conv3x3_direct<1,2>", "conv1": "k_conv3x3_small<8,1,13,1>", "conv2": "k_conv3x3_small<8,1,9,2>"}
 
 CONVNET_LAYERS = [  # (name, B-relative shape) of configuration 4

@@ -263,6 +263,11 @@ int gh_memcpy_d2d(gh_ctx* ctx, gh_devptr dst, gh_devptr src, int64_t bytes) {
 }
 
 static int dispatch(gh_ctx* ctx, const gh_cmd& c) {
+  // the streaming kernels keep their own account of what they touch; everything else marks its
+  // operands as recently used (sizes unknown here: by start address), so that an elementwise
+  // kernel behind a product or a convolution reads the result as the cache-resident data it is
+  if (c.opcode != GH_OP_ELEM_BIN && c.opcode != GH_OP_ELEM_UNARY && c.opcode != GH_OP_BCAST_BIN && c.opcode != GH_OP_NOP)
+    for (uint64_t p : c.ptr) ctx->llc.touch(p, 0, false);
   switch (c.opcode) {
     case GH_OP_NOP: return GH_OK;
     case GH_OP_ELEM_BIN: return gh_launch_elem_bin(ctx, c);

@@ -563,6 +563,16 @@ inline bool stream_bytes(int64_t bytes) {
   return bytes >= limit;
 }
 
+// ... and so are operands the cache has lost by now: every tensor the kernel reads was last
+// touched more than a cache's worth of traffic ago (or never).  Small launches stay plain.
+constexpr uint64_t kWarmWindow = 192ull << 20;
+constexpr int64_t kColdMinBytes = 16ll << 20;
+inline bool cold_inputs(const gh_ctx* ctx, int64_t bytes, uint64_t a, uint64_t b) {
+  static const bool off = getenv("GORGONIA_HIP_EW_NO_RESIDENCY") != nullptr;   // tuning switch: size rule only
+  if (off || bytes < kColdMinBytes) return false;
+  return !(a && ctx->llc.warm(a, kWarmWindow)) && !(b && ctx->llc.warm(b, kWarmWindow));
+}
+
 template <int FN, class T>
 int launch_bin_fn(gh_ctx* ctx, const gh_cmd& c) {
   const T* A = (const T*)(uintptr_t)c.ptr[0];
@@ -582,7 +592,15 @@ int launch_bin_fn(gh_ctx* ctx, const gh_cmd& c) {
   if (mode == GH_SS) vec = false;
   const int gv = grid_chunks(ctx, n / N);
   const int gs = grid_for(ctx, n, 4);
-  const bool stream = stream_bytes((int64_t)sizeof(T) * n * (mode == GH_VV ? 3 : 2));
+  const int64_t tbytes = (int64_t)sizeof(T) * n;
+  const uint64_t va = mode == GH_SV ? 0 : c.ptr[0], vb = mode == GH_VS ? 0 : c.ptr[1];   // the tensor operands
+  const bool stream = stream_bytes(tbytes * (mode == GH_VV ? 3 : 2)) ||
+                      (mode != GH_SS && cold_inputs(ctx, tbytes * (mode == GH_VV ? 3 : 2), va, vb));
+  if (mode != GH_SS) {
+    ctx->llc.touch(va, tbytes, true);
+    ctx->llc.touch(vb, tbytes, true);
+    ctx->llc.touch(dptr, tbytes, dptr != va && dptr != vb);
+  }
 #define GH_LAUNCH_MODE(M)                                                                   \
   if (vec && stream) hipLaunchKernelGGL((k_bin_vec<FN, T, M, true>), dim3(gv), dim3(kBlock), 0, ctx->stream, A, B, Dst, n); \
   else if (vec) hipLaunchKernelGGL((k_bin_vec<FN, T, M, false>), dim3(gv), dim3(kBlock), 0, ctx->stream, A, B, Dst, n); \
@@ -625,8 +643,12 @@ int launch_unary_fn(gh_ctx* ctx, const gh_cmd& c) {
   const int64_t n = c.dim[0];
   constexpr int N = VecOf<T>::N;
   if (n == 0) return GH_OK;
+  const int64_t tbytes = (int64_t)sizeof(T) * n;
+  const bool stream = stream_bytes(tbytes * 2) || cold_inputs(ctx, tbytes * 2, c.ptr[0], 0);
+  ctx->llc.touch(c.ptr[0], tbytes, true);
+  ctx->llc.touch(dptr, tbytes, dptr != c.ptr[0]);
   if (n >= N && aligned16(c.ptr[0]) && aligned16(dptr)) {
-    if (stream_bytes((int64_t)sizeof(T) * n * 2))
+    if (stream)
       hipLaunchKernelGGL((k_unary_vec<FN, T, true>), dim3(grid_chunks(ctx, n / N)), dim3(kBlock), 0, ctx->stream, A, Dst, n);
     else
       hipLaunchKernelGGL((k_unary_vec<FN, T, false>), dim3(grid_chunks(ctx, n / N)), dim3(kBlock), 0, ctx->stream, A, Dst, n);
@@ -668,7 +690,9 @@ int launch_bcast_fn(gh_ctx* ctx, const gh_cmd& c) {
     if (gy > need) gy = need;
     if (gy < 1) gy = 1;
     if (gy > 65535) gy = 65535;
-    const bool stream = stream_bytes(8 * n);
+    const bool stream = stream_bytes(8 * n) || cold_inputs(ctx, 8 * n, c.ptr[1], 0);
+    ctx->llc.touch(c.ptr[1], 4 * n, true);
+    ctx->llc.touch(c.ptr[0], 4 * n, c.ptr[0] != c.ptr[1]);
 #define GH_BCAST_ROW(L_, S_)                                                                              \
   hipLaunchKernelGGL((k_bcast_row<FN, L_, S_>), dim3(gx, (int)gy), dim3(kBlock), 0, ctx->stream, dst, big, \
                      small, outer, colv)

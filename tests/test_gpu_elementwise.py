@@ -233,6 +233,52 @@ def test_broadcast_bit_exact(ctx, fn, shape, left):
     ctx.free(db); ctx.free(ds); ctx.free(dd)
 
 
+def test_large_operands_cold_then_warm_same_bits(ctx):
+    """Tensors of 32 MiB: the first launch finds them nowhere in the library's account of the
+    last-level cache and streams them (non-temporal accesses), the repeat finds them there and
+    uses plain accesses, and a launch behind 400 MiB of other traffic streams again.  Every one
+    stores the oracle's bits, in place and into a separate destination."""
+    n = 8 << 20
+    a, b = _special(n, 61), _special(n, 62)[::-1].copy()
+    row = synth.uniform(63, (4096,), -4, 4)
+    want_mul = O.binop("mul", "vv", a, b)
+    want_tanh = O.unary("tanh", a)
+    want_vs = O.binop("add", "vs", a, np.array([1.5], np.float32))
+    want_bc = O.bcast_binop("add", a, row, n // 4096, 4096, 1, False)
+    da, db, dd, dr = ctx.upload(a), ctx.upload(b), ctx.malloc(4 * n), ctx.upload(row)
+    ds = ctx.upload(np.array([1.5], np.float32))
+    filler = [ctx.malloc(64 << 20) for _ in range(3)]
+
+    def check(tag):
+        ctx.run(D.cmd_bin("mul", "vv", da, db, n, dst=dd))
+        assert_bits_equal(ctx.d2h(dd, (n,)), want_mul, f"mul vv, {tag}")
+        ctx.run(D.cmd_unary("tanh", da, n, dst=dd))
+        assert ulp_diff(ctx.d2h(dd, (n,)), want_tanh).max() <= 2, f"tanh, {tag}"
+        ctx.run(D.cmd_bin("add", "vs", da, ds, n, dst=dd))
+        assert_bits_equal(ctx.d2h(dd, (n,)), want_vs, f"add vs, {tag}")
+        ctx.run(D.cmd_bcast("add", dd, da, dr, n // 4096, 4096, 1))
+        assert_bits_equal(ctx.d2h(dd, (n,)), want_bc, f"broadcast add, {tag}")
+
+    check("never seen")
+    check("just used")
+    for rep in range(3):               # 3 x 3 x 64 MiB through the streaming kernels
+        for f in filler:
+            ctx.run(D.cmd_unary("neg", f, 16 << 20))
+    check("long unused")
+    # in place, cold then warm
+    for tag in ("cold", "warm"):
+        ctx.run(D.cmd_copy(dd, da, 4 * n))
+        if tag == "cold":
+            for f in filler:
+                ctx.run(D.cmd_unary("neg", f, 16 << 20))
+            for f in filler:
+                ctx.run(D.cmd_unary("neg", f, 16 << 20))
+        ctx.run(D.cmd_bin("mul", "vv", dd, db, n))
+        assert_bits_equal(ctx.d2h(dd, (n,)), want_mul, f"mul vv in place, {tag}")
+    for p in [da, db, dd, dr, ds] + filler:
+        ctx.free(p)
+
+
 def test_relu_and_leaky_bit_exact(ctx):
     for n in [1, 7, 4099, (1 << 20) + 1]:
         x = _special(n, 61)
