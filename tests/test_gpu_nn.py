@@ -170,7 +170,7 @@ def test_conv_epilogue_batchnorm_activation_bit_exact(ctx, cfg):
 
 
 @pytest.mark.parametrize("cfg", [(3, 1, 28, 28, 32, 1), (2, 3, 21, 19, 16, 1), (2, 4, 10, 12, 6, 0),
-                                 (1, 2, 7, 7, 9, 1),
+                                 (1, 2, 7, 7, 9, 1), (2, 2, 9, 8, 7, 2), (1, 4, 6, 11, 5, 2),   # padding wider than one
                                  # the matrix-core kernel: blocks of whole rows (even height, blocks crossing
                                  # images), whole images (odd height), 128-pixel blocks, rectangular tiles
                                  (5, 32, 14, 14, 64, 1), (3, 16, 7, 7, 40, 1), (130, 8, 7, 7, 8, 1),

@@ -275,3 +275,40 @@ def test_pooled_rectify_is_folded_only_when_nothing_else_reads_it():
         assert m.fused == (1 if "other_z" in kw else 0) and ("conv2d+rectify" in m.program()) == ("other_z" in kw), kw
         assert "rectify+maxpool2d" not in m.program() and "rectifyDiff" in m.program(), kw
         m.Close()
+
+
+def test_pooling_query_over_random_geometries():
+    """gh_conv2d_can_pool runs every 3x3 kernel's planner on the host.  Over a few thousand random
+    geometries (channel counts around every kernel's limits, images from 3x3 to 500x500) it must
+    answer 0 or 1 without a device, say no to everything the pool cannot follow (other kernel sizes,
+    strides, dilation, float64, results smaller than a window) and give one answer per geometry."""
+    from gorgonia_amd import _ffi, device as D
+    lib = _ffi.load()
+    rng = np.random.default_rng(123)
+    yes = 0
+    for it in range(4000):
+        B = int(rng.choice([1, 2, 3, 8, 16, 128, 130]))
+        C = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 24, 32, 48, 64, 96, 128, 256, 512, 1000]))
+        F = int(rng.choice([1, 5, 16, 17, 32, 40, 64, 128, 425, 1024]))
+        H = int(rng.choice([3, 4, 7, 13, 14, 16, 17, 26, 28, 52, 104, 208, 416, 500]))
+        W = int(rng.choice([3, 4, 7, 13, 14, 16, 17, 26, 28, 52, 104, 208, 416, 500]))
+        k = int(rng.choice([3, 3, 3, 1, 5]))
+        pad = int(rng.choice([0, 1, 1, 2]))
+        stride = int(rng.choice([1, 1, 1, 2]))
+        dil = int(rng.choice([1, 1, 1, 2]))
+        if H + 2 * pad < dil * (k - 1) + 1 or W + 2 * pad < dil * (k - 1) + 1:
+            continue
+        if B * C * H * W >= 2 ** 31 or B * F * H * W >= 2 ** 31:
+            continue
+        cmd = D.cmd_conv2d(0x1000, 0x2000, 0x3000, B, C, H, W, F, k, k, (pad, pad), (stride, stride), (dil, dil))
+        a = lib.gh_conv2d_can_pool(cmd)
+        assert a in (0, 1) and a == lib.gh_conv2d_can_pool(cmd)
+        oh = (H + 2 * pad - (dil * (k - 1) + 1)) // stride + 1
+        ow = (W + 2 * pad - (dil * (k - 1) + 1)) // stride + 1
+        if a:
+            yes += 1
+            assert k == 3 and stride == 1 and dil == 1 and oh >= 2 and ow >= 2, (B, C, H, W, F, k, pad, stride, dil)
+        f64 = D.cmd_conv2d(0x1000, 0x2000, 0x3000, B, C, H, W, F, k, k, (pad, pad), (stride, stride), (dil, dil),
+                           dtype=_ffi.F64)
+        assert lib.gh_conv2d_can_pool(f64) == 0
+    assert yes > 300
