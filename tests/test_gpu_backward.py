@@ -164,6 +164,28 @@ def test_conv_backward_vs_oracle(ctx, cfg):
     assert_bits_equal(dwi, owi, f"integer dw {cfg}")
 
 
+def test_small_image_filter_gradient_random_geometries(ctx):
+    """Forty random geometries in the small-image filter-gradient kernel's domain (and just outside it:
+    fewer than four output pixels, 15 filters) against the oracle: <= 1e-5 on real data, exact on integers."""
+    rng = np.random.default_rng(2024)
+    for it in range(40):
+        B = int(rng.integers(1, 41)); C = int(rng.choice([16, 32, 48, 64])); F = int(rng.integers(15, 101))
+        H = int(rng.integers(3, 17)); W = int(rng.integers(3, 17)); pad = int(rng.integers(0, 2))
+        cfg = (B, C, H, W, F, pad)
+        oh, ow = H + 2 * pad - 2, W + 2 * pad - 2
+        x = synth.uniform(600 + it, (B, C, H, W), -1, 1)
+        w = synth.he_normal(700 + it, (F, C, 3, 3))
+        dy = synth.normal(800 + it, (B, F, oh, ow))
+        _, dw = gpu_conv_bwd(ctx, x, w, dy, (pad, pad), (1, 1), (1, 1))
+        _, rw = O.conv2d_bwd(x, w, dy, (pad, pad), (1, 1), (1, 1))
+        assert rel_frobenius(dw, rw) <= TOL, f"dw {cfg}: {rel_frobenius(dw, rw):.3e}"
+        xi = rng.integers(-3, 4, x.shape).astype(np.float32)
+        di = rng.integers(-2, 3, dy.shape).astype(np.float32)
+        _, dwi = gpu_conv_bwd(ctx, xi, w, di, (pad, pad), (1, 1), (1, 1))
+        _, owi = O.conv2d_bwd(xi, w, di, (pad, pad), (1, 1), (1, 1))
+        assert_bits_equal(dwi, owi, f"integer dw {cfg}")
+
+
 BN_CASES = [(3, 2, 1), (6, 4, 1), (2, 2, 4), (4, 3, 25), (8, 16, 26 * 26), (2, 32, 104 * 104), (128, 10, 1)]
 
 
