@@ -176,8 +176,8 @@ __device__ __forceinline__ float sigmoid_f32_fast(float x) {
   const float e_lo = ldexpf(tl, p.n);
   const float d_hi = 1.0f + e_hi;
   const float d_lo = (e_hi - (d_hi - 1.0f)) + e_lo;
-  float r = __builtin_amdgcn_rcpf(d_hi);
-  r = __builtin_fmaf(__builtin_fmaf(-d_hi, r, 1.0f), r, r);
+  // the hardware estimate of 1/d is good to an ulp; the residual step below squares that error away
+  const float r = __builtin_amdgcn_rcpf(d_hi);
   const bool neg = x < 0.0f;
   const float num_hi = neg ? e_hi : 1.0f, num_lo = neg ? e_lo : 0.0f;
   const float q0 = num_hi * r;
