@@ -12,9 +12,12 @@
 //     images.  It takes the images a few at a time (as many as give about 200 output pixels):
 //     their dy rows go to LDS as dyL[filter][k] with k = (image, pixel) and a pitch of 4 mod
 //     64, so the 64 lanes of an A fetch hit 64 banks; their x planes go to LDS with a zero
-//     halo, so a B fetch is one ds_read at (channel, tap) offset + pixel position, no test.
-//     A table gives the position of every k.  Per step of four k: one A read, one table
-//     read and nine B reads feed nine MFMAs.
+//     halo, rows at a fixed pitch of 18 and planes at a pitch of 4 mod 32.  The tile's 144
+//     columns are taken tap-major: MFMA tile t is tap t and lane column c is channel c, so a
+//     step's nine B fetches are one address - channel plane + the pixel position a table
+//     gives for every k - plus nine compile-time offsets (tap row * 18 + tap column), and
+//     the 64 lanes of each land in 64 banks.  Per step of four k: one A read, one table read,
+//     one address add and nine B reads feed nine MFMAs.
 //   * The tile is accumulated in registers over all of the workgroup's images and stored
 //     once, as slab `split` of the workspace; slabs are summed in slab order by the
 //     reduction kernel the other filter-gradient kernels use, so results repeat bit for bit.
@@ -46,7 +49,7 @@ struct WgGeom {
   int KW;           // K rounded up to a multiple of 4
   int DP;           // pitch of a dyL row, = 4 mod 64, >= KW
   int PW, PH, PP;   // padded plane: (W + 2 pad) x (H + 2 pad), PP = PH * PW
-  int XP;           // plane pitch in LDS (odd, >= PP)
+  int XP;           // plane pitch in LDS (= 4 mod 32, >= PH * kRowPitch)
   int HW;
   int CKK;          // C * 9
   int ngroups;      // ceil(B / nb)
@@ -57,6 +60,7 @@ struct WgGeom {
 constexpr int kCT = 16;          // channels per workgroup
 constexpr int kBM = 64;          // filters per workgroup
 constexpr int kThreads = 256;
+constexpr int kRowPitch = 18;    // row pitch of a staged plane: the widest padded image (16 + 2)
 constexpr int kU = 8;            // loads a thread has in flight while staging
 
 __global__ __launch_bounds__(kThreads) void k_conv3x3_wgrad_small(const float* __restrict__ x,
@@ -78,20 +82,12 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_wgrad_small(const float* _
     if (p < g.K) {
       const int img = mdiv(p, g.mNPX), r = p - img * g.npx;
       const int row = mdiv(r, g.mOW), col = r - row * g.ow;
-      pos = img * (kCT * g.XP) + row * g.PW + col;
+      pos = img * (kCT * g.XP) + row * kRowPitch + col;
     }
     ptab[p] = pos;
   }
-  // this lane's nine B columns: n = 16 t + li -> (channel, tap) -> offset inside an image's planes
-  int xoff[9];
-#pragma unroll
-  for (int t = 0; t < 9; t++) {
-    const int n = 16 * t + li;
-    const int c = (n * 57) >> 9;   // n / 9 for n < 144
-    const int tap = n - 9 * c;
-    const int kr = (tap * 11) >> 5;   // tap / 3 for tap < 9
-    xoff[t] = c * g.XP + kr * g.PW + (tap - 3 * kr);
-  }
+  // B column of (tile t, lane li) is (tap t, channel li): the lane's plane, the tile's tap offset
+  const int xlane = li * g.XP;
   f32x4 acc[9];
 #pragma unroll
   for (int t = 0; t < 9; t++) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -152,7 +148,7 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_wgrad_small(const float* _
           const int py = mdiv(q, g.mPW), px = q - py * g.PW;
           const int img = ic >> 4, c = ic & 15;
           const int iy = py - g.pad, ix = px - g.pad;
-          dst[u] = ic * g.XP + q;
+          dst[u] = ic * g.XP + py * kRowPitch + px;
           if (b0 + img < g.B && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W)
             v[u] = x[((int64_t)(b0 + img) * g.C + c0 + c) * g.HW + iy * g.W + ix];
         }
@@ -174,17 +170,17 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_wgrad_small(const float* _
     float a0 = arow[0], a1;
     float b0v[9], b1v[9];
     {
-      const float* const xb = xL + prow[0];
+      const float* const xb = xL + xlane + prow[0];
 #pragma unroll
-      for (int t = 0; t < 9; t++) b0v[t] = xb[xoff[t]];
+      for (int t = 0; t < 9; t++) b0v[t] = xb[(t / 3) * kRowPitch + t % 3];
     }
     int pn = prow[min(4, klast)];
     for (int k0 = 0; k0 < g.KW; k0 += 8) {
       {
         a1 = arow[min(k0 + 4, klast)];
-        const float* const xb = xL + pn;
+        const float* const xb = xL + xlane + pn;
 #pragma unroll
-        for (int t = 0; t < 9; t++) b1v[t] = xb[xoff[t]];
+        for (int t = 0; t < 9; t++) b1v[t] = xb[(t / 3) * kRowPitch + t % 3];
         pn = prow[min(k0 + 8, klast)];
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -194,9 +190,9 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_wgrad_small(const float* _
       if (k0 + 4 >= g.KW) break;
       {
         a0 = arow[min(k0 + 8, klast)];
-        const float* const xb = xL + pn;
+        const float* const xb = xL + xlane + pn;
 #pragma unroll
-        for (int t = 0; t < 9; t++) b0v[t] = xb[xoff[t]];
+        for (int t = 0; t < 9; t++) b0v[t] = xb[(t / 3) * kRowPitch + t % 3];
         pn = prow[min(k0 + 12, klast)];
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -207,15 +203,16 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_wgrad_small(const float* _
     __syncthreads();   // every wavefront is done with the planes before the next group lands
   }
 
-  // ---- register v of acc[t] is filter f0 + 16 wave + 4 lk + v, column c0 * 9 + 16 t + li
+  // ---- register v of acc[t] is filter f0 + 16 wave + 4 lk + v, channel c0 + li, tap t: nine
+  // consecutive floats of dW per lane and filter
   float* const o = out + (int64_t)split * slab;
 #pragma unroll
   for (int v = 0; v < 4; v++) {
     const int f = f0 + 16 * wave + 4 * lk + v;
     if (f >= g.F) continue;
-    float* const row = o + (int64_t)f * g.CKK + c0 * 9 + li;
+    float* const row = o + (int64_t)f * g.CKK + (c0 + li) * 9;
 #pragma unroll
-    for (int t = 0; t < 9; t++) row[16 * t] = acc[t][v];
+    for (int t = 0; t < 9; t++) row[t] = acc[t][v];
   }
 }
 
@@ -245,7 +242,9 @@ bool wgrad_small_plan(const gh_ctx* ctx, const gh_cmd& c, WgPlan* out) {
   if (g.nb > g.B) g.nb = g.B;
   g.K = g.nb * g.npx; g.KW = (g.K + 3) & ~3;
   g.DP = g.KW + ((4 - g.KW % 64) + 64) % 64;
-  g.PW = g.W + 2 * g.pad; g.PH = g.H + 2 * g.pad; g.PP = g.PH * g.PW; g.XP = g.PP | 1;
+  g.PW = g.W + 2 * g.pad; g.PH = g.H + 2 * g.pad; g.PP = g.PH * g.PW;
+  g.XP = g.PH * kRowPitch;
+  while (g.XP % 32 != 4) g.XP++;
   g.HW = g.H * g.W; g.CKK = g.C * 9;
   g.ngroups = (g.B + g.nb - 1) / g.nb;
   const int64_t tiles = (C / kCT) * ((F + kBM - 1) / kBM);
