@@ -7,9 +7,11 @@
 // N = C * 9 in the reference's (c, kr, kc) order, K = B * oh * ow: a small result summed over
 // a long K, so K is what gets divided among workgroups.
 //
-//   * One workgroup of four wavefronts owns 64 filters x 16 channels (a 64 x 144 tile of dW:
-//     wavefront w has filter rows 16 w .. 16 w + 15 and all nine 16-column tiles) and a run of
-//     images.  It takes the images a few at a time (as many as give about 200 output pixels):
+//   * One workgroup of eight wavefronts owns 64 filters x 16 channels (a 64 x 144 tile of dW:
+//     wavefront w has filter rows 16 (w & 3) .. + 15, all nine 16-column tiles and one half
+//     of every group's k steps; the two halves meet through LDS at the end, second onto
+//     first, a fixed order) and a run of images.  Two wavefronts per SIMD: one's LDS and
+//     issue latencies run under the other's MFMAs.  It takes the images a few at a time (as many as give about 200 output pixels):
 //     their dy rows go to LDS as dyL[filter][k] with k = (image, pixel) and a pitch of 4 mod
 //     64, so the 64 lanes of an A fetch hit 64 banks; their x planes go to LDS with a zero
 //     halo, rows at a fixed pitch of 18 and planes at a pitch of 4 mod 32.  The tile's 144
@@ -59,11 +61,12 @@ struct WgGeom {
 
 constexpr int kCT = 16;          // channels per workgroup
 constexpr int kBM = 64;          // filters per workgroup
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
 constexpr int kRowPitch = 18;    // row pitch of a staged plane: the widest padded image (16 + 2)
-constexpr int kU = 8;            // loads a thread has in flight while staging
+constexpr int kU = 6;            // loads a thread has in flight while staging
 
-__global__ __launch_bounds__(kThreads) void k_conv3x3_wgrad_small(const float* __restrict__ x,
+// Held to 128 registers: two workgroups then share a compute unit where their LDS allows (long K, few images).
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void k_conv3x3_wgrad_small(const float* __restrict__ x,
                                                                   const float* __restrict__ dy,
                                                                   float* __restrict__ out, WgGeom g,
                                                                   int64_t slab) {
@@ -73,6 +76,7 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_wgrad_small(const float* _
   int* const ptab = reinterpret_cast<int*>(xL + g.nb * kCT * g.XP);   // [KW]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int mt = wave & 3, khalf = wave >> 2;   // tile row, half of the k steps
   const int li = lane & 15, lk = lane >> 4;
   const int split = blockIdx.x, c0 = blockIdx.y * kCT, f0 = blockIdx.z * kBM;
 
@@ -162,53 +166,69 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_wgrad_small(const float* _
     // operands of step s + 1 and the position of step s + 2 are fetched before the MFMAs of
     // step s: a position leads to nine B reads, two LDS latencies that would otherwise sit
     // between the steps of a wavefront that has its SIMD to itself.
-    const float* const arow = dyL + (16 * wave + li) * g.DP + lk;
+    // this wavefront's half of the group's steps: [kb, ke)
+    const int nsteps = g.KW >> 2, half = (nsteps + 1) >> 1;
+    const int kb = 4 * (khalf ? half : 0), ke = 4 * (khalf ? nsteps : half);
+    const float* const arow = dyL + (16 * mt + li) * g.DP + lk;
     const int* const prow = ptab + lk;
-    const int klast = g.KW - 4;
-    // two operand sets, used in turn: while one feeds the MFMAs the other is being read.
-    // (The fences keep the reads of a set in front of the MFMAs they are meant to run under.)
-    float a0 = arow[0], a1;
-    float b0v[9], b1v[9];
-    {
-      const float* const xb = xL + xlane + prow[0];
-#pragma unroll
-      for (int t = 0; t < 9; t++) b0v[t] = xb[(t / 3) * kRowPitch + t % 3];
-    }
-    int pn = prow[min(4, klast)];
-    for (int k0 = 0; k0 < g.KW; k0 += 8) {
+    if (kb < ke) {
+      const int klast = ke - 4;
+      // two operand sets, used in turn: while one feeds the MFMAs the other is being read.
+      // (The fences keep the reads of a set in front of the MFMAs they are meant to run under.)
+      float a0 = arow[kb], a1;
+      float b0v[9], b1v[9];
       {
-        a1 = arow[min(k0 + 4, klast)];
-        const float* const xb = xL + xlane + pn;
-#pragma unroll
-        for (int t = 0; t < 9; t++) b1v[t] = xb[(t / 3) * kRowPitch + t % 3];
-        pn = prow[min(k0 + 8, klast)];
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int t = 0; t < 9; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0v[t], acc[t], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      if (k0 + 4 >= g.KW) break;
-      {
-        a0 = arow[min(k0 + 8, klast)];
-        const float* const xb = xL + xlane + pn;
+        const float* const xb = xL + xlane + prow[kb];
 #pragma unroll
         for (int t = 0; t < 9; t++) b0v[t] = xb[(t / 3) * kRowPitch + t % 3];
-        pn = prow[min(k0 + 12, klast)];
       }
-      __builtin_amdgcn_sched_barrier(0);
+      int pn = prow[min(kb + 4, klast)];
+      for (int k0 = kb; k0 < ke; k0 += 8) {
+        {
+          a1 = arow[min(k0 + 4, klast)];
+          const float* const xb = xL + xlane + pn;
 #pragma unroll
-      for (int t = 0; t < 9; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1v[t], acc[t], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
+          for (int t = 0; t < 9; t++) b1v[t] = xb[(t / 3) * kRowPitch + t % 3];
+          pn = prow[min(k0 + 8, klast)];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 9; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0v[t], acc[t], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (k0 + 4 >= ke) break;
+        {
+          a0 = arow[min(k0 + 8, klast)];
+          const float* const xb = xL + xlane + pn;
+#pragma unroll
+          for (int t = 0; t < 9; t++) b0v[t] = xb[(t / 3) * kRowPitch + t % 3];
+          pn = prow[min(k0 + 12, klast)];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 9; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1v[t], acc[t], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
     __syncthreads();   // every wavefront is done with the planes before the next group lands
   }
 
-  // ---- register v of acc[t] is filter f0 + 16 wave + 4 lk + v, channel c0 + li, tap t: nine
+  // ---- the second half's partial tile onto the first's, through LDS (the last barrier of the
+  // loop has every wavefront past its reads of dyL): [tile row][t][lane] as 128-bit values
+  f32x4* const red = reinterpret_cast<f32x4*>(dyL) + (mt * 9) * 64 + lane;
+  if (khalf) {
+#pragma unroll
+    for (int t = 0; t < 9; t++) red[t * 64] = acc[t];
+  }
+  __syncthreads();
+  if (khalf) return;
+#pragma unroll
+  for (int t = 0; t < 9; t++) acc[t] = acc[t] + red[t * 64];
+  // ---- register v of acc[t] is filter f0 + 16 mt + 4 lk + v, channel c0 + li, tap t: nine
   // consecutive floats of dW per lane and filter
   float* const o = out + (int64_t)split * slab;
 #pragma unroll
   for (int v = 0; v < 4; v++) {
-    const int f = f0 + 16 * wave + 4 * lk + v;
+    const int f = f0 + 16 * mt + 4 * lk + v;
     if (f >= g.F) continue;
     float* const row = o + (int64_t)f * g.CKK + (c0 + li) * 9;
 #pragma unroll
@@ -259,6 +279,7 @@ bool wgrad_small_plan(const gh_ctx* ctx, const gh_cmd& c, WgPlan* out) {
   out->g = g;
   out->splits = (int)splits;
   out->lds = ((size_t)kBM * g.DP + (size_t)g.nb * kCT * g.XP + g.KW) * 4;
+  out->lds = std::max<size_t>(out->lds, (size_t)4 * 9 * 64 * 16);   // the two halves' partial tiles meet in it
   return out->lds <= 150 * 1024;
 }
 
