@@ -2933,6 +2933,8 @@ int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
   if (rcp >= 0) return rcp;
   const int rcw = gh_try_launch_conv_wide(ctx, c);
   if (rcw >= 0) return rcw;
+  const int rc1 = gh_try_launch_conv_pointwise(ctx, c);
+  if (rc1 >= 0) return rc1;
   const int rc3 = try_launch_conv3(ctx, c);
   if (rc3 >= 0) return rc3;
   if (c.flags & GH_FLAG_CONV_POOL2)

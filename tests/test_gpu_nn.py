@@ -323,6 +323,41 @@ def test_conv_patch_kernel(ctx, cfg):
                           O.maxpool2d(leaky, (2, 2), (0, 0), (2, 2)), f"patch conv+bn+leaky+pool {cfg}")
 
 
+# shapes the 1x1 kernel takes (stride 1, no padding, channels a multiple of 256, four pixels or more per image, too
+# few 64x64 tiles to fill the device): ragged filter and pixel tiles, tiles crossing images, image sizes of every
+# remainder mod 4 (the last quad of an image overlaps the one before), two and four channel groups in flight,
+# every filter-tile height; and two the tiled kernel keeps (one pixel per image, 384 channels)
+POINTWISE_CASES = [(2, 1024, 13, 13, 425), (8, 256, 13, 13, 40), (3, 512, 7, 9, 33), (1, 512, 26, 26, 255),
+                   (5, 768, 5, 3, 17), (2, 256, 31, 29, 96), (9, 256, 2, 3, 150), (3, 1024, 2, 2, 48), (4, 512, 5, 5, 300),
+                   (70, 256, 1, 1, 64), (3, 384, 7, 9, 33)]
+
+
+@pytest.mark.parametrize("cfg", POINTWISE_CASES)
+def test_conv_pointwise_kernel(ctx, cfg):
+    """The 1x1 convolution kernel against the oracle (<= 1e-5, exact on integers), and its epilogues against the
+    oracle's operators applied to its own plain result, bit for bit."""
+    B, C, H, W, F = cfg
+    x = synth.uniform(51, (B, C, H, W), -1, 1)
+    w = synth.he_normal(52, (F, C, 1, 1))
+    plain = gpu_conv(ctx, x, w, (0, 0), (1, 1), (1, 1))
+    ref = O.conv2d_direct_f64(x, w, (0, 0), (1, 1), (1, 1))
+    err = rel_frobenius(plain, ref)
+    assert err <= TOL, f"1x1 conv {cfg}: rel frobenius {err:.3e}"
+    rng = np.random.default_rng(11)
+    xi = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+    wi = rng.integers(-3, 4, (F, C, 1, 1)).astype(np.float32)
+    assert_bits_equal(gpu_conv(ctx, xi, wi, (0, 0), (1, 1), (1, 1)), O.conv2d(xi, wi, (0, 0), (1, 1), (1, 1)),
+                      f"integer 1x1 conv {cfg}")
+    mean, var = synth.normal(53, (F,), 0.0, 0.1), synth.uniform(54, (F,), 0.5, 1.5)
+    gamma, beta = synth.uniform(55, (F,), 0.5, 1.5), synth.normal(56, (F,), 0.0, 0.1)
+    bn = O.bn_infer(plain, mean, var, 1e-5, gamma, beta)
+    assert_bits_equal(gpu_conv_tail(ctx, x, w, (0, 0), bn=(mean, var, gamma, beta)), bn, f"1x1 conv+bn {cfg}")
+    assert_bits_equal(gpu_conv_tail(ctx, x, w, (0, 0), bn=(mean, var, gamma, beta), act="leaky", alpha=0.1),
+                      O.leaky_relu(bn, 0.1).reshape(plain.shape), f"1x1 conv+bn+leaky {cfg}")
+    assert_bits_equal(gpu_conv_tail(ctx, x, w, (0, 0), act="relu"), O.relu(plain).reshape(plain.shape), f"1x1 conv+relu {cfg}")
+    assert ctx.lib.gh_conv2d_can_pool(D.cmd_conv2d(1, 1, 1, B, C, H, W, F, 1, 1, (0, 0))) == 0
+
+
 # shapes the wide-image kernel takes (3x3, at most 64 channels, enough pixels that patches alone fill the
 # device; whole K per wavefront): channel counts that are not multiples of four, ragged filter tiles,
 # partial patches on both axes, no padding, pooled extents odd and even
