@@ -2328,9 +2328,24 @@ TilePlan plan_tiles(gh_ctx* ctx, int64_t M, int64_t N, int64_t K, int64_t batch,
   const int64_t blocks = p.tile == kTile64 ? cdiv(M, 64) * cdiv(N, 64) * batch : cdiv(M, 32) * cdiv(N, 256);
   if (batch == 1 && blocks < 2 * cus) {
     const int64_t nk = cdiv(K, 16);
-    int64_t sp = cdiv(2 * cus, blocks);
-    const int64_t max_sp = nk / 4 > 0 ? nk / 4 : 1;  // at least 4 k-tiles per slice
-    if (sp > max_sp) sp = max_sp;
+    int64_t sp = 1;
+    if (!allow_32x256) {
+      // matrix product on 64x64 tiles: a compute unit works through its workgroups' k-tiles at about
+      // 0.8 us each however many share it, and a second launch to add the slabs costs 3.5 us plus
+      // 1 us per slab and million results (1152 x 625 results, K = 128 ... 2048: this picks the
+      // measured best count, one slice up to K = 256 and four from 512 on, where
+      // cdiv(2 cus, blocks) = 3 lost 8-25 %)
+      double best = 0;
+      const double slab_us = (double)M * (double)N * 1e-6;
+      for (int64_t s = 1; s <= 16 && (s == 1 || 2 * s <= nk); s++) {
+        const double est = (double)(cdiv(blocks * s, cus) * cdiv(nk, s)) * 0.8 + (s > 1 ? 3.5 + slab_us * (double)s : 0.0);
+        if (s == 1 || est < best) { best = est; sp = s; }
+      }
+    } else {
+      sp = cdiv(2 * cus, blocks);
+      const int64_t max_sp = nk / 4 > 0 ? nk / 4 : 1;  // at least 4 k-tiles per slice
+      if (sp > max_sp) sp = max_sp;
+    }
     p.splits = clamp_splits(ctx, sp, M, N, K, batch);
   }
   return p;
