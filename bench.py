@@ -231,7 +231,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 # SQ_VALU_MFMA_BUSY_CYCLES / (128 * GRBM_GUI_ACTIVE) of the same kernels in a rocprofv3 --pmc run of this
 # script (eager launches, one at a time: launch and drain are inside GUI_ACTIVE, clocks are not sustained)
-MEASURED_MFMA_BUSY = {"conv0": 0.0, "conv1": 0.288, "conv2": 0.226}
+MEASURED_MFMA_BUSY = {"conv0": 0.0, "conv1": 0.283, "conv2": 0.223}
 CONV_KERNEL_NAME = {"conv0": "k_conv3x3_direct<1,2>", "conv1": "k_conv3x3_small<8,1,13,1>", "conv2": "k_conv3x3_small<8,1,9,2>"}
 
 CONVNET_LAYERS = [  # (name, B-relative shape) of configuration 4
