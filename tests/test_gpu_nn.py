@@ -431,6 +431,30 @@ def test_conv_random_geometry_sweep(ctx):
     assert pooled >= 8
 
 
+def test_conv_pointwise_random_geometries(ctx):
+    """Seeded sweep over 1x1 convolutions with 256-1024 channels (the K-split 1x1 kernel, every filter-tile height,
+    images of every size mod 4): against the float64 sum, exact on small integers, and conv+LeakyReLU against the
+    oracle's LeakyReLU of the plain result bit for bit."""
+    rng = np.random.default_rng(78)
+    for case in range(14):
+        B = int(rng.integers(1, 10))
+        C = int(rng.choice([256, 512, 768, 1024]))
+        H, W = int(rng.integers(1, 20)), int(rng.integers(2, 20))
+        F = int(rng.integers(1, 200))
+        x = synth.uniform(5000 + case, (B, C, H, W), -1, 1)
+        w = synth.he_normal(6000 + case, (F, C, 1, 1))
+        got = gpu_conv(ctx, x, w, (0, 0), (1, 1), (1, 1))
+        ref = np.einsum("fc,bchw->bfhw", w[:, :, 0, 0].astype(np.float64), x.astype(np.float64))
+        err = rel_frobenius(got, ref)
+        assert err <= TOL, f"case {case}: B{B} C{C} {H}x{W} F{F}: {err:.3e}"
+        xi = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+        wi = rng.integers(-3, 4, (F, C, 1, 1)).astype(np.float32)
+        want = np.einsum("fc,bchw->bfhw", wi[:, :, 0, 0].astype(np.float64), xi.astype(np.float64)).astype(np.float32)
+        assert_bits_equal(gpu_conv(ctx, xi, wi, (0, 0), (1, 1), (1, 1)), want, f"case {case}: integer 1x1 conv")
+        assert_bits_equal(gpu_conv_tail(ctx, x, w, (0, 0), act="leaky", alpha=0.1), O.leaky_relu(got, 0.1).reshape(got.shape),
+                          f"case {case}: 1x1 conv+leaky")
+
+
 def test_conv_pool_flag_needs_a_pooling_kernel(ctx):
     # 13 rows of 13: no block of at most 128 pixels holds a whole image
     cmd = D.cmd_conv2d(0x1000, 0x2000, 0x3000, 2, 8, 13, 13, 16, 3, 3, (1, 1), pool2=True)
