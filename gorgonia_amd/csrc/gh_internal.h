@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <cstdint>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "gorgonia_hip.h"
@@ -61,6 +62,8 @@ struct gh_ctx {
   bool ws_strict = false;
   bool sync_spin = false;  // gh_sync polls the stream instead of blocking in the runtime
   gh_llc_model llc;
+  // pinned host buffers handed out by gh_host_alloc: [start, end)
+  std::vector<std::pair<uint64_t, uint64_t>> host_ranges;
 };
 
 // A launcher calls this where `need` bytes of scratch do not fit the workspace,

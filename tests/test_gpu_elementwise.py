@@ -279,6 +279,26 @@ def test_large_operands_cold_then_warm_same_bits(ctx):
         ctx.free(p)
 
 
+def test_copy_command_from_pinned_host_memory(ctx):
+    """GH_OP_MEMCPY_D2D with pinned host memory on the source side, as the tape machine's uploads use it:
+    the small sizes go through the copy kernels (128-bit, word and odd-tail forms), the large one through
+    the copy engine; every one lands byte for byte."""
+    import ctypes as C
+    rng = np.random.default_rng(5)
+    for nbytes in (64, 4096 + 8, 401408, (4 << 20) - 4, 4 << 20, (6 << 20) + 12, 17 << 20):
+        host = C.c_void_p()
+        assert ctx.lib.gh_host_alloc(ctx.h, C.c_int64(nbytes), C.byref(host)) == 0
+        src = rng.integers(0, 2 ** 32, nbytes // 4, dtype=np.uint32)
+        C.memmove(host, src.ctypes.data, nbytes)
+        dev = ctx.malloc(nbytes)
+        ctx.run(D.cmd_fill(dev, nbytes // 4, 0.0))
+        ctx.run(D.cmd_copy(dev, host.value, nbytes))
+        got = ctx.d2h(dev, (nbytes // 4,), np.uint32)
+        assert np.array_equal(got, src), f"{nbytes} bytes"
+        ctx.free(dev)
+        assert ctx.lib.gh_host_free(ctx.h, host) == 0
+
+
 def test_relu_and_leaky_bit_exact(ctx):
     for n in [1, 7, 4099, (1 << 20) + 1]:
         x = _special(n, 61)
