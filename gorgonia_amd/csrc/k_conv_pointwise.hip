@@ -183,9 +183,15 @@ bool pointwise_plan(const gh_cmd& c, int cus, PwPlan* out) {
   if ((c.ptr[1] & 15) != 0) return false;                       // 128-bit loads of filter rows
   const int64_t HW = H * W, P = B * HW;
   if (HW < 4) return false;                                     // a quad of pixels per lane
+  if (getenv("GORGONIA_HIP_CONV_NO_POINTWISE")) return false;   // tuning switch: the tiled kernel only
   if (B * C * HW * 4 >= (1ll << 32) || P * F >= (1ll << 31) || P >= (1 << 24)) return false;
-  // only where 64x64 tiles would leave compute units idle without cutting K across workgroups
-  if (((F + 63) / 64) * ((P + 63) / 64) >= 2 * cus) return false;
+  // only where 64x64 tiles would leave compute units idle, or nearly, without cutting K across workgroups
+  // measured against the tiled kernel (batch 8): ahead up to about 2 cus of its tiles, by up to 2x below
+  // one per compute unit; with 256 channels (few k-tiles for the tiled kernel to overlap its loads with)
+  // up to about 8 cus (256 -> 256 at 52 x 52: 40.6 us against 52.8), level at 2700 tiles
+  int64_t max_tiles = (C <= 256 ? 8 : 2) * (int64_t)cus;
+  if (const char* e = getenv("GORGONIA_HIP_CONV_POINTWISE_TILES")) max_tiles = atoll(e);   // tuning override
+  if (((F + 63) / 64) * ((P + 63) / 64) >= max_tiles) return false;
   PwGeom g{};
   g.B = (int)B; g.C = (int)C; g.F = (int)F; g.HW = (int)HW;
   g.QI = (int)((HW + 3) / 4); g.NQ = g.B * g.QI;

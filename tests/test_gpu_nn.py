@@ -328,7 +328,7 @@ def test_conv_patch_kernel(ctx, cfg):
 # remainder mod 4 (the last quad of an image overlaps the one before), two and four channel groups in flight,
 # every filter-tile height; and two the tiled kernel keeps (one pixel per image, 384 channels)
 POINTWISE_CASES = [(2, 1024, 13, 13, 425), (8, 256, 13, 13, 40), (3, 512, 7, 9, 33), (1, 512, 26, 26, 255),
-                   (5, 768, 5, 3, 17), (2, 256, 31, 29, 96), (9, 256, 2, 3, 150), (3, 1024, 2, 2, 48), (4, 512, 5, 5, 300),
+                   (5, 768, 5, 3, 17), (2, 256, 31, 29, 96), (9, 256, 2, 3, 150), (3, 1024, 2, 2, 48), (4, 512, 5, 5, 300), (2, 256, 104, 100, 24),
                    (70, 256, 1, 1, 64), (3, 384, 7, 9, 33)]
 
 
