@@ -15,6 +15,9 @@ static constexpr int64_t kStageLimit = 8 << 20;
 // inputs re-uploaded on every run are staged through pinned memory up to these sizes
 static constexpr int64_t kStageInLimit = 16 << 20;    // per input (what one copy kernel moves)
 static constexpr int64_t kStageInTotal = 512ll << 20; // per machine
+// inputs from this size on are uploaded in pieces, the host copy into pinned memory overlapping the bus
+static constexpr int64_t kPipelinedUpload = 4 << 20;
+static constexpr int64_t kUploadPiece = 2 << 20;
 
 static Status bad(const std::string& m) { return Status::Err(GH_EINVAL, m); }
 
@@ -1095,6 +1098,21 @@ Status TapeMachine::RunAll() {
         if (void* pinned = stage_in_[(size_t)in.node]) {
           // host value -> pinned buffer now, pinned buffer -> register as a command of
           // the segment: the upload is captured and replayed with the operators
+          if (!n.host_borrowed && in.size >= kPipelinedUpload && eng_.Segment().empty()) {
+            // a large value at the front of its segment: piece by piece, the host copy of one
+            // piece runs while the copy engine moves the piece before it (stream order puts the
+            // segment's operators behind the last piece)
+            const char* src = static_cast<const char*>(n.host);
+            char* stg = static_cast<char*>(pinned);
+            for (int64_t off = 0; off < in.size; off += kUploadPiece) {
+              const int64_t len = std::min(kUploadPiece, in.size - off);
+              std::memcpy(stg + off, src + off, (size_t)len);
+              st = eng_.MemcpyHtoD(regs_[(size_t)in.reg].mem + (uint64_t)off, stg + off, len);
+              if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": devTrans");
+            }
+            resident_done_[(size_t)in.node] = 1;
+            break;
+          }
           if (!n.host_borrowed) std::memcpy(pinned, n.host, (size_t)in.size);
           eng_.RecordCopy(regs_[(size_t)in.reg].mem, (uint64_t)(uintptr_t)pinned, in.size);
           resident_done_[(size_t)in.node] = 1;

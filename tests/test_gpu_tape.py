@@ -328,6 +328,28 @@ def test_borrowed_inputs_upload_what_the_caller_wrote(ctx):
         m.Close()
 
 
+def test_large_input_uploaded_in_pieces_each_run(ctx):
+    """An input of several megabytes that is uploaded on every run travels in pieces (host copy into pinned
+    memory overlapping the bus): every byte arrives, on plain, replayed and measured runs, with the value changed
+    between runs, for a size that is no multiple of the piece."""
+    n = (5 << 20) // 4 + 1234 * 4
+    yv = synth.uniform(8, (n,), -2, 2)
+    for mode in (False, True, "measured"):
+        g = G.NewGraph()
+        x = G.NewTensor(g, synth.uniform(7, (n,), -2, 2))
+        y = G.NewTensor(g, yv, resident=True)
+        out = G.Read(G.Rectify(G.Add(G.HadamardProd(x, y), x)))
+        m = G.NewTapeMachine(g, graph_replay=mode)
+        for it in range(7):
+            a = synth.uniform(100 + it, (n,), -2, 2)
+            G.Let(x, a)
+            m.RunAll()
+            v = a * yv + a                      # two float32 roundings, as the two operators make them
+            want = v * (v >= 0).astype(np.float32)
+            assert_bits_equal(out, want.reshape(out.shape), f"large input, replay={mode}, run {it}")
+        m.Close()
+
+
 def test_measured_replay_keeps_results_and_settles(ctx):
     """graph_replay="measured": the machine times plain submits against replays of a segment on
     its first runs and keeps the quicker; every run along the way, and after the verdict, stores
