@@ -118,6 +118,7 @@ bool gh_conv_wide_takes(const gh_cmd& c);
 bool gh_conv_wide_can_pool(const gh_cmd& c);
 // k_conv_pointwise.hip: 1x1 stride-1 convolution whose result is too small for K-wide 64x64 tiles to fill the device
 int gh_try_launch_conv_pointwise(gh_ctx* ctx, const gh_cmd& c);
+bool gh_conv_pointwise_takes(const gh_cmd& c, int cus);
 int gh_launch_maxpool2d(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_bn_infer(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_softmax(gh_ctx* ctx, const gh_cmd& c);

@@ -230,6 +230,11 @@ int launch_pointwise(gh_ctx* ctx, const gh_cmd& c, const PwPlan& p) {
 
 }  // namespace
 
+bool gh_conv_pointwise_takes(const gh_cmd& c, int cus) {
+  PwPlan p;
+  return pointwise_plan(c, cus, &p);
+}
+
 // Returns -1 when the shape is not one this kernel takes.
 int gh_try_launch_conv_pointwise(gh_ctx* ctx, const gh_cmd& c) {
   PwPlan p;

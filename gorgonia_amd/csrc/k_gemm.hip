@@ -3175,6 +3175,22 @@ extern "C" int gh_gemm_can_softmax(const gh_cmd* c) {
   return c->dim[1] >= 1 && c->dim[1] <= 32 && c->dim[0] >= 1 && c->dim[0] <= 2048 && c->dim[2] >= 32;
 }
 
+// The dispatch order of gh_launch_conv2d, asked without launching.  The plans are functions of the
+// command; the one figure of the device they use, its compute units, is the MI355X's here.
+extern "C" int gh_conv2d_route(const gh_cmd* c) {
+  if (!c || c->opcode != GH_OP_CONV2D || gh_dtype_of(c->flags) != GH_F32) return -1;
+  if (conv_direct_takes(*c)) return GH_CONV_ROUTE_DIRECT;
+  if (gh_conv_small_takes(*c)) return GH_CONV_ROUTE_SMALL;
+  if (gh_conv_patch_takes(*c)) return GH_CONV_ROUTE_PATCH;
+  if (gh_conv_wide_takes(*c)) return GH_CONV_ROUTE_WIDE;
+  if (gh_conv_pointwise_takes(*c, 256)) return GH_CONV_ROUTE_POINTWISE;
+  Conv3Geom g;
+  int BM, BN, per_thread;
+  size_t lds;
+  if (conv3_plan<8>(*c, false, &g, &BM, &BN, &lds, &per_thread)) return GH_CONV_ROUTE_TILED;
+  return GH_CONV_ROUTE_GATHER;
+}
+
 extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {
   if (!c || c->opcode != GH_OP_CONV2D || gh_dtype_of(c->flags) != GH_F32) return 0;
   if (conv_direct_takes(*c)) {

@@ -296,6 +296,21 @@ GH_API int gh_validate(const gh_cmd* cmds, int n, char* msg, int msg_len);
  * reference has no fused form: this folds maxpool.CUDADo
  * (ops/nn/maxpool_cuda.go:94-111) into convolution.CUDADo (convolution_cuda.go:95-121). */
 GH_API int gh_conv2d_can_pool(const gh_cmd* conv);
+/* Which of the library's convolution kernels gh_submit runs this float32 CONV2D command on, a
+ * function of its shape, its flags and (for the filter operand's alignment) its pointers: one of
+ * GH_CONV_ROUTE_*, or -1 for a command that is no float32 CONV2D.  Host only.  The reference
+ * leaves this choice to cuDNN (algorithm ImplicitGemm, ops/nn/convolution_cuda.go:111-117); here
+ * the summing order, and with it the bits, belong to the kernel, so tests and callers can ask. */
+enum gh_conv_route {
+  GH_CONV_ROUTE_DIRECT = 0,     /* 3x3, at most four channels: vector ALUs               */
+  GH_CONV_ROUTE_SMALL = 1,      /* 3x3 over images up to 16 x 16, K split over wavefronts */
+  GH_CONV_ROUTE_PATCH = 2,      /* 3x3, 64 channels or more, patch per workgroup          */
+  GH_CONV_ROUTE_WIDE = 3,       /* 3x3 over large images, persistent workgroups           */
+  GH_CONV_ROUTE_POINTWISE = 4,  /* 1x1 with a small result                                */
+  GH_CONV_ROUTE_TILED = 5,      /* 3x3 staged through LDS tiles (+ K slices)              */
+  GH_CONV_ROUTE_GATHER = 6      /* every other geometry                                   */
+};
+GH_API int gh_conv2d_route(const gh_cmd* conv);
 
 /* 1 when this GEMM command may carry GH_FLAG_GEMM_SOFTMAX: a float32 product of
  * untransposed operands with at most 32 columns and at most 2048 rows, whose

@@ -97,3 +97,64 @@ def test_headers_are_plain_c99(tmp_path):
     src = os.path.join(ROOT, "tests", "c_consumer", "consumer.c")
     p = subprocess.run([gcc] + flags + ["-c", src, "-o", str(tmp_path / "consumer.o")], capture_output=True, text=True)
     assert p.returncode == 0, p.stderr
+
+
+ROUTE = {"direct": 0, "small": 1, "patch": 2, "wide": 3, "pointwise": 4, "tiled": 5, "gather": 6}
+
+
+def _route(B, C, H, W, F, k, pad, stride=(1, 1), dil=(1, 1), pool2=False):
+    lib = _ffi.load()
+    cmd = D.cmd_conv2d(0x10000, 0x20000, 0x30000, B, C, H, W, F, k[0], k[1], pad, stride, dil, pool2=pool2)
+    return lib.gh_conv2d_route(C_byref(cmd))
+
+
+def C_byref(cmd):
+    return C.byref(cmd)
+
+
+def test_conv_routes_of_the_benchmark_layers():
+    """gh_conv2d_route: every layer of the two convolutional configurations runs on the kernel the
+    design names for it."""
+    # convnet (configuration 4), batch 128
+    assert _route(128, 1, 28, 28, 32, (3, 3), (1, 1)) == ROUTE["direct"]
+    assert _route(128, 32, 14, 14, 64, (3, 3), (1, 1)) == ROUTE["small"]
+    assert _route(128, 64, 7, 7, 128, (3, 3), (1, 1)) == ROUTE["small"]
+    # tiny-yolo-shaped (configuration 5), batch 8
+    for (Cn, F, S) in ((3, 16, 416), (16, 32, 208), (32, 64, 104)):
+        assert _route(8, Cn, S, S, F, (3, 3), (1, 1)) == ROUTE["wide"], (Cn, F, S)
+    for (Cn, F, S) in ((64, 128, 52), (128, 256, 26), (256, 512, 13), (512, 1024, 13)):
+        assert _route(8, Cn, S, S, F, (3, 3), (1, 1)) == ROUTE["patch"], (Cn, F, S)
+    assert _route(8, 1024, 13, 13, 425, (1, 1), (0, 0)) == ROUTE["pointwise"]
+    # and what the specialised kernels leave: other filter sizes, strides, Conv1d
+    assert _route(2, 5, 9, 9, 7, (5, 5), (2, 2)) == ROUTE["gather"]
+    assert _route(2, 2, 10, 11, 3, (3, 2), (2, 1), (2, 3)) == ROUTE["gather"]
+    assert _route(2, 8, 1, 64, 16, (1, 5), (0, 2), (1, 2)) == ROUTE["gather"]
+    assert _route(1, 4, 7, 7, 6, (1, 1), (0, 0)) == ROUTE["gather"]          # 1x1 with few channels
+    assert _route(2, 16, 66, 68, 40, (3, 3), (0, 0)) in (ROUTE["tiled"], ROUTE["wide"])
+    lib = _ffi.load()
+    assert lib.gh_conv2d_route(C.byref(D.cmd_relu(0x1000, 0x2000, 16))) == -1
+
+
+def test_conv_route_of_every_parity_case_list():
+    """The case lists of the GPU parity tests reach the kernels they are written for."""
+    from tests import test_gpu_nn as T
+    for (B, Cn, H, W, F, pad) in T.SMALL_IMAGE_CASES:
+        assert _route(B, Cn, H, W, F, (3, 3), (pad, pad)) == ROUTE["small"], (B, Cn, H, W, F, pad)
+    for (B, Cn, H, W, F, pad) in T.PATCH_CASES:
+        assert _route(B, Cn, H, W, F, (3, 3), (pad, pad)) == ROUTE["patch"], (B, Cn, H, W, F, pad)
+    for (B, Cn, H, W, F, pad) in T.WIDE_CASES:
+        assert _route(B, Cn, H, W, F, (3, 3), (pad, pad)) == ROUTE["wide"], (B, Cn, H, W, F, pad)
+    taken = [c for c in T.POINTWISE_CASES if c[1] % 256 == 0 and c[2] * c[3] >= 4]
+    assert len(taken) >= 9 and len(taken) < len(T.POINTWISE_CASES)
+    for (B, Cn, H, W, F) in T.POINTWISE_CASES:
+        want = ROUTE["pointwise"] if (B, Cn, H, W, F) in taken else ROUTE["gather"]
+        assert _route(B, Cn, H, W, F, (1, 1), (0, 0)) == want, (B, Cn, H, W, F)
+    # the general lists between them reach all seven kernels
+    seen = set()
+    for (B, Cn, H, W, F, kh, kw, pad, stride, dil) in T.CONV_CASES:
+        seen.add(_route(B, Cn, H, W, F, (kh, kw), pad, stride, dil))
+    for (B, Cn, H, W, F, k, pad) in T.TAIL_CASES:
+        seen.add(_route(B, Cn, H, W, F, (k, k), (pad, pad)))
+    for (B, Cn, H, W, F, pad) in T.WIDE_CASES[:1]:
+        seen.add(_route(B, Cn, H, W, F, (3, 3), (pad, pad)))
+    assert seen == set(ROUTE.values()), seen

@@ -361,8 +361,8 @@ def test_conv_pointwise_kernel(ctx, cfg):
 # shapes the wide-image kernel takes (3x3, at most 64 channels, enough pixels that patches alone fill the
 # device; whole K per wavefront): channel counts that are not multiples of four, ragged filter tiles,
 # partial patches on both axes, no padding, pooled extents odd and even
-WIDE_CASES = [(2, 16, 130, 131, 32, 1), (1, 32, 104, 104, 64, 1), (3, 3, 120, 96, 16, 1), (40, 1, 28, 28, 32, 1),
-              (2, 8, 129, 140, 5, 0), (1, 24, 181, 190, 40, 1), (1, 64, 190, 181, 21, 1), (2, 12, 150, 111, 70, 0),
+WIDE_CASES = [(2, 16, 130, 131, 32, 1), (4, 32, 104, 104, 64, 1), (3, 3, 120, 96, 16, 1), (8, 5, 64, 66, 32, 1),
+              (2, 8, 129, 140, 5, 0), (1, 24, 181, 190, 40, 1), (1, 48, 190, 181, 21, 1), (3, 12, 150, 111, 70, 0),
               (1, 6, 200, 170, 33, 1),
               # three and four channels (one quad of planes, the last one padding for C = 3), taken from the direct kernel
               (2, 4, 140, 130, 20, 1), (1, 3, 260, 270, 16, 0)]
