@@ -106,6 +106,7 @@ int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c);
 // small-image 3x3 convolution (k_conv_small.hip): -1 when the shape is not one it takes
 int gh_try_launch_conv_small(gh_ctx* ctx, const gh_cmd& c);
 int gh_try_launch_conv_wgrad_small(gh_ctx* ctx, const gh_cmd& c, int* splits);
+bool gh_conv_wgrad_small_takes(const gh_cmd& c);
 bool gh_conv_small_takes(const gh_cmd& c);
 bool gh_conv_small_can_pool(const gh_cmd& c);
 // 3x3 convolution over patches with K split across wavefronts (k_conv_patch.hip), same conventions

@@ -258,13 +258,19 @@ bool wgrad_small_plan(const gh_ctx* ctx, const gh_cmd& c, WgPlan* out) {
   g.oh = g.H + 2 * g.pad - 2; g.ow = g.W + 2 * g.pad - 2;
   if (g.oh <= 0 || g.ow <= 0 || g.oh * g.ow < 4) return false;   // a 128-bit piece of dy spans at most two rows
   g.npx = g.oh * g.ow;
-  g.nb = g.npx >= 208 ? 1 : 208 / g.npx;
-  if (g.nb > g.B) g.nb = g.B;
-  g.K = g.nb * g.npx; g.KW = (g.K + 3) & ~3;
-  g.DP = g.KW + ((4 - g.KW % 64) + 64) % 64;
   g.PW = g.W + 2 * g.pad; g.PH = g.H + 2 * g.pad; g.PP = g.PH * g.PW;
   g.XP = g.PH * kRowPitch;
   while (g.XP % 32 != 4) g.XP++;
+  // images staged at a time: about 208 output pixels, fewer where their padded planes (tiny images
+  // have more halo than pixels) would not fit LDS beside the dy rows
+  constexpr size_t kLdsLimit = 150 * 1024;
+  g.nb = g.npx >= 208 ? 1 : 208 / g.npx;
+  if (g.nb > g.B) g.nb = g.B;
+  for (;; g.nb--) {
+    g.K = g.nb * g.npx; g.KW = (g.K + 3) & ~3;
+    g.DP = g.KW + ((4 - g.KW % 64) + 64) % 64;
+    if (g.nb == 1 || ((size_t)kBM * g.DP + (size_t)g.nb * kCT * g.XP + g.KW) * 4 <= kLdsLimit) break;
+  }
   g.HW = g.H * g.W; g.CKK = g.C * 9;
   g.ngroups = (g.B + g.nb - 1) / g.nb;
   const int64_t tiles = (C / kCT) * ((F + kBM - 1) / kBM);
@@ -280,10 +286,17 @@ bool wgrad_small_plan(const gh_ctx* ctx, const gh_cmd& c, WgPlan* out) {
   out->splits = (int)splits;
   out->lds = ((size_t)kBM * g.DP + (size_t)g.nb * kCT * g.XP + g.KW) * 4;
   out->lds = std::max<size_t>(out->lds, (size_t)4 * 9 * 64 * 16);   // the two halves' partial tiles meet in it
-  return out->lds <= 150 * 1024;
+  return out->lds <= kLdsLimit;
 }
 
 }  // namespace
+
+// Whether the kernel takes the command: a function of its shape alone.
+bool gh_conv_wgrad_small_takes(const gh_cmd& c) {
+  gh_ctx probe;   // only its compute-unit count is read, for the slab count
+  WgPlan p;
+  return wgrad_small_plan(&probe, c, &p);
+}
 
 // Returns -1 when the shape is not one this kernel takes (or its slabs do not fit the
 // workspace); otherwise the partial sums are in the workspace as *splits slabs of F x C*9

@@ -3191,6 +3191,15 @@ extern "C" int gh_conv2d_route(const gh_cmd* c) {
   return GH_CONV_ROUTE_GATHER;
 }
 
+// The dispatch order of gh_launch_conv2d_bwd_filter, asked without launching.
+extern "C" int gh_conv2d_bwd_filter_route(const gh_cmd* c) {
+  if (!c || c->opcode != GH_OP_CONV2D_BWD_FILTER) return -1;
+  if (gh_dtype_of(c->flags) == GH_F64) return GH_WGRAD_ROUTE_F64;
+  if (conv_direct_shape(*c) && c->dim[4] <= 65535) return GH_WGRAD_ROUTE_DIRECT;
+  if (gh_conv_wgrad_small_takes(*c)) return GH_WGRAD_ROUTE_SMALL;
+  return GH_WGRAD_ROUTE_GEMM;
+}
+
 extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {
   if (!c || c->opcode != GH_OP_CONV2D || gh_dtype_of(c->flags) != GH_F32) return 0;
   if (conv_direct_takes(*c)) {

@@ -311,6 +311,15 @@ enum gh_conv_route {
   GH_CONV_ROUTE_GATHER = 6      /* every other geometry                                   */
 };
 GH_API int gh_conv2d_route(const gh_cmd* conv);
+/* The same for a CONV2D_BWD_FILTER command (ConvolutionBackwardFilter,
+ * ops/nn/convolution_cuda.go:230-267): GH_WGRAD_ROUTE_*, or -1. */
+enum gh_wgrad_route {
+  GH_WGRAD_ROUTE_DIRECT = 0,  /* 3x3, at most four channels: reduction on the vector ALUs     */
+  GH_WGRAD_ROUTE_SMALL = 1,   /* 3x3 over images up to 16 x 16: dy and x in LDS, MFMA          */
+  GH_WGRAD_ROUTE_GEMM = 2,    /* every other geometry: implicit GEMM over the output pixels    */
+  GH_WGRAD_ROUTE_F64 = 3      /* float64 (its own kernels)                                     */
+};
+GH_API int gh_conv2d_bwd_filter_route(const gh_cmd* conv_bwd_filter);
 
 /* 1 when this GEMM command may carry GH_FLAG_GEMM_SOFTMAX: a float32 product of
  * untransposed operands with at most 32 columns and at most 2048 rows, whose

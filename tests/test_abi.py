@@ -158,3 +158,29 @@ def test_conv_route_of_every_parity_case_list():
     for (B, Cn, H, W, F, pad) in T.WIDE_CASES[:1]:
         seen.add(_route(B, Cn, H, W, F, (3, 3), (pad, pad)))
     assert seen == set(ROUTE.values()), seen
+
+
+def test_filter_gradient_routes():
+    """gh_conv2d_bwd_filter_route: the backward case table reaches all three float32 kernels, the cases written
+    for the small-image kernel run on it, and the training configurations' layers run where the design says."""
+    from tests import test_gpu_backward as T
+    lib = _ffi.load()
+
+    def route(B, Cn, H, W, F, kh, kw, pad, stride=(1, 1), dil=(1, 1), dtype=_ffi.F32):
+        cmd = D.cmd_conv2d_bwd_filter(0x10000, 0x20000, 0x30000, B, Cn, H, W, F, kh, kw, pad, stride, dil, dtype=dtype)
+        return lib.gh_conv2d_bwd_filter_route(C.byref(cmd))
+
+    DIRECT, SMALL, GEMM, F64 = 0, 1, 2, 3
+    seen = [route(*c) for c in T.CONV_BWD_CASES]
+    assert set(seen) == {DIRECT, SMALL, GEMM}
+    small = [c for c in T.CONV_BWD_CASES if c[1] % 16 == 0 and c[2] <= 16 and c[3] <= 16 and c[4] >= 16 and c[5] == 3]
+    assert len(small) >= 8
+    for c in small:
+        assert route(*c) == SMALL, c
+    assert route(128, 1, 28, 28, 32, 3, 3, (1, 1)) == DIRECT          # convnet conv0
+    assert route(128, 32, 14, 14, 64, 3, 3, (1, 1)) == SMALL          # conv1
+    assert route(128, 64, 7, 7, 128, 3, 3, (1, 1)) == SMALL           # conv2
+    assert route(8, 512, 13, 13, 1024, 3, 3, (1, 1)) == SMALL         # yolo-shaped layer 6
+    assert route(8, 64, 52, 52, 128, 3, 3, (1, 1)) == GEMM            # layer 3: images too large for LDS
+    assert route(128, 32, 14, 14, 64, 3, 3, (1, 1), dtype=_ffi.F64) == F64
+    assert lib.gh_conv2d_bwd_filter_route(C.byref(D.cmd_relu(0x1000, 0x2000, 16))) == -1
