@@ -92,6 +92,7 @@ SYMBOLS = {
     "gh_conv2d_can_pool": (C.c_int, [C.POINTER(GhCmd)]),
     "gh_conv2d_route": (C.c_int, [C.POINTER(GhCmd)]),
     "gh_conv2d_bwd_filter_route": (C.c_int, [C.POINTER(GhCmd)]),
+    "gh_gemm_route": (C.c_int, [C.POINTER(GhCmd), C.POINTER(C.c_int)]),
     "gh_gemm_can_softmax": (C.c_int, [C.POINTER(GhCmd)]),
     "gh_sync": (C.c_int, [_P]),
     "gh_graph_begin": (C.c_int, [_P]),

@@ -2883,6 +2883,25 @@ int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
   return launch_sgemm_cfg<64, 64, 2>(ctx, c, p.splits);
 }
 
+// The choices of gh_launch_gemm for a float32 product, asked without launching (MI355X's
+// compute-unit count, a workspace of the default size).
+extern "C" int gh_gemm_route(const gh_cmd* c, int* splits) {
+  if (splits) *splits = 1;
+  if (!c || c->opcode != GH_OP_GEMM) return -1;
+  if (gh_dtype_of(c->flags) == GH_F64) return GH_GEMM_ROUTE_F64;
+  const int64_t batch = c->dim[6] <= 0 ? 1 : c->dim[6];
+  const bool ta = c->flags & GH_FLAG_TRANS_A, tb = c->flags & GH_FLAG_TRANS_B;
+  gh_ctx probe;
+  probe.workspace = &probe;   // never dereferenced: only "there is one" and its size are read
+  probe.workspace_bytes = 64ll << 20;
+  if (batch == 1 && !(ta && tb) && cdiv(c->dim[0], 32) * cdiv(c->dim[1], 32) <= probe.cu_count && c->dim[2] >= 32 &&
+      !getenv("GORGONIA_HIP_GEMM_PLAN"))
+    return GH_GEMM_ROUTE_SMALL_OUTPUT;
+  const TilePlan p = plan_tiles(&probe, c->dim[0], c->dim[1], c->dim[2], batch, false);
+  if (splits) *splits = p.splits;
+  return p.tile == kTile128 ? GH_GEMM_ROUTE_TILE128 : p.tile == kTile128x64 ? GH_GEMM_ROUTE_TILE128X64 : GH_GEMM_ROUTE_TILE64;
+}
+
 // The direct kernel's shapes: 3x3, stride 1, no dilation, square padding, at
 // most four input channels.
 static bool conv_direct_shape(const gh_cmd& c) {

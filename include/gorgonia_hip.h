@@ -320,6 +320,17 @@ enum gh_wgrad_route {
   GH_WGRAD_ROUTE_F64 = 3      /* float64 (its own kernels)                                     */
 };
 GH_API int gh_conv2d_bwd_filter_route(const gh_cmd* conv_bwd_filter);
+/* The same for a GEMM command (Engine.MatMul, cuda/linalg.go:110-229, where cuBLAS chooses):
+ * GH_GEMM_ROUTE_*, or -1; *splits (may be null) receives the number of K slices whose slabs a
+ * second launch adds, 1 for a single launch. */
+enum gh_gemm_route {
+  GH_GEMM_ROUTE_SMALL_OUTPUT = 0, /* few output tiles: K split over the wavefronts of a workgroup */
+  GH_GEMM_ROUTE_TILE128 = 1,      /* 128 x 128 tiles through LDS                                 */
+  GH_GEMM_ROUTE_TILE64 = 2,       /* 64 x 64 tiles (+ K slices)                                  */
+  GH_GEMM_ROUTE_TILE128X64 = 3,
+  GH_GEMM_ROUTE_F64 = 4           /* float64 (its own kernels)                                   */
+};
+GH_API int gh_gemm_route(const gh_cmd* gemm, int* splits);
 
 /* 1 when this GEMM command may carry GH_FLAG_GEMM_SOFTMAX: a float32 product of
  * untransposed operands with at most 32 columns and at most 2048 rows, whose

@@ -184,3 +184,33 @@ def test_filter_gradient_routes():
     assert route(8, 64, 52, 52, 128, 3, 3, (1, 1)) == GEMM            # layer 3: images too large for LDS
     assert route(128, 32, 14, 14, 64, 3, 3, (1, 1), dtype=_ffi.F64) == F64
     assert lib.gh_conv2d_bwd_filter_route(C.byref(D.cmd_relu(0x1000, 0x2000, 16))) == -1
+
+
+def test_gemm_routes():
+    """gh_gemm_route: the matrix-product case table reaches the small-output kernel and the tiled one with and
+    without K slices; the benchmark's products run where the design says."""
+    from tests import test_gpu_linalg as T
+    lib = _ffi.load()
+
+    def route(m, k, n, ta=False, tb=False, batch=1, dtype=_ffi.F32):
+        sp = C.c_int(0)
+        kind = lib.gh_gemm_route(C.byref(D.cmd_gemm(0x1000, 0x2000, 0x3000, m, n, k, trans_a=ta, trans_b=tb, batch=batch,
+                                                    dtype=dtype)), C.byref(sp))
+        return kind, sp.value
+
+    SMALL, T128, T64, T128X64, F64 = range(5)
+    seen = set()
+    for (m, k, n) in T.SHAPES:
+        for ta in (False, True):
+            for tb in (False, True):
+                kind, sp = route(m, k, n, ta, tb)
+                seen.add((kind, sp > 1))
+    assert {(SMALL, False), (T64, False), (T64, True)} <= seen, seen
+    assert route(4096, 4096, 4096) == (T128, 1)                      # configuration 3
+    assert route(512, 512, 512, batch=64) == (T128, 1)
+    for (m, k, n) in ((256, 784, 300), (256, 300, 100), (256, 100, 10), (128, 1152, 625), (128, 625, 10)):
+        assert route(m, k, n) == (SMALL, 1), (m, k, n)               # dense layers of configurations 1 and 4
+    assert route(1152, 128, 625, ta=True) == (T64, 1)                # a dense layer's weight gradient: K = batch
+    assert route(1152, 2048, 625)[0] == T64 and route(1152, 2048, 625)[1] > 1
+    assert route(64, 64, 64, dtype=_ffi.F64)[0] == F64
+    assert lib.gh_gemm_route(C.byref(D.cmd_relu(0x1000, 0x2000, 16)), None) == -1
