@@ -31,8 +31,27 @@
  *   tanh / exp f32                         - PARITY UNPINNED bit-for-bit: the
  *                                            reference routes these through
  *                                            math32 (not vendored).  Oracle is
- *                                            float64 libm rounded once; the
- *                                            2-ulp budget covers the gap.
+ *                                            float64 libm rounded once (checked
+ *                                            against 200-bit values rounded once);
+ *                                            the 2-ulp budget covers the gap.
+ *   abs neg square cube ceil floor sqrt    - single IEEE operations: numpy's bits,
+ *   inverse invsqrt (f32 and f64)            signed zeros, NaN, infinities, denormals
+ *   sin cos exp ln log2 log1p expm1 tanh   - 200-bit mpmath values rounded once
+ *   (f32 and f64)                            (<= 1 ulp, f32 equal on > 99.9 %), and
+ *                                            known values that tell the codes apart
+ *   softplus, float64 sigmoid              - cut-offs of math.go:50-68 and
+ *                                            math_nooptim.go:25-34 at their
+ *                                            neighbours, where cut-off and formula
+ *                                            differ; values as above
+ *   sign                                   - numpy sign on non-zero numbers; at +-0
+ *                                            and NaN the device kernel's form
+ *                                            (elemunaryop.cu:125-131) gives +0.  The
+ *                                            CPU engine's tensor.Signer is not
+ *                                            vendored: PARITY UNPINNED at +-0 / NaN
+ *   pow (general)                          - exact cases (integer powers, square
+ *                                            roots of squares, powers of two,
+ *                                            C99 / Go special cases), 200-bit
+ *                                            values rounded once, exact integers
  *   batch norm backward                    - nn_amd64_test.go ExpectedInputGrad
  *                                            goldens; finite differences of the
  *                                            training forward

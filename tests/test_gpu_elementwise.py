@@ -176,6 +176,63 @@ def test_unary_bit_exact(ctx, fn):
         ctx.free(d)
 
 
+UNARY_SPECIALS = [0.0, -0.0, np.nan, np.inf, -np.inf, 1e-42, -1e-42, 1.0, -1.0, 2.5, -2.5, 0.5, -0.5,
+                  3.0e38, -3.0e38, 16777216.0]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("fn", EXACT_UNARY)
+def test_unary_special_values_bit_exact(ctx, fn, dtype):
+    """Signed zeros, NaN, infinities and denormals through the single-operation codes, both
+    widths.  sign follows the device kernel form (x > 0) - (x < 0) of
+    "cuda modules/src/elemunaryop.cu":125-131: +0 for +0, -0 and NaN."""
+    x = np.array(UNARY_SPECIALS, dtype=dtype)
+    d = ctx.upload(x)
+    ctx.run(D.cmd_unary(fn, d, x.size, dtype=_ffi.F32 if dtype == np.float32 else _ffi.F64))
+    got = ctx.d2h(d, (x.size,), dtype)
+    ctx.free(d)
+    with np.errstate(all="ignore"):
+        want = O.unary(fn, x)
+    assert_bits_equal(got, want, f"{fn} {dtype.__name__}")
+    if fn == "sign":
+        z = got[:3].view(np.uint32 if dtype == np.float32 else np.uint64)
+        assert (z == 0).all(), "sign(+0), sign(-0), sign(NaN) must be +0"
+
+
+@pytest.mark.parametrize("fn", ULP2 + EXACT_UNARY)
+def test_unary_float64(ctx, fn):
+    """The float64 twins: single-operation codes bit-exact, the transcendental ones within
+    2 float64 ulp of the oracle (float64 libm), cut-offs of the reference's scalar forms
+    (math.go:50-58, math_nooptim.go:25-34) included in the inputs."""
+    n = 20011
+    x = _unary_input(fn, n, 53).astype(np.float64)
+    x[16:] += np.random.default_rng(54).uniform(-1e-9, 1e-9, n - 16) * np.abs(x[16:])  # use the low mantissa bits
+    if fn == "sigmoid":
+        x[16:32] = [-709.0, -709.5, np.nextafter(-709.0, -800.0), -708.9, 19.0, 19.5, np.nextafter(19.0, 20.0), 16.0,
+                    -100.0, -88.5, 15.5, 18.99, -700.0, 0.0, 40.0, -800.0]
+    if fn == "softplus":
+        x[16:32] = [-708.0, -708.5, np.nextafter(-708.0, -800.0), -707.9, 16.0, 16.5, np.nextafter(16.0, 17.0), 15.0,
+                    -200.0, -103.5, 14.5, 15.99, -700.0, 0.0, 40.0, -800.0]
+    d = ctx.upload(x)
+    ctx.run(D.cmd_unary(fn, d, n, dtype=_ffi.F64))
+    got = ctx.d2h(d, (n,), np.float64)
+    ctx.free(d)
+    with np.errstate(all="ignore"):
+        want = O.unary(fn, x)
+    if fn in EXACT_UNARY:
+        assert_bits_equal(got, want, f"{fn} float64")
+        return
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    gi, wi = got[ok].view(np.int64), want[ok].view(np.int64)
+    gi = np.where(gi < 0, -(gi & 0x7FFFFFFFFFFFFFFF), gi)
+    wi = np.where(wi < 0, -(wi & 0x7FFFFFFFFFFFFFFF), wi)
+    u = np.abs(gi - wi)
+    assert u.max() <= 2, f"{fn}: {u.max()} ulp at x={x[ok][int(u.argmax())]!r}"
+    if fn in ("sigmoid", "softplus"):   # the cut-offs store exact values
+        assert_bits_equal(got[16:32][[1, 2, 5, 6, 15]], want[16:32][[1, 2, 5, 6, 15]], f"{fn} cut-offs")
+
+
 @pytest.mark.parametrize("fn", ["sigmoid", "tanh"])
 def test_sigmoid_tanh_dense_sweep(ctx, fn):
     """Every 61st float32 bit pattern of both signs (70 million values, NaNs and infinities
