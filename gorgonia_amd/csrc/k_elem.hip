@@ -127,15 +127,21 @@ __device__ __forceinline__ double tanh_f64_for_f32(double x) {
 // ---- float32 sigmoid / tanh without float64 ---------------------------------------
 // The float64 forms above are within half an ulp but cost two quarter-rate
 // conversions, a float64 reciprocal and ~20 half-rate FMAs per element, which
-// makes a streaming kernel ALU-bound on this part.  These stay in float32 and
-// within 2 ulp of the correctly rounded result (measured: the dense sweep in
-// the GPU tests), and leave the kernels memory-bound.
+// makes a streaming kernel ALU-bound on this part.  These stay in float32, take
+// about twenty instructions each and stay within 2 ulp of the correctly rounded
+// result over every float32 input (measured exhaustively; the dense sweep in the
+// GPU tests repeats it against the CPU oracle): sigmoid at most 2, tanh at most 1.
+// With fewer instructions the kernels stay memory-bound at the clocks a device
+// holds after minutes of load as well.
 //
 // exp(t) = 2^n * (1 + q): n = round(t / ln2) through the 1.5*2^23 shift (the
-// integer also sits in the low mantissa bits), Cody-Waite reduction with a
-// short-mantissa ln2 high part so that n*ln2_hi is exact, and
-// exp(r) - 1 = r + r^2 P(r) with the classic degree-5 float32 coefficients.
-struct ExpF { float q; int n; };
+// integer also sits in the low mantissa bits of `shifted`), Cody-Waite reduction
+// with a short-mantissa ln2 high part so that n*ln2_hi is exact, and
+// exp(r) - 1 = r + r^2 P(r) with a degree-4 minimax P on |r| <= ln2/2 (relative
+// error of exp below 2^-28).
+struct ExpF { float q; int shbits; };
+
+constexpr unsigned kShiftBits = 0x4B400000u;   // bits of 1.5 * 2^23
 
 __device__ __forceinline__ ExpF expf_parts(float t) {
   const float kShift = 12582912.0f;  // 1.5 * 2^23
@@ -143,71 +149,69 @@ __device__ __forceinline__ ExpF expf_parts(float t) {
   const float nf = shifted - kShift;
   float r = __builtin_fmaf(-nf, 0.693145751953125f, t);
   r = __builtin_fmaf(-nf, 1.428606765330187e-06f, r);
-  float p = 1.9875691500e-4f;
-  p = __builtin_fmaf(p, r, 1.3981999507e-3f);
-  p = __builtin_fmaf(p, r, 8.3334519073e-3f);
-  p = __builtin_fmaf(p, r, 4.1665795894e-2f);
-  p = __builtin_fmaf(p, r, 1.6666665459e-1f);
-  p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+  float p = 0.0013813756f;
+  p = __builtin_fmaf(p, r, 0.008369124f);
+  p = __builtin_fmaf(p, r, 0.041668426f);
+  p = __builtin_fmaf(p, r, 0.16666517f);
+  p = __builtin_fmaf(p, r, 0.49999994f);
   ExpF e;
   e.q = __builtin_fmaf(r * r, p, r);
-  e.n = __float_as_int(shifted) - __float_as_int(kShift);
+  e.shbits = __float_as_int(shifted);
   return e;
 }
 
-// 1/d to about half an ulp (hardware estimate + one Newton step), then corrected
-// for `derr`, the rounding error of d itself: 1/(d + derr) = r - r^2 derr.
-__device__ __forceinline__ float rcp_f32_comp(float d, float derr) {
-  float r = __builtin_amdgcn_rcpf(d);
-  r = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
-  return __builtin_fmaf(-(r * r), derr, r);
+// 2^(n + bias) as a float from the shifted sum's bits: one shift-and-add.
+template <int BIAS>
+__device__ __forceinline__ float pow2_of(int shbits) {
+  return __int_as_float((shbits << 23) + (int)(((unsigned)(127 + BIAS) << 23) - (kShiftBits << 23)));
 }
 
-// sigmoid with the reference's cut-offs (math_nooptim.go:36-44): with
-// e = exp(-|x|) <= 1, 1/(1+e) for x >= 0 and e/(1+e) for x < 0.  e and 1+e are
-// carried as (high, low) pairs and the quotient gets one residual correction,
-// which leaves the polynomial's own error (about 0.3 ulp) plus the final
-// rounding: within 1 ulp of the correctly rounded value over the dense sweep.
+// sigmoid with the reference's cut-offs (math_nooptim.go:36-44).  With E = exp(|x|) =
+// 2^n (1 + q), r = 1 / (1 + E) is sigmoid(-|x|) and 1 - r is sigmoid(|x|).  The sum
+// 1 + E is formed scaled by 2^-64, as (2^(n-64) q + 2^-64) + 2^(n-64): two roundings
+// of at most 0.9 ulp together for every n (adding the 1 to 2^n first would lose it
+// from n = 24 on), and the scaling keeps the hardware reciprocal's result normal
+// where r itself is subnormal (x below -87.3); the final multiply-add by 2^-64
+// rounds once.  Beyond the cut-offs r is replaced by 0, which gives exactly 0 and 1.
+// NaN fails the compare and propagates through r.
 __device__ __forceinline__ float sigmoid_f32_fast(float x) {
-  const ExpF p = expf_parts(-fabsf(x));
-  const float t = 1.0f + p.q;
-  const float tl = p.q - (t - 1.0f);           // exact: |q| < 1
-  const float e_hi = ldexpf(t, p.n);           // denormal below exp(-87.3), rounded once
-  const float e_lo = ldexpf(tl, p.n);
-  const float d_hi = 1.0f + e_hi;
-  const float d_lo = (e_hi - (d_hi - 1.0f)) + e_lo;
-  // the hardware estimate of 1/d is good to an ulp; the residual step below squares that error away
-  const float r = __builtin_amdgcn_rcpf(d_hi);
-  const bool neg = x < 0.0f;
-  const float num_hi = neg ? e_hi : 1.0f, num_lo = neg ? e_lo : 0.0f;
-  const float q0 = num_hi * r;
-  const float rem = __builtin_fmaf(-q0, d_hi, num_hi);          // exact remainder of the first quotient
-  float s = __builtin_fmaf((rem + num_lo) - q0 * d_lo, r, q0);
-  s = x < -88.0f ? 0.0f : s;
-  s = x > 15.0f ? 1.0f : s;
-  return s;                                    // NaN fails every compare and propagates
+  const float a = fabsf(x);
+  const ExpF p = expf_parts(a);
+  const float s = pow2_of<-64>(p.shbits);
+  const float c = 5.421010862427522e-20f;                       // 2^-64
+  const float d = __builtin_fmaf(s, p.q, c) + s;
+  float rc = __builtin_amdgcn_rcpf(d);                          // 2^64 / (1 + E), within an ulp
+  const float cs = copysignf(c, x);
+  const float lim = __builtin_fmaf(cs, -36.5f * 18446744073709551616.0f, 51.5f);   // 15 right of zero, 88 left
+  const float base = __builtin_fmaf(cs, 0.5f * 18446744073709551616.0f, 0.5f);     // 1 right of zero, 0 left
+  rc = a > lim ? 0.0f : rc;
+  return __builtin_fmaf(-cs, rc, base);
 }
 
 // tanh: below 0.55 an odd polynomial x + x^3 R(x^2) (R fitted on [0, 0.56^2],
 // approximation error 0.07 ulp); above it 1 - 2/(e^(2|x|) + 1), where the result
-// is at least 0.5 and the subtraction costs no accuracy.
+// is at least 0.5 and the quotient's error (the sum's single rounding and the
+// hardware reciprocal's ulp) shrinks by the factor 2/(e^(2|x|) + 1) <= 1/2.
+// The exponential's argument is clamped (tanh(22) rounds to 1); the clamp drops a
+// NaN, so the choice between the two forms is written to fall to the polynomial,
+// which keeps it, when the compare fails.
 __device__ __forceinline__ float tanh_f32_fast(float x) {
   const float ax = fabsf(x);
-  const float s = ax * ax;
+  const float s2 = ax * ax;
   float R = 0.0024976127315312624f;
-  R = __builtin_fmaf(R, s, -0.008506525307893753f);
-  R = __builtin_fmaf(R, s, 0.02181374467909336f);
-  R = __builtin_fmaf(R, s, -0.05396425351500511f);
-  R = __builtin_fmaf(R, s, 0.133333221077919f);
-  R = __builtin_fmaf(R, s, -0.3333333432674408f);
-  const float small = __builtin_fmaf(ax * s, R, ax);
-  const float a = (ax > 10.0f ? 10.0f : ax) * 2.0f;   // tanh(10) rounds to 1; NaN stays NaN
-  const ExpF p = expf_parts(a);
-  const float e = ldexpf(1.0f + p.q, p.n);
-  const float d = e + 1.0f;
-  const float r = rcp_f32_comp(d, 1.0f - (d - e));
-  const float large = __builtin_fmaf(-2.0f, r, 1.0f);
-  return copysignf(ax < 0.55f ? small : large, x);
+  R = __builtin_fmaf(R, s2, -0.008506525307893753f);
+  R = __builtin_fmaf(R, s2, 0.02181374467909336f);
+  R = __builtin_fmaf(R, s2, -0.05396425351500511f);
+  R = __builtin_fmaf(R, s2, 0.133333221077919f);
+  R = __builtin_fmaf(R, s2, -0.3333333432674408f);
+  const float small = __builtin_fmaf(ax * s2, R, ax);
+  const float ac = fminf(ax, 22.0f);
+  const ExpF p = expf_parts(ac + ac);
+  const float s = pow2_of<0>(p.shbits);
+  const float d = __builtin_fmaf(s, p.q, s + 1.0f);             // e^(2|x|) + 1 in one rounding (n <= 64 / ln2)
+  const float rc = __builtin_amdgcn_rcpf(d);
+  const float large = __builtin_fmaf(-2.0f, rc, 1.0f);
+  return copysignf(ax >= 0.55f ? large : small, x);
 }
 
 template <int FN>
