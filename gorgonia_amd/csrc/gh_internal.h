@@ -2,6 +2,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <cstdint>
+#include <cstring>
+#include <mutex>
 #include <string>
 #include <utility>
 #include <vector>
@@ -109,6 +111,10 @@ int gh_try_launch_conv_wgrad_small(gh_ctx* ctx, const gh_cmd& c, int* splits);
 bool gh_conv_wgrad_small_takes(const gh_cmd& c);
 bool gh_conv_small_takes(const gh_cmd& c);
 bool gh_conv_small_can_pool(const gh_cmd& c);
+// its 32- and 64-channel kernel (k_conv_rows.hip), same conventions
+int gh_try_launch_conv_rows(gh_ctx* ctx, const gh_cmd& c);
+bool gh_conv_rows_takes(const gh_cmd& c);
+bool gh_conv_rows_can_pool(const gh_cmd& c);
 // 3x3 convolution over patches with K split across wavefronts (k_conv_patch.hip), same conventions
 int gh_try_launch_conv_patch(gh_ctx* ctx, const gh_cmd& c);
 bool gh_conv_patch_takes(const gh_cmd& c);
@@ -144,6 +150,37 @@ bool gh_try_launch_conv2d_bwd_data_f64_mfma(gh_ctx* ctx, const gh_cmd& c);
 bool gh_try_launch_conv2d_bwd_filter_f64_mfma(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_dropout(gh_ctx* ctx, const gh_cmd& c);
 int gh_launch_dropout_bwd(gh_ctx* ctx, const gh_cmd& c);
+
+// A convolution kernel's plan (geometry and workgroup shape) is a function of the command's shape,
+// its dtype and of whether a pooling rides in the epilogue - and of tuning switches in the environment,
+// which are read when a shape is first seen.  Finding one costs tens of microseconds on the host and a
+// command asks several times (validation, the pooling query, the launcher), which an eager submit
+// cannot hide behind kernels of a few microseconds: gh_plan_memo keeps the answers.  One table per call
+// site (the lambda's type makes the instantiation unique); bounded, cleared when full.
+template <class Plan, class Fn>
+bool gh_plan_memo(const gh_cmd& c, bool pool, Plan* out, Fn&& compute) {
+  struct Entry { int64_t dim[13]; uint32_t dtype; bool pool, ok; Plan plan; };
+  static std::mutex mu;
+  static std::vector<Entry> table;
+  const uint32_t dtype = (c.flags >> 12) & 0xfu;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    for (const Entry& e : table)
+      if (e.pool == pool && e.dtype == dtype && memcmp(e.dim, c.dim, sizeof(e.dim)) == 0) {
+        if (e.ok) *out = e.plan;
+        return e.ok;
+      }
+  }
+  Entry e;
+  memcpy(e.dim, c.dim, sizeof(e.dim));
+  e.dtype = dtype; e.pool = pool;
+  e.ok = compute(&e.plan);
+  std::lock_guard<std::mutex> lock(mu);
+  if (table.size() >= 256) table.clear();
+  table.push_back(e);
+  if (e.ok) *out = e.plan;
+  return e.ok;
+}
 
 static inline uint32_t gh_fn(uint32_t flags) { return flags & 0xffu; }
 static inline uint32_t gh_mode(uint32_t flags) { return (flags >> 8) & 0xfu; }

@@ -284,7 +284,7 @@ constexpr int kTileMenu[] = {4, 7, 9, 11};   // instantiated N extents (in 16-pi
 
 // Geometry and workgroup shape for one command, a function of its shape and of `pool`
 // only; false when the kernel does not take the shape.
-bool patch_plan(const gh_cmd& c, bool pool, PatchPlan* out) {
+bool patch_plan_compute(const gh_cmd& c, bool pool, PatchPlan* out) {
   if (gh_dtype_of(c.flags) != GH_F32) return false;
   const int64_t B = c.dim[0], C = c.dim[1], H = c.dim[2], W = c.dim[3], F = c.dim[4];
   const int64_t pad = c.dim[7];
@@ -340,6 +340,11 @@ bool patch_plan(const gh_cmd& c, bool pool, PatchPlan* out) {
   lds += (size_t)4 * 16 * TM * 4;
   out->g = g; out->TM = TM; out->TN = bTN; out->lds = lds;
   return lds <= 150 * 1024;
+}
+
+// The plan of a command, remembered per shape (the search over patch shapes costs tens of microseconds).
+bool patch_plan(const gh_cmd& c, bool pool, PatchPlan* out) {
+  return gh_plan_memo(c, pool, out, [&](PatchPlan* p) { return patch_plan_compute(c, pool, p); });
 }
 
 template <int TM, int TN>

@@ -323,7 +323,7 @@ constexpr int kTileMenu[] = {4, 7, 9, 13};       // instantiated N extents (in 1
 
 // Geometry and workgroup shape for one command, a function of its shape and of
 // `pool` only; false when the kernel does not take the shape.
-bool small_plan(const gh_cmd& c, bool pool, SmallPlan* out) {
+bool small_plan_compute(const gh_cmd& c, bool pool, SmallPlan* out) {
   if (gh_dtype_of(c.flags) != GH_F32) return false;
   const int64_t B = c.dim[0], C = c.dim[1], H = c.dim[2], W = c.dim[3], F = c.dim[4];
   const int64_t pad = c.dim[7];
@@ -395,6 +395,11 @@ bool small_plan(const gh_cmd& c, bool pool, SmallPlan* out) {
   return true;
 }
 
+// The plan of a command, remembered per shape.
+bool small_plan(const gh_cmd& c, bool pool, SmallPlan* out) {
+  return gh_plan_memo(c, pool, out, [&](SmallPlan* p) { return small_plan_compute(c, pool, p); });
+}
+
 template <int WV, int TM, int TN, int NQ>
 int launch_small(gh_ctx* ctx, const gh_cmd& c, const SmallPlan& p) {
   // more than 64 KB of dynamic LDS has to be allowed per kernel, once
@@ -428,20 +433,28 @@ int launch_small_tile(gh_ctx* ctx, const gh_cmd& c, const SmallPlan& p) {
 
 }  // namespace
 
-// 1 when the small-image kernel takes this convolution (without fused pooling).
+// The small-image route is two kernels: 32 and 64 channels go to k_conv3x3_rows (k_conv_rows.hip, pixels
+// on the MFMA rows, no K split for regular tiles), the other channel counts to the K-split kernel above.
+// Which of the two runs depends on the command's shape alone.
+
+// 1 when the small-image route takes this convolution (without fused pooling).
 bool gh_conv_small_takes(const gh_cmd& c) {
+  if (gh_conv_rows_takes(c)) return true;
   SmallPlan p;
   return small_plan(c, false, &p);
 }
 
 // 1 when it also takes it with the 2x2 pooling in its epilogue.
 bool gh_conv_small_can_pool(const gh_cmd& c) {
+  if (gh_conv_rows_takes(c)) return gh_conv_rows_can_pool(c);
   SmallPlan p;
   return small_plan(c, false, &p) && small_plan(c, true, &p);
 }
 
-// Returns -1 when the shape is not one this kernel takes.
+// Returns -1 when the shape is not one this route takes.
 int gh_try_launch_conv_small(gh_ctx* ctx, const gh_cmd& c) {
+  const int rows = gh_try_launch_conv_rows(ctx, c);
+  if (rows >= 0) return rows;
   SmallPlan p;
   const bool pool = c.flags & GH_FLAG_CONV_POOL2;
   // a pooled command only rides here when the plain one would too: both then sum in the same order

@@ -390,7 +390,7 @@ inline size_t wide_lds(const WideGeom& g, int TM, int TN, int PL, bool db) {
 
 // Geometry and workgroup shape for one command, a function of its shape and of `pool`
 // only; false when the kernel does not take the shape.
-bool wide_plan(const gh_cmd& c, bool pool, WidePlan* out) {
+bool wide_plan_compute(const gh_cmd& c, bool pool, WidePlan* out) {
   if (gh_dtype_of(c.flags) != GH_F32) return false;
   const int64_t B = c.dim[0], C = c.dim[1], H = c.dim[2], W = c.dim[3], F = c.dim[4];
   const int64_t pad = c.dim[7];
@@ -473,6 +473,11 @@ bool wide_plan(const gh_cmd& c, bool pool, WidePlan* out) {
       }
     }
   return found;
+}
+
+// The plan of a command, remembered per shape (the search over patch shapes costs 60-150 microseconds).
+bool wide_plan(const gh_cmd& c, bool pool, WidePlan* out) {
+  return gh_plan_memo(c, pool, out, [&](WidePlan* p) { return wide_plan_compute(c, pool, p); });
 }
 
 template <int TM, int TN, int XS, bool DB>
