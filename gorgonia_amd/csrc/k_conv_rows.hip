@@ -221,7 +221,8 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
   const int outplane = g.outplane;
   const float alpha = tail.alpha;
   // the epilogue of one tile: four N entries of filter `fcol` in v
-  auto finish = [&](auto bn_c, auto act_c, f32x4 v, int pt, int fcol, const float (&k)[4]) {
+  // (o1: the window's result offset when pooling, read from the table by the caller)
+  auto finish = [&](auto bn_c, auto act_c, f32x4 v, int pt, int o1, int fcol, const float (&k)[4]) {
     constexpr bool BN = decltype(bn_c)::value;
     constexpr int ACT = decltype(act_c)::value;
     const bool ok = fcol < g.F;
@@ -231,8 +232,7 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
       float best = -3.402823466e+38f;
 #pragma unroll
       for (int r = 0; r < 4; r++) if (v[r] > best) best = v[r];   // window positions in scan order
-      const int o = tabO[4 * pt + lk];
-      if (ok && o >= 0) ybase[o + fcol * outplane] = best;
+      if (ok && o1 >= 0) ybase[o1 + fcol * outplane] = best;
     } else {
       const i32x4 o = *reinterpret_cast<const i32x4*>(tabO + 16 * pt + 4 * lk);
 #pragma unroll
@@ -241,36 +241,45 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
     }
   };
 
-  // ---- leftover units: this wavefront's quads [wave * QW, +QW) of every leftover (pixel tile, filter tile),
-  // RC units per round: partial tiles to LDS, barrier, wavefront j adds unit j's eight in wavefront order
+  // ---- leftover pixel tiles: this wavefront's quads [wave * QW, +QW) of each, for every filter tile of the
+  // workgroup (a unit = pixel tile x filter tile); RC units per round: partial tiles to LDS, barrier,
+  // wavefront j adds unit j's eight in wavefront order
   if (g.LU > 0) {
     const float* const lf = Wl + wave * QW * 9 * 64 + lane;
-    for (int u0 = 0; u0 < g.LU; u0 += g.RC) {
-      const int nu = min(g.RC, g.LU - u0);
-      if (u0 > 0) __syncthreads();   // the last round's sums are done with the slots
-      for (int j = 0; j < nu; j++) {
-        const int u = u0 + j, t = u / TFB, fi = u - t * TFB;
-        const float* const lp = Ps + tabP[(g.PTR + t) * 16 + li] + lkoff + wave * QW * QPs;
-        const float* const lfu = lf + fi * NQ * 9 * 64;
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    const int tiles_per_round = g.RC / TFB;   // RC is a multiple of TFB
+    const int ntiles = g.LU / TFB;
+    for (int t0 = 0; t0 < ntiles; t0 += tiles_per_round) {
+      const int nt = min(tiles_per_round, ntiles - t0);
+      if (t0 > 0) __syncthreads();   // the last round's sums are done with the slots
+      for (int j = 0; j < nt; j++) {
+        const float* const lp = Ps + tabP[(g.PTR + t0 + j) * 16 + li] + lkoff + wave * QW * QPs;
+        f32x4 acc[TFB];
+#pragma unroll
+        for (int fi = 0; fi < TFB; fi++) acc[fi] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int qq = 0; qq < QW; qq++)
 #pragma unroll
-          for (int tap = 0; tap < 9; tap++)
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(lp[qq * QPs + (tap / 3) * Wps + (tap % 3)],
-                                                       lfu[(qq * 9 + tap) * 64], acc, 0, 0, 0);
-        *reinterpret_cast<f32x4*>(Red + (j * kWaves + wave) * 256 + lane * 4) = acc;
+          for (int tap = 0; tap < 9; tap++) {
+            const float pv = lp[qq * QPs + (tap / 3) * Wps + (tap % 3)];
+#pragma unroll
+            for (int fi = 0; fi < TFB; fi++)
+              acc[fi] = __builtin_amdgcn_mfma_f32_16x16x4f32(pv, lf[((fi * NQ + qq) * 9 + tap) * 64], acc[fi], 0, 0, 0);
+          }
+#pragma unroll
+        for (int fi = 0; fi < TFB; fi++)
+          *reinterpret_cast<f32x4*>(Red + ((j * TFB + fi) * kWaves + wave) * 256 + lane * 4) = acc[fi];
       }
       __syncthreads();
-      if (wave < nu) {
-        const int u = u0 + wave, t = u / TFB, fi = u - t * TFB;
+      if (wave < nt * TFB) {
+        const int t = t0 + wave / TFB, fi = wave % TFB;
         f32x4 s = *reinterpret_cast<const f32x4*>(Red + (wave * kWaves) * 256 + lane * 4);
 #pragma unroll
         for (int k = 1; k < kWaves; k++) s = s + *reinterpret_cast<const f32x4*>(Red + (wave * kWaves + k) * 256 + lane * 4);
         const int fcol = m0 + fi * 16 + li;
+        const int o1 = POOL ? tabO[4 * (g.PTR + t) + lk] : 0;
         conv_tail_dispatch(tail, [&](auto bn_c, auto act_c) {
-          if (TFB == 1 || fi == 0) finish(bn_c, act_c, s, g.PTR + t, fcol, bn[0]);
-          else finish(bn_c, act_c, s, g.PTR + t, fcol, bn[TFB - 1]);
+          if (TFB == 1 || fi == 0) finish(bn_c, act_c, s, g.PTR + t, o1, fcol, bn[0]);
+          else finish(bn_c, act_c, s, g.PTR + t, o1, fcol, bn[TFB - 1]);
         });
       }
     }
@@ -281,8 +290,10 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
   if constexpr (A > 0) {
     const float* const fbase = Wl + ft * NQ * 9 * 64 + lane;
     const float* pb[A][FIXED ? 1 : 3];
+    int otab[A];
 #pragma unroll
     for (int t = 0; t < A; t++) {
+      otab[t] = POOL ? tabO[4 * (pg * A + t) + lk] : 0;
       const float* p = Ps + tabP[(pg * A + t) * 16 + li] + lkoff;
       pb[t][0] = p;
       if constexpr (!FIXED) { pb[t][1] = p + Wps; pb[t][2] = p + 2 * Wps; }
@@ -331,8 +342,8 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
     conv_tail_dispatch(tail, [&](auto bn_c, auto act_c) {
 #pragma unroll
       for (int t = 0; t < A; t++) {
-        if (TFB == 1 || ft == 0) finish(bn_c, act_c, acc[t], pg * A + t, fcol, bn[0]);
-        else finish(bn_c, act_c, acc[t], pg * A + t, fcol, bn[TFB - 1]);
+        if (TFB == 1 || ft == 0) finish(bn_c, act_c, acc[t], pg * A + t, otab[t], fcol, bn[0]);
+        else finish(bn_c, act_c, acc[t], pg * A + t, otab[t], fcol, bn[TFB - 1]);
       }
     });
   }
@@ -415,13 +426,16 @@ bool rows_plan_compute(const gh_cmd& c, bool pool, RowsPlan* out) {
       if (A > 4) break;
       const int LUu = (PTu - A * wave_groups) * TFB;
       size_t fl = (size_t)TFB * NQ * 576 + (size_t)IPB * NQ * g.QP + 32 * (size_t)PTu + 4;
-      if ((fl + (LUu ? 2048 : 0)) * 4 > kLdsBudget) break;
+      if ((fl + (LUu ? 2048 * TFB : 0)) * 4 > kLdsBudget) break;
       const size_t lds = (fl + (size_t)LUu * 2048) * 4 > kLdsBudget ? kLdsBudget : (fl + (size_t)LUu * 2048) * 4;
       const int64_t blocks = ((F + 16 * TFB - 1) / (16 * TFB)) * ((B + IPB - 1) / IPB);
       const int coresident = lds <= 79 * 1024 ? 2 : 1;
       const int64_t rounds = (blocks + 256 * coresident - 1) / (256 * coresident);
       const double mfma_us = (double)PTw * TFB * NQ * 9 / 4 * 32.0 / 2100.0;
-      const double est = rounds * (3.0 + coresident * mfma_us);
+      // what a workgroup does before its first MFMA grows with what it stages (measured on the convnet's
+      // layers: 32 filters x 1 image against 16 x 2 at 14 x 14, 16 x 4 against 32 x 2 at 7 x 7)
+      const double stage_us = 2.0 + 0.035 * (TFB * NQ * 576 * 4 / 1024.0) + 0.03 * ((double)IPB * NQ * g.QP * 4 / 1024.0);
+      const double est = rounds * (stage_us + coresident * mfma_us);
       if (!bestTFB || est < best) { best = est; bestTFB = TFB; bestIPB = IPB; }
     }
   }
@@ -449,8 +463,9 @@ bool rows_plan_compute(const gh_cmd& c, bool pool, RowsPlan* out) {
   // as many leftover units per round as the rest of LDS holds
   const int room = (int)((kLdsBudget / 4 - (size_t)off) / 2048);
   g.RC = g.LU < room ? g.LU : room;
-  if (g.LU > 0 && g.RC < 1) return false;
   if (g.RC > kWaves) g.RC = kWaves;
+  g.RC -= g.RC % TFB;   // whole pixel tiles per round
+  if (g.LU > 0 && g.RC < TFB) return false;
   off += g.RC * 2048;
   g.mW = magic_of(g.W); g.mNWIN = magic_of(g.nwin); g.mPW = magic_of(g.pw); g.mPER = magic_of(g.per);
   out->g = g; out->NQ = NQ; out->A = A; out->TFB = TFB; out->lds = (size_t)off * 4;
