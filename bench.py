@@ -44,6 +44,7 @@ def replay_mode():
 
 
 SUSTAIN_MS = 40.0   # a kernel is timed after this much back-to-back work of its own, over this much more
+IN_FLIGHT = 32      # graph replays queued between two host waits of the sustained loop
 
 
 def time_cmds(ctx, cmds, iters, warm=3):
@@ -79,11 +80,24 @@ def time_cmds(ctx, cmds, iters, warm=3):
         ctx.graph_destroy(gid)
         return time_cmds.last_burst_ms
     reps = max(1, min(4000, int(SUSTAIN_MS / max(one, 1e-3)) + 1))
-    for _ in range(reps):
-        ctx.graph_launch(gid)
+
+    def replay(n):
+        # At most 2 * IN_FLIGHT replays are ever queued: every IN_FLIGHT launches an event goes into the
+        # stream and the host waits for the event of the batch before (the device never runs dry: a whole
+        # batch is still queued behind the one it waits for).  Thousands of graph launches queued at
+        # once are what a run of this loop under a tracing profiler died of.
+        slot = 2
+        for i in range(n):
+            ctx.graph_launch(gid)
+            if (i + 1) % IN_FLIGHT == 0:
+                ctx.event(slot)
+                if i + 1 >= 2 * IN_FLIGHT:
+                    ctx.elapsed_ms(5 - slot, 5 - slot)   # the other slot: the batch before this one
+                slot = 5 - slot
+
+    replay(reps)
     ctx.event(0)
-    for _ in range(reps):
-        ctx.graph_launch(gid)
+    replay(reps)
     ctx.event(1)
     ms = ctx.elapsed_ms(0, 1) / (iters * reps)
     ctx.graph_destroy(gid)

@@ -5,6 +5,8 @@
 #include <cstdio>
 #include <cstring>
 
+#include <mutex>
+
 #include "gh_internal.h"
 
 int gh_fail(gh_ctx* ctx, int code, const std::string& msg) {
@@ -29,6 +31,8 @@ static void* g_scratch_ptr[kMaxDevices] = {};   // address of `scratch` on devic
 // once per device (every GPU holds its own copy at its own address).
 static hipError_t static_scratch(int device, void** out) {
   if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  static std::mutex mu;   // contexts may be opened from several host threads at once
+  std::lock_guard<std::mutex> lock(mu);
   if (!g_scratch_ptr[device]) {
     void* p = nullptr;
     hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));

@@ -598,7 +598,11 @@ int gh_launch_bn_train(gh_ctx* ctx, const gh_cmd& c) {
   const int G = bn_groups(n, S);
   // scratch: [C][G] sums, [C][G] squared deviations, [C] batch variance
   const int64_t need = (2 * C * G + C) * 4;
-  if (need > ctx->workspace_bytes) return gh_fail(ctx, GH_ESTATE, "batchnorm: reduction scratch does not fit the workspace");
+  if (need > ctx->workspace_bytes) {
+    // under gh_submit_noalloc: the refusal that names the need; there is no smaller plan to fall back to
+    if (const int rc = gh_ws_short(ctx, need)) return rc;
+    return gh_fail(ctx, GH_ESTATE, "batchnorm: reduction scratch does not fit the workspace");
+  }
   float* part_sum = (float*)ctx->workspace;
   float* part_sq = part_sum + C * G;
   float* batch_var = part_sq + C * G;
@@ -625,7 +629,10 @@ int gh_launch_bn_bwd(gh_ctx* ctx, const gh_cmd& c) {
   if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_bn_bwd_f64(ctx, c);
   const int64_t B = c.dim[0], C = c.dim[1], S = c.dim[2], n = B * S;
   const int G = bn_groups(n, S);
-  if (2 * C * G * 4 > ctx->workspace_bytes) return gh_fail(ctx, GH_ESTATE, "batchnorm: reduction scratch does not fit the workspace");
+  if (2 * C * G * 4 > ctx->workspace_bytes) {
+    if (const int rc = gh_ws_short(ctx, 2 * C * G * 4)) return rc;
+    return gh_fail(ctx, GH_ESTATE, "batchnorm: reduction scratch does not fit the workspace");
+  }
   float* part = (float*)ctx->workspace;
   const float* x = (const float*)(uintptr_t)c.ptr[0];
   const float* dy = (const float*)(uintptr_t)c.ptr[1];

@@ -177,10 +177,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
       // (The fences keep the reads of a set in front of the MFMAs they are meant to run under.)
       float a0 = arow[kb], a1;
       float b0v[9], b1v[9];
+      // The k that pad the last step (K..KW) carry dy = 0 and table position 0, so their B operand is
+      // real x data; an Inf there would put 0 * Inf = NaN into the sum where the reference has Inf or a
+      // number.  Those lanes' B registers are cleared instead, in the one step that has them.
+      const int kpad = g.KW > g.K ? g.KW - 4 : -1;
+      const bool lane_pad = g.KW - 4 + lk >= g.K;
+      auto clear_pad = [&](int ks, float (&bv)[9]) {
+        if (ks == kpad && lane_pad) {
+#pragma unroll
+          for (int t = 0; t < 9; t++) bv[t] = 0.f;
+        }
+      };
       {
         const float* const xb = xL + xlane + prow[kb];
 #pragma unroll
         for (int t = 0; t < 9; t++) b0v[t] = xb[(t / 3) * kRowPitch + t % 3];
+        clear_pad(kb, b0v);
       }
       int pn = prow[min(kb + 4, klast)];
       for (int k0 = kb; k0 < ke; k0 += 8) {
@@ -189,6 +201,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
           const float* const xb = xL + xlane + pn;
 #pragma unroll
           for (int t = 0; t < 9; t++) b1v[t] = xb[(t / 3) * kRowPitch + t % 3];
+          clear_pad(min(k0 + 4, klast), b1v);
           pn = prow[min(k0 + 8, klast)];
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -201,6 +214,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
           const float* const xb = xL + xlane + pn;
 #pragma unroll
           for (int t = 0; t < 9; t++) b0v[t] = xb[(t / 3) * kRowPitch + t % 3];
+          clear_pad(min(k0 + 8, klast), b0v);
           pn = prow[min(k0 + 12, klast)];
         }
         __builtin_amdgcn_sched_barrier(0);

@@ -2644,14 +2644,24 @@ static const char* force_tile() { return getenv("GORGONIA_HIP_SKINNY_TILE"); }
 // against 7 us for the 32x32 tile: every B load touches 64 different lines.)
 // Small-output products (dense layers of a small batch): returns -1 when the
 // shape belongs to the tiled kernel.
-static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
+// Whether the small-output kernels take a product, on a device of `cus` compute units: the one test
+// behind the launcher and the route query.
+static bool gemm_skinny_takes(const gh_cmd& c, int cus) {
   const int64_t batch = c.dim[6] <= 0 ? 1 : c.dim[6];
   const bool ta = c.flags & GH_FLAG_TRANS_A, tb = c.flags & GH_FLAG_TRANS_B;
-  if (batch != 1 || (ta && tb)) return -1;
+  if (batch != 1 || (ta && tb)) return false;
+  if (cdiv(c.dim[0], 32) * cdiv(c.dim[1], 32) > cus || c.dim[2] < 32) return false;
+  if (getenv("GORGONIA_HIP_GEMM_PLAN")) return false;  // a forced tile plan means the tiled kernel
+  // transposed views only have the 16-row kernel, which wants 16 rows and has no softmax for them
+  if ((ta || tb) && (c.dim[0] < 16 || (c.flags & GH_FLAG_GEMM_SOFTMAX))) return false;
+  return true;
+}
+
+static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
+  if (!gemm_skinny_takes(c, ctx->cu_count)) return -1;
+  const bool ta = c.flags & GH_FLAG_TRANS_A, tb = c.flags & GH_FLAG_TRANS_B;
   const int M = (int)c.dim[0], N = (int)c.dim[1], K = (int)c.dim[2];
   const int64_t tiles = cdiv(M, 32) * cdiv(N, 32);
-  if (tiles > ctx->cu_count || K < 32) return -1;
-  if (getenv("GORGONIA_HIP_GEMM_PLAN")) return -1;  // a forced tile plan means the tiled kernel
   const int lda = (int)c.dim[3], ldb = (int)c.dim[4], ldc = (int)c.dim[5];
   const int act = (c.flags & GH_FLAG_ACT_RELU) ? 1 : (c.flags & GH_FLAG_ACT_LEAKY) ? 2 : 0;
   constexpr int WV = 8;  // 512 threads leave each wavefront 256 registers for the grouped loads
@@ -2668,7 +2678,6 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
   // gradients of a dense layer) only have the 16-row kernel.
   const char* force = force_tile();
   const bool transposed = ta || tb;
-  if (transposed && (M < 16 || softmax)) return -1;
   const bool tiles16 = N <= 16 || (N > 32 && tiles * 2 <= ctx->cu_count);
   if (transposed || (M >= 16 && tiles16 && !(force && !strcmp(force, "32")))) {
     // 16x32 tiles read whole 128-byte lines of B; when even those leave half the
@@ -2890,13 +2899,10 @@ extern "C" int gh_gemm_route(const gh_cmd* c, int* splits) {
   if (!c || c->opcode != GH_OP_GEMM) return -1;
   if (gh_dtype_of(c->flags) == GH_F64) return GH_GEMM_ROUTE_F64;
   const int64_t batch = c->dim[6] <= 0 ? 1 : c->dim[6];
-  const bool ta = c->flags & GH_FLAG_TRANS_A, tb = c->flags & GH_FLAG_TRANS_B;
   gh_ctx probe;
   probe.workspace = &probe;   // never dereferenced: only "there is one" and its size are read
   probe.workspace_bytes = 64ll << 20;
-  if (batch == 1 && !(ta && tb) && cdiv(c->dim[0], 32) * cdiv(c->dim[1], 32) <= probe.cu_count && c->dim[2] >= 32 &&
-      !getenv("GORGONIA_HIP_GEMM_PLAN"))
-    return GH_GEMM_ROUTE_SMALL_OUTPUT;
+  if (gemm_skinny_takes(*c, probe.cu_count)) return GH_GEMM_ROUTE_SMALL_OUTPUT;
   const TilePlan p = plan_tiles(&probe, c->dim[0], c->dim[1], c->dim[2], batch, false);
   if (splits) *splits = p.splits;
   return p.tile == kTile128 ? GH_GEMM_ROUTE_TILE128 : p.tile == kTile128x64 ? GH_GEMM_ROUTE_TILE128X64 : GH_GEMM_ROUTE_TILE64;

@@ -26,7 +26,7 @@ class GhhOp(C.Structure):
                 ("ints", C.c_int64 * 16), ("f0", C.c_double), ("f1", C.c_double), ("fs", C.c_double * 10)]
 
 
-T_NOT_MANAGED, T_TRANSPOSED, T_NEEDS_ITER = 1, 2, 4
+T_NOT_MANAGED, T_TRANSPOSED, T_NEEDS_ITER, T_COL_MAJOR = 1, 2, 4, 8
 _P = C.c_void_p
 _TP = C.POINTER(GhhTensor)
 
@@ -141,13 +141,14 @@ class Tensor:
     """A dense tensor in the engine's arena (shape () = scalar)."""
 
     def __init__(self, mem, shape, dtype=np.float32, transposed=False, managed=True,
-                 needs_iterator=False):
+                 needs_iterator=False, col_major=False):
         self.mem = int(mem)
         self.shape = tuple(int(s) for s in shape)
         self.dtype = np.dtype(dtype)
         self.transposed = transposed
         self.managed = managed
         self.needs_iterator = needs_iterator
+        self.col_major = col_major   # DataOrder.IsColMajor: element (i, j) of an (r, c) matrix at j * r + i
 
     @property
     def size(self):
@@ -160,7 +161,8 @@ class Tensor:
     def T(self):
         """Transposed view of a matrix (tensor.T(): shape swapped, data order flagged)."""
         assert len(self.shape) == 2
-        return Tensor(self.mem, self.shape[::-1], self.dtype, not self.transposed, self.managed)
+        return Tensor(self.mem, self.shape[::-1], self.dtype, not self.transposed, self.managed,
+                      col_major=self.col_major)
 
     def desc(self):
         d = GhhTensor()
@@ -170,7 +172,7 @@ class Tensor:
         for i, s in enumerate(self.shape):
             d.shape[i] = s
         d.flags = ((0 if self.managed else T_NOT_MANAGED) | (T_TRANSPOSED if self.transposed else 0) |
-                   (T_NEEDS_ITER if self.needs_iterator else 0))
+                   (T_NEEDS_ITER if self.needs_iterator else 0) | (T_COL_MAJOR if self.col_major else 0))
         return d
 
 

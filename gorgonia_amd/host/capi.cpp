@@ -20,6 +20,7 @@ static Tensor to_tensor(const ghh_tensor* t) {
   for (int i = 0; i < t->ndim && i < 8; i++) r.shape.d.push_back(t->shape[i]);
   r.manually_managed = !(t->flags & GHH_T_NOT_MANAGED);
   r.transposed = t->flags & GHH_T_TRANSPOSED;
+  r.col_major = t->flags & GHH_T_COL_MAJOR;
   r.requires_iterator = t->flags & GHH_T_NEEDS_ITER;
   return r;
 }

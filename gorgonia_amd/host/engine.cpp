@@ -393,7 +393,10 @@ Status Engine::MatVecMul(Tensor& a, Tensor& b, Tensor& prealloc) {
   c.opcode = GH_OP_GEMV;
   c.ptr[0] = a.mem; c.ptr[1] = b.mem; c.ptr[2] = prealloc.mem;
   c.flags = GH_FLAG_DTYPE(a.dt == Dtype::Float64 ? GH_F64 : GH_F32);  // Dgemv / Sgemv, cuda/linalg.go:94-127
-  if (a.transposed) {  // stored (n x m) row-major: y = A_stored^T x
+  // The four cases of cuda/linalg.go:57-75.  A column-major (m, n) matrix is the row-major matrix
+  // (n, m) in memory, and so is a transposed view of a row-major one; column-major and transposed
+  // together is plain row-major again.
+  if (a.transposed != a.col_major) {  // stored (n x m) row-major: y = A_stored^T x
     c.flags |= GH_FLAG_TRANS_A;
     c.dim[0] = n; c.dim[1] = m; c.dim[2] = m;
   } else {
@@ -417,21 +420,44 @@ Status Engine::MatMul(Tensor& a, Tensor& b, Tensor& prealloc, int act, float alp
     return Status::Err(GH_EINVAL, fmt2(kShapeMismatch, Shape{k, n}.String(), b.shape.String()));
   if (prealloc.shape[0] != m || prealloc.shape[1] != n)
     return Status::Err(GH_EINVAL, fmt2(kShapeMismatch, Shape{m, n}.String(), prealloc.shape.String()));
-  // Row-major case table of cuda/linalg.go:161-202 without the operand swap:
-  // the kernel is row-major itself, so a transposed view just flips the flag
-  // and takes the stored width as its leading dimension.
+  if (a.col_major != b.col_major)   // cuda/linalg.go:118-122
+    return Status::Err(GH_EINVAL, std::string("a does not have the same data order as b. a is ") +
+                                      (a.col_major ? "ColMajor" : "RowMajor") + ". b is " +
+                                      (b.col_major ? "ColMajor" : "RowMajor"));
   gh_cmd c{};
   c.opcode = GH_OP_GEMM;
-  c.flags = (a.transposed ? GH_FLAG_TRANS_A : 0) | (b.transposed ? GH_FLAG_TRANS_B : 0) |
-            (act == 1 ? GH_FLAG_ACT_RELU : act == 2 ? GH_FLAG_ACT_LEAKY : 0) |
+  c.flags = (act == 1 ? GH_FLAG_ACT_RELU : act == 2 ? GH_FLAG_ACT_LEAKY : 0) |
             (softmax ? GH_FLAG_GEMM_SOFTMAX : 0) | (bias ? GH_FLAG_GEMM_BIAS : 0) |
             GH_FLAG_DTYPE(a.dt == Dtype::Float64 ? GH_F64 : GH_F32);  // Dgemm / Sgemm, cuda/linalg.go:204-227
   c.f[0] = alpha;
-  c.ptr[0] = a.mem; c.ptr[1] = b.mem; c.ptr[2] = prealloc.mem; c.ptr[3] = bias;
-  c.dim[0] = m; c.dim[1] = n; c.dim[2] = k;
-  c.dim[3] = a.transposed ? m : k;
-  c.dim[4] = b.transposed ? k : n;
-  c.dim[5] = prealloc.shape[1];
+  c.ptr[2] = prealloc.mem; c.ptr[3] = bias;
+  c.dim[2] = k;
+  c.dim[6] = 1;
+  if (!a.col_major) {
+    // Row-major case table of cuda/linalg.go:161-202 without the operand swap: the kernel is
+    // row-major itself, so a transposed view just flips the flag and takes the stored width as
+    // its leading dimension.
+    c.flags |= (a.transposed ? GH_FLAG_TRANS_A : 0) | (b.transposed ? GH_FLAG_TRANS_B : 0);
+    c.ptr[0] = a.mem; c.ptr[1] = b.mem;
+    c.dim[0] = m; c.dim[1] = n;
+    c.dim[3] = a.transposed ? m : k;
+    c.dim[4] = b.transposed ? k : n;
+    c.dim[5] = prealloc.shape[1];
+  } else {
+    // Column-major case table of cuda/linalg.go:142-160 (the result is column-major too, leading
+    // dimension its row count): in row-major terms the memory holds C^T = B^T A^T, and a
+    // column-major (r, c) operand is the row-major (c, r) matrix - the reference's operand swap the
+    // other way round.  B^T (n x k) is the left operand, A^T (k x m) the right one; an operand whose
+    // transposed flag is set is stored the other way and becomes a transposed view of that.
+    if (act || bias || softmax)
+      return Status::Err(GH_EINVAL, "MatMul: no fused bias, activation or softmax for column-major operands");
+    c.flags |= (b.transposed ? GH_FLAG_TRANS_A : 0) | (a.transposed ? GH_FLAG_TRANS_B : 0);
+    c.ptr[0] = b.mem; c.ptr[1] = a.mem;
+    c.dim[0] = n; c.dim[1] = m;
+    c.dim[3] = b.transposed ? n : k;   // ldb of the reference's table
+    c.dim[4] = a.transposed ? k : m;   // lda
+    c.dim[5] = prealloc.shape[0];      // ldc
+  }
   c.dim[6] = 1;
   Enqueue(c);
   return Status::OK();

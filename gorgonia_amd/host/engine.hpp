@@ -44,6 +44,7 @@ struct Tensor {
   Shape shape;
   bool manually_managed = true;
   bool transposed = false;
+  bool col_major = false;          // DataOrder.IsColMajor: element (i, j) of an untransposed (r, c) matrix at j * r + i
   bool requires_iterator = false;  // views the engine cannot walk (cuda/utils.go:83-89)
   int64_t DataSize() const { return shape.IsScalar() ? 1 : shape.TotalSize(); }
   int64_t MemSize() const { return DataSize() * dtype_size(dt); }
@@ -140,8 +141,9 @@ class Engine {
   GORGONIA_BINOP(Lte, GH_LTE) GORGONIA_BINOP(Gt, GH_GT) GORGONIA_BINOP(Gte, GH_GTE)
   GORGONIA_BINOP(ElEq, GH_EQ) GORGONIA_BINOP(ElNe, GH_NE)
 #undef GORGONIA_BINOP
-  // Mod: the reference engine declares it but ships no kernel; here it runs
-  // (cuda/arith.go:589-701, elembinop.cu:201-210): same error here.
+  // Mod: the reference engine declares the methods but ships no kernel, so its calls stop at
+  // "does not have the function" (cuda/arith.go:589-701, elembinop.cu:201-210); here the
+  // kernel exists and the call runs, with math.Mod's semantics.
   Status Mod(Tensor& a, Tensor& b, const FuncOpts& o, Tensor** ret = nullptr);
 
   // Unary kernels by the reference's op name ("tanh", "sigmoid", "inv" ...):

@@ -1118,6 +1118,13 @@ Status TapeMachine::RunAll() {
           resident_done_[(size_t)in.node] = 1;
           break;
         }
+        // a borrowed input has no host value of its own (Node::host is a marker): without the machine's
+        // pinned buffer - LetBorrowed after Init, on an input this machine does not stage - there is
+        // nothing to upload
+        if (n.host_borrowed)
+          return Status::Err(GH_ESTATE, "PC " + std::to_string(pc) + ": devTrans: input " + std::to_string(in.node) +
+                                            " was lent (LetBorrowed) but this machine holds no pinned buffer for it; "
+                                            "lend inputs before the machine is created");
         st = eng_.MemcpyHtoD(regs_[(size_t)in.reg].mem, n.host, in.size);
         if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": devTrans");
         resident_done_[(size_t)in.node] = 1;

@@ -33,6 +33,7 @@ typedef struct ghh_tensor {
 #define GHH_T_NOT_MANAGED  1u  /* host memory: !IsManuallyManaged (cuda/linalg.go:19-29) */
 #define GHH_T_TRANSPOSED   2u  /* DataOrder.IsTransposed (cuda/linalg.go:57,135) */
 #define GHH_T_NEEDS_ITER   4u  /* RequiresIterator (cuda/utils.go:83-89) */
+#define GHH_T_COL_MAJOR    8u  /* DataOrder.IsColMajor (cuda/linalg.go:57-75,118-160) */
 
 /* ---- bfc: cuda/bfc.go, cuda/bfc_test.go (no GPU needed) ------------------- */
 typedef struct ghh_bfc ghh_bfc;

@@ -213,4 +213,6 @@ def test_gemm_routes():
     assert route(1152, 128, 625, ta=True) == (T64, 1)                # a dense layer's weight gradient: K = batch
     assert route(1152, 2048, 625)[0] == T64 and route(1152, 2048, 625)[1] > 1
     assert route(64, 64, 64, dtype=_ffi.F64)[0] == F64
+    # a transposed view with fewer than 16 rows has no small-output kernel: the launcher takes the tiled one
+    assert route(8, 128, 64, ta=True)[0] == T64 and route(8, 128, 64)[0] == SMALL and route(16, 128, 64, ta=True)[0] == SMALL
     assert lib.gh_gemm_route(C.byref(D.cmd_relu(0x1000, 0x2000, 16)), None) == -1

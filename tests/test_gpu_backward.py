@@ -186,6 +186,28 @@ def test_small_image_filter_gradient_random_geometries(ctx):
         assert_bits_equal(dwi, owi, f"integer dw {cfg}")
 
 
+@pytest.mark.parametrize("cfg", [(3, 16, 5, 5, 32, 1), (5, 32, 7, 7, 64, 1), (2, 16, 6, 5, 16, 0)])
+def test_small_image_filter_gradient_keeps_infinities(ctx, cfg):
+    """An infinite input value makes the filter-gradient entries it reaches infinite and leaves every
+    other entry as it was (geometries whose pixel count per staged group is no multiple of four, so the
+    last MFMA step has padding k: those must not multiply a zero gradient by the infinity)."""
+    B, C, H, W, F, pad = cfg
+    oh, ow = H + 2 * pad - 2, W + 2 * pad - 2
+    x = synth.uniform(900, (B, C, H, W), -1, 1)
+    w = synth.he_normal(901, (F, C, 3, 3))
+    dy = np.abs(synth.normal(902, (B, F, oh, ow))) + 0.25     # positive: an infinite term stays +inf in the sum
+    _, clean = gpu_conv_bwd(ctx, x, w, dy, (pad, pad), (1, 1), (1, 1))
+    x[0, :, 0, 0] = np.inf
+    _, dw = gpu_conv_bwd(ctx, x, w, dy, (pad, pad), (1, 1), (1, 1))
+    with np.errstate(all="ignore"):
+        _, rw = O.conv2d_bwd(x, w, dy, (pad, pad), (1, 1), (1, 1))
+    assert not np.isnan(rw).any() and np.isinf(rw).any()
+    assert np.array_equal(np.isnan(dw), np.isnan(rw)), f"{int(np.isnan(dw).sum())} NaN in the device's dW"
+    assert np.array_equal(np.isposinf(dw), np.isposinf(rw)) and np.array_equal(np.isneginf(dw), np.isneginf(rw))
+    fin = np.isfinite(rw)
+    assert np.allclose(dw[fin], clean[fin], rtol=1e-4, atol=1e-5)
+
+
 BN_CASES = [(3, 2, 1), (6, 4, 1), (2, 2, 4), (4, 3, 25), (8, 16, 26 * 26), (2, 32, 104 * 104), (128, 10, 1)]
 
 

@@ -137,6 +137,66 @@ def test_matmul_case_table(eng, za, zb):
     assert rel_frobenius(eng.to_host(tc), ref) <= 1e-5
 
 
+def _col_major(eng, logical, transposed):
+    """A column-major tensor of logical shape `logical.shape` on the device.  Without the
+    transposed flag its memory is that of logical.T laid out row by row (column-major:
+    element (i, j) at j * rows + i); with it, the tensor is the transposed view of the
+    column-major matrix logical.T, whose memory is logical row by row."""
+    from gorgonia_amd.engine import Tensor
+    stored = logical.copy() if transposed else logical.T.copy()
+    t = eng.to_device(stored.reshape(-1))
+    return Tensor(t.mem, logical.shape, logical.dtype, transposed=transposed, col_major=True)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("za,zb", [(False, False), (True, False), (False, True), (True, True)])
+def test_matmul_column_major_case_table(eng, za, zb, dtype):
+    """cuda/linalg.go:142-160: column-major operands, each optionally flagged transposed; the
+    result is column-major with its row count as leading dimension."""
+    from gorgonia_amd.engine import Tensor
+    m, k, n = 70, 45, 52
+    A = synth.normal(5, (m, k)).astype(dtype)
+    B = synth.normal(6, (k, n)).astype(dtype)
+    ta, tb = _col_major(eng, A, za), _col_major(eng, B, zb)
+    tc = eng.new_tensor((m, n), dtype)
+    tc = Tensor(tc.mem, (m, n), dtype, col_major=True)
+    eng.MatMul(ta, tb, tc)
+    eng.DoWork()
+    got = eng.to_host(Tensor(tc.mem, (n, m), dtype)).T   # column-major (m, n) = row-major (n, m), transposed
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    assert rel_frobenius(got, ref) <= (1e-5 if dtype == np.float32 else 1e-13)
+    # on integer data every summing order is exact: the same bits as the row-major product of the same values
+    Ai = np.round(A * 4).astype(dtype)
+    Bi = np.round(B * 4).astype(dtype)
+    ta, tb = _col_major(eng, Ai, za), _col_major(eng, Bi, zb)
+    eng.MatMul(ta, tb, tc)
+    eng.DoWork()
+    got = eng.to_host(Tensor(tc.mem, (n, m), dtype)).T
+    assert np.array_equal(got, (Ai.astype(np.float64) @ Bi.astype(np.float64)).astype(dtype))
+
+
+def test_matmul_rejects_mixed_data_orders(eng):
+    """cuda/linalg.go:118-122."""
+    from gorgonia_amd.engine import Tensor, EngineError
+    a = eng.to_device(synth.normal(1, (8, 6)))
+    b = eng.to_device(synth.normal(2, (6, 5)))
+    bc = Tensor(b.mem, (6, 5), np.float32, col_major=True)
+    c = eng.new_tensor((8, 5))
+    with pytest.raises(EngineError, match="does not have the same data order"):
+        eng.MatMul(a, bc, c)
+
+
+@pytest.mark.parametrize("z", [False, True])
+def test_matvec_column_major(eng, z):
+    """cuda/linalg.go:57-75: the column-major cases of MatVecMul."""
+    A = synth.normal(7, (33, 47))
+    x = synth.normal(8, (47,))
+    ta, tx, ty = _col_major(eng, A, z), eng.to_device(x), eng.new_tensor((33,))
+    eng.MatVecMul(ta, tx, ty)
+    eng.DoWork()
+    assert rel_frobenius(eng.to_host(ty), A.astype(np.float64) @ x) <= 1e-5
+
+
 def test_matvec_and_outer(eng):
     A = synth.normal(7, (33, 47))
     x = synth.normal(8, (47,))

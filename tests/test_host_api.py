@@ -81,6 +81,12 @@ def test_linalg_checks(eng):
     eng.MatVecMul(a, T((4,)), T((3,)))
     eng.Outer(T((3,)), T((5,)), c)
     assert eng.pending() == 4
+    # data orders (cuda/linalg.go:118-122): both operands row-major or both column-major
+    with pytest.raises(EngineError, match="a does not have the same data order as b. a is RowMajor. b is ColMajor"):
+        eng.MatMul(a, T((4, 5), col_major=True), c)
+    eng.MatMul(T((3, 4), col_major=True), T((4, 5), col_major=True), T((3, 5), col_major=True))
+    eng.MatVecMul(T((3, 4), col_major=True), T((4,)), T((3,)))
+    assert eng.pending() == 6
 
 
 def test_has_func_and_unknown_unary(eng):
