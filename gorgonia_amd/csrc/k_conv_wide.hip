@@ -48,6 +48,7 @@ struct WideGeom {
   int npix;                       // TH * TW
   int pool, ph, pw, HTW;          // fused 2x2 / stride-2 max-pool: pooled extents of y, TW / 2
   unsigned mTXY, mTX, mPP, mPW, mTW, mHTW;   // magics: tiles_x*tiles_y, tiles_x, PP, PW, TW, HTW
+  int xcd_walk;                   // workgroups of one XCD walk one contiguous eighth of the tiles
 };
 
 constexpr int kWaves = 8;
@@ -174,9 +175,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
     for (int u = 0; u < XS; u++) buf[xpk[u] & 0xffff] = xv[u];
   };
 
+  // Which tiles this workgroup walks.  Workgroup ids are dealt round-robin over the 8 XCDs, each with
+  // its own L2: with tiles id, id + G, ... neighbouring patches - which share halo rows and cache
+  // lines, and whose results share cache lines - would land on different XCDs, every L2 would fetch
+  // nearly the whole input and no L2 would see a whole line of results.  Instead the workgroups of
+  // XCD j (ids = j mod 8; the launch has a multiple of 8 in x) share the j-th contiguous eighth
+  // of the tiles, whole images where the batch allows.
   const int ntiles = g.B * g.tiles_x * g.tiles_y;
-  int tile = blockIdx.x;                 // the launch has no more workgroups than tiles
-  load_patch(tile);
+  int tile, tile_end, tile_step;
+  if (g.xcd_walk) {
+    const int xcd = blockIdx.x & 7;
+    tile_end = (int)(((int64_t)ntiles * (xcd + 1)) >> 3);
+    tile = (int)(((int64_t)ntiles * xcd) >> 3) + (blockIdx.x >> 3);
+    tile_step = gridDim.x >> 3;
+  } else {
+    tile = blockIdx.x; tile_end = ntiles; tile_step = gridDim.x;
+  }
+  load_patch(tile);                      // the launch leaves no workgroup without a tile
   store_patch(P0);
   __syncthreads();
 
@@ -191,8 +206,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
   int cur = 0;
 
   for (;;) {
-    const int next = tile + gridDim.x;
-    const bool more = next < ntiles;
+    const int next = tile + tile_step;
+    const bool more = next < tile_end;
     if (more) load_patch(next);          // in flight during this tile's MFMAs
 
     f32x4 acc[TM][TN];
@@ -498,15 +513,29 @@ int launch_wide(gh_ctx* ctx, const gh_cmd& c, const WidePlan& p) {
   const int per_cu = (XS == 12 && TM * TN <= 4 && 2 * p.lds <= 158 * 1024) ? 2 : 1;
   int64_t G = std::max<int64_t>(1, (int64_t)ctx->cu_count * per_cu / ft);
   if (G > ntiles) G = ntiles;
-  const int64_t rounds = (ntiles + G - 1) / G;
-  G = (ntiles + rounds - 1) / rounds;
+  WideGeom geom = p.g;
+  static const bool no_xcd = getenv("GORGONIA_HIP_CONV_WIDE_NO_XCD") != nullptr;   // tuning switch: tiles id, id + G, ...
+  if (ntiles >= 64 && G >= 8 && !no_xcd) {
+    // one contiguous eighth of the tiles per XCD (see the kernel): Gx workgroups per XCD, lowered to
+    // the fewest that need no more rounds, and never more than the smallest eighth has tiles
+    const int64_t t8 = (ntiles + 7) / 8, t8min = ntiles / 8;
+    int64_t Gx = std::max<int64_t>(1, G / 8);
+    const int64_t rounds = (t8 + Gx - 1) / Gx;
+    Gx = std::min((t8 + rounds - 1) / rounds, t8min);
+    G = 8 * Gx;
+    geom.xcd_walk = 1;
+  } else {
+    const int64_t rounds = (ntiles + G - 1) / G;
+    G = (ntiles + rounds - 1) / rounds;
+    geom.xcd_walk = 0;
+  }
   const dim3 grid((unsigned)G, (unsigned)ft);
   if (getenv("GORGONIA_HIP_CONV_WIDE_DEBUG"))
     fprintf(stderr, "wide conv: TM=%d TN=%d XS=%d DB=%d patch %dx%d tiles %lld G=%lld ft=%d lds=%zu\n", TM, TN, XS, (int)DB,
             p.g.TH, p.g.TW, (long long)ntiles, (long long)G, ft, p.lds);
   hipLaunchKernelGGL((k_conv3x3_wide<TM, TN, XS, DB>), grid, dim3(kThreads), p.lds, ctx->stream,
                      (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
-                     (float*)(uintptr_t)c.ptr[2], p.g, conv_tail(c));
+                     (float*)(uintptr_t)c.ptr[2], geom, conv_tail(c));
   return gh_check_hip(ctx, hipGetLastError(), "conv3x3 wide launch");
 }
 
