@@ -89,8 +89,9 @@ __device__ __forceinline__ float tail_reg(float v, const float (&k)[4], float al
 
 // NQ channel quads; A regular pixel tiles per wavefront; TFB filter tiles per workgroup; WPT / QPT: padded
 // row and quad pitch as compile-time constants (0: taken from g, then three row pointers per tile advance
-// quad by quad).  Wavefront w: filter tile w % TFB, regular pixel tiles [(w / TFB) * A, +A).
-template <int NQ, int A, int TFB, bool POOL, int WPT, int QPT>
+// quad by quad); NLDT: image load instructions per wavefront as a constant (0: g.NLD, at most kMaxLoads).
+// Wavefront w: filter tile w % TFB, regular pixel tiles [(w / TFB) * A, +A).
+template <int NQ, int A, int TFB, bool POOL, int WPT, int QPT, int NLDT>
 __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restrict__ x, const float* __restrict__ w,
                                                            float* __restrict__ y, RowsGeom g, ConvTail tail) {
   static_assert((TFB * NQ) % kWaves == 0 && NQ % kWaves == 0, "quads divide over the wavefronts");
@@ -130,7 +131,8 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
     }
   }
   // image: lane = chunk * planes-per-load + plane in the group; chunk c covers floats [min(4c, HW-4), +4)
-  f32x4 xv[kMaxLoads];
+  constexpr int NLDMAX = NLDT ? NLDT : kMaxLoads;
+  f32x4 xv[NLDMAX];
   const int pl = lane & ((1 << g.ppl_shift) - 1), ch = lane >> g.ppl_shift;
   const bool lane_loads = ch < g.CH;
   const int e0 = min(4 * ch, g.HW - 4);
@@ -139,8 +141,8 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
     const int sstep = (kWaves << g.ppl_shift) * g.HW * 4;
     int soff = (wave << g.ppl_shift) * g.HW * 4;
 #pragma unroll
-    for (int i = 0; i < kMaxLoads; i++, soff += sstep)
-      if (i < g.NLD) xv[i] = bload4(rx, voff, soff);
+    for (int i = 0; i < NLDMAX; i++, soff += sstep)
+      if (NLDT || i < g.NLD) xv[i] = bload4(rx, voff, soff);
   }
   // a lane stores results of filter li of a filter tile: its BatchNorm constants, per filter tile
   float bn[TFB][4];
@@ -206,8 +208,8 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
     }
     const int istep = ((kWaves << g.ppl_shift) >> 2) * QPs;   // eight groups further: whole quads
 #pragma unroll
-    for (int i = 0; i < kMaxLoads; i++) {
-      if (i < g.NLD && ((wave + kWaves * i) << g.ppl_shift) < g.nplanes) {
+    for (int i = 0; i < NLDMAX; i++) {
+      if ((NLDT || i < g.NLD) && ((wave + kWaves * i) << g.ppl_shift) < g.nplanes) {
 #pragma unroll
         for (int e = 0; e < 4; e++) d[e][i * istep] = xv[i][e];
       }
@@ -477,18 +479,18 @@ bool rows_plan(const gh_cmd& c, bool pool, RowsPlan* out) {
   return gh_plan_memo(c, pool, out, [&](RowsPlan* p) { return rows_plan_compute(c, pool, p); });
 }
 
-template <int NQ, int A, int TFB, bool POOL, int WPT, int QPT>
+template <int NQ, int A, int TFB, bool POOL, int WPT, int QPT, int NLDT>
 int launch_rows(gh_ctx* ctx, const gh_cmd& c, const RowsPlan& p) {
   // more than 64 KB of dynamic LDS has to be allowed per kernel, once
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
   std::call_once(once, [] {
-    attr_rc = hipFuncSetAttribute((const void*)k_conv3x3_rows<NQ, A, TFB, POOL, WPT, QPT>,
+    attr_rc = hipFuncSetAttribute((const void*)k_conv3x3_rows<NQ, A, TFB, POOL, WPT, QPT, NLDT>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
   });
   if (attr_rc != hipSuccess) return gh_check_hip(ctx, attr_rc, "hipFuncSetAttribute(conv3x3 rows)");
   const dim3 grid((unsigned)((p.g.B + p.g.IPB - 1) / p.g.IPB), (unsigned)((p.g.F + 16 * TFB - 1) / (16 * TFB)));
-  hipLaunchKernelGGL((k_conv3x3_rows<NQ, A, TFB, POOL, WPT, QPT>), grid, dim3(kThreads), p.lds, ctx->stream,
+  hipLaunchKernelGGL((k_conv3x3_rows<NQ, A, TFB, POOL, WPT, QPT, NLDT>), grid, dim3(kThreads), p.lds, ctx->stream,
                      (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
                      (float*)(uintptr_t)c.ptr[2], p.g, conv_tail(c));
   return gh_check_hip(ctx, hipGetLastError(), "conv3x3 rows launch");
@@ -498,20 +500,20 @@ template <int NQ, int TFB, bool POOL>
 int launch_rows_a(gh_ctx* ctx, const gh_cmd& c, const RowsPlan& p) {
   // 16 x 16 and 9 x 9 padded planes (14 x 14 and 7 x 7 images with padding 1) have their pitches compiled in
   if constexpr (NQ == 8 && TFB == 2) {
-    if (p.g.Wp == 16 && p.g.QP == 1088 && p.A == 3) return launch_rows<NQ, 3, TFB, POOL, 16, 1088>(ctx, c, p);
+    if (p.g.Wp == 16 && p.g.QP == 1088 && p.A == 3 && p.g.NLD == 4) return launch_rows<NQ, 3, TFB, POOL, 16, 1088, 4>(ctx, c, p);
   }
   if constexpr (NQ == 16 && TFB == 1) {
-    if (p.g.Wp == 9 && p.g.QP == 336 && p.A == 1) return launch_rows<NQ, 1, TFB, POOL, 9, 336>(ctx, c, p);
+    if (p.g.Wp == 9 && p.g.QP == 336 && p.A == 1 && p.g.NLD == 8) return launch_rows<NQ, 1, TFB, POOL, 9, 336, 8>(ctx, c, p);
     if constexpr (!POOL) {
-      if (p.g.Wp == 16 && p.g.QP == 1088 && p.A == 1) return launch_rows<NQ, 1, TFB, POOL, 16, 1088>(ctx, c, p);
+      if (p.g.Wp == 16 && p.g.QP == 1088 && p.A == 1 && p.g.NLD == 8) return launch_rows<NQ, 1, TFB, POOL, 16, 1088, 8>(ctx, c, p);
     }
   }
   switch (p.A) {
-    case 0: return launch_rows<NQ, 0, TFB, POOL, 0, 0>(ctx, c, p);
-    case 1: return launch_rows<NQ, 1, TFB, POOL, 0, 0>(ctx, c, p);
-    case 2: return launch_rows<NQ, 2, TFB, POOL, 0, 0>(ctx, c, p);
-    case 3: return launch_rows<NQ, 3, TFB, POOL, 0, 0>(ctx, c, p);
-    default: return launch_rows<NQ, 4, TFB, POOL, 0, 0>(ctx, c, p);
+    case 0: return launch_rows<NQ, 0, TFB, POOL, 0, 0, 0>(ctx, c, p);
+    case 1: return launch_rows<NQ, 1, TFB, POOL, 0, 0, 0>(ctx, c, p);
+    case 2: return launch_rows<NQ, 2, TFB, POOL, 0, 0, 0>(ctx, c, p);
+    case 3: return launch_rows<NQ, 3, TFB, POOL, 0, 0, 0>(ctx, c, p);
+    default: return launch_rows<NQ, 4, TFB, POOL, 0, 0, 0>(ctx, c, p);
   }
 }
 
