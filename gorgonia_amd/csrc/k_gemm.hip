@@ -1233,9 +1233,19 @@ __global__ __launch_bounds__(256) void k_conv3x3_direct(const float* __restrict_
                                                         int F, int pad, int yh, int yw, int fper,
                                                         ConvTail tail) {
   constexpr int PS = WS + 2;
-  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (t >= (int64_t)B * yh * yw) return;
-  const int px = (int)(t % yw), py = (int)((t / yw) % yh), b = (int)(t / ((int64_t)yw * yh));
+  // gridDim.z > 1: one image per z, the x blocks walk that image's stored pixels (one 32-bit division
+  // per thread; the 64-bit divisions of the flat numbering were a quarter of a small layer's run).
+  // gridDim.z == 1: stored pixels numbered over the whole batch (more images than z can count).
+  int px, py, b;
+  if (gridDim.z > 1 || B == 1) {
+    const unsigned t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= (unsigned)(yh * yw)) return;
+    py = (int)(t / (unsigned)yw); px = (int)(t - (unsigned)py * (unsigned)yw); b = blockIdx.z;
+  } else {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= (int64_t)B * yh * yw) return;
+    px = (int)(t % yw); py = (int)((t / yw) % yh); b = (int)(t / ((int64_t)yw * yh));
+  }
   const int iy0 = py * WS - pad, ix0 = px * WS - pad;
   float patch[C][PS][PS];
 #pragma unroll
@@ -2934,13 +2944,18 @@ static int launch_conv_direct(gh_ctx* ctx, const gh_cmd& c) {
   const int yh = pool ? oh / 2 : oh, yw = pool ? ow / 2 : ow;
   const int64_t pix = (int64_t)B * yh * yw;
   if (pix == 0 || F == 0) return GH_OK;
-  const int64_t bx = cdiv(pix, 256);
+  // one image per grid z where z can count them and an image's stored pixels fill most of their
+  // workgroups' lanes; else the batch's stored pixels in one numbering
+  const bool per_image = B <= 65535 && (int64_t)yh * yw < (1ll << 31) &&
+                         cdiv((int64_t)yh * yw, 256) * 256 * 10 <= (int64_t)yh * yw * 14;
+  const int64_t bx = per_image ? cdiv((int64_t)yh * yw, 256) : cdiv(pix, 256);
+  const int64_t nblocks = per_image ? bx * B : bx;
   // enough filter groups to give every SIMD a few wavefronts, at least 4 filters each
-  int64_t groups = cdiv((int64_t)ctx->cu_count * 16, bx * 4);
+  int64_t groups = cdiv((int64_t)ctx->cu_count * 16, nblocks * 4);
   if (groups > F / 4) groups = F / 4;
   if (groups < 1) groups = 1;
   const int fper = (int)cdiv(F, groups);
-  const dim3 grid((unsigned)bx, (unsigned)cdiv(F, fper));
+  const dim3 grid((unsigned)bx, (unsigned)cdiv(F, fper), per_image ? (unsigned)B : 1u);
   const float* x = (const float*)(uintptr_t)c.ptr[0];
   const float* w = (const float*)(uintptr_t)c.ptr[1];
   float* y = (float*)(uintptr_t)c.ptr[2];
