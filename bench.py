@@ -523,6 +523,10 @@ def main():
     ap.add_argument("--short-timing", action="store_true",
                     help="time each kernel over one graph replay only (no sustained-clock loop): for runs under a "
                          "tracing profiler, which records every launch")
+    ap.add_argument("--sustain-ms", type=float, default=None,
+                    help="length of the warm-up and of the timed loop of each kernel measurement (default 40)")
+    ap.add_argument("--in-flight", type=int, default=None,
+                    help="graph replays queued between two host waits of a kernel measurement (default 32)")
     ap.add_argument("--only", default="", help="comma list of: convnet,elementwise,linalg,mlp,yolo,train")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -532,6 +536,11 @@ def main():
     EAGER_TIMING = a.eager_timing
     if a.short_timing:
         SUSTAIN_MS = 0.0
+    elif a.sustain_ms is not None:
+        SUSTAIN_MS = a.sustain_ms
+    global IN_FLIGHT
+    if a.in_flight:
+        IN_FLIGHT = max(1, a.in_flight)
 
     from gorgonia_amd.device import Context
     ctx = Context(0, 0)
