@@ -235,18 +235,32 @@ def bench_linalg(ctx, iters):
 
 
 # HBM bytes per launch of each conv layer's kernel as the step issues it (conv +
-# ReLU + 2x2 max-pool in one launch), from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs of this script (KiB per dispatch; FETCH_SIZE scaled by 2.0,
-# WRITE_SIZE by 1.0, the factors a 64 MiB device copy in the same runs gives).
+# ReLU + 2x2 max-pool in one launch): constants read off rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs of this script, not measured by this run (KiB per dispatch;
+# FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0, the factors a 64 MiB device copy
+# in the same runs gives).  TRAFFIC_SOURCE names the summary that holds the runs.
 MEASURED_TRAFFIC_BYTES = {
-    "conv0": (2 * 937.5 + 3232.0) * 1024,
-    "conv1": (2 * 1953.6 + 1568.0) * 1024,
-    "conv2": (2 * 2033.1 + 576.0) * 1024,
+    "conv0": (2 * 1614.4 + 3136.0) * 1024,
+    "conv1": (2 * 1977.1 + 1568.0) * 1024,
+    "conv2": (2 * 2028.6 + 576.0) * 1024,
 }
+TRAFFIC_SOURCE = ("constant from profiles/convnet_yolo_elementwise_hbm_traffic_pmc.txt: rocprofv3 --pmc FETCH_SIZE "
+                  "(x2.0) + WRITE_SIZE (x1.0), KiB per dispatch of this kernel in `bench.py --skip-cpu --skip-machines "
+                  "--eager-timing --steps 5 --warmup 3 --only convnet,elementwise,yolo`")
 # SQ_VALU_MFMA_BUSY_CYCLES / (128 * GRBM_GUI_ACTIVE) of the same kernels in a rocprofv3 --pmc run of this
 # script (eager launches, one at a time: launch and drain are inside GUI_ACTIVE, clocks are not sustained)
-MEASURED_MFMA_BUSY = {"conv0": 0.0, "conv1": 0.283, "conv2": 0.223}
-CONV_KERNEL_NAME = {"conv0": "k_conv3x3_direct<1,2>", "conv1": "k_conv3x3_small<8,1,13,1>", "conv2": "k_conv3x3_small<8,1,9,2>"}
+MEASURED_MFMA_BUSY = {"conv0": 0.0, "conv1": 0.317, "conv2": 0.243}
+MFMA_BUSY_SOURCE = ("constant from profiles/mfma_utilisation_pmc.txt: SQ_VALU_MFMA_BUSY_CYCLES / (128 x GRBM_GUI_ACTIVE) "
+                    "per dispatch in `bench.py --skip-cpu --skip-machines --eager-timing --steps 5 --warmup 3 --only "
+                    "convnet,linalg,yolo` (one eager launch at a time; launch and drain are inside GUI_ACTIVE)")
+CONV_KERNEL_NAME = {"conv0": "k_conv3x3_direct<1,2>", "conv1": "k_conv3x3_rows<8,3,2,true,16,1088,4>",
+                    "conv2": "k_conv3x3_rows<16,1,1,true,9,336,8>"}
+# gh_conv2d_route's answer -> the kernel family it names
+CONV_ROUTE_KERNEL = {0: "k_conv3x3_direct", 1: "k_conv3x3_small", 2: "k_conv3x3_patch", 3: "k_conv3x3_wide",
+                     4: "k_conv1x1", 5: "k_conv3x3_tiled", 6: "k_conv2d_gather", 7: "k_conv3x3_rows"}
+# where the launch time of the dominant kernel can be checked: a kernel trace of the convnet legs alone
+TRACE_SOURCE = ("profiles/convnet_step_kernel_trace.txt: rocprofv3 --kernel-trace --stats of `bench.py --skip-cpu "
+                "--skip-machines --only convnet --sustain-ms 15 --in-flight 2`, average duration of this kernel")
 
 CONVNET_LAYERS = [  # (name, B-relative shape) of configuration 4
     ("conv0", 1, 28, 32), ("conv1", 32, 14, 64), ("conv2", 64, 7, 128),
@@ -263,13 +277,15 @@ def bench_convnet_kernels(ctx, batch, iters):
         x = ctx.upload(synth.uniform01(1, (batch * cin * hw * hw,)))
         w = ctx.upload(synth.normal(2, (f * cin * 9,)))
         y = ctx.malloc(batch * f * hw * hw * 4)
-        pool = bool(ctx.lib.gh_conv2d_can_pool(D.cmd_conv2d(x, w, y, batch, cin, hw, hw, f, 3, 3, (1, 1))))
+        plain = D.cmd_conv2d(x, w, y, batch, cin, hw, hw, f, 3, 3, (1, 1))
+        pool = bool(ctx.lib.gh_conv2d_can_pool(plain))
+        route = int(ctx.lib.gh_conv2d_route(plain))
         ms = time_cmds(ctx, [D.cmd_conv2d(x, w, y, batch, cin, hw, hw, f, 3, 3, (1, 1), act="relu", pool2=pool)], iters)
         fl = 2.0 * batch * hw * hw * f * cin * 9
         out_hw = (hw // 2) if pool else hw
         nb = 4 * (batch * cin * hw * hw + f * cin * 9 + batch * f * out_hw * out_hw)
         out[name] = {"us": round(ms * 1e3, 2), "TFLOPs": round(fl / ms / 1e9, 2), "flop": fl,
-                     "GBps": round(nb / ms / 1e6, 1), "bytes": nb, "pool_fused": pool,
+                     "GBps": round(nb / ms / 1e6, 1), "bytes": nb, "pool_fused": pool, "route": CONV_ROUTE_KERNEL.get(route, str(route)),
                      "us_short_burst": round(time_cmds.last_burst_ms * 1e3, 2)}
         for q in (x, w, y):
             ctx.free(q)
@@ -352,7 +368,7 @@ def bench_convnet_machines(steps, warmup, count=2, batch=128):
     return count * steps * batch / dt, results
 
 
-def bench_yolo(steps, warmup, resident_input=True, borrow_output=True, borrow_input=False):
+def bench_yolo(steps, warmup, resident_input=True, borrow_output=True, borrow_input=False, graph_replay=None):
     """Config 5: Tiny-YOLO-v2-shaped forward, batch 8 x 3 x 416 x 416, on the tape
     machine with conv+BatchNorm+LeakyReLU(+MaxPool) folded, graph replay,
     weights and input resident.  borrow_output: the 8 x 425 x 13 x 13 result (2.3 MB) is read
@@ -362,7 +378,7 @@ def bench_yolo(steps, warmup, resident_input=True, borrow_output=True, borrow_in
     inp = configs.yolo_inputs(8, 416)
     g, outs = configs.build_yolo(inp, resident_input=resident_input, borrow_output=borrow_output,
                                  borrow_input=borrow_input)
-    m = G.NewTapeMachine(g, graph_replay=replay_mode(), fuse_activations=True)
+    m = G.NewTapeMachine(g, graph_replay=replay_mode() if graph_replay is None else graph_replay, fuse_activations=True)
     if borrow_input:
         m.input(g.x_node)[...] = inp["x"]
     for _ in range(max(warmup, WARM_RUNS)):
@@ -375,7 +391,8 @@ def bench_yolo(steps, warmup, resident_input=True, borrow_output=True, borrow_in
     eng.DoWork()
     dt = time.perf_counter() - t0
     result = (m.value(outs["out"]) if borrow_output else outs["out"]).copy()
-    VERDICTS["yolo" if resident_input else "yolo_input_h2d"] = m.segment_verdict()
+    if graph_replay is None:
+        VERDICTS["yolo" if resident_input else "yolo_input_h2d"] = m.segment_verdict()
     m.Close()
     return dt / steps * 1e3, result, inp
 
@@ -570,12 +587,16 @@ def main():
         ms_yolo_h2d, _, _ = bench_yolo(max(10, a.steps // 8), a.warmup, resident_input=False)
         ms_yolo_copy, yolo_out_copy, _ = bench_yolo(max(10, a.steps // 8), a.warmup, borrow_output=False)
         ms_yolo_h2d_b, yolo_out_b, _ = bench_yolo(max(10, a.steps // 8), a.warmup, resident_input=False, borrow_input=True)
+        # every command submitted one by one (no hipGraph): the host cost of the library's kernel plans shows here
+        ms_yolo_eager, yolo_out_eager, _ = bench_yolo(max(10, a.steps // 8), a.warmup, graph_replay=False)
         yolo = {"ms_per_step": round(ms_yolo, 4), "images_s": round(8 / ms_yolo * 1e3, 1),
                 "TFLOPs": round(31_080_857_600 / ms_yolo / 1e9, 2), "flop_per_step": 31_080_857_600,
                 "ms_per_step_with_input_h2d": round(ms_yolo_h2d, 4),
                 "ms_per_step_with_input_h2d_from_borrowed_pinned_buffer": round(ms_yolo_h2d_b, 4),
                 "borrowed_input_output_equals_resident": bool(np.array_equal(yolo_out, yolo_out_b)),
                 "output": "read in the machine's pinned buffer (ReadBorrowed), 2298400 bytes",
+                "ms_per_step_eager_no_graph": round(ms_yolo_eager, 4),
+                "eager_output_equals_replayed": bool(np.array_equal(yolo_out, yolo_out_eager)),
                 "ms_per_step_output_copied_to_caller": round(ms_yolo_copy, 4),
                 "copied_output_equals_borrowed": bool(np.array_equal(yolo_out, yolo_out_copy))}
         log(f"yolo-shaped: {ms_yolo:.4f} ms/step  {8 / ms_yolo * 1e3:.0f} images/s")
@@ -629,11 +650,16 @@ def main():
         name = max(conv_k, key=lambda k: conv_k[k]["us"])
         r = conv_k[name]
         kname = CONV_KERNEL_NAME[name]
+        if not kname.startswith(r["route"]):   # the library chose another kernel than the one the constants are for
+            kname = r["route"] + " (traffic and mfma_busy constants are not this kernel's)"
         tail = "ReLU and the 2x2 max-pool in the epilogue" if r["pool_fused"] else "ReLU in the epilogue"
         roofline = {"kernel": f"{kname}: {name} of the convnet step with {tail}", "bound": "mfma",
                     "achieved": r["TFLOPs"], "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(r["TFLOPs"] / MFMA_F32_PEAK_TFLOPS, 4),
-                    "traffic": int(MEASURED_TRAFFIC_BYTES[name]), "mfma_busy": MEASURED_MFMA_BUSY[name],
+                    "traffic": int(MEASURED_TRAFFIC_BYTES[name]), "traffic_source": TRAFFIC_SOURCE,
+                    "mfma_busy": MEASURED_MFMA_BUSY[name], "mfma_busy_source": MFMA_BUSY_SOURCE,
+                    "launch_us_source": "HIP events around back-to-back launches of this kernel on the library's "
+                                        "stream in this run; cross-check: " + TRACE_SOURCE,
                     "launch_us": r["us"], "launch_us_short_burst": r.get("us_short_burst"),
                     "algorithmic_flop": r["flop"]}
 

@@ -3220,6 +3220,7 @@ extern "C" int gh_gemm_can_softmax(const gh_cmd* c) {
 extern "C" int gh_conv2d_route(const gh_cmd* c) {
   if (!c || c->opcode != GH_OP_CONV2D || gh_dtype_of(c->flags) != GH_F32) return -1;
   if (conv_direct_takes(*c)) return GH_CONV_ROUTE_DIRECT;
+  if (gh_conv_rows_takes(*c)) return GH_CONV_ROUTE_ROWS;
   if (gh_conv_small_takes(*c)) return GH_CONV_ROUTE_SMALL;
   if (gh_conv_patch_takes(*c)) return GH_CONV_ROUTE_PATCH;
   if (gh_conv_wide_takes(*c)) return GH_CONV_ROUTE_WIDE;

@@ -59,6 +59,9 @@ CONV_CASES = [
     (16, 1, 28, 28, 32, 3, 3, (1, 1), (1, 1), (1, 1)),
     (16, 32, 14, 14, 64, 3, 3, (1, 1), (1, 1), (1, 1)),
     (16, 64, 7, 7, 128, 3, 3, (1, 1), (1, 1), (1, 1)),
+    # small images with 16 and 128 channels (the K-split small-image kernel)
+    (9, 16, 12, 12, 33, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (4, 128, 6, 6, 24, 3, 3, (0, 0), (1, 1), (1, 1)),
     # tiny-yolo-shaped layers (configuration 5) at reduced spatial size / batch
     (1, 3, 104, 104, 16, 3, 3, (1, 1), (1, 1), (1, 1)),
     (2, 16, 52, 52, 32, 3, 3, (1, 1), (1, 1), (1, 1)),
@@ -249,17 +252,23 @@ def test_conv_epilogue_special_values_bit_exact(ctx, cfg):
                                   O.maxpool2d(want, (2, 2), (0, 0), (2, 2)), f"conv+bn+leaky({alpha})+pool {cfg}")
 
 
-# shapes the small-image kernel takes (3x3, images up to 16x16, 16/32/64/128 channels): ragged filter
+# shapes the K-split small-image kernel takes (3x3, images up to 16x16, 16 or 128 channels): ragged filter
 # tiles, batches that do not fill the last workgroup, no padding, odd and even extents, H != W
-SMALL_IMAGE_CASES = [(7, 16, 7, 7, 10, 1), (5, 32, 14, 14, 50, 1), (9, 64, 7, 7, 33, 1), (3, 128, 5, 6, 20, 1),
-                     (6, 32, 16, 16, 16, 0), (2, 64, 9, 13, 17, 0), (1, 16, 4, 4, 5, 1), (11, 32, 6, 11, 64, 1),
-                     (130, 64, 7, 7, 8, 1)]
+SMALL_IMAGE_CASES = [(7, 16, 7, 7, 10, 1), (3, 128, 5, 6, 20, 1), (1, 16, 4, 4, 5, 1), (4, 128, 6, 6, 24, 0),
+                     (9, 16, 8, 15, 33, 1), (6, 16, 10, 9, 17, 0)]
+# and those of the kernel with the pixels on the MFMA rows (32 or 64 channels, 4 to 16 pixels wide): the
+# same kinds, plus the smallest and largest images it takes, odd output extents on either axis (the
+# pixels outside every pooling window), more filters than one round of workgroups, and a batch that
+# leaves the last workgroup's image slots partly empty
+ROWS_CASES = [(5, 32, 14, 14, 50, 1), (9, 64, 7, 7, 33, 1), (6, 32, 16, 16, 16, 0), (2, 64, 9, 13, 17, 0),
+              (11, 32, 6, 11, 64, 1), (130, 64, 7, 7, 8, 1), (3, 32, 4, 4, 20, 1), (2, 64, 16, 16, 40, 1),
+              (1, 32, 3, 5, 7, 1), (17, 64, 2, 16, 130, 1), (4, 32, 5, 4, 33, 0), (35, 64, 8, 5, 300, 1)]
 
 
-@pytest.mark.parametrize("cfg", SMALL_IMAGE_CASES)
+@pytest.mark.parametrize("cfg", SMALL_IMAGE_CASES + ROWS_CASES)
 def test_conv_small_images(ctx, cfg):
-    """The small-image convolution kernel against the oracle (<= 1e-5, exact on integers), and every
-    epilogue it can carry against the separate commands bit for bit."""
+    """The two small-image convolution kernels against the oracle (<= 1e-5, exact on integers), and every
+    epilogue they can carry against the separate commands bit for bit."""
     B, C, H, W, F, pad = cfg
     x = synth.uniform(31, (B, C, H, W), -1, 1)
     w = synth.he_normal(32, (F, C, 3, 3))
