@@ -42,7 +42,7 @@ HIP_FLAGS = [
     "-I", INCLUDE, "-I", CSRC,
 ]
 
-HIP_SOURCES = ["gh_api.hip", "gh_validate.cpp", "k_elem.hip", "k_gemm.hip", "k_conv_small.hip", "k_conv_rows.hip", "k_conv_patch.hip", "k_conv_wide.hip", "k_conv_pointwise.hip", "k_conv_wgrad_small.hip", "k_nn.hip", "k_nn64.hip", "k_bwd.hip", "k_bwd64.hip"]
+HIP_SOURCES = ["gh_api.hip", "gh_validate.cpp", "k_elem.hip", "k_gemm.hip", "k_conv_small.hip", "k_conv_rows.hip", "k_conv_rows1.hip", "k_conv_patch.hip", "k_conv_wide.hip", "k_conv_pointwise.hip", "k_conv_wgrad_small.hip", "k_nn.hip", "k_nn64.hip", "k_bwd.hip", "k_bwd64.hip"]
 
 HOST_FLAGS = [
     "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wextra",

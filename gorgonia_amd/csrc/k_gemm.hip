@@ -2981,6 +2981,8 @@ static int launch_conv_direct(gh_ctx* ctx, const gh_cmd& c) {
 
 int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
   if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_conv2d_f64(ctx, c);
+  const int rc0 = gh_try_launch_conv_rows1(ctx, c);
+  if (rc0 >= 0) return rc0;
   if (conv_direct_takes(c)) return launch_conv_direct(ctx, c);
   const int rcs = gh_try_launch_conv_small(ctx, c);
   if (rcs >= 0) return rcs;
@@ -3219,6 +3221,7 @@ extern "C" int gh_gemm_can_softmax(const gh_cmd* c) {
 // command; the one figure of the device they use, its compute units, is the MI355X's here.
 extern "C" int gh_conv2d_route(const gh_cmd* c) {
   if (!c || c->opcode != GH_OP_CONV2D || gh_dtype_of(c->flags) != GH_F32) return -1;
+  if (gh_conv_rows1_takes(*c)) return GH_CONV_ROUTE_ROWS1;
   if (conv_direct_takes(*c)) return GH_CONV_ROUTE_DIRECT;
   if (gh_conv_rows_takes(*c)) return GH_CONV_ROUTE_ROWS;
   if (gh_conv_small_takes(*c)) return GH_CONV_ROUTE_SMALL;
@@ -3243,6 +3246,7 @@ extern "C" int gh_conv2d_bwd_filter_route(const gh_cmd* c) {
 
 extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {
   if (!c || c->opcode != GH_OP_CONV2D || gh_dtype_of(c->flags) != GH_F32) return 0;
+  if (gh_conv_rows1_takes(*c)) return 1;   // even output extents are part of what it takes
   if (conv_direct_takes(*c)) {
     const int64_t oh = c->dim[2] + 2 * c->dim[7] - 2, ow = c->dim[3] + 2 * c->dim[7] - 2;
     return oh >= 2 && ow >= 2;

@@ -309,8 +309,10 @@ enum gh_conv_route {
   GH_CONV_ROUTE_POINTWISE = 4,  /* 1x1 with a small result                                */
   GH_CONV_ROUTE_TILED = 5,      /* 3x3 staged through LDS tiles (+ K slices)              */
   GH_CONV_ROUTE_GATHER = 6,     /* every other geometry                                   */
-  GH_CONV_ROUTE_ROWS = 7        /* 3x3, 32 or 64 channels, images up to 16 x 16: pixels on
+  GH_CONV_ROUTE_ROWS = 7,       /* 3x3, 32 or 64 channels, images up to 16 x 16: pixels on
                                    the MFMA rows, the 2x2 pool inside a lane's registers  */
+  GH_CONV_ROUTE_ROWS1 = 8       /* 3x3, one channel, images up to 64 x 64 with even output
+                                   extents: the same layout, K = 9 taps                   */
 };
 GH_API int gh_conv2d_route(const gh_cmd* conv);
 /* The same for a CONV2D_BWD_FILTER command (ConvolutionBackwardFilter,

@@ -99,7 +99,7 @@ def test_headers_are_plain_c99(tmp_path):
     assert p.returncode == 0, p.stderr
 
 
-ROUTE = {"direct": 0, "small": 1, "patch": 2, "wide": 3, "pointwise": 4, "tiled": 5, "gather": 6, "rows": 7}
+ROUTE = {"direct": 0, "small": 1, "patch": 2, "wide": 3, "pointwise": 4, "tiled": 5, "gather": 6, "rows": 7, "rows1": 8}
 
 
 def _route(B, C, H, W, F, k, pad, stride=(1, 1), dil=(1, 1), pool2=False):
@@ -116,7 +116,7 @@ def test_conv_routes_of_the_benchmark_layers():
     """gh_conv2d_route: every layer of the two convolutional configurations runs on the kernel the
     design names for it."""
     # convnet (configuration 4), batch 128
-    assert _route(128, 1, 28, 28, 32, (3, 3), (1, 1)) == ROUTE["direct"]
+    assert _route(128, 1, 28, 28, 32, (3, 3), (1, 1)) == ROUTE["rows1"]
     assert _route(128, 32, 14, 14, 64, (3, 3), (1, 1)) == ROUTE["rows"]
     assert _route(128, 64, 7, 7, 128, (3, 3), (1, 1)) == ROUTE["rows"]
     # tiny-yolo-shaped (configuration 5), batch 8
@@ -142,6 +142,8 @@ def test_conv_route_of_every_parity_case_list():
         assert _route(B, Cn, H, W, F, (3, 3), (pad, pad)) == ROUTE["small"], (B, Cn, H, W, F, pad)
     for (B, Cn, H, W, F, pad) in T.ROWS_CASES:
         assert _route(B, Cn, H, W, F, (3, 3), (pad, pad)) == ROUTE["rows"], (B, Cn, H, W, F, pad)
+    for (B, Cn, H, W, F, pad) in T.ROWS1_CASES:
+        assert _route(B, Cn, H, W, F, (3, 3), (pad, pad)) == ROUTE["rows1"], (B, Cn, H, W, F, pad)
     for (B, Cn, H, W, F, pad) in T.PATCH_CASES:
         assert _route(B, Cn, H, W, F, (3, 3), (pad, pad)) == ROUTE["patch"], (B, Cn, H, W, F, pad)
     for (B, Cn, H, W, F, pad) in T.WIDE_CASES:
@@ -151,7 +153,7 @@ def test_conv_route_of_every_parity_case_list():
     for (B, Cn, H, W, F) in T.POINTWISE_CASES:
         want = ROUTE["pointwise"] if (B, Cn, H, W, F) in taken else ROUTE["gather"]
         assert _route(B, Cn, H, W, F, (1, 1), (0, 0)) == want, (B, Cn, H, W, F)
-    # the general lists between them reach all eight kernels
+    # the general lists between them reach all nine kernels
     seen = set()
     for (B, Cn, H, W, F, kh, kw, pad, stride, dil) in T.CONV_CASES:
         seen.add(_route(B, Cn, H, W, F, (kh, kw), pad, stride, dil))

@@ -265,7 +265,13 @@ ROWS_CASES = [(5, 32, 14, 14, 50, 1), (9, 64, 7, 7, 33, 1), (6, 32, 16, 16, 16, 
               (1, 32, 3, 5, 7, 1), (17, 64, 2, 16, 130, 1), (4, 32, 5, 4, 33, 0), (35, 64, 8, 5, 300, 1)]
 
 
-@pytest.mark.parametrize("cfg", SMALL_IMAGE_CASES + ROWS_CASES)
+# single-channel images on the matrix cores (even output extents, 16 to 256 filters): the smallest and the
+# largest image, ragged filter tiles, a last pixel tile that is partly empty, no padding, H != W
+ROWS1_CASES = [(3, 1, 28, 28, 32, 1), (2, 1, 6, 6, 16, 0), (5, 1, 64, 64, 40, 1), (1, 1, 2, 2, 16, 1),
+               (4, 1, 10, 30, 256, 1), (7, 1, 8, 12, 17, 1), (2, 1, 6, 8, 20, 0), (130, 1, 4, 6, 33, 1)]
+
+
+@pytest.mark.parametrize("cfg", SMALL_IMAGE_CASES + ROWS_CASES + ROWS1_CASES)
 def test_conv_small_images(ctx, cfg):
     """The two small-image convolution kernels against the oracle (<= 1e-5, exact on integers), and every
     epilogue they can carry against the separate commands bit for bit."""
