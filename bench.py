@@ -240,24 +240,26 @@ def bench_linalg(ctx, iters):
 # FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0, the factors a 64 MiB device copy
 # in the same runs gives).  TRAFFIC_SOURCE names the summary that holds the runs.
 MEASURED_TRAFFIC_BYTES = {
-    "conv0": (2 * 1614.4 + 3136.0) * 1024,
-    "conv1": (2 * 1977.1 + 1568.0) * 1024,
+    "conv0": (2 * 1419.1 + 3584.0) * 1024,
+    "conv1": (2 * 1969.1 + 1568.0) * 1024,
     "conv2": (2 * 2028.6 + 576.0) * 1024,
+    "conv0+conv1": (2 * 627.7 + 1568.0) * 1024,
 }
 TRAFFIC_SOURCE = ("constant from profiles/convnet_yolo_elementwise_hbm_traffic_pmc.txt: rocprofv3 --pmc FETCH_SIZE "
                   "(x2.0) + WRITE_SIZE (x1.0), KiB per dispatch of this kernel in `bench.py --skip-cpu --skip-machines "
                   "--eager-timing --steps 5 --warmup 3 --only convnet,elementwise,yolo`")
 # SQ_VALU_MFMA_BUSY_CYCLES / (128 * GRBM_GUI_ACTIVE) of the same kernels in a rocprofv3 --pmc run of this
 # script (eager launches, one at a time: launch and drain are inside GUI_ACTIVE, clocks are not sustained)
-MEASURED_MFMA_BUSY = {"conv0": 0.0, "conv1": 0.317, "conv2": 0.243}
+MEASURED_MFMA_BUSY = {"conv0": 0.036, "conv1": 0.310, "conv2": 0.236, "conv0+conv1": 0.325}
 MFMA_BUSY_SOURCE = ("constant from profiles/mfma_utilisation_pmc.txt: SQ_VALU_MFMA_BUSY_CYCLES / (128 x GRBM_GUI_ACTIVE) "
                     "per dispatch in `bench.py --skip-cpu --skip-machines --eager-timing --steps 5 --warmup 3 --only "
                     "convnet,linalg,yolo` (one eager launch at a time; launch and drain are inside GUI_ACTIVE)")
-CONV_KERNEL_NAME = {"conv0": "k_conv3x3_direct<1,2>", "conv1": "k_conv3x3_rows<8,3,2,true,16,1088,4>",
-                    "conv2": "k_conv3x3_rows<16,1,1,true,9,336,8>"}
+CONV_KERNEL_NAME = {"conv0": "k_conv3x3_rows1<true>", "conv1": "k_conv3x3_rows<8,3,2,true,16,1088,4,false>",
+                    "conv2": "k_conv3x3_rows<16,1,1,true,9,336,8,false>",
+                    "conv0+conv1": "k_conv3x3_rows<8,3,2,true,16,1088,4,true>"}
 # gh_conv2d_route's answer -> the kernel family it names
 CONV_ROUTE_KERNEL = {0: "k_conv3x3_direct", 1: "k_conv3x3_small", 2: "k_conv3x3_patch", 3: "k_conv3x3_wide",
-                     4: "k_conv1x1", 5: "k_conv3x3_tiled", 6: "k_conv2d_gather", 7: "k_conv3x3_rows"}
+                     4: "k_conv1x1", 5: "k_conv3x3_tiled", 6: "k_conv2d_gather", 7: "k_conv3x3_rows", 8: "k_conv3x3_rows1"}
 # where the launch time of the dominant kernel can be checked: a kernel trace of the convnet legs alone
 TRACE_SOURCE = ("profiles/convnet_step_kernel_trace.txt: rocprofv3 --kernel-trace --stats of `bench.py --skip-cpu "
                 "--skip-machines --only convnet --sustain-ms 15 --in-flight 2`, average duration of this kernel")
@@ -270,7 +272,9 @@ CONVNET_LAYERS = [  # (name, B-relative shape) of configuration 4
 def bench_convnet_kernels(ctx, batch, iters):
     """Per-kernel time of the conv layers of the convnet step (for the roofline object):
     the commands the step itself issues - conv + ReLU + 2x2 max-pool in one launch where
-    the library offers it.  FLOPs are the convolution's own (2*B*oh*ow*F*C*9)."""
+    the library offers it, and layers 0 and 1 as one launch where it folds them
+    ("conv0+conv1"; "in_step" marks the entries a fused step runs).  FLOPs are the
+    convolutions' own (2*B*oh*ow*F*C*9)."""
     from gorgonia_amd import device as D, synth
     out = {}
     for name, cin, hw, f in CONVNET_LAYERS:
@@ -286,8 +290,27 @@ def bench_convnet_kernels(ctx, batch, iters):
         nb = 4 * (batch * cin * hw * hw + f * cin * 9 + batch * f * out_hw * out_hw)
         out[name] = {"us": round(ms * 1e3, 2), "TFLOPs": round(fl / ms / 1e9, 2), "flop": fl,
                      "GBps": round(nb / ms / 1e6, 1), "bytes": nb, "pool_fused": pool, "route": CONV_ROUTE_KERNEL.get(route, str(route)),
-                     "us_short_burst": round(time_cmds.last_burst_ms * 1e3, 2)}
+                     "us_short_burst": round(time_cmds.last_burst_ms * 1e3, 2), "in_step": True}
         for q in (x, w, y):
+            ctx.free(q)
+    # layers 0 and 1 in one launch: the first layer's result is made in LDS and never stored
+    (_, c0, hw0, f0), (_, c1, hw1, f1) = CONVNET_LAYERS[0], CONVNET_LAYERS[1]
+    probe = D.cmd_conv2d(1, 1, 1, batch, c1, hw1, hw1, f1, 3, 3, (1, 1))
+    if c0 == 1 and f0 == c1 and hw0 == 2 * hw1 and ctx.lib.gh_conv2d_can_pre(probe) and out["conv0"]["pool_fused"]:
+        x = ctx.upload(synth.uniform01(1, (batch * hw0 * hw0,)))
+        w0 = ctx.upload(synth.normal(2, (f0 * 9,)))
+        w1 = ctx.upload(synth.normal(3, (f1 * c1 * 9,)))
+        y = ctx.malloc(batch * f1 * hw1 * hw1 * 4)
+        pool = out["conv1"]["pool_fused"]
+        ms = time_cmds(ctx, [D.cmd_conv2d(x, w1, y, batch, c1, hw1, hw1, f1, 3, 3, (1, 1), act="relu", pool2=pool, pre=w0)], iters)
+        fl = out["conv0"]["flop"] + out["conv1"]["flop"]
+        out_hw = (hw1 // 2) if pool else hw1
+        nb = 4 * (batch * hw0 * hw0 + f0 * 9 + f1 * c1 * 9 + batch * f1 * out_hw * out_hw)
+        out["conv0+conv1"] = {"us": round(ms * 1e3, 2), "TFLOPs": round(fl / ms / 1e9, 2), "flop": fl,
+                              "GBps": round(nb / ms / 1e6, 1), "bytes": nb, "pool_fused": pool, "route": out["conv1"]["route"],
+                              "us_short_burst": round(time_cmds.last_burst_ms * 1e3, 2), "in_step": True}
+        out["conv0"]["in_step"] = out["conv1"]["in_step"] = False
+        for q in (x, w0, w1, y):
             ctx.free(q)
     return out
 
@@ -647,17 +670,20 @@ def main():
     # the dominant kernel of the step: the conv layer with the largest time
     roofline = None
     if conv_k:
-        name = max(conv_k, key=lambda k: conv_k[k]["us"])
+        name = max((k for k in conv_k if conv_k[k]["in_step"]), key=lambda k: conv_k[k]["us"])
         r = conv_k[name]
         kname = CONV_KERNEL_NAME[name]
         if not kname.startswith(r["route"]):   # the library chose another kernel than the one the constants are for
             kname = r["route"] + " (traffic and mfma_busy constants are not this kernel's)"
         tail = "ReLU and the 2x2 max-pool in the epilogue" if r["pool_fused"] else "ReLU in the epilogue"
+        if name == "conv0+conv1":
+            tail += "; conv0 + ReLU + pool computed in LDS in front of it, its result never stored"
         roofline = {"kernel": f"{kname}: {name} of the convnet step with {tail}", "bound": "mfma",
                     "achieved": r["TFLOPs"], "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(r["TFLOPs"] / MFMA_F32_PEAK_TFLOPS, 4),
-                    "traffic": int(MEASURED_TRAFFIC_BYTES[name]), "traffic_source": TRAFFIC_SOURCE,
-                    "mfma_busy": MEASURED_MFMA_BUSY[name], "mfma_busy_source": MFMA_BUSY_SOURCE,
+                    "traffic": int(MEASURED_TRAFFIC_BYTES[name]) if name in MEASURED_TRAFFIC_BYTES else None,
+                    "traffic_source": TRAFFIC_SOURCE,
+                    "mfma_busy": MEASURED_MFMA_BUSY.get(name), "mfma_busy_source": MFMA_BUSY_SOURCE,
                     "launch_us_source": "HIP events around back-to-back launches of this kernel on the library's "
                                         "stream in this run; cross-check: " + TRACE_SOURCE,
                     "launch_us": r["us"], "launch_us_short_burst": r.get("us_short_burst"),

@@ -115,6 +115,7 @@ bool gh_conv_small_can_pool(const gh_cmd& c);
 int gh_try_launch_conv_rows(gh_ctx* ctx, const gh_cmd& c);
 bool gh_conv_rows_takes(const gh_cmd& c);
 bool gh_conv_rows_can_pool(const gh_cmd& c);
+bool gh_conv_rows_can_pre(const gh_cmd& c);
 // single-channel 3x3 convolution on the matrix cores (k_conv_rows1.hip), same conventions
 int gh_try_launch_conv_rows1(gh_ctx* ctx, const gh_cmd& c);
 bool gh_conv_rows1_takes(const gh_cmd& c);

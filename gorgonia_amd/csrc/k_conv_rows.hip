@@ -30,6 +30,7 @@
 #include <mutex>
 
 #include "gh_conv_common.h"
+#include "gh_conv_rows1.h"
 #include "gh_internal.h"
 
 namespace {
@@ -65,6 +66,13 @@ struct RowsGeom {
   int nwin, wpart;    // windows per image; N entries of the window part
   int per, er;        // other pixels per image (not pooled), of which in the last row
   unsigned mW, mNWIN, mPW, mPER;
+  // GH_FLAG_CONV_PRE: the input is computed in LDS from single-channel images of 2H x 2W (3x3 convolution with
+  // C filters and padding 1, Rectify, 2x2 max-pool) instead of being loaded
+  int preRW, preRP, preZP;   // padded row pitch, floats per padded image, zero floats in front
+  int preOff, preFloats;     // LDS offset and size of the padded images, floats
+  int preTab;                // LDS offset of the window tables: [4 prePT] patch offsets, [4 prePT] plane offsets
+  int preHW, preNL, prePT;   // pixels of a single-channel image; loads per thread; 16-pixel tiles of its convolution
+  unsigned mHW, mPreHW, mPreW;
 };
 
 __device__ __forceinline__ f32x4 bload4(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
@@ -90,10 +98,12 @@ __device__ __forceinline__ float tail_reg(float v, const float (&k)[4], float al
 // NQ channel quads; A regular pixel tiles per wavefront; TFB filter tiles per workgroup; WPT / QPT: padded
 // row and quad pitch as compile-time constants (0: taken from g, then three row pointers per tile advance
 // quad by quad); NLDT: image load instructions per wavefront as a constant (0: g.NLD, at most kMaxLoads).
+// PRE: x holds single-channel images and w0 the C 3x3 filters that make this convolution's input from them.
 // Wavefront w: filter tile w % TFB, regular pixel tiles [(w / TFB) * A, +A).
-template <int NQ, int A, int TFB, bool POOL, int WPT, int QPT, int NLDT>
+template <int NQ, int A, int TFB, bool POOL, int WPT, int QPT, int NLDT, bool PRE>
 __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restrict__ x, const float* __restrict__ w,
-                                                           float* __restrict__ y, RowsGeom g, ConvTail tail) {
+                                                           float* __restrict__ y, RowsGeom g, ConvTail tail,
+                                                           const float* __restrict__ w0) {
   static_assert((TFB * NQ) % kWaves == 0 && NQ % kWaves == 0, "quads divide over the wavefronts");
   constexpr int NFP = TFB * NQ / kWaves;      // filter (tile, quad) pairs staged per wavefront
   constexpr int QW = NQ / kWaves;             // quads of a leftover unit per wavefront
@@ -115,8 +125,9 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
   // ---- global loads, all issued before anything waits.  Buffer loads: filter rows past F and planes of
   // images past B lie beyond the descriptors' ranges and read as zero.
   const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void*)w, 0, g.F * g.K * 4, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void*)(x + (int64_t)b0 * g.C * g.HW), 0,
-                                                                     nimg * g.C * g.HW * 4, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rx =
+      PRE ? __builtin_amdgcn_make_buffer_rsrc((void*)(x + (int64_t)b0 * g.preHW), 0, nimg * g.preHW * 4, 0x00020000)
+          : __builtin_amdgcn_make_buffer_rsrc((void*)(x + (int64_t)b0 * g.C * g.HW), 0, nimg * g.C * g.HW * 4, 0x00020000);
   float wf[NFP][9];
   {
     const int voff = (li * g.K + lk * 9) * 4;
@@ -131,12 +142,24 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
     }
   }
   // image: lane = chunk * planes-per-load + plane in the group; chunk c covers floats [min(4c, HW-4), +4)
-  constexpr int NLDMAX = NLDT ? NLDT : kMaxLoads;
+  constexpr int NLDMAX = PRE ? 1 : NLDT ? NLDT : kMaxLoads;
   f32x4 xv[NLDMAX];
   const int pl = lane & ((1 << g.ppl_shift) - 1), ch = lane >> g.ppl_shift;
   const bool lane_loads = ch < g.CH;
   const int e0 = min(4 * ch, g.HW - 4);
-  {
+  // PRE: the single-channel images instead, element tid + 512 i per thread, and the first convolution's
+  // filters as this lane's operand of channel tile ct (channels ct * 16 + li)
+  constexpr int CT = NQ / 4;
+  float rawv[PRE ? kMaxLoads : 1];
+  float w0b[PRE ? CT : 1][3];
+  if constexpr (PRE) {
+#pragma unroll
+    for (int i = 0; i < kMaxLoads; i++)
+      if (i < g.preNL) rawv[i] = bload1(rx, (tid + kThreads * i) * 4, 0);
+    const __amdgpu_buffer_rsrc_t rw0 = __builtin_amdgcn_make_buffer_rsrc((void*)w0, 0, g.C * 36, 0x00020000);
+#pragma unroll
+    for (int ct = 0; ct < CT; ct++) rows1::filter_operand(rw0, ct * 16 + li, lk, w0b[ct]);
+  } else {
     const int voff = lane_loads ? (pl * g.HW + e0) * 4 : 0x7ffffff0;
     const int sstep = (kWaves << g.ppl_shift) * g.HW * 4;
     int soff = (wave << g.ppl_shift) * g.HW * 4;
@@ -162,6 +185,22 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
     f32x4* p4 = reinterpret_cast<f32x4*>(Ps);
     const int n4 = g.IPB * NQ * QPs / 4;
     for (int i = tid; i < n4; i += kThreads) p4[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if constexpr (PRE) {
+      f32x4* r4 = reinterpret_cast<f32x4*>(lds + g.preOff);
+      for (int i = tid; i < g.preFloats / 4; i += kThreads) r4[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+      // per pooling window of the first convolution (= input pixel of this one): where its 4x4 patch starts in
+      // the padded single-channel image, and where its result goes in the planes; windows past the workgroup's
+      // images read the zeros at offset 0 and store nothing
+      int* const tabA = reinterpret_cast<int*>(lds + g.preTab);
+      int* const tabD = tabA + 4 * g.prePT;
+      for (int gw = tid; gw < 4 * g.prePT; gw += kThreads) {
+        const int im = mdiv(gw, g.mHW), wi = gw - im * g.HW;
+        const int py = mdiv(wi, g.mW), px = wi - py * g.W;
+        const bool ok = gw < g.IPB * g.HW;
+        tabA[gw] = ok ? g.preZP + im * g.preRP + 2 * py * g.preRW + 2 * px : 0;
+        tabD[gw] = ok ? im * NQ * QPs + (py + g.pad) * Wps + px + g.pad : -1;
+      }
+    }
   }
   for (int n = tid; n < 16 * g.PT; n += kThreads) {
     // window part: IPB * nwin windows in order, four positions each; then (not pooled) the other pixels
@@ -187,14 +226,27 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
   }
   __syncthreads();
   // ---- stage: filters (lane order is the MFMA operand order), image interiors
-  {
+  auto stage_filters = [&]() {
     float* d = Wl + wave * NFP * 9 * 64 + lane;
 #pragma unroll
     for (int i = 0; i < NFP; i++)
 #pragma unroll
       for (int t = 0; t < 9; t++) d[(i * 9 + t) * 64] = wf[i][t];
-  }
-  if (lane_loads) {
+  };
+  if constexpr (!PRE) stage_filters();
+  if constexpr (PRE) {
+    // the single-channel images into their zeroed padded frames
+    float* const Raw = lds + g.preOff;
+#pragma unroll
+    for (int i = 0; i < kMaxLoads; i++) {
+      const int e = tid + kThreads * i;
+      if (i < g.preNL && e < g.IPB * g.preHW) {
+        const int im = mdiv(e, g.mPreHW), k = e - im * g.preHW;
+        const int r = mdiv(k, g.mPreW), c = k - r * (2 * g.W);
+        Raw[g.preZP + im * g.preRP + (r + 1) * g.preRW + c + 1] = rawv[i];
+      }
+    }
+  } else if (lane_loads) {
     // plane p = ((wave + 8 i) << ppl_shift) + pl sits at (p >> 2) * QP + (p & 3) * PP
     const int pw0 = (wave << g.ppl_shift) + pl;
     const int r0 = mdiv(e0, g.mW), c0 = e0 - r0 * g.W;
@@ -216,6 +268,35 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
     }
   }
   __syncthreads();
+  if constexpr (PRE) {
+    // ---- the first convolution, Rectify and the 2x2 pool (gh_conv_rows1.h), straight into the planes: a wavefront
+    // takes 16-pixel tiles of the single-channel images in turn and walks the channel tiles with the pixel operand;
+    // a lane's four accumulator registers are the pooling window that becomes one input pixel of a channel
+    const float* const Raw = lds + g.preOff;
+    const rows1::LaneTaps L = rows1::lane_taps(lk, g.preRW);
+    int coff[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ct++) coff[ct] = ((ct * 16 + li) >> 2) * QPs + ((ct * 16 + li) & 3) * PP;
+    const int* const tabA = reinterpret_cast<const int*>(lds + g.preTab);
+    const int* const tabD = tabA + 4 * g.prePT;
+    const int posoff = ((li & 3) >> 1) * g.preRW + (li & 1);   // the lane's position in its window, operand side
+    for (int pt = wave; pt < g.prePT; pt += kWaves) {
+      float a[3];
+      rows1::pixel_operand(Raw, tabA[pt * 4 + (li >> 2)] + posoff, L, a);
+      const int od = tabD[pt * 4 + lk];
+#pragma unroll
+      for (int ct = 0; ct < CT; ct++) {
+        f32x4 v = rows1::tile(a, w0b[ct]);
+#pragma unroll
+        for (int r = 0; r < 4; r++) v[r] = act_apply(v[r], 1, 0.0f);
+        const float best = rows1::pool_window(v);
+        if (od >= 0) Ps[od + coff[ct]] = best;
+      }
+    }
+    // this convolution's filters have had the first one's time to arrive
+    stage_filters();
+    __syncthreads();
+  }
 
   const int ft = wave % TFB, pg = wave / TFB;
   const int lkoff = lk * PP;
@@ -479,28 +560,69 @@ bool rows_plan(const gh_cmd& c, bool pool, RowsPlan* out) {
   return gh_plan_memo(c, pool, out, [&](RowsPlan* p) { return rows_plan_compute(c, pool, p); });
 }
 
-template <int NQ, int A, int TFB, bool POOL, int WPT, int QPT, int NLDT>
+// The command of the single-channel convolution a GH_FLAG_CONV_PRE command stands for.
+gh_cmd pre_command(const gh_cmd& c) {
+  gh_cmd q{};
+  q.opcode = GH_OP_CONV2D;
+  q.flags = GH_FLAG_DTYPE(GH_F32) | GH_FLAG_ACT_RELU | GH_FLAG_CONV_POOL2;
+  q.dim[0] = c.dim[0]; q.dim[1] = 1; q.dim[2] = 2 * c.dim[2]; q.dim[3] = 2 * c.dim[3]; q.dim[4] = c.dim[1];
+  q.dim[5] = 3; q.dim[6] = 3; q.dim[7] = 1; q.dim[8] = 1;
+  q.dim[9] = 1; q.dim[10] = 1; q.dim[11] = 1; q.dim[12] = 1;
+  return q;
+}
+
+// Extends a plan by the padded single-channel images of GH_FLAG_CONV_PRE.  False when the fold is not offered:
+// 32 channels only, the single-channel convolution must be one k_conv3x3_rows1 takes (so that it sums as it
+// would on its own), a workgroup's images at most 8 loads per thread, everything within LDS.
+bool rows_pre_plan(const gh_cmd& c, RowsPlan* p) {
+  if (p->NQ != 8 || !gh_conv_rows1_takes(pre_command(c))) return false;
+  RowsGeom& g = p->g;
+  g.preHW = 4 * g.HW;
+  if ((int64_t)g.IPB * g.preHW > (int64_t)kMaxLoads * kThreads) return false;
+  g.preNL = (g.IPB * g.preHW + kThreads - 1) / kThreads;
+  g.preRW = 2 * g.W + 2;
+  g.preRP = (2 * g.H + 2) * g.preRW;
+  g.preZP = (3 * g.preRW + 8 + 3) & ~3;   // a window past the images reads at its position's offset from 0
+  g.preFloats = (g.preZP + g.IPB * g.preRP + 3) & ~3;
+  g.preOff = (int)((p->lds / 4 + 3) & ~(size_t)3);
+  g.prePT = (g.IPB * g.preHW + 15) / 16;
+  g.preTab = g.preOff + g.preFloats;
+  g.mHW = magic_of((unsigned)g.HW); g.mPreHW = magic_of((unsigned)g.preHW); g.mPreW = magic_of((unsigned)(2 * g.W));
+  p->lds = ((size_t)g.preTab + 8 * (size_t)g.prePT) * 4;
+  return p->lds <= kLdsBudget;
+}
+
+template <int NQ, int A, int TFB, bool POOL, int WPT, int QPT, int NLDT, bool PRE = false>
 int launch_rows(gh_ctx* ctx, const gh_cmd& c, const RowsPlan& p) {
   // more than 64 KB of dynamic LDS has to be allowed per kernel, once
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
   std::call_once(once, [] {
-    attr_rc = hipFuncSetAttribute((const void*)k_conv3x3_rows<NQ, A, TFB, POOL, WPT, QPT, NLDT>,
+    attr_rc = hipFuncSetAttribute((const void*)k_conv3x3_rows<NQ, A, TFB, POOL, WPT, QPT, NLDT, PRE>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
   });
   if (attr_rc != hipSuccess) return gh_check_hip(ctx, attr_rc, "hipFuncSetAttribute(conv3x3 rows)");
   const dim3 grid((unsigned)((p.g.B + p.g.IPB - 1) / p.g.IPB), (unsigned)((p.g.F + 16 * TFB - 1) / (16 * TFB)));
-  hipLaunchKernelGGL((k_conv3x3_rows<NQ, A, TFB, POOL, WPT, QPT, NLDT>), grid, dim3(kThreads), p.lds, ctx->stream,
+  hipLaunchKernelGGL((k_conv3x3_rows<NQ, A, TFB, POOL, WPT, QPT, NLDT, PRE>), grid, dim3(kThreads), p.lds, ctx->stream,
                      (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
-                     (float*)(uintptr_t)c.ptr[2], p.g, conv_tail(c));
+                     (float*)(uintptr_t)c.ptr[2], p.g, conv_tail(c), (const float*)(uintptr_t)c.ptr[7]);
   return gh_check_hip(ctx, hipGetLastError(), "conv3x3 rows launch");
 }
 
-template <int NQ, int TFB, bool POOL>
+template <int NQ, int TFB, bool POOL, bool PRE = false>
 int launch_rows_a(gh_ctx* ctx, const gh_cmd& c, const RowsPlan& p) {
   // 16 x 16 and 9 x 9 padded planes (14 x 14 and 7 x 7 images with padding 1) have their pitches compiled in
   if constexpr (NQ == 8 && TFB == 2) {
-    if (p.g.Wp == 16 && p.g.QP == 1088 && p.A == 3 && p.g.NLD == 4) return launch_rows<NQ, 3, TFB, POOL, 16, 1088, 4>(ctx, c, p);
+    if (p.g.Wp == 16 && p.g.QP == 1088 && p.A == 3 && p.g.NLD == 4) return launch_rows<NQ, 3, TFB, POOL, 16, 1088, 4, PRE>(ctx, c, p);
+  }
+  if constexpr (PRE) {
+    switch (p.A) {
+      case 0: return launch_rows<NQ, 0, TFB, POOL, 0, 0, 0, true>(ctx, c, p);
+      case 1: return launch_rows<NQ, 1, TFB, POOL, 0, 0, 0, true>(ctx, c, p);
+      case 2: return launch_rows<NQ, 2, TFB, POOL, 0, 0, 0, true>(ctx, c, p);
+      case 3: return launch_rows<NQ, 3, TFB, POOL, 0, 0, 0, true>(ctx, c, p);
+      default: return launch_rows<NQ, 4, TFB, POOL, 0, 0, 0, true>(ctx, c, p);
+    }
   }
   if constexpr (NQ == 16 && TFB == 1) {
     if (p.g.Wp == 9 && p.g.QP == 336 && p.A == 1 && p.g.NLD == 8) return launch_rows<NQ, 1, TFB, POOL, 9, 336, 8>(ctx, c, p);
@@ -515,6 +637,11 @@ int launch_rows_a(gh_ctx* ctx, const gh_cmd& c, const RowsPlan& p) {
     case 3: return launch_rows<NQ, 3, TFB, POOL, 0, 0, 0>(ctx, c, p);
     default: return launch_rows<NQ, 4, TFB, POOL, 0, 0, 0>(ctx, c, p);
   }
+}
+
+int launch_rows_pre(gh_ctx* ctx, const gh_cmd& c, const RowsPlan& p, bool pool) {
+  if (p.TFB == 1) return pool ? launch_rows_a<8, 1, true, true>(ctx, c, p) : launch_rows_a<8, 1, false, true>(ctx, c, p);
+  return pool ? launch_rows_a<8, 2, true, true>(ctx, c, p) : launch_rows_a<8, 2, false, true>(ctx, c, p);
 }
 
 template <int NQ>
@@ -537,6 +664,17 @@ bool gh_conv_rows_can_pool(const gh_cmd& c) {
   return rows_plan(c, false, &p) && rows_plan(c, true, &p);
 }
 
+// 1 when it takes it with its input computed from single-channel images (GH_FLAG_CONV_PRE), pooled or not.
+bool gh_conv_rows_can_pre(const gh_cmd& c) {
+  RowsPlan p;
+  if (!rows_plan(c, false, &p) || !rows_pre_plan(c, &p)) return false;
+  if (gh_conv_rows_can_pool(c)) {
+    RowsPlan q;
+    if (!rows_plan(c, true, &q) || !rows_pre_plan(c, &q)) return false;
+  }
+  return true;
+}
+
 // Returns -1 when the shape is not one this kernel takes.
 int gh_try_launch_conv_rows(gh_ctx* ctx, const gh_cmd& c) {
   RowsPlan p;
@@ -545,5 +683,10 @@ int gh_try_launch_conv_rows(gh_ctx* ctx, const gh_cmd& c) {
   if (!rows_plan(c, false, &p)) return -1;
   if (pool && !rows_plan(c, true, &p))
     return gh_fail(ctx, GH_EINVAL, "conv2d: no fused pooling for this shape (see gh_conv2d_can_pool)");
+  if (c.flags & GH_FLAG_CONV_PRE) {
+    if (!rows_pre_plan(c, &p) || !c.ptr[7])
+      return gh_fail(ctx, GH_EINVAL, "conv2d: the single-channel convolution cannot be folded in front of this one (see gh_conv2d_can_pre)");
+    return launch_rows_pre(ctx, c, p, pool);
+  }
   return p.NQ == 8 ? launch_rows_q<8>(ctx, c, p, pool) : launch_rows_q<16>(ctx, c, p, pool);
 }

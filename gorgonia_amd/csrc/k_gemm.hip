@@ -2981,6 +2981,11 @@ static int launch_conv_direct(gh_ctx* ctx, const gh_cmd& c) {
 
 int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
   if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_conv2d_f64(ctx, c);
+  if (c.flags & GH_FLAG_CONV_PRE) {
+    const int rcp = gh_conv2d_can_pre(&c) ? gh_try_launch_conv_rows(ctx, c) : -1;
+    if (rcp >= 0) return rcp;
+    return gh_fail(ctx, GH_EINVAL, "conv2d: no folded first layer for this shape (see gh_conv2d_can_pre)");
+  }
   const int rc0 = gh_try_launch_conv_rows1(ctx, c);
   if (rc0 >= 0) return rc0;
   if (conv_direct_takes(c)) return launch_conv_direct(ctx, c);
@@ -3242,6 +3247,12 @@ extern "C" int gh_conv2d_bwd_filter_route(const gh_cmd* c) {
   if (conv_direct_shape(*c) && c->dim[4] <= 65535) return GH_WGRAD_ROUTE_DIRECT;
   if (gh_conv_wgrad_small_takes(*c)) return GH_WGRAD_ROUTE_SMALL;
   return GH_WGRAD_ROUTE_GEMM;
+}
+
+extern "C" int gh_conv2d_can_pre(const gh_cmd* c) {
+  if (!c || c->opcode != GH_OP_CONV2D || gh_dtype_of(c->flags) != GH_F32) return 0;
+  if (getenv("GORGONIA_HIP_CONV_NO_PRE")) return 0;   // tuning switch: the first layer stays a kernel of its own
+  return gh_conv_rows_takes(*c) && gh_conv_rows_can_pre(*c) ? 1 : 0;
 }
 
 extern "C" int gh_conv2d_can_pool(const gh_cmd* c) {

@@ -289,7 +289,7 @@ static std::string op_name(const OpSpec& op) {
     case OpKind::Outer: return "outer";
     case OpKind::BatchedMatMul: return "batchedmatmul";
     case OpKind::Conv2d:
-      return std::string("conv2d") + (op.fuse_bn ? "+batchnorm(eval)" : "") +
+      return std::string(op.fuse_pre ? "conv2d+rectify+maxpool2d+conv2d" : "conv2d") + (op.fuse_bn ? "+batchnorm(eval)" : "") +
              (op.fuse_act_relu ? "+rectify" : op.fuse_act_leaky ? "+leakyrelu" : "") +
              (op.fuse_pool2 ? "+maxpool2d" : "");
     case OpKind::MaxPool2D: return op.relu_input ? "rectify+maxpool2d" : "maxpool2d";
@@ -364,18 +364,19 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       const Tensor& x = *in[0];
       const Tensor& w = *in[1];
       if (x.dt == Dtype::Other || w.dt != x.dt) return bad("Conv2d: Unsupported Dtype");
-      if (x.dt == Dtype::Float64 && (op.fuse_bn || op.fuse_act_relu || op.fuse_act_leaky || op.fuse_pool2))
+      if (x.dt == Dtype::Float64 && (op.fuse_bn || op.fuse_act_relu || op.fuse_act_leaky || op.fuse_pool2 || op.fuse_pre))
         return bad("Conv2d: no epilogue operators for float64");
+      const size_t nin = in.size() - (op.fuse_pre ? 1 : 0);   // a folded first layer's filters come last
       gh_cmd c{};
       c.opcode = GH_OP_CONV2D;
       c.flags = (op.fuse_act_relu ? GH_FLAG_ACT_RELU : op.fuse_act_leaky ? GH_FLAG_ACT_LEAKY : 0) | dtype_flag(x.dt);
       c.f[0] = (float)op.f0;
       c.ptr[0] = x.mem; c.ptr[1] = w.mem; c.ptr[2] = prealloc.mem;
       if (op.fuse_bn) {
-        if (in.size() != 4 && in.size() != 6) return bad("Conv2d: fused BatchNorm needs mean, var[, scale, bias]");
+        if (nin != 4 && nin != 6) return bad("Conv2d: fused BatchNorm needs mean, var[, scale, bias]");
         c.flags |= GH_FLAG_CONV_BN;
         c.ptr[3] = in[2]->mem; c.ptr[4] = in[3]->mem;
-        if (in.size() == 6) {
+        if (nin == 6) {
           c.flags |= GH_FLAG_HAS_GAMMA | GH_FLAG_HAS_BETA;
           c.ptr[5] = in[4]->mem; c.ptr[6] = in[5]->mem;
         }
@@ -383,6 +384,13 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       }
       if (op.fuse_pool2) c.flags |= GH_FLAG_CONV_POOL2;
       for (int i = 0; i < 4; i++) c.dim[i] = x.shape[i];
+      if (op.fuse_pre) {
+        // x holds the single-channel images; the command's B,C,H,W describe the input that is never stored
+        if (nin < 2 || x.shape[1] != 1 || (x.shape[2] & 1) || (x.shape[3] & 1)) return bad("Conv2d: folded first layer needs B x 1 x 2H x 2W images");
+        c.flags |= GH_FLAG_CONV_PRE;
+        c.ptr[7] = in.back()->mem;
+        c.dim[1] = w.shape[1]; c.dim[2] = x.shape[2] / 2; c.dim[3] = x.shape[3] / 2;
+      }
       c.dim[4] = w.shape[0];
       for (int i = 0; i < 8; i++) c.dim[5 + i] = op.ints[(size_t)i];
       e.Enqueue(c);
@@ -726,6 +734,46 @@ int Graph::FuseActivations() {
     fused++;
   }
   fused += fuse_pooled_rectify();
+  fused += fuse_first_layer();
+  return fused;
+}
+
+// conv(conv+rectify+pool(x0, w0), w1, ...) where the inner node is a single-channel 3x3 / pad 1 / stride 1
+// convolution with Rectify and the 2x2 pool already in its epilogue, read by nothing but the outer convolution,
+// and the library folds the pair (gh_conv2d_can_pre): the outer node takes x0 as input 0 and w0 as its last
+// input; the tensor between the two layers is never stored.
+int Graph::fuse_first_layer() {
+  int fused = 0;
+  std::vector<int> uses(nodes_.size(), 0);
+  for (auto& n : nodes_)
+    if (!n.fused_away) for (int i : n.inputs) uses[(size_t)i]++;
+  for (auto& n : nodes_) {
+    if (n.is_input || n.fused_away || n.op.kind != OpKind::Conv2d || n.op.fuse_pre || n.inputs.size() < 2) continue;
+    if (n.dt != Dtype::Float32) continue;
+    Node& p = nodes_[(size_t)n.inputs[0]];
+    if (p.is_input || p.fused_away || p.read_into || uses[(size_t)p.id] != 1 || p.op.kind != OpKind::Conv2d) continue;
+    const OpSpec& q = p.op;
+    if (!q.fuse_act_relu || !q.fuse_pool2 || q.fuse_bn || q.fuse_act_leaky || q.fuse_pre || p.inputs.size() != 2) continue;
+    static const int64_t first[8] = {3, 3, 1, 1, 1, 1, 1, 1};   // kernel, pad, stride, dilation
+    bool plain = q.ints.size() >= 8;
+    for (size_t i = 0; plain && i < 8; i++) plain = q.ints[i] == first[i];
+    if (!plain) continue;
+    const Shape& x0 = nodes_[(size_t)p.inputs[0]].shape;
+    const Shape& ws = nodes_[(size_t)n.inputs[1]].shape;
+    if (x0.Dims() != 4 || x0[1] != 1 || (x0[2] & 1) || (x0[3] & 1) || p.shape.Dims() != 4 || ws.Dims() != 4) continue;
+    if (p.shape[2] != x0[2] / 2 || p.shape[3] != x0[3] / 2 || ws[1] != p.shape[1]) continue;
+    gh_cmd c{};
+    c.opcode = GH_OP_CONV2D;
+    for (int i = 0; i < 4; i++) c.dim[i] = p.shape[i];
+    c.dim[4] = ws[0];
+    for (int i = 0; i < 8; i++) c.dim[5 + i] = n.op.ints[(size_t)i];
+    if (!gh_conv2d_can_pre(&c)) continue;
+    n.op.fuse_pre = true;
+    n.inputs[0] = p.inputs[0];
+    n.inputs.push_back(p.inputs[1]);
+    p.fused_away = true;
+    fused++;
+  }
   return fused;
 }
 

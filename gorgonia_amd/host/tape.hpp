@@ -79,6 +79,10 @@ struct OpSpec {
   bool fuse_pool2 = false;
   bool fuse_bias = false;     // MatMul only: the BroadcastAdd of a row vector that follows (last input)
   bool fuse_softmax = false;  // MatMul only: the SoftMax that follows, where gh_gemm_can_softmax allows
+  // Conv2d only: the operators in FRONT of it ride along (GH_FLAG_CONV_PRE).  Input 0 is then a batch of
+  // single-channel images and the last input the filters of Conv2d 3x3 pad 1 -> Rectify -> MaxPool2D 2x2/2
+  // whose result this convolution reads without it ever being stored.
+  bool fuse_pre = false;
   // MaxPool2D / MaxPool2DDiff: input 0 is the value before a Rectify and is read through it; the
   // diff also applies the Rectify's own gradient (it stands for RectifyDiff(z, MaxPool2DDiff(Rectify(z), g)))
   bool relu_input = false;
@@ -129,6 +133,7 @@ class Graph {
   // Returns the number of operators folded away.
   int FuseActivations();
   int fuse_pooled_rectify();   // part of FuseActivations: the Rectify between a pool and both gradients
+  int fuse_first_layer();      // part of FuseActivations: a single-channel first layer folded into the next convolution
   const std::vector<Node>& Nodes() const { return nodes_; }
   std::vector<Node>& Nodes() { return nodes_; }
 

@@ -133,6 +133,7 @@ enum gh_unaryfn {
 #define GH_FLAG_BN_EVAL      (1u << 26)   /* BN_BWD: eval-mode gradient dy/sqrt(var+eps)       */
 #define GH_FLAG_CONV_POOL2   (1u << 25)   /* CONV2D: 2x2 stride-2 unpadded MaxPool2D on the result */
 #define GH_FLAG_GEMM_SOFTMAX (1u << 27)   /* GEMM: row SoftMax on the result (after the activation) */
+#define GH_FLAG_CONV_PRE     (1u << 29)   /* CONV2D: the input is made on the fly from single-channel images, see below */
 #define GH_FLAG_GEMM_BIAS    (1u << 28)   /* GEMM (untransposed): ptr[3] = N floats added to every row of the product (before the activation) */
 
 /*
@@ -169,6 +170,11 @@ enum gh_unaryfn {
  *             with HAS_BETA ptr[6]=beta, f[1]=eps; BN_INFER's arithmetic per filter),
  *             then ACT_RELU / ACT_LEAKY, then CONV_POOL2 (y then has the pooled
  *             shape B,F,oh/2,ow/2; only where gh_conv2d_can_pool says so)
+ *             CONV_PRE (float32, only where gh_conv2d_can_pre says so): the operators in front
+ *             of the convolution ride along too.  ptr[0] then holds single-channel images
+ *             (B,1,2H,2W) and ptr[7] C filters (C,1,3,3); the convolution's input (B,C,H,W) is
+ *             MaxPool2D 2x2/2 (Rectify (Conv2d 3x3 pad 1 (ptr[0], ptr[7]))), computed where it is
+ *             needed and never stored; y holds the bits the three commands would give
  * MAXPOOL2D   ptr[0]=x ptr[1]=y            dim[0..3]=B,C,H,W dim[4..5]=kh,kw
  *             dim[6..9]=padN,padS,padW,padE dim[10..11]=strideH,strideW
  *             GH_FLAG_ACT_RELU (float32): x is read through Rectify, y = pool(x*(x>=0));
@@ -296,6 +302,11 @@ GH_API int gh_validate(const gh_cmd* cmds, int n, char* msg, int msg_len);
  * reference has no fused form: this folds maxpool.CUDADo
  * (ops/nn/maxpool_cuda.go:94-111) into convolution.CUDADo (convolution_cuda.go:95-121). */
 GH_API int gh_conv2d_can_pool(const gh_cmd* conv);
+/* 1 when gh_submit accepts GH_FLAG_CONV_PRE on this float32 CONV2D command (dims as for the
+ * unfolded command: B,C,H,W describe the input that is never stored).  Host only.  The reference
+ * runs the first layer of its convolutional example as three operators with two stored tensors
+ * between them (examples/convnet/main.go:86-112); folded, a step has one kernel and one tensor less. */
+GH_API int gh_conv2d_can_pre(const gh_cmd* conv);
 /* Which of the library's convolution kernels gh_submit runs this float32 CONV2D command on, a
  * function of its shape, its flags and (for the filter operand's alignment) its pointers: one of
  * GH_CONV_ROUTE_*, or -1 for a command that is no float32 CONV2D.  Host only.  The reference

@@ -304,6 +304,76 @@ def test_conv_small_images(ctx, cfg):
                           O.maxpool2d(leaky, (2, 2), (0, 0), (2, 2)), f"small conv+bn+leaky+pool {cfg}")
 
 
+# (B, H, W, F, pad) of the second convolution of a folded first layer: its input has 32 channels and is
+# Conv2d 3x3 pad 1 -> Rectify -> MaxPool2D 2x2 of single-channel images of 2H x 2W.  The convnet's own
+# layer, ragged filter counts, several images per workgroup, no padding, the smallest and the largest
+# images, H != W, a batch that leaves the last workgroup partly empty
+PRE_CASES = [(5, 14, 14, 64, 1), (3, 7, 7, 33, 1), (9, 4, 4, 16, 1), (2, 16, 16, 40, 1), (6, 6, 11, 50, 0),
+             (130, 5, 8, 20, 1), (1, 14, 14, 64, 1), (4, 9, 13, 130, 0)]
+
+
+@pytest.mark.parametrize("cfg", PRE_CASES)
+def test_conv_folded_first_layer_bit_exact(ctx, cfg):
+    """GH_FLAG_CONV_PRE: one command stores the bits of the three it stands for (single-channel
+    convolution + Rectify + pool, then the convolution), with and without followers of its own, and
+    special values in the image and the first filters travel as they do through the separate commands."""
+    B, H, W, F, pad = cfg
+    C = 32
+    x0 = synth.uniform(71, (B, 1, 2 * H, 2 * W), -1, 1)
+    w0 = synth.he_normal(72, (C, 1, 3, 3))
+    w1 = synth.he_normal(73, (F, C, 3, 3))
+    probe = D.cmd_conv2d(1, 1, 1, B, C, H, W, F, 3, 3, (pad, pad))
+    assert ctx.lib.gh_conv2d_can_pre(probe) == 1, cfg
+    mean, var = synth.normal(74, (F,), 0.0, 0.1), synth.uniform(75, (F,), 0.5, 1.5)
+    gamma, beta = synth.uniform(76, (F,), 0.5, 1.5), synth.normal(77, (F,), 0.0, 0.1)
+
+    def folded(x0, w0, w1=w1, **kw):
+        oh, ow = H + 2 * pad - 2, W + 2 * pad - 2
+        yh, yw = (oh // 2, ow // 2) if kw.get("pool2") else (oh, ow)
+        held = [ctx.upload(x0), ctx.upload(w1), ctx.upload(w0)]
+        dbn = None
+        if kw.get("bn") is not None:
+            dbn = tuple(ctx.upload(a) for a in kw["bn"])
+            held += list(dbn)
+        dy = ctx.malloc(B * F * yh * yw * 4)
+        held.append(dy)
+        ctx.run(D.cmd_fill(dy, B * F * yh * yw, np.nan))
+        ctx.run(D.cmd_conv2d(held[0], held[1], dy, B, C, H, W, F, 3, 3, (pad, pad), act=kw.get("act"),
+                             alpha=kw.get("alpha", 0.0), bn=dbn, pool2=bool(kw.get("pool2")), pre=held[2]))
+        y = ctx.d2h(dy, (B, F, yh, yw))
+        for p in held:
+            ctx.free(p)
+        return y
+
+    mid = gpu_conv_tail(ctx, x0, w0, (1, 1), act="relu", pool2=True)
+    assert mid.shape == (B, C, H, W)
+    ref = O.maxpool2d(O.relu(O.conv2d(x0, w0, (1, 1), (1, 1), (1, 1))).reshape(B, C, 2 * H, 2 * W), (2, 2), (0, 0), (2, 2))
+    assert rel_frobenius(mid, ref) <= TOL
+    assert_bits_equal(folded(x0, w0), gpu_conv(ctx, mid, w1, (pad, pad), (1, 1), (1, 1)), f"folded {cfg}")
+    if H + 2 * pad - 2 >= 2 and W + 2 * pad - 2 >= 2:
+        assert_bits_equal(folded(x0, w0, act="relu", pool2=True),
+                          gpu_conv_tail(ctx, mid, w1, (pad, pad), act="relu", pool2=True), f"folded+relu+pool {cfg}")
+        assert_bits_equal(folded(x0, w0, bn=(mean, var, gamma, beta), act="leaky", alpha=0.1, pool2=True),
+                          gpu_conv_tail(ctx, mid, w1, (pad, pad), bn=(mean, var, gamma, beta), act="leaky", alpha=0.1,
+                                        pool2=True), f"folded+bn+leaky+pool {cfg}")
+    # integers: exact against the oracle's chain
+    rng = np.random.default_rng(5)
+    xi = rng.integers(-3, 4, x0.shape).astype(np.float32)
+    w0i = rng.integers(-2, 3, w0.shape).astype(np.float32)
+    w1i = rng.integers(-2, 3, w1.shape).astype(np.float32)
+    midi = O.maxpool2d(O.relu(O.conv2d(xi, w0i, (1, 1), (1, 1), (1, 1))).reshape(B, C, 2 * H, 2 * W), (2, 2), (0, 0), (2, 2))
+    assert_bits_equal(folded(xi, w0i, w1i), O.conv2d(midi.reshape(B, C, H, W), w1i, (pad, pad), (1, 1), (1, 1)), f"folded integers {cfg}")
+    # special values in the image and in the first filters
+    xs = x0.copy()
+    flat = xs.reshape(-1)
+    flat[::37] = np.inf; flat[5::41] = -np.inf; flat[11::43] = np.nan; flat[3::29] = -0.0; flat[7::31] = 0.0
+    ws = w0.copy()
+    ws.reshape(-1)[4::19] = -0.0
+    ws.reshape(-1)[9::23] = np.inf
+    mids = gpu_conv_tail(ctx, xs, ws, (1, 1), act="relu", pool2=True)
+    assert_bits_equal(folded(xs, ws), gpu_conv(ctx, mids, w1, (pad, pad), (1, 1), (1, 1)), f"folded special values {cfg}")
+
+
 # shapes the patch kernel takes (3x3, 64 channels or more, K split over eight wavefronts): partial
 # patches on both axes, ragged filter tiles, no padding, pooled extents odd and even
 PATCH_CASES = [(2, 64, 20, 17, 40, 1), (2, 64, 28, 28, 32, 1), (1, 64, 24, 14, 20, 0), (1, 96, 26, 26, 48, 1), (3, 128, 13, 13, 70, 1), (1, 64, 31, 18, 16, 0),

@@ -63,7 +63,7 @@ def test_convnet_forward_fused_and_unfused(ctx):
     m2, _, r2 = run_once(configs.build_convnet, inp, fuse_activations=True)
     assert rel_frobenius(r1["out"], want) <= 1e-5
     assert_bits_equal(r1["out"], r2["out"], "fused activations change nothing")
-    assert m2.fused == 8  # 4 activations, the three pools and the softmax
+    assert m2.fused == 9  # 4 activations, the three pools, the softmax, the first layer into the second
     m1.Close(); m2.Close()
 
 

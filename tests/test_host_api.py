@@ -181,11 +181,22 @@ def test_tape_program_convnet_fusion():
     inp = configs.convnet_inputs(2)
     g, _ = configs.build_convnet(inp)
     m = G.NewTapeMachine(g, compile_only=True, fuse_activations=True)
-    assert m.fused == 8  # 4 activations, the three pools and the softmax
+    assert m.fused == 9  # 4 activations, the three pools, the softmax, and the first layer into the second
     prog = m.program()
-    assert prog.count("conv2d+rectify") == 3 and prog.count(" rectify") == 0
+    assert prog.count("conv2d+rectify+maxpool2d+conv2d+rectify+maxpool2d") == 1   # layers 0 and 1: one command
+    assert prog.count("execOp") == 4 and prog.count(" rectify") == 0
     assert prog.count("maxpool2d") == 3 and prog.count("softmax") == 1
     m.Close()
+    # a first layer whose result something else reads as well stays a command of its own
+    g3 = G.NewGraph()
+    x = G.NewTensor(g3, inp["x"], True)
+    h = G.MaxPool2D(G.Rectify(G.Conv2d(x, G.NewTensor(g3, inp["w0"], True), (3, 3), (1, 1), (1, 1), (1, 1))), (2, 2), (0, 0), (2, 2))
+    y = G.Conv2d(h, G.NewTensor(g3, inp["w1"], True), (3, 3), (1, 1), (1, 1), (1, 1))
+    G.Read(y)
+    G.Read(h)
+    m3 = G.NewTapeMachine(g3, compile_only=True, fuse_activations=True)
+    assert m3.program().count("conv2d+rectify+maxpool2d+conv2d") == 0 and m3.program().count("execOp") == 2
+    m3.Close()
     g2, _ = configs.build_convnet(inp)
     m2 = G.NewTapeMachine(g2, compile_only=True)
     assert m2.program().count(" rectify") == 4
