@@ -7,9 +7,9 @@
 // a few hundred at most, the whole filter tile and every channel of the padded patch fit
 // in LDS at once, so there is one staging phase, one barrier, and then nothing but
 // operand fetches and MFMAs; the results leave from the accumulators, no partial sums
-// cross wavefronts.  Same GEMM view as the other convolution kernels (M = filters, N =
-// output pixels, K in the reference's (c, kr, kc) order, op_nn.go:418-437), results
-// written straight into NCHW.
+// cross wavefronts.  The output pixels are the MFMA's rows and the filters its columns
+// (K in the reference's (c, kr, kc) order, op_nn.go:418-437): a lane holds four consecutive
+// N entries of one filter, and results are written straight into NCHW.
 //
 //   * One output is one accumulator chain over K, channel quad by channel quad, tap by
 //     tap, whatever the patch shape and whether or not the pooling below is fused: the
@@ -17,9 +17,11 @@
 //   * A channel count that is not a multiple of four is padded with zero planes and zero
 //     filter columns in LDS (a first layer's 3 channels or 1).
 //   * With GH_FLAG_CONV_POOL2 the patch has even extents and the N axis enumerates (pooled
-//     pixel, position in the 2x2 window), so a window is four adjacent lanes of one
-//     accumulator register: the maximum is taken across them in scan order with strict >
-//     (the pooling kernel's rule, op_nn.go:860-907) and one lane stores it.
+//     pixel, position in the 2x2 window), so a window is the four accumulator registers of
+//     one lane: the maximum is a scan over them in order with strict > (the pooling kernel's
+//     rule, op_nn.go:860-907), no lane waits for another, and every lane stores a result.
+//     Without it a lane's four entries are four pixels of a row wherever the patch is a
+//     multiple of four wide, and leave as one 128-bit store where the result allows.
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
@@ -53,12 +55,6 @@ struct WideGeom {
 
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
-
-// A 2x2 window's four positions sit in the four lanes of a quad, in scan order.
-template <int A, int B, int C, int D>
-__device__ __forceinline__ float quad_perm(float v) {   // lane i of each quad reads lane (A,B,C,D)[i] of it
-  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), A | (B << 2) | (C << 4) | (D << 6), 0xf, 0xf, true));
-}
 
 // XS: patch cells each thread stages per tile (4 NQ PP <= XS * kThreads); DB: two patch buffers.
 // The 12-slot kernels are held to 128 registers so that two workgroups share a compute unit
@@ -259,7 +255,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
         for (int a = 0; a < TM; a++)
 #pragma unroll
           for (int t = 0; t < TN; t++)
-            acc[a][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[tap % 3][a], bf[tap % 3][t], acc[a][t], 0, 0, 0);
+            acc[a][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf[tap % 3][t], af[tap % 3][a], acc[a][t], 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < TM * TN; i++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
@@ -269,8 +265,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
       }
     }
 
-    // ---- epilogue from the accumulators: register v of acc[a][t] is filter m0 + 16 a + 4 lk + v
-    // at N entry n0 + 16 t + li
+    // ---- epilogue from the accumulators.  The pixels are the MFMA's rows and the filters its columns:
+    // register v of acc[a][t] is N entry n0 + 16 t + 4 lk + v of filter m0 + 16 a + li.  With the pool fused
+    // the N order is window-major, so those four entries are one 2x2 window and the pool is a scan over
+    // the lane's own registers; a lane needs the BatchNorm constants of one filter per filter tile.
     {
       // The lane's coordinates pass through an empty asm here, so that what the epilogue derives
       // from them is computed per tile and does not sit in registers through the MFMA loop.
@@ -280,92 +278,89 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
       const int trem = tile - bimg * (g.tiles_x * g.tiles_y);
       const int tyi = mdiv(trem, g.mTX), txi = trem - tyi * g.tiles_x;
       const int oy0 = tyi * g.TH, ox0 = txi * g.TW;
-      // where each N tile's value goes (element offset inside a filter's plane), -1: nowhere
-      int yoff[TN];
       const int plane = g.pool ? g.ph * g.pw : g.oh * g.ow;
-#pragma unroll
-      for (int t = 0; t < TN; t++) {
-        const int n = n0 + 16 * t + eli;
-        if (g.pool) {
-          const int q = n >> 2;
-          const int py = mdiv(q, g.mHTW), px = q - py * g.HTW;
-          const int oy = (oy0 >> 1) + py, ox = (ox0 >> 1) + px;
-          yoff[t] = ((n & 3) == 0 && n < g.npix && oy < g.ph && ox < g.pw) ? oy * g.pw + ox : -1;
-        } else {
-          const int ty = mdiv(n, g.mTW), tx = n - ty * g.TW;
-          const int oy = oy0 + ty, ox = ox0 + tx;
-          yoff[t] = (n < g.npix && oy < g.oh && ox < g.ow) ? oy * g.ow + ox : -1;
-        }
-      }
       // one 64-bit base per tile, 32-bit byte offsets per lane (a filter tile's planes span < 2 GB)
       char* const ytile = reinterpret_cast<char*>(y + ((int64_t)bimg * g.F + m0) * plane);
       const unsigned pbytes = 4u * (unsigned)plane;
-      const bool all4 = (g.F & 3) == 0;   // then a lane's four filters exist or not together
       const float alpha = tail.alpha;
+      const int nb = n0 + 4 * elk;   // the lane's first N entry of N tile 0
       // What the epilogue consists of is uniform over the launch: the value loops are compiled
       // once per combination and the combination is chosen once per tile, not once per value.
       auto values = [&](auto bn_c, auto act_c, auto pool_c) {
         constexpr bool BN = decltype(bn_c)::value;
         constexpr int ACT = decltype(act_c)::value;
         constexpr bool POOL = decltype(pool_c)::value;
+        // where the lane's entries of each N tile go (element offset inside a filter's plane)
+        int yoff[TN];        // pooled: the window; else the first of four pixels in a row (row4); -1: nowhere
+        int nval[TN];        // row4: how many of the four pixels lie inside the image
+        const bool row4 = !POOL && (g.TW & 3) == 0;
+#pragma unroll
+        for (int t = 0; t < TN; t++) {
+          const int n = nb + 16 * t;
+          if constexpr (POOL) {
+            const int q = n >> 2;
+            const int py = mdiv(q, g.mHTW), px = q - py * g.HTW;
+            const int oy = (oy0 >> 1) + py, ox = (ox0 >> 1) + px;
+            yoff[t] = (n < g.npix && oy < g.ph && ox < g.pw) ? oy * g.pw + ox : -1;
+            nval[t] = 0;
+          } else {
+            const int ty = mdiv(n, g.mTW), tx = n - ty * g.TW;
+            const int oy = oy0 + ty, ox = ox0 + tx;
+            yoff[t] = (n < g.npix && oy < g.oh && ox < g.ow) ? oy * g.ow + ox : -1;
+            nval[t] = min(g.ow - ox, 4);
+          }
+        }
+        const bool vec4 = row4 && (g.ow & 3) == 0 && (plane & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
 #pragma unroll
         for (int a = 0; a < TM; a++) {
-          // BatchNorm constants of this lane's filters 16 a + 4 lk + (0..3): one 128-bit read
-          // each; an absent gamma is 1 and an absent beta -0 in the table, which change no bits
-          const float* const fp = ftab + 16 * a + 4 * elk;
-          if constexpr (BN) {   // two constants at a time, so that eight registers hold them, not sixteen
-            const f32x4 ca = *reinterpret_cast<const f32x4*>(fp);
-            const f32x4 cb = *reinterpret_cast<const f32x4*>(fp + BM);
-#pragma unroll
-            for (int t = 0; t < TN; t++)
-#pragma unroll
-              for (int v = 0; v < 4; v++) {
-                acc[a][t][v] = acc[a][t][v] * ca[v];
-                acc[a][t][v] = acc[a][t][v] + cb[v];
-              }
-            const f32x4 cg = *reinterpret_cast<const f32x4*>(fp + 2 * BM);
-            const f32x4 ce = *reinterpret_cast<const f32x4*>(fp + 3 * BM);
-#pragma unroll
-            for (int t = 0; t < TN; t++)
-#pragma unroll
-              for (int v = 0; v < 4; v++) {
-                acc[a][t][v] = cg[v] * acc[a][t][v];
-                acc[a][t][v] = acc[a][t][v] + ce[v];
-              }
+          const int fl = 16 * a + eli;                 // the lane's filter inside the workgroup's tile
+          const bool fok = m0 + fl < g.F;
+          const unsigned foff = (unsigned)fl * pbytes;
+          float ka = 0.f, kb = 0.f, kg = 0.f, ke = 0.f;
+          if constexpr (BN) {   // an absent gamma is 1 and an absent beta -0 in the table, which change no bits
+            ka = ftab[fl]; kb = ftab[BM + fl]; kg = ftab[2 * BM + fl]; ke = ftab[3 * BM + fl];
           }
-          const int fl = 16 * a + 4 * elk;             // first of the lane's four filters, inside the tile
-          const int nf = min(max(g.F - (m0 + fl), 0), 4);   // how many of them exist
 #pragma unroll
           for (int t = 0; t < TN; t++) {
-            unsigned off = (unsigned)fl * pbytes + 4u * (unsigned)max(yoff[t], 0);
-            const bool live = yoff[t] >= 0 && nf > 0;
-            float res[4];
+            f32x4 v = acc[a][t];
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-              float val = act_apply(acc[a][t][v], ACT, alpha);
-              if constexpr (POOL) {
-                // The reference scans the window in order from -FLT_MAX, taking a value only if it
-                // is greater.  The same in three steps: each lane clamps its own value the way the
-                // scan would (NaN and anything <= -FLT_MAX never enter), then a tree over the quad
-                // in which the earlier position keeps a tie (it matters between +0 and -0).  Lane
-                // 0 of the quad ends with the window's value; the others are not stored.
-                val = val > -3.402823466e+38f ? val : -3.402823466e+38f;
-                const float nb = quad_perm<1, 0, 3, 2>(val);
-                val = nb > val ? nb : val;          // lanes 0 and 2: pairs (0,1) and (2,3)
-                const float far = quad_perm<2, 3, 0, 1>(val);
-                val = far > val ? far : val;        // lane 0: the whole window
+            for (int r = 0; r < 4; r++) {
+              if constexpr (BN) {
+                v[r] = v[r] * ka;
+                v[r] = v[r] + kb;
+                v[r] = kg * v[r];
+                v[r] = v[r] + ke;
               }
-              res[v] = val;
+              v[r] = act_apply(v[r], ACT, alpha);
             }
-            if (all4) {
-              if (live) {   // one test for the four stores
+            if constexpr (POOL) {
+              // the reference's scan of the window from -FLT_MAX with a strict compare, positions in order
+              float best = -3.402823466e+38f;
 #pragma unroll
-                for (int v = 0; v < 4; v++) *reinterpret_cast<float*>(ytile + (off + v * pbytes)) = res[v];
+              for (int r = 0; r < 4; r++)
+                if (v[r] > best) best = v[r];
+              if (fok && yoff[t] >= 0) *reinterpret_cast<float*>(ytile + (foff + 4u * (unsigned)yoff[t])) = best;
+            } else if (row4) {
+              if (fok && yoff[t] >= 0) {
+                char* const yp = ytile + (foff + 4u * (unsigned)yoff[t]);
+                if (vec4 && nval[t] >= 4) {
+                  *reinterpret_cast<f32x4*>(yp) = v;
+                } else {
+#pragma unroll
+                  for (int r = 0; r < 4; r++)
+                    if (r < nval[t]) reinterpret_cast<float*>(yp)[r] = v[r];
+                }
               }
             } else {
+              // a patch row is no multiple of four pixels: each of the lane's entries has its own row and column
 #pragma unroll
-              for (int v = 0; v < 4; v++)
-                if (live && v < nf) *reinterpret_cast<float*>(ytile + (off + v * pbytes)) = res[v];
+              for (int r = 0; r < 4; r++) {
+                const int n = nb + 16 * t + r;
+                const int ty = mdiv(n, g.mTW), tx = n - ty * g.TW;
+                const int oy = oy0 + ty, ox = ox0 + tx;
+                if (fok && n < g.npix && oy < g.oh && ox < g.ow)
+                  *reinterpret_cast<float*>(ytile + (foff + 4u * (unsigned)(oy * g.ow + ox))) = v[r];
+              }
             }
           }
         }
