@@ -76,36 +76,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
   const int m0 = blockIdx.y * BM;
   if (tid < BM) conv_tail_table(tail, ftab, BM, tid, min(m0 + tid, g.F - 1));
 
-  // ---- the filter tile, once: As[a][k][f] = w[m0 + 16 a + f][k], zero for k >= K
-  {
-    const int f = tid & (BM - 1), j0 = tid / BM;
-    const float* const wrow = w + (int64_t)min(m0 + f, g.F - 1) * g.K;
-    float* const ad = As + (f >> 4) * g.KP * 16 + (f & 15);
-    constexpr int JS = kThreads / BM;    // 128-bit columns in flight per pass
-    const int ncol = g.KP / 4;
-    if ((g.K & 3) == 0) {
-      // every workgroup reads the same filter rows at the same moment: each starts at a column
-      // of its own (and wraps), so that their loads spread over the cache channels
-      const int rot = (int)((blockIdx.x * 5u) % (unsigned)ncol);
-      for (int j = j0; j < ncol; j += 4 * JS) {
-        f32x4 v[4];
-        int jj[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-          const int jc = min(j + u * JS, ncol - 1) + rot;   // passes past the end rewrite the last column
-          jj[u] = jc >= ncol ? jc - ncol : jc;
-          v[u] = *reinterpret_cast<const f32x4_a4*>(wrow + 4 * jj[u]);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-#pragma unroll
-          for (int e = 0; e < 4; e++) ad[(4 * jj[u] + e) * 16] = v[u][e];
-        }
-      }
-    } else {
-      for (int k = j0; k < g.KP; k += JS) ad[k * 16] = k < g.K ? wrow[k] : 0.f;
-    }
-  }
   // ---- per-thread patch cells, the same for every tile: source offset relative to the patch
   // origin, row and column inside the padded patch, destination in the buffer.  Slots past the
   // last cell and cells of padded channels are flagged: they load nothing that matters and
@@ -128,22 +98,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
     for (int bsel = 0; bsel < (DB ? 2 : 1); bsel++)
       for (int i = zero0 + tid; i < zero1; i += kThreads) P0[bsel * plane_floats + i] = 0.f;
   }
-  // ---- table of patch cells of the N entries
-  for (int n = tid; n < NB; n += kThreads) {
-    const int nn = n < g.npix ? n : 0;   // idle column: any valid cell
-    int ty, tx;
-    if (g.pool) {
-      const int q = nn >> 2, wpos = nn & 3;
-      const int py = mdiv(q, g.mHTW), px = q - py * g.HTW;
-      ty = 2 * py + (wpos >> 1);
-      tx = 2 * px + (wpos & 1);
-    } else {
-      ty = mdiv(nn, g.mTW);
-      tx = nn - ty * g.TW;
-    }
-    tab[n] = ty * g.PW + tx;
-  }
-
   float xv[XS];
   // global loads of one tile's patch into registers.  A patch that lies inside the image, halo
   // and all, needs no test: every load is base + per-thread offset.  At the image border each
@@ -188,6 +142,53 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(XS == 
     tile = blockIdx.x; tile_end = ntiles; tile_step = gridDim.x;
   }
   load_patch(tile);                      // the launch leaves no workgroup without a tile
+  // (the first patch is on its way while the filter tile is fetched and the table is filled)
+  // ---- the filter tile, once: As[a][k][f] = w[m0 + 16 a + f][k], zero for k >= K
+  {
+    const int f = tid & (BM - 1), j0 = tid / BM;
+    const float* const wrow = w + (int64_t)min(m0 + f, g.F - 1) * g.K;
+    float* const ad = As + (f >> 4) * g.KP * 16 + (f & 15);
+    constexpr int JS = kThreads / BM;    // 128-bit columns in flight per pass
+    const int ncol = g.KP / 4;
+    if ((g.K & 3) == 0) {
+      // every workgroup reads the same filter rows at the same moment: each starts at a column
+      // of its own (and wraps), so that their loads spread over the cache channels
+      const int rot = (int)((blockIdx.x * 5u) % (unsigned)ncol);
+      for (int j = j0; j < ncol; j += 4 * JS) {
+        f32x4 v[4];
+        int jj[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          const int jc = min(j + u * JS, ncol - 1) + rot;   // passes past the end rewrite the last column
+          jj[u] = jc >= ncol ? jc - ncol : jc;
+          v[u] = *reinterpret_cast<const f32x4_a4*>(wrow + 4 * jj[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) ad[(4 * jj[u] + e) * 16] = v[u][e];
+        }
+      }
+    } else {
+      for (int k = j0; k < g.KP; k += JS) ad[k * 16] = k < g.K ? wrow[k] : 0.f;
+    }
+  }
+  // ---- table of patch cells of the N entries
+  for (int n = tid; n < NB; n += kThreads) {
+    const int nn = n < g.npix ? n : 0;   // idle column: any valid cell
+    int ty, tx;
+    if (g.pool) {
+      const int q = nn >> 2, wpos = nn & 3;
+      const int py = mdiv(q, g.mHTW), px = q - py * g.HTW;
+      ty = 2 * py + (wpos >> 1);
+      tx = 2 * px + (wpos & 1);
+    } else {
+      ty = mdiv(nn, g.mTW);
+      tx = nn - ty * g.TW;
+    }
+    tab[n] = ty * g.PW + tx;
+  }
+
   store_patch(P0);
   __syncthreads();
 
