@@ -47,6 +47,9 @@ struct PatchGeom {
   int pool, ph, pw, HTW;          // fused 2x2 / stride-2 max-pool: pooled extents of y, TW / 2
   int epi_off;                    // float offset in LDS of the per-filter epilogue table (past every other use)
   unsigned mTXY, mTX, mPP, mPW, mTW, mHTW, mNPIX, mNPOOL;   // magics: tiles_x*tiles_y, tiles_x, PP, PW, TW, HTW, npix, npix/4
+  // the launch is one-dimensional: workgroup id -> (patch, filter tile), see the kernel
+  int ntiles, ftiles, nwg;        // patches of the batch, filter tiles, their product
+  int ft_major;                   // 1: an XCD owns whole filter tiles (all patches of each); 0: whole patches (all filter tiles)
 };
 
 constexpr int kWaves = 8;
@@ -73,11 +76,24 @@ __global__ __launch_bounds__(kWaves * 64) void k_conv3x3_patch(const float* __re
   float* const Pw = Aw + 36 * SA;                 // [4][PL]
   int* const tab = reinterpret_cast<int*>(lds + kWaves * wsize);   // [16 TN] cell of N entry n inside the padded patch
 
-  const int bimg = mdiv(blockIdx.x, g.mTXY);
-  const int trem = blockIdx.x - bimg * (g.tiles_x * g.tiles_y);
+  // Workgroup ids are dealt round-robin over the 8 XCDs, each with its own L2.  An XCD gets one contiguous
+  // run of the (patch, filter tile) pairs, ordered so that what the run shares is the larger operand:
+  // patch-major where the images outweigh the filters (the workgroups of a patch and of its neighbours,
+  // whose halos overlap, then meet in one L2), filter-tile-major where the filters do (a filter tile is
+  // then fetched from memory by one XCD instead of by every one that holds an image).
+  int wpatch, wft;
+  {
+    const int id = blockIdx.x, xcd = id & 7, per = g.nwg >> 3, extra = g.nwg & 7;
+    const int lin = xcd * per + min(xcd, extra) + (id >> 3);
+    // (a true division, once per workgroup: the multiply-shift form is exact only while id x divisor < 2^32)
+    if (g.ft_major) { wft = (int)((unsigned)lin / (unsigned)g.ntiles); wpatch = lin - wft * g.ntiles; }
+    else { wpatch = (int)((unsigned)lin / (unsigned)g.ftiles); wft = lin - wpatch * g.ftiles; }
+  }
+  const int bimg = mdiv(wpatch, g.mTXY);
+  const int trem = wpatch - bimg * (g.tiles_x * g.tiles_y);
   const int tyi = mdiv(trem, g.mTX), txi = trem - tyi * g.tiles_x;
   const int oy0 = tyi * g.TH, ox0 = txi * g.TW;
-  const int m0 = blockIdx.y * BM;
+  const int m0 = wft * BM;
   const int c0 = wave * (4 * g.NQ);
   float* const ftab = lds + g.epi_off;            // [4][BM] BatchNorm constants of this workgroup's filters
   if (tid < BM) conv_tail_table(tail, ftab, BM, tid, min(m0 + tid, g.F - 1));
@@ -357,10 +373,18 @@ int launch_patch(gh_ctx* ctx, const gh_cmd& c, const PatchPlan& p) {
                                   160 * 1024);
   });
   if (attr_rc != hipSuccess) return gh_check_hip(ctx, attr_rc, "hipFuncSetAttribute(conv3x3 patch)");
-  const dim3 grid((unsigned)(p.g.B * p.g.tiles_x * p.g.tiles_y), (unsigned)((p.g.F + 16 * TM - 1) / (16 * TM)));
-  hipLaunchKernelGGL((k_conv3x3_patch<TM, TN>), grid, dim3(kWaves * 64), p.lds, ctx->stream,
+  PatchGeom g = p.g;
+  g.ntiles = g.B * g.tiles_x * g.tiles_y;
+  g.ftiles = (g.F + 16 * TM - 1) / (16 * TM);
+  const int64_t nwg = (int64_t)g.ntiles * g.ftiles;
+  if (nwg >= (1ll << 31)) return gh_fail(ctx, GH_EINVAL, "conv2d: too many workgroups for the patch kernel");
+  g.nwg = (int)nwg;
+  static const bool no_xcd = getenv("GORGONIA_HIP_CONV_PATCH_ORDER") != nullptr;   // tuning switch: "0" patch-major, "1" filter-tile-major
+  g.ft_major = (int64_t)g.F * g.K > (int64_t)g.B * g.C * g.HW ? 1 : 0;
+  if (no_xcd) g.ft_major = atoi(getenv("GORGONIA_HIP_CONV_PATCH_ORDER")) != 0;
+  hipLaunchKernelGGL((k_conv3x3_patch<TM, TN>), dim3((unsigned)g.nwg), dim3(kWaves * 64), p.lds, ctx->stream,
                      (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
-                     (float*)(uintptr_t)c.ptr[2], p.g, conv_tail(c));
+                     (float*)(uintptr_t)c.ptr[2], g, conv_tail(c));
   return gh_check_hip(ctx, hipGetLastError(), "conv3x3 patch launch");
 }
 
