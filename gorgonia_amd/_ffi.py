@@ -44,6 +44,7 @@ FLAG_BN_EVAL = 1 << 26
 FLAG_GEMM_SOFTMAX = 1 << 27
 FLAG_GEMM_BIAS = 1 << 28
 FLAG_CONV_PRE = 1 << 29
+FLAG_CONV_KEEP = 1 << 30
 
 
 def flag_fn(f):
@@ -92,6 +93,7 @@ SYMBOLS = {
     "gh_validate": (C.c_int, [C.POINTER(GhCmd), C.c_int, C.c_char_p, C.c_int]),
     "gh_conv2d_can_pool": (C.c_int, [C.POINTER(GhCmd)]),
     "gh_conv2d_can_pre": (C.c_int, [C.POINTER(GhCmd)]),
+    "gh_conv2d_can_keep": (C.c_int, [C.POINTER(GhCmd)]),
     "gh_conv2d_route": (C.c_int, [C.POINTER(GhCmd)]),
     "gh_conv2d_bwd_filter_route": (C.c_int, [C.POINTER(GhCmd)]),
     "gh_gemm_route": (C.c_int, [C.POINTER(GhCmd), C.POINTER(C.c_int)]),

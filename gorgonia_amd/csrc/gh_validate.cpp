@@ -81,7 +81,7 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       return GH_OK;
     case GH_OP_CONV2D_BWD_DATA:
     case GH_OP_CONV2D_BWD_FILTER:
-      if (c.flags & (GH_FLAG_CONV_BN | GH_FLAG_CONV_POOL2 | GH_FLAG_ACT_RELU | GH_FLAG_ACT_LEAKY | GH_FLAG_CONV_PRE))
+      if (c.flags & (GH_FLAG_CONV_BN | GH_FLAG_CONV_POOL2 | GH_FLAG_ACT_RELU | GH_FLAG_ACT_LEAKY | GH_FLAG_CONV_PRE | GH_FLAG_CONV_KEEP))
         return bad("conv2d backward takes no epilogue flags");
       [[fallthrough]];
     case GH_OP_CONV2D: {
@@ -110,6 +110,12 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
         return bad("conv2d: no epilogue operators for float64");
       if ((c.flags & GH_FLAG_CONV_POOL2) && !gh_conv2d_can_pool(&c))
         return bad("conv2d: no fused pooling for this shape");
+      if (c.flags & GH_FLAG_CONV_KEEP) {
+        if (c.opcode != GH_OP_CONV2D || dt != GH_F32 || !(c.flags & GH_FLAG_CONV_POOL2) || (c.flags & GH_FLAG_CONV_PRE))
+          return bad("conv2d: keeping the unpooled result is for the float32 forward command with fused pooling, without a folded first layer");
+        if (!c.ptr[7]) return bad("conv2d: the tensor for the unpooled result (ptr[7]) is null");
+        if (!gh_conv2d_can_keep(&c)) return bad("conv2d: the unpooled result cannot be kept for this shape");
+      }
       if (c.flags & GH_FLAG_CONV_PRE) {
         if (c.opcode != GH_OP_CONV2D || dt != GH_F32) return bad("conv2d: a folded first layer is for the float32 forward command");
         if (!c.ptr[7]) return bad("conv2d: the folded first layer's filters (ptr[7]) are null");

@@ -71,6 +71,10 @@ struct RowsGeom {
   int preRW, preRP, preZP;   // padded row pitch, floats per padded image, zero floats in front
   int preOff, preFloats;     // LDS offset and size of the padded images, floats
   int preTab;                // LDS offset of the window tables: [4 prePT] patch offsets, [4 prePT] plane offsets
+  // GH_FLAG_CONV_KEEP (the kernel then runs its unpooled form): y gets the pooled result of the window part as
+  // well, the convolution's own values go to `keep`
+  int keep, offTabO2;        // flag; LDS offset of [4 PT] pooled result offsets per window (-1: none)
+  int poolplane;             // floats per pooled plane
   int preHW, preNL, prePT;   // pixels of a single-channel image; loads per thread; 16-pixel tiles of its convolution
   unsigned mHW, mPreHW, mPreW;
 };
@@ -103,7 +107,7 @@ __device__ __forceinline__ float tail_reg(float v, const float (&k)[4], float al
 template <int NQ, int A, int TFB, bool POOL, int WPT, int QPT, int NLDT, bool PRE>
 __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restrict__ x, const float* __restrict__ w,
                                                            float* __restrict__ y, RowsGeom g, ConvTail tail,
-                                                           const float* __restrict__ w0) {
+                                                           const float* __restrict__ w0, float* __restrict__ keep) {
   static_assert((TFB * NQ) % kWaves == 0 && NQ % kWaves == 0, "quads divide over the wavefronts");
   constexpr int NFP = TFB * NQ / kWaves;      // filter (tile, quad) pairs staged per wavefront
   constexpr int QW = NQ / kWaves;             // quads of a leftover unit per wavefront
@@ -223,6 +227,10 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
     tabP[n] = img * NQ * QPs + oy * Wps + ox;
     if (!POOL) tabO[n] = valid ? (img * g.F) * g.outplane + oy * g.ow + ox : -1;
     else if ((n & 3) == 0) tabO[n >> 2] = valid ? (img * g.F) * g.outplane + wi : -1;
+    if constexpr (!POOL) {
+      if (g.keep && (n & 3) == 0)
+        reinterpret_cast<int*>(lds + g.offTabO2)[n >> 2] = (valid && n < g.wpart) ? (img * g.F) * g.poolplane + wi : -1;
+    }
   }
   __syncthreads();
   // ---- stage: filters (lane order is the MFMA operand order), image interiors
@@ -300,7 +308,10 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
 
   const int ft = wave % TFB, pg = wave / TFB;
   const int lkoff = lk * PP;
-  float* const ybase = y + (int64_t)b0 * g.F * g.outplane;
+  // (with `keep` the unpooled values go there and y takes the pooled ones)
+  float* const ybase = (!POOL && g.keep ? keep : y) + (int64_t)b0 * g.F * g.outplane;
+  float* const pbase = y + (int64_t)b0 * g.F * g.poolplane;
+  const int* const tabO2 = reinterpret_cast<const int*>(lds + g.offTabO2);
   const int outplane = g.outplane;
   const float alpha = tail.alpha;
   // the epilogue of one tile: four N entries of filter `fcol` in v
@@ -309,6 +320,26 @@ __global__ __launch_bounds__(kThreads) void k_conv3x3_rows(const float* __restri
     constexpr bool BN = decltype(bn_c)::value;
     constexpr int ACT = decltype(act_c)::value;
     const bool ok = fcol < g.F;
+    if constexpr (!POOL) {
+      if (g.keep) {
+        // the convolution's own values (after BatchNorm) as the plain command stores them, then the activation
+        // and the pooling scan of the window the lane holds
+#pragma unroll
+        for (int r = 0; r < 4; r++) v[r] = tail_reg<BN, 0>(v[r], k, alpha);
+        const i32x4 o = *reinterpret_cast<const i32x4*>(tabO + 16 * pt + 4 * lk);
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          if (ok && o[r] >= 0) ybase[o[r] + fcol * outplane] = v[r];
+        const int o2 = tabO2[4 * pt + lk];
+#pragma unroll
+        for (int r = 0; r < 4; r++) v[r] = act_apply(v[r], ACT, alpha);
+        float best = -3.402823466e+38f;
+#pragma unroll
+        for (int r = 0; r < 4; r++) if (v[r] > best) best = v[r];
+        if (ok && o2 >= 0) pbase[o2 + fcol * g.poolplane] = best;
+        return;
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 4; r++) v[r] = tail_reg<BN, ACT>(v[r], k, alpha);
     if constexpr (POOL) {
@@ -508,7 +539,7 @@ bool rows_plan_compute(const gh_cmd& c, bool pool, RowsPlan* out) {
       const int A = PTw / wave_groups;
       if (A > 4) break;
       const int LUu = (PTu - A * wave_groups) * TFB;
-      size_t fl = (size_t)TFB * NQ * 576 + (size_t)IPB * NQ * g.QP + 32 * (size_t)PTu + 4;
+      size_t fl = (size_t)TFB * NQ * 576 + (size_t)IPB * NQ * g.QP + 36 * (size_t)PTu + 4;
       if ((fl + (LUu ? 2048 * TFB : 0)) * 4 > kLdsBudget) break;
       const size_t lds = (fl + (size_t)LUu * 2048) * 4 > kLdsBudget ? kLdsBudget : (fl + (size_t)LUu * 2048) * 4;
       const int64_t blocks = ((F + 16 * TFB - 1) / (16 * TFB)) * ((B + IPB - 1) / IPB);
@@ -541,6 +572,8 @@ bool rows_plan_compute(const gh_cmd& c, bool pool, RowsPlan* out) {
   g.offP = off; off += g.IPB * NQ * g.QP;
   g.offTabP = off; off += 16 * g.PT;
   g.offTabO = off; off += pool ? 4 * g.PT : 16 * g.PT;
+  g.offTabO2 = off; off += pool ? 0 : 4 * g.PT;   // used by GH_FLAG_CONV_KEEP; part of every plain plan, so the flag changes no plan
+  g.poolplane = g.ph * g.pw;
   off = (off + 3) & ~3;
   g.offRed = off;
   // as many leftover units per round as the rest of LDS holds
@@ -605,7 +638,8 @@ int launch_rows(gh_ctx* ctx, const gh_cmd& c, const RowsPlan& p) {
   const dim3 grid((unsigned)((p.g.B + p.g.IPB - 1) / p.g.IPB), (unsigned)((p.g.F + 16 * TFB - 1) / (16 * TFB)));
   hipLaunchKernelGGL((k_conv3x3_rows<NQ, A, TFB, POOL, WPT, QPT, NLDT, PRE>), grid, dim3(kThreads), p.lds, ctx->stream,
                      (const float*)(uintptr_t)c.ptr[0], (const float*)(uintptr_t)c.ptr[1],
-                     (float*)(uintptr_t)c.ptr[2], p.g, conv_tail(c), (const float*)(uintptr_t)c.ptr[7]);
+                     (float*)(uintptr_t)c.ptr[2], p.g, conv_tail(c), PRE ? (const float*)(uintptr_t)c.ptr[7] : nullptr,
+                     p.g.keep ? (float*)(uintptr_t)c.ptr[7] : nullptr);
   return gh_check_hip(ctx, hipGetLastError(), "conv3x3 rows launch");
 }
 
@@ -678,9 +712,16 @@ bool gh_conv_rows_can_pre(const gh_cmd& c) {
 // Returns -1 when the shape is not one this kernel takes.
 int gh_try_launch_conv_rows(gh_ctx* ctx, const gh_cmd& c) {
   RowsPlan p;
-  const bool pool = c.flags & GH_FLAG_CONV_POOL2;
+  bool pool = c.flags & GH_FLAG_CONV_POOL2;
   // a pooled command only rides here when the plain one would too: both then sum in the same order
   if (!rows_plan(c, false, &p)) return -1;
+  if (pool && (c.flags & GH_FLAG_CONV_KEEP)) {
+    // the plain command's plan and kernel, which then stores the pooled windows as well
+    if (!gh_conv_rows_can_pool(c) || !c.ptr[7] || (c.flags & GH_FLAG_CONV_PRE))
+      return gh_fail(ctx, GH_EINVAL, "conv2d: the convolution's own result cannot be kept next to the pooled one here (see gh_conv2d_can_keep)");
+    p.g.keep = 1;
+    pool = false;
+  }
   if (pool && !rows_plan(c, true, &p))
     return gh_fail(ctx, GH_EINVAL, "conv2d: no fused pooling for this shape (see gh_conv2d_can_pool)");
   if (c.flags & GH_FLAG_CONV_PRE) {

@@ -44,9 +44,12 @@ struct Rows1Geom {
   unsigned mW, mPW;
 };
 
+// keep: with POOL, where the convolution's own result goes as well (B x F x oh x ow, the values the activation
+// and the pool read), or null.
 template <bool POOL>
 __global__ __launch_bounds__(kThreads1) void k_conv3x3_rows1(const float* __restrict__ x, const float* __restrict__ w,
-                                                             float* __restrict__ y, Rows1Geom g, ConvTail tail) {
+                                                             float* __restrict__ y, Rows1Geom g, ConvTail tail,
+                                                             float* __restrict__ keep) {
   extern __shared__ float lds[];
   float* const Raw = lds;
   float* const Wl = lds + g.offW;   // [FT][3][64]
@@ -94,6 +97,7 @@ __global__ __launch_bounds__(kThreads1) void k_conv3x3_rows1(const float* __rest
     const bool wok = gwd < g.ph * g.pw;
     const int pyd = mdiv(gwd, g.mPW), pxd = gwd - pyd * g.pw;
     const int o = POOL ? gwd : 2 * pyd * g.ow + 2 * pxd;
+    const int okeep = 2 * pyd * g.ow + 2 * pxd;
     for (int ft = 0; ft < g.FT; ft++) {
       float b[3];
       const float* const wl = Wl + ft * 192 + lane;
@@ -117,6 +121,17 @@ __global__ __launch_bounds__(kThreads1) void k_conv3x3_rows1(const float* __rest
             t = t + kb;
             t = kg * t;
             v[r] = t + kbeta;
+          }
+        }
+        if constexpr (POOL) {
+          if (keep && ok) {   // the pair stores of the plain command
+            float* const kp = keep + ((int64_t)img * g.F + col) * (g.oh * g.ow) + okeep;
+            if (g.y8) {
+              *reinterpret_cast<f32x2*>(kp) = f32x2{v[0], v[1]};
+              *reinterpret_cast<f32x2*>(kp + g.ow) = f32x2{v[2], v[3]};
+            } else {
+              kp[0] = v[0]; kp[1] = v[1]; kp[g.ow] = v[2]; kp[g.ow + 1] = v[3];
+            }
           }
         }
 #pragma unroll
@@ -183,16 +198,17 @@ int gh_try_launch_conv_rows1(gh_ctx* ctx, const gh_cmd& c) {
   if (parts < 1) parts = 1;
   g.TPP = (g.PT + parts - 1) / parts;
   parts = (g.PT + g.TPP - 1) / g.TPP;
-  g.y8 = (c.ptr[2] & 7) == 0;
   const bool pool = c.flags & GH_FLAG_CONV_POOL2;
+  float* const keep = (pool && (c.flags & GH_FLAG_CONV_KEEP)) ? (float*)(uintptr_t)c.ptr[7] : nullptr;
+  g.y8 = ((keep ? c.ptr[7] : c.ptr[2]) & 7) == 0;   // of the tensor that gets the unpooled pairs
   const size_t lds = ((size_t)g.offW + (size_t)g.FT * 192) * 4;
   const dim3 grid((unsigned)parts, (unsigned)g.B);
   const float* x = (const float*)(uintptr_t)c.ptr[0];
   const float* w = (const float*)(uintptr_t)c.ptr[1];
   float* y = (float*)(uintptr_t)c.ptr[2];
   if (pool)
-    hipLaunchKernelGGL((k_conv3x3_rows1<true>), grid, dim3(kThreads1), lds, ctx->stream, x, w, y, g, conv_tail(c));
+    hipLaunchKernelGGL((k_conv3x3_rows1<true>), grid, dim3(kThreads1), lds, ctx->stream, x, w, y, g, conv_tail(c), keep);
   else
-    hipLaunchKernelGGL((k_conv3x3_rows1<false>), grid, dim3(kThreads1), lds, ctx->stream, x, w, y, g, conv_tail(c));
+    hipLaunchKernelGGL((k_conv3x3_rows1<false>), grid, dim3(kThreads1), lds, ctx->stream, x, w, y, g, conv_tail(c), keep);
   return gh_check_hip(ctx, hipGetLastError(), "conv3x3 rows1 launch");
 }

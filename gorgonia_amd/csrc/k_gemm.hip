@@ -2986,6 +2986,8 @@ int gh_launch_conv2d(gh_ctx* ctx, const gh_cmd& c) {
     if (rcp >= 0) return rcp;
     return gh_fail(ctx, GH_EINVAL, "conv2d: no folded first layer for this shape (see gh_conv2d_can_pre)");
   }
+  if ((c.flags & GH_FLAG_CONV_KEEP) && !((c.flags & GH_FLAG_CONV_POOL2) && gh_conv2d_can_keep(&c)))
+    return gh_fail(ctx, GH_EINVAL, "conv2d: the unpooled result cannot be kept for this command (see gh_conv2d_can_keep)");
   const int rc0 = gh_try_launch_conv_rows1(ctx, c);
   if (rc0 >= 0) return rc0;
   if (conv_direct_takes(c)) return launch_conv_direct(ctx, c);
@@ -3247,6 +3249,13 @@ extern "C" int gh_conv2d_bwd_filter_route(const gh_cmd* c) {
   if (conv_direct_shape(*c) && c->dim[4] <= 65535) return GH_WGRAD_ROUTE_DIRECT;
   if (gh_conv_wgrad_small_takes(*c)) return GH_WGRAD_ROUTE_SMALL;
   return GH_WGRAD_ROUTE_GEMM;
+}
+
+extern "C" int gh_conv2d_can_keep(const gh_cmd* c) {
+  if (!c || c->opcode != GH_OP_CONV2D || gh_dtype_of(c->flags) != GH_F32) return 0;
+  if (getenv("GORGONIA_HIP_CONV_NO_KEEP")) return 0;   // tuning switch: the pool stays a kernel of its own
+  if (gh_conv_rows1_takes(*c)) return 1;
+  return gh_conv_rows_takes(*c) && gh_conv_rows_can_pool(*c) ? 1 : 0;
 }
 
 extern "C" int gh_conv2d_can_pre(const gh_cmd* c) {

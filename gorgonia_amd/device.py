@@ -192,12 +192,14 @@ def _double_bits(v):
 
 
 def cmd_conv2d(x, w, y, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dilation=(1, 1),
-               act=None, alpha=0.0, bn=None, eps=1e-5, pool2=False, dtype=_ffi.F32, pre=None):
+               act=None, alpha=0.0, bn=None, eps=1e-5, pool2=False, dtype=_ffi.F32, pre=None, keep=None):
     """bn = (mean, var, gamma or 0, beta or 0) device pointers: BatchNorm (eval)
     on the result; pool2: 2x2 stride-2 MaxPool2D on the result (y is then
     B x F x oh/2 x ow/2).  Order: conv, bn, activation, pool.
     pre = w0 (Cin x 1 x 3 x 3 filters): x holds single-channel images B x 1 x 2H x 2W and the
-    convolution's input is MaxPool2D(Rectify(Conv2d(x, w0, pad 1))), never stored."""
+    convolution's input is MaxPool2D(Rectify(Conv2d(x, w0, pad 1))), never stored.
+    keep (with pool2): a B x F x oh x ow tensor that also receives the unpooled result as the
+    activation reads it."""
     fl = {None: 0, "relu": _ffi.FLAG_ACT_RELU, "leaky": _ffi.FLAG_ACT_LEAKY}[act] | _ffi.flag_dtype(dtype)
     ptrs = [x, w, y]
     if bn is not None:
@@ -209,6 +211,9 @@ def cmd_conv2d(x, w, y, B, Cin, H, W, F, kh, kw, pad=(0, 0), stride=(1, 1), dila
     if pre is not None:
         fl |= _ffi.FLAG_CONV_PRE
         ptrs = (ptrs + [0] * 7)[:7] + [pre]
+    if keep is not None:
+        fl |= _ffi.FLAG_CONV_KEEP
+        ptrs = (ptrs + [0] * 7)[:7] + [keep]
     return make_cmd(_ffi.OP_CONV2D, fl, ptrs,
                     (B, Cin, H, W, F, kh, kw, pad[0], pad[1], stride[0], stride[1], dilation[0],
                      dilation[1]), (alpha, eps))

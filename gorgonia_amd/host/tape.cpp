@@ -289,7 +289,7 @@ static std::string op_name(const OpSpec& op) {
     case OpKind::Outer: return "outer";
     case OpKind::BatchedMatMul: return "batchedmatmul";
     case OpKind::Conv2d:
-      return std::string(op.fuse_pre ? "conv2d+rectify+maxpool2d+conv2d" : "conv2d") + (op.fuse_bn ? "+batchnorm(eval)" : "") +
+      return std::string(op.fuse_pre ? "conv2d+rectify+maxpool2d+conv2d" : op.fuse_keep ? "conv2d(kept)" : "conv2d") + (op.fuse_bn ? "+batchnorm(eval)" : "") +
              (op.fuse_act_relu ? "+rectify" : op.fuse_act_leaky ? "+leakyrelu" : "") +
              (op.fuse_pool2 ? "+maxpool2d" : "");
     case OpKind::MaxPool2D: return op.relu_input ? "rectify+maxpool2d" : "maxpool2d";
@@ -366,7 +366,8 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
       if (x.dt == Dtype::Other || w.dt != x.dt) return bad("Conv2d: Unsupported Dtype");
       if (x.dt == Dtype::Float64 && (op.fuse_bn || op.fuse_act_relu || op.fuse_act_leaky || op.fuse_pool2 || op.fuse_pre))
         return bad("Conv2d: no epilogue operators for float64");
-      const size_t nin = in.size() - (op.fuse_pre ? 1 : 0);   // a folded first layer's filters come last
+      if (op.fuse_pre && op.fuse_keep) return bad("Conv2d: a folded first layer and a kept result exclude each other");
+      const size_t nin = in.size() - (op.fuse_pre || op.fuse_keep ? 1 : 0);   // a folded first layer's filters, or the tensor for the kept result, come last
       gh_cmd c{};
       c.opcode = GH_OP_CONV2D;
       c.flags = (op.fuse_act_relu ? GH_FLAG_ACT_RELU : op.fuse_act_leaky ? GH_FLAG_ACT_LEAKY : 0) | dtype_flag(x.dt);
@@ -390,6 +391,11 @@ Status CUDADo(Engine& e, const OpSpec& op, Tensor& prealloc, const std::vector<T
         c.flags |= GH_FLAG_CONV_PRE;
         c.ptr[7] = in.back()->mem;
         c.dim[1] = w.shape[1]; c.dim[2] = x.shape[2] / 2; c.dim[3] = x.shape[3] / 2;
+      }
+      if (op.fuse_keep) {
+        if (!op.fuse_pool2 || nin < 2) return bad("Conv2d: a kept result goes with fused pooling");
+        c.flags |= GH_FLAG_CONV_KEEP;
+        c.ptr[7] = in.back()->mem;
       }
       c.dim[4] = w.shape[0];
       for (int i = 0; i < 8; i++) c.dim[5 + i] = op.ints[(size_t)i];
@@ -735,6 +741,52 @@ int Graph::FuseActivations() {
   }
   fused += fuse_pooled_rectify();
   fused += fuse_first_layer();
+  fused += fuse_kept_conv();
+  return fused;
+}
+
+// z = Conv2d(x, w); p = MaxPool2D(z) 2x2/2 (read through a Rectify or not) where other nodes read z as well -
+// a training graph, whose backward pass needs the unpooled values - and the library's kernel for the shape
+// can store both (gh_conv2d_can_keep): p takes over the convolution, with z as its last input, the tensor the
+// unpooled values go to; z keeps its register and loses its instruction.  Nothing may read z between the two.
+int Graph::fuse_kept_conv() {
+  int fused = 0;
+  for (auto& pn : nodes_) {
+    if (pn.is_input || pn.fused_away || pn.deferred || pn.op.kind != OpKind::MaxPool2D || pn.inputs.size() != 1) continue;
+    if (pn.dt != Dtype::Float32 || pn.shape.Dims() != 4) continue;
+    const auto& q = pn.op.ints;  // kh kw npad pads... sh sw
+    bool plain = q.size() >= 5 && q[0] == 2 && q[1] == 2;
+    for (size_t i = 3; plain && i < q.size(); i++) plain = q[i] == (i >= 3 + (size_t)q[2] ? 2 : 0);
+    if (!plain) continue;
+    Node& z = nodes_[(size_t)pn.inputs[0]];
+    if (z.is_input || z.fused_away || z.deferred || z.alias_of >= 0 || z.op.kind != OpKind::Conv2d || z.inputs.size() != 2) continue;
+    const OpSpec& zo = z.op;
+    if (zo.fuse_bn || zo.fuse_act_relu || zo.fuse_act_leaky || zo.fuse_pool2 || zo.fuse_pre || zo.fuse_keep) continue;
+    if (z.dt != Dtype::Float32 || z.id >= pn.id) continue;
+    bool read_between = false;
+    for (int j = z.id + 1; j < pn.id && !read_between; j++) {
+      const Node& o = nodes_[(size_t)j];
+      if (o.fused_away) continue;
+      for (int in : o.inputs) if (in == z.id || nodes_[(size_t)in].alias_of == z.id) read_between = true;
+    }
+    if (read_between) continue;
+    const Shape& xs = nodes_[(size_t)z.inputs[0]].shape;
+    const Shape& ws = nodes_[(size_t)z.inputs[1]].shape;
+    gh_cmd c{};
+    c.opcode = GH_OP_CONV2D;
+    for (int i = 0; i < 4; i++) c.dim[i] = xs[i];
+    c.dim[4] = ws[0];
+    for (int i = 0; i < 8; i++) c.dim[5 + i] = zo.ints[(size_t)i];
+    if (!gh_conv2d_can_pool(&c) || !gh_conv2d_can_keep(&c)) continue;
+    OpSpec op = zo;
+    op.fuse_pool2 = true;
+    op.fuse_keep = true;
+    op.fuse_act_relu = pn.op.relu_input;
+    pn.op = op;
+    pn.inputs = {z.inputs[0], z.inputs[1], z.id};
+    z.deferred = true;
+    fused++;
+  }
   return fused;
 }
 
@@ -925,7 +977,7 @@ Status TapeMachine::Compile() {
         reg_bytes[(size_t)r] = bytes;
         gpumem_ += bytes;
       }
-      prog_.push_back({InstrKind::ExecOp, i, r, bytes, inplace[(size_t)i] != 0});
+      if (!n.deferred) prog_.push_back({InstrKind::ExecOp, i, r, bytes, inplace[(size_t)i] != 0});
     }
     // registers whose last use is this instruction die here
     for (int q = 0; q < nreg; q++)

@@ -83,6 +83,10 @@ struct OpSpec {
   // single-channel images and the last input the filters of Conv2d 3x3 pad 1 -> Rectify -> MaxPool2D 2x2/2
   // whose result this convolution reads without it ever being stored.
   bool fuse_pre = false;
+  // Conv2d only, with fuse_pool2: the convolution's own result is stored as well (GH_FLAG_CONV_KEEP), into the
+  // register of the node given as the last input - a Conv2d node whose work this node has taken over
+  // (Node::deferred) because other nodes, a backward pass, read the unpooled values too.
+  bool fuse_keep = false;
   // MaxPool2D / MaxPool2DDiff: input 0 is the value before a Rectify and is read through it; the
   // diff also applies the Rectify's own gradient (it stands for RectifyDiff(z, MaxPool2DDiff(Rectify(z), g)))
   bool relu_input = false;
@@ -110,6 +114,7 @@ struct Node {
   void* read_into = nullptr;      // Read(node, &host) target
   bool read_borrowed = false;     // ReadBorrowed: the value stays in the machine's own pinned buffer
   bool fused_away = false;        // absorbed into the follower that now computes both: no register, no instruction
+  bool deferred = false;          // keeps its register, but a later node (which lists it as its last input) writes it: no instruction
   int alias_of = -1;              // Reshape shares its input's register
 };
 
@@ -134,6 +139,7 @@ class Graph {
   int FuseActivations();
   int fuse_pooled_rectify();   // part of FuseActivations: the Rectify between a pool and both gradients
   int fuse_first_layer();      // part of FuseActivations: a single-channel first layer folded into the next convolution
+  int fuse_kept_conv();        // part of FuseActivations: a pool into the convolution whose result other nodes read too
   const std::vector<Node>& Nodes() const { return nodes_; }
   std::vector<Node>& Nodes() { return nodes_; }
 

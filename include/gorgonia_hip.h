@@ -134,6 +134,7 @@ enum gh_unaryfn {
 #define GH_FLAG_CONV_POOL2   (1u << 25)   /* CONV2D: 2x2 stride-2 unpadded MaxPool2D on the result */
 #define GH_FLAG_GEMM_SOFTMAX (1u << 27)   /* GEMM: row SoftMax on the result (after the activation) */
 #define GH_FLAG_CONV_PRE     (1u << 29)   /* CONV2D: the input is made on the fly from single-channel images, see below */
+#define GH_FLAG_CONV_KEEP    (1u << 30)   /* CONV2D with CONV_POOL2: ptr[7] also receives the unpooled result, see below */
 #define GH_FLAG_GEMM_BIAS    (1u << 28)   /* GEMM (untransposed): ptr[3] = N floats added to every row of the product (before the activation) */
 
 /*
@@ -170,6 +171,11 @@ enum gh_unaryfn {
  *             with HAS_BETA ptr[6]=beta, f[1]=eps; BN_INFER's arithmetic per filter),
  *             then ACT_RELU / ACT_LEAKY, then CONV_POOL2 (y then has the pooled
  *             shape B,F,oh/2,ow/2; only where gh_conv2d_can_pool says so)
+ *             CONV_KEEP (float32, with CONV_POOL2, only where gh_conv2d_can_keep says so): ptr[7] =
+ *             a (B,F,oh,ow) tensor that also receives the convolution's result as the activation
+ *             and the pool read it (after a fused BatchNorm, before the activation) - what a
+ *             training step keeps for the backward pass; both tensors hold the bits of the
+ *             separate commands.  Not together with CONV_PRE.
  *             CONV_PRE (float32, only where gh_conv2d_can_pre says so): the operators in front
  *             of the convolution ride along too.  ptr[0] then holds single-channel images
  *             (B,1,2H,2W) and ptr[7] C filters (C,1,3,3); the convolution's input (B,C,H,W) is
@@ -307,6 +313,10 @@ GH_API int gh_conv2d_can_pool(const gh_cmd* conv);
  * runs the first layer of its convolutional example as three operators with two stored tensors
  * between them (examples/convnet/main.go:86-112); folded, a step has one kernel and one tensor less. */
 GH_API int gh_conv2d_can_pre(const gh_cmd* conv);
+/* 1 when gh_submit accepts GH_FLAG_CONV_KEEP on this float32 CONV2D command with CONV_POOL2.  Host only.
+ * The reference's training graph stores the convolution's result and runs the activation and the pool
+ * as operators of their own (examples/convnet/main.go:86-112); here the convolution stores both. */
+GH_API int gh_conv2d_can_keep(const gh_cmd* conv);
 /* Which of the library's convolution kernels gh_submit runs this float32 CONV2D command on, a
  * function of its shape, its flags and (for the filter operand's alignment) its pointers: one of
  * GH_CONV_ROUTE_*, or -1 for a command that is no float32 CONV2D.  Host only.  The reference

@@ -374,6 +374,44 @@ def test_conv_folded_first_layer_bit_exact(ctx, cfg):
     assert_bits_equal(folded(xs, ws), gpu_conv(ctx, mids, w1, (pad, pad), (1, 1), (1, 1)), f"folded special values {cfg}")
 
 
+@pytest.mark.parametrize("cfg", ROWS_CASES + ROWS1_CASES)
+def test_conv_keeps_unpooled_result_bit_exact(ctx, cfg):
+    """GH_FLAG_CONV_KEEP: one command stores the pooled activation and the convolution's own result, each with
+    the bits of the separate commands (what a training step keeps for its backward pass)."""
+    B, C, H, W, F, pad = cfg
+    oh, ow = H + 2 * pad - 2, W + 2 * pad - 2
+    probe = D.cmd_conv2d(1, 1, 1, B, C, H, W, F, 3, 3, (pad, pad))
+    if not ctx.lib.gh_conv2d_can_pool(probe):
+        assert ctx.lib.gh_conv2d_can_keep(probe) == 0
+        return
+    assert ctx.lib.gh_conv2d_can_keep(probe) == 1
+    x = synth.uniform(81, (B, C, H, W), -1, 1)
+    w = synth.he_normal(82, (F, C, 3, 3))
+    x.reshape(-1)[::53] = np.inf; x.reshape(-1)[7::59] = np.nan; x.reshape(-1)[3::31] = -0.0
+    mean, var = synth.normal(83, (F,), 0.0, 0.1), synth.uniform(84, (F,), 0.5, 1.5)
+    gamma, beta = synth.uniform(85, (F,), 0.5, 1.5), synth.normal(86, (F,), 0.0, 0.1)
+    for bn, act in ((None, "relu"), ((mean, var, gamma, beta), "leaky"), (None, None)):
+        held = [ctx.upload(x), ctx.upload(w)]
+        dbn = None
+        if bn is not None:
+            dbn = tuple(ctx.upload(a) for a in bn)
+            held += list(dbn)
+        dp = ctx.malloc(B * F * (oh // 2) * (ow // 2) * 4)
+        dz = ctx.malloc(B * F * oh * ow * 4)
+        held += [dp, dz]
+        ctx.run(D.cmd_fill(dp, B * F * (oh // 2) * (ow // 2), np.nan))
+        ctx.run(D.cmd_fill(dz, B * F * oh * ow, np.nan))
+        ctx.run(D.cmd_conv2d(held[0], held[1], dp, B, C, H, W, F, 3, 3, (pad, pad), act=act, alpha=0.1, bn=dbn,
+                             pool2=True, keep=dz))
+        p = ctx.d2h(dp, (B, F, oh // 2, ow // 2))
+        z = ctx.d2h(dz, (B, F, oh, ow))
+        for q in held:
+            ctx.free(q)
+        assert_bits_equal(z, gpu_conv_tail(ctx, x, w, (pad, pad), bn=bn), f"kept result {cfg} bn={bn is not None}")
+        assert_bits_equal(p, gpu_conv_tail(ctx, x, w, (pad, pad), bn=bn, act=act, alpha=0.1, pool2=True),
+                          f"pooled result next to a kept one {cfg} act={act}")
+
+
 # shapes the patch kernel takes (3x3, 64 channels or more, K split over eight wavefronts): partial
 # patches on both axes, ragged filter tiles, no padding, pooled extents odd and even
 PATCH_CASES = [(2, 64, 20, 17, 40, 1), (2, 64, 28, 28, 32, 1), (1, 64, 24, 14, 20, 0), (1, 96, 26, 26, 48, 1), (3, 128, 13, 13, 70, 1), (1, 64, 31, 18, 16, 0),

@@ -53,12 +53,14 @@ def test_training_step_with_folded_operators_keeps_every_bit(ctx):
         m0 = G.NewTapeMachine(g0)
         g1, outs1 = configs.build_convnet_train(inp, y, 0.05)
         m1 = G.NewTapeMachine(g1, fuse_activations=True, graph_replay=replay)
-        assert m1.fused == 7           # 3 x (Rectify, MaxPool2DDiff) + the SoftMax
+        assert m1.fused == 10          # 3 x (Rectify, MaxPool2DDiff) + the SoftMax + 3 x (pool into its convolution)
         prog = m1.program()
-        assert prog.count("rectify+maxpool2d.diff") == 3 and prog.count("rectify+maxpool2d") == 6
+        assert prog.count("rectify+maxpool2d.diff") == 3
+        # every convolution stores its own result (the backward pass reads it) and the pooled activation
+        assert prog.count("conv2d(kept)+rectify+maxpool2d") == 3 and prog.count(" rectify+maxpool2d ") == 0
         assert prog.count("rectifyDiff") == 1       # the dense layer's activation is not pooled
         ops = lambda m: len([l for l in m.program().splitlines() if "execOp" in l])
-        assert ops(m1) == ops(m0) - 7
+        assert ops(m1) == ops(m0) - 10
         for step in range(3):
             m0.RunAll(); m1.RunAll()
             for k in outs0:
