@@ -157,6 +157,12 @@ def bench_elementwise(ctx, iters):
         total_ms += ms_cold
         total_ms_warm += ms_warm
         total_bytes += nbytes
+    # what a one-read-one-write kernel with no arithmetic at all reaches on the same rotating sets: the
+    # ceiling Sigmoid, Tanh and Pow2 (same traffic) are measured against
+    ms_neg = time_cmds(ctx, [D.cmd_unary("neg", xs[i], N, dst=ps[i]) for i in range(S)], passes) / S
+    no_arith = {"us": round(ms_neg * 1e3, 2), "GBps": round(2 * 4 * N / ms_neg / 1e6, 1),
+                "frac_hbm": round(2 * 4 * N / ms_neg / 1e6 / HBM_PEAK_GBPS, 4), "bytes": 2 * 4 * N,
+                "kernel": "Neg, same tensors and rotation as Sigmoid"}
     # the chain as configuration 2 issues it - five launches in order on one set of tensors
     # (x, y, z, t, p: 320 MiB, intermediates re-read straight after they were written)
     z, t, p = ys[1], ps[0], ps[1]
@@ -187,7 +193,7 @@ def bench_elementwise(ctx, iters):
             "chain_in_sequence_us": round(ms_seq * 1e3, 1), "chain_in_sequence_GBps": round(total_bytes / ms_seq / 1e6, 1),
             "streaming_8192": streaming, "operand_sets": S, "footprint_bytes": 3 * S * 4 * N,
             "device_copy_GBps": round(copy_gbps, 1), "device_copy_GBps_llc_assisted": round(copy_gbps_warm, 1),
-            "kernels": out}
+            "kernels": out, "one_read_one_write_without_arithmetic": no_arith}
 
 
 def bench_linalg(ctx, iters):
