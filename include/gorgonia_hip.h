@@ -321,7 +321,11 @@ GH_API int gh_conv2d_can_keep(const gh_cmd* conv);
  * function of its shape, its flags and (for the filter operand's alignment) its pointers: one of
  * GH_CONV_ROUTE_*, or -1 for a command that is no float32 CONV2D.  Host only.  The reference
  * leaves this choice to cuDNN (algorithm ImplicitGemm, ops/nn/convolution_cuda.go:111-117); here
- * the summing order, and with it the bits, belong to the kernel, so tests and callers can ask. */
+ * the summing order, and with it the bits, belong to the kernel, so tests and callers can ask.
+ * The three route queries take no context: where a launcher's choice depends on the number of
+ * compute units (the 1x1 kernel, the small-output product, the K slices of a product) they
+ * answer for 256 of them, the MI355X's count; on a device with another count gh_submit may
+ * choose differently there. */
 enum gh_conv_route {
   GH_CONV_ROUTE_DIRECT = 0,     /* 3x3, at most four channels: vector ALUs               */
   GH_CONV_ROUTE_SMALL = 1,      /* 3x3 over images up to 16 x 16, K split over wavefronts */
