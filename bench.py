@@ -752,8 +752,10 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "convnet forward, float32 NCHW batch 128x1x28x28 (config 4): "
                                "3x[Conv2d 3x3 pad1 + ReLU + MaxPool 2x2] -> Dense 625 ReLU -> Dense 10 SoftMax; "
-                               "tape machine, one segment, run the quicker of plain submits and hipGraph replay "
-                               "(timed by the machine on its first runs), weights and input resident",
+                               "tape machine, one segment of four commands (layers 0 and 1 folded into one), submitted "
+                               "plainly - segments of five commands and more run the quicker of plain submits and "
+                               "hipGraph replay, timed by the machine on its first runs; weights and input resident, "
+                               "every step ends with the output on the host",
                    "batch": 128, "flop_per_step": 2_093_410_816},
         "roofline": roofline,
         "cpu_baseline": cpu,
