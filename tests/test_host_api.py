@@ -294,6 +294,33 @@ def test_pooled_rectify_is_folded_only_when_nothing_else_reads_it():
         m.Close()
 
 
+def test_pool_is_folded_into_a_convolution_whose_result_is_kept():
+    """Graph::fuse_kept_conv: where a convolution's result has other readers than its 2x2 pool (a backward pass,
+    a host read) and the kernel for the shape stores both, the pool's node runs the convolution and the
+    convolution's node keeps its register without an instruction; not when something reads the result in
+    between, and not for shapes whose kernel cannot keep it."""
+    def build(C=32, between=False):
+        g = G.NewGraph()
+        x = G.NewTensor(g, np.zeros((2, C, 8, 8), np.float32))
+        w = G.NewTensor(g, np.zeros((16, C, 3, 3), np.float32), resident=True)
+        z = G.Conv2d(x, w, (3, 3), (1, 1), (1, 1), (1, 1))
+        if between:
+            G.Read(G.Rectify(z))
+        p = G.MaxPool2D(z, (2, 2), (0, 0), (2, 2))
+        G.Read(p)
+        G.Read(z)
+        return g
+    m = G.NewTapeMachine(build(), compile_only=True, fuse_activations=True)
+    prog = m.program()
+    assert m.fused == 1 and prog.count("conv2d(kept)+maxpool2d") == 1 and prog.count("execOp") == 1, prog
+    assert "alloc node 2" in prog and "execOp node 2" not in prog and "execOp node 3" in prog   # z: a register, no instruction
+    m.Close()
+    for kw in (dict(between=True), dict(C=3)):
+        m = G.NewTapeMachine(build(**kw), compile_only=True, fuse_activations=True)
+        assert "conv2d(kept)" not in m.program() and " maxpool2d" in m.program(), kw
+        m.Close()
+
+
 def test_pooling_query_over_random_geometries():
     """gh_conv2d_can_pool runs every 3x3 kernel's planner on the host.  Over a few thousand random
     geometries (channel counts around every kernel's limits, images from 3x3 to 500x500) it must
