@@ -346,8 +346,7 @@ def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=Tr
     eng = m.engine()
     eng.DoWork()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        m.RunAll()
+    m.RunAllN(steps)   # the steps back to back as a compiled caller would issue them
     eng.DoWork()
     dt = time.perf_counter() - t0
     result = out.copy()
@@ -378,8 +377,7 @@ def bench_convnet_machines(steps, warmup, count=2, batch=128):
 
     def loop(m):
         gate.wait()
-        for _ in range(steps):
-            m.RunAll()
+        m.RunAllN(steps)
         gate.wait()
 
     threads = [threading.Thread(target=loop, args=(m,)) for _, m, _ in machines]
@@ -415,8 +413,7 @@ def bench_yolo(steps, warmup, resident_input=True, borrow_output=True, borrow_in
     eng = m.engine()
     eng.DoWork()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        m.RunAll()
+    m.RunAllN(steps)   # the steps back to back as a compiled caller would issue them
     eng.DoWork()
     dt = time.perf_counter() - t0
     result = (m.value(outs["out"]) if borrow_output else outs["out"]).copy()
@@ -439,8 +436,7 @@ def bench_mlp(steps, warmup, resident_input=True):
     eng = m.engine()
     eng.DoWork()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        m.RunAll()
+    m.RunAllN(steps)   # the steps back to back as a compiled caller would issue them
     eng.DoWork()
     dt = time.perf_counter() - t0
     result = outs["out"].copy()
@@ -464,8 +460,7 @@ def bench_convnet_train(steps, warmup, batch=128, dtype=np.float32):
     eng = m.engine()
     eng.DoWork()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        m.RunAll()
+    m.RunAllN(steps)   # the steps back to back as a compiled caller would issue them
     eng.DoWork()
     dt = time.perf_counter() - t0
     VERDICTS["convnet_train" + ("_f64" if dtype == np.float64 else "")] = m.segment_verdict()

@@ -357,6 +357,10 @@ class TapeMachine:
     def RunAll(self):
         self._check(self.lib.ghh_tape_run_all(self.h))
 
+    def RunAllN(self, n):
+        """n RunAll calls in one call into the library (no interpreter between the steps)."""
+        self._check(self.lib.ghh_tape_run_all_n(self.h, int(n)))
+
     def Reset(self):
         self._check(self.lib.ghh_tape_reset(self.h))
 

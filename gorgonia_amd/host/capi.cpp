@@ -258,6 +258,13 @@ const char* ghh_tape_last_error(ghh_tape* t) { return t->err.c_str(); }
 int ghh_tape_init(ghh_tape* t, int device) { return ret(t, t->t->Init(device)); }
 int ghh_tape_compile_only(ghh_tape* t) { return ret(t, t->t->Compile()); }
 int ghh_tape_run_all(ghh_tape* t) { return ret(t, t->t->RunAll()); }
+int ghh_tape_run_all_n(ghh_tape* t, int n) {
+  for (int i = 0; i < n; i++) {
+    const int rc = ret(t, t->t->RunAll());
+    if (rc) return rc;
+  }
+  return 0;
+}
 int ghh_tape_reset(ghh_tape* t) { return ret(t, t->t->Reset()); }
 int ghh_tape_close(ghh_tape* t) { return ret(t, t->t->Close()); }
 int64_t ghh_tape_gpumem(ghh_tape* t) { return t->t->GpuMem(); }

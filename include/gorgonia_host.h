@@ -160,6 +160,10 @@ GH_API void ghh_tape_destroy(ghh_tape* t);
 GH_API const char* ghh_tape_last_error(ghh_tape* t);
 GH_API int ghh_tape_init(ghh_tape* t, int device);   /* compile + engine init */
 GH_API int ghh_tape_run_all(ghh_tape* t);            /* RunAll */
+/* n RunAll calls one after the other, stopping at the first error: the loop of a compiled caller
+ * (`for i := 0; i < n; i++ { vm.RunAll(); vm.Reset() }`, cuda_test.go:125-141) without an
+ * interpreter's call overhead between the steps; every step still ends with its results on the host. */
+GH_API int ghh_tape_run_all_n(ghh_tape* t, int n);
 GH_API int ghh_tape_reset(ghh_tape* t);              /* Reset */
 GH_API int ghh_tape_close(ghh_tape* t);
 GH_API int64_t ghh_tape_gpumem(ghh_tape* t);
