@@ -329,7 +329,7 @@ def test_pooling_query_over_random_geometries():
     from gorgonia_amd import _ffi, device as D
     lib = _ffi.load()
     rng = np.random.default_rng(123)
-    yes = 0
+    yes = kept = folded = 0
     for it in range(4000):
         B = int(rng.choice([1, 2, 3, 8, 16, 128, 130]))
         C = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 24, 32, 48, 64, 96, 128, 256, 512, 1000]))
@@ -355,4 +355,15 @@ def test_pooling_query_over_random_geometries():
         f64 = D.cmd_conv2d(0x1000, 0x2000, 0x3000, B, C, H, W, F, k, k, (pad, pad), (stride, stride), (dil, dil),
                            dtype=_ffi.F64)
         assert lib.gh_conv2d_can_pool(f64) == 0
-    assert yes > 300
+        # the folds that only the small-image kernels offer: a kept result goes with a pool, a folded first layer
+        # with 32 channels on small images; both queries answer without a device and never for float64
+        keep, pre = lib.gh_conv2d_can_keep(cmd), lib.gh_conv2d_can_pre(cmd)
+        assert keep in (0, 1) and pre in (0, 1)
+        if keep:
+            kept += 1
+            assert a == 1 and C in (1, 32, 64) and H <= 64 and W <= 64, (B, C, H, W, F, k, pad, stride, dil)
+        if pre:
+            folded += 1
+            assert C == 32 and k == 3 and stride == 1 and dil == 1 and pad <= 1 and 4 <= W <= 16 and H <= 16, (B, C, H, W, F, pad)
+        assert lib.gh_conv2d_can_keep(f64) == 0 and lib.gh_conv2d_can_pre(f64) == 0
+    assert yes > 300 and kept > 20 and folded > 5, (yes, kept, folded)
