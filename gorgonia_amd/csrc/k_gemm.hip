@@ -2700,9 +2700,20 @@ static int try_launch_gemm_skinny(gh_ctx* ctx, const gh_cmd& c) {
       hipLaunchKernelGGL(kernel, dim3((N + bn - 1) / bn, (M + 15) / 16), dim3(WV * 64), 0, ctx->stream, A, B, C, M,
                          N, K, lda, ldb, ldc, act, c.f[0], bias, softmax);
     };
+    // Sixteen wavefronts share the K of a long contraction (a function of the shape alone, like the tile): each
+    // wavefront's chain of grouped loads is half as long (measured: 128x1152x625 7.8 -> 7.2 us, 256x784x300
+    // 5.8 -> 5.3, 128x625x10 4.3 -> 4.1; nothing below K = 512, where a wavefront has four chunks or fewer).
+    static const bool no16 = getenv("GORGONIA_HIP_SKINNY_WAVES8") != nullptr;   // tuning switch
+    const bool wide16 = K >= 512 && !no16;
+    auto launch16w = [&](auto kernel, int bn) {
+      hipLaunchKernelGGL(kernel, dim3((N + bn - 1) / bn, (M + 15) / 16), dim3(16 * 64), 0, ctx->stream, A, B, C, M,
+                         N, K, lda, ldb, ldc, act, c.f[0], bias, softmax);
+    };
 #define GH_SKINNY16(TA_, TB_)                                                               \
   do {                                                                                      \
-    if (narrow) launch16(k_gemm_skinny16<WV, 1, TA_, TB_>, 16);                             \
+    if (wide16 && !narrow) launch16w(k_gemm_skinny16<16, 2, TA_, TB_>, 32);                 \
+    else if (wide16) launch16w(k_gemm_skinny16<16, 1, TA_, TB_>, 16);                       \
+    else if (narrow) launch16(k_gemm_skinny16<WV, 1, TA_, TB_>, 16);                        \
     else launch16(k_gemm_skinny16<WV, 2, TA_, TB_>, 32);                                    \
   } while (0)
     if (ta) GH_SKINNY16(true, false);
