@@ -26,6 +26,7 @@
 //   * The prologue is kept short (a wavefront's instructions are time the matrix pipe stands idle
 //     for all eight): buffer loads whose descriptors' ranges stand for the bounds tests, every
 //     staging address a per-lane constant plus an immediate.
+#include <cstdio>
 #include <cstdlib>
 #include <mutex>
 
@@ -550,7 +551,12 @@ bool rows_plan_compute(const gh_cmd& c, bool pool, RowsPlan* out) {
       // layers: 32 filters x 1 image against 16 x 2 at 14 x 14, 16 x 4 against 32 x 2 at 7 x 7)
       const double stage_us = 2.0 + 0.035 * (TFB * NQ * 576 * 4 / 1024.0) + 0.03 * ((double)IPB * NQ * g.QP * 4 / 1024.0);
       const double est = rounds * (stage_us + coresident * mfma_us);
-      if (!bestTFB || est < best) { best = est; bestTFB = TFB; bestIPB = IPB; }
+      double score = est;
+      if (const char* e = getenv("GORGONIA_HIP_CONV_ROWS_PLAN")) {   // tuning override: "TFB,IPB"
+        int ft = 0, ip = 0;
+        if (sscanf(e, "%d,%d", &ft, &ip) == 2 && ft == TFB && ip == IPB) score = -1.0;
+      }
+      if (!bestTFB || score < best) { best = score; bestTFB = TFB; bestIPB = IPB; }
     }
   }
   if (!bestTFB) return false;
