@@ -140,7 +140,8 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       if (c.dim[0] * c.dim[1] * c.dim[2] * c.dim[3] > INT32_MAX)
         return bad("maxpool2d: tensor too large for 32-bit indexing");
       if (dt > GH_F64) return bad("Unsupported Dtype");
-      if (dt == GH_F64 && (c.flags & GH_FLAG_ACT_RELU)) return bad("maxpool2d: no Rectify on the input for float64");
+      if (dt == GH_F64 && (c.flags & GH_FLAG_ACT_RELU) && c.opcode == GH_OP_MAXPOOL2D_BWD)
+        return bad("maxpool2d gradient: no Rectify on the input for float64");
       return GH_OK;
     }
     case GH_OP_BN_INFER:

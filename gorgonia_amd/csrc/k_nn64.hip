@@ -46,7 +46,9 @@ struct Pool64 {
 };
 
 // Reference scan: window clipped to the image, row-major, strict >, start
-// value -maxFloat64 (op_nn.go:916-950).
+// value -maxFloat64 (op_nn.go:916-950).  RELU: x is read through Rectify (x * (x >= 0), nn.go:136-163), whose
+// result is then never stored.
+template <bool RELU>
 __global__ __launch_bounds__(kBlock) void k_maxpool2d_f64(const double* __restrict__ x, double* __restrict__ y,
                                                           Pool64 g, int64_t total) {
   const int64_t stride = (int64_t)gridDim.x * kBlock;
@@ -63,7 +65,8 @@ __global__ __launch_bounds__(kBlock) void k_maxpool2d_f64(const double* __restri
     double best = -DBL_MAX;
     for (int hi = hs; hi < he; hi++)
       for (int wi = ws; wi < we; wi++) {
-        const double v = in[hi * g.W + wi];
+        double v = in[hi * g.W + wi];
+        if constexpr (RELU) v = v * (v >= 0.0 ? 1.0 : 0.0);
         if (v > best) best = v;
       }
     y[i] = best;
@@ -246,8 +249,12 @@ int gh_launch_maxpool2d_f64(gh_ctx* ctx, const gh_cmd& c) {
   g.padW = (int)(explicit_pad ? padE : padW);
   const int64_t total = B * C * g.oh * g.ow;
   if (total <= 0) return GH_OK;
-  hipLaunchKernelGGL(k_maxpool2d_f64, dim3(blocks_for(ctx, total)), dim3(kBlock), 0, ctx->stream,
-                     (const double*)(uintptr_t)c.ptr[0], (double*)(uintptr_t)c.ptr[1], g, total);
+  if (c.flags & GH_FLAG_ACT_RELU)
+    hipLaunchKernelGGL(k_maxpool2d_f64<true>, dim3(blocks_for(ctx, total)), dim3(kBlock), 0, ctx->stream,
+                       (const double*)(uintptr_t)c.ptr[0], (double*)(uintptr_t)c.ptr[1], g, total);
+  else
+    hipLaunchKernelGGL(k_maxpool2d_f64<false>, dim3(blocks_for(ctx, total)), dim3(kBlock), 0, ctx->stream,
+                       (const double*)(uintptr_t)c.ptr[0], (double*)(uintptr_t)c.ptr[1], g, total);
   return gh_check_hip(ctx, hipGetLastError(), "maxpool2d launch");
 }
 

@@ -739,6 +739,7 @@ int Graph::FuseActivations() {
     p.fused_away = true;
     fused++;
   }
+  fused += fuse_rectify_into_pool();
   fused += fuse_pooled_rectify();
   fused += fuse_first_layer();
   fused += fuse_kept_conv();
@@ -785,6 +786,28 @@ int Graph::fuse_kept_conv() {
     pn.op = op;
     pn.inputs = {z.inputs[0], z.inputs[1], z.id};
     z.deferred = true;
+    fused++;
+  }
+  return fused;
+}
+
+// p = MaxPool2D(Rectify(z)) where nothing else reads the activation and no producer took it into an epilogue
+// (a float64 convolution has none): the pool reads z through the activation, whose result is never stored.
+// The pooled values are those of the two operators: the same scan over the same x * (x >= 0).
+int Graph::fuse_rectify_into_pool() {
+  int fused = 0;
+  std::vector<int> uses(nodes_.size(), 0);
+  for (auto& n : nodes_)
+    if (!n.fused_away) for (int i : n.inputs) uses[(size_t)i]++;
+  for (auto& pn : nodes_) {
+    if (pn.is_input || pn.fused_away || pn.op.kind != OpKind::MaxPool2D || pn.inputs.size() != 1 || pn.op.relu_input) continue;
+    Node& a = nodes_[(size_t)pn.inputs[0]];
+    if (a.is_input || a.fused_away || a.deferred || a.read_into || a.alias_of >= 0 || uses[(size_t)a.id] != 1) continue;
+    if (a.op.kind != OpKind::Rectify || a.inputs.size() != 1) continue;
+    if (a.dt != Dtype::Float32 && a.dt != Dtype::Float64) continue;
+    pn.inputs[0] = a.inputs[0];
+    pn.op.relu_input = true;
+    a.fused_away = true;
     fused++;
   }
   return fused;

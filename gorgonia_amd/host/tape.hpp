@@ -139,6 +139,7 @@ class Graph {
   int FuseActivations();
   int fuse_pooled_rectify();   // part of FuseActivations: the Rectify between a pool and both gradients
   int fuse_first_layer();      // part of FuseActivations: a single-channel first layer folded into the next convolution
+  int fuse_rectify_into_pool();   // part of FuseActivations: a Rectify read by nothing but a pool (float64 convolutions have no epilogue)
   int fuse_kept_conv();        // part of FuseActivations: a pool into the convolution whose result other nodes read too
   const std::vector<Node>& Nodes() const { return nodes_; }
   std::vector<Node>& Nodes() { return nodes_; }

@@ -183,7 +183,7 @@ enum gh_unaryfn {
  *             needed and never stored; y holds the bits the three commands would give
  * MAXPOOL2D   ptr[0]=x ptr[1]=y            dim[0..3]=B,C,H,W dim[4..5]=kh,kw
  *             dim[6..9]=padN,padS,padW,padE dim[10..11]=strideH,strideW
- *             GH_FLAG_ACT_RELU (float32): x is read through Rectify, y = pool(x*(x>=0));
+ *             GH_FLAG_ACT_RELU: x is read through Rectify, y = pool(x*(x>=0));
  *             the activation's result is never stored
  * BN_INFER    ptr[0]=x ptr[1]=y ptr[2]=mean ptr[3]=var [ptr[4]=gamma ptr[5]=beta]
  *             dim[0..2]=B,C,S  f[0]=eps

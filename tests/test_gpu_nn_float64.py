@@ -103,6 +103,17 @@ def test_maxpool_float64_bit_exact(ctx, cfg):
     got = ctx.d2h(dy, want.shape, np.float64)
     ctx.free(dx); ctx.free(dy)
     assert_bits_equal(got, want, f"float64 maxpool {cfg}")
+    # the same pool reading its input through Rectify: the bits of the two operators, the activation never stored
+    xs = x.copy()
+    xs.reshape(-1)[5::13] = np.inf; xs.reshape(-1)[9::17] = -np.inf; xs.reshape(-1)[1::19] = np.nan
+    want = O.maxpool2d(O.relu(xs).reshape(xs.shape), kernel, pad, stride)
+    dx, dy = ctx.upload(xs), ctx.malloc(want.size * 8)
+    cmd = D.cmd_maxpool2d(dx, dy, B, C, H, W, kernel[0], kernel[1], pad, stride, dtype=F64)
+    cmd.flags |= _ffi.FLAG_ACT_RELU
+    ctx.run(cmd)
+    got = ctx.d2h(dy, want.shape, np.float64)
+    ctx.free(dx); ctx.free(dy)
+    assert_bits_equal(got, want, f"float64 rectify+maxpool {cfg}")
 
 
 @pytest.mark.parametrize("shape", [(4, 6), (2, 5, 7, 3)])
@@ -177,6 +188,25 @@ def test_tape_float64_network(ctx):
     want = O.softmax(ref.reshape(2, 64) @ w2)
     assert np.allclose(out, want, rtol=1e-12, atol=1e-15)
     m.Close()
+
+
+def test_tape_float64_convnet_folds_rectify_into_pool(ctx):
+    """The convnet in float64 (the reference example's default dtype, examples/convnet/main.go:28): the
+    convolutions have no epilogue there, so FuseActivations lets each pool read through the Rectify in front
+    of it; the output keeps the bits of the unfolded machine."""
+    from gorgonia_amd import configs
+    inp = {k: v.astype(np.float64) for k, v in configs.convnet_inputs(8).items()}
+    outs = []
+    for fuse in (False, True):
+        g, o = configs.build_convnet(inp)
+        m = G.NewTapeMachine(g, fuse_activations=fuse)
+        if fuse:
+            assert m.fused == 3 and m.program().count("rectify+maxpool2d") == 3, m.program()
+        m.RunAll()
+        outs.append(o["out"].copy())
+        m.Close()
+    assert outs[0].dtype == np.float64
+    assert_bits_equal(outs[1], outs[0], "float64 convnet, Rectify folded into the pools")
 
 
 def test_conv2d_float64_seeded_geometry_sweep(ctx):
