@@ -36,7 +36,7 @@ int gh_validate_cmd(const gh_cmd& c, std::string& msg) {
       return GH_OK;
     case GH_OP_BCAST_BIN:
       if (fn >= GH_BINFN__COUNT) { msg = "unknown binary function"; return GH_ENOFUNC; }
-      if (dt != GH_F32) return bad("broadcast ops are float32 only");
+      if (dt > GH_F64) return bad("Unsupported Dtype");
       if (!c.ptr[0] || !c.ptr[1] || !c.ptr[2]) return bad("null operand");
       if (c.dim[0] < 0 || c.dim[1] <= 0 || c.dim[2] <= 0) return bad("bad broadcast shape");
       return GH_OK;

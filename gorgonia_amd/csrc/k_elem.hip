@@ -408,14 +408,15 @@ __global__ __launch_bounds__(kBlock) void k_unary_scalar(const T* A, T* D, int64
 
 // ---- fused broadcast --------------------------------------------------------
 // dst[o,m,i] = big[o,m,i] op small[m]  (or small op big with SMALL_LEFT).
-// Row form (inner == 1, mid % 4 == 0): each thread owns one float4 column
-// group, keeps its slice of `small` in registers and walks rows.
-template <int FN, bool LEFT, bool STREAM>
-__global__ __launch_bounds__(kBlock) void k_bcast_row(float* __restrict__ dst,
-                                                      const float* __restrict__ big,
-                                                      const float* __restrict__ small,
+// Row form (inner == 1, mid a multiple of the vector width): each thread owns one 128-bit
+// column group, keeps its slice of `small` in registers and walks rows.
+template <int FN, class T, bool LEFT, bool STREAM>
+__global__ __launch_bounds__(kBlock) void k_bcast_row(T* __restrict__ dst,
+                                                      const T* __restrict__ big,
+                                                      const T* __restrict__ small,
                                                       int64_t rows, int64_t colv) {
-  typedef float V __attribute__((ext_vector_type(4)));
+  typedef typename VecOf<T>::type V;
+  constexpr int N = VecOf<T>::N;
   const int64_t cv = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (cv >= colv) return;
   const V s = reinterpret_cast<const V*>(small)[cv];
@@ -424,7 +425,7 @@ __global__ __launch_bounds__(kBlock) void k_bcast_row(float* __restrict__ dst,
   auto apply = [&](V a) {
     V o;
 #pragma unroll
-    for (int e = 0; e < 4; e++) o[e] = LEFT ? bin_apply<FN, float>(s[e], a[e]) : bin_apply<FN, float>(a[e], s[e]);
+    for (int e = 0; e < N; e++) o[e] = LEFT ? bin_apply<FN, T>(s[e], a[e]) : bin_apply<FN, T>(a[e], s[e]);
     return o;
   };
   // a workgroup takes kUnroll adjacent rows per step
@@ -443,15 +444,15 @@ __global__ __launch_bounds__(kBlock) void k_bcast_row(float* __restrict__ dst,
 }
 
 // General form: one element per thread, small index = (idx / inner) % mid.
-template <int FN, bool LEFT>
-__global__ __launch_bounds__(kBlock) void k_bcast_generic(float* dst, const float* big,
-                                                          const float* small, int64_t n,
+template <int FN, class T, bool LEFT>
+__global__ __launch_bounds__(kBlock) void k_bcast_generic(T* dst, const T* big,
+                                                          const T* small, int64_t n,
                                                           int64_t mid, int64_t inner) {
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
-    const float s = small[(i / inner) % mid];
-    const float a = big[i];
-    dst[i] = LEFT ? bin_apply<FN, float>(s, a) : bin_apply<FN, float>(a, s);
+    const T s = small[(i / inner) % mid];
+    const T a = big[i];
+    dst[i] = LEFT ? bin_apply<FN, T>(s, a) : bin_apply<FN, T>(a, s);
   }
 }
 
@@ -675,30 +676,32 @@ int launch_unary(gh_ctx* ctx, const gh_cmd& c) {
   return gh_fail(ctx, GH_ENOFUNC, "unknown unary function");
 }
 
-template <int FN>
+template <int FN, class T>
 int launch_bcast_fn(gh_ctx* ctx, const gh_cmd& c) {
-  float* dst = (float*)(uintptr_t)c.ptr[0];
-  const float* big = (const float*)(uintptr_t)c.ptr[1];
-  const float* small = (const float*)(uintptr_t)c.ptr[2];
+  T* dst = (T*)(uintptr_t)c.ptr[0];
+  const T* big = (const T*)(uintptr_t)c.ptr[1];
+  const T* small = (const T*)(uintptr_t)c.ptr[2];
+  constexpr int N = VecOf<T>::N;
   const int64_t outer = c.dim[0], mid = c.dim[1], inner = c.dim[2];
   const int64_t n = outer * mid * inner;
+  const int64_t tbytes = (int64_t)sizeof(T) * n;
   const bool left = c.flags & GH_FLAG_SMALL_LEFT;
   if (n == 0) return GH_OK;
-  const bool row = inner == 1 && (mid % 4) == 0 && aligned16(c.ptr[0]) && aligned16(c.ptr[1]) &&
+  const bool row = inner == 1 && (mid % N) == 0 && aligned16(c.ptr[0]) && aligned16(c.ptr[1]) &&
                    aligned16(c.ptr[2]);
   if (row) {
-    const int64_t colv = mid / 4;
+    const int64_t colv = mid / N;
     const int gx = (int)((colv + kBlock - 1) / kBlock);
     int64_t gy = ((int64_t)ctx->cu_count * 16 + gx - 1) / gx;
     const int64_t need = (outer + kUnroll - 1) / kUnroll;
     if (gy > need) gy = need;
     if (gy < 1) gy = 1;
     if (gy > 65535) gy = 65535;
-    const bool stream = stream_bytes(8 * n) || cold_inputs(ctx, 8 * n, c.ptr[1], 0);
-    ctx->llc.touch(c.ptr[1], 4 * n, true);
-    ctx->llc.touch(c.ptr[0], 4 * n, c.ptr[0] != c.ptr[1]);
-#define GH_BCAST_ROW(L_, S_)                                                                              \
-  hipLaunchKernelGGL((k_bcast_row<FN, L_, S_>), dim3(gx, (int)gy), dim3(kBlock), 0, ctx->stream, dst, big, \
+    const bool stream = stream_bytes(2 * tbytes) || cold_inputs(ctx, 2 * tbytes, c.ptr[1], 0);
+    ctx->llc.touch(c.ptr[1], tbytes, true);
+    ctx->llc.touch(c.ptr[0], tbytes, c.ptr[0] != c.ptr[1]);
+#define GH_BCAST_ROW(L_, S_)                                                                                 \
+  hipLaunchKernelGGL((k_bcast_row<FN, T, L_, S_>), dim3(gx, (int)gy), dim3(kBlock), 0, ctx->stream, dst, big, \
                      small, outer, colv)
     if (left) { if (stream) GH_BCAST_ROW(true, true); else GH_BCAST_ROW(true, false); }
     else { if (stream) GH_BCAST_ROW(false, true); else GH_BCAST_ROW(false, false); }
@@ -706,13 +709,32 @@ int launch_bcast_fn(gh_ctx* ctx, const gh_cmd& c) {
   } else {
     const int g = grid_for(ctx, n, 4);
     if (left)
-      hipLaunchKernelGGL((k_bcast_generic<FN, true>), dim3(g), dim3(kBlock), 0, ctx->stream, dst, big,
+      hipLaunchKernelGGL((k_bcast_generic<FN, T, true>), dim3(g), dim3(kBlock), 0, ctx->stream, dst, big,
                          small, n, mid, inner);
     else
-      hipLaunchKernelGGL((k_bcast_generic<FN, false>), dim3(g), dim3(kBlock), 0, ctx->stream, dst, big,
+      hipLaunchKernelGGL((k_bcast_generic<FN, T, false>), dim3(g), dim3(kBlock), 0, ctx->stream, dst, big,
                          small, n, mid, inner);
   }
   return gh_check_hip(ctx, hipGetLastError(), "broadcast launch");
+}
+
+template <class T>
+int launch_bcast(gh_ctx* ctx, const gh_cmd& c) {
+  switch (gh_fn(c.flags)) {
+    case GH_ADD: return launch_bcast_fn<GH_ADD, T>(ctx, c);
+    case GH_SUB: return launch_bcast_fn<GH_SUB, T>(ctx, c);
+    case GH_MUL: return launch_bcast_fn<GH_MUL, T>(ctx, c);
+    case GH_DIV: return launch_bcast_fn<GH_DIV, T>(ctx, c);
+    case GH_POW: return launch_bcast_fn<GH_POW, T>(ctx, c);
+    case GH_LT: return launch_bcast_fn<GH_LT, T>(ctx, c);
+    case GH_LTE: return launch_bcast_fn<GH_LTE, T>(ctx, c);
+    case GH_GT: return launch_bcast_fn<GH_GT, T>(ctx, c);
+    case GH_GTE: return launch_bcast_fn<GH_GTE, T>(ctx, c);
+    case GH_EQ: return launch_bcast_fn<GH_EQ, T>(ctx, c);
+    case GH_NE: return launch_bcast_fn<GH_NE, T>(ctx, c);
+    case GH_MOD: return launch_bcast_fn<GH_MOD, T>(ctx, c);
+  }
+  return gh_fail(ctx, GH_ENOFUNC, "unknown binary function");
 }
 
 }  // namespace
@@ -726,21 +748,7 @@ int gh_launch_elem_unary(gh_ctx* ctx, const gh_cmd& c) {
 }
 
 int gh_launch_bcast_bin(gh_ctx* ctx, const gh_cmd& c) {
-  switch (gh_fn(c.flags)) {
-    case GH_ADD: return launch_bcast_fn<GH_ADD>(ctx, c);
-    case GH_SUB: return launch_bcast_fn<GH_SUB>(ctx, c);
-    case GH_MUL: return launch_bcast_fn<GH_MUL>(ctx, c);
-    case GH_DIV: return launch_bcast_fn<GH_DIV>(ctx, c);
-    case GH_POW: return launch_bcast_fn<GH_POW>(ctx, c);
-    case GH_LT: return launch_bcast_fn<GH_LT>(ctx, c);
-    case GH_LTE: return launch_bcast_fn<GH_LTE>(ctx, c);
-    case GH_GT: return launch_bcast_fn<GH_GT>(ctx, c);
-    case GH_GTE: return launch_bcast_fn<GH_GTE>(ctx, c);
-    case GH_EQ: return launch_bcast_fn<GH_EQ>(ctx, c);
-    case GH_NE: return launch_bcast_fn<GH_NE>(ctx, c);
-    case GH_MOD: return launch_bcast_fn<GH_MOD>(ctx, c);
-  }
-  return gh_fail(ctx, GH_ENOFUNC, "unknown binary function");
+  return gh_dtype_of(c.flags) == GH_F64 ? launch_bcast<double>(ctx, c) : launch_bcast<float>(ctx, c);
 }
 
 int gh_launch_relu(gh_ctx* ctx, const gh_cmd& c) {

@@ -152,8 +152,8 @@ def cmd_unary(fn, a, n, dtype=_ffi.F32, dst=0):
     return make_cmd(_ffi.OP_ELEM_UNARY, fl, (a, dst), (n,))
 
 
-def cmd_bcast(fn, dst, big, small, outer, mid, inner, small_left=False):
-    fl = _ffi.flag_fn(_ffi.BIN_FN[fn]) | (_ffi.FLAG_SMALL_LEFT if small_left else 0)
+def cmd_bcast(fn, dst, big, small, outer, mid, inner, small_left=False, dtype=_ffi.F32):
+    fl = _ffi.flag_fn(_ffi.BIN_FN[fn]) | _ffi.flag_dtype(dtype) | (_ffi.FLAG_SMALL_LEFT if small_left else 0)
     return make_cmd(_ffi.OP_BCAST_BIN, fl, (dst, big, small), (outer, mid, inner))
 
 

@@ -322,13 +322,12 @@ Status Engine::UnaryTo(const std::string& op_name, Tensor& a, uint64_t dst_mem) 
 Status Engine::BroadcastBinOp(int fn, Tensor& big, Tensor& small, int64_t outer, int64_t mid,
                               int64_t inner, bool small_left, uint64_t dst_mem) {
   if (fn < 0 || fn >= GH_BINFN__COUNT) return Status::Err(GH_ENOFUNC, "unknown binary function");
-  if (big.dt != Dtype::Float32 || small.dt != Dtype::Float32)
-    return Status::Err(GH_EINVAL, "Unsupported Dtype for broadcast");
+  if (big.dt != small.dt) return Status::Err(GH_EINVAL, "broadcast: operands of different Dtypes");
   if (big.DataSize() != outer * mid * inner || small.DataSize() != mid)
     return Status::Err(GH_EINVAL, fmt2(kShapeMismatch, big.shape.String(), small.shape.String()));
   gh_cmd c{};
   c.opcode = GH_OP_BCAST_BIN;
-  c.flags = GH_FLAG_FN(fn) | (small_left ? GH_FLAG_SMALL_LEFT : 0);
+  c.flags = GH_FLAG_FN(fn) | GH_FLAG_DTYPE(big.dt == Dtype::Float64 ? GH_F64 : GH_F32) | (small_left ? GH_FLAG_SMALL_LEFT : 0);
   c.ptr[0] = dst_mem; c.ptr[1] = big.mem; c.ptr[2] = small.mem;
   c.dim[0] = outer; c.dim[1] = mid; c.dim[2] = inner;
   Enqueue(c);

@@ -652,8 +652,14 @@ Status Graph::LetBorrowed(int node) {
 
 Status Graph::Read(int node, void* host_out) {
   if (node < 0 || node >= (int)nodes_.size()) return bad("Read: unknown node");
-  nodes_[(size_t)node].read_into = host_out;
-  nodes_[(size_t)node].read_borrowed = false;
+  Node& n = nodes_[(size_t)node];
+  if (n.read_into && host_out != n.read_into) {   // a node may be read more than once (gorgonia.Read makes a readOp node per call, gorgonia.go:311-318)
+    if (n.read_borrowed) return bad("Read: the node's value is lent out (ReadBorrowed)");
+    n.read_also.push_back(host_out);
+    return Status::OK();
+  }
+  n.read_into = host_out;
+  n.read_borrowed = false;
   return Status::OK();
 }
 
@@ -661,6 +667,7 @@ Status Graph::ReadBorrowed(int node) {
   static char marker;   // read_into only has to be non-null: nothing is ever copied there
   if (node < 0 || node >= (int)nodes_.size()) return bad("ReadBorrowed: unknown node");
   Node& n = nodes_[(size_t)node];
+  if (n.read_into && !n.read_borrowed) return bad("ReadBorrowed: the node already has a Read");
   n.read_into = &marker;
   n.read_borrowed = true;
   return Status::OK();
@@ -1298,9 +1305,12 @@ Status TapeMachine::RunAll() {
           // the flush in front of the reads has waited for the staging copy; a borrowed
           // read is finished with that
           if (!n.read_borrowed) std::memcpy(n.read_into, stage_[(size_t)in.node], (size_t)in.size);
+          for (void* more : n.read_also) std::memcpy(more, stage_[(size_t)in.node], (size_t)in.size);
           break;
         }
         st = eng_.MemcpyDtoH(n.read_into, regs_[(size_t)in.reg].mem, in.size, false);
+        for (void* more : n.read_also)
+          if (st.ok()) st = eng_.MemcpyDtoH(more, regs_[(size_t)in.reg].mem, in.size, false);
         if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": read");
         bool last = pc + 1 >= prog_.size() || prog_[pc + 1].kind != InstrKind::Read;
         if (last) {

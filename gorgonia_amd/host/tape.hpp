@@ -112,6 +112,7 @@ struct Node {
   OpSpec op;
   std::vector<int> inputs;
   void* read_into = nullptr;      // Read(node, &host) target
+  std::vector<void*> read_also;   // further Reads of the same node: each gets the value too
   bool read_borrowed = false;     // ReadBorrowed: the value stays in the machine's own pinned buffer
   bool fused_away = false;        // absorbed into the follower that now computes both: no register, no instruction
   bool deferred = false;          // keeps its register, but a later node (which lists it as its last input) writes it: no instruction

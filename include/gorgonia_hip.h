@@ -147,7 +147,8 @@ enum gh_unaryfn {
  * ELEM_UNARY  ptr[0]=A [ptr[1]=dst]        dim[0]=n ; in place without dst
  * BCAST_BIN   ptr[0]=dst ptr[1]=big ptr[2]=small
  *             dim[0]=outer dim[1]=mid dim[2]=inner; small has `mid` elements,
- *             element (o,m,i) pairs big[o,m,i] with small[m]
+ *             element (o,m,i) pairs big[o,m,i] with small[m]; float32 or
+ *             float64 by the dtype field, both operands alike
  * MEMCPY_D2D  ptr[0]=dst ptr[1]=src        dim[0]=bytes
  *             either side may be pinned host memory from gh_host_alloc (the
  *             device reads or writes it over the bus): this is how a segment

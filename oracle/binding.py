@@ -59,11 +59,12 @@ def binop(fn, mode, a, b):
 
 
 def bcast_binop(fn, big, small, outer, mid, inner, small_left=False):
-    big = np.ascontiguousarray(big, dtype=np.float32)
-    small = np.ascontiguousarray(small, dtype=np.float32)
-    dst = np.empty(outer * mid * inner, dtype=np.float32)
-    lib().oracle_bcast_binop_f32(BIN[fn], int(small_left), _p(dst), _p(big), _p(small),
-                                 *_i64(outer, mid, inner))
+    dt = np.float64 if np.asarray(big).dtype == np.float64 else np.float32
+    big = np.ascontiguousarray(big, dtype=dt)
+    small = np.ascontiguousarray(small, dtype=dt)
+    dst = np.empty(outer * mid * inner, dtype=dt)
+    f = lib().oracle_bcast_binop_f64 if dt == np.float64 else lib().oracle_bcast_binop_f32
+    f(BIN[fn], int(small_left), _p(dst), _p(big), _p(small), *_i64(outer, mid, inner))
     return dst
 
 

@@ -192,6 +192,16 @@ EXPORT void oracle_bcast_binop_f32(int op, int small_left, float* dst, const flo
   free(rep);
 }
 
+EXPORT void oracle_bcast_binop_f64(int op, int small_left, double* dst, const double* big,
+                                   const double* small, int64_t outer, int64_t mid, int64_t inner) {
+  int64_t n = outer * mid * inner, i;
+  double* rep = (double*)malloc((size_t)(n > 0 ? n : 1) * sizeof(double));
+  for (i = 0; i < n; i++) rep[i] = small[(i / inner) % mid]; /* tensor.Repeat */
+  for (i = 0; i < n; i++)
+    dst[i] = small_left ? binop_f64(op, rep[i], big[i]) : binop_f64(op, big[i], rep[i]);
+  free(rep);
+}
+
 /* ------------------------------------------------------------------ */
 /* Unary ops, in place.  elemunaryop.cu:109-193 names; CPU semantics   */
 /* operatorPointwise_unary.go:30-101, math.go:13-68,                   */

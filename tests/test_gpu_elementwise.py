@@ -290,6 +290,22 @@ def test_broadcast_bit_exact(ctx, fn, shape, left):
     ctx.free(db); ctx.free(ds); ctx.free(dd)
 
 
+@pytest.mark.parametrize("fn", ["add", "mul", "sub", "div", "lt", "gte"])
+@pytest.mark.parametrize("shape", [(64, 4096, 1), (7, 13, 1), (8, 16, 169), (1, 4098, 1), (4097, 2, 1)])
+@pytest.mark.parametrize("left", [False, True])
+def test_broadcast_float64_bit_exact(ctx, fn, shape, left):
+    """The float64 twin: the same repeat-then-operate result (broadcast.go:69-129), one IEEE operation per element."""
+    outer, mid, inner = shape
+    big = synth.uniform(53, (outer * mid * inner,), -4, 4).astype(np.float64) + 2.0 ** -40
+    small = synth.uniform(54, (mid,), -4, 4).astype(np.float64) - 2.0 ** -41
+    db, ds = ctx.upload(big), ctx.upload(small)
+    dd = ctx.malloc(big.nbytes)
+    ctx.run(D.cmd_bcast(fn, dd, db, ds, outer, mid, inner, small_left=left, dtype=_ffi.F64))
+    got = ctx.d2h(dd, big.shape, np.float64)
+    assert_bits_equal(got, O.bcast_binop(fn, big, small, outer, mid, inner, left), f"bcast f64 {fn}")
+    ctx.free(db); ctx.free(ds); ctx.free(dd)
+
+
 def test_large_operands_cold_then_warm_same_bits(ctx):
     """Tensors of 32 MiB: the first launch finds them nowhere in the library's account of the
     last-level cache and streams them (non-temporal accesses), the repeat finds them there and

@@ -379,6 +379,26 @@ def test_measured_replay_keeps_results_and_settles(ctx, monkeypatch):
         m.Close()
 
 
+def test_a_node_read_twice_fills_both_values(ctx):
+    """gorgonia.Read makes a readOp node per call (gorgonia.go:311-318): two Reads of one node fill two values,
+    whether the value reaches the host through the staging copy of the segment or a copy after the flush."""
+    for n in (64, (9 << 20) // 4):
+        xv = synth.uniform(3, (n,), -2, 2)
+        for lisp in (False, True):
+            g = G.NewGraph()
+            y = G.Neg(G.NewTensor(g, xv))
+            a, b = G.Read(y), G.Read(y)
+            z = G.Read(G.Square(y))
+            m = G.NewLispMachine(g) if lisp else G.NewTapeMachine(g)
+            for _ in range(2):
+                a[...] = 0; b[...] = 0
+                m.RunAll()
+                assert_bits_equal(a, -xv, "first Read")
+                assert_bits_equal(b, -xv, "second Read")
+                assert_bits_equal(z, xv * xv, "a reader of the read value")
+            m.Close()
+
+
 def test_lisp_machine_differential(ctx):
     """The reference's main test pattern (nn_test.go:25-79, operatorPointwise_unary_test.go:14-95):
     one graph on the TapeMachine and on the LispMachine, equal values required.  Here the second
