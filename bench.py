@@ -137,8 +137,8 @@ def bench_elementwise(ctx, iters):
             return D.cmd_bin("mul", "vv", x, zs[i], N, dst=p)
         if name == "BroadcastAdd":
             return D.cmd_bcast("add", p, x, b, 4096, 4096, 1)
-        if name == "Sigmoid":
-            return D.cmd_unary("sigmoid", x, N, dst=p)
+        if name == "Sigmoid":   # in place, as the tape machine runs it in this chain: its operand x*y + b is dead
+            return D.cmd_unary("sigmoid", z, N)
         if name == "Tanh":
             return D.cmd_unary("tanh", z, N, dst=p)
         return D.cmd_bin("pow", "vs", z, two, N, dst=p)

@@ -524,34 +524,63 @@ def test_conv_wide_kernel(ctx, cfg):
 
 
 def test_conv_random_geometry_sweep(ctx):
-    """Seeded sweep over 3x3 and other geometries (all three convolution kernels, ragged sizes,
-    batch boundaries inside blocks): the plain convolution against the oracle, and wherever the
-    pool may ride in the epilogue, conv+ReLU+pool against the separate commands bit for bit."""
-    rng = np.random.default_rng(77)
-    pooled = 0
-    for case in range(36):
-        B = int(rng.integers(1, 7))
-        C = int(rng.choice([1, 3, 4, 8, 16, 24, 40]))
-        H, W = int(rng.integers(3, 34)), int(rng.integers(3, 34))
-        F = int(rng.integers(1, 90))
-        k = 3 if case % 5 else int(rng.choice([1, 2, 5]))
-        pad = int(rng.integers(0, 2)) if k == 3 else int(rng.integers(0, k))
-        if H + 2 * pad < k or W + 2 * pad < k:
+    """Seeded sweep over geometries nobody picked by hand - 3x3 / stride 1 on small and large images, 1x1 over
+    many channels, and kernels, strides, dilations and paddings of every kind - whichever kernel each one
+    reaches: the plain convolution against the oracle (as a norm, and value by value), BatchNorm and an
+    activation in the epilogue against the separate commands bit for bit, and the pool on top wherever
+    gh_conv2d_can_pool allows it."""
+    routes, pooled, tails = set(), 0, 0
+    for case in range(160):
+        rng = np.random.default_rng(case)
+        B = int(rng.integers(1, 9))
+        C = int(rng.choice([1, 2, 3, 4, 7, 8, 16, 24, 32, 48, 64, 96, 128, 256]))
+        large = rng.random() < 0.25 and C <= 64
+        H, W = (int(rng.integers(20, 120)), int(rng.integers(20, 120))) if large else \
+               (int(rng.integers(1, 34)), int(rng.integers(1, 34)))
+        F = int(rng.choice([1, 3, 8, 15, 16, 17, 31, 32, 33, 48, 64, 65, 100, 128, 130, 256]))
+        if case % 4 == 3:
+            kh, kw = int(rng.choice([1, 2, 3, 5])), int(rng.choice([1, 2, 3, 4]))
+            pad = (int(rng.integers(0, kh)), int(rng.integers(0, kw)))
+            stride = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+            dil = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        elif case % 4 == 2 and C >= 64:
+            kh = kw = 1; pad = (0, 0); stride = dil = (1, 1)
+        else:
+            kh = kw = 3; pad = (int(rng.integers(0, 2)),) * 2; stride = dil = (1, 1)
+        oh, ow = O.conv_out_hw(H, W, kh, kw, pad, stride, dil)
+        if oh < 1 or ow < 1 or B * C * H * W > 6_000_000 or B * F * oh * ow > 6_000_000:
             continue
+        tag = f"case {case}: B{B} C{C} {H}x{W} F{F} k{kh}x{kw} pad{pad} stride{stride} dilation{dil}"
         x = synth.uniform(3000 + case, (B, C, H, W), -1, 1)
-        w = synth.he_normal(4000 + case, (F, C, k, k))
-        got = gpu_conv(ctx, x, w, (pad, pad), (1, 1), (1, 1))
-        ref = O.conv2d(x, w, (pad, pad), (1, 1), (1, 1))
+        w = synth.he_normal(4000 + case, (F, C, kh, kw))
+        routes.add(ctx.lib.gh_conv2d_route(D.cmd_conv2d(1, 1, 1, B, C, H, W, F, kh, kw, pad, stride, dil)))
+        got = gpu_conv(ctx, x, w, pad, stride, dil)
+        ref = O.conv2d(x, w, pad, stride, dil)
         err = rel_frobenius(got, ref)
-        assert err <= TOL, f"case {case}: B{B} C{C} {H}x{W} F{F} k{k} pad{pad}: {err:.3e}"
-        cmd = D.cmd_conv2d(1, 1, 1, B, C, H, W, F, k, k, (pad, pad))
-        if k == 3 and ctx.lib.gh_conv2d_can_pool(cmd) == 1:
+        assert err <= TOL, f"{tag}: {err:.3e}"
+        assert np.abs(got.astype(np.float64) - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max()), f"{tag}: a value is off"
+        if stride != (1, 1) or dil != (1, 1) or pad[0] != pad[1] or kh != kw:
+            continue
+        use_bn = rng.random() < 0.5
+        act = [None, "relu", "leaky"][int(rng.integers(0, 3))]
+        bn = None
+        h = got
+        if use_bn:
+            bn = (synth.normal(13 + case, (F,), 0.0, 0.1), synth.uniform(14 + case, (F,), 0.5, 1.5),
+                  synth.uniform(15 + case, (F,), 0.5, 1.5), synth.normal(16 + case, (F,), 0.0, 0.1))
+            h = gpu_bn(ctx, h.copy(), bn[0], bn[1], bn[2], bn[3], 1e-5)
+        if act == "relu":
+            h = O.relu(h).reshape(h.shape)
+        elif act == "leaky":
+            h = O.leaky_relu(h, 0.1).reshape(h.shape)
+        if use_bn or act:
+            tails += 1
+            assert_bits_equal(gpu_conv_tail(ctx, x, w, pad, bn=bn, act=act, alpha=0.1), h, f"{tag}: bn {use_bn}, {act}")
+        if ctx.lib.gh_conv2d_can_pool(D.cmd_conv2d(1, 1, 1, B, C, H, W, F, kh, kw, pad, pool2=True)) == 1:
             pooled += 1
-            act = gpu_conv(ctx, x, w, (pad, pad), (1, 1), (1, 1), act="relu")
-            want = gpu_pool(ctx, act, (2, 2), (0, 0), (2, 2))
-            assert_bits_equal(gpu_conv_tail(ctx, x, w, (pad, pad), act="relu", pool2=True), want,
-                              f"case {case}: conv+relu+pool B{B} C{C} {H}x{W} F{F} pad{pad}")
-    assert pooled >= 8
+            assert_bits_equal(gpu_conv_tail(ctx, x, w, pad, bn=bn, act=act, alpha=0.1, pool2=True),
+                              gpu_pool(ctx, h, (2, 2), (0, 0), (2, 2)), f"{tag}: bn {use_bn}, {act}, pool")
+    assert pooled >= 40 and tails >= 40 and len(routes) >= 6, (pooled, tails, routes)
 
 
 def test_conv_pointwise_random_geometries(ctx):
