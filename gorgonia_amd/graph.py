@@ -142,8 +142,64 @@ def _un(name):
     return lambda a: a.g.apply(K_ELEMUNARY, [a], name=name)
 
 
+def _calc_broadcast_shape(shape, expected_dims, along):
+    """calcBroadcastShape (shape.go:38-68): the operand's shape in `expected_dims` dimensions with
+    ones at the axes it is repeated along and its own extents, in order, in the free slots."""
+    if len(shape) == expected_dims:
+        return tuple(shape)
+    if len(shape) == 0:
+        return (1,) * expected_dims
+    new = [0] * expected_dims
+    for i in along:
+        new[i] = 1
+    for s in shape:
+        for j in range(expected_dims):
+            if new[j] == 0:
+                new[j] = s
+                break
+    return tuple(new)
+
+
 def _bc(fn):
-    return lambda a, b: a.g.apply(K_BCAST, [a, b], fn=_ffi.BIN_FN[fn])
+    def op(a, b, leftPattern=None, rightPattern=None):
+        """Broadcast<Op>(a, b, leftPattern, rightPattern) (api_gen.go:129-135 over Broadcast, broadcast.go:69-129):
+        a is repeated along the axes of leftPattern and b along those of rightPattern, then the plain operator
+        runs.  Here nothing is repeated in memory: the device operator reads the small operand where the
+        repeated one would hold its copy.  Without patterns the operand with extents of one is the small one."""
+        left, right = list(leftPattern or ()), list(rightPattern or ())
+        if not left and not right:
+            return a.g.apply(K_BCAST, [a, b], fn=_ffi.BIN_FN[fn])
+        ashape, bshape = a.Shape(), b.Shape()
+        x, y = a, b
+        xs, ys = list(ashape), list(bshape)
+        if left:
+            for ax in left:
+                if ax >= len(bshape):
+                    raise EngineError(_ffi.GH_EINVAL, f"Attempting to broadcast a on axis {ax} of b. But b has shape {bshape}")
+            xs = list(_calc_broadcast_shape(ashape, len(bshape), left))
+            if tuple(xs) != tuple(ashape):
+                x = Reshape(a, xs)
+        if right:
+            for ax in right:
+                if ax >= len(ashape):
+                    raise EngineError(_ffi.GH_EINVAL, f"Attempting to broadcast b on axis {ax} of a. But a has shape {ashape}")
+            ys = list(_calc_broadcast_shape(bshape, len(ashape), right))
+            if tuple(ys) != tuple(bshape):
+                y = Reshape(b, ys)
+        # the shapes the repeats would give (repeatOp multiplies the extent of its axis, op_tensor.go:175-188)
+        xr, yr = list(xs), list(ys)
+        for ax in left:
+            xr[ax] *= bshape[ax]
+        for ax in right:
+            yr[ax] *= ashape[ax]
+        if xr != yr:
+            raise EngineError(_ffi.GH_EINVAL, f"Shape mismatch. Expected {tuple(xr)}. Got {tuple(yr)}")
+        if left and right and tuple(xs) != tuple(xr) and tuple(ys) != tuple(yr):
+            # both operands grow: the left one first, as a product with ones (exact), then the right one
+            ones = NewTensor(a.g, np.ones(tuple(xr), dtype=a.Dtype()), resident=True)
+            x = a.g.apply(K_BCAST, [ones, x], fn=_ffi.BIN_FN["mul"])
+        return a.g.apply(K_BCAST, [x, y], fn=_ffi.BIN_FN[fn])
+    return op
 
 
 # api_gen.go names

@@ -379,6 +379,46 @@ def test_measured_replay_keeps_results_and_settles(ctx, monkeypatch):
         m.Close()
 
 
+# operations_broadcast_test.go:24-71 (broadcastAddTests) and :183-230 (broadcastMulTests): name, a, b,
+# leftPattern, rightPattern, expected a op b
+BROADCAST_TABLE = [
+    ("vec-mat", ([100, 200], (2,)), ([1, 2, 3, 4], (2, 2)), [1], None, [101, 102, 203, 204], [10, 20, 60, 80]),
+    ("mat-vec", ([1, 2, 3, 4], (2, 2)), ([100, 200], (2,)), None, [1], [101, 102, 203, 204], [10, 20, 60, 80]),
+    ("rowvec-mat", ([100, 200], (2, 1)), ([1, 2, 3, 4], (2, 2)), [1], None, [101, 102, 203, 204], [10, 20, 60, 80]),
+    ("mat-rowvec", ([1, 2, 3, 4], (2, 2)), ([100, 200], (2, 1)), None, [1], [101, 102, 203, 204], [10, 20, 60, 80]),
+    ("colvec-mat", ([100, 200], (1, 2)), ([1, 2, 3, 4], (2, 2)), [0], None, [101, 202, 103, 204], [10, 40, 30, 80]),
+    ("mat-colvec", ([1, 2, 3, 4], (2, 2)), ([100, 200], (1, 2)), None, [0], [101, 202, 103, 204], [10, 40, 30, 80]),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_broadcast_pattern_table(ctx, dtype):
+    """TestBroadcastAdd / TestBroadcastHadamardProd (operations_broadcast_test.go:167-183, 262-280): the reference's
+    tables (float64 there) through BroadcastAdd / BroadcastHadamardProd with explicit patterns on the tape
+    machine; the multiplication table holds the addition table's operands scaled by ten."""
+    for name, (av, ashp), (bv, bshp), left, right, want_add, want_mul in BROADCAST_TABLE:
+        for fn, scale, want in ((G.BroadcastAdd, 1, want_add), (G.BroadcastHadamardProd, 10, want_mul)):
+            def operand(v, shp):   # the multiplication table's vector is 10, 20 where the addition table's is 100, 200
+                v = np.array(v, dtype=dtype)
+                return (v / scale if v.max() >= 100 else v).astype(dtype).reshape(shp)
+            g = G.NewGraph()
+            a, b = G.NewTensor(g, operand(av, ashp)), G.NewTensor(g, operand(bv, bshp))
+            out = G.Read(fn(a, b, left, right))
+            m = G.NewTapeMachine(g)
+            m.RunAll()
+            assert out.shape == (2, 2) and out.reshape(-1).tolist() == [float(v) for v in want], f"{name} {fn}"
+            m.Close()
+    # both operands repeated: a (2, 1) along axis 1, b (1, 3) along axis 0; subtraction keeps the operand order
+    g = G.NewGraph()
+    a = G.NewTensor(g, np.array([[10], [20]], dtype=dtype))
+    b = G.NewTensor(g, np.array([[1, 2, 3]], dtype=dtype))
+    out = G.Read(G.BroadcastSub(a, b, [1], [0]))
+    m = G.NewTapeMachine(g)
+    m.RunAll()
+    assert out.tolist() == [[9, 8, 7], [19, 18, 17]]
+    m.Close()
+
+
 def test_a_node_read_twice_fills_both_values(ctx):
     """gorgonia.Read makes a readOp node per call (gorgonia.go:311-318): two Reads of one node fill two values,
     whether the value reaches the host through the staging copy of the segment or a copy after the flush."""

@@ -367,3 +367,29 @@ def test_pooling_query_over_random_geometries():
             assert C == 32 and k == 3 and stride == 1 and dil == 1 and pad <= 1 and 4 <= W <= 16 and H <= 16, (B, C, H, W, F, pad)
         assert lib.gh_conv2d_can_keep(f64) == 0 and lib.gh_conv2d_can_pre(f64) == 0
     assert yes > 300 and kept > 20 and folded > 5, (yes, kept, folded)
+
+
+def test_broadcast_patterns_shapes_and_errors():
+    """Broadcast (broadcast.go:69-129) with explicit patterns, graph construction only: the result shapes of the
+    reference's table and its two error cases (operations_broadcast_test.go:147-164: an axis the other operand
+    does not have; repeats that do not reach the other operand's shape)."""
+    from gorgonia_amd import graph as G
+    from gorgonia_amd.engine import EngineError
+
+    def shapes(ashp, bshp, left, right):
+        g = G.NewGraph()
+        a, b = G.NewTensor(g, np.zeros(ashp)), G.NewTensor(g, np.zeros(bshp))
+        return G.BroadcastAdd(a, b, left, right).Shape()
+
+    assert shapes((2,), (2, 2), [1], None) == (2, 2)
+    assert shapes((2, 2), (2,), None, [1]) == (2, 2)
+    assert shapes((1, 2), (2, 2), [0], None) == (2, 2)
+    assert shapes((2, 1), (1, 3), [1], [0]) == (2, 3)
+    assert shapes((), (3, 4), [0, 1], None) == (3, 4)          # a scalar is all ones (shape.go:50-53)
+    assert shapes((4,), (3, 4, 5), [0, 2], None) == (3, 4, 5)  # the operand's extent takes the free slot
+    with pytest.raises(EngineError, match="axis 2 of b"):
+        shapes((2, 1), (2, 2), [2], None)                      # "rowvec-mat: wrong axis"
+    with pytest.raises(EngineError, match="Shape mismatch"):
+        shapes((2, 4), (1, 2), None, [0, 1])                   # "impossible mat-mat"
+    with pytest.raises(EngineError):
+        shapes((3,), (2, 2), [1], None)                        # three values do not fill (?, 1) of a (2, 2)
