@@ -207,7 +207,24 @@ Add, Sub, HadamardProd, HadamardDiv, Pow = _bin("add"), _bin("sub"), _bin("mul")
 Lt, Lte, Gt, Gte, Eq, Ne = _bin("lt"), _bin("lte"), _bin("gt"), _bin("gte"), _bin("eq"), _bin("ne")
 Mod = _bin("mod")
 BroadcastAdd, BroadcastSub = _bc("add"), _bc("sub")
-BroadcastHadamardProd, BroadcastHadamardDiv = _bc("mul"), _bc("div")
+BroadcastHadamardProd, BroadcastHadamardDiv, BroadcastPow = _bc("mul"), _bc("div"), _bc("pow")
+
+
+def _bc_cmp(fn):
+    plain = _bc(fn)
+
+    def op(a, b, retSame=True, leftPattern=None, rightPattern=None):
+        """Broadcast<Cmp>(a, b, retSame, leftPattern, rightPattern) (api_gen.go:174-227).  The device operators
+        write 1 / 0 in the operands' own type (cuda/cmp.go:14-701), which is retSame = true; a Bool result does
+        not exist on this path."""
+        if not retSame:
+            raise EngineError(_ffi.GH_EINVAL, "comparison on the device path returns the operands' type (retSame)")
+        return plain(a, b, leftPattern, rightPattern)
+    return op
+
+
+BroadcastLt, BroadcastGt, BroadcastLte, BroadcastGte = _bc_cmp("lt"), _bc_cmp("gt"), _bc_cmp("lte"), _bc_cmp("gte")
+BroadcastEq, BroadcastNe = _bc_cmp("eq"), _bc_cmp("ne")
 Abs, Sign, Ceil, Floor, Sin, Cos, Exp, Log, Log2 = (_un(n) for n in
                                                      ("abs", "sign", "ceil", "floor", "sin", "cos", "exp", "ln", "log2"))
 Neg, Square, Sqrt, Inverse, InverseSqrt, Cube = (_un(n) for n in

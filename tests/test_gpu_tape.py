@@ -408,7 +408,18 @@ def test_broadcast_pattern_table(ctx, dtype):
             m.RunAll()
             assert out.shape == (2, 2) and out.reshape(-1).tolist() == [float(v) for v in want], f"{name} {fn}"
             m.Close()
-    # both operands repeated: a (2, 1) along axis 1, b (1, 3) along axis 0; subtraction keeps the operand order
+    # ExampleBroadcastGte_creatingTriangleMatrices (example_broadcast_op_test.go:62-105): both operands repeated,
+    # a = 0..2 as (3, 1) along axis 1, b = 0..3 as (1, 4) along axis 0
+    g = G.NewGraph()
+    a = G.NewTensor(g, np.arange(3, dtype=dtype).reshape(3, 1))
+    b = G.NewTensor(g, np.arange(4, dtype=dtype).reshape(1, 4))
+    tl, tu = G.Read(G.BroadcastGte(a, b, True, [1], [0])), G.Read(G.BroadcastLt(a, b, True, [1], [0]))
+    m = G.NewTapeMachine(g)
+    m.RunAll()
+    assert tl.tolist() == [[1, 0, 0, 0], [1, 1, 0, 0], [1, 1, 1, 0]]
+    assert tu.tolist() == [[0, 1, 1, 1], [0, 0, 1, 1], [0, 0, 0, 1]]
+    m.Close()
+    # a (2, 1) along axis 1, b (1, 3) along axis 0; subtraction keeps the operand order
     g = G.NewGraph()
     a = G.NewTensor(g, np.array([[10], [20]], dtype=dtype))
     b = G.NewTensor(g, np.array([[1, 2, 3]], dtype=dtype))
