@@ -430,6 +430,25 @@ def test_broadcast_pattern_table(ctx, dtype):
     m.Close()
 
 
+def test_dev_cuda_graph(ctx):
+    """TestDevCUDA (cuda_test.go:14-58): x = 2 and y = 8 as 1024 x 100 float64 matrices, x + y, x - y and their
+    squares read back (the test's Slice has no device operator in the reference either)."""
+    g = G.NewGraph()
+    x = G.NewTensor(g, np.full((1024, 100), 2.0))
+    y = G.NewTensor(g, np.full((1024, 100), 8.0))
+    xpy, xmy = G.Add(x, y), G.Sub(x, y)
+    outs = [G.Read(n) for n in (xpy, xmy, G.Square(xpy), G.Square(xmy))]
+    for kw in (dict(), dict(graph_replay=True)):
+        m = G.NewTapeMachine(g, **kw)
+        for _ in range(3):
+            for o in outs:
+                o[...] = 0
+            m.RunAll()
+            for o, want in zip(outs, (10.0, -6.0, 100.0, 36.0)):
+                assert o.dtype == np.float64 and (o == want).all()
+        m.Close()
+
+
 def test_a_node_read_twice_fills_both_values(ctx):
     """gorgonia.Read makes a readOp node per call (gorgonia.go:311-318): two Reads of one node fill two values,
     whether the value reaches the host through the staging copy of the segment or a copy after the flush."""
