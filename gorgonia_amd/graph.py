@@ -425,6 +425,8 @@ class TapeMachine:
 
     def _check(self, rc):
         if rc != 0:
+            if not self.h:
+                raise EngineError(rc, "the machine is closed")
             raise EngineError(rc, self.lib.ghh_tape_last_error(self.h).decode(errors="replace"))
 
     def RunAll(self):

@@ -254,33 +254,36 @@ void ghh_tape_destroy(ghh_tape* t) {
   delete t->t;
   delete t;
 }
-const char* ghh_tape_last_error(ghh_tape* t) { return t->err.c_str(); }
-int ghh_tape_init(ghh_tape* t, int device) { return ret(t, t->t->Init(device)); }
-int ghh_tape_compile_only(ghh_tape* t) { return ret(t, t->t->Compile()); }
-int ghh_tape_run_all(ghh_tape* t) { return ret(t, t->t->RunAll()); }
+const char* ghh_tape_last_error(ghh_tape* t) { return t ? t->err.c_str() : "null machine handle"; }
+// (a null handle - a machine that was never made, or one already destroyed by the caller - is an argument error)
+int ghh_tape_init(ghh_tape* t, int device) { return t ? ret(t, t->t->Init(device)) : GH_EINVAL; }
+int ghh_tape_compile_only(ghh_tape* t) { return t ? ret(t, t->t->Compile()) : GH_EINVAL; }
+int ghh_tape_run_all(ghh_tape* t) { return t ? ret(t, t->t->RunAll()) : GH_EINVAL; }
 int ghh_tape_run_all_n(ghh_tape* t, int n) {
+  if (!t) return GH_EINVAL;
   for (int i = 0; i < n; i++) {
     const int rc = ret(t, t->t->RunAll());
     if (rc) return rc;
   }
   return 0;
 }
-int ghh_tape_reset(ghh_tape* t) { return ret(t, t->t->Reset()); }
-int ghh_tape_close(ghh_tape* t) { return ret(t, t->t->Close()); }
-int64_t ghh_tape_gpumem(ghh_tape* t) { return t->t->GpuMem(); }
-int ghh_tape_segments(ghh_tape* t) { return t->t->Segments(); }
-int ghh_tape_graph_launches(ghh_tape* t) { return t->t->GraphLaunches(); }
-int64_t ghh_tape_submit_calls(ghh_tape* t) { return t->t->Eng().SubmitCalls(); }
-uint64_t ghh_tape_register_address(ghh_tape* t, int node) { return t->t->RegisterAddress(node); }
-const void* ghh_tape_read_buffer(ghh_tape* t, int node) { return t->t->ReadBuffer(node); }
-void* ghh_tape_input_buffer(ghh_tape* t, int node) { return t->t->InputBuffer(node); }
+int ghh_tape_reset(ghh_tape* t) { return t ? ret(t, t->t->Reset()) : GH_EINVAL; }
+int ghh_tape_close(ghh_tape* t) { return t ? ret(t, t->t->Close()) : GH_EINVAL; }
+int64_t ghh_tape_gpumem(ghh_tape* t) { return t ? t->t->GpuMem() : 0; }
+int ghh_tape_segments(ghh_tape* t) { return t ? t->t->Segments() : 0; }
+int ghh_tape_graph_launches(ghh_tape* t) { return t ? t->t->GraphLaunches() : 0; }
+int64_t ghh_tape_submit_calls(ghh_tape* t) { return t ? t->t->Eng().SubmitCalls() : 0; }
+uint64_t ghh_tape_register_address(ghh_tape* t, int node) { return t ? t->t->RegisterAddress(node) : 0; }
+const void* ghh_tape_read_buffer(ghh_tape* t, int node) { return t ? t->t->ReadBuffer(node) : nullptr; }
+void* ghh_tape_input_buffer(ghh_tape* t, int node) { return t ? t->t->InputBuffer(node) : nullptr; }
 int ghh_tape_program_string(ghh_tape* t, char* buf, int cap) {
+  if (!t) return 0;
   std::string s = t->t->ProgramString();
   if (buf && cap > 0) snprintf(buf, (size_t)cap, "%s", s.c_str());
   return (int)s.size();
 }
-ghh_engine* ghh_tape_engine(ghh_tape* t) { return &t->eng; }
-int ghh_tape_segment_verdict(ghh_tape* t, int segment) { return t->t->SegmentVerdict(segment); }
-void ghh_tape_phase_ns(ghh_tape* t, int64_t* out3) { t->t->PhaseNs(out3); }
+ghh_engine* ghh_tape_engine(ghh_tape* t) { return t ? &t->eng : nullptr; }
+int ghh_tape_segment_verdict(ghh_tape* t, int segment) { return t ? t->t->SegmentVerdict(segment) : 0; }
+void ghh_tape_phase_ns(ghh_tape* t, int64_t* out3) { if (t) t->t->PhaseNs(out3); }
 
 }  // extern "C"

@@ -430,6 +430,29 @@ def test_broadcast_pattern_table(ctx, dtype):
     m.Close()
 
 
+def test_run_all_n_is_n_run_alls(ctx):
+    """RunAllN(n): n whole RunAll calls - as many submits and waits, the last step's values on the host - and it
+    stops at the first error."""
+    inp = configs.convnet_inputs(8)
+    m0, _, want = run_once(configs.build_convnet, inp, fuse_activations=True)
+    m0.Close()
+    g, outs = configs.build_convnet(inp)
+    m = G.NewTapeMachine(g, fuse_activations=True)
+    m.RunAll()                      # the first run also uploads the resident weights
+    before = m.submit_calls()
+    m.RunAll()
+    per_run = m.submit_calls() - before
+    outs["out"][...] = -1.0
+    m.RunAllN(5)
+    assert per_run >= 1 and m.submit_calls() == before + 6 * per_run
+    assert_bits_equal(outs["out"], want["out"], "after RunAllN(5)")
+    m.RunAllN(0)
+    assert m.submit_calls() == before + 6 * per_run
+    m.Close()
+    with pytest.raises(Exception):
+        m.RunAllN(2)   # a closed machine
+
+
 def test_dev_cuda_graph(ctx):
     """TestDevCUDA (cuda_test.go:14-58): x = 2 and y = 8 as 1024 x 100 float64 matrices, x + y, x - y and their
     squares read back (the test's Slice has no device operator in the reference either)."""
