@@ -622,6 +622,17 @@ Status Graph::Apply(const OpSpec& op, const std::vector<int>& inputs, int* out) 
     if (i < 0 || i >= (int)nodes_.size()) return bad("Apply: unknown input node");
     shapes.push_back(&nodes_[(size_t)i].shape);
   }
+  // the reference's type inference refuses operands of different Dtypes when the graph is built
+  // ("Unification Fail: Float64 ~ Float32 cannot be unified"); so does this
+  switch (op.kind) {
+    case OpKind::ElemBin: case OpKind::BroadcastBin: case OpKind::MatMul: case OpKind::MatVecMul: case OpKind::Outer:
+    case OpKind::BatchedMatMul: case OpKind::Conv2d: case OpKind::BatchNorm:
+      for (size_t i = 1; i < inputs.size(); i++)
+        if (nodes_[(size_t)inputs[i]].dt != nodes_[(size_t)inputs[0]].dt)
+          return bad("Apply: operands of different Dtypes cannot be unified (input 0 and input " + std::to_string(i) + ")");
+      break;
+    default: break;
+  }
   Node n;
   Status st = InferShape(op, shapes, &n.shape);
   if (!st.ok()) return st;
