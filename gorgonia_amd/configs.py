@@ -115,8 +115,9 @@ def build_convnet_train(inp, onehot, lr, read_grads=True, solver="set"):
     x = G.NewTensor(g, inp["x"], True)
     y = G.NewTensor(g, onehot, True)
     w = [G.NewTensor(g, inp[f"w{i}"], True) for i in range(5)]
-    lr_s = G.NewScalar(g, lr)
-    scale = G.NewScalar(g, -1.0 / onehot.size)
+    dt = np.asarray(inp["x"]).dtype   # the scalars in the tensors' own type, as the reference's type inference demands
+    lr_s = G.NewScalar(g, lr, dtype=dt)
+    scale = G.NewScalar(g, -1.0 / onehot.size, dtype=dt)
     conv = dict(kernelShape=(3, 3), pad=(1, 1), stride=(1, 1), dilation=(1, 1))
     acts, h = [], x
     for i in range(3):
