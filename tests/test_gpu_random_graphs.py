@@ -7,7 +7,8 @@ tape machine batches, overwrites dead operands, folds followers into their produ
 (BatchNorm, activation, pooling, bias, SoftMax, a first layer into the second, a kept
 pre-activation value) and replays.  Every value a graph reads must come out with the same bits
 either way, on every run: what a random graph adds to the hand-written ones is intermediate values
-with a second reader or a Read, created before or after the node that would otherwise swallow them."""
+with a second reader or a Read, created before or after the node that would otherwise swallow them,
+and (every fifth graph) the gradient operators behind a stack of conv -> Rectify -> pool layers."""
 import numpy as np
 import pytest
 
@@ -172,9 +173,60 @@ def elementwise_web(b):
     return vals[-1]
 
 
+def training_stack(b):
+    """Forward layers conv -> Rectify [-> pool] and the diff operators symbolic differentiation would insert
+    behind them, from a drawn gradient of the last value: the values between the layers have readers in both
+    directions, which is where the pool takes over a kept convolution and reads through a Rectify."""
+    rng = b.rng
+    B = int(rng.integers(1, 5))
+    C = b.pick([1, 3, 8, 16, 32])
+    H, W = int(rng.integers(6, 20)), int(rng.integers(6, 20))
+    h = b.tensor((B, C, H, W), 0.0, 1.0, resident=False)
+    layers = []
+    for layer in range(int(rng.integers(1, 4))):
+        _, C, H, W = h.Shape()
+        pad = b.pick([0, 1])
+        if H + 2 * pad - 2 < 2 or W + 2 * pad - 2 < 2:
+            break
+        F = b.pick([8, 16, 32, 64])
+        w = b.tensor((F, C, 3, 3), -0.5, 0.5, resident=True)
+        z = G.Conv2d(h, w, (3, 3), (pad, pad), (1, 1), (1, 1))
+        a = G.Rectify(z)
+        pooled = None
+        kind = b.pick(["2x2", "2x2", "3x3", None])
+        if kind == "2x2":
+            pooled = G.MaxPool2D(a, (2, 2), (0, 0), (2, 2))
+        elif kind == "3x3" and a.Shape()[2] >= 3 and a.Shape()[3] >= 3:
+            pooled = G.MaxPool2D(a, (3, 3), (1, 1), (2, 2))
+        else:
+            kind = None
+        layers.append((h, w, z, a, pooled, kind, pad))
+        h = pooled if pooled is not None else a
+        if b.chance(0.2):
+            b.read(h, f"fwd{layer}")
+    b.read(h, "fwd")
+    grad = b.tensor(h.Shape(), -1.0, 1.0, resident=False)
+    for layer in reversed(range(len(layers))):
+        x_in, w, z, a, pooled, kind, pad = layers[layer]
+        if kind == "2x2":
+            grad = G.MaxPool2DDiff(a, grad, (2, 2), (0, 0), (2, 2))
+        elif kind == "3x3":
+            grad = G.MaxPool2DDiff(a, grad, (3, 3), (1, 1), (2, 2))
+        dz = G.RectifyDiff(z, grad)
+        b.read(G.Conv2dDiffFilter(x_in, dz, (3, 3), (pad, pad), (1, 1), (1, 1)), f"dw{layer}")
+        if layer or b.chance(0.5):
+            grad = G.Conv2dDiffImage(dz, w, x_in.Shape(), (3, 3), (pad, pad), (1, 1), (1, 1))
+            if layer == 0:
+                b.read(grad, "dx")
+    return None
+
+
 def build(seed, dtype):
     b = Builder(seed, dtype)
-    shape = seed % 4
+    shape = seed % 5
+    if shape == 4:
+        training_stack(b)
+        return b.g, b.reads
     if shape == 3:
         out = elementwise_web(b)
     else:
