@@ -85,6 +85,8 @@ def NewTensor(g, value, resident=False):
     dt = {np.dtype(np.float32): 0, np.dtype(np.float64): 1}.get(value.dtype, 2)
     nid = g.lib.ghh_graph_new_tensor(g.h, shp, value.ndim, dt, value.ctypes.data_as(C.c_void_p),
                                      int(resident))
+    if nid < 0:
+        raise EngineError(_ffi.GH_EINVAL, g.lib.ghh_graph_last_error(g.h).decode(errors="replace"))
     node = Node(g, nid)
     node.dtype = value.dtype
     return node

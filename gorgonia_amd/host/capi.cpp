@@ -180,6 +180,10 @@ void ghh_graph_destroy(ghh_graph* g) { delete g; }
 const char* ghh_graph_last_error(ghh_graph* g) { return g->err.c_str(); }
 int ghh_graph_new_tensor(ghh_graph* g, const int64_t* shape, int ndim, int dtype, const void* host,
                          int resident) {
+  if (!g) return -1;
+  if (ndim < 0 || ndim > 8 || (ndim > 0 && !shape)) { g->err = "NewTensor: between 0 and 8 dimensions"; return -1; }
+  for (int i = 0; i < ndim; i++)
+    if (shape[i] <= 0) { g->err = "NewTensor: every extent of a shape must be positive"; return -1; }
   Shape s;
   for (int i = 0; i < ndim; i++) s.d.push_back(shape[i]);
   return g->g.NewTensor(s, dtype == 1 ? Dtype::Float64 : dtype == 0 ? Dtype::Float32 : Dtype::Other, host,

@@ -113,7 +113,8 @@ typedef struct ghh_op {
 GH_API ghh_graph* ghh_graph_new(void);
 GH_API void ghh_graph_destroy(ghh_graph* g);
 GH_API const char* ghh_graph_last_error(ghh_graph* g);
-/* NewTensor + WithValue: an input bound to host memory */
+/* NewTensor + WithValue: an input bound to host memory.  Returns the node, or -1 (message in
+ * ghh_graph_last_error) for more than 8 dimensions or an extent that is not positive. */
 GH_API int ghh_graph_new_tensor(ghh_graph* g, const int64_t* shape, int ndim, int dtype,
                                 const void* host, int resident);
 GH_API int ghh_graph_apply(ghh_graph* g, const ghh_op* op, const int* inputs, int n_inputs, int* out);

@@ -408,3 +408,15 @@ def test_operands_of_different_dtypes_are_refused_when_the_graph_is_built():
         with pytest.raises(EngineError, match="cannot be unified"):
             build()
     assert G.Add(a64, a64).Dtype() == np.float64
+
+
+def test_new_tensor_refuses_shapes_the_machine_cannot_hold():
+    from gorgonia_amd import graph as G
+    from gorgonia_amd.engine import EngineError
+    g = G.NewGraph()
+    with pytest.raises(EngineError, match="positive"):
+        G.NewTensor(g, np.ones((0, 3), np.float32))
+    with pytest.raises(EngineError, match="8 dimensions"):
+        G.NewTensor(g, np.ones((1,) * 9, np.float32))
+    assert G.NewTensor(g, np.ones((1,) * 8, np.float32)).Shape() == (1,) * 8
+    assert G.NewScalar(g, 2.0).Shape() == ()
