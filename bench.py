@@ -36,6 +36,16 @@ EAGER_TIMING = False  # --eager-timing: no hipGraph anywhere (for hardware-count
 # A tape machine in "measured" mode runs a segment plainly three times, captures it, replays it twice
 # and then keeps the quicker way: the timed loops start after that.
 WARM_RUNS = 8
+
+
+def warm_up(m, warmup):
+    """The untimed steps in front of a timed loop: the `warmup` asked for (at least WARM_RUNS), then more
+    until SUSTAIN_MS of steps have run - the GPU raises its clocks only under load that lasts, and a timed
+    loop of a few dozen 50 us steps would otherwise be measured on the ramp (time_cmds warms the same way)."""
+    m.RunAllN(max(warmup, WARM_RUNS))
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < SUSTAIN_MS:
+        m.RunAllN(16)
 VERDICTS = {}  # workload -> how its segment ended up being run ("plain" / "replay")
 
 
@@ -341,8 +351,7 @@ def bench_convnet(steps, warmup, batch=128, resident_input=True, graph_replay=Tr
     m = G.NewTapeMachine(g, graph_replay=graph_replay, fuse_activations=True, reupload_resident=reupload_all)
     if borrow_input:
         m.input(xin)[...] = inp["x"]
-    for _ in range(max(warmup, WARM_RUNS)):
-        m.RunAll()
+    warm_up(m, warmup)
     eng = m.engine()
     eng.DoWork()
     t0 = time.perf_counter()
@@ -370,8 +379,7 @@ def bench_convnet_machines(steps, warmup, count=2, batch=128):
     for _ in range(count):
         g, outs = configs.build_convnet(inp, resident_input=True)
         m = G.NewTapeMachine(g, graph_replay=replay_mode(), fuse_activations=True)
-        for _ in range(max(warmup, WARM_RUNS)):
-            m.RunAll()
+        warm_up(m, warmup)
         machines.append((g, m, outs))
     gate = threading.Barrier(count + 1)
 
@@ -408,8 +416,7 @@ def bench_yolo(steps, warmup, resident_input=True, borrow_output=True, borrow_in
     m = G.NewTapeMachine(g, graph_replay=replay_mode() if graph_replay is None else graph_replay, fuse_activations=True)
     if borrow_input:
         m.input(g.x_node)[...] = inp["x"]
-    for _ in range(max(warmup, WARM_RUNS)):
-        m.RunAll()
+    warm_up(m, warmup)
     eng = m.engine()
     eng.DoWork()
     t0 = time.perf_counter()
@@ -431,8 +438,7 @@ def bench_mlp(steps, warmup, resident_input=True):
     inp = configs.mlp_inputs(256)
     g, outs = configs.build_mlp(inp, resident_input=resident_input)
     m = G.NewTapeMachine(g, graph_replay=replay_mode(), fuse_activations=True)
-    for _ in range(max(warmup, WARM_RUNS)):
-        m.RunAll()
+    warm_up(m, warmup)
     eng = m.engine()
     eng.DoWork()
     t0 = time.perf_counter()
@@ -455,8 +461,7 @@ def bench_convnet_train(steps, warmup, batch=128, dtype=np.float32):
     onehot[np.arange(batch), np.arange(batch) % 10] = 1.0
     g, outs = configs.build_convnet_train(inp, onehot, 0.01, read_grads=False, solver="rmsprop")
     m = G.NewTapeMachine(g, graph_replay=replay_mode(), fuse_activations=True)
-    for _ in range(max(warmup, WARM_RUNS)):
-        m.RunAll()
+    warm_up(m, warmup)
     eng = m.engine()
     eng.DoWork()
     t0 = time.perf_counter()
@@ -751,7 +756,9 @@ def main():
                                "plainly - segments of five commands and more run the quicker of plain submits and "
                                "hipGraph replay, timed by the machine on its first runs; weights and input resident, "
                                "every step ends with the output on the host",
-                   "batch": 128, "flop_per_step": 2_093_410_816},
+                   "batch": 128, "flop_per_step": 2_093_410_816,
+                   "untimed_warmup": f"max({a.warmup}, {WARM_RUNS}) steps, then steps until {SUSTAIN_MS:g} ms have passed "
+                                     "(the clocks' ramp), then the timed steps"},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "extra": {
