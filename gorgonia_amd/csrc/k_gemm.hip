@@ -1589,7 +1589,7 @@ __global__ __launch_bounds__(kThreads) void k_dgemm(const double* __restrict__ A
 // transpose is the same code); loads are unconditional at clamped addresses and
 // masked afterwards, so they all stay in flight.  The slices are added in LDS in
 // wavefront order: the result does not depend on scheduling.
-template <int WV>
+template <int WV, bool AV, bool BV>
 __global__ __launch_bounds__(WV * 64) void k_dgemm_skinny(const double* __restrict__ A,
                                                           const double* __restrict__ B,
                                                           double* __restrict__ C, int M, int N, int K,
@@ -1601,25 +1601,53 @@ __global__ __launch_bounds__(WV * 64) void k_dgemm_skinny(const double* __restri
   const int m0 = blockIdx.y * 16, n0 = blockIdx.x * 16;
   const double* ap = A + (int64_t)min(m0 + lr, M - 1) * sai;
   const double* bp = B + (int64_t)min(n0 + lr, N - 1) * sbj;
-  const int kper = (((K + WV - 1) / WV) + 3) & ~3;
+  const int kper = (((K + WV - 1) / WV) + 7) & ~7;
   const int k0 = wave * kper, k1 = min(K, k0 + kper);
   f64x4 acc = {0.0, 0.0, 0.0, 0.0};
-  for (int k = k0; k < k1; k += 16) {
-    double a[4], b[4];
+  if constexpr (AV || BV) {
+    // An operand that is k-contiguous (16-byte aligned rows, K even): a lane fetches two consecutive k of its
+    // row or column in one load (the sixteen k of a step are then two 64-byte pieces instead of sixteen 8-byte
+    // ones); which k a lane group multiplies in which MFMA is the same for both operands - k0 + 8 u + 2 lk + e
+    for (int k = k0; k < k1; k += 16) {
+      f64x2 a[2], b[2];
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
-      const int kc = min(k + 4 * u + lk, K - 1);
-      a[u] = ap[kc * sak];
-      b[u] = bp[kc * sbk];
+      for (int u = 0; u < 2; u++) {
+        const int kk = k + 8 * u + 2 * lk;
+        if constexpr (AV) a[u] = *reinterpret_cast<const f64x2*>(ap + min(kk, K - 2));
+        if constexpr (BV) b[u] = *reinterpret_cast<const f64x2*>(bp + min(kk, K - 2));
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+          if constexpr (!AV) a[u][e] = ap[(int64_t)min(kk + e, K - 1) * sak];
+          if constexpr (!BV) b[u][e] = bp[(int64_t)min(kk + e, K - 1) * sbk];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 2; u++)
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+          const bool ok = k + 8 * u + 2 * lk + e < k1;
+          const double av = ok ? a[u][e] : 0.0, bv = ok ? b[u][e] : 0.0;
+          acc = __builtin_amdgcn_mfma_f64_16x16x4f64(av, bv, acc, 0, 0, 0);
+        }
     }
+  } else {
+    for (int k = k0; k < k1; k += 16) {
+      double a[4], b[4];
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
-      const bool ok = k + 4 * u + lk < k1;
-      a[u] = ok ? a[u] : 0.0;
-      b[u] = ok ? b[u] : 0.0;
+      for (int u = 0; u < 4; u++) {
+        const int kc = min(k + 4 * u + lk, K - 1);
+        a[u] = ap[kc * sak];
+        b[u] = bp[kc * sbk];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const bool ok = k + 4 * u + lk < k1;
+        a[u] = ok ? a[u] : 0.0;
+        b[u] = ok ? b[u] : 0.0;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) acc = __builtin_amdgcn_mfma_f64_16x16x4f64(a[u], b[u], acc, 0, 0, 0);
     }
-#pragma unroll
-    for (int u = 0; u < 4; u++) acc = __builtin_amdgcn_mfma_f64_16x16x4f64(a[u], b[u], acc, 0, 0, 0);
   }
 #pragma unroll
   for (int v = 0; v < 4; v++) part[wave][v * 64 + lane] = acc[v];
@@ -2887,12 +2915,26 @@ int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
       const double* A = (const double*)(uintptr_t)c.ptr[0];
       const double* B = (const double*)(uintptr_t)c.ptr[1];
       double* C = (double*)(uintptr_t)c.ptr[2];
-      if (K >= 256)
-        hipLaunchKernelGGL((k_dgemm_skinny<8>), grid, dim3(512), 0, ctx->stream, A, B, C, M, N, K, ta ? 1 : lda,
-                           ta ? lda : 1, tb ? 1 : ldb, tb ? ldb : 1, (int)c.dim[5]);
-      else
-        hipLaunchKernelGGL((k_dgemm_skinny<4>), grid, dim3(256), 0, ctx->stream, A, B, C, M, N, K, ta ? 1 : lda,
-                           ta ? lda : 1, tb ? 1 : ldb, tb ? ldb : 1, (int)c.dim[5]);
+      // (which wavefront sums which k, and with AV which k shares an MFMA, depends on the shape and the operands'
+      // layout only: a product's bits repeat from run to run)
+      const bool pairs = (K & 1) == 0 && !getenv("GORGONIA_HIP_DGEMM_SKINNY_SCALAR");   // (tuning switch)
+      const bool av = pairs && !ta && (lda & 1) == 0 && (c.ptr[0] & 15) == 0;
+      const bool bv = pairs && tb && (ldb & 1) == 0 && (c.ptr[1] & 15) == 0;
+#define GH_DSK(WV_, AV_, BV_)                                                                                          \
+  hipLaunchKernelGGL((k_dgemm_skinny<WV_, AV_, BV_>), grid, dim3(WV_ * 64), 0, ctx->stream, A, B, C, M, N, K,           \
+                     ta ? 1 : lda, ta ? lda : 1, tb ? 1 : ldb, tb ? ldb : 1, (int)c.dim[5])
+#define GH_DSK_W(WV_)                                            \
+  do {                                                           \
+    if (av && bv) GH_DSK(WV_, true, true);                       \
+    else if (av) GH_DSK(WV_, true, false);                       \
+    else if (bv) GH_DSK(WV_, false, true);                       \
+    else GH_DSK(WV_, false, false);                              \
+  } while (0)
+      if (K >= 512 && !getenv("GORGONIA_HIP_SKINNY_WAVES8")) GH_DSK_W(16);
+      else if (K >= 256) GH_DSK_W(8);
+      else GH_DSK_W(4);
+#undef GH_DSK_W
+#undef GH_DSK
       return gh_check_hip(ctx, hipGetLastError(), "dgemm launch");
     }
     // 128x128 tiles once they fill the device, 64x64 with a longer k-tile below that
