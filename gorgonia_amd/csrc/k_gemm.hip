@@ -2930,8 +2930,7 @@ int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
     else if (bv) GH_DSK(WV_, false, true);                       \
     else GH_DSK(WV_, false, false);                              \
   } while (0)
-      if (K >= 512 && !getenv("GORGONIA_HIP_SKINNY_WAVES8")) GH_DSK_W(16);
-      else if (K >= 256) GH_DSK_W(8);
+      if (K >= 256) GH_DSK_W(8);   // (sixteen wavefronts, as the float32 kernel has them from K = 512, are slower here: 15.7 us against 14.4)
       else GH_DSK_W(4);
 #undef GH_DSK_W
 #undef GH_DSK
