@@ -2806,6 +2806,14 @@ bool gh_try_launch_conv2d_f64_mfma(gh_ctx* ctx, const gh_cmd& c) {
   const int64_t tiles128 = (int64_t)((g.F + 127) / 128) * ((P + 127) / 128);
   // the smaller tiles do less per k-tile, so they take twice the k range per barrier
   const int64_t tiles64 = (int64_t)((g.F + 63) / 64) * ((P + 63) / 64);
+  if (const char* e = getenv("GORGONIA_HIP_CONV64_TILE")) {   // tuning override: 0 32x128, 1 128x128, 2 64x64, 3 32x64
+    switch (atoi(e)) {
+      case 0: launch_conv64_cfg<32, 128, 16>(ctx, c, g); return true;
+      case 1: launch_conv64_cfg<128, 128, 8>(ctx, c, g); return true;
+      case 2: launch_conv64_cfg<64, 64, 16>(ctx, c, g); return true;
+      default: launch_conv64_cfg<32, 64, 16>(ctx, c, g); return true;
+    }
+  }
   if (g.F <= 32) launch_conv64_cfg<32, 128, 16>(ctx, c, g);
   else if (tiles128 >= ctx->cu_count) launch_conv64_cfg<128, 128, 8>(ctx, c, g);
   else if (tiles64 >= ctx->cu_count) launch_conv64_cfg<64, 64, 16>(ctx, c, g);
