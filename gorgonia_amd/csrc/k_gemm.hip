@@ -1605,16 +1605,25 @@ __global__ __launch_bounds__(WV * 64) void k_dgemm_skinny(const double* __restri
   const int k0 = wave * kper, k1 = min(K, k0 + kper);
   f64x4 acc = {0.0, 0.0, 0.0, 0.0};
   if constexpr (AV || BV) {
-    // An operand that is k-contiguous (16-byte aligned rows, K even): a lane fetches two consecutive k of its
-    // row or column in one load (the sixteen k of a step are then two 64-byte pieces instead of sixteen 8-byte
-    // ones); which k a lane group multiplies in which MFMA is the same for both operands - k0 + 8 u + 2 lk + e
+    // An operand that is k-contiguous: a lane fetches two consecutive k of its row or column in one load (the
+    // sixteen k of a step are then two 64-byte pieces instead of sixteen 8-byte ones; 8-byte alignment is all
+    // the load needs); which k a lane group multiplies in which MFMA is the same for both operands -
+    // k0 + 8 u + 2 lk + e.  The pair that would start at the last k of an odd K starts one earlier and is
+    // shifted into place.
     for (int k = k0; k < k1; k += 16) {
       f64x2 a[2], b[2];
 #pragma unroll
       for (int u = 0; u < 2; u++) {
         const int kk = k + 8 * u + 2 * lk;
-        if constexpr (AV) a[u] = *reinterpret_cast<const f64x2*>(ap + min(kk, K - 2));
-        if constexpr (BV) b[u] = *reinterpret_cast<const f64x2*>(bp + min(kk, K - 2));
+        const bool last = kk > K - 2;   // kk == K - 1 (its second k does not exist), or past the end (masked below)
+        if constexpr (AV) {
+          const f64x2 v = *reinterpret_cast<const f64x2_a8*>(ap + min(kk, K - 2));
+          a[u] = last ? f64x2{v[1], 0.0} : v;
+        }
+        if constexpr (BV) {
+          const f64x2 v = *reinterpret_cast<const f64x2_a8*>(bp + min(kk, K - 2));
+          b[u] = last ? f64x2{v[1], 0.0} : v;
+        }
 #pragma unroll
         for (int e = 0; e < 2; e++) {
           if constexpr (!AV) a[u][e] = ap[(int64_t)min(kk + e, K - 1) * sak];
@@ -2925,9 +2934,8 @@ int gh_launch_gemm(gh_ctx* ctx, const gh_cmd& c) {
       double* C = (double*)(uintptr_t)c.ptr[2];
       // (which wavefront sums which k, and with AV which k shares an MFMA, depends on the shape and the operands'
       // layout only: a product's bits repeat from run to run)
-      const bool pairs = (K & 1) == 0 && !getenv("GORGONIA_HIP_DGEMM_SKINNY_SCALAR");   // (tuning switch)
-      const bool av = pairs && !ta && (lda & 1) == 0 && (c.ptr[0] & 15) == 0;
-      const bool bv = pairs && tb && (ldb & 1) == 0 && (c.ptr[1] & 15) == 0;
+      const bool pairs = K >= 2 && !getenv("GORGONIA_HIP_DGEMM_SKINNY_SCALAR");   // (tuning switch)
+      const bool av = pairs && !ta, bv = pairs && tb;
 #define GH_DSK(WV_, AV_, BV_)                                                                                          \
   hipLaunchKernelGGL((k_dgemm_skinny<WV_, AV_, BV_>), grid, dim3(WV_ * 64), 0, ctx->stream, A, B, C, M, N, K,           \
                      ta ? 1 : lda, ta ? lda : 1, tb ? 1 : ldb, tb ? ldb : 1, (int)c.dim[5])
