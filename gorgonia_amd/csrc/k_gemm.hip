@@ -2134,6 +2134,62 @@ __global__ __launch_bounds__(256) void k_conv3x3_wgrad_direct(const float* __res
   }
 }
 
+// The same reduction for a single input channel (a network's first layer): the padded image sits in LDS
+// with a zero halo, so a pixel's nine taps are nine reads at fixed offsets and no bounds test; a wavefront owns
+// one filter and walks the pixels 64 at a time (one coalesced read of dy), nine accumulators per lane; four
+// filters per workgroup, workgroup (g, fb) takes every G-th image.  Slab g of the [G][F][9] workspace gets the
+// lanes' sums folded by a fixed tree; the split-K reduce kernel adds the slabs in order.
+__global__ __launch_bounds__(256) void k_conv3x3_wgrad_c1(const float* __restrict__ x, const float* __restrict__ dy,
+                                                          float* __restrict__ ws, int B, int H, int W, int F, int pad,
+                                                          int oh, int ow, unsigned m_ow, unsigned m_pw) {
+  extern __shared__ float img[];   // (H + 2 pad) rows of W + 2 pad
+  const int PW = W + 2 * pad, PH = H + 2 * pad;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int f = blockIdx.y * 4 + wave;
+  const bool fok = f < F;
+  const int plane = oh * ow;
+  float acc[9];
+#pragma unroll
+  for (int q = 0; q < 9; q++) acc[q] = 0.f;
+  for (int b = blockIdx.x; b < B; b += gridDim.x) {
+    __syncthreads();   // every wavefront is done with the image before
+    const float* xb = x + (int64_t)b * H * W;
+    for (int i = threadIdx.x; i < PH * PW; i += 256) {
+      const int r = (int)__umulhi((unsigned)i, m_pw), c = i - r * PW;
+      const int iy = r - pad, ix = c - pad;
+      img[i] = (iy >= 0 && iy < H && ix >= 0 && ix < W) ? xb[iy * W + ix] : 0.f;
+    }
+    __syncthreads();
+    const float* gy = dy + ((int64_t)b * F + (fok ? f : F - 1)) * plane;
+    // eight pixels per lane at a time: their dy loads are all in flight before the first is used
+    for (int p0 = lane; p0 < plane; p0 += 8 * 64) {
+      float g[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int p = p0 + 64 * u;
+        g[u] = (fok && p < plane) ? gy[p] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int p = min(p0 + 64 * u, plane - 1);   // (a pixel past the end multiplies a zero)
+        const int oy = (int)__umulhi((unsigned)p, m_ow), ox = p - oy * ow;
+        const float* ip = img + oy * PW + ox;
+#pragma unroll
+        for (int kr = 0; kr < 3; kr++)
+#pragma unroll
+          for (int kc = 0; kc < 3; kc++) acc[kr * 3 + kc] = __builtin_fmaf(g[u], ip[kr * PW + kc], acc[kr * 3 + kc]);
+      }
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 9; q++) {
+    float v = acc[q];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    if (lane == 0 && fok) ws[((int64_t)blockIdx.x * F + f) * 9 + q] = v;
+  }
+}
+
 // Input gradient, stride 1: dX is the forward convolution of dy with the
 // filters mirrored and their channel axes swapped, under padding
 // dil*(k-1) - pad, so the forward kernels compute it.  This writes those filters:
@@ -3136,6 +3192,30 @@ int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
     float* wsd = (float*)ctx->workspace;
     const float* xd = (const float*)(uintptr_t)c.ptr[0];
     const float* dyd = (const float*)(uintptr_t)c.ptr[1];
+    const size_t img_bytes = (size_t)(g.H + 2 * g.padH) * (g.W + 2 * g.padH) * 4;
+    if (g.C == 1 && img_bytes <= 60 * 1024 && g.oh * g.ow >= 64 && g.ow >= 2 && !getenv("GORGONIA_HIP_WGRAD_NO_C1")) {   // (tuning switch)
+      // as many slabs as give every compute unit a workgroup, within what the images and the workspace allow
+      const int fby = (int)cdiv(F, 4);
+      // a workgroup's images follow each other (stage, barrier, sum), so few per workgroup; 128 images of 28 x 28,
+      // 32 filters: 25.8 us with 16 slabs, 16.0 with 32, 12.5 with 64, 13.0 with 128 (slab sum included; 15.8 on the
+      // kernel below)
+      int G1 = 64;
+      if (const char* e = getenv("GORGONIA_HIP_WGRAD_C1_SLABS")) G1 = atoi(e);   // tuning override
+      if (G1 > 256) G1 = 256;
+      if (G1 > B) G1 = B;
+      while (G1 > 1 && (int64_t)G1 * F * CKK * 4 > ctx->workspace_bytes) G1--;
+      if (G1 < 1) G1 = 1;
+      // exact while i * d < 2^32: ceil(2^32 / d)
+      auto magic = [](int d) { return (unsigned)((0x100000000ull + (unsigned)d - 1) / (unsigned)d); };
+      const int PW = g.W + 2 * g.padH;
+      hipLaunchKernelGGL(k_conv3x3_wgrad_c1, dim3((unsigned)G1, (unsigned)fby), dim3(256), img_bytes, ctx->stream, xd, dyd,
+                         wsd, B, g.H, g.W, F, g.padH, g.oh, g.ow, magic(g.ow), magic(PW));
+      int rc1 = gh_check_hip(ctx, hipGetLastError(), "single-channel filter-gradient launch");
+      if (rc1) return rc1;
+      hipLaunchKernelGGL((k_splitk_reduce_lanes<StoreRowMajor, 4>), dim3((int)cdiv((int64_t)F * CKK * 4, 256)), dim3(256),
+                         0, ctx->stream, wsd, G1, F, CKK, StoreRowMajor{(float*)(uintptr_t)c.ptr[2], CKK}, 0, 0.f);
+      return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
+    }
 #define GH_WGRAD_DIRECT(C_, FB_)                                                                             \
   hipLaunchKernelGGL((k_conv3x3_wgrad_direct<C_, FB_>), dim3((unsigned)G, (unsigned)cdiv(F, FB_)), dim3(256), 0, \
                      ctx->stream, xd, dyd, wsd, B, g.H, g.W, F, g.padH, g.oh, g.ow)
