@@ -3175,6 +3175,15 @@ static int launch_slab_reduce(gh_ctx* ctx, const float* ws, int splits, int F, i
   return gh_check_hip(ctx, hipGetLastError(), "split-K reduce launch");
 }
 
+// The direct kernel's shapes that k_conv3x3_wgrad_c1 takes: one channel, a padded image of at most 60 KB, at least
+// a wavefront of output pixels.
+static bool wgrad_c1_takes(const gh_cmd& c) {
+  if (!conv_direct_shape(c) || c.dim[1] != 1 || c.dim[4] > 65535) return false;
+  const ConvGeom g = conv_geom(c);
+  const size_t img_bytes = (size_t)(g.H + 2 * g.padH) * (g.W + 2 * g.padH) * 4;
+  return img_bytes <= 60 * 1024 && g.oh * g.ow >= 64 && g.ow >= 2 && !getenv("GORGONIA_HIP_WGRAD_NO_C1");   // (tuning switch)
+}
+
 // dW = dY2d^T . col  (ptr[0] = x, ptr[1] = dy, ptr[2] = dw)
 int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
   if (gh_dtype_of(c.flags) == GH_F64) return gh_launch_conv2d_bwd_filter_f64(ctx, c);
@@ -3193,7 +3202,7 @@ int gh_launch_conv2d_bwd_filter(gh_ctx* ctx, const gh_cmd& c) {
     const float* xd = (const float*)(uintptr_t)c.ptr[0];
     const float* dyd = (const float*)(uintptr_t)c.ptr[1];
     const size_t img_bytes = (size_t)(g.H + 2 * g.padH) * (g.W + 2 * g.padH) * 4;
-    if (g.C == 1 && img_bytes <= 60 * 1024 && g.oh * g.ow >= 64 && g.ow >= 2 && !getenv("GORGONIA_HIP_WGRAD_NO_C1")) {   // (tuning switch)
+    if (wgrad_c1_takes(c)) {
       // as many slabs as give every compute unit a workgroup, within what the images and the workspace allow
       const int fby = (int)cdiv(F, 4);
       // a workgroup's images follow each other (stage, barrier, sum), so few per workgroup; 128 images of 28 x 28,
@@ -3394,6 +3403,7 @@ extern "C" int gh_conv2d_route(const gh_cmd* c) {
 extern "C" int gh_conv2d_bwd_filter_route(const gh_cmd* c) {
   if (!c || c->opcode != GH_OP_CONV2D_BWD_FILTER) return -1;
   if (gh_dtype_of(c->flags) == GH_F64) return GH_WGRAD_ROUTE_F64;
+  if (wgrad_c1_takes(*c)) return GH_WGRAD_ROUTE_SINGLE_CHANNEL;
   if (conv_direct_shape(*c) && c->dim[4] <= 65535) return GH_WGRAD_ROUTE_DIRECT;
   if (gh_conv_wgrad_small_takes(*c)) return GH_WGRAD_ROUTE_SMALL;
   return GH_WGRAD_ROUTE_GEMM;

@@ -347,7 +347,8 @@ enum gh_wgrad_route {
   GH_WGRAD_ROUTE_DIRECT = 0,  /* 3x3, at most four channels: reduction on the vector ALUs     */
   GH_WGRAD_ROUTE_SMALL = 1,   /* 3x3 over images up to 16 x 16: dy and x in LDS, MFMA          */
   GH_WGRAD_ROUTE_GEMM = 2,    /* every other geometry: implicit GEMM over the output pixels    */
-  GH_WGRAD_ROUTE_F64 = 3      /* float64 (its own kernels)                                     */
+  GH_WGRAD_ROUTE_F64 = 3,     /* float64 (its own kernels)                                     */
+  GH_WGRAD_ROUTE_SINGLE_CHANNEL = 4   /* 3x3 over one channel: the image in LDS, a wavefront per filter */
 };
 GH_API int gh_conv2d_bwd_filter_route(const gh_cmd* conv_bwd_filter);
 /* The same for a GEMM command (Engine.MatMul, cuda/linalg.go:110-229, where cuBLAS chooses):

@@ -165,7 +165,7 @@ def test_conv_route_of_every_parity_case_list():
 
 
 def test_filter_gradient_routes():
-    """gh_conv2d_bwd_filter_route: the backward case table reaches all three float32 kernels, the cases written
+    """gh_conv2d_bwd_filter_route: the backward case table reaches all four float32 kernels, the cases written
     for the small-image kernel run on it, and the training configurations' layers run where the design says."""
     from tests import test_gpu_backward as T
     lib = _ffi.load()
@@ -174,14 +174,17 @@ def test_filter_gradient_routes():
         cmd = D.cmd_conv2d_bwd_filter(0x10000, 0x20000, 0x30000, B, Cn, H, W, F, kh, kw, pad, stride, dil, dtype=dtype)
         return lib.gh_conv2d_bwd_filter_route(C.byref(cmd))
 
-    DIRECT, SMALL, GEMM, F64 = 0, 1, 2, 3
+    DIRECT, SMALL, GEMM, F64, SINGLE = 0, 1, 2, 3, 4
     seen = [route(*c) for c in T.CONV_BWD_CASES]
-    assert set(seen) == {DIRECT, SMALL, GEMM}
+    assert set(seen) == {DIRECT, SMALL, GEMM, SINGLE}
     small = [c for c in T.CONV_BWD_CASES if c[1] % 16 == 0 and c[2] <= 16 and c[3] <= 16 and c[4] >= 16 and c[5] == 3]
     assert len(small) >= 8
     for c in small:
         assert route(*c) == SMALL, c
-    assert route(128, 1, 28, 28, 32, 3, 3, (1, 1)) == DIRECT          # convnet conv0
+    assert route(128, 1, 28, 28, 32, 3, 3, (1, 1)) == SINGLE          # convnet conv0
+    assert route(4, 1, 6, 6, 8, 3, 3, (0, 0)) == DIRECT               # sixteen output pixels: less than a wavefront
+    assert route(2, 1, 130, 130, 8, 3, 3, (1, 1)) == DIRECT           # the padded image does not fit the LDS budget
+    assert route(2, 3, 28, 28, 8, 3, 3, (1, 1)) == DIRECT
     assert route(128, 32, 14, 14, 64, 3, 3, (1, 1)) == SMALL          # conv1
     assert route(128, 64, 7, 7, 128, 3, 3, (1, 1)) == SMALL           # conv2
     assert route(8, 512, 13, 13, 1024, 3, 3, (1, 1)) == SMALL         # yolo-shaped layer 6
