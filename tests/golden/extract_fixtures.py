@@ -10,7 +10,7 @@ Writes next to this script:
     leaky_relu.json    nn_test.go TestLeakyRelu (float32 case)
     conv.json          known_issues_test.go TestIssue233_F32, blas_test.go TestUse
     softmax_do.json    op_softmax_test.go testCasesSoftMaxDo
-    binop.json         op_math_test.go binOpTests (values only, no gradients)
+    binop.json         op_math_test.go binOpTests (operands, result, the two derivatives)
     batchnorm.json     nn_amd64_test.go bnAllCases (float32 cases)
 """
 import json
@@ -123,12 +123,12 @@ def binop():
                 vals.append({"bits": int(m.group(1)), "scalar": True, "v": [float(m.group(2))]})
             else:
                 vals.append({"bits": int(m.group(3)), "scalar": False, "v": nums(m.group(4))})
-            if len(vals) == 3:
+            if len(vals) == 5:
                 break
-        a, b, correct = vals
-        out.append({"op": op, "a": a, "b": b, "correct": correct})
+        a, b, correct, deriv_a, deriv_b = vals
+        out.append({"op": op, "a": a, "b": b, "correct": correct, "deriv_a": deriv_a, "deriv_b": deriv_b})
     assert len(out) == 32, len(out)
-    dump("binop.json", {"source": "op_math_test.go:23-360 binOpTests (a, b, correct)", "cases": out})
+    dump("binop.json", {"source": "op_math_test.go:23-360 binOpTests (a, b, correct, correctDerivA, correctDerivB)", "cases": out})
 
 
 def batchnorm():

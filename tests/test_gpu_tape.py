@@ -523,3 +523,62 @@ def test_lisp_machine_differential(ctx):
             for k in outs2:
                 assert_bits_equal(outs2[k], want[k], f"{build.__name__}.{k}: tape {kw} == lisp")
             m.Close()
+
+
+def test_cuda_basic_arithmetic_table_with_gradients(ctx):
+    """TestCUDABasicArithmetic (op_math_cuda_test.go:44-99) at graph level: every entry of binOpTests
+    (op_math_test.go:23-360) as a graph on the tape machine, its value and the two derivatives of
+    Sum(result) equal to the table's, exactly.  The derivative nodes are the ones the reference's
+    symbolic differentiation inserts, built here from the same device operators: addDiffExpr,
+    subDiffExpr, hadamardProdDiffExpr, hadamardDivDiffExpr (operatorPointwise_binary.go:430-840) on
+    a gradient of ones; a scalar operand's derivative is the sum of the elementwise one
+    (elemBinOp.SymDiff, op_math.go:232-240), taken on the host as the reference takes it (Sum has no
+    device function there).  The vector-vector Mul entries are inner products, another operator."""
+    import json
+    import os
+    cases = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "binop.json")))["cases"]
+    ops = {"Add": G.Add, "Sub": G.Sub, "Mul": G.HadamardProd, "HadamardProd": G.HadamardProd,
+           "Div": G.HadamardDiv, "HadamardDiv": G.HadamardDiv}
+    ran = 0
+    for n, c in enumerate(cases):
+        sa, sb = c["a"]["scalar"], c["b"]["scalar"]
+        if c["op"] == "Mul" and not (sa or sb):
+            continue
+        dt = np.float32 if c["a"]["bits"] == 32 else np.float64
+
+        def node(g, side):
+            v = np.array(side["v"], dtype=dt)
+            return G.NewScalar(g, v[0], dtype=dt) if side["scalar"] else G.NewTensor(g, v)
+
+        g = G.NewGraph()
+        x, y = node(g, c["a"]), node(g, c["b"])
+        z = ops[c["op"]](x, y)
+        ones = np.ones(z.Shape(), dtype=dt)
+        grad = G.NewScalar(g, 1.0, dtype=dt) if z.Shape() == () else G.NewTensor(g, ones)
+        kind = ops[c["op"]]
+        if kind is G.Add:
+            dx, dy = grad, grad
+        elif kind is G.Sub:
+            dx, dy = grad, G.Neg(grad)
+        elif kind is G.HadamardProd:
+            dx, dy = G.HadamardProd(y, grad), G.HadamardProd(x, grad)
+        else:
+            dx, dy = G.HadamardDiv(grad, y), G.HadamardProd(G.Neg(G.HadamardDiv(z, y)), grad)
+        got = {"z": G.Read(z)}
+        if dx is not grad:
+            got["dx"] = G.Read(dx)
+        if dy is not grad:
+            got["dy"] = G.Read(dy)
+        m = G.NewTapeMachine(g)
+        m.RunAll()
+        m.Close()
+        assert got["z"].dtype == dt
+        assert np.array_equal(got["z"].reshape(-1), np.array(c["correct"]["v"], dtype=dt)), (n, c["op"], got["z"])
+        for name, operand_is_scalar, key in (("dx", sa, "deriv_a"), ("dy", sb, "deriv_b")):
+            d = got.get(name, ones).reshape(-1)
+            if operand_is_scalar and d.size > 1:
+                d = np.array([d.sum(dtype=dt)], dtype=dt)
+            want = np.array(c[key]["v"], dtype=dt)
+            assert d.dtype == dt and np.array_equal(d, want), (n, c["op"], name, d, want)
+        ran += 1
+    assert ran >= 26
