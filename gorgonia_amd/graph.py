@@ -235,15 +235,25 @@ Tanh, Sigmoid, Log1p, Expm1, Softplus = (_un(n) for n in ("tanh", "sigmoid", "lo
 
 
 def Mul(a, b, transA=False, transB=False):
-    """operations.go:52-130: matrix-matrix, matrix-vector or vector-vector (outer) product."""
+    """operations.go:52-74: scalar operand -> HadamardProd; vector . vector -> the inner product (a scalar);
+    vector x matrix -> matVecMul of the transposed matrix; matrix x vector; matrix x matrix.  transA / transB are
+    the flags the reference's linAlgBinOp carries when its differentiation builds the gradient products
+    (operatorLinAlg.go:14-68)."""
     sa, sb = a.Shape(), b.Shape()
+    if sa == () or sb == ():
+        return HadamardProd(a, b)
     if len(sa) == 2 and len(sb) == 2:
         return a.g.apply(K_MATMUL, [a, b], trans_a=transA, trans_b=transB)
     if len(sa) == 2 and len(sb) == 1:
         return a.g.apply(K_MATVEC, [a, b], trans_a=transA)
+    if len(sa) == 1 and len(sb) == 2:
+        return a.g.apply(K_MATVEC, [b, a], trans_a=True)
     if len(sa) == 1 and len(sb) == 1:
-        return a.g.apply(K_OUTER, [a, b])
-    raise EngineError(_ffi.GH_EINVAL, f"Mul: unsupported shapes {sa} x {sb}")
+        if sa != sb:
+            raise EngineError(_ffi.GH_EINVAL, f"Mul: vectors of different lengths {sa} . {sb}")
+        # the engine has MatVecMul, MatMul and Outer (cuda/linalg.go:47-260): the inner product is the 1 x n matrix a times b
+        return Reshape(a.g.apply(K_MATVEC, [Reshape(a, (1, sa[0])), b]), ())
+    raise EngineError(_ffi.GH_EINVAL, f"Mul: not yet implemented for a {sa} b {sb}")
 
 
 def OuterProd(a, b):

@@ -582,3 +582,47 @@ def test_cuda_basic_arithmetic_table_with_gradients(ctx):
             assert d.dtype == dt and np.array_equal(d, want), (n, c["op"], name, d, want)
         ran += 1
     assert ran >= 26
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_mul_table_with_gradients(ctx, dt):
+    """TestMul (operations_test.go:43-110) over mulTests: Mul of a vector and a matrix, two matrices, two vectors
+    on RangedFrom(0) operands, and the gradients of Sum(result) - of the inner product itself for two vectors -
+    equal to the table.  The gradient nodes are those of matVecMulDiffExpr, matMulDiffExpr and vecDotDiffExpr
+    (operatorLinAlg.go:51-101, 181-202, 232-244) on a gradient of ones."""
+    def ranged(g, shape):
+        return G.NewTensor(g, np.arange(int(np.prod(shape)), dtype=dt).reshape(shape))
+
+    # x vector: Mul(x, w) is the matrix-vector product of w transposed (operations.go:62-64)
+    g = G.NewGraph()
+    x, w = ranged(g, (2,)), ranged(g, (2, 3))
+    z = G.Mul(x, w)
+    assert z.Shape() == (3,)
+    grad = G.NewTensor(g, np.ones(3, dtype=dt))
+    got = {"z": G.Read(z), "dw": G.Read(G.OuterProd(x, grad)), "dx": G.Read(G.Mul(w, grad))}
+    m = G.NewTapeMachine(g); m.RunAll(); m.Close()
+    assert np.array_equal(got["z"], [3, 4, 5])
+    assert np.array_equal(got["dx"], [3, 12]) and got["dx"].shape == (2,)
+    assert np.array_equal(got["dw"].reshape(-1), [0, 0, 0, 1, 1, 1]) and got["dw"].shape == (2, 3)
+
+    # x mat
+    g = G.NewGraph()
+    x, w = ranged(g, (3, 2)), ranged(g, (2, 3))
+    z = G.Mul(x, w)
+    grad = G.NewTensor(g, np.ones((3, 3), dtype=dt))
+    got = {"z": G.Read(z), "dx": G.Read(G.Mul(grad, w, transB=True)), "dw": G.Read(G.Mul(x, grad, transA=True))}
+    m = G.NewTapeMachine(g); m.RunAll(); m.Close()
+    assert np.array_equal(got["z"], np.arange(6).reshape(3, 2) @ np.arange(6).reshape(2, 3))
+    assert np.array_equal(got["dx"].reshape(-1), [3, 12, 3, 12, 3, 12]) and got["dx"].shape == (3, 2)
+    assert np.array_equal(got["dw"].reshape(-1), [6, 6, 6, 9, 9, 9]) and got["dw"].shape == (2, 3)
+
+    # x_vec_w_vec: the inner product, a scalar, differentiated itself
+    g = G.NewGraph()
+    x, w = ranged(g, (6,)), ranged(g, (6,))
+    z = G.Mul(x, w)
+    assert z.Shape() == ()
+    grad = G.NewScalar(g, 1.0, dtype=dt)
+    got = {"z": G.Read(z), "dx": G.Read(G.HadamardProd(w, grad)), "dw": G.Read(G.HadamardProd(x, grad))}
+    m = G.NewTapeMachine(g); m.RunAll(); m.Close()
+    assert got["z"].dtype == dt and got["z"].reshape(-1)[0] == 55
+    assert np.array_equal(got["dx"], np.arange(6)) and np.array_equal(got["dw"], np.arange(6))

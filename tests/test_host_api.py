@@ -420,3 +420,21 @@ def test_new_tensor_refuses_shapes_the_machine_cannot_hold():
         G.NewTensor(g, np.ones((1,) * 9, np.float32))
     assert G.NewTensor(g, np.ones((1,) * 8, np.float32)).Shape() == (1,) * 8
     assert G.NewScalar(g, 2.0).Shape() == ()
+
+
+def test_mul_follows_the_reference_dispatch():
+    """operations.go:52-74: a scalar operand makes a HadamardProd, two vectors the inner product (a scalar),
+    vector x matrix the product with the transposed matrix; anything else is refused."""
+    g = G.NewGraph()
+    v6, m23, v2, v3 = (G.NewTensor(g, np.zeros(s, np.float32)) for s in ((6,), (2, 3), (2,), (3,)))
+    s = G.NewScalar(g, 2.0)
+    assert G.Mul(s, m23).Shape() == (2, 3) and G.Mul(m23, s).Shape() == (2, 3) and G.Mul(s, s).Shape() == ()
+    assert G.Mul(v6, v6).Shape() == ()
+    assert G.Mul(v2, m23).Shape() == (3,)
+    assert G.Mul(m23, v3).Shape() == (2,)
+    with pytest.raises(G.EngineError):
+        G.Mul(v2, v3)
+    with pytest.raises(G.EngineError):
+        G.Mul(v3, m23)          # 3 against the 2 rows of the matrix
+    with pytest.raises(G.EngineError):
+        G.Mul(G.NewTensor(g, np.zeros((2, 2, 2), np.float32)), m23)
