@@ -206,8 +206,32 @@ def _bc(fn):
 
 # api_gen.go names
 Add, Sub, HadamardProd, HadamardDiv, Pow = _bin("add"), _bin("sub"), _bin("mul"), _bin("div"), _bin("pow")
-Lt, Lte, Gt, Gte, Eq, Ne = _bin("lt"), _bin("lte"), _bin("gt"), _bin("gte"), _bin("eq"), _bin("ne")
 Mod = _bin("mod")
+
+
+def _cmp(fn):
+    plain = _bin(fn)
+
+    def op(a, b, retSame=True):
+        """<Cmp>(a, b, retSame) (api_gen.go:80-127).  The device operators write 1 / 0 in the operands' own type
+        (cuda/cmp.go:14-701), which is retSame = true; a Bool result does not exist on this path."""
+        if not retSame:
+            raise EngineError(_ffi.GH_EINVAL, "comparison on the device path returns the operands' type (retSame)")
+        return plain(a, b)
+    return op
+
+
+Lt, Lte, Gt, Gte, Eq, Ne = _cmp("lt"), _cmp("lte"), _cmp("gt"), _cmp("gte"), _cmp("eq"), _cmp("ne")
+
+
+def Div(a, b):
+    """operations.go:114-122: HadamardDiv for a scalar operand or equal shapes; matrix division does not exist
+    (the reference panics with "Unhandled")."""
+    if a.Shape() == () or b.Shape() == () or a.Shape() == b.Shape():
+        return HadamardDiv(a, b)
+    raise EngineError(_ffi.GH_EINVAL, f"Div: unhandled for shapes {a.Shape()} and {b.Shape()}")
+
+
 BroadcastAdd, BroadcastSub = _bc("add"), _bc("sub")
 BroadcastHadamardProd, BroadcastHadamardDiv, BroadcastPow = _bc("mul"), _bc("div"), _bc("pow")
 
@@ -280,6 +304,11 @@ def Conv1d(im, filter, kernel, pad, stride, dilation):
 def MaxPool2D(x, kernel, pad, stride):
     """nnops.MaxPool2D (nn.go:322-375): pad has 2 values (symmetric) or 4 (N, S, W, E)."""
     return x.g.apply(K_MAXPOOL, [x], ints=list(kernel) + [len(pad)] + list(pad) + list(stride))
+
+
+def MaxPool1D(x, kernel, pad, stride):
+    """nn.go:378-380: MaxPool2D over (B, C, 1, W) with kernel {1, kernel}, pad {0, pad}, stride {1, stride}."""
+    return MaxPool2D(x, (1, kernel), (0, pad), (1, stride))
 
 
 def BatchNorm(x, scale, bias, runningMean, runningVariance, epsilon=1e-5):

@@ -249,6 +249,34 @@ def test_conv1d_on_the_tape(ctx):
         m.Close()
 
 
+def test_maxpool1d_on_the_tape(ctx):
+    """MaxPool1D (nn.go:378-380) is MaxPool2D over a height-1 image: the oracle's bits, and behind a Conv1d
+    whose result it may take over."""
+    from oracle import binding as O
+    x = synth.uniform(13, (3, 8, 1, 97), -1, 1)
+    for kernel, pad, stride in ((2, 0, 2), (3, 1, 2), (4, 2, 3), (2, 1, 1)):
+        g = G.NewGraph()
+        out = G.Read(G.MaxPool1D(G.NewTensor(g, x), kernel, pad, stride))
+        m = G.NewTapeMachine(g, fuse_activations=True)
+        m.RunAll()
+        want = O.maxpool2d(x, (1, kernel), (0, pad), (1, stride))
+        assert out.shape == want.shape and want.shape[2] == 1
+        assert_bits_equal(out, want, f"{kernel} {pad} {stride}")
+        m.Close()
+    w = synth.he_normal(14, (12, 8, 1, 3))
+    res = []
+    for kw in (dict(), dict(fuse_activations=True)):
+        g = G.NewGraph()
+        y = G.Rectify(G.Conv1d(G.NewTensor(g, x), G.NewTensor(g, w, resident=True), 3, 1, 1, 1))
+        out = G.Read(G.MaxPool1D(y, 2, 0, 2))
+        m = G.NewTapeMachine(g, **kw)
+        m.RunAll()
+        res.append(out.copy())
+        m.Close()
+    assert res[0].shape == (3, 12, 1, 48)
+    assert_bits_equal(res[1], res[0], "folded against plain")
+
+
 def test_borrowed_reads_hold_what_read_copies(ctx):
     """ReadBorrowed leaves a value in the machine's pinned buffer; Read copies it out.  Same bits,
     for a value only the host reads (written there by its kernel), one that other nodes also

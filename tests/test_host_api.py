@@ -438,3 +438,16 @@ def test_mul_follows_the_reference_dispatch():
         G.Mul(v3, m23)          # 3 against the 2 rows of the matrix
     with pytest.raises(G.EngineError):
         G.Mul(G.NewTensor(g, np.zeros((2, 2, 2), np.float32)), m23)
+
+
+def test_comparisons_take_ret_same_and_div_is_hadamard_div():
+    """api_gen.go:80-127 (retSame), operations.go:114-122 (Div)."""
+    g = G.NewGraph()
+    a, b = G.NewTensor(g, np.zeros((2, 3), np.float32)), G.NewTensor(g, np.ones((2, 3), np.float32))
+    for cmp in (G.Lt, G.Lte, G.Gt, G.Gte, G.Eq, G.Ne):
+        assert cmp(a, b, True).Shape() == (2, 3)
+        with pytest.raises(G.EngineError):
+            cmp(a, b, False)
+    assert G.Div(a, b).Shape() == (2, 3) and G.Div(a, G.NewScalar(g, 2.0)).Shape() == (2, 3)
+    with pytest.raises(G.EngineError):
+        G.Div(a, G.NewTensor(g, np.ones((3, 2), np.float32)))
