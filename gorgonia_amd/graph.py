@@ -326,7 +326,11 @@ def LeakyRelu(x, alpha):
     return x.g.apply(K_LEAKY, [x], f0=alpha)
 
 
-def SoftMax(x):
+def SoftMax(x, *axes):
+    """SoftMax(x, axes...) (op_softmax.go:13-17, 33-43): over the last axis, the reference's default, which is
+    the only one the device operator has; another axis is refused."""
+    if axes and axes[0] not in (-1, len(x.Shape()) - 1):
+        raise EngineError(_ffi.GH_EINVAL, f"SoftMax: axis {axes[0]} of a {len(x.Shape())}-d value is not on the device path (last axis only)")
     return x.g.apply(K_SOFTMAX, [x])
 
 

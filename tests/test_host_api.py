@@ -451,3 +451,11 @@ def test_comparisons_take_ret_same_and_div_is_hadamard_div():
     assert G.Div(a, b).Shape() == (2, 3) and G.Div(a, G.NewScalar(g, 2.0)).Shape() == (2, 3)
     with pytest.raises(G.EngineError):
         G.Div(a, G.NewTensor(g, np.ones((3, 2), np.float32)))
+
+
+def test_softmax_takes_the_last_axis_only():
+    g = G.NewGraph()
+    a = G.NewTensor(g, np.zeros((4, 6), np.float32))
+    assert G.SoftMax(a).Shape() == G.SoftMax(a, -1).Shape() == G.SoftMax(a, 1).Shape() == (4, 6)
+    with pytest.raises(G.EngineError):
+        G.SoftMax(a, 0)
