@@ -95,6 +95,7 @@ HOST_SYMBOLS = {
     "ghh_tape_compile_only": (C.c_int, [_P]),
     "ghh_tape_run_all": (C.c_int, [_P]),
     "ghh_tape_run_all_n": (C.c_int, [_P, C.c_int]),
+    "ghh_tape_watch": (C.c_int, [_P, C.c_int, C.c_int]),
     "ghh_tape_reset": (C.c_int, [_P]),
     "ghh_tape_close": (C.c_int, [_P]),
     "ghh_tape_gpumem": (C.c_int64, [_P]),

@@ -449,7 +449,7 @@ class TapeMachine:
     """NewTapeMachine(g, ...) / RunAll / Reset / Close (vm_tape.go:45-249)."""
 
     def __init__(self, g, graph_replay=False, reupload_resident=False, fuse_activations=False,
-                 device=0, compile_only=False, engine=None, node_at_a_time=False):
+                 device=0, compile_only=False, engine=None, node_at_a_time=False, watch_nan=False, watch_inf=False):
         self.g = g
         self.lib = g.lib
         self.fused = self.lib.ghh_graph_fuse_activations(g.h) if fuse_activations else 0
@@ -463,6 +463,8 @@ class TapeMachine:
             self.h = self.lib.ghh_tape_new_with_engine(g.h, engine.h, mode, int(reupload_resident))
         else:
             self.h = self.lib.ghh_tape_new(g.h, mode, int(reupload_resident))
+        if watch_nan or watch_inf:
+            self._check(self.lib.ghh_tape_watch(self.h, int(watch_nan), int(watch_inf)))
         if compile_only:
             self._check(self.lib.ghh_tape_compile_only(self.h))
         else:
@@ -546,15 +548,27 @@ class TapeMachine:
         return buf.value.decode()
 
 
-def NewLispMachine(g, **kw):
+def NewLispMachine(g, *opts, **kw):
     """NewLispMachine(g) (vm_genera.go:43-120), forward execution: every node is run and waited for
     on its own.  The reference's tests run one graph on both machines and compare."""
+    for o in opts:
+        kw.update(o)
     return TapeMachine(g, node_at_a_time=True, **kw)
 
 
 def WithEngine(e):
     """VMOpt of the reference (vm.go:318-329): NewTapeMachine(g, WithEngine(e))."""
     return {"engine": e}
+
+
+def WithNaNWatch():
+    """VMOpt of the reference (vm.go:138-151): watch for NaNs when executing; this slows the execution down."""
+    return {"watch_nan": True}
+
+
+def WithInfWatch():
+    """VMOpt of the reference (vm.go:153-166): watch for +Inf and -Inf when executing."""
+    return {"watch_inf": True}
 
 
 def NewTapeMachine(g, *opts, **kw):

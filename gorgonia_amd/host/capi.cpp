@@ -271,6 +271,11 @@ int ghh_tape_run_all_n(ghh_tape* t, int n) {
   }
   return 0;
 }
+int ghh_tape_watch(ghh_tape* t, int nan, int inf) {
+  if (!t) return GH_EINVAL;
+  t->t->SetWatch(nan != 0, inf != 0);
+  return 0;
+}
 int ghh_tape_reset(ghh_tape* t) { return t ? ret(t, t->t->Reset()) : GH_EINVAL; }
 int ghh_tape_close(ghh_tape* t) { return t ? ret(t, t->t->Close()) : GH_EINVAL; }
 int64_t ghh_tape_gpumem(ghh_tape* t) { return t ? t->t->GpuMem() : 0; }

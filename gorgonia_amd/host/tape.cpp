@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <chrono>
+#include <cstdio>
 #include <cstring>
 #include <sstream>
 
@@ -1135,7 +1136,7 @@ Status TapeMachine::flush() {
     return st;
   };
   auto eager = [&]() { return launch_and_wait([&]() { return eng_.SubmitPending(); }); };
-  if (!opt_.graph_replay) return eager();
+  if (!opt_.graph_replay || opt_.watch_nan || opt_.watch_inf) return eager();
   const size_t idx = (size_t)seg_index_++;
   if (seg_cache_.size() <= idx) seg_cache_.resize(idx + 1);
   SegCache& sc = seg_cache_[idx];
@@ -1291,6 +1292,26 @@ Status TapeMachine::RunAll() {
         if (opt_.node_at_a_time) {
           st = flush();  // DoWork after every node (vm_genera.go:144)
           if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": " + op_name(n.op) + ": DoWork failed");
+        }
+        if (opt_.watch_nan || opt_.watch_inf) {
+          // the value just written, checked before anything else runs (vm_tape.go:271-315)
+          if (!opt_.node_at_a_time) {
+            st = flush();
+            if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": " + op_name(n.op) + ": DoWork failed");
+          }
+          char idhex[24];
+          std::snprintf(idhex, sizeof idhex, "%x", (unsigned)n.id);
+          bool hit = false;
+          if (opt_.watch_nan && n.dt != Dtype::Other) {
+            st = eng_.HasNaN(out, &hit);
+            if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": watchNaN");
+            if (hit) return Status::Err(GH_ESTATE, "NaN found in value. Node: " + op_name(n.op) + "(" + idhex + ")");
+          }
+          if (opt_.watch_inf && n.dt != Dtype::Other) {
+            st = eng_.HasInf(out, &hit);
+            if (!st.ok()) return st.Wrap("PC " + std::to_string(pc) + ": watchInf");
+            if (hit) return Status::Err(GH_ESTATE, "Inf found in value. Node: " + op_name(n.op) + "(" + idhex + ")");
+          }
         }
         break;
       }

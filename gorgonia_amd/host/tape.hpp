@@ -173,6 +173,13 @@ struct TapeOptions {
   // an input's register.  Same operators, same kernels: the values are those of
   // the batched machine, which is what running one graph on both machines checks.
   bool node_at_a_time = false;
+  // WithNaNWatch() / WithInfWatch() (vm.go:138-166; the checks of vm_tape.go:271-315): after every operator
+  // its value is searched for NaN / +-Inf on the device (the engine's HasNaN / HasInf) and the run stops
+  // at the first hit with "NaN found in value. Node: ..." - later operators, weight updates included,
+  // do not run.  Every operator is then submitted and waited for on its own, which "slows the execution
+  // down" here as it does there; segments are neither batched across operators nor replayed.
+  bool watch_nan = false;
+  bool watch_inf = false;
 };
 
 class TapeMachine {
@@ -192,6 +199,7 @@ class TapeMachine {
   Status Init(int device);
   Status Compile();  // program only, no device
   Status RunAll();
+  void SetWatch(bool nan, bool inf) { opt_.watch_nan = nan; opt_.watch_inf = inf; }
   Status Reset();   // vm_tape.go:123-134: pc = 0, arena reset
   Status Close();
   Engine& Eng() { return eng_; }

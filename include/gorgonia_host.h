@@ -161,6 +161,12 @@ GH_API void ghh_tape_destroy(ghh_tape* t);
 GH_API const char* ghh_tape_last_error(ghh_tape* t);
 GH_API int ghh_tape_init(ghh_tape* t, int device);   /* compile + engine init */
 GH_API int ghh_tape_run_all(ghh_tape* t);            /* RunAll */
+/* WithNaNWatch() / WithInfWatch() (vm.go:138-166; vm_tape.go:271-315): from the next RunAll on, every
+ * operator is submitted and waited for on its own and its value searched for NaN / +-Inf on the device;
+ * the run stops at the first hit with GH_ESTATE and "NaN found in value. Node: <operator>(<id>)" (or
+ * "Inf found ..."), the operators behind it - weight updates included - not run.  nan = inf = 0 turns
+ * the watch off again. */
+GH_API int ghh_tape_watch(ghh_tape* t, int nan, int inf);
 /* n RunAll calls one after the other, stopping at the first error: the loop of a compiled caller
  * (`for i := 0; i < n; i++ { vm.RunAll(); vm.Reset() }`, cuda_test.go:125-141) without an
  * interpreter's call overhead between the steps; every step still ends with its results on the host. */

@@ -654,3 +654,55 @@ def test_mul_table_with_gradients(ctx, dt):
     m = G.NewTapeMachine(g); m.RunAll(); m.Close()
     assert got["z"].dtype == dt and got["z"].reshape(-1)[0] == 55
     assert np.array_equal(got["dx"], np.arange(6)) and np.array_equal(got["dw"], np.arange(6))
+
+
+@pytest.mark.parametrize("machine", [G.NewTapeMachine, G.NewLispMachine])
+def test_nan_and_inf_watch(ctx, machine):
+    """WithNaNWatch / WithInfWatch (vm.go:138-166, vm_tape.go:271-315): the run stops at the first operator
+    whose value holds a NaN / an Inf, naming it; what comes after it is not run.  Without the watch the same
+    graph runs through, and on a clean graph the watch changes no bit."""
+    x = synth.uniform(71, (37, 129), 0.5, 2.0)
+
+    def build(poison):
+        g = G.NewGraph()
+        v = x.copy()
+        if poison == "nan":
+            v[17, 5] = -1.0          # ln of a negative number
+        if poison == "inf":
+            v[3, 100] = 0.0          # ln 0
+        a = G.NewTensor(g, v)
+        b = G.Log(a)
+        c = G.Square(G.Add(b, b))
+        return g, {"log": G.Read(b), "after": G.Read(c)}
+
+    g, want = build(None)
+    m = machine(g); m.RunAll(); m.Close()
+    g, got = build(None)
+    m = machine(g, G.WithNaNWatch(), G.WithInfWatch())
+    m.RunAll(); m.RunAll()
+    m.Close()
+    assert_bits_equal(got["log"], want["log"], "log")
+    assert_bits_equal(got["after"], want["after"], "after")
+
+    for poison, opt, other, word in (("nan", G.WithNaNWatch, G.WithInfWatch, "NaN"), ("inf", G.WithInfWatch, G.WithNaNWatch, "Inf")):
+        g, got = build(poison)
+        for v in got.values():
+            v[...] = -7.0
+        m = machine(g, opt())
+        with pytest.raises(G.EngineError) as e:
+            m.RunAll()
+        assert f"{word} found in value. Node: elemunary.ln(1)" in str(e.value), str(e.value)
+        assert np.all(got["after"] == -7.0) and np.all(got["log"] == -7.0)   # nothing behind the hit ran
+        m.Close()
+        # the other watch lets this value pass at the logarithm; unwatched, the graph runs through
+        g, got = build(poison)
+        m = machine(g)
+        m.RunAll()
+        assert (np.isnan(got["log"]).sum() == 1) if poison == "nan" else (np.isinf(got["log"]).sum() == 1)
+        m.Close()
+    # -Inf squared is +Inf, a NaN stays a NaN: the Inf watch alone sees the NaN graph through
+    g, got = build("nan")
+    m = machine(g, G.WithInfWatch())
+    m.RunAll()
+    assert np.isnan(got["after"]).sum() == 1
+    m.Close()

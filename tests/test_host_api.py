@@ -459,3 +459,14 @@ def test_softmax_takes_the_last_axis_only():
     assert G.SoftMax(a).Shape() == G.SoftMax(a, -1).Shape() == G.SoftMax(a, 1).Shape() == (4, 6)
     with pytest.raises(G.EngineError):
         G.SoftMax(a, 0)
+
+
+def test_watch_options_reach_the_machine():
+    """WithNaNWatch / WithInfWatch (vm.go:138-166) are options of both machines; the C entry refuses a null handle."""
+    from gorgonia_amd import engine as E
+    assert G.WithNaNWatch() == {"watch_nan": True} and G.WithInfWatch() == {"watch_inf": True}
+    assert E.load_host().ghh_tape_watch(None, 1, 1) != 0
+    g = G.NewGraph()
+    G.Read(G.Neg(G.NewTensor(g, np.zeros((2, 2), np.float32))))
+    m = G.NewTapeMachine(g, G.WithNaNWatch(), G.WithInfWatch(), compile_only=True)
+    assert "neg" in m.program()
