@@ -145,8 +145,15 @@ def dense_tail(b, h):
             h = G.Rectify(h)
             b.tap(h, f"relu{layer}", 0.15, 0.15)
         cols = n
-    if b.chance(0.6):
+    kind = b.pick(["softmax", "softmax", "softmax", "matvec", "vecmat", None])
+    if kind == "softmax":
         h = G.SoftMax(h)
+    elif kind == "matvec":      # matrix x vector, then the inner product with a vector (operations.go:52-74)
+        h = G.Mul(h, b.tensor((cols,), -0.5, 0.5))
+        b.tap(h, "matvec", 0.3, 0.0)
+        h = G.Mul(h, b.tensor((rows,), -0.5, 0.5))
+    elif kind == "vecmat":      # vector x matrix: the product with the transposed matrix
+        h = G.Mul(b.tensor((rows,), -0.5, 0.5), h)
     return h
 
 
