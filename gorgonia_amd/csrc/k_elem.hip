@@ -528,12 +528,33 @@ __global__ void k_set_flag(int* flag, int v) { *flag = v; }
 // counter without atomics; here any matching lane stores 1 (a benign race on
 // a single value).
 template <class T, bool NAN_CHECK>
+__device__ __forceinline__ bool has_hit(T v) {
+  return NAN_CHECK ? (v != v) : (v == (T)INFINITY || v == -(T)INFINITY);
+}
+template <class T, bool NAN_CHECK>
 __global__ __launch_bounds__(kBlock) void k_has(const T* __restrict__ A, int64_t n, int* flag) {
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   bool hit = false;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
-    const T v = A[i];
-    hit |= NAN_CHECK ? (v != v) : (v == (T)INFINITY || v == -(T)INFINITY);
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) hit |= has_hit<T, NAN_CHECK>(A[i]);
+  if (hit) *flag = 1;
+}
+// The same search over 16-byte vectors (A aligned to 16 bytes, nv whole vectors), four loads in flight per lane:
+// a value this large is a stream out of HBM and nothing else.
+template <class T, bool NAN_CHECK>
+__global__ __launch_bounds__(kBlock) void k_has_vec(const T* __restrict__ A, int64_t nv, int* flag) {
+  typedef typename VecOf<T>::type V;
+  constexpr int N = VecOf<T>::N, U = 4;
+  const V* Av = reinterpret_cast<const V*>(A);
+  const int64_t stride = (int64_t)gridDim.x * kBlock * U;
+  bool hit = false;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock * U + threadIdx.x; i < nv; i += stride) {
+    V v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = Av[min(i + (int64_t)u * kBlock, nv - 1)];   // past the end: the last vector again
+#pragma unroll
+    for (int u = 0; u < U; u++)
+#pragma unroll
+      for (int e = 0; e < N; e++) hit |= has_hit<T, NAN_CHECK>(v[u][e]);
   }
   if (hit) *flag = 1;
 }
@@ -792,22 +813,40 @@ int gh_launch_fill(gh_ctx* ctx, const gh_cmd& c) {
   return gh_check_hip(ctx, hipGetLastError(), "fill launch");
 }
 
+template <class T>
+static void launch_has(gh_ctx* ctx, const T* A, int64_t n, int* flag, bool nanc) {
+  constexpr int N = VecOf<T>::N;
+  // whole 16-byte vectors from the first aligned element on; the few elements in front of them and behind, one by one
+  int64_t head = 0;
+  while (head < n && (((uintptr_t)(A + head)) & 15u)) head++;
+  const int64_t nv = (n - head) / N, tail0 = head + nv * N;
+  if (nv >= 4 * kBlock) {
+    const int g = grid_for(ctx, nv, 4);
+    if (nanc) hipLaunchKernelGGL((k_has_vec<T, true>), dim3(g), dim3(kBlock), 0, ctx->stream, A + head, nv, flag);
+    else hipLaunchKernelGGL((k_has_vec<T, false>), dim3(g), dim3(kBlock), 0, ctx->stream, A + head, nv, flag);
+    if (head) {
+      if (nanc) hipLaunchKernelGGL((k_has<T, true>), dim3(1), dim3(kBlock), 0, ctx->stream, A, head, flag);
+      else hipLaunchKernelGGL((k_has<T, false>), dim3(1), dim3(kBlock), 0, ctx->stream, A, head, flag);
+    }
+    if (tail0 < n) {
+      if (nanc) hipLaunchKernelGGL((k_has<T, true>), dim3(1), dim3(kBlock), 0, ctx->stream, A + tail0, n - tail0, flag);
+      else hipLaunchKernelGGL((k_has<T, false>), dim3(1), dim3(kBlock), 0, ctx->stream, A + tail0, n - tail0, flag);
+    }
+    return;
+  }
+  const int g = grid_for(ctx, n, 8);
+  if (nanc) hipLaunchKernelGGL((k_has<T, true>), dim3(g), dim3(kBlock), 0, ctx->stream, A, n, flag);
+  else hipLaunchKernelGGL((k_has<T, false>), dim3(g), dim3(kBlock), 0, ctx->stream, A, n, flag);
+}
+
 int gh_launch_has_nan_inf(gh_ctx* ctx, const gh_cmd& c) {
   const int64_t n = c.dim[0];
   int* flag = (int*)(uintptr_t)c.ptr[1];
   hipLaunchKernelGGL(k_set_flag, dim3(1), dim3(1), 0, ctx->stream, flag, 0);
   if (n > 0) {
-    const int g = grid_for(ctx, n, 8);
     const bool nanc = c.opcode == GH_OP_HAS_NAN;
-    if (gh_dtype_of(c.flags) == GH_F64) {
-      const double* A = (const double*)(uintptr_t)c.ptr[0];
-      if (nanc) hipLaunchKernelGGL((k_has<double, true>), dim3(g), dim3(kBlock), 0, ctx->stream, A, n, flag);
-      else hipLaunchKernelGGL((k_has<double, false>), dim3(g), dim3(kBlock), 0, ctx->stream, A, n, flag);
-    } else {
-      const float* A = (const float*)(uintptr_t)c.ptr[0];
-      if (nanc) hipLaunchKernelGGL((k_has<float, true>), dim3(g), dim3(kBlock), 0, ctx->stream, A, n, flag);
-      else hipLaunchKernelGGL((k_has<float, false>), dim3(g), dim3(kBlock), 0, ctx->stream, A, n, flag);
-    }
+    if (gh_dtype_of(c.flags) == GH_F64) launch_has(ctx, (const double*)(uintptr_t)c.ptr[0], n, flag, nanc);
+    else launch_has(ctx, (const float*)(uintptr_t)c.ptr[0], n, flag, nanc);
   }
   return gh_check_hip(ctx, hipGetLastError(), "hasNaN/hasInf launch");
 }

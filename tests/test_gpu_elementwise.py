@@ -411,6 +411,38 @@ def test_has_nan_inf(ctx):
     ctx.free(flag)
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_has_nan_inf_finds_one_value_anywhere(ctx, dt):
+    """One NaN / Inf at the first element, the last, in the unaligned elements in front of the 16-byte vectors,
+    behind them and in the middle, of tensors at every 4- or 8-byte offset: found; absent: not found; values next
+    to the tensor never looked at."""
+    code = _ffi.F32 if dt == np.float32 else _ffi.F64
+    size = np.dtype(dt).itemsize
+    flag = ctx.malloc(4)
+    rng = np.random.default_rng(5)
+    for n in (1, 3, 4100, 65537, 1 << 20):
+        for off in range(0, 16 // size + 1):
+            host = synth.uniform(80 + off, (n + 8,), -4, 4).astype(dt)
+            host[:off] = np.nan                  # outside the tensor: must not be seen
+            host[off + n:] = np.inf
+            d = ctx.upload(host)
+            a = d + off * size
+            for kind in ("nan", "inf"):
+                ctx.run(D.cmd_has(kind, a, flag, n, dtype=code))
+                assert ctx.d2h(flag, (1,), np.int32)[0] == 0, (n, off, kind)
+            for pos in sorted({0, n - 1, min(n - 1, 2), max(0, n - 3), int(rng.integers(n))}):
+                for kind, val in (("nan", np.nan), ("inf", -np.inf)):
+                    y = host.copy()
+                    y[off + pos] = val
+                    ctx.h2d(d, y)
+                    ctx.run(D.cmd_has(kind, a, flag, n, dtype=code))
+                    assert ctx.d2h(flag, (1,), np.int32)[0] == 1, (n, off, pos, kind)
+                    ctx.run(D.cmd_has("inf" if kind == "nan" else "nan", a, flag, n, dtype=code))
+                    assert ctx.d2h(flag, (1,), np.int32)[0] == 0, (n, off, pos, kind, "other")
+            ctx.free(d)
+    ctx.free(flag)
+
+
 def test_denormals_and_division_are_ieee(ctx):
     """No flush-to-zero, correctly rounded division (the reference builds its
     kernels with -ftz=false -prec-div=true, cmd/cudagen/main.go:41-43)."""
