@@ -452,7 +452,9 @@ class TapeMachine:
                  device=0, compile_only=False, engine=None, node_at_a_time=False, watch_nan=False, watch_inf=False):
         self.g = g
         self.lib = g.lib
-        self.fused = self.lib.ghh_graph_fuse_activations(g.h) if fuse_activations else 0
+        # a watched machine checks every operator's own value, so nothing is folded into its producer (a pool
+        # drops the NaN its input held: the folded command's result would hide it)
+        self.fused = self.lib.ghh_graph_fuse_activations(g.h) if fuse_activations and not (watch_nan or watch_inf) else 0
         self._shared_engine = engine  # WithEngine(e) (vm.go:318-329): kept alive, never closed here
         # graph_replay: False, True (capture on the second run, replay from then on) or
         # "measured" (time plain submits against replays first, keep the quicker)

@@ -165,7 +165,9 @@ GH_API int ghh_tape_run_all(ghh_tape* t);            /* RunAll */
  * operator is submitted and waited for on its own and its value searched for NaN / +-Inf on the device;
  * the run stops at the first hit with GH_ESTATE and "NaN found in value. Node: <operator>(<id>)" (or
  * "Inf found ..."), the operators behind it - weight updates included - not run.  nan = inf = 0 turns
- * the watch off again. */
+ * the watch off again.  The values checked are those of the graph's commands: after
+ * ghh_graph_fuse_activations a folded command is checked as one (a max-pool folded behind a convolution
+ * drops a NaN the convolution produced), so watch graphs that were not folded. */
 GH_API int ghh_tape_watch(ghh_tape* t, int nan, int inf);
 /* n RunAll calls one after the other, stopping at the first error: the loop of a compiled caller
  * (`for i := 0; i < n; i++ { vm.RunAll(); vm.Reset() }`, cuda_test.go:125-141) without an

@@ -706,3 +706,29 @@ def test_nan_and_inf_watch(ctx, machine):
     m.RunAll()
     assert np.isnan(got["after"]).sum() == 1
     m.Close()
+
+
+def test_watch_sees_a_nan_a_pool_would_drop(ctx):
+    """A max-pool never selects a NaN (strict >), so the pooled value of a convolution that produced one is clean:
+    a watched machine folds nothing and stops at the convolution."""
+    x = synth.uniform(91, (2, 8, 12, 12), 0, 1)
+    x[1, 3, 5, 5] = np.nan
+    w = synth.he_normal(92, (16, 8, 3, 3))
+
+    def build():
+        g = G.NewGraph()
+        h = G.Conv2d(G.NewTensor(g, x), G.NewTensor(g, w, resident=True), (3, 3), (1, 1), (1, 1), (1, 1))
+        return g, G.Read(G.MaxPool2D(G.Rectify(h), (2, 2), (0, 0), (2, 2)))
+
+    g, out = build()
+    m = G.NewTapeMachine(g, fuse_activations=True)
+    assert m.fused > 0
+    m.RunAll(); m.Close()
+    assert not np.isnan(out).any()
+    g, out = build()
+    m = G.NewTapeMachine(g, G.WithNaNWatch(), fuse_activations=True)
+    assert m.fused == 0
+    with pytest.raises(G.EngineError) as e:
+        m.RunAll()
+    assert "NaN found in value. Node: conv2d(" in str(e.value), str(e.value)
+    m.Close()
