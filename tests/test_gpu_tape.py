@@ -732,3 +732,87 @@ def test_watch_sees_a_nan_a_pool_would_drop(ctx):
         m.RunAll()
     assert "NaN found in value. Node: conv2d(" in str(e.value), str(e.value)
     m.Close()
+
+
+UNARY_API = {"Abs": "abs", "Sign": "sign", "Ceil": "ceil", "Floor": "floor", "Sin": "sin", "Cos": "cos", "Exp": "exp",
+             "Log": "ln", "Log2": "log2", "Neg": "neg", "Square": "square", "Sqrt": "sqrt", "Inverse": "inverse",
+             "InverseSqrt": "invsqrt", "Cube": "cube", "Tanh": "tanh", "Sigmoid": "sigmoid", "Log1p": "log1p",
+             "Expm1": "expm1", "Softplus": "softplus"}
+BINARY_API = {"Add": "add", "Sub": "sub", "HadamardProd": "mul", "HadamardDiv": "div", "Pow": "pow", "Mod": "mod",
+              "Lt": "lt", "Lte": "lte", "Gt": "gt", "Gte": "gte", "Eq": "eq", "Ne": "ne"}
+
+
+def _ulps(got, want):
+    """Distance in units in the last place of the arrays' own type; equal NaNs and equal zeros count as 0."""
+    it = np.int32 if got.dtype == np.float32 else np.int64
+    top = np.iinfo(it).max
+    gi, wi = got.reshape(-1).view(it).astype(np.int64), want.reshape(-1).view(it).astype(np.int64)
+    gi = np.where(gi < 0, -(gi & top), gi)
+    wi = np.where(wi < 0, -(wi & top), wi)
+    d = np.abs(gi - wi)
+    d[np.isnan(got.reshape(-1)) & np.isnan(want.reshape(-1))] = 0
+    return d
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_every_pointwise_name_on_both_machines(ctx, dt):
+    """Every unary and binary name of api_gen.go:6-127 as a graph on the tape machine and on the lisp machine
+    (operatorPointwise_unary_test.go:14-95 runs each unary operator on both): the two machines agree bit for bit
+    and stand within 2 ulp of the oracle's function of that name (0 for the single-operation ones), tensor with
+    tensor, tensor with scalar and scalar with tensor."""
+    from oracle import binding as O
+    x = synth.uniform(111, (33, 65), 0.25, 3.0).astype(dt)
+    y = synth.uniform(112, (33, 65), 0.5, 2.5).astype(dt)
+    y[::7, ::5] = x[::7, ::5]                      # equal pairs for the comparisons
+    s = np.array(1.75, dtype=dt)
+    exact = {"abs", "sign", "ceil", "floor", "neg", "square", "sqrt", "inverse", "cube"} | (set(BINARY_API.values()) - {"pow"})
+
+    def run(machine, build):
+        g = G.NewGraph()
+        out = G.Read(build(g))
+        m = machine(g)
+        m.RunAll()
+        m.Close()
+        return out
+
+    def check(name, fn, build, want):
+        a, b = run(G.NewTapeMachine, build), run(G.NewLispMachine, build)
+        assert a.dtype == dt and a.shape == x.shape
+        assert_bits_equal(a, b, f"{name}: tape against lisp")
+        u = _ulps(a, np.asarray(want, dtype=dt).reshape(x.shape))
+        assert u.max() <= (0 if fn in exact else 2), f"{name} ({np.dtype(dt).name}): {u.max()} ulp"
+
+    with np.errstate(all="ignore"):
+        for name, fn in UNARY_API.items():
+            check(name, fn, lambda g: getattr(G, name)(G.NewTensor(g, x)), O.unary(fn, x))
+        for name, fn in BINARY_API.items():
+            op = getattr(G, name)
+            check(name + " vv", fn, lambda g: op(G.NewTensor(g, x), G.NewTensor(g, y)), O.binop(fn, "vv", x, y))
+            check(name + " vs", fn, lambda g: op(G.NewTensor(g, x), G.NewScalar(g, s, dtype=dt)),
+                  O.binop(fn, "vs", x, s.reshape(1)))
+            check(name + " sv", fn, lambda g: op(G.NewScalar(g, s, dtype=dt), G.NewTensor(g, y)),
+                  O.binop(fn, "sv", s.reshape(1), y))
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_batched_matmul_graph(ctx, dt):
+    """BatchedMatMul(a, b, transes...) (operations.go:76-98) as a graph operator on both machines, all four
+    transpose combinations, leading dimensions of rank 1 and 2, against the float64 product."""
+    tol = 1e-5 if dt == np.float32 else 1e-12
+    for lead in ((5,), (2, 3)):
+        for ta in (False, True):
+            for tb in (False, True):
+                a = synth.uniform(121, lead + ((9, 7) if ta else (7, 9)), -1, 1).astype(dt)
+                b = synth.uniform(122, lead + ((11, 9) if tb else (9, 11)), -1, 1).astype(dt)
+                want = np.matmul(np.swapaxes(a, -1, -2) if ta else a, np.swapaxes(b, -1, -2) if tb else b, dtype=np.float64)
+                res = []
+                for machine in (G.NewTapeMachine, G.NewLispMachine):
+                    g = G.NewGraph()
+                    out = G.Read(G.BatchedMatMul(G.NewTensor(g, a), G.NewTensor(g, b), ta, tb))
+                    m = machine(g)
+                    m.RunAll()
+                    m.Close()
+                    assert out.dtype == dt and out.shape == lead + (7, 11)
+                    assert rel_frobenius(out, want) <= tol, (lead, ta, tb)
+                    res.append(out)
+                assert_bits_equal(res[0], res[1], f"{lead} {ta} {tb}: tape against lisp")

@@ -166,3 +166,42 @@ def test_adam_steps_replay_with_corrections_from_memory(ctx, dtype):
         assert_bits_equal(r2, c2, f"adam v, iteration {t + 1}")
     assert m.graph_launches() >= 4, "the step did not stay the same command"
     m.Close()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("machine", [G.NewTapeMachine, G.NewLispMachine])
+def test_batchnorm_training_graph(ctx, dt, machine):
+    """BatchNorm in training mode and its gradient as graph operators on both machines: the oracle's values; the
+    running statistics live in resident tensors and carry over from run to run; and what the reference's own
+    (commented-out) device test asks of the result (ops/nn/api_cuda_test.go:24-75): on Gaussian input of shape
+    (5, 2, 3, 4) every channel of the output has mean 0 within 1e-5 and mean square 1 within 1e-4."""
+    from oracle import binding as O
+    shape = (5, 2, 3, 4)
+    x = synth.normal(61, shape).astype(dt)
+    dy = synth.uniform(62, shape, -1, 1).astype(dt)
+    Cn = shape[1]
+    g = G.NewGraph()
+    xn = G.NewTensor(g, x)
+    rm = G.NewTensor(g, np.zeros(Cn, dt), resident=True)
+    rv = G.NewTensor(g, np.ones(Cn, dt), resident=True)
+    sm = G.NewTensor(g, np.zeros(Cn, dt), resident=True)
+    sv = G.NewTensor(g, np.zeros(Cn, dt), resident=True)
+    y = G.BatchNormTrain(xn, rm, rv, sm, sv, momentum=0.9, epsilon=1e-5)
+    dx = G.BatchNormDiff(xn, G.NewTensor(g, dy), sm, sv, epsilon=1e-5)
+    got = {"y": G.Read(y), "dx": G.Read(dx), "rm": G.Read(rm), "rv": G.Read(rv)}
+    m = machine(g)
+    tol = 1e-5 if dt == np.float32 else 1e-12
+    want_rm, want_rv = np.zeros(Cn, dt), np.ones(Cn, dt)
+    for run in range(3):
+        m.RunAll()
+        want_y, want_rm, want_rv, w_sm, w_sv = O.bn_train_stats(x, want_rm, want_rv, 0.9, 1e-5)
+        want_dx = O.bn_bwd(x, dy, w_sm, w_sv, 1e-5, True)
+        for k, want in (("y", want_y), ("dx", want_dx), ("rm", want_rm), ("rv", want_rv)):
+            assert got[k].dtype == dt
+            assert np.linalg.norm(got[k].astype(np.float64) - want) <= tol * np.linalg.norm(want), (run, k)
+    m.Close()
+    yv = got["y"].astype(np.float64)
+    mean = yv.mean(axis=(0, 2, 3))
+    mean_sq = (yv * yv).mean(axis=(0, 2, 3))
+    assert np.all(np.abs(mean) < 1e-5), mean
+    assert np.all(np.abs(mean_sq - 1.0) < 1e-4), mean_sq
